@@ -1,0 +1,125 @@
+/* C ABI of the gfx950 (MI355X) ragged-dot library, libtkx_ragged_dot.so.
+ *
+ * This is the drop-in boundary for `implementation="hip"` of tokamax.ragged_dot.  Every entry point
+ * takes plain device pointers, sizes and a HIP stream; none of them allocates, frees, synchronises
+ * or touches any stream other than the one passed in, so they can be bound from ctypes, cgo-style
+ * FFIs or an XLA FFI handler alike.  Return value: 0 on success, a TKX_ERR_* code otherwise
+ * (tkx_last_error() then holds a thread-local message).  TKX_ERR_UNSUPPORTED is the C-side twin of
+ * the reference's `NotImplementedError`: the caller may fall through to another implementation.
+ *
+ * Reference interfaces replaced (paths relative to the openxla/tokamax tree):
+ *   tkx_ragged_dot_schedule     tokamax/_src/ops/ragged_dot/pallas_mosaic_gpu_common.py:87-151
+ *                               (GroupInfo.create_aligned) + the offsets of :119-121
+ *   tkx_ragged_dot_fwd          tokamax/_src/ops/ragged_dot/base.py:291-360 (RaggedDot._fwd) as
+ *                               dispatched by pallas_mosaic_gpu.py:103-244, for
+ *                               DEFAULT_RAGGED_DOT_DIM_NUMS (base.py:40-44) and
+ *                               TRANS_RHS_RAGGED_DOT_DIM_NUMS (base.py:45-49, the dlhs of base.py:434-446)
+ *   tkx_ragged_dot_drhs         RAGGED_CONTRACTING_DOT_DIM_NUMS (base.py:50-54), the drhs of
+ *                               base.py:448-461; kernel counterpart pallas_mosaic_gpu_kernel_sm90.py:184-285
+ *   TkxConfig                   pallas_mosaic_gpu_common.py:45-73 (Config)
+ */
+#ifndef TKX_RAGGED_DOT_H_
+#define TKX_RAGGED_DOT_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* tkx_stream_t; /* a hipStream_t */
+
+enum TkxStatus {
+  TKX_OK = 0,
+  TKX_ERR_INVALID = 1,     /* bad argument (the reference raises ValueError) */
+  TKX_ERR_UNSUPPORTED = 2, /* valid but not implemented here (the reference raises NotImplementedError) */
+  TKX_ERR_RUNTIME = 3      /* HIP launch/runtime failure */
+};
+
+enum TkxDtype {
+  TKX_F32 = 0,
+  TKX_BF16 = 1,
+  TKX_F16 = 2,
+  TKX_F8E4M3FN = 3, /* OCP float8_e4m3fn */
+  TKX_I8 = 4
+};
+
+enum TkxMode {
+  TKX_MODE_DEFAULT = 0,  /* out[m,n] = lhs[m,k] . rhs[g,k,n]              (base.py:40-44) */
+  TKX_MODE_TRANS_RHS = 1 /* out[m,k] = lhs[m,n] . rhs[g,k,n]^T  (dlhs)    (base.py:45-49) */
+};
+
+enum TkxActivation { TKX_ACT_NONE = 0, TKX_ACT_RELU = 1, TKX_ACT_TANH = 2, TKX_ACT_SILU = 3, TKX_ACT_GELU_TANH = 4 };
+
+/* Tunables; the gfx950 counterpart of the reference's Config (pallas_mosaic_gpu_common.py:45-73).
+ * (block_m, block_n, block_k, waves_m, waves_n) must name a compiled kernel variant
+ * (see tkx_ragged_dot_num_variants / tkx_ragged_dot_variant). */
+typedef struct TkxConfig {
+  int32_t block_m;         /* rows of lhs per task (multiple of 8) */
+  int32_t block_n;         /* output columns per tile */
+  int32_t block_k;         /* contraction elements per LDS stage */
+  int32_t waves_m;         /* wavefronts along m in a workgroup */
+  int32_t waves_n;         /* wavefronts along n in a workgroup */
+  int32_t grid_tile_width; /* m-tasks that share an n-panel in launch order (L2 reuse) */
+  int32_t align_tile;      /* task starts are aligned down to this many rows (reference default 8) */
+  int32_t reserved;
+} TkxConfig;
+
+/* Library / ABI version (major*1000 + minor). */
+int32_t tkx_version(void);
+
+/* Thread-local message for the last non-zero status returned on this thread. */
+const char* tkx_last_error(void);
+
+/* Number of task slots the schedule uses for (m, G, block_m): cdiv(m, block_m) + G - 1
+ * (pallas_mosaic_gpu_kernel_sm90.py:54). */
+int64_t tkx_ragged_dot_tid_size(int64_t m, int64_t num_groups, int32_t block_m);
+
+/* Bytes of device workspace needed by schedule/fwd/drhs for these sizes (int32 arrays, 256-aligned). */
+int64_t tkx_ragged_dot_workspace_bytes(int64_t m, int64_t num_groups, int32_t block_m);
+
+/* Word offsets (int32 units) inside the workspace, for callers/tests that read the schedule back:
+ * which = 0 num_tasks (1 word), 1 total_rows (1 word), 2 group_offsets (G+1 words),
+ * 3..8 = group_id, block_start, actual_start, actual_end, start_within_block, actual_size
+ * (tid_size words each). Returns -1 for an unknown `which`. */
+int64_t tkx_ragged_dot_workspace_offset(int64_t m, int64_t num_groups, int32_t block_m, int32_t which);
+
+/* Part (1): group-offset prefix sum + tile schedule, one small kernel on `stream`.
+ * group_sizes: device int32[G] (negative entries count as 0). Fills `workspace`. */
+int32_t tkx_ragged_dot_schedule(const int32_t* group_sizes, int64_t num_groups, int64_t m, int32_t block_m,
+                                int32_t align_tile, void* workspace, tkx_stream_t stream);
+
+/* Parts (2),(3),(4-dlhs): grouped GEMM over the rows of each group.
+ *   mode DEFAULT:   lhs [m,k] row-major, rhs [G,k,n] row-major, out [m,n]
+ *   mode TRANS_RHS: lhs [m,n] row-major, rhs [G,k,n] row-major, out [m,k]  (rhs read transposed in-kernel)
+ * lhs_scale: f32[m] per-row scale or NULL; rhs_scale: f32[G,n] per-(group, column) scale or NULL
+ * (both applied to the f32 accumulator in the epilogue; DEFAULT mode only).
+ * Supported (lhs_dtype, rhs_dtype): (f32,f32) (bf16,bf16) (f16,f16) (f8e4m3fn,f8e4m3fn) (bf16,i8).
+ * out_dtype: f32, bf16 or f16. Rows >= sum(group_sizes) of `out` are set to zero.
+ * Runs the schedule kernel itself (workspace must hold tkx_ragged_dot_workspace_bytes bytes). */
+int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* group_sizes,
+                           const float* lhs_scale, const float* rhs_scale, void* out, void* workspace,
+                           int64_t m, int64_t k, int64_t n, int64_t num_groups, int32_t lhs_dtype,
+                           int32_t rhs_dtype, int32_t out_dtype, int32_t mode, int32_t activation,
+                           const TkxConfig* config, tkx_stream_t stream);
+
+/* Part (4-drhs): out[G,k,n] = lhs[rows_g, k]^T . dout[rows_g, n], zeros for empty groups.
+ * lhs [m,k], dout [m,n] row-major of `dtype` (f32/bf16/f16); out_dtype f32/bf16/f16.
+ * Deterministic: one workgroup owns each output tile, no atomics. block_m/block_n of `config`
+ * tile the (k, n) output; block_k rows of the ragged dimension are contracted per stage. */
+int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* group_sizes, void* out,
+                            void* workspace, int64_t m, int64_t k, int64_t n, int64_t num_groups,
+                            int32_t dtype, int32_t out_dtype, const TkxConfig* config, tkx_stream_t stream);
+
+/* Enumerates compiled kernel variants, for the autotuner's search space.
+ * kind: 0 = fwd/dlhs variants, 1 = drhs variants.  Returns the count; tkx_ragged_dot_variant fills
+ * `config` (tile + wave fields) and the dtype pair of variant `index`, returning 0, or TKX_ERR_INVALID. */
+int32_t tkx_ragged_dot_num_variants(int32_t kind);
+int32_t tkx_ragged_dot_variant(int32_t kind, int32_t index, TkxConfig* config, int32_t* lhs_dtype,
+                               int32_t* rhs_dtype, int32_t* mode);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TKX_RAGGED_DOT_H_ */

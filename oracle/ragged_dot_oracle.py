@@ -1,0 +1,295 @@
+"""CPU oracle for tokamax.ragged_dot -- TEST INFRASTRUCTURE ONLY.
+
+This file restates, in NumPy, the algorithm of the reference's
+`implementation="xla"` ragged dot and of its GPU tile scheduler.  Nothing in the
+shipped package imports it: only `tests/`, `__graft_entry__.smoke()` and the
+`cpu_baseline` leg of `bench.py` do, and only as the checker / the timed CPU
+baseline.
+
+The arithmetic of the reference's XLA path lives in un-vendored third-party
+packages (`jax>=0.11.0`: `jax.lax.ragged_dot_general`; `qwix>=0.1.2`:
+`dequantize`), which are not installed here, and the reference's own tests hold
+no stored floating-point outputs (they compare against JAX live).  Each function
+below therefore cites the reference call site it follows, and says what pins it:
+
+  function                     follows (reference file:line)                      pinned by
+  ---------------------------  -------------------------------------------------  ------------------------------------
+  group_offsets                pallas_mosaic_gpu_common.py:119-121                closed form (np.cumsum), brute force
+  group_info_create_aligned    pallas_mosaic_gpu_common.py:87-151                 the 4 known-answer tests of
+                                                                                  pallas_mosaic_gpu_common_test.py:27-84
+  ragged_dot (3 dim-number     base.py:291-360 (+ :40-54 dim numbers); jax doc    brute-force loops on tiny inputs; G=1
+    sets)                      of lax.ragged_dot_general                          -> plain GEMM; equal groups -> batched
+                                                                                  GEMM (bench.py:43-49); all rows in
+                                                                                  group 0 (bench.py:35-39); autograd of
+                                                                                  the forward for dlhs/drhs
+  dequantize                   quantization.py:80-83;                             the in-repo restatement
+                               ..._sm100_fp8_quant_test.py:229-232                q.astype(f32)*repeat(scale, tile)
+  round_to_bf16 / e4m3fn       base.py:342-354 (.astype(out_dtype))               torch's bf16 / float8_e4m3fn casts
+                                                                                  (library routine), exhaustive for fp8
+  generate_group_sizes         base.py:171-196                                    invariants of base_test.py:45-51
+                                                                                  (len == G, sum == m) + literal restatement
+
+Status of "parity unpinned": `qwix.quantize` (absmax calibration / rounding) is
+NOT restated -- quantised inputs are generated directly as (qvalue, scale) pairs.
+Everything else above has a pin listed.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+# Dimension-number sets of the reference (base.py:40-54), named by what they compute.
+DEFAULT = "default"  # lhs[m,k] . rhs[g,k,n] -> [m,n]        (base.py:40-44)
+TRANS_RHS = "trans_rhs"  # lhs[m,n'] . rhs[g,k',n'] -> [m,k']   (base.py:45-49)  (dlhs)
+RAGGED_CONTRACTING = "ragged_contracting"  # lhs[m,k] , rhs[m,n] -> [g,k,n]  (base.py:50-54)  (drhs)
+
+
+# ----------------------------------------------------------------------------
+# Integer part: offsets and tile schedule (bit-exact contract)
+# ----------------------------------------------------------------------------
+def group_offsets(group_sizes) -> np.ndarray:
+  """Exclusive prefix sum of clamped group sizes, length G+1.
+
+  Follows pallas_mosaic_gpu_common.py:119-121: sizes are clamped at 0, cast to
+  int32, `cumulative_sum(include_initial=True)`.
+  """
+  gs = np.maximum(np.asarray(group_sizes).astype(np.int64), 0).astype(np.int32)
+  out = np.zeros(gs.shape[0] + 1, np.int32)
+  np.cumsum(gs, out=out[1:])
+  return out
+
+
+def _cdiv(a, b):
+  return -(-a // b)
+
+
+def group_info_create_aligned(group_sizes, tile: int, tid_size: int, align_tile: int = 8):
+  """Tile schedule; literal restatement of `GroupInfo.create_aligned`.
+
+  Follows pallas_mosaic_gpu_common.py:119-151 line by line.  Returns a dict of six
+  int32 arrays of length `tid_size`: group_id, block_start, actual_start,
+  actual_end, start_within_block, actual_size -- plus `num_tasks` (the number of
+  tasks that belong to some non-empty group = group_start_tasks[-1]).
+  """
+  gs = np.asarray(group_sizes)
+  gs = np.maximum(np.zeros_like(gs), gs).astype(np.int32)  # :119-120
+  G = gs.shape[0]
+  group_starts = np.zeros(G + 1, np.int32)  # :121
+  np.cumsum(gs, out=group_starts[1:])
+  group_starts_aligned = (group_starts[:-1] // align_tile) * align_tile  # :122
+  group_ends = group_starts[:-1] + gs  # :124
+  group_num_blocks = np.where(gs == 0, 0, _cdiv(group_ends - group_starts_aligned, tile))  # :125-127
+  group_start_tasks = np.zeros(G + 1, np.int32)  # :128-130
+  np.cumsum(group_num_blocks, out=group_start_tasks[1:])
+  group_end_tasks = group_start_tasks[:-1] + group_num_blocks  # :132
+  task_idx = np.arange(tid_size, dtype=np.int32)  # :133
+  task_group_idx = np.searchsorted(group_end_tasks[:-1], task_idx, side="right").astype(np.int32)  # :136-138
+  task_block_idx = task_idx - group_start_tasks[task_group_idx]  # :139
+  task_starts = group_starts_aligned[task_group_idx] + tile * task_block_idx  # :140
+  task_valid_starts = np.maximum(task_starts, group_starts[task_group_idx])  # :141
+  task_valid_ends = np.minimum(task_starts + tile, group_ends[task_group_idx])  # :142
+  task_valid_size = np.maximum(0, task_valid_ends - task_valid_starts)  # :143
+  i32 = lambda x: np.asarray(x, np.int32)
+  return dict(
+      group_id=i32(task_group_idx),
+      block_start=i32(task_starts),
+      actual_start=i32(task_valid_starts),
+      actual_end=i32(task_valid_ends),
+      start_within_block=i32(task_valid_starts - task_starts),
+      actual_size=i32(task_valid_size),
+      num_tasks=int(group_start_tasks[-1]),
+  )
+
+
+def generate_group_sizes(*, m: int, num_groups: int, p=None, seed: int = 0):
+  """Restatement of base.py:171-196 (`generate_group_sizes`)."""
+  rng = np.random.default_rng(seed)
+  group_ids = rng.choice(num_groups, (m,), p=p, replace=True)
+  return tuple(map(int, np.bincount(group_ids, minlength=num_groups)))
+
+
+# ----------------------------------------------------------------------------
+# Dtype helpers
+# ----------------------------------------------------------------------------
+def round_to_bf16(x) -> np.ndarray:
+  """float32 -> nearest-even bfloat16, returned as float32 holding the bf16 value."""
+  x = np.ascontiguousarray(x, np.float32)
+  u = x.view(np.uint32).astype(np.uint64)
+  rounded = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+  out = rounded.astype(np.uint32).view(np.float32)
+  return np.where(np.isnan(x), x, out)
+
+
+def bf16_bits(x) -> np.ndarray:
+  """float32 -> uint16 bf16 bit patterns (round to nearest even)."""
+  return (round_to_bf16(x).view(np.uint32) >> 16).astype(np.uint16)
+
+
+def bf16_from_bits(bits) -> np.ndarray:
+  return (np.asarray(bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def _e4m3fn_table() -> np.ndarray:
+  """All 256 OCP float8_e4m3fn values (bias 7, no inf, 0x7f/0xff = NaN)."""
+  t = np.zeros(256, np.float32)
+  for b in range(256):
+    s = -1.0 if b & 0x80 else 1.0
+    e = (b >> 3) & 0xF
+    m = b & 0x7
+    if e == 0xF and m == 0x7:
+      v = np.nan
+    elif e == 0:
+      v = s * (m / 8.0) * 2.0 ** (-6)
+    else:
+      v = s * (1.0 + m / 8.0) * 2.0 ** (e - 7)
+    t[b] = v
+  return t
+
+
+E4M3FN_TABLE = _e4m3fn_table()
+
+
+def e4m3fn_decode(bits) -> np.ndarray:
+  return E4M3FN_TABLE[np.asarray(bits, np.uint8)]
+
+
+def e4m3fn_encode(x) -> np.ndarray:
+  """float32 -> uint8 e4m3fn bits, round to nearest even, saturating to +-448."""
+  x = np.asarray(x, np.float32)
+  pos = E4M3FN_TABLE[:0x7F].astype(np.float64)  # 0 .. 448, ascending
+  a = np.minimum(np.abs(x).astype(np.float64), 448.0)
+  hi = np.searchsorted(pos, a, side="left").clip(0, 0x7E)
+  lo = (hi - 1).clip(0, 0x7E)
+  dlo, dhi = np.abs(a - pos[lo]), np.abs(pos[hi] - a)
+  pick_hi = (dhi < dlo) | ((dhi == dlo) & (hi % 2 == 0))
+  code = np.where(pick_hi, hi, lo).astype(np.uint8)
+  code = np.where(np.signbit(x), code | 0x80, code).astype(np.uint8)
+  return np.where(np.isnan(x), np.uint8(0x7F), code)
+
+
+def dequantize(qvalue, scale) -> np.ndarray:
+  """`qvalue.astype(f32) * broadcast(scale)` with tile-repeat broadcasting.
+
+  Follows quantization.py:80-83 (`qwix.dequantize`, zero_point=None) as restated in
+  the reference's own test, pallas_mosaic_gpu_kernel_sm100_fp8_quant_test.py:229-232:
+  `scale.shape[i]` divides `qvalue.shape[i]`; each scale entry covers a tile of
+  `qvalue.shape[i] // scale.shape[i]` along axis i.
+  """
+  q = np.asarray(qvalue, np.float32)
+  s = np.asarray(scale, np.float32)
+  assert q.ndim == s.ndim, (q.shape, s.shape)
+  for ax in range(q.ndim):
+    assert q.shape[ax] % s.shape[ax] == 0, (q.shape, s.shape)
+    s = np.repeat(s, q.shape[ax] // s.shape[ax], axis=ax)
+  return q * s
+
+
+# ----------------------------------------------------------------------------
+# Floating-point part
+# ----------------------------------------------------------------------------
+def _round_out(x, out_dtype: str):
+  if out_dtype in ("f32", "float32"):
+    return x.astype(np.float32)
+  if out_dtype in ("f64", "float64"):
+    return x.astype(np.float64)
+  if out_dtype in ("bf16", "bfloat16"):
+    return round_to_bf16(x.astype(np.float32))
+  if out_dtype in ("f16", "float16"):
+    return x.astype(np.float16).astype(np.float32)
+  raise ValueError(out_dtype)
+
+
+def ragged_dot(lhs, rhs, group_sizes, mode: str = DEFAULT, *, acc_dtype=np.float32, out_dtype: str = "f32"):
+  """Per-group GEMM restating `RaggedDot._fwd` (base.py:291-360).
+
+  `lhs`/`rhs` are float arrays already holding the (de-quantised) input values.
+  Accumulates in `acc_dtype` (f32 = the reference's accumulator, base.py:345-346;
+  f64 = a tighter yardstick) and rounds once to `out_dtype` (base.py:354).  Rows
+  `>= sum(group_sizes)` are zero for DEFAULT/TRANS_RHS, as in the XLA path; groups
+  with no rows give a zero [k,n] block for RAGGED_CONTRACTING.
+  """
+  off = group_offsets(group_sizes)
+  G = len(off) - 1
+  lhs = np.asarray(lhs, acc_dtype)
+  rhs = np.asarray(rhs, acc_dtype)
+  if mode == DEFAULT:
+    m, k = lhs.shape
+    g2, k2, n = rhs.shape
+    assert g2 == G and k2 == k
+    out = np.zeros((m, n), acc_dtype)
+    for g in range(G):
+      s, e = int(off[g]), min(int(off[g + 1]), m)
+      if e > s:
+        out[s:e] = lhs[s:e] @ rhs[g]
+  elif mode == TRANS_RHS:
+    m, n = lhs.shape
+    g2, k, n2 = rhs.shape
+    assert g2 == G and n2 == n
+    out = np.zeros((m, k), acc_dtype)
+    for g in range(G):
+      s, e = int(off[g]), min(int(off[g + 1]), m)
+      if e > s:
+        out[s:e] = lhs[s:e] @ rhs[g].T
+  elif mode == RAGGED_CONTRACTING:
+    m, k = lhs.shape
+    m2, n = rhs.shape
+    assert m2 == m
+    out = np.zeros((G, k, n), acc_dtype)
+    for g in range(G):
+      s, e = int(off[g]), min(int(off[g + 1]), m)
+      if e > s:
+        out[g] = lhs[s:e].T @ rhs[s:e]
+  else:
+    raise ValueError(mode)
+  return _round_out(out, out_dtype)
+
+
+def ragged_dot_bruteforce(lhs, rhs, group_sizes, mode: str = DEFAULT):
+  """Element-by-element float64 loops (tiny inputs only): the pin for `ragged_dot`."""
+  lhs = np.asarray(lhs, np.float64)
+  rhs = np.asarray(rhs, np.float64)
+  gs = [max(int(x), 0) for x in group_sizes]
+  G = len(gs)
+  row_group = []
+  for g, s in enumerate(gs):
+    row_group += [g] * s
+  if mode == DEFAULT:
+    m, k = lhs.shape
+    n = rhs.shape[2]
+    out = np.zeros((m, n))
+    for i in range(min(m, len(row_group))):
+      for j in range(n):
+        acc = 0.0
+        for kk in range(k):
+          acc += lhs[i, kk] * rhs[row_group[i], kk, j]
+        out[i, j] = acc
+  elif mode == TRANS_RHS:
+    m, n = lhs.shape
+    k = rhs.shape[1]
+    out = np.zeros((m, k))
+    for i in range(min(m, len(row_group))):
+      for kk in range(k):
+        acc = 0.0
+        for j in range(n):
+          acc += lhs[i, j] * rhs[row_group[i], kk, j]
+        out[i, kk] = acc
+  elif mode == RAGGED_CONTRACTING:
+    m, k = lhs.shape
+    n = rhs.shape[1]
+    out = np.zeros((G, k, n))
+    for i in range(min(m, len(row_group))):
+      g = row_group[i]
+      for kk in range(k):
+        for j in range(n):
+          out[g, kk, j] += lhs[i, kk] * rhs[i, j]
+  else:
+    raise ValueError(mode)
+  return out
+
+
+def rel_l2(actual, expected) -> float:
+  """Relative L2 error ||a-e|| / ||e|| in float64 (the tolerance metric of the spec)."""
+  a = np.asarray(actual, np.float64).ravel()
+  e = np.asarray(expected, np.float64).ravel()
+  den = np.linalg.norm(e)
+  return float(np.linalg.norm(a - e) / (den if den > 0 else 1.0))

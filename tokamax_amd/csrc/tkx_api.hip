@@ -1,0 +1,280 @@
+// extern "C" entry points of libtkx_ragged_dot.so (declared in include/tkx_ragged_dot.h).
+#include <cstdarg>
+#include <cstdio>
+#include <mutex>
+#include <vector>
+
+#include "tkx_common.h"
+
+namespace tkx {
+
+static thread_local char g_err[512] = "";
+
+int32_t set_error(int32_t code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+namespace {
+
+struct Registry {
+  std::vector<Variant> all;
+  Registry() {
+    int n = 0;
+    const Variant* v;
+    v = variants_bf16(&n); all.insert(all.end(), v, v + n);
+    v = variants_f16(&n);  all.insert(all.end(), v, v + n);
+    v = variants_f32(&n);  all.insert(all.end(), v, v + n);
+    v = variants_f8(&n);   all.insert(all.end(), v, v + n);
+    v = variants_i8w(&n);  all.insert(all.end(), v, v + n);
+  }
+};
+
+const Registry& registry() {
+  static Registry r;
+  return r;
+}
+
+const Variant* find_variant(int mode, int a_dtype, int b_dtype, const TkxConfig& c) {
+  for (const Variant& v : registry().all)
+    if (v.mode == mode && v.a_dtype == a_dtype && v.b_dtype == b_dtype && v.block_m == c.block_m &&
+        v.block_n == c.block_n && v.block_k == c.block_k && v.waves_m == c.waves_m && v.waves_n == c.waves_n)
+      return &v;
+  return nullptr;
+}
+
+int dtype_bytes(int d) { return d == TKX_F32 ? 4 : (d == TKX_BF16 || d == TKX_F16) ? 2 : 1; }
+
+// Raises the dynamic-LDS limit of a kernel once per (device, kernel).
+int32_t prepare(const Variant* v) {
+  static std::mutex mu;
+  static std::vector<std::pair<int, const void*>> done;
+  int dev = 0;
+  TKX_HIP_CHECK(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  for (auto& d : done)
+    if (d.first == dev && d.second == v->fn) return TKX_OK;
+  TKX_HIP_CHECK(hipFuncSetAttribute(v->fn, hipFuncAttributeMaxDynamicSharedMemorySize, v->smem_bytes));
+  done.emplace_back(dev, v->fn);
+  return TKX_OK;
+}
+
+int32_t launch(const Variant* v, const GemmParams& p, int64_t grid, hipStream_t stream) {
+  int32_t st = prepare(v);
+  if (st != TKX_OK) return st;
+  if (grid <= 0 || grid > 0x7fffffffLL) return set_error(TKX_ERR_INVALID, "grid size %lld out of range", (long long)grid);
+  GemmParams params = p;
+  void* args[] = {&params};
+  const int threads = v->waves_m * v->waves_n * 64;
+  TKX_HIP_CHECK(hipLaunchKernel(v->fn, dim3((unsigned)grid), dim3(threads), args, (size_t)v->smem_bytes, stream));
+  return TKX_OK;
+}
+
+bool valid_out_dtype(int d) { return d == TKX_F32 || d == TKX_BF16 || d == TKX_F16; }
+
+}  // namespace
+}  // namespace tkx
+
+using namespace tkx;
+
+extern "C" {
+
+int32_t tkx_version(void) { return 1000; }
+
+const char* tkx_last_error(void) { return g_err; }
+
+int64_t tkx_ragged_dot_tid_size(int64_t m, int64_t num_groups, int32_t block_m) {
+  if (m < 0 || num_groups < 1 || block_m < 1) return -1;
+  return ws_layout(m, num_groups, block_m).tid_size;
+}
+
+int64_t tkx_ragged_dot_workspace_bytes(int64_t m, int64_t num_groups, int32_t block_m) {
+  if (m < 0 || num_groups < 1 || block_m < 1) return -1;
+  return ws_layout(m, num_groups, block_m).words * 4;
+}
+
+int64_t tkx_ragged_dot_workspace_offset(int64_t m, int64_t num_groups, int32_t block_m, int32_t which) {
+  if (m < 0 || num_groups < 1 || block_m < 1) return -1;
+  const WsLayout L = ws_layout(m, num_groups, block_m);
+  if (which == 0) return 0;
+  if (which == 1) return 1;
+  if (which == 2) return L.offsets;
+  if (which >= 3 && which <= 8) return L.task[which - 3];
+  return -1;
+}
+
+int32_t tkx_ragged_dot_schedule(const int32_t* group_sizes, int64_t num_groups, int64_t m, int32_t block_m,
+                                int32_t align_tile, void* workspace, tkx_stream_t stream) {
+  if (group_sizes == nullptr || workspace == nullptr) return set_error(TKX_ERR_INVALID, "null pointer argument");
+  if (num_groups < 1 || m < 0) return set_error(TKX_ERR_INVALID, "bad sizes m=%lld G=%lld", (long long)m, (long long)num_groups);
+  if (block_m < 1 || align_tile < 1) return set_error(TKX_ERR_INVALID, "block_m and align_tile must be positive");
+  const WsLayout L = ws_layout(m, num_groups, block_m);
+  return launch_schedule(group_sizes, num_groups, m, block_m, align_tile, static_cast<int32_t*>(workspace), L,
+                         static_cast<hipStream_t>(stream));
+}
+
+int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* group_sizes, const float* lhs_scale,
+                           const float* rhs_scale, void* out, void* workspace, int64_t m, int64_t k, int64_t n,
+                           int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype, int32_t mode,
+                           int32_t activation, const TkxConfig* config, tkx_stream_t stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (!lhs || !rhs || !group_sizes || !out || !workspace || !config)
+    return set_error(TKX_ERR_INVALID, "null pointer argument");
+  if (m < 1 || k < 1 || n < 1 || num_groups < 1)
+    return set_error(TKX_ERR_INVALID, "bad sizes m=%lld k=%lld n=%lld G=%lld", (long long)m, (long long)k,
+                     (long long)n, (long long)num_groups);
+  if (mode != TKX_MODE_DEFAULT && mode != TKX_MODE_TRANS_RHS) return set_error(TKX_ERR_INVALID, "bad mode %d", mode);
+  if (!valid_out_dtype(out_dtype)) return set_error(TKX_ERR_UNSUPPORTED, "out dtype %d not supported", out_dtype);
+  if (activation < TKX_ACT_NONE || activation > TKX_ACT_GELU_TANH)
+    return set_error(TKX_ERR_INVALID, "bad activation %d", activation);
+  if (m > 0x7fffffffLL / 2 || k > 0x7fffffffLL / 2 || n > 0x7fffffffLL / 2)
+    return set_error(TKX_ERR_UNSUPPORTED, "dimension too large");
+  const TkxConfig& c = *config;
+  if (c.block_m < 8 || c.block_m % 8 != 0) return set_error(TKX_ERR_INVALID, "block_m must be a positive multiple of 8");
+  if (c.grid_tile_width < 1 || c.align_tile < 1) return set_error(TKX_ERR_INVALID, "grid_tile_width/align_tile must be >= 1");
+  const bool dlhs = mode == TKX_MODE_TRANS_RHS;
+  if (dlhs && (lhs_scale || rhs_scale)) return set_error(TKX_ERR_UNSUPPORTED, "scales are not supported with TRANS_RHS");
+  const Variant* v = find_variant(dlhs ? kDlhs : kFwd, lhs_dtype, rhs_dtype, c);
+  if (v == nullptr)
+    return set_error(TKX_ERR_UNSUPPORTED, "no kernel variant for mode=%d dtypes=(%d,%d) tile=%dx%dx%d waves=%dx%d", mode,
+                     lhs_dtype, rhs_dtype, c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n);
+  // In C terms: rows = m; cols = n (fwd) or k (dlhs); contraction = k (fwd) or n (dlhs).
+  const int64_t cols = dlhs ? k : n, contraction = dlhs ? n : k;
+  const int lb = dtype_bytes(lhs_dtype), rb = dtype_bytes(rhs_dtype), ob = dtype_bytes(out_dtype);
+  // 16-byte vector accesses: every row of every operand must start 16-byte aligned and the tile
+  // loaders move whole 16-byte chunks along the contiguous axis.
+  if (contraction % c.block_k != 0)
+    return set_error(TKX_ERR_UNSUPPORTED, "contraction size %lld is not a multiple of block_k=%d", (long long)contraction, c.block_k);
+  if ((k * lb) % 16 != 0 && !dlhs) return set_error(TKX_ERR_UNSUPPORTED, "k*sizeof(lhs) must be a multiple of 16");
+  if ((n * rb) % 16 != 0 || (dlhs && (n * lb) % 16 != 0)) return set_error(TKX_ERR_UNSUPPORTED, "n*sizeof(elem) must be a multiple of 16");
+  if ((cols * ob) % 16 != 0 || cols % 8 != 0) return set_error(TKX_ERR_UNSUPPORTED, "output row size must be a multiple of 8 elements");
+  if (((uintptr_t)lhs | (uintptr_t)rhs | (uintptr_t)out | (uintptr_t)workspace) % 16 != 0 ||
+      (rhs_scale && (uintptr_t)rhs_scale % 16 != 0))
+    return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
+
+  const WsLayout L = ws_layout(m, num_groups, c.block_m);
+  int32_t st = launch_schedule(group_sizes, num_groups, m, c.block_m, c.align_tile, static_cast<int32_t*>(workspace), L, stream);
+  if (st != TKX_OK) return st;
+
+  GemmParams p = {};
+  p.A = lhs;
+  p.B = rhs;
+  p.C = out;
+  p.a_scale = lhs_scale;
+  p.b_scale = rhs_scale;
+  p.ws = static_cast<const int32_t*>(workspace);
+  p.lda = dlhs ? n : k;
+  p.ldb = n;
+  p.ldc = cols;
+  p.b_group_stride = k * n;
+  p.c_group_stride = 0;
+  p.m_ext = (int32_t)m;
+  p.n_ext = (int32_t)cols;
+  p.k_ext = (int32_t)contraction;
+  p.num_groups = (int32_t)num_groups;
+  p.n_tiles = (int32_t)((cols + c.block_n - 1) / c.block_n);
+  p.m_tiles = 0;
+  const int64_t slots = ((int64_t)L.tid_size * p.n_tiles + 7) / 8 * 8;
+  p.real_slots = (int32_t)slots;
+  p.grid_tile_width = c.grid_tile_width;
+  p.out_dtype = out_dtype;
+  p.activation = activation;
+  p.ws_offsets = (int32_t)L.offsets;
+  p.ws_gid = (int32_t)L.task[0];
+  p.ws_bstart = (int32_t)L.task[1];
+  p.ws_astart = (int32_t)L.task[2];
+  p.ws_aend = (int32_t)L.task[3];
+  if (slots > 0x7fffff00LL) return set_error(TKX_ERR_UNSUPPORTED, "too many tiles");
+  // Extra workgroups zero the rows past sum(group_sizes); they exit at once when there are none.
+  int64_t zero_wgs = (m * cols * ob + (64 << 10) - 1) / (64 << 10);
+  if (zero_wgs > 256) zero_wgs = 256;
+  if (zero_wgs < 1) zero_wgs = 1;
+  return launch(v, p, slots + zero_wgs, stream);
+}
+
+int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* group_sizes, void* out, void* workspace,
+                            int64_t m, int64_t k, int64_t n, int64_t num_groups, int32_t dtype, int32_t out_dtype,
+                            const TkxConfig* config, tkx_stream_t stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (!lhs || !dout || !group_sizes || !out || !workspace || !config)
+    return set_error(TKX_ERR_INVALID, "null pointer argument");
+  if (m < 1 || k < 1 || n < 1 || num_groups < 1)
+    return set_error(TKX_ERR_INVALID, "bad sizes m=%lld k=%lld n=%lld G=%lld", (long long)m, (long long)k,
+                     (long long)n, (long long)num_groups);
+  if (!valid_out_dtype(out_dtype)) return set_error(TKX_ERR_UNSUPPORTED, "out dtype %d not supported", out_dtype);
+  if (m > 0x7fffffffLL / 2 || k > 0x7fffffffLL / 2 || n > 0x7fffffffLL / 2)
+    return set_error(TKX_ERR_UNSUPPORTED, "dimension too large");
+  const TkxConfig& c = *config;
+  if (c.align_tile < 1) return set_error(TKX_ERR_INVALID, "align_tile must be >= 1");
+  const Variant* v = find_variant(kDrhs, dtype, dtype, c);
+  if (v == nullptr)
+    return set_error(TKX_ERR_UNSUPPORTED, "no drhs kernel variant for dtype=%d tile=%dx%dx%d waves=%dx%d", dtype,
+                     c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n);
+  const int eb = dtype_bytes(dtype), ob = dtype_bytes(out_dtype);
+  if ((k * eb) % 16 != 0 || (n * eb) % 16 != 0 || (n * ob) % 16 != 0 || n % 8 != 0)
+    return set_error(TKX_ERR_UNSUPPORTED, "k and n row sizes must be multiples of 16 bytes (n of 8 elements)");
+  if (((uintptr_t)lhs | (uintptr_t)dout | (uintptr_t)out | (uintptr_t)workspace) % 16 != 0)
+    return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
+
+  // Only the group offsets are needed; block_m of the schedule is irrelevant here, use a fixed one
+  // so the workspace size depends on (m, G) alone.
+  const int32_t sched_bm = 128;
+  const WsLayout L = ws_layout(m, num_groups, sched_bm);
+  int32_t st = launch_schedule(group_sizes, num_groups, m, sched_bm, c.align_tile, static_cast<int32_t*>(workspace), L, stream);
+  if (st != TKX_OK) return st;
+
+  GemmParams p = {};
+  p.A = lhs;
+  p.B = dout;
+  p.C = out;
+  p.ws = static_cast<const int32_t*>(workspace);
+  p.lda = k;
+  p.ldb = n;
+  p.ldc = n;
+  p.c_group_stride = k * n;
+  p.m_ext = (int32_t)k;
+  p.n_ext = (int32_t)n;
+  p.k_ext = (int32_t)m;
+  p.num_groups = (int32_t)num_groups;
+  p.n_tiles = (int32_t)((n + c.block_n - 1) / c.block_n);
+  p.m_tiles = (int32_t)((k + c.block_m - 1) / c.block_m);
+  p.grid_tile_width = 1;
+  p.out_dtype = out_dtype;
+  p.activation = TKX_ACT_NONE;
+  p.ws_offsets = (int32_t)L.offsets;
+  return launch(v, p, (int64_t)num_groups * p.m_tiles * p.n_tiles, stream);
+}
+
+int32_t tkx_ragged_dot_num_variants(int32_t kind) {
+  int32_t n = 0;
+  for (const Variant& v : registry().all) n += ((v.mode == kDrhs) == (kind == 1));
+  return n;
+}
+
+int32_t tkx_ragged_dot_variant(int32_t kind, int32_t index, TkxConfig* config, int32_t* lhs_dtype, int32_t* rhs_dtype,
+                               int32_t* mode) {
+  if (!config || !lhs_dtype || !rhs_dtype || !mode) return set_error(TKX_ERR_INVALID, "null pointer argument");
+  int32_t i = 0;
+  for (const Variant& v : registry().all) {
+    if ((v.mode == kDrhs) != (kind == 1)) continue;
+    if (i++ != index) continue;
+    config->block_m = v.block_m;
+    config->block_n = v.block_n;
+    config->block_k = v.block_k;
+    config->waves_m = v.waves_m;
+    config->waves_n = v.waves_n;
+    config->grid_tile_width = 1;
+    config->align_tile = 8;
+    config->reserved = 0;
+    *lhs_dtype = v.a_dtype;
+    *rhs_dtype = v.b_dtype;
+    *mode = v.mode;
+    return TKX_OK;
+  }
+  return set_error(TKX_ERR_INVALID, "variant index %d out of range", index);
+}
+
+}  // extern "C"

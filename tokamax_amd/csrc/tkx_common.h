@@ -1,0 +1,92 @@
+// Shared declarations of the gfx950 ragged-dot library (host + device).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tkx_ragged_dot.h"
+
+namespace tkx {
+
+// ---- workspace layout (int32 words) -----------------------------------------------------------
+// [0] num_tasks  [1] total_rows  [kWsHeader ..) group_offsets[G+1]  then six task arrays of
+// tid_size words each (group_id, block_start, actual_start, actual_end, start_within_block,
+// actual_size); every array starts on a 64-word boundary.
+constexpr int64_t kWsHeader = 64;
+
+struct WsLayout {
+  int64_t offsets;   // word offset of group_offsets
+  int64_t task[6];   // word offsets of the six task arrays
+  int64_t words;     // total words
+  int32_t tid_size;
+};
+
+inline int64_t round_up64(int64_t x) { return (x + 63) / 64 * 64; }
+
+inline WsLayout ws_layout(int64_t m, int64_t G, int32_t block_m) {
+  WsLayout L;
+  L.tid_size = (int32_t)((m + block_m - 1) / block_m + G - 1);
+  if (L.tid_size < 1) L.tid_size = 1;
+  int64_t w = kWsHeader;
+  L.offsets = w;
+  w += round_up64(G + 1);
+  for (int i = 0; i < 6; ++i) {
+    L.task[i] = w;
+    w += round_up64(L.tid_size);
+  }
+  L.words = w;
+  return L;
+}
+
+// ---- error reporting ----------------------------------------------------------------------------
+int32_t set_error(int32_t code, const char* fmt, ...);
+
+#define TKX_HIP_CHECK(expr)                                                                      \
+  do {                                                                                           \
+    hipError_t _e = (expr);                                                                      \
+    if (_e != hipSuccess)                                                                        \
+      return ::tkx::set_error(TKX_ERR_RUNTIME, "%s failed: %s", #expr, hipGetErrorString(_e));   \
+  } while (0)
+
+// ---- schedule -------------------------------------------------------------------------------------
+int32_t launch_schedule(const int32_t* group_sizes, int64_t G, int64_t m, int32_t block_m, int32_t align_tile,
+                        int32_t* ws, const WsLayout& L, hipStream_t stream);
+
+// ---- grouped GEMM -----------------------------------------------------------------------------
+enum KernelMode { kFwd = 0, kDlhs = 1, kDrhs = 2 };
+
+struct GemmParams {
+  const void* A;
+  const void* B;
+  void* C;
+  const float* a_scale;  // per A row, or null
+  const float* b_scale;  // per (group, column), or null
+  const int32_t* ws;
+  int64_t lda, ldb, ldc;            // leading dimensions, elements
+  int64_t b_group_stride;           // elements between consecutive groups of B (fwd/dlhs)
+  int64_t c_group_stride;           // elements between consecutive groups of C (drhs)
+  int32_t m_ext, n_ext, k_ext;      // extents of the C rows, C columns and the contraction
+  int32_t num_groups;
+  int32_t n_tiles, m_tiles;         // tiles along C columns; along C rows (drhs only)
+  int32_t real_slots;               // fwd/dlhs: workgroups that may own a task tile (multiple of 8)
+  int32_t grid_tile_width;
+  int32_t out_dtype, activation;
+  int32_t ws_offsets, ws_gid, ws_bstart, ws_astart, ws_aend;  // word offsets into ws
+};
+
+struct Variant {
+  int32_t mode;  // KernelMode
+  int32_t a_dtype, b_dtype;
+  int32_t block_m, block_n, block_k, waves_m, waves_n;
+  int32_t smem_bytes;
+  const void* fn;  // __global__ void (*)(GemmParams)
+};
+
+// Each dtype family registers its variants from its own translation unit.
+const Variant* variants_bf16(int* count);
+const Variant* variants_f16(int* count);
+const Variant* variants_f32(int* count);
+const Variant* variants_f8(int* count);
+const Variant* variants_i8w(int* count);
+
+}  // namespace tkx

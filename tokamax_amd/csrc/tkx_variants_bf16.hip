@@ -1,0 +1,29 @@
+// bf16 x bf16 kernel variants (forward, dlhs, drhs).
+#include "tkx_gemm.hip.h"
+
+namespace tkx {
+#define FWD_DLHS(BM, BN, BK, WM, WN) \
+  TKX_VARIANT(kFwd, kEBF16, kEBF16, BM, BN, BK, WM, WN), TKX_VARIANT(kDlhs, kEBF16, kEBF16, BM, BN, BK, WM, WN)
+
+static const Variant kVariants[] = {
+    FWD_DLHS(256, 256, 64, 2, 2),
+    FWD_DLHS(256, 256, 64, 2, 4),
+    FWD_DLHS(128, 256, 64, 2, 2),
+    FWD_DLHS(128, 256, 64, 2, 4),
+    FWD_DLHS(128, 128, 64, 2, 2),
+    FWD_DLHS(64, 256, 64, 2, 2),
+    FWD_DLHS(64, 128, 64, 2, 2),
+    FWD_DLHS(32, 256, 64, 1, 4),
+    FWD_DLHS(32, 128, 64, 1, 4),
+    TKX_VARIANT(kDrhs, kEBF16, kEBF16, 256, 256, 64, 2, 2),
+    TKX_VARIANT(kDrhs, kEBF16, kEBF16, 256, 256, 64, 2, 4),
+    TKX_VARIANT(kDrhs, kEBF16, kEBF16, 128, 256, 64, 2, 2),
+    TKX_VARIANT(kDrhs, kEBF16, kEBF16, 128, 128, 64, 2, 2),
+    TKX_VARIANT(kDrhs, kEBF16, kEBF16, 64, 128, 64, 2, 2),
+};
+
+const Variant* variants_bf16(int* count) {
+  *count = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
+  return kVariants;
+}
+}  // namespace tkx

@@ -1,0 +1,155 @@
+"""Thin adapters from torch device tensors to the C ABI (pointers + sizes + stream).
+
+PyTorch is used for device memory and streams only; all arithmetic happens in the HIP library.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import dataclasses
+
+import torch
+
+from tokamax_amd import _lib
+
+_DTYPE_CODE = {
+    torch.float32: _lib.TKX_F32,
+    torch.bfloat16: _lib.TKX_BF16,
+    torch.float16: _lib.TKX_F16,
+    torch.float8_e4m3fn: _lib.TKX_F8E4M3FN,
+    torch.int8: _lib.TKX_I8,
+}
+
+SCHEDULE_FIELDS = ("group_id", "block_start", "actual_start", "actual_end", "start_within_block", "actual_size")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+  try:
+    return _DTYPE_CODE[dtype]
+  except KeyError:
+    raise NotImplementedError(f"dtype {dtype} is not supported by the hip implementation") from None
+
+
+@dataclasses.dataclass(frozen=True)
+class KernelConfig:
+  """Launch parameters handed to the C ABI (see TkxConfig in include/tkx_ragged_dot.h)."""
+
+  block_m: int
+  block_n: int
+  block_k: int
+  waves_m: int
+  waves_n: int
+  grid_tile_width: int = 1
+  align_tile: int = 8
+
+  def to_c(self) -> _lib.TkxConfig:
+    return _lib.TkxConfig(self.block_m, self.block_n, self.block_k, self.waves_m, self.waves_n,
+                          self.grid_tile_width, self.align_tile, 0)
+
+
+def _require_cuda(*tensors):
+  for t in tensors:
+    if t is not None and not t.is_cuda:
+      raise NotImplementedError("the hip implementation needs tensors on an AMD GPU (got a CPU tensor)")
+
+
+def _ptr(t):
+  return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream(device) -> ctypes.c_void_p:
+  return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _group_sizes_i32(group_sizes: torch.Tensor) -> torch.Tensor:
+  if group_sizes.dtype != torch.int32:
+    group_sizes = group_sizes.to(torch.int32)  # uint32 / int64 inputs are legal in the reference
+  return group_sizes.contiguous()
+
+
+def workspace(m: int, num_groups: int, block_m: int, device) -> torch.Tensor:
+  nbytes = _lib.load().tkx_ragged_dot_workspace_bytes(m, num_groups, block_m)
+  if nbytes < 0:
+    raise ValueError(f"bad sizes m={m} G={num_groups} block_m={block_m}")
+  return torch.empty(nbytes // 4, dtype=torch.int32, device=device)
+
+
+def schedule(group_sizes: torch.Tensor, m: int, block_m: int, align_tile: int = 8):
+  """Runs the on-device scheduler; returns (dict of the six task arrays + group_offsets, num_tasks)."""
+  _require_cuda(group_sizes)
+  lib = _lib.load()
+  gs = _group_sizes_i32(group_sizes)
+  G = gs.numel()
+  ws = workspace(m, G, block_m, gs.device)
+  _lib.check(lib.tkx_ragged_dot_schedule(_ptr(gs), G, m, block_m, align_tile, _ptr(ws), _stream(gs.device)))
+  tid_size = lib.tkx_ragged_dot_tid_size(m, G, block_m)
+  out = {}
+  for i, name in enumerate(SCHEDULE_FIELDS):
+    off = lib.tkx_ragged_dot_workspace_offset(m, G, block_m, 3 + i)
+    out[name] = ws[off:off + tid_size]
+  off = lib.tkx_ragged_dot_workspace_offset(m, G, block_m, 2)
+  out["group_offsets"] = ws[off:off + G + 1]
+  out["num_tasks"] = ws[0:1]
+  out["total_rows"] = ws[1:2]
+  return out
+
+
+def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: torch.dtype, trans_rhs: bool = False,
+                   lhs_scale=None, rhs_scale=None, activation: str | None = None) -> torch.Tensor:
+  """out[m,n] = lhs[m,k] . rhs[g,k,n]   (trans_rhs: out[m,k] = lhs[m,n] . rhs[g,k,n]^T)."""
+  _require_cuda(lhs, rhs, group_sizes, lhs_scale, rhs_scale)
+  lib = _lib.load()
+  if lhs.dim() != 2 or rhs.dim() != 3:
+    raise ValueError(f"expected lhs [m,k] and rhs [g,k,n], got {tuple(lhs.shape)} and {tuple(rhs.shape)}")
+  lhs, rhs = lhs.contiguous(), rhs.contiguous()
+  gs = _group_sizes_i32(group_sizes)
+  G, k, n = rhs.shape
+  m = lhs.shape[0]
+  if gs.numel() != G:
+    raise ValueError(f"group_sizes has {gs.numel()} entries, rhs has {G} groups")
+  if lhs.shape[1] != (n if trans_rhs else k):
+    raise ValueError("contraction sizes of lhs and rhs differ")
+  if lhs_scale is not None:
+    lhs_scale = lhs_scale.to(torch.float32).contiguous().view(-1)
+    if lhs_scale.numel() != m:
+      raise NotImplementedError("lhs scale must be one f32 per row")
+  if rhs_scale is not None:
+    rhs_scale = rhs_scale.to(torch.float32).contiguous().view(-1)
+    if rhs_scale.numel() != G * n:
+      raise NotImplementedError("rhs scale must be one f32 per (group, column)")
+  out = torch.empty((m, k if trans_rhs else n), dtype=out_dtype, device=lhs.device)
+  ws = workspace(m, G, config.block_m, lhs.device)
+  cfg = config.to_c()
+  with torch.cuda.device(lhs.device):
+    st = lib.tkx_ragged_dot_fwd(
+        _ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(out), _ptr(ws), m, k, n, G,
+        dtype_code(lhs.dtype), dtype_code(rhs.dtype), dtype_code(out_dtype),
+        _lib.TKX_MODE_TRANS_RHS if trans_rhs else _lib.TKX_MODE_DEFAULT, _lib.ACTIVATIONS[activation],
+        ctypes.byref(cfg), _stream(lhs.device))
+  _lib.check(st)
+  return out
+
+
+def ragged_dot_drhs(lhs, dout, group_sizes, num_groups: int, *, config: KernelConfig,
+                    out_dtype: torch.dtype) -> torch.Tensor:
+  """out[g,k,n] = lhs[rows_g,k]^T . dout[rows_g,n]."""
+  _require_cuda(lhs, dout, group_sizes)
+  lib = _lib.load()
+  if lhs.dim() != 2 or dout.dim() != 2 or lhs.shape[0] != dout.shape[0]:
+    raise ValueError(f"expected lhs [m,k] and dout [m,n], got {tuple(lhs.shape)} and {tuple(dout.shape)}")
+  if lhs.dtype != dout.dtype:
+    raise NotImplementedError("lhs and dout must have the same dtype")
+  lhs, dout = lhs.contiguous(), dout.contiguous()
+  gs = _group_sizes_i32(group_sizes)
+  if gs.numel() != num_groups:
+    raise ValueError("group_sizes length differs from num_groups")
+  m, k = lhs.shape
+  n = dout.shape[1]
+  out = torch.empty((num_groups, k, n), dtype=out_dtype, device=lhs.device)
+  ws = workspace(m, num_groups, 128, lhs.device)
+  cfg = config.to_c()
+  with torch.cuda.device(lhs.device):
+    st = lib.tkx_ragged_dot_drhs(_ptr(lhs), _ptr(dout), _ptr(gs), _ptr(out), _ptr(ws), m, k, n, num_groups,
+                                 dtype_code(lhs.dtype), dtype_code(out_dtype), ctypes.byref(cfg), _stream(lhs.device))
+  _lib.check(st)
+  return out
