@@ -1,0 +1,222 @@
+"""Benchmark of the hip ragged dot on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+Prints ONE JSON line. A step is one pass of the hot path (scheduler kernel + grouped-GEMM kernel)
+over one seeded synthetic batch that is already resident in HBM. The headline workload is the
+Mixtral-8x7B-shaped prefill grouped GEMM (m=16384, k=4096, n=14336, G=8, bf16, top-2 router group
+sizes); `value` is its throughput in TFLOP/s with FLOPs = 2 * sum(group_sizes) * k * n. The other
+measured configurations (DeepSeek-V3 shape, int8-weight decode, fp8, bf16 VJP) are reported under
+"extras" with their own roofline figures. `cpu_baseline` times the CPU oracle (per-group f32 GEMM
+through NumPy's BLAS) on this box's host cores; it is a reported baseline, not the thing measured.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+# MI355X published peaks (dense).
+PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "f32": 157.3}
+PEAK_HBM_GBS = 8000.0
+
+
+def _time_steps(fn, steps, warmup, stream):
+  """Total and per-step device time (ms) of `steps` calls, HIP events on the launch stream."""
+  for _ in range(warmup):
+    fn()
+  stream.synchronize()
+  torch.cuda.synchronize()
+  starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+  ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+  t0 = time.perf_counter()
+  for i in range(steps):
+    starts[i].record(stream)
+    fn()
+    ends[i].record(stream)
+  stream.synchronize()
+  torch.cuda.synchronize()
+  wall_ms = (time.perf_counter() - t0) * 1e3
+  per = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+  total = starts[0].elapsed_time(ends[-1])
+  return total, per, wall_ms
+
+
+def _roofline(bound, flops, nbytes, ms, dtype_key):
+  if bound == "mfma":
+    achieved = flops / ms / 1e9
+    peak = PEAK_TFLOPS[dtype_key]
+    return dict(bound="mfma", achieved=round(achieved, 2), peak=peak, unit="TFLOP/s", frac=round(achieved / peak, 4),
+                traffic=None)
+  achieved = nbytes / ms / 1e6
+  return dict(bound="hbm", achieved=round(achieved, 2), peak=PEAK_HBM_GBS, unit="GB/s",
+              frac=round(achieved / PEAK_HBM_GBS, 4), traffic=None)
+
+
+def _cpu_baseline(w):
+  """Times the CPU oracle (per-group f32 GEMM, NumPy BLAS) on the full Mixtral workload."""
+  from oracle import ragged_dot_oracle as O
+
+  lhs = w.lhs.float().cpu().numpy()
+  rhs = w.rhs.float().cpu().numpy()
+  gs = w.group_sizes
+  O.ragged_dot(lhs[:256], rhs, np.minimum(gs, 32), acc_dtype=np.float32)  # warm the BLAS threads
+  times = []
+  t_all = time.perf_counter()
+  while len(times) < 3 or (time.perf_counter() - t_all < 10.0 and len(times) < 10):
+    t0 = time.perf_counter()
+    O.ragged_dot(lhs, rhs, gs, acc_dtype=np.float32, out_dtype="f32")
+    times.append(time.perf_counter() - t0)
+  try:
+    from threadpoolctl import threadpool_info
+
+    cores = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+  except Exception:  # pylint: disable=broad-exception-caught
+    cores = os.cpu_count() or 1
+  sec = statistics.median(times)
+  return dict(value=round(w.flops / sec / 1e12, 4), unit="TFLOP/s", cores=int(cores), kind="port",
+              sample=f"full {w.name} workload (m={w.m}, k={w.k}, n={w.n}, G={w.num_groups}), f32 NumPy-BLAS per-group "
+                     f"GEMM, median of {len(times)} runs, {sec:.3f} s each")
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=20)
+  ap.add_argument("--warmup", type=int, default=5)
+  ap.add_argument("--no-extras", action="store_true", help="headline workload only")
+  ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+  args = ap.parse_args()
+  if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+    print("bench.py: ragged_dot is a single-device operator and this build measures ONE GPU; "
+          "run with --gpus 1 (no multi-GPU figure exists).", file=sys.stderr)
+    sys.exit(2)
+  if not torch.cuda.is_available():
+    print("bench.py: no GPU visible; the hip implementation has no CPU fallback.", file=sys.stderr)
+    sys.exit(2)
+
+  import tokamax_amd
+  from tokamax_amd.ragged_dot import base, workloads
+
+  device = torch.device("cuda:0")
+  torch.cuda.set_device(device)
+  stream = torch.cuda.current_stream(device)
+  op = tokamax_amd.HipRaggedDot()
+
+  # ---- headline: Mixtral prefill ----------------------------------------------------------------
+  w = workloads.make("mixtral", device, seed=0)
+  gs = torch.tensor(w.group_sizes, device=device)
+  config = op.bind(w.lhs, w.rhs, group_sizes=gs).default_config
+  run = lambda: op(w.lhs, w.rhs, group_sizes=gs)
+  total_ms, per, wall_ms = _time_steps(run, args.steps, args.warmup, stream)
+  ms = total_ms / args.steps
+  result = {
+      "metric": "ragged_dot TFLOP/s (% MFMA peak) prefill; GB/s (% HBM peak) decode, 1 GPU",
+      "value": round(w.flops / ms / 1e9, 2),
+      "unit": "TFLOP/s",
+      "n_gpus": 1,
+      "steps": args.steps,
+      "warmup": args.warmup,
+      "ms_per_step": round(ms, 5),
+      "higher_is_better": True,
+      "scaling": "weak",
+      "vs_baseline": None,
+      "dtype": "bf16",
+      "data": "synthetic",
+      "config": {
+          "workload": "mixtral-8x7b prefill grouped GEMM: m=16384 (8192 tokens x top-2), k=4096, n=14336, G=8, "
+                      "bf16 in / f32 accumulate / bf16 out, group_sizes from a top-2 router over Gaussian logits",
+          "group_sizes": w.group_sizes.tolist(),
+          "seed": 0,
+          "kernel_config": {k: getattr(config, k) for k in ("block_m", "block_n", "block_k", "waves_m", "waves_n",
+                                                            "grid_tile_width")},
+      },
+      "roofline": _roofline("mfma", w.flops, w.algorithmic_bytes(), ms, "bf16"),
+      "ms_median_step": round(statistics.median(per), 5),
+      "ms_min_step": round(min(per), 5),
+      "wall_ms_per_step": round(wall_ms / args.steps, 5),
+      "pct_mfma_peak": round(100 * w.flops / ms / 1e9 / PEAK_TFLOPS["bf16"], 2),
+      "device": tokamax_amd.op.device_kind(),
+  }
+
+  if not args.no_cpu:
+    result["cpu_baseline"] = _cpu_baseline(w)
+  del w
+
+  # ---- the other measured configurations ----------------------------------------------------------
+  if not args.no_extras:
+    extras = {}
+    steps, warm = max(5, args.steps), max(2, args.warmup)
+
+    def measure(name, fn, flops, nbytes, bound, dtype_key, cfg):
+      t, p, _ = _time_steps(fn, steps, warm, stream)
+      m_ = t / steps
+      extras[name] = dict(ms_per_step=round(m_, 5), ms_min_step=round(min(p), 5), tflops=round(flops / m_ / 1e9, 2),
+                          gbs=round(nbytes / m_ / 1e6, 2), roofline=_roofline(bound, flops, nbytes, m_, dtype_key),
+                          kernel_config=None if cfg is None else
+                          [cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.grid_tile_width])
+
+    w = workloads.make("deepseek", device, seed=0)
+    gs = torch.tensor(w.group_sizes, device=device)
+    cfg = op.bind(w.lhs, w.rhs, group_sizes=gs).default_config
+    measure("deepseek_v3_prefill_bf16", lambda: op(w.lhs, w.rhs, group_sizes=gs), w.flops, w.algorithmic_bytes(),
+            "hbm", "bf16", cfg)
+    extras["deepseek_v3_prefill_bf16"]["pct_mfma_peak"] = round(
+        100 * extras["deepseek_v3_prefill_bf16"]["tflops"] / PEAK_TFLOPS["bf16"], 2)
+    del w
+
+    # decode: 4 rotating copies of the weights defeat the 256 MB last-level cache ("cold"); the same
+    # copy every step is the "warm" figure.
+    w = workloads.make("decode", device, seed=0)
+    gs = torch.tensor(w.group_sizes, device=device)
+    copies = [tokamax_amd.QArray(w.rhs.clone(), w.rhs_scale.clone()) for _ in range(4)]
+    cfg = op.bind(w.lhs, copies[0], group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    state = {"i": 0}
+
+    def decode_cold():
+      state["i"] = (state["i"] + 1) % len(copies)
+      return op(w.lhs, copies[state["i"]], group_sizes=gs, preferred_element_type=torch.bfloat16)
+
+    measure("decode_int8_cold", decode_cold, w.flops, w.algorithmic_bytes(), "hbm", "bf16", cfg)
+    measure("decode_int8_warm", lambda: op(w.lhs, copies[0], group_sizes=gs, preferred_element_type=torch.bfloat16),
+            w.flops, w.algorithmic_bytes(), "hbm", "bf16", cfg)
+    extras["decode_int8_cold"]["touched_experts"] = w.nonempty_groups
+    del w, copies
+
+    w = workloads.make("fp8", device, seed=0)
+    gs = torch.tensor(w.group_sizes, device=device)
+    ql, qr = tokamax_amd.QArray(w.lhs, w.lhs_scale), tokamax_amd.QArray(w.rhs, w.rhs_scale)
+    cfg = op.bind(ql, qr, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_prefill_fp8", lambda: op(ql, qr, group_sizes=gs, preferred_element_type=torch.bfloat16), w.flops,
+            w.algorithmic_bytes(), "mfma", "fp8", cfg)
+    del w, ql, qr
+
+    w = workloads.make("vjp", device, seed=0)
+    gs = torch.tensor(w.group_sizes, device=device)
+    cfg = op.bind(w.dout, w.rhs, group_sizes=gs, ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS).default_config
+    nb = (w.m * w.n + w.nonempty_groups * w.k * w.n + w.m * w.k) * 2
+    measure("vjp_dlhs_bf16", lambda: op(w.dout, w.rhs, group_sizes=gs, ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS),
+            w.flops, nb, "mfma", "bf16", cfg)
+    cfg = op.bind(w.lhs, w.dout, group_sizes=gs, ragged_dot_dimension_numbers=base.RAGGED_CONTRACTING_DOT_DIM_NUMS).default_config
+    nb = (w.m * w.k + w.m * w.n + w.num_groups * w.k * w.n) * 2
+    measure("vjp_drhs_bf16", lambda: op(w.lhs, w.dout, group_sizes=gs, ragged_dot_dimension_numbers=base.RAGGED_CONTRACTING_DOT_DIM_NUMS),
+            w.flops, nb, "mfma", "bf16", cfg)
+    del w
+    result["extras"] = extras
+
+  print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+  main()

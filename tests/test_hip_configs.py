@@ -1,0 +1,133 @@
+"""The five measured configurations at full size, checked through size-independent properties.
+
+The CPU oracle cannot run a 2 TFLOP problem in seconds, so at full size each configuration is checked
+by (a) the oracle on a seeded sample of rows of every non-empty group, (b) exact linearity under a
+power-of-two scaling of lhs, (c) zero rows past sum(group_sizes) and untouched-by-construction empty
+groups, (d) run-twice bit equality. The fp32 configuration is small enough to compare in full.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import tokamax_amd
+from oracle import ragged_dot_oracle as O
+from tokamax_amd.ragged_dot import base, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def _np(x):
+  return x.detach().float().cpu().numpy()
+
+
+def _sample_rows(gs, per_group, seed):
+  rng = np.random.default_rng(seed)
+  off = O.group_offsets(gs)
+  rows, groups = [], []
+  for g in range(len(gs)):
+    s, e = int(off[g]), int(off[g + 1])
+    if e > s:
+      # first and last row of the group (tile-straddling edges) plus random interior rows
+      pick = {s, e - 1} | set(rng.integers(s, e, per_group).tolist())
+      rows += sorted(pick)
+      groups += [g] * len(pick)
+  return np.array(rows), np.array(groups)
+
+
+def _check_rows(out, lhs_f, rhs_of_group, rows, groups, tol):
+  got = _np(out[torch.as_tensor(rows, device=out.device)])
+  want = np.stack([lhs_f[i].astype(np.float64) @ rhs_of_group(g).astype(np.float64) for i, g in enumerate(groups)])
+  err = O.rel_l2(got, want)
+  assert err <= tol, f"rel_l2 {err:.3e} > {tol}"
+
+
+def test_fp32_config_in_full(device):
+  w = workloads.make("fp32", device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  out = tokamax_amd.ragged_dot(w.lhs, w.rhs, gs, precision="highest")
+  assert out.dtype == torch.float32
+  want = O.ragged_dot(_np(w.lhs), _np(w.rhs), w.group_sizes, acc_dtype=np.float32, out_dtype="f32")
+  assert O.rel_l2(_np(out), want) <= 1e-5
+  want64 = O.ragged_dot(_np(w.lhs), _np(w.rhs), w.group_sizes, acc_dtype=np.float64, out_dtype="f64")
+  assert O.rel_l2(_np(out), want64) <= 1e-5
+
+
+@pytest.mark.parametrize("name,per_group", [("mixtral", 6), ("deepseek", 1)])
+def test_bf16_prefill_configs(name, per_group, device):
+  w = workloads.make(name, device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  out = tokamax_amd.ragged_dot(w.lhs, w.rhs, gs)
+  assert out.dtype == torch.bfloat16 and tuple(out.shape) == (w.m, w.n)
+  rows, groups = _sample_rows(w.group_sizes, per_group, 0)
+  lhs_f = _np(w.lhs[torch.as_tensor(rows, device=device)])
+  _check_rows(out, lhs_f, lambda g: _np(w.rhs[g]), rows, groups, 2e-3)
+  # linearity: scaling lhs by 2 scales every output by exactly 2 (power of two: no rounding anywhere)
+  out2 = tokamax_amd.ragged_dot(w.lhs * 2, w.rhs, gs)
+  assert torch.equal(out2, out * 2)
+  assert torch.equal(tokamax_amd.ragged_dot(w.lhs, w.rhs, gs), out)  # deterministic
+  if name == "deepseek":
+    assert (w.group_sizes == 0).sum() >= 8
+  del out2
+  # a shorter total leaves a zero tail
+  short = w.group_sizes.copy()
+  short[np.argmax(short)] -= 100
+  out3 = tokamax_amd.ragged_dot(w.lhs, w.rhs, torch.tensor(short, device=device))
+  assert torch.count_nonzero(out3[int(short.sum()):]) == 0
+
+
+def test_decode_int8_config(device):
+  w = workloads.make("decode", device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  rhs = tokamax_amd.QArray(w.rhs, w.rhs_scale)
+  out = tokamax_amd.ragged_dot(w.lhs, rhs, gs, preferred_element_type=torch.bfloat16)
+  want = O.ragged_dot(_np(w.lhs), O.dequantize(w.rhs.cpu().numpy(), _np(w.rhs_scale)), w.group_sizes,
+                      acc_dtype=np.float64, out_dtype="f64")
+  assert O.rel_l2(_np(out), want) <= 3e-2
+  assert O.rel_l2(_np(out), want) <= 3e-3  # in fact bf16-rounding accurate: int8 -> bf16 is exact
+  out32 = tokamax_amd.ragged_dot(w.lhs, rhs, gs, preferred_element_type=torch.float32)
+  assert O.rel_l2(_np(out32), want) <= 1e-5
+  assert (w.group_sizes == 0).any() and w.group_sizes.sum() == w.m
+
+
+def test_fp8_config(device):
+  w = workloads.make("fp8", device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  out = tokamax_amd.ragged_dot(tokamax_amd.QArray(w.lhs, w.lhs_scale), tokamax_amd.QArray(w.rhs, w.rhs_scale), gs,
+                               preferred_element_type=torch.bfloat16)
+  rows, groups = _sample_rows(w.group_sizes, 4, 1)
+  idx = torch.as_tensor(rows, device=device)
+  lhs_f = _np(w.lhs[idx]) * _np(w.lhs_scale[idx])
+  _check_rows(out, lhs_f, lambda g: _np(w.rhs[g]) * _np(w.rhs_scale[g]), rows, groups, 3e-3)
+  assert torch.equal(tokamax_amd.ragged_dot(tokamax_amd.QArray(w.lhs, w.lhs_scale), tokamax_amd.QArray(w.rhs, w.rhs_scale),
+                                            gs, preferred_element_type=torch.bfloat16), out)
+
+
+def test_vjp_config(device):
+  w = workloads.make("vjp", device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  dlhs = tokamax_amd.ragged_dot_general(w.dout, w.rhs, gs, base.TRANS_RHS_RAGGED_DOT_DIM_NUMS)
+  assert dlhs.dtype == torch.bfloat16 and tuple(dlhs.shape) == (w.m, w.k)
+  rows, groups = _sample_rows(w.group_sizes, 6, 2)
+  dout_f = _np(w.dout[torch.as_tensor(rows, device=device)])
+  _check_rows(dlhs, dout_f, lambda g: _np(w.rhs[g]).T, rows, groups, 2e-3)
+  drhs = tokamax_amd.ragged_dot_general(w.lhs, w.dout, gs, base.RAGGED_CONTRACTING_DOT_DIM_NUMS)
+  assert drhs.dtype == torch.bfloat16 and tuple(drhs.shape) == (w.num_groups, w.k, w.n)
+  # drhs[g][kk, :] = lhs[rows_g, kk]^T . dout[rows_g, :] for sampled (g, kk)
+  off = O.group_offsets(w.group_sizes)
+  rng = np.random.default_rng(3)
+  got, want = [], []
+  for g in range(w.num_groups):
+    s, e = int(off[g]), int(off[g + 1])
+    for kk in rng.integers(0, w.k, 3):
+      got.append(_np(drhs[g, int(kk)]))
+      want.append(_np(w.lhs[s:e, int(kk)]).astype(np.float64) @ _np(w.dout[s:e]).astype(np.float64))
+  assert O.rel_l2(np.stack(got), np.stack(want)) <= 2e-3
+  # the same gradients through autograd of the public API
+  lhs = w.lhs[:512].clone().requires_grad_(True)
+  rhs = w.rhs.clone().requires_grad_(True)
+  small = np.array([64] * 8, np.int32)
+  out = tokamax_amd.ragged_dot(lhs, rhs, torch.tensor(small, device=device))
+  out.backward(w.dout[:512])
+  want_dlhs = tokamax_amd.ragged_dot_general(w.dout[:512], w.rhs, torch.tensor(small, device=device), base.TRANS_RHS_RAGGED_DOT_DIM_NUMS)
+  assert torch.equal(lhs.grad, want_dlhs)

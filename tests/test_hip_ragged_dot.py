@@ -1,0 +1,358 @@
+"""GPU parity tests: the HIP path (through the C ABI) against the CPU oracle.
+
+Case list and tolerances follow the reference's shared suite
+(tokamax/_src/ops/ragged_dot/test_base.py:97-344) and scheduler test
+(pallas_mosaic_gpu_common_test.py:27-84). Bars: offsets and tile schedule bit-exact; relative L2
+error vs an f32/f64-accumulated reference <= 1e-5 (f32), <= 2e-3 (bf16/f16), <= 3e-2 (fp8, int8-dequant).
+"""
+
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import tokamax_amd
+from oracle import ragged_dot_oracle as O
+from tokamax_amd import _lib
+from tokamax_amd.ragged_dot import base, hip, hip_ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-3, torch.float16: 2e-3, "fp8": 3e-2, "int8": 3e-2}
+OP = hip.HipRaggedDot()
+
+
+def _np(x):
+  return x.detach().float().cpu().numpy()
+
+
+def _inputs(name, G, m, k, n, dtype, device, random_groups=False, std=0.1):
+  """Same recipe as test_base.py:108-150: rng seeded by the test name, N(0, std^2) cast to dtype."""
+  rng = np.random.default_rng(sum(name.encode()))
+  a = torch.tensor(rng.normal(0.0, std, (m, k)).astype(np.float32)).to(dtype).to(device)
+  b = torch.tensor(rng.normal(0.0, std, (G, k, n)).astype(np.float32)).to(dtype).to(device)
+  if random_groups:
+    gs = rng.integers(0, m // G, (G,)).astype(np.int32)
+  else:
+    gs = np.array([m // G] * G, np.int32)
+  return a, b, gs
+
+
+def _ref(a, b, gs, mode=O.DEFAULT):
+  return O.ragged_dot(_np(a), _np(b), gs, mode, acc_dtype=np.float64, out_dtype="f64")
+
+
+def _check(actual, expected, tol, rows=None):
+  a, e = _np(actual), np.asarray(expected)
+  if rows is not None:
+    a, e = a[:rows], e[:rows]
+  err = O.rel_l2(a, e)
+  assert err <= tol, f"rel_l2 {err:.3e} > {tol}"
+
+
+# ---- part (1): offsets and tile schedule, bit exact ----------------------------------------------
+with open(os.path.join(GOLDEN, "scheduler_kat.json")) as _f:
+  KAT = json.load(_f)
+
+
+@pytest.mark.parametrize("case", KAT, ids=[c["name"] for c in KAT])
+def test_schedule_known_answers(case, device):
+  gs = torch.tensor(case["group_sizes"], dtype=torch.int32, device=device)
+  m = sum(case["group_sizes"])
+  lib = _lib.load()
+  # the C ABI derives tid_size = cdiv(m, tile) + G - 1; compare on the common prefix
+  got = hip_ops.schedule(gs, m, case["tile"], case["align_tile"])
+  tid = min(case["tid_size"], got["group_id"].numel())
+  want = O.group_info_create_aligned(case["group_sizes"], case["tile"], got["group_id"].numel(), case["align_tile"])
+  for f in hip_ops.SCHEDULE_FIELDS:
+    np.testing.assert_array_equal(got[f].cpu().numpy()[:tid], np.array(case[f], np.int32)[:tid], err_msg=f)
+    np.testing.assert_array_equal(got[f].cpu().numpy(), want[f], err_msg=f)
+  assert lib.tkx_ragged_dot_tid_size(m, len(case["group_sizes"]), case["tile"]) == got["group_id"].numel()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_schedule_random_bit_exact(seed, device):
+  rng = np.random.default_rng(seed)
+  G = int(rng.choice([1, 2, 7, 8, 64, 128, 256, 300, 1000]))
+  gs = rng.integers(0, 400, G).astype(np.int32)
+  gs[rng.random(G) < 0.3] = 0
+  if seed % 2:
+    gs[rng.integers(0, G)] = -3  # negative sizes are clamped to zero
+  tile = int(rng.choice([8, 16, 32, 64, 128, 256]))
+  m = int(np.maximum(gs, 0).sum()) + int(rng.integers(0, 300))
+  got = hip_ops.schedule(torch.tensor(gs, device=device), max(m, 1), tile, 8)
+  want = O.group_info_create_aligned(gs, tile, got["group_id"].numel(), 8)
+  for f in hip_ops.SCHEDULE_FIELDS:
+    np.testing.assert_array_equal(got[f].cpu().numpy(), want[f], err_msg=f)
+  np.testing.assert_array_equal(got["group_offsets"].cpu().numpy(), O.group_offsets(gs))
+  assert int(got["num_tasks"].item()) == want["num_tasks"]
+  assert int(got["total_rows"].item()) == int(np.maximum(gs, 0).sum())
+
+
+@pytest.mark.parametrize("name,block_m", [("mixtral", 256), ("deepseek", 128), ("decode", 32)])
+def test_schedule_of_benchmark_group_sizes(name, block_m, device):
+  gs = {"mixtral": lambda: workloads.router_top2_group_sizes(8192, 8, 0),
+        "deepseek": lambda: workloads.zipf_group_sizes(65536, 256, 0),
+        "decode": lambda: workloads.decode_group_sizes(32, 8, 128, 0)}[name]()
+  m = int(gs.sum())
+  got = hip_ops.schedule(torch.tensor(gs, device=device), m, block_m, 8)
+  want = O.group_info_create_aligned(gs, block_m, got["group_id"].numel(), 8)
+  for f in hip_ops.SCHEDULE_FIELDS:
+    np.testing.assert_array_equal(got[f].cpu().numpy(), want[f], err_msg=f)
+  if name == "deepseek":
+    assert (gs == 0).sum() >= 10  # empty experts produce no task
+    assert set(got["group_id"].cpu().numpy()[:want["num_tasks"]].tolist()) == set(np.nonzero(gs)[0].tolist())
+
+
+# ---- the reference's shared suite -----------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_simple(dtype, device):
+  a, b, gs = _inputs("test_simple", 8, 1024, 128, 256, dtype, device)
+  # uint32 group sizes are legal input (test_base.py:137)
+  out = tokamax_amd.ragged_dot(a, b, torch.tensor(gs.astype(np.uint32), device=device), preferred_element_type=torch.float32)
+  assert out.dtype == torch.float32
+  _check(out, _ref(a, b, gs), TOL[dtype])
+
+
+def test_padded(device):
+  a, b, gs = _inputs("test_padded", 8, 1024, 128, 256, torch.bfloat16, device, random_groups=True)
+  out = tokamax_amd.ragged_dot(a, b, torch.tensor(gs, device=device), preferred_element_type=torch.float32)
+  count = int(gs.sum())
+  _check(out, _ref(a, b, gs), TOL[torch.bfloat16], rows=count)
+  assert torch.count_nonzero(out[count:]) == 0  # rows past sum(group_sizes) are zero, as in the XLA path
+
+
+def test_zero_group_sizes(device):
+  a, b, gs = _inputs("test_zero_group_sizes", 8, 1024, 128, 256, torch.bfloat16, device, random_groups=True)
+  for i in range(2 ** 8):  # every zero / non-zero pattern (test_base.py:172-185)
+    mask = np.unpackbits(np.uint8(i)).astype(bool)
+    gs_ = np.where(mask, gs, 0).astype(np.int32)
+    out = tokamax_amd.ragged_dot(a, b, torch.tensor(gs_, device=device), preferred_element_type=torch.float32)
+    count = int(gs_.sum())
+    err = O.rel_l2(_np(out), _ref(a, b, gs_))
+    assert err <= TOL[torch.bfloat16], (gs_.tolist(), err)
+    assert torch.count_nonzero(out[count:]) == 0, gs_.tolist()
+
+
+@pytest.mark.parametrize("out_type", [None, torch.bfloat16, torch.float32])
+def test_preferred_element_type(out_type, device):
+  a, b, gs = _inputs("test_preferred_element_type", 8, 1024, 128, 256, torch.bfloat16, device)
+  out = tokamax_amd.ragged_dot(a, b, torch.tensor(gs, device=device), preferred_element_type=out_type)
+  assert out.dtype == (out_type or torch.bfloat16)
+  want = O.ragged_dot(_np(a), _np(b), gs, acc_dtype=np.float32, out_dtype="bf16" if out.dtype == torch.bfloat16 else "f32")
+  _check(out, want, 2e-3)
+  if out.dtype == torch.bfloat16:
+    # one rounding of an f32 accumulator: at most 1 bf16 ulp from the oracle's rounding
+    ulp = np.abs(_np(out) - want) / np.maximum(np.abs(want), 1e-30)
+    assert float(np.quantile(ulp, 0.999)) <= 2 ** -7
+
+
+def test_group_sizes_wrapper(device):
+  a, b, gs = _inputs("test_group_sizes", 8, 1024, 128, 256, torch.bfloat16, device)
+  wrapped = base.GroupSizes(torch.tensor(gs, device=device), (1,) * 8)
+  out = tokamax_amd.ragged_dot(a, b, wrapped, preferred_element_type=torch.float32)
+  _check(out, _ref(a, b, gs), TOL[torch.bfloat16])
+
+
+@pytest.mark.parametrize("activation", [None, torch.relu, torch.tanh, torch.nn.functional.silu, torch.sigmoid])
+def test_activation(activation, device):
+  a, b, gs = _inputs("test_activation", 8, 512, 128, 256, torch.bfloat16, device, std=0.3)
+  out = tokamax_amd.ragged_dot(a, b, torch.tensor(gs, device=device), preferred_element_type=torch.float32, activation=activation)
+  want = torch.tensor(_ref(a, b, gs))
+  if activation is not None:
+    want = activation(want)
+  _check(out, want.numpy(), 2e-3)
+
+
+@pytest.mark.parametrize("m,k,n", list(itertools.product((1024, 128), (128, 64), (256, 128))))
+@pytest.mark.parametrize("activation", [None, torch.relu, torch.tanh])
+def test_vjp(m, k, n, activation, device):
+  """test_base.py:259-293: bf16 inputs, f32 reference, grads within atol=0.02, rtol=0.005."""
+  G = 8
+  a, b, gs = _inputs("test_vjp", G, m, k, n, torch.bfloat16, device)
+  gst = torch.tensor(gs, device=device)
+  a_ref = a.detach().float().cpu().double().requires_grad_(True)
+  b_ref = b.detach().float().cpu().double().requires_grad_(True)
+  off = O.group_offsets(gs)
+  ref_out = torch.cat([a_ref[int(off[g]):int(off[g + 1])] @ b_ref[g] for g in range(G)])
+  if activation is not None:
+    ref_out = activation(ref_out)
+  a_t = a.clone().requires_grad_(True)
+  b_t = b.clone().requires_grad_(True)
+  out = tokamax_amd.ragged_dot(a_t, b_t, gst, precision="BF16_BF16_F32", preferred_element_type=torch.float32,
+                               activation=activation)
+  np.testing.assert_allclose(_np(out), ref_out.detach().numpy(), atol=1e-5 + 2e-3 * float(ref_out.detach().abs().max()))
+  dout = (ref_out.detach() - ref_out.detach().mean()) / ref_out.detach().std()
+  dout = dout.to(torch.bfloat16).double()  # bottleneck the precision as the reference's test does
+  ref_out.backward(dout)
+  out.backward(dout.float().to(device))
+  assert a_t.grad.dtype == torch.bfloat16 and b_t.grad.dtype == torch.bfloat16
+  np.testing.assert_allclose(_np(a_t.grad), a_ref.grad.numpy(), atol=0.02, rtol=0.005)
+  np.testing.assert_allclose(_np(b_t.grad), b_ref.grad.numpy(), atol=0.02, rtol=0.005)
+  assert O.rel_l2(_np(a_t.grad), a_ref.grad.numpy()) <= 4e-3  # bf16 dout . bf16 rhs, rounded to bf16
+  assert O.rel_l2(_np(b_t.grad), b_ref.grad.numpy()) <= 4e-3
+
+
+@pytest.mark.parametrize("b_tile_shape,supported", [((1, 256, 1), True), ((1, 16, 1), False), ((1, 1, 16), False)])
+def test_quantized_int8_weights(b_tile_shape, supported, device):
+  """bf16 x int8: per-(group, column) scales run natively; other scale tilings are declined."""
+  G, m, k, n = 8, 512, 256, 512
+  a, _, gs = _inputs("test_quantized", G, m, k, n, torch.bfloat16, device, random_groups=True)
+  rng = np.random.default_rng(11)
+  q = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+  sshape = tuple(d // t for d, t in zip((G, k, n), b_tile_shape))
+  scale = torch.tensor((rng.uniform(0.5, 1.5, sshape) / 127 * 0.1).astype(np.float32), device=device)
+  rhs = tokamax_amd.QArray(q, scale)
+  gst = torch.tensor(gs, device=device)
+  if not supported:
+    with pytest.raises(NotImplementedError):
+      tokamax_amd.ragged_dot(a, rhs, gst)
+    return
+  for act in (None, torch.relu, torch.tanh):
+    out = tokamax_amd.ragged_dot(a, rhs, gst, activation=act, preferred_element_type=torch.float32)
+    want = torch.tensor(O.ragged_dot(_np(a), O.dequantize(q.cpu().numpy(), _np(scale)), gs, acc_dtype=np.float64, out_dtype="f64"))
+    want = act(want) if act is not None else want
+    count = int(gs.sum())
+    _check(out, want.numpy(), TOL["int8"], rows=count)
+    np.testing.assert_allclose(_np(out)[:count], want.numpy()[:count], atol=0.01, rtol=0.005)  # test_base.py:240-242
+  with pytest.raises(NotImplementedError):
+    tokamax_amd.ragged_dot(a, tokamax_amd.AsQArray(q.to(torch.bfloat16), torch.int8), gst)
+
+
+def test_fp8_with_row_and_column_scales(device):
+  G, m, k, n = 8, 512, 256, 512
+  rng = np.random.default_rng(12)
+  x = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device)
+  w = torch.tensor(rng.normal(0, k ** -0.5, (G, k, n)).astype(np.float32), device=device)
+  xs, ws = x.abs().amax(1, keepdim=True) / 448, w.abs().amax(1, keepdim=True) / 448
+  xq, wq = (x / xs).to(torch.float8_e4m3fn), (w / ws).to(torch.float8_e4m3fn)
+  gs = np.array([33, 67, 50, 80, 70, 60, 90, 62], np.int32)
+  out = tokamax_amd.ragged_dot(tokamax_amd.QArray(xq, xs), tokamax_amd.QArray(wq, ws), torch.tensor(gs, device=device),
+                               preferred_element_type=torch.bfloat16)
+  assert out.dtype == torch.bfloat16
+  # against the same quantised values (kernel arithmetic) ...
+  want_q = O.ragged_dot(O.dequantize(O.e4m3fn_decode(xq.view(torch.uint8).cpu().numpy()), _np(xs)),
+                        O.dequantize(O.e4m3fn_decode(wq.view(torch.uint8).cpu().numpy()), _np(ws)), gs,
+                        acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want_q, 2e-3)
+  _check(out, want_q, TOL["fp8"])
+  # ... and, for scale, against the unquantised problem: two e4m3 operands (3 mantissa bits each)
+  # put about 2^-4.7 of relative noise on every product, which no kernel can remove
+  _check(out, O.ragged_dot(_np(x), _np(w), gs, acc_dtype=np.float64, out_dtype="f64"), 6e-2)
+
+
+@pytest.mark.parametrize("group_sizes", [(33, 67, 50, 80, 70, 60, 90, 62), (1, 7, 199, 1, 100, 50, 151, 3),
+                                         (0, 130, 0, 200, 0, 98, 84, 0)])
+@pytest.mark.parametrize("block_m", [32, 64, 128, 256])
+def test_straddling_groups(group_sizes, block_m, device):
+  """..._sm100_fp8_quant_test.py:313-331: tiles that straddle two groups; no write outside a task's rows."""
+  G, m, k, n = 8, 512, 128, 256
+  a, b, _ = _inputs("test_straddling", G, m, k, n, torch.bfloat16, device)
+  gs = np.array(group_sizes, np.int32)
+  table = hip._variant_table()[(0, _lib.TKX_BF16, _lib.TKX_BF16)]
+  bm, bn, bk, wm, wn = next(v for v in table if v[0] == block_m)
+  op = hip.HipRaggedDot(config=hip.Config(bm, bn, bk, wm, wn, grid_tile_width=2))
+  out = op(a, b, group_sizes=torch.tensor(gs, device=device), preferred_element_type=torch.float32)
+  _check(out, _ref(a, b, gs), TOL[torch.bfloat16])
+  again = op(a, b, group_sizes=torch.tensor(gs, device=device), preferred_element_type=torch.float32)
+  assert torch.equal(out, again)  # run-twice bit equality (..._fp8_quant_test.py:274-280)
+
+
+def test_golden_fixtures(device):
+  z = np.load(os.path.join(GOLDEN, "ragged_dot_small.npz"))
+  gs = torch.tensor(z["gs"], device=device)
+  bf = lambda x: torch.tensor(x).to(torch.bfloat16).to(device)
+  lhs, rhs, dout = bf(z["lhs"]), bf(z["rhs"]), bf(z["dout"])
+  f32 = torch.float32
+  _check(tokamax_amd.ragged_dot(lhs, rhs, gs, preferred_element_type=f32), z["fwd"], 1e-5)
+  _check(tokamax_amd.ragged_dot_general(dout, rhs, gs, base.TRANS_RHS_RAGGED_DOT_DIM_NUMS, preferred_element_type=f32), z["dlhs"], 1e-5)
+  _check(tokamax_amd.ragged_dot_general(lhs, dout, gs, base.RAGGED_CONTRACTING_DOT_DIM_NUMS, preferred_element_type=f32), z["drhs"], 1e-5)
+  q8 = tokamax_amd.QArray(torch.tensor(z["q8"], device=device), torch.tensor(z["q8_scale"], device=device))
+  _check(tokamax_amd.ragged_dot(lhs, q8, gs, preferred_element_type=f32), z["fwd_q8"], 1e-5)
+  x8 = tokamax_amd.QArray(torch.tensor(z["x8"], device=device).view(torch.float8_e4m3fn), torch.tensor(z["x8_scale"], device=device))
+  w8 = tokamax_amd.QArray(torch.tensor(z["w8"], device=device).view(torch.float8_e4m3fn), torch.tensor(z["w8_scale"], device=device))
+  _check(tokamax_amd.ragged_dot(x8, w8, gs, preferred_element_type=f32), z["fwd_f8"], 1e-4)
+
+
+def _variant_cases():
+  cases = []
+  for kind in (0, 1):
+    for v in _lib.variants(kind):
+      cases.append(pytest.param(v, id="mode{mode}-d{lhs_dtype}x{rhs_dtype}-{block_m}x{block_n}x{block_k}-w{waves_m}x{waves_n}".format(**v)))
+  return cases
+
+
+_TORCH_DTYPE = {_lib.TKX_F32: torch.float32, _lib.TKX_BF16: torch.bfloat16, _lib.TKX_F16: torch.float16,
+                _lib.TKX_F8E4M3FN: torch.float8_e4m3fn, _lib.TKX_I8: torch.int8}
+
+
+@pytest.mark.parametrize("v", _variant_cases())
+def test_every_kernel_variant_through_c_abi(v, device):
+  """Each compiled tile shape, called through the C ABI, on ragged groups with an empty one and a tail."""
+  rng = np.random.default_rng(v["block_m"] * 7 + v["block_n"] + v["mode"])
+  G, m, k, n = 6, 640, 256, 384
+  gs = np.array([100, 0, 257, 9, 130, 80], np.int32)  # sum 576 < m
+  gst = torch.tensor(gs, device=device)
+  cfg = hip_ops.KernelConfig(v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"], grid_tile_width=3)
+  lt, rt = _TORCH_DTYPE[v["lhs_dtype"]], _TORCH_DTYPE[v["rhs_dtype"]]
+  mk = lambda shape, std: torch.tensor(rng.normal(0, std, shape).astype(np.float32), device=device)
+  if v["mode"] == 2:
+    lhs, dout = mk((m, k), 1.0).to(lt), mk((m, n), 1.0).to(lt)
+    out = hip_ops.ragged_dot_drhs(lhs, dout, gst, G, config=cfg, out_dtype=torch.float32)
+    _check(out, _ref(lhs, dout, gs, O.RAGGED_CONTRACTING), TOL[lt])
+    return
+  lhs_scale = rhs_scale = None
+  if rt == torch.int8:
+    rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+    rhs_scale = mk((G, 1, n), 0.01).abs() + 1e-3
+    rhs_f = O.dequantize(rhs.cpu().numpy(), _np(rhs_scale))
+    lhs = mk((m, k), 1.0).to(lt)
+    lhs_f = _np(lhs)
+    tol = 1e-5
+  elif lt == torch.float8_e4m3fn:
+    lhs, rhs = mk((m, k), 1.0).to(lt), mk((G, k, n), 1.0).to(rt)
+    lhs_scale, rhs_scale = mk((m, 1), 0.1).abs() + 0.05, mk((G, 1, n), 0.1).abs() + 0.05
+    lhs_f, rhs_f = _np(lhs) * _np(lhs_scale), _np(rhs) * _np(rhs_scale)
+    tol = 1e-4
+  else:
+    trans = v["mode"] == 1
+    lhs, rhs = mk((m, n if trans else k), 1.0).to(lt), mk((G, k, n), k ** -0.5).to(rt)
+    lhs_f, rhs_f = _np(lhs), _np(rhs)
+    tol = TOL[lt] if lt == torch.float32 else 1e-5  # f32 output of exact bf16/f16 products
+  out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, trans_rhs=(v["mode"] == 1),
+                               lhs_scale=lhs_scale, rhs_scale=rhs_scale)
+  want = O.ragged_dot(lhs_f, rhs_f, gs, O.TRANS_RHS if v["mode"] == 1 else O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, tol)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+
+
+def test_unsupported_inputs_are_declined(device):
+  a = torch.zeros(64, 100, dtype=torch.bfloat16, device=device)  # k not a multiple of any block_k
+  b = torch.zeros(2, 100, 64, dtype=torch.bfloat16, device=device)
+  gs = torch.tensor([32, 32], dtype=torch.int32, device=device)
+  with pytest.raises(NotImplementedError):
+    tokamax_amd.ragged_dot(a, b, gs)
+  with pytest.raises(NotImplementedError):  # mixed dtypes have no kernel
+    tokamax_amd.ragged_dot(torch.zeros(64, 128, device=device), torch.zeros(2, 128, 64, dtype=torch.bfloat16, device=device), gs)
+  calls = []
+  fallback = lambda lhs, rhs, **kw: calls.append(1) or "fallback"
+  assert tokamax_amd.ragged_dot(a, b, gs, implementation=["hip", fallback]) == "fallback" and calls
+
+
+def test_autotune_on_device(device):
+  a, b, gs = _inputs("test_autotune", 8, 1024, 128, 256, torch.bfloat16, device)
+  ba = OP.bind(a, b, group_sizes=torch.tensor(gs, device=device))
+  configs = {c for c in ba.autotuning_configs if c.grid_tile_width in (1, 8)}
+  bad = hip.Config(block_m=8, block_n=8, block_k=8)  # names no compiled kernel: recorded, not raised
+  data = ba.autotune(configs | {bad}, cache_results=False)
+  assert isinstance(data[bad], NotImplementedError)
+  best = data.fastest_config
+  assert best in configs and data[best].median_evaluation_time_ms > 0
+  res = tokamax_amd.AutotuningResult(tokamax_amd.op.device_kind(), ((ba, data),))
+  with res:
+    assert ba.default_config == best
+  assert tokamax_amd.op.device_kind() == "AMD Instinct MI355X"

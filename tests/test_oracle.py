@@ -1,0 +1,201 @@
+"""Pins the CPU oracle before anything is compared against it (no GPU needed).
+
+Integer part: the literal known-answer vectors of the reference's own scheduler test
+(tests/golden/scheduler_kat.json, from pallas_mosaic_gpu_common_test.py:27-84) plus invariants.
+Floating-point part: the reference stores no outputs, so `ragged_dot` is pinned by what the
+mathematics fixes -- brute-force loops, special cases that reduce to a library GEMM, autograd of the
+forward for the two backward contractions -- each chosen so that a dropped term, a wrong index or a
+transposed operand fails.
+"""
+
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import ragged_dot_oracle as O
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+FIELDS = ("group_id", "block_start", "actual_start", "actual_end", "start_within_block", "actual_size")
+
+with open(os.path.join(GOLDEN, "scheduler_kat.json")) as _f:
+  KAT = json.load(_f)
+
+
+@pytest.mark.parametrize("case", KAT, ids=[c["name"] for c in KAT])
+@pytest.mark.parametrize("impl", ["numpy", "c"])
+def test_scheduler_known_answers(case, impl):
+  fn = O.group_info_create_aligned if impl == "numpy" else c_oracle.create_aligned
+  got = fn(np.array(case["group_sizes"], np.int32), case["tile"], case["tid_size"], case["align_tile"])
+  for f in FIELDS:
+    np.testing.assert_array_equal(got[f], np.array(case[f], np.int32), err_msg=f)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_scheduler_invariants_and_c_agrees(seed):
+  rng = np.random.default_rng(seed)
+  G = int(rng.integers(1, 40))
+  gs = rng.integers(0, 70, G).astype(np.int32)
+  gs[rng.random(G) < 0.3] = 0
+  if seed == 0:
+    gs[0] = -5  # negative sizes count as zero (pallas_mosaic_gpu_common.py:119)
+  tile = int(rng.choice([8, 16, 32, 64]))
+  total = int(np.maximum(gs, 0).sum())
+  m = total + int(rng.integers(0, 20))
+  tid = -(-m // tile) + G - 1
+  a = O.group_info_create_aligned(gs, tile, tid, 8)
+  b = c_oracle.create_aligned(gs, tile, tid, 8)
+  for f in FIELDS:
+    np.testing.assert_array_equal(a[f], b[f], err_msg=f)
+  assert a["num_tasks"] == b["num_tasks"] <= tid
+  nt = a["num_tasks"]
+  off = O.group_offsets(gs)
+  np.testing.assert_array_equal(off, c_oracle.group_offsets(gs))
+  np.testing.assert_array_equal(off, np.concatenate([[0], np.cumsum(np.maximum(gs, 0))]))
+  # store ranges of the real tasks partition [0, total) in order
+  assert int(a["actual_size"][:nt].sum()) == total
+  pos = 0
+  for t in range(nt):
+    assert a["actual_start"][t] == pos and a["actual_size"][t] > 0
+    pos = a["actual_end"][t]
+    assert a["block_start"][t] % 8 == 0
+    assert 0 <= a["start_within_block"][t] < 8
+    g = a["group_id"][t]
+    assert off[g] <= a["actual_start"][t] and a["actual_end"][t] <= off[g + 1]
+    assert a["actual_end"][t] <= a["block_start"][t] + tile
+  assert pos == total
+  assert np.all(np.diff(a["group_id"][:nt]) >= 0)  # tasks of a group are contiguous
+  assert np.all(a["actual_size"][nt:] == 0)
+
+
+def test_generate_group_sizes():
+  gs = O.generate_group_sizes(m=1024, num_groups=8)
+  assert len(gs) == 8 and sum(gs) == 1024  # base_test.py:45-51
+  assert gs == tuple(np.bincount(np.random.default_rng(0).choice(8, (1024,)), minlength=8))
+
+
+@pytest.mark.parametrize("mode", [O.DEFAULT, O.TRANS_RHS, O.RAGGED_CONTRACTING])
+def test_ragged_dot_vs_bruteforce(mode):
+  rng = np.random.default_rng(3)
+  G, m, k, n = 3, 13, 5, 7
+  gs = [4, 0, 6]  # 3 trailing rows belong to no group
+  lhs = rng.normal(size=(m, n if mode == O.TRANS_RHS else k))
+  rhs = rng.normal(size=(m, n)) if mode == O.RAGGED_CONTRACTING else rng.normal(size=(G, k, n))
+  want = O.ragged_dot_bruteforce(lhs, rhs, gs, mode)
+  got = O.ragged_dot(lhs, rhs, gs, mode, acc_dtype=np.float64, out_dtype="f64")
+  np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-12)
+  got32 = c_oracle.ragged_dot_f32(lhs, rhs, np.array(gs, np.int32), {O.DEFAULT: 0, O.TRANS_RHS: 1, O.RAGGED_CONTRACTING: 2}[mode])
+  np.testing.assert_allclose(got32, want, rtol=2e-5, atol=2e-5)
+  if mode != O.RAGGED_CONTRACTING:
+    assert np.all(got[10:] == 0)  # rows past sum(group_sizes) are zero
+  else:
+    assert np.all(got[1] == 0)  # empty group
+
+
+def test_special_cases_reduce_to_library_gemm():
+  rng = np.random.default_rng(4)
+  G, m, k, n = 4, 32, 16, 24
+  lhs, rhs = rng.normal(size=(m, k)), rng.normal(size=(G, k, n))
+  # one group -> plain GEMM
+  np.testing.assert_allclose(O.ragged_dot(lhs, rhs[:1], [m], acc_dtype=np.float64, out_dtype="f64"), lhs @ rhs[0], rtol=1e-12)
+  # all rows in group 0 (bench.py:35-39)
+  np.testing.assert_allclose(O.ragged_dot(lhs, rhs, [m, 0, 0, 0], acc_dtype=np.float64, out_dtype="f64"), lhs @ rhs[0], rtol=1e-12)
+  # even groups -> batched GEMM (bench.py:43-49)
+  want = np.einsum("gmk,gkn->gmn", lhs.reshape(G, m // G, k), rhs).reshape(m, n)
+  np.testing.assert_allclose(O.ragged_dot(lhs, rhs, [m // G] * G, acc_dtype=np.float64, out_dtype="f64"), want, rtol=1e-12)
+  # the group of each row matters: permuting the weights of two groups changes exactly their rows
+  swapped = rhs[[1, 0, 2, 3]]
+  a = O.ragged_dot(lhs, rhs, [8] * 4, acc_dtype=np.float64, out_dtype="f64")
+  b = O.ragged_dot(lhs, swapped, [8] * 4, acc_dtype=np.float64, out_dtype="f64")
+  np.testing.assert_allclose(a[:8], lhs[:8] @ rhs[0], rtol=1e-12)
+  np.testing.assert_allclose(b[:8], lhs[:8] @ rhs[1], rtol=1e-12)
+  np.testing.assert_array_equal(a[16:], b[16:])
+
+
+def test_backward_contractions_match_autograd_of_forward():
+  rng = np.random.default_rng(5)
+  G, m, k, n = 3, 20, 6, 9
+  gs = [7, 0, 9]
+  lhs = torch.tensor(rng.normal(size=(m, k)), requires_grad=True)
+  rhs = torch.tensor(rng.normal(size=(G, k, n)), requires_grad=True)
+  dout = rng.normal(size=(m, n))
+  off = O.group_offsets(gs)
+  out = torch.zeros(m, n, dtype=torch.float64)
+  pieces = []
+  for g in range(G):
+    s, e = int(off[g]), int(off[g + 1])
+    pieces.append(lhs[s:e] @ rhs[g])
+  out = torch.cat(pieces + [torch.zeros(m - int(off[-1]), n, dtype=torch.float64)])
+  out.backward(torch.tensor(dout))
+  np.testing.assert_allclose(O.ragged_dot(dout, rhs.detach().numpy(), gs, O.TRANS_RHS, acc_dtype=np.float64, out_dtype="f64"),
+                             lhs.grad.numpy(), rtol=1e-12, atol=1e-12)
+  np.testing.assert_allclose(
+      O.ragged_dot(lhs.detach().numpy(), dout, gs, O.RAGGED_CONTRACTING, acc_dtype=np.float64, out_dtype="f64"),
+      rhs.grad.numpy(), rtol=1e-12, atol=1e-12)
+
+
+def test_f32_accumulation_and_single_rounding():
+  rng = np.random.default_rng(6)
+  lhs = O.round_to_bf16(rng.normal(size=(16, 64)).astype(np.float32))
+  rhs = O.round_to_bf16(rng.normal(size=(2, 64, 8)).astype(np.float32))
+  f64 = O.ragged_dot(lhs, rhs, [9, 7], acc_dtype=np.float64, out_dtype="f64")
+  f32 = O.ragged_dot(lhs, rhs, [9, 7], acc_dtype=np.float32, out_dtype="f32")
+  assert f32.dtype == np.float32 and O.rel_l2(f32, f64) < 1e-6
+  bf = O.ragged_dot(lhs, rhs, [9, 7], acc_dtype=np.float32, out_dtype="bf16")
+  np.testing.assert_array_equal(bf, torch.tensor(f32).to(torch.bfloat16).float().numpy())
+
+
+def test_bf16_rounding_matches_torch():
+  rng = np.random.default_rng(7)
+  x = np.concatenate([rng.normal(size=4096).astype(np.float32) * 10.0 ** rng.integers(-20, 20, 4096),
+                      np.array([0.0, -0.0, 1.0, 65504.0, 3.3895314e38, 1.0000001, 1.00390625, 1.01171875], np.float32)])
+  want = torch.tensor(x).to(torch.bfloat16)
+  np.testing.assert_array_equal(O.round_to_bf16(x), want.float().numpy())
+  np.testing.assert_array_equal(O.bf16_bits(x), want.view(torch.int16).numpy().view(np.uint16))
+  np.testing.assert_array_equal(O.bf16_from_bits(O.bf16_bits(x)), want.float().numpy())
+
+
+def test_e4m3fn_matches_torch_exhaustively():
+  bits = np.arange(256, dtype=np.uint8)
+  want = torch.tensor(bits).view(torch.float8_e4m3fn).float().numpy()
+  got = O.e4m3fn_decode(bits)
+  np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+  np.testing.assert_array_equal(got[~np.isnan(want)], want[~np.isnan(want)])
+  rng = np.random.default_rng(8)
+  x = np.concatenate([rng.normal(size=20000).astype(np.float32) * 10.0 ** rng.integers(-4, 3, 20000),
+                      got[~np.isnan(got)], np.array([448.0, -448.0, 464.0, 0.0009765625, 0.0029296875], np.float32)])
+  x = x[np.abs(x) <= 464]  # torch saturates differently above the last rounding boundary; stay in range
+  enc = O.e4m3fn_encode(x)
+  tw = torch.tensor(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+  np.testing.assert_array_equal(O.e4m3fn_decode(enc), O.e4m3fn_decode(tw))
+
+
+def test_dequantize_is_tile_repeat():
+  rng = np.random.default_rng(9)
+  q = rng.integers(-127, 128, (2, 8, 6)).astype(np.int8)
+  s = rng.uniform(0.5, 1.5, (2, 2, 6)).astype(np.float32)
+  want = q.astype(np.float32) * np.repeat(s, 4, axis=1)  # ..._sm100_fp8_quant_test.py:229-232
+  np.testing.assert_array_equal(O.dequantize(q, s), want)
+  # scales constant along k commute with the contraction (the epilogue-scale identity)
+  lhs = rng.normal(size=(5, 8))
+  s1 = rng.uniform(0.5, 1.5, (2, 1, 6)).astype(np.float32)
+  a = O.ragged_dot(lhs, O.dequantize(q, s1), [3, 2], acc_dtype=np.float64, out_dtype="f64")
+  b = O.ragged_dot(lhs, q.astype(np.float64), [3, 2], acc_dtype=np.float64, out_dtype="f64")
+  b[:3] *= s1[0, 0]
+  b[3:] *= s1[1, 0]
+  np.testing.assert_allclose(a, b, rtol=2e-6)  # dequantize rounds q*s to f32
+
+
+def test_golden_fixtures_match_oracle():
+  z = np.load(os.path.join(GOLDEN, "ragged_dot_small.npz"))
+  gs = z["gs"]
+  f = lambda *a, **kw: O.ragged_dot(*a, acc_dtype=np.float64, out_dtype="f64", **kw)
+  np.testing.assert_allclose(f(z["lhs"], z["rhs"], gs), z["fwd"], rtol=1e-12, atol=1e-12)
+  np.testing.assert_allclose(f(z["dout"], z["rhs"], gs, mode=O.TRANS_RHS), z["dlhs"], rtol=1e-12, atol=1e-12)
+  np.testing.assert_allclose(f(z["lhs"], z["dout"], gs, mode=O.RAGGED_CONTRACTING), z["drhs"], rtol=1e-12, atol=1e-12)
+  np.testing.assert_allclose(f(z["lhs"], O.dequantize(z["q8"], z["q8_scale"]), gs), z["fwd_q8"], rtol=1e-12, atol=1e-12)
+  # the brute-force loops agree with the stored vectors too (small enough to run here)
+  np.testing.assert_allclose(O.ragged_dot_bruteforce(z["lhs"][:40], z["rhs"], [23, 0, 17, 0]), z["fwd"][:40], rtol=1e-10, atol=1e-10)

@@ -1,0 +1,31 @@
+"""MI355X-native `ragged_dot` behind the tokamax operator API.
+
+Public names follow tokamax/__init__.py:18-41 for this operator: `ragged_dot`,
+`ragged_dot_general`, `RaggedDotGroupSizes`, `Op`, `BoundArguments`, `autotune`,
+`AutotuningResult`, and the config options.
+"""
+
+from tokamax_amd import config
+from tokamax_amd.autotuning.api import AutotuningResult, autotune
+from tokamax_amd.op import AUTO, BoundArguments, NullConfig, Op
+from tokamax_amd.quantization import AsQArray, QArray
+from tokamax_amd.ragged_dot.api import IMPLEMENTATIONS as RAGGED_DOT_IMPLEMENTATIONS
+from tokamax_amd.ragged_dot.api import ragged_dot, ragged_dot_general
+from tokamax_amd.ragged_dot.base import (
+    DEFAULT_RAGGED_DOT_DIM_NUMS,
+    RAGGED_CONTRACTING_DOT_DIM_NUMS,
+    TRANS_RHS_RAGGED_DOT_DIM_NUMS,
+    GroupSizes as RaggedDotGroupSizes,
+    RaggedDotDimensionNumbers,
+    generate_group_sizes,
+)
+from tokamax_amd.ragged_dot.hip import Config as HipRaggedDotConfig
+from tokamax_amd.ragged_dot.hip import HipRaggedDot
+
+__all__ = [
+    "AUTO", "AsQArray", "AutotuningResult", "BoundArguments", "DEFAULT_RAGGED_DOT_DIM_NUMS", "HipRaggedDot",
+    "HipRaggedDotConfig", "NullConfig", "Op", "QArray", "RAGGED_CONTRACTING_DOT_DIM_NUMS",
+    "RAGGED_DOT_IMPLEMENTATIONS", "RaggedDotDimensionNumbers", "RaggedDotGroupSizes",
+    "TRANS_RHS_RAGGED_DOT_DIM_NUMS", "autotune", "config", "generate_group_sizes", "ragged_dot",
+    "ragged_dot_general",
+]

@@ -145,9 +145,9 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   const int64_t cols = dlhs ? k : n, contraction = dlhs ? n : k;
   const int lb = dtype_bytes(lhs_dtype), rb = dtype_bytes(rhs_dtype), ob = dtype_bytes(out_dtype);
   // 16-byte vector accesses: every row of every operand must start 16-byte aligned and the tile
-  // loaders move whole 16-byte chunks along the contiguous axis.
-  if (contraction % c.block_k != 0)
-    return set_error(TKX_ERR_UNSUPPORTED, "contraction size %lld is not a multiple of block_k=%d", (long long)contraction, c.block_k);
+  // loaders move whole 16-byte chunks along the contiguous axis. The contraction size itself need
+  // not be a multiple of block_k: the last k-step is zero-filled.
+  (void)contraction;
   if ((k * lb) % 16 != 0 && !dlhs) return set_error(TKX_ERR_UNSUPPORTED, "k*sizeof(lhs) must be a multiple of 16");
   if ((n * rb) % 16 != 0 || (dlhs && (n * lb) % 16 != 0)) return set_error(TKX_ERR_UNSUPPORTED, "n*sizeof(elem) must be a multiple of 16");
   if ((cols * ob) % 16 != 0 || cols % 8 != 0) return set_error(TKX_ERR_UNSUPPORTED, "output row size must be a multiple of 8 elements");

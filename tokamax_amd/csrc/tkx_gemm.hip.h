@@ -188,8 +188,9 @@ __device__ __forceinline__ typename Mma<EC>::Frag load_frag(const unsigned char*
 // ---- global -> register -> LDS staging ------------------------------------------------------
 // One operand tile of a k-step, moved in 16-byte chunks; chunk q of the tile belongs to thread
 // (q % THREADS). Out-of-range rows/columns are clamped to valid memory (their products are never
-// stored); out-of-range contraction rows (kDrhs) are zero-filled.
-template <int LAYOUT, int ES, int RC /* rows or cols of C covered */, int BK, int THREADS, bool MASK_K>
+// stored); contraction indices at or past `k_hi` are zero-filled, which only the last k-step of
+// a tile can need (a workgroup-uniform test keeps the other steps free of per-lane masking).
+template <int LAYOUT, int ES, int RC /* rows or cols of C covered */, int BK, int THREADS>
 struct TileStage {
   static constexpr int ESZ = elem_bytes(ES);
   static constexpr int ROW_BYTES = (LAYOUT == kKC) ? BK * ESZ : RC * ESZ;
@@ -204,9 +205,11 @@ struct TileStage {
 
   // base: operand pointer already offset to the group; ld in elements; rc0 = first row/col of the
   // tile; rc_ext = extent of that axis; kc0 = first contraction index of this k-step;
-  // [k_lo, k_hi) = valid contraction range (only used when MASK_K).
-  __device__ __forceinline__ void load(const unsigned char* base, int64_t ld, int rc0, int rc_ext, int kc0, int k_lo,
-                                       int k_hi, int tid) {
+  // k_hi = end of the valid contraction range.
+  __device__ __forceinline__ void load(const unsigned char* base, int64_t ld, int rc0, int rc_ext, int kc0, int k_hi,
+                                       int tid) {
+    const bool full = kc0 + BK <= k_hi;  // uniform across the workgroup
+    const i32x4 z = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int q = tid + i * THREADS;
@@ -215,21 +218,25 @@ struct TileStage {
       if constexpr (LAYOUT == kKC) {
         int row = rc0 + r;
         row = row < rc_ext ? row : rc_ext - 1;
-        const unsigned char* p = base + ((int64_t)row * ld + kc0) * ESZ + c * 16;
-        regs[i] = *reinterpret_cast<const i32x4*>(p);
+        const int kcol = kc0 + c * (16 / ESZ);
+        const unsigned char* p = base + ((int64_t)row * ld + kcol) * ESZ;
+        if (full) {
+          regs[i] = *reinterpret_cast<const i32x4*>(p);
+        } else {
+          regs[i] = z;
+          if (kcol < k_hi) regs[i] = *reinterpret_cast<const i32x4*>(p);
+        }
       } else {
         const int krow = kc0 + r;
         int colb = rc0 * ESZ + c * 16;
         const int lim = rc_ext * ESZ - 16;
         colb = colb < lim ? colb : lim;
-        if constexpr (MASK_K) {
-          const bool ok = krow >= k_lo && krow < k_hi;
-          const int kr = ok ? krow : k_lo;
-          i32x4 v = *reinterpret_cast<const i32x4*>(base + (int64_t)kr * ld * ESZ + colb);
-          const i32x4 z = {0, 0, 0, 0};
-          regs[i] = ok ? v : z;
+        const unsigned char* p = base + (int64_t)krow * ld * ESZ + colb;
+        if (full) {
+          regs[i] = *reinterpret_cast<const i32x4*>(p);
         } else {
-          regs[i] = *reinterpret_cast<const i32x4*>(base + (int64_t)krow * ld * ESZ + colb);
+          regs[i] = z;
+          if (krow < k_hi) regs[i] = *reinterpret_cast<const i32x4*>(p);
         }
       }
     }
@@ -289,8 +296,8 @@ struct GemmKernel {
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int TM = WTM / 32, TN = WTN / 32;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % KA == 0, "tile does not split into 32x32 atoms");
-  typedef TileStage<LA, EA, BM, BK, THREADS, MODE == kDrhs> StageA;
-  typedef TileStage<LB, EB, BN, BK, THREADS, MODE == kDrhs> StageB;
+  typedef TileStage<LA, EA, BM, BK, THREADS> StageA;
+  typedef TileStage<LB, EB, BN, BK, THREADS> StageB;
   static constexpr int STAGE_BYTES = StageA::BYTES + StageB::BYTES;
   static constexpr int SMEM_BYTES = 2 * STAGE_BYTES;
 
@@ -366,8 +373,8 @@ struct GemmKernel {
     StageA sa;
     StageB sb;
     if (nk > 0) {
-      sa.load(Ab, p.lda, row0, p.m_ext, kc_begin, kc_begin, kc_end, tid);
-      sb.load(Bb, p.ldb, col0, p.n_ext, kc_begin, kc_begin, kc_end, tid);
+      sa.load(Ab, p.lda, row0, p.m_ext, kc_begin, kc_end, tid);
+      sb.load(Bb, p.ldb, col0, p.n_ext, kc_begin, kc_end, tid);
       sa.store(smem, tid);
       sb.store(smem + StageA::BYTES, tid);
     }
@@ -379,8 +386,8 @@ struct GemmKernel {
       const bool more = kt + 1 < nk;
       if (more) {
         const int kc0 = kc_begin + (kt + 1) * BK;
-        sa.load(Ab, p.lda, row0, p.m_ext, kc0, kc_begin, kc_end, tid);
-        sb.load(Bb, p.ldb, col0, p.n_ext, kc0, kc_begin, kc_end, tid);
+        sa.load(Ab, p.lda, row0, p.m_ext, kc0, kc_end, tid);
+        sb.load(Bb, p.ldb, col0, p.n_ext, kc0, kc_end, tid);
       }
 #pragma unroll
       for (int kk = 0; kk < BK / KA; ++kk) {

@@ -1,0 +1,356 @@
+"""Base class for ops: bind -> pick a config -> run `_fwd`, with a custom VJP.
+
+Restates tokamax/_src/ops/op.py for torch tensors. Kept identical in behaviour:
+  * `Op.__call__` (op.py:196-307): bind, device check (`NotImplementedError("Not supported on ...")`,
+    :209-211), config selection through `BoundArguments.default_config`, `_fwd`, and the op's own
+    `vjp` for gradients (here via `torch.autograd.Function` instead of `jax.custom_vjp`).
+  * `BoundArguments.get_config` (op.py:477-516): `op.config` -> NullConfig shortcut -> overlay stack
+    (innermost first) -> shipped JSON cache (fastest config by median) -> autotune -> heuristics ->
+    `ValueError("No config found ...")`.
+  * `autotuning_configs = {heuristics_config} | op._get_autotuning_configs(ba)` (op.py:558-561).
+Not restated: the vmap capture and the HLO metadata payload, which only exist under JAX tracing.
+"""
+
+from __future__ import annotations
+
+import abc
+import collections
+import contextvars
+import dataclasses
+import inspect
+import json
+import logging
+from typing import Any, Callable, ClassVar, Mapping
+
+import torch
+
+from tokamax_amd import benchmarking
+from tokamax_amd import config as config_lib
+from tokamax_amd import serialization
+from tokamax_amd.autotuning import autotuner as autotuner_lib
+from tokamax_amd.autotuning import cache as autotuning_cache
+
+AutotuningData = autotuner_lib.AutotuningData
+DeviceKind = str
+logger = logging.getLogger("tokamax_amd")
+
+
+@dataclasses.dataclass(frozen=True)
+class NullConfig:
+  ...
+
+
+_NULL_CONFIG = NullConfig()
+
+
+class AUTO:
+  """Sentinel: autotune over `BoundArguments.autotuning_configs`."""
+
+
+# Names of GPUs whose marketing name the runtime may not report (it needs a PCI-id table that
+# is not always installed): fall back to the architecture.
+_ARCH_DEVICE_KINDS = {"gfx950": "AMD Instinct MI355X", "gfx942": "AMD Instinct MI300X", "gfx90a": "AMD Instinct MI250X"}
+
+
+def device_kind(device=None) -> DeviceKind:
+  """The key autotuning caches are filed under (the role of `jax.Device.device_kind`)."""
+  if not torch.cuda.is_available():
+    return "cpu"
+  props = torch.cuda.get_device_properties(device)
+  arch = getattr(props, "gcnArchName", "").split(":")[0]
+  if arch in _ARCH_DEVICE_KINDS:
+    return _ARCH_DEVICE_KINDS[arch]
+  return props.name
+
+
+def default_device() -> torch.device:
+  if torch.cuda.is_available():
+    return torch.device("cuda", torch.cuda.current_device())
+  return torch.device("cpu")
+
+
+@dataclasses.dataclass(frozen=True)
+class Op(abc.ABC):
+  """Base class for operations (see module docstring)."""
+
+  config_cls: ClassVar[type] = NullConfig
+  supports_symbolic_shapes: ClassVar[bool] = True
+
+  config: Any = None
+  _: dataclasses.KW_ONLY
+  # `vjp(residuals, out, dout, *args, **kwargs)` returns gradients for the positional arguments,
+  # as a tuple, or as a dict {"argname": gradient}.
+  vjp: Callable[..., Any] | None = None
+
+  def __call__(self, *args, return_residuals: bool = False, **kwargs):
+    ba = self.bind(*args, return_residuals=return_residuals, **kwargs)
+    for device in infer_devices(ba) or {default_device()}:
+      if not self.supported_on(device):
+        raise NotImplementedError(f"Not supported on {device_kind(device) if device.type == 'cuda' else device}.")
+    config = ba.default_config
+
+    tensors = [x for x in _leaves(dict(ba.arguments)) if isinstance(x, torch.Tensor)]
+    needs_grad = self.vjp is not None and torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+    if not needs_grad:
+      out, residuals = self._fwd(*ba.args, config=config, **ba.kwargs)
+      return (out, residuals) if return_residuals else out
+    return _call_with_vjp(self, ba, config, return_residuals)
+
+  def bind(self, *args, return_residuals: bool = False, **kwargs) -> "BoundArguments":
+    """Binds the op to the given arguments."""
+    ba = self._fwd_signature.bind(*args, return_residuals=return_residuals, **kwargs)
+    ba.apply_defaults()
+    return BoundArguments(self, ba.arguments)
+
+  def replace(self, **kwargs) -> "Op":
+    new_op = dataclasses.replace(self, **kwargs)
+    # Ops may install a default VJP in `__post_init__`; an explicit `vjp=None` must win.
+    if "vjp" in kwargs:
+      object.__setattr__(new_op, "vjp", kwargs["vjp"])
+    return new_op
+
+  def get_autotuning_cache(self, device_kind_: DeviceKind | None = None) -> dict:
+    self_no_vjp = self.replace(vjp=None)
+    if device_kind_ is None:
+      device_kind_ = device_kind()
+    if config_lib.ignore_autotuning_cache.value:
+      logger.warning("Ignoring autotuning cache for %s", self_no_vjp)
+      return {}
+    cache = _AUTOTUNING_CACHE.get(self_no_vjp)
+    if cache is None:
+      cache = autotuning_cache.AutotuningCache(self_no_vjp)
+      _AUTOTUNING_CACHE[self_no_vjp] = cache
+    return cache[device_kind_]
+
+  @abc.abstractmethod
+  def _fwd(self, *args, **kwargs):
+    ...
+
+  def _get_heuristics_config(self, ba: "BoundArguments"):
+    del ba
+    if type(self).config_cls is NullConfig:
+      return _NULL_CONFIG
+    raise NotImplementedError("`_get_heuristics_config` not implemented.")
+
+  def _get_autotuning_cache_key(self, ba: "BoundArguments"):
+    return CacheKey(tuple((k, serialization.abstractify(v)) for k, v in ba.arguments.items()))
+
+  def _get_autotuning_configs(self, ba: "BoundArguments") -> set:
+    del ba
+    return set()
+
+  @property
+  def signature(self) -> inspect.Signature:
+    if type(self).bind is not Op.bind:
+      return inspect.signature(self.bind)
+    return self._fwd_signature
+
+  @property
+  def _fwd_signature(self) -> inspect.Signature:
+    sig = inspect.signature(self._fwd)
+    params = dict(sig.parameters)
+    del params["config"]
+    return sig.replace(parameters=tuple(params.values()))
+
+  def supported_on(self, device: torch.device) -> bool:
+    del device
+    return True
+
+
+class CacheKey(tuple):
+  """Hashable (name, abstract value) pairs in signature order; JSON form = the cache-file key."""
+
+  def to_json(self) -> str:
+    return json.dumps({k: serialization.to_jsonable(v) for k, v in self}, separators=(",", ":"))
+
+  def __repr__(self):
+    return f"CacheKey({self.to_json()})"
+
+
+_AUTOTUNING_CACHE: dict = {}
+# Stack of {op: {device_kind: {key: AutotuningData}}} overlays pushed by `AutotuningResult`.
+AUTOTUNING_CACHE_OVERLAY_STACK: contextvars.ContextVar[tuple] = contextvars.ContextVar(
+    "AUTOTUNING_CACHE_OVERLAY_STACK", default=()
+)
+
+
+@dataclasses.dataclass(frozen=True)
+class BoundArguments:
+  """Bound arguments for an op's `__call__` method."""
+
+  op: Op
+  arguments: Mapping[str, Any]
+
+  def __post_init__(self):
+    object.__setattr__(self, "arguments", collections.OrderedDict(self.arguments))
+
+  def __hash__(self):
+    return hash((self.op.replace(vjp=None), self.autotuning_cache_key))
+
+  def __eq__(self, other):
+    return (isinstance(other, BoundArguments) and self.op.replace(vjp=None) == other.op.replace(vjp=None)
+            and self.autotuning_cache_key == other.autotuning_cache_key)
+
+  @property
+  def signature(self) -> inspect.Signature:
+    return self.op._fwd_signature  # pylint: disable=protected-access
+
+  @property
+  def _bound_args(self) -> inspect.BoundArguments:
+    return inspect.BoundArguments(self.signature, collections.OrderedDict(self.arguments))
+
+  @property
+  def args(self) -> tuple:
+    return self._bound_args.args
+
+  @property
+  def kwargs(self) -> dict:
+    return self._bound_args.kwargs
+
+  @property
+  def default_config(self):
+    """`op.config`, else cache, else autotune / heuristics / error by the cache-miss option."""
+    fallback = config_lib.autotuning_cache_miss_fallback.value
+    return self.get_config(
+        autotune_configs=AUTO if fallback == "autotune" else None,
+        allow_heuristics=fallback != "error",
+    )
+
+  def get_config(self, check_autotuning_cache: bool = True, autotune_configs=None,
+                 cache_autotuning_results: bool = True, allow_heuristics: bool = True):
+    if (config := self.op.config) is not None:
+      return config
+    if (heuristics_config := self.heuristics_config) is _NULL_CONFIG:
+      return heuristics_config
+    if check_autotuning_cache:
+      data = self.cached_autotuning_data
+      if data is not None and len(data):
+        return data.fastest_config
+    if autotune_configs is not None:
+      return self.autotune(autotune_configs, cache_results=cache_autotuning_results).fastest_config
+    if allow_heuristics:
+      return heuristics_config
+    raise ValueError(f"No config found for {self}.")
+
+  @property
+  def heuristics_config(self):
+    return self.op._get_heuristics_config(self)  # pylint: disable=protected-access
+
+  @property
+  def autotuning_cache_key(self):
+    return self.op._get_autotuning_cache_key(self)  # pylint: disable=protected-access
+
+  @property
+  def cached_autotuning_data(self) -> AutotuningData | None:
+    if config_lib.ignore_autotuning_cache.value:
+      return None
+    kind = infer_device_kind(self) or device_kind()
+    key = self.autotuning_cache_key
+    op_no_vjp = self.op.replace(vjp=None)
+    for overlay in reversed(AUTOTUNING_CACHE_OVERLAY_STACK.get()):
+      data = overlay.get(op_no_vjp, {}).get(kind, {}).get(key)
+      if data is not None:
+        return data
+    try:
+      return self.op.get_autotuning_cache(kind)[key]
+    except KeyError:
+      logger.info("Autotuning cache miss for %s on %s with key %s", self.op, kind, key)
+      return None
+
+  @property
+  def autotuning_configs(self) -> set:
+    return {self.heuristics_config} | self.op._get_autotuning_configs(self)  # pylint: disable=protected-access
+
+  def benchmark(self, iterations: int = 5) -> benchmarking.BenchmarkData:
+    args, kwargs = self.args, self.kwargs
+    return benchmarking.benchmark(lambda: self.op(*args, **kwargs), iterations=iterations)
+
+  def autotune(self, configs=AUTO, autotuner: autotuner_lib.Autotuner = autotuner_lib.Autotuner(),
+               cache_results: bool = True, timeout: float | None = None) -> AutotuningData:
+    if configs is AUTO:
+      configs = self.autotuning_configs
+    op_fn = lambda config: self.op.replace(config=config)
+    data = autotuner.autotune(op_fn, configs, *self.args, timeout=timeout, **self.kwargs)
+    if cache_results:
+      self.op.get_autotuning_cache()[self.autotuning_cache_key] = data
+    return data
+
+  def to_json_dict(self) -> dict:
+    """`{"op": ..., "arguments": ...}` with abstract arguments (the reference's BOUND_ARGS_ADAPTER form)."""
+    op = self.op.replace(vjp=None)
+    op_json = {"__class__": type(op).__name__}
+    for f in dataclasses.fields(op):
+      if f.name not in ("_", "vjp"):
+        op_json[f.name] = serialization.to_jsonable(getattr(op, f.name))
+    return dict(op=op_json, arguments=json.loads(self.autotuning_cache_key.to_json()))
+
+  def replace(self, **kwargs) -> "BoundArguments":
+    return dataclasses.replace(self, **kwargs)
+
+
+def _leaves(x):
+  if isinstance(x, dict):
+    for v in x.values():
+      yield from _leaves(v)
+  elif isinstance(x, (tuple, list)):
+    for v in x:
+      yield from _leaves(v)
+  elif dataclasses.is_dataclass(x) and not isinstance(x, type):
+    for f in dataclasses.fields(x):
+      yield from _leaves(getattr(x, f.name))
+  elif hasattr(x, "_leaves"):
+    yield from x._leaves()  # pylint: disable=protected-access
+  else:
+    yield x
+
+
+def infer_devices(ba: BoundArguments) -> set:
+  return {x.device for x in _leaves(dict(ba.arguments)) if isinstance(x, torch.Tensor)}
+
+
+def infer_device_kind(ba: BoundArguments) -> DeviceKind | None:
+  kinds = {device_kind(d) if d.type == "cuda" else "cpu" for d in infer_devices(ba)}
+  if not kinds:
+    return None
+  if len(kinds) == 1:
+    return kinds.pop()
+  raise ValueError(f"Multiple device kinds found: {kinds}")
+
+
+def _call_with_vjp(op: Op, ba: BoundArguments, config, return_residuals: bool):
+  """Runs `_fwd` under a torch.autograd.Function whose backward is `op.vjp` (op.py:276-307)."""
+  arguments = dict(ba.arguments)
+  names = [k for k, v in arguments.items() if isinstance(v, torch.Tensor) and v.is_floating_point()]
+  tensors = [arguments[k] for k in names]
+  pos_names = [
+      n for n, p in ba.signature.parameters.items()
+      if p.kind in (p.POSITIONAL_ONLY, p.POSITIONAL_OR_KEYWORD)
+  ]
+
+  class _Fn(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, *ts):
+      full = dict(arguments)
+      full.update(zip(names, ts))
+      bound = BoundArguments(op, full)
+      kwargs = dict(bound.kwargs)
+      kwargs["return_residuals"] = True
+      out, residuals = op._fwd(*bound.args, config=config, **kwargs)  # pylint: disable=protected-access
+      ctx.bound, ctx.out, ctx.residuals = bound, out, residuals
+      if return_residuals:
+        ctx.mark_non_differentiable(residuals)
+        return out, residuals
+      return out
+
+    @staticmethod
+    def backward(ctx, dout, *unused):
+      bound = ctx.bound
+      kwargs = dict(bound.kwargs)
+      kwargs.pop("return_residuals")
+      with torch.no_grad():
+        grads = op.vjp(ctx.residuals, ctx.out, dout, *bound.args, **kwargs)
+      by_name = dict(grads) if isinstance(grads, dict) else dict(zip(pos_names, grads))
+      return tuple(by_name.get(n) for n in names)
+
+  return _Fn.apply(*tensors)

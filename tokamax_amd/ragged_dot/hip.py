@@ -1,0 +1,278 @@
+"""Ragged dot on gfx950 (MI355X): `implementation="hip"`.
+
+Slots into the operator framework the way the reference's GPU backend does
+(tokamax/_src/ops/ragged_dot/pallas_mosaic_gpu.py:85-518): a `RaggedDot` subclass with its own
+`Config`, `_fwd`, heuristics, autotuning search space and `supported_on`; anything it cannot run
+raises `NotImplementedError` so that the dispatcher may try the next implementation. All three
+dimension-number sets run natively: the transposed-rhs case (dlhs) reads rhs in place instead
+of materialising `rhs.mT` as the reference does (pallas_mosaic_gpu.py:148-150).
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import functools
+from functools import partial
+from typing import ClassVar
+
+import torch
+
+from tokamax_amd import _lib
+from tokamax_amd import config as config_lib
+from tokamax_amd import op
+from tokamax_amd import precision as precision_lib
+from tokamax_amd.ragged_dot import base
+from tokamax_amd.ragged_dot import hip_ops
+
+QArray = base.QArray
+AsQArray = base.AsQArray
+GroupSizes = base.GroupSizes
+
+
+@dataclasses.dataclass(frozen=True)
+class Config:
+  """Tunables of the hip kernels; counterpart of pallas_mosaic_gpu_common.py:45-73.
+
+  (block_m, block_n, block_k, waves_m, waves_n) selects a precompiled kernel variant;
+  `grid_tile_width` m-tasks share one n-panel of rhs in launch order (L2 reuse);
+  `align_tile` is the row alignment of task starts (the reference's `align_tile`, default 8).
+  """
+
+  block_m: int
+  block_n: int
+  block_k: int
+  waves_m: int = 2
+  waves_n: int = 2
+  grid_tile_width: int = 8
+  align_tile: int = 8
+
+  def __post_init__(self):
+    for f in dataclasses.fields(self):
+      v = getattr(self, f.name)
+      if not isinstance(v, int) or isinstance(v, bool) or v <= 0:
+        raise ValueError(f"Config.{f.name} must be a positive int, got {v!r}")
+    if self.block_m % 8 != 0:
+      raise ValueError(f"Config.block_m must be a multiple of 8, got {self.block_m}")
+
+  def to_kernel_config(self) -> hip_ops.KernelConfig:
+    return hip_ops.KernelConfig(self.block_m, self.block_n, self.block_k, self.waves_m, self.waves_n,
+                                self.grid_tile_width, self.align_tile)
+
+
+_ACTIVATION_NAMES = {
+    torch.relu: "relu",
+    torch.nn.functional.relu: "relu",
+    torch.tanh: "tanh",
+    torch.nn.functional.tanh: "tanh",
+    torch.nn.functional.silu: "silu",
+}
+
+
+def _fused_activation_name(activation) -> str | None:
+  """Name of the in-kernel epilogue for a known activation callable, else None."""
+  try:
+    return _ACTIVATION_NAMES.get(activation)
+  except TypeError:  # unhashable callable
+    return None
+
+
+def _dtype_of(x) -> torch.dtype:
+  return x.qtype if isinstance(x, (QArray, AsQArray)) else x.dtype
+
+
+@functools.lru_cache(maxsize=None)
+def _variant_table():
+  """{(mode, lhs dtype code, rhs dtype code): [(bm, bn, bk, wm, wn), ...]} from the library."""
+  table: dict = {}
+  for kind in (0, 1):
+    for v in _lib.variants(kind):
+      key = (v["mode"], v["lhs_dtype"], v["rhs_dtype"])
+      table.setdefault(key, []).append((v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"]))
+  return table
+
+
+_MODE_OF_DIMS = {
+    base.DEFAULT_RAGGED_DOT_DIM_NUMS: 0,
+    base.TRANS_RHS_RAGGED_DOT_DIM_NUMS: 1,
+    base.RAGGED_CONTRACTING_DOT_DIM_NUMS: 2,
+}
+
+
+@dataclasses.dataclass(frozen=True)
+class HipRaggedDot(base.RaggedDot):
+  """Hand-written HIP ragged dot for gfx950. Physical layout `mk,gkn->mn`, rhs never transposed."""
+
+  config_cls: ClassVar[type] = Config
+  supports_symbolic_shapes: ClassVar[bool] = False
+
+  def __post_init__(self):
+    if self.vjp is None:
+      # A fresh op per call avoids infinite recursion (pallas_mosaic_gpu.py:95-100).
+      fn = lambda *a, **kw: HipRaggedDot()(*a, **kw)  # pylint: disable=unnecessary-lambda
+      object.__setattr__(self, "vjp", partial(base.vjp, dlhs_ragged_dot=fn, drhs_ragged_dot=fn))
+
+  # -- forward ---------------------------------------------------------------------------------
+  def _fwd(
+      self,
+      lhs,
+      rhs,
+      *,
+      group_sizes,
+      ragged_dot_dimension_numbers,
+      precision,
+      preferred_element_type,
+      return_residuals,
+      config: Config,
+      activation=None,
+      manual_axis_type=None,
+      group_offset=None,
+      rhs_scale=None,
+      rhs_bias=None,
+      maybe_quantize_lhs=False,
+      zero_initialize=True,
+      fuse_gateup_activation=None,
+      lhs_quantization_dtype=None,
+      rhs_quantization_dtype=None,
+  ):
+    del manual_axis_type  # sharding annotation only; no meaning on a single device
+    if (group_offset is not None or rhs_scale is not None or rhs_bias is not None or maybe_quantize_lhs
+        or not zero_initialize or fuse_gateup_activation is not None or lhs_quantization_dtype is not None
+        or rhs_quantization_dtype is not None):
+      raise NotImplementedError(
+          "The hip implementation does not support group_offset, rhs_scale, rhs_bias, maybe_quantize_lhs,"
+          " zero_initialize, fuse_gateup_activation, lhs_quantization_dtype, or rhs_quantization_dtype."
+      )
+    if isinstance(lhs, AsQArray) or isinstance(rhs, AsQArray):
+      raise NotImplementedError("The hip implementation does not quantise inputs on the fly (AsQArray).")
+    mode = _MODE_OF_DIMS.get(ragged_dot_dimension_numbers)
+    if mode is None:
+      raise NotImplementedError("Unsupported ragged dot dimension numbers.")
+
+    lhs_scale = rhs_scale_ = None
+    if isinstance(lhs, QArray):
+      if mode != 0 or lhs.zero_point is not None:
+        raise NotImplementedError("Quantised lhs: default dimension numbers without zero point only.")
+      m, k = lhs.qvalue.shape
+      if tuple(lhs.scale.shape) != (m, 1):
+        raise NotImplementedError(f"lhs scale must have shape [m,1] (one per row), got {tuple(lhs.scale.shape)}")
+      lhs_scale, lhs_v = lhs.scale, lhs.qvalue
+    else:
+      lhs_v = lhs
+    if isinstance(rhs, QArray):
+      if mode != 0 or rhs.zero_point is not None:
+        raise NotImplementedError("Quantised rhs: default dimension numbers without zero point only.")
+      g, k, n = rhs.qvalue.shape
+      if tuple(rhs.scale.shape) != (g, 1, n):
+        raise NotImplementedError(
+            f"rhs scale must have shape [g,1,n] (one per group and column), got {tuple(rhs.scale.shape)}")
+      rhs_scale_, rhs_v = rhs.scale, rhs.qvalue
+    else:
+      rhs_v = rhs
+
+    in_dtype = lhs.dtype if isinstance(lhs, QArray) else lhs_v.dtype
+    w_dtype = rhs.dtype if isinstance(rhs, QArray) else rhs_v.dtype
+    if not precision_lib.is_default(in_dtype, w_dtype, precision):
+      if precision == precision_lib.DotAlgorithmPreset.BF16_BF16_F32 and not isinstance(lhs, QArray) \
+          and not isinstance(rhs, QArray):
+        lhs_v, rhs_v = lhs_v.to(torch.bfloat16), rhs_v.to(torch.bfloat16)
+      else:
+        raise NotImplementedError(f"{precision=} not supported.")
+
+    if preferred_element_type is None:
+      preferred_element_type = torch.promote_types(in_dtype, w_dtype)
+    if preferred_element_type == torch.float8_e4m3fn:
+      preferred_element_type = w_dtype  # widened, as pallas_mosaic_gpu.py:197-205
+    if preferred_element_type not in (torch.float32, torch.bfloat16, torch.float16):
+      raise NotImplementedError(f"Output dtype {preferred_element_type} not supported.")
+
+    device = lhs_v.device
+    gs = group_sizes.to_tensor(device) if isinstance(group_sizes, GroupSizes) else group_sizes
+    if not isinstance(gs, torch.Tensor):
+      gs = torch.as_tensor(gs, dtype=torch.int32, device=device)
+
+    kcfg = config.to_kernel_config()
+    fused = None
+    if activation is not None and not return_residuals:
+      fused = _fused_activation_name(activation)
+
+    if mode == 2:
+      if isinstance(lhs, QArray) or isinstance(rhs, QArray):
+        raise NotImplementedError("Quantised inputs are not supported with ragged contracting dimensions.")
+      dot_out = hip_ops.ragged_dot_drhs(lhs_v, rhs_v, gs, gs.numel(), config=kcfg, out_dtype=preferred_element_type)
+    else:
+      # A callable with no in-kernel twin is applied to an f32 result, i.e. still in the accumulator
+      # dtype, and cast afterwards.
+      unfused = activation is not None and not return_residuals and fused is None
+      kernel_out = torch.float32 if unfused else preferred_element_type
+      dot_out = hip_ops.ragged_dot_fwd(lhs_v, rhs_v, gs, config=kcfg, out_dtype=kernel_out, trans_rhs=(mode == 1),
+                                       lhs_scale=lhs_scale, rhs_scale=rhs_scale_, activation=fused)
+      if unfused:
+        dot_out = activation(dot_out).to(preferred_element_type)
+
+    residuals = dot_out
+    if activation is not None and return_residuals:
+      dot_out = activation(dot_out)
+    elif activation is not None and mode == 2:
+      dot_out = activation(dot_out)
+    return dot_out, residuals if return_residuals else None
+
+  # -- configs ---------------------------------------------------------------------------------
+  def _problem(self, ba: op.BoundArguments):
+    lhs, rhs = ba.args[:2]
+    dims = ba.kwargs["ragged_dot_dimension_numbers"]
+    mode = _MODE_OF_DIMS.get(dims)
+    if mode is None:
+      raise NotImplementedError("Unsupported ragged dot dimension numbers.")
+    lhs_shape = tuple(lhs.shape)
+    rhs_shape = tuple(rhs.shape)
+    if mode == 2:
+      num_groups = int(ba.kwargs["group_sizes"].shape[0])
+      rows, cols, contraction = lhs_shape[1], rhs_shape[1], lhs_shape[0]
+    elif mode == 1:
+      num_groups = rhs_shape[0]
+      rows, cols, contraction = lhs_shape[0], rhs_shape[1], rhs_shape[2]
+    else:
+      num_groups = rhs_shape[0]
+      rows, cols, contraction = lhs_shape[0], rhs_shape[2], rhs_shape[1]
+    lhs_dt, rhs_dt = _dtype_of(lhs), _dtype_of(rhs)
+    if (ba.kwargs.get("precision") == precision_lib.DotAlgorithmPreset.BF16_BF16_F32
+        and not isinstance(lhs, (QArray, AsQArray)) and not isinstance(rhs, (QArray, AsQArray))):
+      lhs_dt = rhs_dt = torch.bfloat16  # `_fwd` casts both operands for this preset
+    key = (mode, hip_ops.dtype_code(lhs_dt), hip_ops.dtype_code(rhs_dt))
+    return mode, key, num_groups, rows, cols, contraction
+
+  def _get_heuristics_config(self, ba: op.BoundArguments) -> Config:
+    mode, key, num_groups, rows, cols, contraction = self._problem(ba)
+    variants = _variant_table().get(key)
+    if not variants:
+      raise NotImplementedError(f"No hip kernel for dtypes/mode {key}.")
+    usable = list(variants)
+    # Rows per group decide the m-tile: a tile much taller than a group wastes MFMA work on rows
+    # that are masked out at the store; a short tile re-reads the weights more often.
+    rows_per_group = rows / max(num_groups, 1) if mode != 2 else rows
+    want_m = 256 if rows_per_group >= 1024 else 128 if rows_per_group >= 192 else 64 if rows_per_group >= 48 else 32
+    want_n = 256 if cols >= 2048 else 128
+
+    def score(v):
+      bm, bn, bk, wm, wn = v
+      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -bk)
+
+    bm, bn, bk, wm, wn = min(usable, key=score)
+    return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, grid_tile_width=8, align_tile=8)
+
+  def _get_autotuning_configs(self, ba: op.BoundArguments) -> set[Config]:
+    mode, key, _, _, _, _ = self._problem(ba)
+    configs = set()
+    for bm, bn, bk, wm, wn in _variant_table().get(key, []):
+      widths = (1,) if mode == 2 else (1, 2, 4, 8, 16)
+      for w in widths:
+        configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, grid_tile_width=w))
+    return configs
+
+  def supported_on(self, device: torch.device) -> bool:
+    if config_lib.cross_compile.value:
+      return True
+    if device.type != "cuda" or not torch.cuda.is_available() or torch.version.hip is None:
+      return False
+    arch = getattr(torch.cuda.get_device_properties(device), "gcnArchName", "")
+    return arch.split(":")[0] == "gfx950"
