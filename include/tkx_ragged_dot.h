@@ -53,7 +53,7 @@ enum TkxMode {
 enum TkxActivation { TKX_ACT_NONE = 0, TKX_ACT_RELU = 1, TKX_ACT_TANH = 2, TKX_ACT_SILU = 3, TKX_ACT_GELU_TANH = 4 };
 
 /* Tunables; the gfx950 counterpart of the reference's Config (pallas_mosaic_gpu_common.py:45-73).
- * (block_m, block_n, block_k, waves_m, waves_n) must name a compiled kernel variant
+ * (block_m, block_n, block_k, waves_m, waves_n, num_stages) must name a compiled kernel variant
  * (see tkx_ragged_dot_num_variants / tkx_ragged_dot_variant). */
 typedef struct TkxConfig {
   int32_t block_m;         /* rows of lhs per task (multiple of 8) */
@@ -63,7 +63,7 @@ typedef struct TkxConfig {
   int32_t waves_n;         /* wavefronts along n in a workgroup */
   int32_t grid_tile_width; /* m-tasks that share an n-panel in launch order (L2 reuse) */
   int32_t align_tile;      /* task starts are aligned down to this many rows (reference default 8) */
-  int32_t reserved;
+  int32_t num_stages;      /* LDS stages of block_k contraction elements kept in flight */
 } TkxConfig;
 
 /* Library / ABI version (major*1000 + minor). */

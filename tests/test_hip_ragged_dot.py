@@ -254,8 +254,8 @@ def test_straddling_groups(group_sizes, block_m, device):
   a, b, _ = _inputs("test_straddling", G, m, k, n, torch.bfloat16, device)
   gs = np.array(group_sizes, np.int32)
   table = hip._variant_table()[(0, _lib.TKX_BF16, _lib.TKX_BF16)]
-  bm, bn, bk, wm, wn = next(v for v in table if v[0] == block_m)
-  op = hip.HipRaggedDot(config=hip.Config(bm, bn, bk, wm, wn, grid_tile_width=2))
+  bm, bn, bk, wm, wn, ns = next(v for v in table if v[0] == block_m)
+  op = hip.HipRaggedDot(config=hip.Config(bm, bn, bk, wm, wn, ns, grid_tile_width=2))
   out = op(a, b, group_sizes=torch.tensor(gs, device=device), preferred_element_type=torch.float32)
   _check(out, _ref(a, b, gs), TOL[torch.bfloat16])
   again = op(a, b, group_sizes=torch.tensor(gs, device=device), preferred_element_type=torch.float32)
@@ -282,7 +282,7 @@ def _variant_cases():
   cases = []
   for kind in (0, 1):
     for v in _lib.variants(kind):
-      cases.append(pytest.param(v, id="mode{mode}-d{lhs_dtype}x{rhs_dtype}-{block_m}x{block_n}x{block_k}-w{waves_m}x{waves_n}".format(**v)))
+      cases.append(pytest.param(v, id="mode{mode}-d{lhs_dtype}x{rhs_dtype}-{block_m}x{block_n}x{block_k}-w{waves_m}x{waves_n}-s{num_stages}".format(**v)))
   return cases
 
 
@@ -297,7 +297,8 @@ def test_every_kernel_variant_through_c_abi(v, device):
   G, m, k, n = 6, 640, 256, 384
   gs = np.array([100, 0, 257, 9, 130, 80], np.int32)  # sum 576 < m
   gst = torch.tensor(gs, device=device)
-  cfg = hip_ops.KernelConfig(v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"], grid_tile_width=3)
+  cfg = hip_ops.KernelConfig(v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"], v["num_stages"],
+                             grid_tile_width=3)
   lt, rt = _TORCH_DTYPE[v["lhs_dtype"]], _TORCH_DTYPE[v["rhs_dtype"]]
   mk = lambda shape, std: torch.tensor(rng.normal(0, std, shape).astype(np.float32), device=device)
   if v["mode"] == 2:

@@ -66,7 +66,7 @@ def test_variant_enumeration_matches_config_space():
 
 def test_c_abi_argument_errors_without_gpu():
   lib = _lib.load()
-  cfg = _lib.TkxConfig(128, 128, 64, 2, 2, 1, 8, 0)
+  cfg = _lib.TkxConfig(128, 128, 64, 2, 2, 1, 8, 2)
   st = lib.tkx_ragged_dot_fwd(None, None, None, None, None, None, None, 8, 8, 8, 1, 1, 1, 1, 0, 0, ctypes.byref(cfg), None)
   assert st == _lib.TKX_ERR_INVALID and "null" in _lib.last_error()
   with pytest.raises(ValueError):
@@ -315,7 +315,7 @@ def test_cache_file_name_and_json_round_trip(tmp_path):
   assert parsed["group_sizes"] == {"num_groups": 256, "total_size": 131072}
   assert parsed["ragged_dot_dimension_numbers"]["dot_dimension_numbers"] == [[[1], [1]], [[], []]]
   assert parsed["precision"] == ["DEFAULT", "DEFAULT"] and parsed["preferred_element_type"] is None
-  cfg = hip.Config(block_m=128, block_n=256, block_k=64, waves_m=2, waves_n=4)
+  cfg = hip.Config(block_m=128, block_n=256, block_k=64, waves_m=2, waves_n=4, num_stages=3)
   text = cache_lib.dumps(op, {ba.autotuning_cache_key: autotuner_lib.AutotuningData({cfg: _bench(1.5), hip.Config(64, 128, 64): RuntimeError("x")})})
   loaded = cache_lib.loads(op, text)
   assert list(loaded) == [ba.autotuning_cache_key]
@@ -337,7 +337,7 @@ def test_cache_file_name_and_json_round_trip(tmp_path):
     tiles = {v for vs in table.values() for v in vs}
     for data in entries.values():
       for c in data:
-        assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n) in tiles
+        assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages) in tiles
 
 
 def test_bound_args_and_autotuning_result_round_trip():
@@ -365,7 +365,7 @@ def test_hip_config_validation_and_heuristics():
   for spec in arg_specs.ARG_SPECS:
     ba = op.bind(**spec.args)
     c = ba.heuristics_config
-    assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n) in table[(0, _lib.TKX_BF16, _lib.TKX_BF16)]
+    assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages) in table[(0, _lib.TKX_BF16, _lib.TKX_BF16)]
     configs = ba.autotuning_configs
     assert c in configs and len(configs) > 10
   # decode-like int8 weights pick a short m-tile; unsupported dtypes raise NotImplementedError

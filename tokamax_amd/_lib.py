@@ -46,7 +46,7 @@ class TkxConfig(ctypes.Structure):
       ("waves_n", ctypes.c_int32),
       ("grid_tile_width", ctypes.c_int32),
       ("align_tile", ctypes.c_int32),
-      ("reserved", ctypes.c_int32),
+      ("num_stages", ctypes.c_int32),
   ]
 
 
@@ -125,5 +125,5 @@ def variants(kind: int):
     a, b, mode = ctypes.c_int32(), ctypes.c_int32(), ctypes.c_int32()
     check(lib.tkx_ragged_dot_variant(kind, i, ctypes.byref(cfg), ctypes.byref(a), ctypes.byref(b), ctypes.byref(mode)))
     out.append(dict(block_m=cfg.block_m, block_n=cfg.block_n, block_k=cfg.block_k, waves_m=cfg.waves_m,
-                    waves_n=cfg.waves_n, lhs_dtype=a.value, rhs_dtype=b.value, mode=mode.value))
+                    waves_n=cfg.waves_n, num_stages=cfg.num_stages, lhs_dtype=a.value, rhs_dtype=b.value, mode=mode.value))
   return out

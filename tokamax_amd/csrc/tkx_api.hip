@@ -41,7 +41,8 @@ const Registry& registry() {
 const Variant* find_variant(int mode, int a_dtype, int b_dtype, const TkxConfig& c) {
   for (const Variant& v : registry().all)
     if (v.mode == mode && v.a_dtype == a_dtype && v.b_dtype == b_dtype && v.block_m == c.block_m &&
-        v.block_n == c.block_n && v.block_k == c.block_k && v.waves_m == c.waves_m && v.waves_n == c.waves_n)
+        v.block_n == c.block_n && v.block_k == c.block_k && v.waves_m == c.waves_m && v.waves_n == c.waves_n &&
+        v.num_stages == c.num_stages)
       return &v;
   return nullptr;
 }
@@ -130,7 +131,8 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   if (!valid_out_dtype(out_dtype)) return set_error(TKX_ERR_UNSUPPORTED, "out dtype %d not supported", out_dtype);
   if (activation < TKX_ACT_NONE || activation > TKX_ACT_GELU_TANH)
     return set_error(TKX_ERR_INVALID, "bad activation %d", activation);
-  if (m > 0x7fffffffLL / 2 || k > 0x7fffffffLL / 2 || n > 0x7fffffffLL / 2)
+  // Per-lane byte offsets inside a tile are 32-bit: (256 rows) x (row bytes) must stay below 2^31.
+  if (m > 0x7fffffffLL / 2 || k >= (1 << 21) || n >= (1 << 21))
     return set_error(TKX_ERR_UNSUPPORTED, "dimension too large");
   const TkxConfig& c = *config;
   if (c.block_m < 8 || c.block_m % 8 != 0) return set_error(TKX_ERR_INVALID, "block_m must be a positive multiple of 8");
@@ -139,8 +141,8 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   if (dlhs && (lhs_scale || rhs_scale)) return set_error(TKX_ERR_UNSUPPORTED, "scales are not supported with TRANS_RHS");
   const Variant* v = find_variant(dlhs ? kDlhs : kFwd, lhs_dtype, rhs_dtype, c);
   if (v == nullptr)
-    return set_error(TKX_ERR_UNSUPPORTED, "no kernel variant for mode=%d dtypes=(%d,%d) tile=%dx%dx%d waves=%dx%d", mode,
-                     lhs_dtype, rhs_dtype, c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n);
+    return set_error(TKX_ERR_UNSUPPORTED, "no kernel variant for mode=%d dtypes=(%d,%d) tile=%dx%dx%d waves=%dx%d stages=%d",
+                     mode, lhs_dtype, rhs_dtype, c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages);
   // In C terms: rows = m; cols = n (fwd) or k (dlhs); contraction = k (fwd) or n (dlhs).
   const int64_t cols = dlhs ? k : n, contraction = dlhs ? n : k;
   const int lb = dtype_bytes(lhs_dtype), rb = dtype_bytes(rhs_dtype), ob = dtype_bytes(out_dtype);
@@ -205,14 +207,14 @@ int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* gr
     return set_error(TKX_ERR_INVALID, "bad sizes m=%lld k=%lld n=%lld G=%lld", (long long)m, (long long)k,
                      (long long)n, (long long)num_groups);
   if (!valid_out_dtype(out_dtype)) return set_error(TKX_ERR_UNSUPPORTED, "out dtype %d not supported", out_dtype);
-  if (m > 0x7fffffffLL / 2 || k > 0x7fffffffLL / 2 || n > 0x7fffffffLL / 2)
+  if (m > 0x7fffffffLL / 2 || k >= (1 << 21) || n >= (1 << 21))
     return set_error(TKX_ERR_UNSUPPORTED, "dimension too large");
   const TkxConfig& c = *config;
   if (c.align_tile < 1) return set_error(TKX_ERR_INVALID, "align_tile must be >= 1");
   const Variant* v = find_variant(kDrhs, dtype, dtype, c);
   if (v == nullptr)
-    return set_error(TKX_ERR_UNSUPPORTED, "no drhs kernel variant for dtype=%d tile=%dx%dx%d waves=%dx%d", dtype,
-                     c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n);
+    return set_error(TKX_ERR_UNSUPPORTED, "no drhs kernel variant for dtype=%d tile=%dx%dx%d waves=%dx%d stages=%d", dtype,
+                     c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages);
   const int eb = dtype_bytes(dtype), ob = dtype_bytes(out_dtype);
   if ((k * eb) % 16 != 0 || (n * eb) % 16 != 0 || (n * ob) % 16 != 0 || n % 8 != 0)
     return set_error(TKX_ERR_UNSUPPORTED, "k and n row sizes must be multiples of 16 bytes (n of 8 elements)");
@@ -268,7 +270,7 @@ int32_t tkx_ragged_dot_variant(int32_t kind, int32_t index, TkxConfig* config, i
     config->waves_n = v.waves_n;
     config->grid_tile_width = 1;
     config->align_tile = 8;
-    config->reserved = 0;
+    config->num_stages = v.num_stages;
     *lhs_dtype = v.a_dtype;
     *rhs_dtype = v.b_dtype;
     *mode = v.mode;

@@ -77,7 +77,7 @@ struct GemmParams {
 struct Variant {
   int32_t mode;  // KernelMode
   int32_t a_dtype, b_dtype;
-  int32_t block_m, block_n, block_k, waves_m, waves_n;
+  int32_t block_m, block_n, block_k, waves_m, waves_n, num_stages;
   int32_t smem_bytes;
   const void* fn;  // __global__ void (*)(GemmParams)
 };

@@ -9,8 +9,8 @@
 //                (C[g][k,n] = lhs[rows_g]^T . dout[rows_g]; contraction = the group's row range)
 //
 // A workgroup owns one BM x BN tile of C. k-steps of BK contraction elements are staged through
-// two LDS buffers (global -> registers -> LDS, the next step's global loads in flight during the
-// MFMAs of the current one). Operands that are contraction-contiguous are read from LDS with
+// two LDS buffers with direct-to-LDS loads (global_load_lds_dwordx4): the next step's loads are in
+// flight during the MFMAs of the current one, and fragments are double-buffered in registers. Operands that are contraction-contiguous are read from LDS with
 // ds_read_b128; operands that are contiguous along the other axis are read with the gfx950
 // transposing LDS loads (ds_read_b64_tr_b16 / _tr_b8), so no operand is ever transposed in memory.
 // The 32x32 MFMA is issued with its operands swapped (B-fragment first) so that each lane ends up
@@ -79,22 +79,29 @@ __device__ __forceinline__ f32x16 mma_atom(const typename Mma<EA>::Frag& first, 
 // Contraction-contiguous tile: [rows][ROW_BYTES], 16-byte chunks XOR-swizzled by the row so that the
 // 16/32 lanes of one ds_read_b128 phase touch distinct banks.
 template <int ROW_BYTES>
-__device__ __forceinline__ int kc_offset(int row, int chunk) {
+__device__ __forceinline__ int kc_swizzle(int row) {
   constexpr int CPR = ROW_BYTES / 16;
-  const int s = ((row & 7) ^ ((row >> 3) & 1)) & (CPR - 1);
-  return row * ROW_BYTES + ((chunk ^ s) << 4);
+  return ((row & 7) ^ ((row >> 3) & 1)) & (CPR - 1);
+}
+template <int ROW_BYTES>
+__device__ __forceinline__ int kc_offset(int row, int chunk) {
+  return row * ROW_BYTES + ((chunk ^ kc_swizzle<ROW_BYTES>(row)) << 4);
 }
 
 // Row/column-contiguous tile: [BK rows of k][ROW_BYTES], 32-byte granules XOR-swizzled by k.
 // E selects the pattern that suits the read instruction used for that element size.
 template <int ROW_BYTES, int E>
-__device__ __forceinline__ int mc_offset(int krow, int byte_in_row) {
+__device__ __forceinline__ int mc_swizzle(int krow) {
   constexpr int NG = ROW_BYTES / 32;
   int f;
   if constexpr (E == kEF32) f = ((krow >> 2) & 1) << 2;
   else if constexpr (E == kEBF16 || E == kEF16) f = ((krow & 3) << 1) ^ ((krow >> 1) & 1);
   else f = krow & 7;
-  const int g = (byte_in_row >> 5) ^ (f & (NG - 1));
+  return f & (NG - 1);
+}
+template <int ROW_BYTES, int E>
+__device__ __forceinline__ int mc_offset(int krow, int byte_in_row) {
+  const int g = (byte_in_row >> 5) ^ mc_swizzle<ROW_BYTES, E>(krow);
   return krow * ROW_BYTES + (g << 5) + (byte_in_row & 31);
 }
 
@@ -185,12 +192,129 @@ __device__ __forceinline__ typename Mma<EC>::Frag load_frag(const unsigned char*
   }
 }
 
-// ---- global -> register -> LDS staging ------------------------------------------------------
-// One operand tile of a k-step, moved in 16-byte chunks; chunk q of the tile belongs to thread
-// (q % THREADS). Out-of-range rows/columns are clamped to valid memory (their products are never
-// stored); contraction indices at or past `k_hi` are zero-filled, which only the last k-step of
-// a tile can need (a workgroup-uniform test keeps the other steps free of per-lane masking).
-template <int LAYOUT, int ES, int RC /* rows or cols of C covered */, int BK, int THREADS>
+// ---- global -> LDS, fast path: direct-to-LDS loads -------------------------------------------
+// global_load_lds_dwordx4 moves 16 bytes per lane straight into LDS; one wave instruction fills
+// 1024 contiguous LDS bytes (lane l lands at base + 16*l). The LDS swizzle is therefore applied
+// on the global side: each lane fetches the chunk that belongs at its fixed LDS position.
+// Out-of-range rows/columns are clamped to valid memory (their products are never stored).
+// Only whole k-steps go this way; a partial last step is zero-filled through TileStage below.
+// The loads are issued from inline assembly on purpose: the compiler guards every LDS read that
+// follows a direct-to-LDS load it can see with a full vmcnt(0) wait (it cannot tell which LDS bytes
+// the load writes), which would serialise each k-step's loads with its MFMAs. Ordering is enforced
+// explicitly instead, by barrier_after_direct_loads(). M0 carries the LDS destination.
+__device__ __forceinline__ unsigned lds_address(const unsigned char* p) {
+  return __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)p);
+}
+__device__ __forceinline__ const unsigned char* uniform_pointer(const unsigned char* p) {
+  const uint64_t v = (uint64_t)(uintptr_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const unsigned char*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+// 16 bytes per lane: LDS[lds + 16*lane] <- *(sbase + voff)
+__device__ __forceinline__ void direct_load_16(const unsigned char* sbase, uint32_t voff, unsigned lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff), "s"(sbase)
+               : "memory", "m0");
+}
+// 4 bytes per lane from a per-lane address (used only to touch cache lines).
+__device__ __forceinline__ void direct_load_4(const unsigned char* vptr, unsigned lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds), "v"(vptr) : "memory", "m0");
+}
+
+// Workgroup barrier that also orders direct-to-LDS loads: a wave's loads count on vmcnt, and other
+// waves read the bytes they deposit, so every wave must drain vmcnt BEFORE it arrives at the
+// barrier (the compiler only guards a wave's own later LDS reads).
+// N = number of this wave's most recent direct loads that may stay in flight (they belong to
+// later stages); loads complete in issue order.
+template <int N>
+__device__ __forceinline__ void barrier_after_direct_loads() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  // s_waitcnt immediate: vmcnt = bits [3:0] and [15:14], expcnt = [6:4] (7: no wait), lgkmcnt = [11:8] (0: all).
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4));
+#if defined(TKX_ABLATE) && (TKX_ABLATE & 8)
+  return;
+#endif
+  __syncthreads();
+}
+
+template <int LAYOUT, int ES, int RC /* rows or cols of C covered */, int BK, int NWAVES>
+struct DirectLoader {
+  static constexpr int ESZ = elem_bytes(ES);
+  static constexpr int ROW_BYTES = (LAYOUT == kKC) ? BK * ESZ : RC * ESZ;
+  static constexpr int ROWS = (LAYOUT == kKC) ? RC : BK;
+  static constexpr int BYTES = ROWS * ROW_BYTES;
+  static constexpr int INSTRS = BYTES / 1024;
+  static constexpr int PER = (INSTRS + NWAVES - 1) / NWAVES;
+  static_assert(BYTES % 1024 == 0, "tile must be a whole number of wave-wide 16-byte loads");
+
+  uint32_t voff[PER];  // per-lane byte offset from the wave-uniform base pointer of a k-step
+
+  // Base pointer of the k-step that starts at contraction index kc0 (uniform across the workgroup).
+  static __device__ __forceinline__ int64_t step_base(int rc0, int64_t ld, int kc0) {
+    if constexpr (LAYOUT == kKC) return ((int64_t)rc0 * ld + kc0) * ESZ;
+    else return (int64_t)kc0 * ld * ESZ;
+  }
+  static __device__ __forceinline__ int64_t step_bytes(int64_t ld) {
+    if constexpr (LAYOUT == kKC) return (int64_t)BK * ESZ;
+    else return (int64_t)BK * ld * ESZ;
+  }
+
+  __device__ __forceinline__ void init(int rc0, int rc_ext, int64_t ld, int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int j = i * NWAVES + wave;
+      const int off = j * 1024 + lane * 16;
+      const int row = off / ROW_BYTES, pc = (off % ROW_BYTES) >> 4;
+      if constexpr (LAYOUT == kKC) {
+        const int lc = pc ^ kc_swizzle<ROW_BYTES>(row);
+        int grow = rc0 + row;
+        grow = (grow < rc_ext ? grow : rc_ext - 1) - rc0;
+        voff[i] = (uint32_t)(grow * (int)ld * ESZ + lc * 16);
+      } else {
+        const int lc = ((((pc >> 1) ^ mc_swizzle<ROW_BYTES, ES>(row))) << 1) | (pc & 1);
+        int colb = rc0 * ESZ + lc * 16;
+        const int lim = rc_ext * ESZ - 16;
+        colb = colb < lim ? colb : lim;
+        voff[i] = (uint32_t)(row * (int)ld * ESZ + colb);
+      }
+    }
+  }
+
+  // Cache lines (128 B, or a whole row when rows are shorter) of one k-step tile, and the byte
+  // offset of line `line` from the k-step base pointer: used to pull a later k-step into L2.
+  static constexpr int LINE = ROW_BYTES < 128 ? ROW_BYTES : 128;
+  static constexpr int LINES = BYTES / LINE;
+  static __device__ __forceinline__ uint32_t line_offset(int line, int rc0, int rc_ext, int64_t ld) {
+    constexpr int LPR = ROW_BYTES / LINE;
+    const int row = line / LPR, seg = line % LPR;
+    if constexpr (LAYOUT == kKC) {
+      int grow = rc0 + row;
+      grow = (grow < rc_ext ? grow : rc_ext - 1) - rc0;
+      return (uint32_t)(grow * (int)ld * ESZ + seg * LINE);
+    } else {
+      int colb = rc0 * ESZ + seg * LINE;
+      const int lim = rc_ext * ESZ - 16;
+      colb = colb < lim ? colb : lim;
+      return (uint32_t)(row * (int)ld * ESZ + colb);
+    }
+  }
+
+  __device__ __forceinline__ void issue(const unsigned char* base, unsigned char* tile, int wave) const {
+#if defined(TKX_ABLATE) && (TKX_ABLATE & 1)
+    return;
+#endif
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int j = i * NWAVES + wave;
+      if (INSTRS % NWAVES != 0 && j >= INSTRS) break;
+      direct_load_16(base, voff[i], lds_address(tile + j * 1024));
+    }
+  }
+};
+
+// ---- global -> register -> LDS, masked path (a partial last k-step) ---------------------------
+// One operand tile moved in 16-byte chunks; chunk q of the tile belongs to thread (q % THREADS).
+// Contraction indices at or past `k_hi` are zero-filled.
+template <int LAYOUT, int ES, int RC, int BK, int THREADS>
 struct TileStage {
   static constexpr int ESZ = elem_bytes(ES);
   static constexpr int ROW_BYTES = (LAYOUT == kKC) ? BK * ESZ : RC * ESZ;
@@ -201,57 +325,33 @@ struct TileStage {
   static constexpr int BYTES = ROWS * ROW_BYTES;
   static_assert(ROW_BYTES % 32 == 0 && (CPR & (CPR - 1)) == 0, "tile rows must be a power-of-two number of chunks");
 
-  i32x4 regs[PER];
-
   // base: operand pointer already offset to the group; ld in elements; rc0 = first row/col of the
-  // tile; rc_ext = extent of that axis; kc0 = first contraction index of this k-step;
-  // k_hi = end of the valid contraction range.
-  __device__ __forceinline__ void load(const unsigned char* base, int64_t ld, int rc0, int rc_ext, int kc0, int k_hi,
-                                       int tid) {
-    const bool full = kc0 + BK <= k_hi;  // uniform across the workgroup
+  // tile; rc_ext = extent of that axis; kc0 = first contraction index of this k-step.
+  static __device__ __forceinline__ void copy(const unsigned char* base, int64_t ld, int rc0, int rc_ext, int kc0,
+                                              int k_hi, unsigned char* tile, int tid) {
     const i32x4 z = {0, 0, 0, 0};
-#pragma unroll
+#pragma unroll 2
     for (int i = 0; i < PER; ++i) {
       const int q = tid + i * THREADS;
       if (CHUNKS % THREADS != 0 && q >= CHUNKS) break;
       const int r = q / CPR, c = q % CPR;
+      i32x4 v = z;
+      int off;
       if constexpr (LAYOUT == kKC) {
         int row = rc0 + r;
         row = row < rc_ext ? row : rc_ext - 1;
         const int kcol = kc0 + c * (16 / ESZ);
-        const unsigned char* p = base + ((int64_t)row * ld + kcol) * ESZ;
-        if (full) {
-          regs[i] = *reinterpret_cast<const i32x4*>(p);
-        } else {
-          regs[i] = z;
-          if (kcol < k_hi) regs[i] = *reinterpret_cast<const i32x4*>(p);
-        }
+        if (kcol < k_hi) v = *reinterpret_cast<const i32x4*>(base + ((int64_t)row * ld + kcol) * ESZ);
+        off = kc_offset<ROW_BYTES>(r, c);
       } else {
         const int krow = kc0 + r;
         int colb = rc0 * ESZ + c * 16;
         const int lim = rc_ext * ESZ - 16;
         colb = colb < lim ? colb : lim;
-        const unsigned char* p = base + (int64_t)krow * ld * ESZ + colb;
-        if (full) {
-          regs[i] = *reinterpret_cast<const i32x4*>(p);
-        } else {
-          regs[i] = z;
-          if (krow < k_hi) regs[i] = *reinterpret_cast<const i32x4*>(p);
-        }
+        if (krow < k_hi) v = *reinterpret_cast<const i32x4*>(base + (int64_t)krow * ld * ESZ + colb);
+        off = mc_offset<ROW_BYTES, ES>(r, c * 16);
       }
-    }
-  }
-
-  __device__ __forceinline__ void store(unsigned char* tile, int tid) const {
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int q = tid + i * THREADS;
-      if (CHUNKS % THREADS != 0 && q >= CHUNKS) break;
-      const int r = q / CPR, c = q % CPR;
-      int off;
-      if constexpr (LAYOUT == kKC) off = kc_offset<ROW_BYTES>(r, c);
-      else off = mc_offset<ROW_BYTES, ES>(r, c * 16);
-      *reinterpret_cast<i32x4*>(tile + off) = regs[i];
+      *reinterpret_cast<i32x4*>(tile + off) = v;
     }
   }
 };
@@ -286,7 +386,7 @@ __device__ __forceinline__ void store4(void* C, int64_t idx, f32x4 v, int out_dt
 }
 
 // ---- the kernel ---------------------------------------------------------------------------------
-template <int MODE, int EA, int EB, int BM, int BN, int BK, int WM, int WN>
+template <int MODE, int EA, int EB, int BM, int BN, int BK, int WM, int WN, int NS>
 struct GemmKernel {
   static constexpr int THREADS = WM * WN * 64;
   static constexpr int LA = (MODE == kDrhs) ? kMC : kKC;
@@ -296,10 +396,29 @@ struct GemmKernel {
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int TM = WTM / 32, TN = WTN / 32;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % KA == 0, "tile does not split into 32x32 atoms");
+  static constexpr int KSTEPS = BK / KA;
+  static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
   typedef TileStage<LA, EA, BM, BK, THREADS> StageA;
   typedef TileStage<LB, EB, BN, BK, THREADS> StageB;
+  // The last wave of the workgroup issues no tile loads: it only prefetches into L2 (see below), so
+  // that a slow prefetch never sits in front of a tile load in a wave's in-order vmcnt queue.
+  static constexpr int NLOAD = WM * WN - 1;
+  typedef DirectLoader<LA, EA, BM, BK, NLOAD> DirA;
+  typedef DirectLoader<LB, EB, BN, BK, NLOAD> DirB;
   static constexpr int STAGE_BYTES = StageA::BYTES + StageB::BYTES;
-  static constexpr int SMEM_BYTES = 2 * STAGE_BYTES;
+  // L2 prefetch. A workgroup can only keep NS-1 k-steps of direct loads in flight (LDS capacity),
+  // which is less than the HBM round trip; so each k-step the prefetch wave touches cache lines of
+  // the k-step PD steps further ahead with 4-byte direct-to-LDS loads into a dump area nobody
+  // reads, pulling them into L2. The workgroups that run side by side on an XCD share panels
+  // (kDedupA n-tiles share an A panel, kDedupB m-tiles share a B panel), so each touches a slice.
+  static constexpr int PD = 2;
+  static constexpr int kDedupA = 4, kDedupB = 8;
+  static constexpr int PF_A = DirA::LINES / kDedupA, PF_B = DirB::LINES / kDedupB;  // lines per workgroup
+  static constexpr int PFI = (PF_A + PF_B + 63) / 64;  // prefetch instructions per k-step
+  static_assert(PF_A >= 1 && PF_B >= 1, "prefetch slices must not be empty");
+  static constexpr int DUMP_BYTES = 256;
+  static constexpr int SMEM_BYTES = NS * STAGE_BYTES + DUMP_BYTES;
+  static_assert(NS >= 2 && SMEM_BYTES <= 160 * 1024, "stages must fit the 160 KB LDS");
 
   static __device__ __forceinline__ void run(const GemmParams& p, unsigned char* smem) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -308,6 +427,7 @@ struct GemmKernel {
     const int b = blockIdx.x;
 
     int group, row0, act_start, act_end, col0, kc_begin, kc_end;
+    int pf_slice_a, pf_slice_b;  // which slice of the shared panels this workgroup prefetches
     if constexpr (MODE != kDrhs) {
       const int num_tasks = ws[0];
       if (b >= p.real_slots) {
@@ -344,6 +464,8 @@ struct GemmKernel {
       col0 = nt * BN;
       kc_begin = 0;
       kc_end = p.k_ext;
+      pf_slice_a = nt & (kDedupA - 1);
+      pf_slice_b = (rem - nt * wcur) & (kDedupB - 1);
     } else {
       const int per_group = p.m_tiles * p.n_tiles;
       group = b / per_group;
@@ -355,6 +477,8 @@ struct GemmKernel {
       act_end = min(row0 + BM, p.m_ext);
       kc_begin = min(ws[p.ws_offsets + group], p.k_ext);
       kc_end = min(ws[p.ws_offsets + group + 1], p.k_ext);
+      pf_slice_a = nt & (kDedupA - 1);
+      pf_slice_b = mt & (kDedupB - 1);
     }
 
     const unsigned char* Ab = reinterpret_cast<const unsigned char*>(p.A);
@@ -369,46 +493,140 @@ struct GemmKernel {
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    const int nk = (kc_end - kc_begin + BK - 1) / BK;
-    StageA sa;
-    StageB sb;
-    if (nk > 0) {
-      sa.load(Ab, p.lda, row0, p.m_ext, kc_begin, kc_end, tid);
-      sb.load(Bb, p.ldb, col0, p.n_ext, kc_begin, kc_end, tid);
-      sa.store(smem, tid);
-      sb.store(smem + StageA::BYTES, tid);
-    }
-    __syncthreads();
+    typedef typename Mma<EC>::Frag Frag;
+    auto load_frags = [&](Frag* fa, Frag* fb, const unsigned char* stage, int kk) {
+#if defined(TKX_ABLATE) && (TKX_ABLATE & 2)
+      return;
+#endif
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        fa[i] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, wm * WTM + i * 32, kk, lane);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        fb[j] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + j * 32, kk, lane);
+    };
+    auto mma_all = [&](const Frag* fa, const Frag* fb) {
+#if defined(TKX_ABLATE) && (TKX_ABLATE & 4)
+      for (int i = 0; i < TM; ++i) asm volatile("" ::"v"(fa[i]));
+      for (int j = 0; j < TN; ++j) asm volatile("" ::"v"(fb[j]));
+      return;
+#endif
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = mma_atom<EC>(fb[j], fa[i], acc[i][j]);
+    };
 
-    for (int kt = 0; kt < nk; ++kt) {
-      const unsigned char* tA = smem + (kt & 1) * STAGE_BYTES;
-      const unsigned char* tB = tA + StageA::BYTES;
-      const bool more = kt + 1 < nk;
-      if (more) {
-        const int kc0 = kc_begin + (kt + 1) * BK;
-        sa.load(Ab, p.lda, row0, p.m_ext, kc0, kc_end, tid);
-        sb.load(Bb, p.ldb, col0, p.n_ext, kc0, kc_end, tid);
+    const int span = kc_end - kc_begin;
+    const int nfull = span > 0 ? span / BK : 0;  // whole k-steps: direct-to-LDS, software pipelined
+    const bool tail = span > nfull * BK;         // partial last k-step: zero-filled through registers
+
+    if (nfull > 0) {
+      DirA da;
+      DirB db;
+      da.init(row0, p.m_ext, p.lda, wave, lane);
+      db.init(col0, p.n_ext, p.ldb, wave, lane);
+      const unsigned char* gA = Ab + DirA::step_base(row0, p.lda, kc_begin);
+      const unsigned char* gB = Bb + DirB::step_base(col0, p.ldb, kc_begin);
+      const int64_t stepA = DirA::step_bytes(p.lda), stepB = DirB::step_bytes(p.ldb);
+      // A load wave may leave the loads of the NS-2 k-steps after the needed one in flight; that
+      // count is only known at compile time when the tile splits evenly over the load waves.
+      constexpr bool kExact = DirA::INSTRS % NLOAD == 0 && DirB::INSTRS % NLOAD == 0;
+      constexpr int kInFlight = kExact ? (NS - 2) * (DirA::PER + DirB::PER) : 0;
+      static_assert(kInFlight < 64, "too many direct loads in flight for vmcnt");
+
+      // L2 prefetch lines of this lane (prefetch wave only; slots past the slice repeat its last line).
+      const bool pf_wave = wave == NLOAD;
+      uint32_t pf_off[PFI];
+      bool pf_is_b[PFI];
+#pragma unroll
+      for (int i = 0; i < PFI; ++i) {
+        int idx = i * 64 + lane;
+        idx = idx < PF_A + PF_B ? idx : PF_A + PF_B - 1;
+        pf_is_b[i] = idx >= PF_A;
+        pf_off[i] = pf_is_b[i] ? DirB::line_offset(pf_slice_b * PF_B + (idx - PF_A), col0, p.n_ext, p.ldb)
+                               : DirA::line_offset(pf_slice_a * PF_A + idx, row0, p.m_ext, p.lda);
       }
+      unsigned char* dump = smem + NS * STAGE_BYTES;
+      const unsigned char* const gA0 = gA;
+      const unsigned char* const gB0 = gB;
+      auto prefetch_step = [&](int step) {
+        if (step >= nfull) return;
+        const unsigned char* a = gA0 + step * stepA;
+        const unsigned char* b = gB0 + step * stepB;
 #pragma unroll
-      for (int kk = 0; kk < BK / KA; ++kk) {
-        typename Mma<EC>::Frag fa[TM], fb[TN];
+        for (int i = 0; i < PFI; ++i)
+          direct_load_4((pf_is_b[i] ? b : a) + pf_off[i], lds_address(dump));
+      };
+      // Tile loads by the load waves, prefetch by the prefetch wave.
+      auto issue_step = [&](int step, int stage) {
+        if (!pf_wave) {
+          da.issue(uniform_pointer(gA0 + step * stepA), smem + stage * STAGE_BYTES, wave);
+          db.issue(uniform_pointer(gB0 + step * stepB), smem + stage * STAGE_BYTES + StageA::BYTES, wave);
+        } else {
+          prefetch_step(step + PD);
+        }
+      };
+      // Load waves drain their tile loads before a barrier; the prefetch wave never waits for its
+      // loads inside the loop (nothing reads what they bring).
+      auto step_barrier = [&](bool partial) {
+        if (pf_wave) barrier_after_direct_loads<63>();
+        else if (partial) barrier_after_direct_loads<kInFlight>();
+        else barrier_after_direct_loads<0>();
+      };
+
+      // Prologue: NS-1 stages in flight, wait for the first.
+      int load_stage = 0;  // stage the next issued k-step goes to
+      int load_step = 0;   // k-step the next issue loads
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
-          fa[i] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(tA, wm * WTM + i * 32, kk, lane);
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          fb[j] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(tB, wn * WTN + j * 32, kk, lane);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j) acc[i][j] = mma_atom<EC>(fb[j], fa[i], acc[i][j]);
+      for (int s_ = 0; s_ < NS - 1; ++s_) {
+        if (s_ < nfull) {
+          issue_step(load_step, load_stage);
+          ++load_step;
+          load_stage = load_stage + 1 == NS ? 0 : load_stage + 1;
+        }
       }
-      if (more) {
-        unsigned char* nA = smem + ((kt + 1) & 1) * STAGE_BYTES;
-        sa.store(nA, tid);
-        sb.store(nA + StageA::BYTES, tid);
+      step_barrier(nfull >= NS - 1);
+
+      Frag fa[2][TM], fb[2][TN];
+      load_frags(fa[0], fb[0], smem, 0);
+      int cur_stage = 0;
+      for (int kt = 0; kt < nfull; ++kt) {
+        const unsigned char* cur = smem + cur_stage * STAGE_BYTES;
+        cur_stage = cur_stage + 1 == NS ? 0 : cur_stage + 1;
+        const unsigned char* nxt = smem + cur_stage * STAGE_BYTES;
+        const bool issue = load_step < nfull;
+        if (issue) {
+          // `load_stage` was last read during step kt-1; every wave passed that step's barrier since.
+          issue_step(load_step, load_stage);
+          ++load_step;
+          load_stage = load_stage + 1 == NS ? 0 : load_stage + 1;
+        }
+#pragma unroll
+        for (int kk = 0; kk + 1 < KSTEPS; ++kk) {
+          load_frags(fa[(kk + 1) & 1], fb[(kk + 1) & 1], cur, kk + 1);
+          mma_all(fa[kk & 1], fb[kk & 1]);
+        }
+        // All LDS reads of `cur` are issued. After the barrier the next stage is complete, so its
+        // first fragments are fetched under the MFMAs of this step's last k-atom.
+        step_barrier(issue);
+        if (kt + 1 < nfull) load_frags(fa[0], fb[0], nxt, 0);
+        mma_all(fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1]);
       }
+      // The dump area may still be receiving prefetched bytes: drain before LDS is reused or freed.
+      if (pf_wave) __builtin_amdgcn_s_waitcnt((0 & 15) | (7 << 4) | (15 << 8));
+    }
+    if (tail) {
+      const int kc0 = kc_begin + nfull * BK;
+      StageA::copy(Ab, p.lda, row0, p.m_ext, kc0, kc_end, smem, tid);
+      StageB::copy(Bb, p.ldb, col0, p.n_ext, kc0, kc_end, smem + StageA::BYTES, tid);
       __syncthreads();
+#pragma unroll
+      for (int kk = 0; kk < KSTEPS; ++kk) {
+        Frag fa[TM], fb[TN];
+        load_frags(fa, fb, smem, kk);
+        mma_all(fa, fb);
+      }
     }
 
     // Epilogue. After the swapped MFMA, lane l of atom (i, j) holds C row (l % 32) and, for
@@ -457,10 +675,10 @@ __global__ __launch_bounds__(K::THREADS) void gemm_entry(const GemmParams p) {
   K::run(p, tkx_smem);
 }
 
-#define TKX_VARIANT(MODE, EA, EB, BM, BN, BK, WM, WN)                                           \
-  {                                                                                             \
-    MODE, EA, EB, BM, BN, BK, WM, WN, ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN>::SMEM_BYTES, \
-        reinterpret_cast<const void*>(&::tkx::gemm_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN>>) \
+#define TKX_VARIANT(MODE, EA, EB, BM, BN, BK, WM, WN, NS)                                            \
+  {                                                                                                  \
+    MODE, EA, EB, BM, BN, BK, WM, WN, NS, ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>::SMEM_BYTES, \
+        reinterpret_cast<const void*>(&::tkx::gemm_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>>) \
   }
 
 }  // namespace tkx

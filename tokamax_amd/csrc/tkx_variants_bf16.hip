@@ -2,24 +2,30 @@
 #include "tkx_gemm.hip.h"
 
 namespace tkx {
-#define FWD_DLHS(BM, BN, BK, WM, WN) \
-  TKX_VARIANT(kFwd, kEBF16, kEBF16, BM, BN, BK, WM, WN), TKX_VARIANT(kDlhs, kEBF16, kEBF16, BM, BN, BK, WM, WN)
+#define FWD_DLHS(BM, BN, BK, WM, WN, NS) \
+  TKX_VARIANT(kFwd, kEBF16, kEBF16, BM, BN, BK, WM, WN, NS), TKX_VARIANT(kDlhs, kEBF16, kEBF16, BM, BN, BK, WM, WN, NS)
+#define DRHS(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kDrhs, kEBF16, kEBF16, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
-    FWD_DLHS(256, 256, 64, 2, 2),
-    FWD_DLHS(256, 256, 64, 2, 4),
-    FWD_DLHS(128, 256, 64, 2, 2),
-    FWD_DLHS(128, 256, 64, 2, 4),
-    FWD_DLHS(128, 128, 64, 2, 2),
-    FWD_DLHS(64, 256, 64, 2, 2),
-    FWD_DLHS(64, 128, 64, 2, 2),
-    FWD_DLHS(32, 256, 64, 1, 4),
-    FWD_DLHS(32, 128, 64, 1, 4),
-    TKX_VARIANT(kDrhs, kEBF16, kEBF16, 256, 256, 64, 2, 2),
-    TKX_VARIANT(kDrhs, kEBF16, kEBF16, 256, 256, 64, 2, 4),
-    TKX_VARIANT(kDrhs, kEBF16, kEBF16, 128, 256, 64, 2, 2),
-    TKX_VARIANT(kDrhs, kEBF16, kEBF16, 128, 128, 64, 2, 2),
-    TKX_VARIANT(kDrhs, kEBF16, kEBF16, 64, 128, 64, 2, 2),
+    FWD_DLHS(256, 256, 64, 2, 4, 2),
+    FWD_DLHS(256, 256, 32, 2, 4, 4),
+    FWD_DLHS(256, 256, 64, 2, 2, 2),
+    FWD_DLHS(256, 256, 32, 2, 2, 4),
+    FWD_DLHS(256, 128, 64, 2, 4, 3),
+    FWD_DLHS(128, 256, 64, 2, 4, 3),
+    FWD_DLHS(128, 256, 64, 2, 2, 3),
+    FWD_DLHS(128, 256, 32, 2, 4, 5),
+    FWD_DLHS(128, 128, 64, 2, 2, 4),
+    FWD_DLHS(128, 128, 64, 2, 2, 2),
+    FWD_DLHS(64, 256, 64, 2, 2, 3),
+    FWD_DLHS(64, 128, 64, 2, 2, 4),
+    FWD_DLHS(32, 256, 64, 1, 4, 3),
+    FWD_DLHS(32, 128, 64, 1, 4, 4),
+    DRHS(256, 256, 64, 2, 4, 2),
+    DRHS(256, 256, 32, 2, 4, 4),
+    DRHS(128, 256, 64, 2, 4, 3),
+    DRHS(128, 128, 64, 2, 2, 4),
+    DRHS(64, 128, 64, 2, 2, 4),
 };
 
 const Variant* variants_bf16(int* count) {

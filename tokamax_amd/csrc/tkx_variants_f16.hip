@@ -2,14 +2,15 @@
 #include "tkx_gemm.hip.h"
 
 namespace tkx {
-#define FWD_DLHS(BM, BN, BK, WM, WN) \
-  TKX_VARIANT(kFwd, kEF16, kEF16, BM, BN, BK, WM, WN), TKX_VARIANT(kDlhs, kEF16, kEF16, BM, BN, BK, WM, WN)
+#define FWD_DLHS(BM, BN, BK, WM, WN, NS) \
+  TKX_VARIANT(kFwd, kEF16, kEF16, BM, BN, BK, WM, WN, NS), TKX_VARIANT(kDlhs, kEF16, kEF16, BM, BN, BK, WM, WN, NS)
+#define DRHS(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kDrhs, kEF16, kEF16, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
-    FWD_DLHS(256, 256, 64, 2, 2),
-    FWD_DLHS(128, 128, 64, 2, 2),
-    FWD_DLHS(32, 128, 64, 1, 4),
-    TKX_VARIANT(kDrhs, kEF16, kEF16, 128, 128, 64, 2, 2),
+    FWD_DLHS(256, 256, 32, 2, 4, 4),
+    FWD_DLHS(128, 128, 64, 2, 2, 4),
+    FWD_DLHS(32, 128, 64, 1, 4, 4),
+    DRHS(128, 128, 64, 2, 2, 4),
 };
 
 const Variant* variants_f16(int* count) {

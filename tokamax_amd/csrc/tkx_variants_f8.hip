@@ -2,13 +2,15 @@
 #include "tkx_gemm.hip.h"
 
 namespace tkx {
+#define FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEF8, kEF8, BM, BN, BK, WM, WN, NS)
+
 static const Variant kVariants[] = {
-    TKX_VARIANT(kFwd, kEF8, kEF8, 256, 256, 128, 2, 2),
-    TKX_VARIANT(kFwd, kEF8, kEF8, 256, 256, 128, 2, 4),
-    TKX_VARIANT(kFwd, kEF8, kEF8, 128, 256, 128, 2, 2),
-    TKX_VARIANT(kFwd, kEF8, kEF8, 128, 128, 128, 2, 2),
-    TKX_VARIANT(kFwd, kEF8, kEF8, 64, 128, 128, 2, 2),
-    TKX_VARIANT(kFwd, kEF8, kEF8, 32, 128, 128, 1, 4),
+    FWD(256, 256, 128, 2, 4, 2),
+    FWD(256, 256, 128, 2, 2, 2),
+    FWD(128, 256, 128, 2, 4, 3),
+    FWD(128, 128, 128, 2, 2, 4),
+    FWD(64, 128, 128, 2, 2, 4),
+    FWD(32, 128, 128, 1, 4, 4),
 };
 
 const Variant* variants_f8(int* count) {

@@ -3,12 +3,15 @@
 #include "tkx_gemm.hip.h"
 
 namespace tkx {
+#define FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEBF16, kEI8, BM, BN, BK, WM, WN, NS)
+
 static const Variant kVariants[] = {
-    TKX_VARIANT(kFwd, kEBF16, kEI8, 128, 128, 64, 2, 2),
-    TKX_VARIANT(kFwd, kEBF16, kEI8, 64, 128, 64, 2, 2),
-    TKX_VARIANT(kFwd, kEBF16, kEI8, 32, 128, 64, 1, 4),
-    TKX_VARIANT(kFwd, kEBF16, kEI8, 32, 256, 64, 1, 4),
-    TKX_VARIANT(kFwd, kEBF16, kEI8, 32, 128, 128, 1, 4),
+    FWD(128, 128, 64, 2, 2, 4),
+    FWD(64, 128, 64, 2, 2, 4),
+    FWD(32, 128, 64, 1, 4, 4),
+    FWD(32, 256, 64, 1, 4, 4),
+    FWD(32, 128, 128, 1, 4, 4),
+    FWD(32, 128, 128, 1, 4, 2),
 };
 
 const Variant* variants_i8w(int* count) {

@@ -33,7 +33,7 @@ GroupSizes = base.GroupSizes
 class Config:
   """Tunables of the hip kernels; counterpart of pallas_mosaic_gpu_common.py:45-73.
 
-  (block_m, block_n, block_k, waves_m, waves_n) selects a precompiled kernel variant;
+  (block_m, block_n, block_k, waves_m, waves_n, num_stages) selects a precompiled kernel variant;
   `grid_tile_width` m-tasks share one n-panel of rhs in launch order (L2 reuse);
   `align_tile` is the row alignment of task starts (the reference's `align_tile`, default 8).
   """
@@ -43,6 +43,7 @@ class Config:
   block_k: int
   waves_m: int = 2
   waves_n: int = 2
+  num_stages: int = 2
   grid_tile_width: int = 8
   align_tile: int = 8
 
@@ -56,7 +57,7 @@ class Config:
 
   def to_kernel_config(self) -> hip_ops.KernelConfig:
     return hip_ops.KernelConfig(self.block_m, self.block_n, self.block_k, self.waves_m, self.waves_n,
-                                self.grid_tile_width, self.align_tile)
+                                self.num_stages, self.grid_tile_width, self.align_tile)
 
 
 _ACTIVATION_NAMES = {
@@ -82,12 +83,12 @@ def _dtype_of(x) -> torch.dtype:
 
 @functools.lru_cache(maxsize=None)
 def _variant_table():
-  """{(mode, lhs dtype code, rhs dtype code): [(bm, bn, bk, wm, wn), ...]} from the library."""
+  """{(mode, lhs dtype code, rhs dtype code): [(bm, bn, bk, wm, wn, stages), ...]} from the library."""
   table: dict = {}
   for kind in (0, 1):
     for v in _lib.variants(kind):
       key = (v["mode"], v["lhs_dtype"], v["rhs_dtype"])
-      table.setdefault(key, []).append((v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"]))
+      table.setdefault(key, []).append((v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"], v["num_stages"]))
   return table
 
 
@@ -254,19 +255,21 @@ class HipRaggedDot(base.RaggedDot):
     want_n = 256 if cols >= 2048 else 128
 
     def score(v):
-      bm, bn, bk, wm, wn = v
-      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -bk)
+      bm, bn, bk, wm, wn, ns = v
+      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -ns, -bk)
 
-    bm, bn, bk, wm, wn = min(usable, key=score)
-    return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, grid_tile_width=8, align_tile=8)
+    bm, bn, bk, wm, wn, ns = min(usable, key=score)
+    return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns, grid_tile_width=8,
+                  align_tile=8)
 
   def _get_autotuning_configs(self, ba: op.BoundArguments) -> set[Config]:
     mode, key, _, _, _, _ = self._problem(ba)
     configs = set()
-    for bm, bn, bk, wm, wn in _variant_table().get(key, []):
+    for bm, bn, bk, wm, wn, ns in _variant_table().get(key, []):
       widths = (1,) if mode == 2 else (1, 2, 4, 8, 16)
       for w in widths:
-        configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, grid_tile_width=w))
+        configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns,
+                           grid_tile_width=w))
     return configs
 
   def supported_on(self, device: torch.device) -> bool:

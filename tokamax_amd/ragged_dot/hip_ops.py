@@ -39,12 +39,13 @@ class KernelConfig:
   block_k: int
   waves_m: int
   waves_n: int
+  num_stages: int = 2
   grid_tile_width: int = 1
   align_tile: int = 8
 
   def to_c(self) -> _lib.TkxConfig:
     return _lib.TkxConfig(self.block_m, self.block_n, self.block_k, self.waves_m, self.waves_n,
-                          self.grid_tile_width, self.align_tile, 0)
+                          self.grid_tile_width, self.align_tile, self.num_stages)
 
 
 def _require_cuda(*tensors):
