@@ -61,7 +61,8 @@ typedef struct TkxConfig {
   int32_t block_k;         /* contraction elements per LDS stage */
   int32_t waves_m;         /* wavefronts along m in a workgroup */
   int32_t waves_n;         /* wavefronts along n in a workgroup */
-  int32_t grid_tile_width; /* m-tasks that share an n-panel in launch order (L2 reuse) */
+  int32_t grid_tile_width; /* m-tasks that share an n-panel in launch order (L2 reuse); unused by the
+                              small-m int8 kernel (block_m == 16) */
   int32_t align_tile;      /* task starts are aligned down to this many rows (reference default 8) */
   int32_t num_stages;      /* LDS stages of block_k contraction elements kept in flight */
 } TkxConfig;

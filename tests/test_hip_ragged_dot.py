@@ -295,6 +295,8 @@ def test_every_kernel_variant_through_c_abi(v, device):
   """Each compiled tile shape, called through the C ABI, on ragged groups with an empty one and a tail."""
   rng = np.random.default_rng(v["block_m"] * 7 + v["block_n"] + v["mode"])
   G, m, k, n = 6, 640, 256, 384
+  if v["block_m"] == 16:
+    k = 1024  # the streaming small-m kernel splits k over 4 waves x 8 steps of 32
   gs = np.array([100, 0, 257, 9, 130, 80], np.int32)  # sum 576 < m
   gst = torch.tensor(gs, device=device)
   cfg = hip_ops.KernelConfig(v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"], v["num_stages"],
@@ -329,6 +331,43 @@ def test_every_kernel_variant_through_c_abi(v, device):
   want = O.ragged_dot(lhs_f, rhs_f, gs, O.TRANS_RHS if v["mode"] == 1 else O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
   _check(out, want, tol)
   assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+
+
+@pytest.mark.parametrize("depth", [2, 4, 8])
+@pytest.mark.parametrize("case", ["ragged", "two_chunks", "all_empty", "one_big_group", "first_and_last_empty"])
+def test_small_m_int8_kernel_edges(case, depth, device):
+  """The streaming small-m kernel: empty groups anywhere, more than 64 groups, groups taller than one
+  16-row pass, a column count that is not a multiple of its 128-column tile, and a zero tail."""
+  rng = np.random.default_rng(len(case) + depth)
+  k, n = 1024, 208
+  if case == "ragged":
+    gs = np.array([3, 0, 0, 17, 1, 0, 16, 2], np.int32)
+  elif case == "two_chunks":
+    gs = rng.integers(0, 4, 70).astype(np.int32)
+    gs[[0, 63, 64, 69]] = [0, 2, 0, 5]
+  elif case == "all_empty":
+    gs = np.zeros(5, np.int32)
+  elif case == "one_big_group":
+    gs = np.array([0, 45, 0], np.int32)
+  else:
+    gs = np.array([0, 4, 9, 0], np.int32)
+  G, m = len(gs), int(gs.sum()) + 11
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  rhs = torch.tensor(rng.integers(-128, 128, (G, k, n)).astype(np.int8), device=device)
+  scale = torch.tensor((np.abs(rng.normal(0, 0.01, (G, 1, n))) + 1e-3).astype(np.float32), device=device)
+  cfg = hip_ops.KernelConfig(16, 128, 32, 1, 4, depth)
+  out = hip_ops.ragged_dot_fwd(lhs, rhs, torch.tensor(gs, device=device), config=cfg, out_dtype=torch.float32,
+                               rhs_scale=scale)
+  want = O.ragged_dot(_np(lhs), O.dequantize(rhs.cpu().numpy(), _np(scale)), gs, O.DEFAULT, acc_dtype=np.float64,
+                      out_dtype="f64")
+  _check(out, want, 1e-5)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  # bf16 output, and the same bits on a second run (fixed reduction order)
+  out16 = hip_ops.ragged_dot_fwd(lhs, rhs, torch.tensor(gs, device=device), config=cfg, out_dtype=torch.bfloat16,
+                                 rhs_scale=scale)
+  assert torch.equal(out16, out.to(torch.bfloat16))
+  assert torch.equal(out, hip_ops.ragged_dot_fwd(lhs, rhs, torch.tensor(gs, device=device), config=cfg,
+                                                 out_dtype=torch.float32, rhs_scale=scale))
 
 
 def test_unsupported_inputs_are_declined(device):

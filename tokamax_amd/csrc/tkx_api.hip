@@ -30,6 +30,11 @@ struct Registry {
     v = variants_f32(&n);  all.insert(all.end(), v, v + n);
     v = variants_f8(&n);   all.insert(all.end(), v, v + n);
     v = variants_i8w(&n);  all.insert(all.end(), v, v + n);
+    // The streaming small-m kernel for int8 weights is not a tile variant of the GEMM template;
+    // it is listed here (fn == nullptr) so that configs can name it.
+    all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, 2, 0, nullptr});
+    all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, 4, 0, nullptr});
+    all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, 8, 0, nullptr});
   }
 };
 
@@ -156,6 +161,17 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   if (((uintptr_t)lhs | (uintptr_t)rhs | (uintptr_t)out | (uintptr_t)workspace) % 16 != 0 ||
       (rhs_scale && (uintptr_t)rhs_scale % 16 != 0))
     return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
+
+  if (v->fn == nullptr) {
+    // Streaming decode kernel: one launch, no schedule.
+    if (lhs_scale != nullptr) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no lhs scale");
+    if (!decode_i8w_supported(m, k, n, num_groups))
+      return set_error(TKX_ERR_UNSUPPORTED,
+                       "decode kernel needs k %% 1024 == 0, n %% 8 == 0 and at most 1024 groups (k=%lld n=%lld G=%lld)",
+                       (long long)k, (long long)n, (long long)num_groups);
+    return launch_decode_i8w(lhs, rhs, rhs_scale, group_sizes, out, m, k, n, num_groups, out_dtype, activation,
+                             c.num_stages, stream);
+  }
 
   const WsLayout L = ws_layout(m, num_groups, c.block_m);
   int32_t st = launch_schedule(group_sizes, num_groups, m, c.block_m, c.align_tile, static_cast<int32_t*>(workspace), L, stream);

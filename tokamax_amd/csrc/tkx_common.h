@@ -82,6 +82,13 @@ struct Variant {
   const void* fn;  // __global__ void (*)(GemmParams)
 };
 
+// ---- decode (small-m, int8 weights) ------------------------------------------------------------
+constexpr int32_t kDecodeBlockM = 16, kDecodeBlockN = 128, kDecodeBlockK = 32, kDecodeWaves = 4, kDecodeStages = 4;
+bool decode_i8w_supported(int64_t m, int64_t k, int64_t n, int64_t G);
+int32_t launch_decode_i8w(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
+                          int64_t m, int64_t k, int64_t n, int64_t G, int32_t out_dtype, int32_t activation,
+                          int32_t depth, hipStream_t stream);
+
 // Each dtype family registers its variants from its own translation unit.
 const Variant* variants_bf16(int* count);
 const Variant* variants_f16(int* count);

@@ -1,0 +1,353 @@
+// Small-m ("decode") ragged dot with int8 weights: bf16 lhs [m,k] x int8 rhs [G,k,n], f32 scales [G,n].
+//
+// This regime is bound by HBM: every touched expert's [k,n] weight panel is read once, and a group
+// has a handful of rows. The kernel is built around streaming those panels:
+//   * one launch, no scheduler kernel: every workgroup reads group_sizes itself, the workgroups are
+//     dealt to the non-empty groups in order, and the surplus ones exit at once (an empty group's
+//     weights are never read);
+//   * a workgroup owns (group, 128 output columns); its 4 waves split the contraction and each
+//     streams its own [k/4, 128] slice of the panel with full 128-byte rows, several steps of
+//     global loads in flight in registers; no workgroup barrier and no LDS inside the loop;
+//   * no transposition is needed: the contraction index of an MFMA is only a label, so lane
+//     (i, q) loads 8 bytes (columns 8i..8i+7) from each of the 8 rows 8q..8q+7 of a 32-row step and
+//     feeds MFMA j (j = 0..7) with byte j of those 8 loads, i.e. 8 contraction values of column
+//     8i+j.  MFMA j therefore produces the output columns {8i+j}; the lhs fragment of lane (r, q) is
+//     lhs[r][8q..8q+7] of the same step, one 16-byte load;
+//   * int8 is widened to bf16 exactly and goes through the 16x16x32 bf16 MFMA with f32 accumulation;
+//   * the four partial tiles are added in a fixed order through LDS (deterministic), scaled per
+//     (group, column), and rows past the group's end are never written.
+#include "tkx_common.h"
+#include "tkx_gemm.hip.h"
+
+namespace tkx {
+namespace {
+
+constexpr int kDecBN = 128;    // output columns per workgroup
+constexpr int kDecWaves = 4;   // waves per workgroup; each takes k / 4 of the contraction
+constexpr int kDecKS = 32;     // contraction elements per step (one 16x16x32 MFMA deep)
+constexpr int kDecRows = 16;   // lhs rows per pass
+constexpr int kDecThreads = kDecWaves * 64;
+constexpr int kDecMaxGroups = 1024;  // group sizes are staged in LDS
+
+struct DecodeParams {
+  const __bf16* lhs;
+  const signed char* rhs;
+  const float* scale;
+  const int32_t* group_sizes;
+  void* out;
+  int32_t m, k, n, num_groups, n_tiles, out_dtype, activation;
+};
+
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+// Buffer loads: wave-uniform descriptor (base + byte count; reads past the end return zero), a
+// 32-bit lane offset and a wave-uniform 32-bit step offset. No 64-bit address arithmetic in VGPRs.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const void* base, uint32_t bytes) {
+  const unsigned char* b = uniform_pointer(static_cast<const unsigned char*>(base));
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(b), 0, __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000);
+}
+// Weights are read exactly once: the non-temporal hint keeps them from displacing reusable lines
+// in the caches, which measurably raises the streaming rate (about 8% on this kernel).
+constexpr int kStreamingLoad = 2;  // cache-policy operand of the buffer load: bit 1 = nt
+__device__ __forceinline__ i32x2 buffer_load_8(__amdgpu_buffer_rsrc_t r, uint32_t lane_offset, uint32_t uniform_offset) {
+  return __builtin_bit_cast(i32x2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)lane_offset, (int)uniform_offset, kStreamingLoad));
+}
+__device__ __forceinline__ i32x4 buffer_load_16(__amdgpu_buffer_rsrc_t r, uint32_t lane_offset, uint32_t uniform_offset) {
+  return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_offset, (int)uniform_offset, 0));
+}
+
+// Sign-extended byte B of a dword -> f32, one SDWA instruction.
+template <int B>
+__device__ __forceinline__ unsigned i8_to_f32_bits(int w) {
+  unsigned f;
+  if constexpr (B == 0) asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(f) : "v"(w));
+  if constexpr (B == 1) asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(f) : "v"(w));
+  if constexpr (B == 2) asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(f) : "v"(w));
+  if constexpr (B == 3) asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(f) : "v"(w));
+  return f;
+}
+
+// Byte J of each of 8 loaded 8-byte rows -> bf16 x8 (exact: |v| <= 128 fits the significand). The
+// upper halves of two f32 are the two bf16, packed with one byte permute.
+template <int J>
+__device__ __forceinline__ bf16x8 column_to_bf16x8(const i32x2 (&rows)[8]) {
+  i32x4 out;
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    const unsigned f0 = i8_to_f32_bits<(J & 3)>(rows[2 * h][J >> 2]);
+    const unsigned f1 = i8_to_f32_bits<(J & 3)>(rows[2 * h + 1][J >> 2]);
+    // v_perm_b32 picks bytes from {first operand: bytes 7..4, second operand: bytes 3..0}.
+    out[h] = (int)__builtin_amdgcn_perm(f1, f0, 0x07060302u);
+  }
+  return __builtin_bit_cast(bf16x8, out);
+}
+
+template <int kDecDepth, int kMinWgs>
+__global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_i8w_kernel(const DecodeParams p) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  __shared__ int s_size[kDecMaxGroups];
+  __shared__ int s_cnt[kDecMaxGroups / 64], s_rows[kDecMaxGroups / 64];
+  __shared__ unsigned long long s_mask[kDecMaxGroups / 64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // The grid is G x n_tiles, but workgroups are handed to the non-empty groups in order: workgroup
+  // w serves the (w / n_tiles)-th non-empty group. The busy workgroups are then the first ones of
+  // the grid, which spreads them evenly over the XCDs and CUs however the empty groups fall; the
+  // rest exit after reading group_sizes. An empty group's weights are never touched.
+  const int t = blockIdx.x / p.n_tiles, nt = blockIdx.x - t * p.n_tiles;
+  const int col0 = nt * kDecBN;
+
+  // Every workgroup reads all group sizes once (G <= 1024): 64 groups per wave pass.
+  const int chunks = (p.num_groups + 63) >> 6;
+  for (int c = wave; c < chunks; c += kDecWaves) {
+    const int j = 64 * c + lane;
+    const int sz = j < p.num_groups ? max(p.group_sizes[j], 0) : 0;
+    s_size[j] = sz;
+    const unsigned long long mask = __ballot(sz > 0);
+    int rows = sz;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) rows += __shfl_xor(rows, off);
+    if (lane == 0) {
+      s_mask[c] = mask;
+      s_cnt[c] = __popcll(mask);
+      s_rows[c] = rows;
+    }
+  }
+  __syncthreads();
+  // Locate the t-th non-empty group: its 64-group chunk, then its bit inside the chunk's mask.
+  int chunk = -1, cnt_before = 0, rows_before = 0, total_cnt = 0, total_rows = 0;
+  for (int c = 0; c < chunks; ++c) {
+    const int cnt = s_cnt[c], rows = s_rows[c];
+    if (chunk < 0 && total_cnt + cnt > t) {
+      chunk = c;
+      cnt_before = total_cnt;
+      rows_before = total_rows;
+    }
+    total_cnt += cnt;
+    total_rows += rows;
+  }
+  // Rows past the last group belong to no group; the workgroups of the last non-empty group (or
+  // of slot 0 when every group is empty) zero their columns of those rows.
+  const bool zeroes_tail = t == max(total_cnt, 1) - 1;
+  if (chunk < 0 && !zeroes_tail) return;
+  int g = 0, start = 0, size = 0;
+  if (chunk >= 0) {
+    const unsigned long long mask = s_mask[chunk];
+    const int r = t - cnt_before;
+    const bool mine = ((mask >> lane) & 1ull) != 0 && __popcll(mask & ((1ull << lane) - 1ull)) == r;
+    const int bit = __builtin_ctzll(__ballot(mine));
+    g = __builtin_amdgcn_readfirstlane(64 * chunk + bit);
+    int rows = lane < bit ? s_size[64 * chunk + lane] : 0;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) rows += __shfl_xor(rows, off);
+    start = __builtin_amdgcn_readfirstlane(rows_before + rows);
+    size = __builtin_amdgcn_readfirstlane(s_size[g]);
+  }
+  const int end = min(start + size, p.m);
+  const int esz = p.out_dtype == TKX_F32 ? 4 : 2;
+
+  const int kw = p.k / kDecWaves;      // contraction slice of this wave
+  const int k_begin = wave * kw;
+  const int steps = kw / kDecKS;       // multiple of kDecDepth (checked on the host)
+  const signed char* wbase = p.rhs + ((int64_t)g * p.k + k_begin) * p.n;
+  // B loads: lane (i = lane % 16, q = lane / 16) -> rows 8q + e (e = 0..7), columns col0 + 8i .. 8i+7,
+  // clamped at the last 8 columns (n is a multiple of 8; clamped lanes feed columns that are never stored).
+  const int li = lane & 15, lq = lane >> 4;
+  int colb = col0 + li * 8;
+  colb = colb < p.n - 8 ? colb : p.n - 8;
+  uint32_t boff[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) boff[e] = (uint32_t)((8 * lq + e) * p.n + colb);
+
+  i32x2 breg[kDecDepth][8];
+  i32x4 areg[kDecDepth];
+  // Nothing looks at a loaded value before its step comes up, so the only waits are the per-step
+  // vmcnt of the oldest group. (A workgroup without a group gets an empty buffer: its loads read zero.)
+  const __amdgpu_buffer_rsrc_t wbuf = buffer_of(wbase, chunk >= 0 ? (uint32_t)kw * (uint32_t)p.n : 0u);
+  const uint32_t step_bytes = (uint32_t)(kDecKS * p.n);
+  auto issue_b = [&](int slot, int step) {
+    const uint32_t so = (uint32_t)__builtin_amdgcn_readfirstlane((int)(step * step_bytes));
+#pragma unroll
+    for (int e = 0; e < 8; ++e) breg[slot][e] = buffer_load_8(wbuf, boff[e], so);
+  };
+#pragma unroll
+  for (int d = 0; d < kDecDepth; ++d) {
+    issue_b(d, d);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // Per-column scales of this thread's 8 epilogue columns, fetched now so that the epilogue does
+  // not end on a dependent memory round trip.
+  f32x4_t scale_lo = {1.f, 1.f, 1.f, 1.f}, scale_hi = {1.f, 1.f, 1.f, 1.f};
+  {
+    const int col = col0 + (tid & 15) * 8;
+    if (p.scale != nullptr && chunk >= 0 && col + 8 <= p.n) {
+      const float* sc = p.scale + (int64_t)g * p.n + col;
+      scale_lo = *reinterpret_cast<const f32x4_t*>(sc);
+      scale_hi = *reinterpret_cast<const f32x4_t*>(sc + 4);
+    }
+  }
+
+  if (zeroes_tail) {
+    const int tail = min(total_rows, p.m);
+    const int ncol = min(kDecBN, p.n - col0);
+    const int pieces = ncol * esz / 16;  // 16-byte pieces per row
+    unsigned char* c = reinterpret_cast<unsigned char*>(p.out);
+    const i32x4 z = {0, 0, 0, 0};
+    for (int idx = tid; idx < (p.m - tail) * pieces; idx += kDecThreads) {
+      const int r = tail + idx / pieces, ch = idx % pieces;
+      *reinterpret_cast<i32x4*>(c + ((int64_t)r * p.n + col0) * esz + ch * 16) = z;
+    }
+  }
+  if (end <= start) return;
+
+  // lhs rows of this group as one buffer: rows at or past the group's end read as zero.
+  const __amdgpu_buffer_rsrc_t abuf = buffer_of(p.lhs + (int64_t)start * p.k, (uint32_t)(end - start) * (uint32_t)p.k * 2u);
+
+  for (int rb = start; rb < end; rb += kDecRows) {
+    // A fragments: lane (i, q) holds lhs[rb + i][k + 8q .. 8q+7].
+    const uint32_t aoff = (uint32_t)((rb + li - start) * p.k + k_begin + 8 * lq) * 2u;
+    auto issue_a = [&](int slot, int step) { areg[slot] = buffer_load_16(abuf, aoff, (uint32_t)(step * (kDecKS * 2))); };
+
+    f32x4_t acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+    for (int d = 0; d < kDecDepth; ++d) {
+      issue_a(d, d);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // One block = kDecDepth steps, each consuming its slot and refilling it kDecDepth steps ahead.
+    // The first block is peeled off the loop: it consumes loads in the order the prologue issued
+    // them (all weight steps, then all lhs steps), while its refills establish the steady-state
+    // order (weights, lhs, weights, lhs, ...) that the loop then sees on entry and on its back edge,
+    // so every wait inside the loop is a partial vmcnt that leaves the younger steps in flight.
+    auto block = [&](int s0) {
+#pragma unroll
+      for (int d = 0; d < kDecDepth; ++d) {
+        const int s = s0 + d;
+        const bf16x8 afrag = __builtin_bit_cast(bf16x8, areg[d]);
+        // MFMA j contracts this step's 32 rows for the columns {8i + j}; operands are swapped, so a
+        // lane ends up with one lhs row and the weight-column indices 4q..4q+3.
+        bf16x8 lo[4], hi[4];
+        lo[0] = column_to_bf16x8<0>(breg[d]);
+        lo[1] = column_to_bf16x8<1>(breg[d]);
+        lo[2] = column_to_bf16x8<2>(breg[d]);
+        lo[3] = column_to_bf16x8<3>(breg[d]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lo[j], afrag, acc[j], 0, 0, 0);
+        hi[0] = column_to_bf16x8<4>(breg[d]);
+        hi[1] = column_to_bf16x8<5>(breg[d]);
+        hi[2] = column_to_bf16x8<6>(breg[d]);
+        hi[3] = column_to_bf16x8<7>(breg[d]);
+        // Refill unconditionally: past the wave's slice the weight buffer reads as zero without
+        // touching memory, and a uniform loop body keeps the waits partial. The scheduling fences
+        // keep the compiler from sinking the loads to the end of the block, which would collapse
+        // the pipeline to a single step in flight.
+        __builtin_amdgcn_sched_barrier(0);
+        issue_b(d, s + kDecDepth);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi[j], afrag, acc[4 + j], 0, 0, 0);
+        // The lhs refill goes into the registers the MFMAs above read, so it follows them.
+        __builtin_amdgcn_sched_barrier(0);
+        issue_a(d, s + kDecDepth);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    block(0);
+#pragma unroll 1
+    for (int s0 = kDecDepth; s0 < steps; s0 += kDecDepth) block(s0);
+
+    // Cross-wave reduction in a fixed order. acc[j][r] of lane (i, q) is row i, column 32 q + 8 r + j.
+    float* part = reinterpret_cast<float*>(smem) + wave * (kDecRows * kDecBN);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float* dst = part + li * kDecBN + 32 * lq + 8 * r;
+      *reinterpret_cast<f32x4_t*>(dst) = (f32x4_t){acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+      *reinterpret_cast<f32x4_t*>(dst + 4) = (f32x4_t){acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
+    }
+    __syncthreads();
+    {
+      const int r = tid >> 4, c8 = (tid & 15) * 8;  // 16 rows x 16 column octets = 256 threads
+      const int row = rb + r, col = col0 + c8;
+      if (row < end && col + 8 <= p.n) {
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = 0.f;
+#pragma unroll
+        for (int w = 0; w < kDecWaves; ++w) {
+          const float* src = reinterpret_cast<const float*>(smem) + w * (kDecRows * kDecBN) + r * kDecBN + c8;
+          const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(src), hi = *reinterpret_cast<const f32x4_t*>(src + 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[e] += lo[e];
+            v[4 + e] += hi[e];
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] *= scale_lo[e];
+          v[4 + e] *= scale_hi[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = apply_activation(v[e], p.activation);
+        const int64_t idx = (int64_t)row * p.n + col;
+        store4(p.out, idx, (f32x4){v[0], v[1], v[2], v[3]}, p.out_dtype);
+        store4(p.out, idx + 4, (f32x4){v[4], v[5], v[6], v[7]}, p.out_dtype);
+      }
+    }
+    __syncthreads();  // partials are consumed before the next pass overwrites them
+    if (rb + kDecRows < end) {
+      // Groups with more than 16 rows stream their panel again for the next 16.
+#pragma unroll
+      for (int d = 0; d < kDecDepth; ++d) {
+        issue_b(d, d);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+}
+
+}  // namespace
+
+// Whether the decode kernel can run this problem (else the caller uses the tiled kernel).
+bool decode_i8w_supported(int64_t m, int64_t k, int64_t n, int64_t G) {
+  (void)m;
+  if (G > kDecMaxGroups || (k / kDecWaves) * n >= (1LL << 31)) return false;
+  return k % (kDecWaves * kDecKS * 8) == 0 && n % 8 == 0 && n >= 8;
+}
+
+int32_t launch_decode_i8w(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
+                          int64_t m, int64_t k, int64_t n, int64_t G, int32_t out_dtype, int32_t activation,
+                          int32_t depth, hipStream_t stream) {
+  DecodeParams p;
+  p.lhs = static_cast<const __bf16*>(lhs);
+  p.rhs = static_cast<const signed char*>(rhs);
+  p.scale = scale;
+  p.group_sizes = group_sizes;
+  p.out = out;
+  p.m = (int32_t)m;
+  p.k = (int32_t)k;
+  p.n = (int32_t)n;
+  p.num_groups = (int32_t)G;
+  p.n_tiles = (int32_t)((n + kDecBN - 1) / kDecBN);
+  p.out_dtype = out_dtype;
+  p.activation = activation;
+  // Dynamic LDS holds only the four partial tiles of the cross-wave reduction (4 x 16 x 128 f32 = 32 KB).
+  const size_t smem = kDecWaves * kDecRows * kDecBN * 4;
+  const int64_t grid = G * p.n_tiles;
+  if (grid > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "too many workgroups");
+  // `depth` = steps of loads in flight per wave; deeper pipelines need more registers and allow
+  // fewer waves per CU.
+  const void* fn = depth <= 2   ? reinterpret_cast<const void*>(&decode_i8w_kernel<2, 4>)
+                   : depth <= 4 ? reinterpret_cast<const void*>(&decode_i8w_kernel<4, 3>)
+                                : reinterpret_cast<const void*>(&decode_i8w_kernel<8, 2>);
+  DecodeParams params = p;
+  void* args[] = {&params};
+  TKX_HIP_CHECK(hipLaunchKernel(fn, dim3((unsigned)grid), dim3(kDecThreads), args, smem, stream));
+  return TKX_OK;
+}
+
+}  // namespace tkx

@@ -109,7 +109,9 @@ __device__ __forceinline__ i32x4 lds_read_b128(const unsigned char* base, int of
   return *reinterpret_cast<const i32x4*>(base + off);
 }
 
-// int8 x8 (two dwords) -> bf16 x8 (exact: |v| <= 128 fits the 8-bit significand of bf16).
+// int8 x8 (two dwords) -> bf16 x8 (exact: |v| <= 128 fits the 8-bit significand of bf16). Each byte is
+// sign-extended and converted to f32 (one SDWA instruction); the upper halves of two f32 are the
+// two bf16 and are packed with one byte permute.
 __device__ __forceinline__ i32x4 i8x8_to_bf16x8(i32x2 v) {
   i32x4 out;
 #pragma unroll
@@ -121,8 +123,9 @@ __device__ __forceinline__ i32x4 i8x8_to_bf16x8(i32x2 v) {
     const float f3 = (float)(signed char)((w >> 24) & 0xff);
     const unsigned u0 = __builtin_bit_cast(unsigned, f0), u1 = __builtin_bit_cast(unsigned, f1);
     const unsigned u2 = __builtin_bit_cast(unsigned, f2), u3 = __builtin_bit_cast(unsigned, f3);
-    out[2 * h] = (int)((u0 >> 16) | (u1 & 0xffff0000u));
-    out[2 * h + 1] = (int)((u2 >> 16) | (u3 & 0xffff0000u));
+    // v_perm_b32 picks bytes from {first operand: bytes 7..4, second operand: bytes 3..0}.
+    out[2 * h] = (int)__builtin_amdgcn_perm(u1, u0, 0x07060302u);
+    out[2 * h + 1] = (int)__builtin_amdgcn_perm(u3, u2, 0x07060302u);
   }
   return out;
 }
@@ -551,6 +554,9 @@ struct GemmKernel {
       const unsigned char* const gA0 = gA;
       const unsigned char* const gB0 = gB;
       auto prefetch_step = [&](int step) {
+#if defined(TKX_ABLATE) && (TKX_ABLATE & 16)
+        return;
+#endif
         if (step >= nfull) return;
         const unsigned char* a = gA0 + step * stepA;
         const unsigned char* b = gB0 + step * stepB;

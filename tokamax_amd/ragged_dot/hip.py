@@ -248,25 +248,31 @@ class HipRaggedDot(base.RaggedDot):
     if not variants:
       raise NotImplementedError(f"No hip kernel for dtypes/mode {key}.")
     usable = list(variants)
+    if key[2] == _lib.TKX_I8:
+      # The streaming small-m kernel (block_m == 16) needs k % 1024 == 0, n % 8 == 0 and G <= 1024.
+      usable = [v for v in usable
+                if v[0] != 16 or (contraction % 1024 == 0 and cols % 8 == 0 and num_groups <= 1024)]
     # Rows per group decide the m-tile: a tile much taller than a group wastes MFMA work on rows
     # that are masked out at the store; a short tile re-reads the weights more often.
     rows_per_group = rows / max(num_groups, 1) if mode != 2 else rows
-    want_m = 256 if rows_per_group >= 1024 else 128 if rows_per_group >= 192 else 64 if rows_per_group >= 48 else 32
+    want_m = (256 if rows_per_group >= 1024 else 128 if rows_per_group >= 192 else 64 if rows_per_group >= 48
+              else 32 if rows_per_group > 16 else 16)
     want_n = 256 if cols >= 2048 else 128
 
     def score(v):
       bm, bn, bk, wm, wn, ns = v
-      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -ns, -bk)
+      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -bk, ns)
 
     bm, bn, bk, wm, wn, ns = min(usable, key=score)
-    return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns, grid_tile_width=8,
+    width = 1 if (bm == 16 and key[2] == _lib.TKX_I8) else 8  # the small-m int8 kernel has no tile order to tune
+    return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns, grid_tile_width=width,
                   align_tile=8)
 
   def _get_autotuning_configs(self, ba: op.BoundArguments) -> set[Config]:
     mode, key, _, _, _, _ = self._problem(ba)
     configs = set()
     for bm, bn, bk, wm, wn, ns in _variant_table().get(key, []):
-      widths = (1,) if mode == 2 else (1, 2, 4, 8, 16)
+      widths = (1,) if (mode == 2 or (bm == 16 and key[2] == _lib.TKX_I8)) else (1, 2, 4, 8, 16)
       for w in widths:
         configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns,
                            grid_tile_width=w))
