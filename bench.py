@@ -1,14 +1,20 @@
 """Benchmark of the hip ragged dot on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--calibration-copy]
 
 Prints ONE JSON line. A step is one pass of the hot path (scheduler kernel + grouped-GEMM kernel)
 over one seeded synthetic batch that is already resident in HBM. The headline workload is the
 Mixtral-8x7B-shaped prefill grouped GEMM (m=16384, k=4096, n=14336, G=8, bf16, top-2 router group
-sizes); `value` is its throughput in TFLOP/s with FLOPs = 2 * sum(group_sizes) * k * n. The other
-measured configurations (DeepSeek-V3 shape, int8-weight decode, fp8, bf16 VJP) are reported under
-"extras" with their own roofline figures. `cpu_baseline` times the CPU oracle (per-group f32 GEMM
-through NumPy's BLAS) on this box's host cores; it is a reported baseline, not the thing measured.
+sizes); `value` is its throughput in TFLOP/s with FLOPs = 2 * sum(group_sizes) * k * n.
+
+`roofline` describes the dominant kernel of a step, the grouped GEMM: its average launch duration is
+the HIP-event time of a step (events recorded on the launch stream) minus the separately measured
+duration of the scheduler kernel, the only other kernel in a step. The other measured
+configurations (DeepSeek-V3 shape, int8-weight decode, fp8, bf16 VJP) are reported under "extras"
+with their own roofline figures; the decode kernel runs for tens of microseconds, less than the
+host needs to issue a launch, so it is timed as a HIP graph of back-to-back launches over rotating
+weight copies. `cpu_baseline` times the CPU oracle (per-group f32 GEMM through NumPy's BLAS) on this
+box's host cores; it is a reported baseline, not the thing measured.
 """
 
 from __future__ import annotations
@@ -30,6 +36,14 @@ if ROOT not in sys.path:
 # MI355X published peaks (dense).
 PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "f32": 157.3}
 PEAK_HBM_GBS = 8000.0
+
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script, each scaled by what the same counter reads for a copy kernel of known size; None
+# where no counter run has been made for the current kernel.
+MEASURED_TRAFFIC_BYTES = {
+    "mixtral": 4.460e9,  # 256x256x64 kernel: 3.968e9 read + 0.492e9 written (algorithmic: 1.543e9)
+    "decode": 1.803e8,   # streaming int8 kernel: 1.799e8 read + 3.9e5 written (algorithmic: 1.748e8)
+}
 
 
 def _time_steps(fn, steps, warmup, stream):
@@ -53,15 +67,43 @@ def _time_steps(fn, steps, warmup, stream):
   return total, per, wall_ms
 
 
-def _roofline(bound, flops, nbytes, ms, dtype_key):
+def _roofline(bound, flops, nbytes, ms, dtype_key, traffic=None):
+  """Roofline record of one kernel launch of `ms` milliseconds; `traffic` = measured HBM bytes per launch."""
   if bound == "mfma":
     achieved = flops / ms / 1e9
     peak = PEAK_TFLOPS[dtype_key]
     return dict(bound="mfma", achieved=round(achieved, 2), peak=peak, unit="TFLOP/s", frac=round(achieved / peak, 4),
-                traffic=None)
+                traffic=traffic, kernel_ms=round(ms, 5))
   achieved = nbytes / ms / 1e6
   return dict(bound="hbm", achieved=round(achieved, 2), peak=PEAK_HBM_GBS, unit="GB/s",
-              frac=round(achieved / PEAK_HBM_GBS, 4), traffic=None)
+              frac=round(achieved / PEAK_HBM_GBS, 4), traffic=traffic, kernel_ms=round(ms, 5))
+
+
+def _time_graph(calls, launches, stream_unused=None):
+  """Average device time (ms) of one call when `launches` of them run back to back in a HIP graph.
+
+  `calls` is a list of zero-argument functions used round-robin (rotating weight copies). The graph
+  is replayed once untimed, then twice between two events."""
+  del stream_unused
+  side = torch.cuda.Stream()
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.stream(side):
+    for c in calls:
+      c()
+    side.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+      for i in range(launches):
+        calls[i % len(calls)]()
+  torch.cuda.synchronize()
+  graph.replay()
+  torch.cuda.synchronize()
+  e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  e0.record()
+  graph.replay()
+  graph.replay()
+  e1.record()
+  torch.cuda.synchronize()
+  return e0.elapsed_time(e1) / (2 * launches)
 
 
 def _cpu_baseline(w):
@@ -97,6 +139,9 @@ def main():
   ap.add_argument("--warmup", type=int, default=5)
   ap.add_argument("--no-extras", action="store_true", help="headline workload only")
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+  ap.add_argument("--calibration-copy", action="store_true",
+                  help="also run one elementwise copy of 1 GiB (reads 1 GiB, writes 1 GiB), the known-size kernel "
+                       "that hardware byte counters are scaled by")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
     print("bench.py: ragged_dot is a single-device operator and this build measures ONE GPU; "
@@ -114,6 +159,13 @@ def main():
   stream = torch.cuda.current_stream(device)
   op = tokamax_amd.HipRaggedDot()
 
+  if args.calibration_copy:
+    src = torch.zeros(1 << 28, dtype=torch.int32, device=device)
+    dst = torch.empty_like(src)
+    torch.add(src, 1, out=dst)  # one elementwise kernel: 2^30 bytes in, 2^30 bytes out
+    torch.cuda.synchronize()
+    del src, dst
+
   # ---- headline: Mixtral prefill ----------------------------------------------------------------
   w = workloads.make("mixtral", device, seed=0)
   gs = torch.tensor(w.group_sizes, device=device)
@@ -121,6 +173,10 @@ def main():
   run = lambda: op(w.lhs, w.rhs, group_sizes=gs)
   total_ms, per, wall_ms = _time_steps(run, args.steps, args.warmup, stream)
   ms = total_ms / args.steps
+  # The scheduler kernel alone (the only other kernel of a step), as a graph of back-to-back launches.
+  from tokamax_amd.ragged_dot import hip_ops
+  sched_ms = _time_graph([lambda: hip_ops.schedule(gs, w.m, config.block_m, config.align_tile)], 20)
+  gemm_ms = statistics.mean(per) - sched_ms
   result = {
       "metric": "ragged_dot TFLOP/s (% MFMA peak) prefill; GB/s (% HBM peak) decode, 1 GPU",
       "value": round(w.flops / ms / 1e9, 2),
@@ -142,7 +198,9 @@ def main():
           "kernel_config": {k: getattr(config, k) for k in ("block_m", "block_n", "block_k", "waves_m", "waves_n",
                                                             "grid_tile_width")},
       },
-      "roofline": _roofline("mfma", w.flops, w.algorithmic_bytes(), ms, "bf16"),
+      "roofline": _roofline("mfma", w.flops, w.algorithmic_bytes(), gemm_ms, "bf16",
+                            traffic=MEASURED_TRAFFIC_BYTES.get("mixtral")),
+      "schedule_kernel_ms": round(sched_ms, 5),
       "ms_median_step": round(statistics.median(per), 5),
       "ms_min_step": round(min(per), 5),
       "wall_ms_per_step": round(wall_ms / args.steps, 5),
@@ -176,21 +234,27 @@ def main():
         100 * extras["deepseek_v3_prefill_bf16"]["tflops"] / PEAK_TFLOPS["bf16"], 2)
     del w
 
-    # decode: 4 rotating copies of the weights defeat the 256 MB last-level cache ("cold"); the same
-    # copy every step is the "warm" figure.
+    # decode: 6 rotating copies of the weights defeat the 256 MB last-level cache ("cold"); the same
+    # copy every launch is the "warm" figure.
     w = workloads.make("decode", device, seed=0)
     gs = torch.tensor(w.group_sizes, device=device)
-    copies = [tokamax_amd.QArray(w.rhs.clone(), w.rhs_scale.clone()) for _ in range(4)]
+    copies = [tokamax_amd.QArray(w.rhs.clone(), w.rhs_scale.clone()) for _ in range(6)]
     cfg = op.bind(w.lhs, copies[0], group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
-    state = {"i": 0}
+    def decode_call(q):
+      return lambda: op(w.lhs, q, group_sizes=gs, preferred_element_type=torch.bfloat16)
 
-    def decode_cold():
-      state["i"] = (state["i"] + 1) % len(copies)
-      return op(w.lhs, copies[state["i"]], group_sizes=gs, preferred_element_type=torch.bfloat16)
+    def measure_graph(name, calls, traffic=None):
+      m_ = _time_graph(calls, 24)
+      extras[name] = dict(ms_per_step=round(m_, 5), tflops=round(w.flops / m_ / 1e9, 2),
+                          gbs=round(w.algorithmic_bytes() / m_ / 1e6, 2), timing="HIP graph of 24 back-to-back launches",
+                          roofline=_roofline("hbm", w.flops, w.algorithmic_bytes(), m_, "bf16", traffic=traffic),
+                          kernel_config=[cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages])
 
-    measure("decode_int8_cold", decode_cold, w.flops, w.algorithmic_bytes(), "hbm", "bf16", cfg)
-    measure("decode_int8_warm", lambda: op(w.lhs, copies[0], group_sizes=gs, preferred_element_type=torch.bfloat16),
-            w.flops, w.algorithmic_bytes(), "hbm", "bf16", cfg)
+    measure_graph("decode_int8_cold", [decode_call(q) for q in copies], MEASURED_TRAFFIC_BYTES.get("decode"))
+    measure_graph("decode_int8_warm", [decode_call(copies[0])])
+    t, p, wall = _time_steps(decode_call(copies[0]), steps, warm, stream)
+    extras["decode_int8_cold"]["eager_wall_ms_per_call"] = round(wall / steps, 5)  # host dispatch included
+    extras["decode_int8_cold"]["algorithmic_bytes"] = int(w.algorithmic_bytes())
     extras["decode_int8_cold"]["touched_experts"] = w.nonempty_groups
     del w, copies
 
