@@ -17,6 +17,8 @@
 // holding runs of 4 consecutive C columns of one C row: the epilogue stores 8/16-byte vectors.
 #pragma once
 
+#include <type_traits>
+
 #include "tkx_common.h"
 
 namespace tkx {
@@ -213,16 +215,15 @@ __device__ __forceinline__ const unsigned char* uniform_pointer(const unsigned c
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
   return (const unsigned char*)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
+// LDS byte address of a pointer into the workgroup's shared memory (wave-uniform).
+__device__ __forceinline__ unsigned lds_address32(const void* p) {
+  return __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)p);  // low half of a generic LDS pointer = LDS offset
+}
 // 16 bytes per lane: LDS[lds + 16*lane] <- *(sbase + voff)
 __device__ __forceinline__ void direct_load_16(const unsigned char* sbase, uint32_t voff, unsigned lds) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff), "s"(sbase)
                : "memory", "m0");
 }
-// 4 bytes per lane from a per-lane address (used only to touch cache lines).
-__device__ __forceinline__ void direct_load_4(const unsigned char* vptr, unsigned lds) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds), "v"(vptr) : "memory", "m0");
-}
-
 // Workgroup barrier that also orders direct-to-LDS loads: a wave's loads count on vmcnt, and other
 // waves read the bytes they deposit, so every wave must drain vmcnt BEFORE it arrives at the
 // barrier (the compiler only guards a wave's own later LDS reads).
@@ -282,35 +283,19 @@ struct DirectLoader {
     }
   }
 
-  // Cache lines (128 B, or a whole row when rows are shorter) of one k-step tile, and the byte
-  // offset of line `line` from the k-step base pointer: used to pull a later k-step into L2.
-  static constexpr int LINE = ROW_BYTES < 128 ? ROW_BYTES : 128;
-  static constexpr int LINES = BYTES / LINE;
-  static __device__ __forceinline__ uint32_t line_offset(int line, int rc0, int rc_ext, int64_t ld) {
-    constexpr int LPR = ROW_BYTES / LINE;
-    const int row = line / LPR, seg = line % LPR;
-    if constexpr (LAYOUT == kKC) {
-      int grow = rc0 + row;
-      grow = (grow < rc_ext ? grow : rc_ext - 1) - rc0;
-      return (uint32_t)(grow * (int)ld * ESZ + seg * LINE);
-    } else {
-      int colb = rc0 * ESZ + seg * LINE;
-      const int lim = rc_ext * ESZ - 16;
-      colb = colb < lim ? colb : lim;
-      return (uint32_t)(row * (int)ld * ESZ + colb);
-    }
-  }
-
-  __device__ __forceinline__ void issue(const unsigned char* base, unsigned char* tile, int wave) const {
+  // Instruction i (0 <= i < PER) of this wave's share: `base` = wave-uniform pointer of the k-step,
+  // `tile_lds` = LDS byte address of the destination tile (wave-uniform).
+  __device__ __forceinline__ void issue_one(int i, const unsigned char* base, unsigned tile_lds, int wave) const {
 #if defined(TKX_ABLATE) && (TKX_ABLATE & 1)
     return;
 #endif
+    const int j = i * NWAVES + wave;
+    if (INSTRS % NWAVES != 0 && j >= INSTRS) return;
+    direct_load_16(base, voff[i], tile_lds + j * 1024);
+  }
+  __device__ __forceinline__ void issue(const unsigned char* base, unsigned tile_lds, int wave) const {
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int j = i * NWAVES + wave;
-      if (INSTRS % NWAVES != 0 && j >= INSTRS) break;
-      direct_load_16(base, voff[i], lds_address(tile + j * 1024));
-    }
+    for (int i = 0; i < PER; ++i) issue_one(i, base, tile_lds, wave);
   }
 };
 
@@ -403,34 +388,22 @@ struct GemmKernel {
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
   typedef TileStage<LA, EA, BM, BK, THREADS> StageA;
   typedef TileStage<LB, EB, BN, BK, THREADS> StageB;
-  // The last wave of the workgroup issues no tile loads: it only prefetches into L2 (see below), so
-  // that a slow prefetch never sits in front of a tile load in a wave's in-order vmcnt queue.
-  static constexpr int NLOAD = WM * WN - 1;
+  // Every wave takes an equal share of a k-step's direct-to-LDS loads.
+  static constexpr int NLOAD = WM * WN;
   typedef DirectLoader<LA, EA, BM, BK, NLOAD> DirA;
   typedef DirectLoader<LB, EB, BN, BK, NLOAD> DirB;
   static constexpr int STAGE_BYTES = StageA::BYTES + StageB::BYTES;
-  // L2 prefetch. A workgroup can only keep NS-1 k-steps of direct loads in flight (LDS capacity),
-  // which is less than the HBM round trip; so each k-step the prefetch wave touches cache lines of
-  // the k-step PD steps further ahead with 4-byte direct-to-LDS loads into a dump area nobody
-  // reads, pulling them into L2. The workgroups that run side by side on an XCD share panels
-  // (kDedupA n-tiles share an A panel, kDedupB m-tiles share a B panel), so each touches a slice.
-  static constexpr int PD = 2;
-  static constexpr int kDedupA = 4, kDedupB = 8;
-  static constexpr int PF_A = DirA::LINES / kDedupA, PF_B = DirB::LINES / kDedupB;  // lines per workgroup
-  static constexpr int PFI = (PF_A + PF_B + 63) / 64;  // prefetch instructions per k-step
-  static_assert(PF_A >= 1 && PF_B >= 1, "prefetch slices must not be empty");
-  static constexpr int DUMP_BYTES = 256;
-  static constexpr int SMEM_BYTES = NS * STAGE_BYTES + DUMP_BYTES;
+  static constexpr int SMEM_BYTES = NS * STAGE_BYTES;
   static_assert(NS >= 2 && SMEM_BYTES <= 160 * 1024, "stages must fit the 160 KB LDS");
 
   static __device__ __forceinline__ void run(const GemmParams& p, unsigned char* smem) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: all that derives from it is uniform
     const int wm = wave / WN, wn = wave % WN;
     const int32_t* ws = p.ws;
     const int b = blockIdx.x;
 
     int group, row0, act_start, act_end, col0, kc_begin, kc_end;
-    int pf_slice_a, pf_slice_b;  // which slice of the shared panels this workgroup prefetches
     if constexpr (MODE != kDrhs) {
       const int num_tasks = ws[0];
       if (b >= p.real_slots) {
@@ -467,8 +440,6 @@ struct GemmKernel {
       col0 = nt * BN;
       kc_begin = 0;
       kc_end = p.k_ext;
-      pf_slice_a = nt & (kDedupA - 1);
-      pf_slice_b = (rem - nt * wcur) & (kDedupB - 1);
     } else {
       const int per_group = p.m_tiles * p.n_tiles;
       group = b / per_group;
@@ -480,8 +451,6 @@ struct GemmKernel {
       act_end = min(row0 + BM, p.m_ext);
       kc_begin = min(ws[p.ws_offsets + group], p.k_ext);
       kc_end = min(ws[p.ws_offsets + group + 1], p.k_ext);
-      pf_slice_a = nt & (kDedupA - 1);
-      pf_slice_b = mt & (kDedupB - 1);
     }
 
     const unsigned char* Ab = reinterpret_cast<const unsigned char*>(p.A);
@@ -497,18 +466,33 @@ struct GemmKernel {
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
     typedef typename Mma<EC>::Frag Frag;
-    auto load_frags = [&](Frag* fa, Frag* fb, const unsigned char* stage, int kk) {
+    // Row blocks (32 rows) of this wave that hold at least one row the task stores. A task at a
+    // group boundary can have only a few such rows; the blocks without any skip their LDS reads and
+    // MFMAs (the wave still takes part in the loads and barriers). `full` selects at compile time
+    // the path without the per-block tests, which whole tiles take.
+    uint32_t rmask = 0;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int r0 = row0 + wm * WTM + i * 32;
+      if (r0 < act_end && r0 + 32 > act_start) rmask |= 1u << i;
+    }
+    rmask = __builtin_amdgcn_readfirstlane(rmask);
+    const bool all_rows = rmask == (1u << TM) - 1u;
+    auto load_frags = [&](auto full, Frag* fa, Frag* fb, const unsigned char* stage, int kk) {
 #if defined(TKX_ABLATE) && (TKX_ABLATE & 2)
       return;
 #endif
 #pragma unroll
       for (int i = 0; i < TM; ++i)
-        fa[i] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, wm * WTM + i * 32, kk, lane);
+        if (decltype(full)::value || ((rmask >> i) & 1u))
+          fa[i] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, wm * WTM + i * 32, kk, lane);
+      if (decltype(full)::value || rmask != 0) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        fb[j] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + j * 32, kk, lane);
+        for (int j = 0; j < TN; ++j)
+          fb[j] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + j * 32, kk, lane);
+      }
     };
-    auto mma_all = [&](const Frag* fa, const Frag* fb) {
+    auto mma_all = [&](auto full, const Frag* fa, const Frag* fb) {
 #if defined(TKX_ABLATE) && (TKX_ABLATE & 4)
       for (int i = 0; i < TM; ++i) asm volatile("" ::"v"(fa[i]));
       for (int j = 0; j < TN; ++j) asm volatile("" ::"v"(fb[j]));
@@ -516,8 +500,10 @@ struct GemmKernel {
 #endif
 #pragma unroll
       for (int i = 0; i < TM; ++i)
+        if (decltype(full)::value || ((rmask >> i) & 1u)) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = mma_atom<EC>(fb[j], fa[i], acc[i][j]);
+          for (int j = 0; j < TN; ++j) acc[i][j] = mma_atom<EC>(fb[j], fa[i], acc[i][j]);
+        }
     };
 
     const int span = kc_end - kc_begin;
@@ -529,98 +515,121 @@ struct GemmKernel {
       DirB db;
       da.init(row0, p.m_ext, p.lda, wave, lane);
       db.init(col0, p.n_ext, p.ldb, wave, lane);
-      const unsigned char* gA = Ab + DirA::step_base(row0, p.lda, kc_begin);
-      const unsigned char* gB = Bb + DirB::step_base(col0, p.ldb, kc_begin);
+      const unsigned char* const gA0 = Ab + DirA::step_base(row0, p.lda, kc_begin);
+      const unsigned char* const gB0 = Bb + DirB::step_base(col0, p.ldb, kc_begin);
       const int64_t stepA = DirA::step_bytes(p.lda), stepB = DirB::step_bytes(p.ldb);
+      const unsigned smem_lds = lds_address32(smem);
       // A load wave may leave the loads of the NS-2 k-steps after the needed one in flight; that
       // count is only known at compile time when the tile splits evenly over the load waves.
       constexpr bool kExact = DirA::INSTRS % NLOAD == 0 && DirB::INSTRS % NLOAD == 0;
       constexpr int kInFlight = kExact ? (NS - 2) * (DirA::PER + DirB::PER) : 0;
       static_assert(kInFlight < 64, "too many direct loads in flight for vmcnt");
 
-      // L2 prefetch lines of this lane (prefetch wave only; slots past the slice repeat its last line).
-      const bool pf_wave = wave == NLOAD;
-      uint32_t pf_off[PFI];
-      bool pf_is_b[PFI];
-#pragma unroll
-      for (int i = 0; i < PFI; ++i) {
-        int idx = i * 64 + lane;
-        idx = idx < PF_A + PF_B ? idx : PF_A + PF_B - 1;
-        pf_is_b[i] = idx >= PF_A;
-        pf_off[i] = pf_is_b[i] ? DirB::line_offset(pf_slice_b * PF_B + (idx - PF_A), col0, p.n_ext, p.ldb)
-                               : DirA::line_offset(pf_slice_a * PF_A + idx, row0, p.m_ext, p.lda);
-      }
-      unsigned char* dump = smem + NS * STAGE_BYTES;
-      const unsigned char* const gA0 = gA;
-      const unsigned char* const gB0 = gB;
-      auto prefetch_step = [&](int step) {
-#if defined(TKX_ABLATE) && (TKX_ABLATE & 16)
-        return;
-#endif
-        if (step >= nfull) return;
-        const unsigned char* a = gA0 + step * stepA;
-        const unsigned char* b = gB0 + step * stepB;
-#pragma unroll
-        for (int i = 0; i < PFI; ++i)
-          direct_load_4((pf_is_b[i] ? b : a) + pf_off[i], lds_address(dump));
+      // One k-step of loads is a list of NLD per-wave instructions; slot q of the list can be issued
+      // on its own, so that the list can be threaded between MFMAs.
+      constexpr int NLD = DirA::PER + DirB::PER;
+      struct StepPtrs { const unsigned char *a, *b; unsigned lds; };
+      auto step_ptrs = [&](int step, int stage) {
+        StepPtrs sp;
+        sp.a = uniform_pointer(gA0 + step * stepA);
+        sp.b = uniform_pointer(gB0 + step * stepB);
+        sp.lds = smem_lds + stage * STAGE_BYTES;
+        return sp;
       };
-      // Tile loads by the load waves, prefetch by the prefetch wave.
-      auto issue_step = [&](int step, int stage) {
-        if (!pf_wave) {
-          da.issue(uniform_pointer(gA0 + step * stepA), smem + stage * STAGE_BYTES, wave);
-          db.issue(uniform_pointer(gB0 + step * stepB), smem + stage * STAGE_BYTES + StageA::BYTES, wave);
-        } else {
-          prefetch_step(step + PD);
-        }
+      auto issue_slot = [&](int q, const StepPtrs& sp) {
+        if (q < DirA::PER) da.issue_one(q, sp.a, sp.lds, wave);
+        else if (q < DirA::PER + DirB::PER) db.issue_one(q - DirA::PER, sp.b, sp.lds + StageA::BYTES, wave);
       };
-      // Load waves drain their tile loads before a barrier; the prefetch wave never waits for its
-      // loads inside the loop (nothing reads what they bring).
+      // Every wave drains the loads the next k-step needs before it arrives at a barrier.
       auto step_barrier = [&](bool partial) {
-        if (pf_wave) barrier_after_direct_loads<63>();
-        else if (partial) barrier_after_direct_loads<kInFlight>();
+        if (partial) barrier_after_direct_loads<kInFlight>();
         else barrier_after_direct_loads<0>();
       };
 
-      // Prologue: NS-1 stages in flight, wait for the first.
-      int load_stage = 0;  // stage the next issued k-step goes to
-      int load_step = 0;   // k-step the next issue loads
+      // Prologue: every stage gets a k-step; wait for the first.
 #pragma unroll
-      for (int s_ = 0; s_ < NS - 1; ++s_) {
+      for (int s_ = 0; s_ < NS; ++s_) {
         if (s_ < nfull) {
-          issue_step(load_step, load_stage);
-          ++load_step;
-          load_stage = load_stage + 1 == NS ? 0 : load_stage + 1;
-        }
-      }
-      step_barrier(nfull >= NS - 1);
-
-      Frag fa[2][TM], fb[2][TN];
-      load_frags(fa[0], fb[0], smem, 0);
-      int cur_stage = 0;
-      for (int kt = 0; kt < nfull; ++kt) {
-        const unsigned char* cur = smem + cur_stage * STAGE_BYTES;
-        cur_stage = cur_stage + 1 == NS ? 0 : cur_stage + 1;
-        const unsigned char* nxt = smem + cur_stage * STAGE_BYTES;
-        const bool issue = load_step < nfull;
-        if (issue) {
-          // `load_stage` was last read during step kt-1; every wave passed that step's barrier since.
-          issue_step(load_step, load_stage);
-          ++load_step;
-          load_stage = load_stage + 1 == NS ? 0 : load_stage + 1;
-        }
+          const StepPtrs sp = step_ptrs(s_, s_);
 #pragma unroll
-        for (int kk = 0; kk + 1 < KSTEPS; ++kk) {
-          load_frags(fa[(kk + 1) & 1], fb[(kk + 1) & 1], cur, kk + 1);
-          mma_all(fa[kk & 1], fb[kk & 1]);
+          for (int q = 0; q < NLD; ++q) issue_slot(q, sp);
         }
-        // All LDS reads of `cur` are issued. After the barrier the next stage is complete, so its
-        // first fragments are fetched under the MFMAs of this step's last k-atom.
-        step_barrier(issue);
-        if (kt + 1 < nfull) load_frags(fa[0], fb[0], nxt, 0);
-        mma_all(fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1]);
       }
-      // The dump area may still be receiving prefetched bytes: drain before LDS is reused or freed.
-      if (pf_wave) __builtin_amdgcn_s_waitcnt((0 & 15) | (7 << 4) | (15 << 8));
+      if (kExact && nfull >= NS) barrier_after_direct_loads<(NS - 1) * (DirA::PER + DirB::PER)>();
+      else barrier_after_direct_loads<0>();
+
+      // The k loop. Each 32-wide (KA-deep) atom is a run of TM*TN MFMAs; the LDS reads of the next
+      // atom's fragments and, in the last atom of a k-step, the global loads that refill the stage
+      // just released are threaded between those MFMAs one by one, so that the matrix pipe is
+      // never left waiting behind a block of memory instructions.
+      auto k_loop = [&](auto full) {
+        constexpr bool F = decltype(full)::value;
+        Frag fa[2][TM], fb[2][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[0][i] = fa[1][i] = Frag{};
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[0][j] = fb[1][j] = Frag{};
+        // Fragment f of an atom: f < TM is the A fragment of row block f, else the B fragment f - TM.
+        auto read_frag = [&](Frag* a, Frag* b, int f, const unsigned char* stage, int kk) {
+#if defined(TKX_ABLATE) && (TKX_ABLATE & 2)
+          return;
+#endif
+          if (f < TM) {
+            if (F || ((rmask >> f) & 1u)) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, wm * WTM + f * 32, kk, lane);
+          } else if (f < TM + TN) {
+            if (F || rmask != 0)
+              b[f - TM] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + (f - TM) * 32, kk, lane);
+          }
+        };
+        constexpr int NM = TM * TN;                      // MFMAs per atom
+        constexpr int RPM = (TM + TN + NM - 1) / NM;     // fragment reads threaded after each MFMA
+        constexpr int LPM = (NLD + NM - 1) / NM;         // load slots threaded after each MFMA
+        auto atom = [&](const Frag* a, const Frag* b, Frag* na, Frag* nb, const unsigned char* rd_stage, int rd_kk,
+                        bool reads, bool loads, const StepPtrs& sp) {
+#pragma unroll
+          for (int t = 0; t < NM; ++t) {
+            const int i = t / TN, j = t % TN;
+#if defined(TKX_ABLATE) && (TKX_ABLATE & 4)
+            asm volatile("" ::"v"(a[i]), "v"(b[j]));
+#else
+            if (F || ((rmask >> i) & 1u)) acc[i][j] = mma_atom<EC>(b[j], a[i], acc[i][j]);
+#endif
+            if (reads) {
+#pragma unroll
+              for (int r = 0; r < RPM; ++r) read_frag(na, nb, t * RPM + r, rd_stage, rd_kk);
+            }
+            if (loads) {
+#pragma unroll
+              for (int q = 0; q < LPM; ++q) issue_slot(t * LPM + q, sp);
+            }
+            if (F) __builtin_amdgcn_sched_barrier(0);
+          }
+        };
+
+#pragma unroll
+        for (int f = 0; f < TM + TN; ++f) read_frag(fa[0], fb[0], f, smem, 0);
+        int cur_stage = 0;
+        const StepPtrs none = {};
+        for (int kt = 0; kt < nfull; ++kt) {
+          const unsigned char* cur = smem + cur_stage * STAGE_BYTES;
+          const int freed = cur_stage;
+          cur_stage = cur_stage + 1 == NS ? 0 : cur_stage + 1;
+          const unsigned char* nxt = smem + cur_stage * STAGE_BYTES;
+          // (Pointers of the refill are computed here, far ahead of the MFMAs they are issued between.)
+          const bool refill = kt + NS < nfull;
+          const StepPtrs sp = refill ? step_ptrs(kt + NS, freed) : none;
+#pragma unroll
+          for (int kk = 0; kk + 1 < KSTEPS; ++kk)
+            atom(fa[kk & 1], fb[kk & 1], fa[(kk + 1) & 1], fb[(kk + 1) & 1], cur, kk + 1, true, false, none);
+          // All LDS reads of `cur` are issued. After the barrier the next stage is complete and `cur`
+          // is free: the last atom's MFMAs cover the first fragment reads of the next stage and the
+          // issue of the loads that refill `cur` with k-step kt + NS.
+          step_barrier(kt + NS - 1 < nfull);
+          atom(fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1], fa[0], fb[0], nxt, 0, kt + 1 < nfull, refill, sp);
+        }
+      };
+      if (all_rows) k_loop(std::true_type{});
+      else k_loop(std::false_type{});
     }
     if (tail) {
       const int kc0 = kc_begin + nfull * BK;
@@ -630,8 +639,12 @@ struct GemmKernel {
 #pragma unroll
       for (int kk = 0; kk < KSTEPS; ++kk) {
         Frag fa[TM], fb[TN];
-        load_frags(fa, fb, smem, kk);
-        mma_all(fa, fb);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[i] = Frag{};
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[j] = Frag{};
+        load_frags(std::false_type{}, fa, fb, smem, kk);
+        mma_all(std::false_type{}, fa, fb);
       }
     }
 

@@ -9,8 +9,7 @@ namespace tkx {
 static const Variant kVariants[] = {
     FWD_DLHS(256, 256, 64, 2, 4, 2),
     FWD_DLHS(256, 256, 32, 2, 4, 4),
-    FWD_DLHS(256, 256, 64, 2, 2, 2),
-    FWD_DLHS(256, 256, 32, 2, 2, 4),
+    FWD_DLHS(256, 256, 32, 2, 4, 5),
     FWD_DLHS(256, 128, 64, 2, 4, 3),
     FWD_DLHS(128, 256, 64, 2, 4, 3),
     FWD_DLHS(128, 256, 64, 2, 2, 3),
