@@ -373,6 +373,26 @@ __device__ __forceinline__ void store4(void* C, int64_t idx, f32x4 v, int out_dt
   }
 }
 
+// 4 consecutive outputs at a byte address, in a compile-time output type. (The pointer is rebuilt
+// from integers upstream, so the global address space is named here: a generic pointer would turn
+// every store into a flat one.)
+template <int OUT>
+__device__ __forceinline__ void store4_as(unsigned char* ptr, f32x4 v) {
+  if constexpr (OUT == TKX_F32) {
+    *(__attribute__((address_space(1))) f32x4*)ptr = v;
+  } else if constexpr (OUT == TKX_BF16) {
+    bf16x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = (__bf16)v[e];
+    *(__attribute__((address_space(1))) bf16x4*)ptr = o;
+  } else {
+    f16x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = (_Float16)v[e];
+    *(__attribute__((address_space(1))) f16x4*)ptr = o;
+  }
+}
+
 // ---- the kernel ---------------------------------------------------------------------------------
 template <int MODE, int EA, int EB, int BM, int BN, int BK, int WM, int WN, int NS>
 struct GemmKernel {
@@ -649,41 +669,84 @@ struct GemmKernel {
     }
 
     // Epilogue. After the swapped MFMA, lane l of atom (i, j) holds C row (l % 32) and, for
-    // t = 0..3, columns 8t + 4*(l / 32) + {0,1,2,3} of that atom.
-    unsigned char* Cb = reinterpret_cast<unsigned char*>(p.C);
-    if constexpr (MODE == kDrhs)
-      Cb += (int64_t)group * p.c_group_stride * (p.out_dtype == TKX_F32 ? 4 : 2);
+    // t = 0..3, columns 8t + 4*(l / 32) + {0,1,2,3} of that atom. Scales and the activation are
+    // applied to the accumulators in registers first (each in one pass, with the run-time choices
+    // made outside the unrolled loops); the stores then only convert and write. A store's address
+    // is the tile's (uniform) base plus one lane offset per row block plus a constant.
+    {
+      unsigned char* Cg = reinterpret_cast<unsigned char*>(p.C);
+      if constexpr (MODE == kDrhs) Cg += (int64_t)group * p.c_group_stride * (p.out_dtype == TKX_F32 ? 4 : 2);
+      const bool inside = col0 + BN <= p.n_ext;
+      const int lane_col = wn * WTN + 4 * (lane >> 5);
+      if (p.a_scale != nullptr) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int row = row0 + wm * WTM + i * 32 + (lane & 31);
-      const bool row_ok = row >= act_start && row < act_end;
-      float rs = 1.f;
-      if (p.a_scale != nullptr && row_ok) rs = p.a_scale[row];
+        for (int i = 0; i < TM; ++i) {
+          const int row = min(row0 + wm * WTM + i * 32 + (lane & 31), p.m_ext - 1);
+          const float rs = p.a_scale[row];
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
+          for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int col = col0 + wn * WTN + j * 32 + 8 * t + 4 * (lane >> 5);
-          if (!row_ok || col + 4 > p.n_ext) continue;
-          f32x4 v;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * t + e];
-          if (p.a_scale != nullptr) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] *= rs;
-          }
-          if (p.b_scale != nullptr) {
-            const f32x4 cs = *reinterpret_cast<const f32x4*>(p.b_scale + (int64_t)group * p.n_ext + col);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] *= cs[e];
-          }
-          if (p.activation != TKX_ACT_NONE) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = apply_activation(v[e], p.activation);
-          }
-          store4(Cb, (int64_t)row * p.ldc + col, v, p.out_dtype);
+            for (int e = 0; e < 16; ++e) acc[i][j][e] *= rs;
         }
       }
+      if (p.b_scale != nullptr) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int col = min(col0 + lane_col + j * 32 + 8 * t, p.n_ext - 4);
+            const f32x4 cs = *reinterpret_cast<const f32x4*>(p.b_scale + (int64_t)group * p.n_ext + col);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[i][j][4 * t + e] *= cs[e];
+          }
+        }
+      }
+      if (p.activation != TKX_ACT_NONE) {
+        auto for_all = [&](auto fn) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) acc[i][j][e] = fn(acc[i][j][e]);
+        };
+        // tanh(x) = 1 - 2 / (exp(2x) + 1): a handful of instructions per element with the hardware
+        // exponential and reciprocal.
+        auto fast_tanh = [](float x) { return 1.f - 2.f * __builtin_amdgcn_rcpf(__expf(2.f * x) + 1.f); };
+        if (p.activation == TKX_ACT_RELU) for_all([](float x) { return x > 0.f ? x : 0.f; });
+        else if (p.activation == TKX_ACT_TANH) for_all(fast_tanh);
+        else if (p.activation == TKX_ACT_SILU) for_all([](float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-x)); });
+        else if (p.activation == TKX_ACT_GELU_TANH)
+          for_all([&](float x) { return 0.5f * x * (1.f + fast_tanh(0.7978845608028654f * (x + 0.044715f * x * x * x))); });
+      }
+      auto emit = [&](auto out_tag) {
+        constexpr int OUT = decltype(out_tag)::value;
+        constexpr int ESZ = OUT == TKX_F32 ? 4 : 2;
+        unsigned char* const tile = const_cast<unsigned char*>(uniform_pointer(Cg + ((int64_t)row0 * p.ldc + col0) * ESZ));
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int lrow = wm * WTM + i * 32 + (lane & 31);
+          const int row = row0 + lrow;
+          if (!(row >= act_start && row < act_end)) continue;
+          const uint32_t voff = (uint32_t)((lrow * (int)p.ldc + lane_col) * ESZ);
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+              if (!inside && col0 + lane_col + j * 32 + 8 * t + 4 > p.n_ext) continue;
+              f32x4 v;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * t + e];
+              store4_as<OUT>(tile + voff + (j * 32 + 8 * t) * ESZ, v);
+            }
+          }
+        }
+      };
+      if (p.out_dtype == TKX_BF16) emit(std::integral_constant<int, TKX_BF16>{});
+      else if (p.out_dtype == TKX_F32) emit(std::integral_constant<int, TKX_F32>{});
+      else emit(std::integral_constant<int, TKX_F16>{});
     }
   }
 };
