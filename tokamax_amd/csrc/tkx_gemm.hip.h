@@ -721,26 +721,68 @@ struct GemmKernel {
         else if (p.activation == TKX_ACT_GELU_TANH)
           for_all([&](float x) { return 0.5f * x * (1.f + fast_tanh(0.7978845608028654f * (x + 0.044715f * x * x * x))); });
       }
+      // The stores go through LDS (free once the k loop is done): as the MFMA leaves them, a
+      // lane's values are 4 columns of one row, so a store straight from registers writes 16-byte
+      // pieces of 32 different rows and the memory pipeline takes it apart line by line. Each wave
+      // lays its part of the tile out row-major in its own slice of LDS and reads it back 16 bytes
+      // per lane, so that a store instruction writes whole 128-byte (or longer) row segments.
+      __syncthreads();  // every wave is done reading the last stage
       auto emit = [&](auto out_tag) {
         constexpr int OUT = decltype(out_tag)::value;
         constexpr int ESZ = OUT == TKX_F32 ? 4 : 2;
+        constexpr int ROW_BYTES = WTN * ESZ;
+        constexpr int PITCH = ROW_BYTES + 16;                     // keeps 16-byte alignment, staggers banks
+        constexpr int WAVE_LDS = (SMEM_BYTES / (WM * WN)) / 16 * 16;
+        constexpr int AP = (WAVE_LDS / PITCH) / 32 < TM ? (WAVE_LDS / PITCH) / 32 : TM;  // atoms (32 rows) per pass
+        static_assert(AP >= 1, "a wave's LDS slice must hold 32 output rows");
+        constexpr int CPR = ROW_BYTES / 16;                       // 16-byte chunks per row
+        constexpr int RPI = 64 / CPR;                             // rows per store instruction
+        static_assert(64 % CPR == 0 && CPR <= 64, "a store instruction must cover whole rows");
+        unsigned char* const slice = smem + wave * WAVE_LDS;
         unsigned char* const tile = const_cast<unsigned char*>(uniform_pointer(Cg + ((int64_t)row0 * p.ldc + col0) * ESZ));
+        const int rd_row = lane / CPR, rd_chunk = lane % CPR;
+        const int gcol = col0 + wn * WTN + rd_chunk * (16 / ESZ);
+        const bool col_ok = inside || gcol + 16 / ESZ <= p.n_ext;
+        const uint32_t voff = (uint32_t)(((wm * WTM + rd_row) * (int)p.ldc + wn * WTN + rd_chunk * (16 / ESZ)) * ESZ);
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const int lrow = wm * WTM + i * 32 + (lane & 31);
-          const int row = row0 + lrow;
-          if (!(row >= act_start && row < act_end)) continue;
-          const uint32_t voff = (uint32_t)((lrow * (int)p.ldc + lane_col) * ESZ);
+        for (int i0 = 0; i0 < TM; i0 += AP) {
 #pragma unroll
-          for (int j = 0; j < TN; ++j) {
+          for (int ii = 0; ii < AP; ++ii) {
+            if (i0 + ii >= TM) break;
+            const int i = i0 + ii;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-              if (!inside && col0 + lane_col + j * 32 + 8 * t + 4 > p.n_ext) continue;
-              f32x4 v;
+            for (int j = 0; j < TN; ++j) {
 #pragma unroll
-              for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * t + e];
-              store4_as<OUT>(tile + voff + (j * 32 + 8 * t) * ESZ, v);
+              for (int t = 0; t < 4; ++t) {
+                f32x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * t + e];
+                unsigned char* dst = slice + (ii * 32 + (lane & 31)) * PITCH + (j * 32 + 8 * t + 4 * (lane >> 5)) * ESZ;
+                if constexpr (OUT == TKX_F32) {
+                  *reinterpret_cast<f32x4*>(dst) = v;
+                } else if constexpr (OUT == TKX_BF16) {
+                  bf16x4 o;
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) o[e] = (__bf16)v[e];
+                  *reinterpret_cast<bf16x4*>(dst) = o;
+                } else {
+                  f16x4 o;
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) o[e] = (_Float16)v[e];
+                  *reinterpret_cast<f16x4*>(dst) = o;
+                }
+              }
             }
+          }
+          constexpr int ROWS = AP * 32;
+#pragma unroll
+          for (int s_ = 0; s_ < ROWS / RPI; ++s_) {
+            const int lrow = i0 * 32 + s_ * RPI + rd_row;            // row inside the wave's part of the tile
+            if (lrow >= WTM) continue;
+            const int row = row0 + wm * WTM + lrow;
+            const i32x4 val = *reinterpret_cast<const i32x4*>(slice + (s_ * RPI + rd_row) * PITCH + rd_chunk * 16);
+            if (row >= act_start && row < act_end && col_ok)
+              *(__attribute__((address_space(1))) i32x4*)(tile + (size_t)(i0 * 32 + s_ * RPI) * p.ldc * ESZ + voff) = val;
           }
         }
       };
