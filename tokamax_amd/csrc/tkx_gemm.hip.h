@@ -781,8 +781,10 @@ struct GemmKernel {
             if (lrow >= WTM) continue;
             const int row = row0 + wm * WTM + lrow;
             const i32x4 val = *reinterpret_cast<const i32x4*>(slice + (s_ * RPI + rd_row) * PITCH + rd_chunk * 16);
+            // (Non-temporal: the output is not read again by this kernel and should not displace
+            // the operand panels the other workgroups of the XCD share in L2.)
             if (row >= act_start && row < act_end && col_ok)
-              *(__attribute__((address_space(1))) i32x4*)(tile + (size_t)(i0 * 32 + s_ * RPI) * p.ldc * ESZ + voff) = val;
+              __builtin_nontemporal_store(val, (__attribute__((address_space(1))) i32x4*)(tile + (size_t)(i0 * 32 + s_ * RPI) * p.ldc * ESZ + voff));
           }
         }
       };
