@@ -167,7 +167,7 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
     if (lhs_scale != nullptr) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no lhs scale");
     if (!decode_i8w_supported(m, k, n, num_groups))
       return set_error(TKX_ERR_UNSUPPORTED,
-                       "decode kernel needs k %% 1024 == 0, n %% 8 == 0 and at most 1024 groups (k=%lld n=%lld G=%lld)",
+                       "decode kernel needs k %% 1024 == 0 and n %% 8 == 0 (k=%lld n=%lld G=%lld)",
                        (long long)k, (long long)n, (long long)num_groups);
     return launch_decode_i8w(lhs, rhs, rhs_scale, group_sizes, out, m, k, n, num_groups, out_dtype, activation,
                              c.num_stages, stream);

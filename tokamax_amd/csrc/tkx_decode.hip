@@ -2,9 +2,9 @@
 //
 // This regime is bound by HBM: every touched expert's [k,n] weight panel is read once, and a group
 // has a handful of rows. The kernel is built around streaming those panels:
-//   * one launch, no scheduler kernel: every workgroup reads group_sizes itself, the workgroups are
-//     dealt to the non-empty groups in order, and the surplus ones exit at once (an empty group's
-//     weights are never read);
+//   * one launch, no scheduler kernel: a workgroup derives its group's row range from group_sizes
+//     itself while its first weight loads are already in flight, and the workgroups of empty groups
+//     exit (all but the first 2% of an empty group's weights are never read);
 //   * a workgroup owns (group, 128 output columns); its 4 waves split the contraction and each
 //     streams its own [k/4, 128] slice of the panel with full 128-byte rows, several steps of
 //     global loads in flight in registers; no workgroup barrier and no LDS inside the loop;
@@ -27,7 +27,6 @@ constexpr int kDecWaves = 4;   // waves per workgroup; each takes k / 4 of the c
 constexpr int kDecKS = 32;     // contraction elements per step (one 16x16x32 MFMA deep)
 constexpr int kDecRows = 16;   // lhs rows per pass
 constexpr int kDecThreads = kDecWaves * 64;
-constexpr int kDecMaxGroups = 1024;  // group sizes are staged in LDS
 
 struct DecodeParams {
   const __bf16* lhs;
@@ -85,65 +84,18 @@ __device__ __forceinline__ bf16x8 column_to_bf16x8(const i32x2 (&rows)[8]) {
 template <int kDecDepth, int kMinWgs>
 __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_i8w_kernel(const DecodeParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  __shared__ int s_size[kDecMaxGroups];
-  __shared__ int s_cnt[kDecMaxGroups / 64], s_rows[kDecMaxGroups / 64];
-  __shared__ unsigned long long s_mask[kDecMaxGroups / 64];
+  __shared__ int s_red[kDecWaves];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  // The grid is G x n_tiles, but workgroups are handed to the non-empty groups in order: workgroup
-  // w serves the (w / n_tiles)-th non-empty group. The busy workgroups are then the first ones of
-  // the grid, which spreads them evenly over the XCDs and CUs however the empty groups fall; the
-  // rest exit after reading group_sizes. An empty group's weights are never touched.
-  const int t = blockIdx.x / p.n_tiles, nt = blockIdx.x - t * p.n_tiles;
+  const int g = blockIdx.x / p.n_tiles, nt = blockIdx.x - g * p.n_tiles;
   const int col0 = nt * kDecBN;
+  const bool last_group = g == p.num_groups - 1;
 
-  // Every workgroup reads all group sizes once (G <= 1024): 64 groups per wave pass.
-  const int chunks = (p.num_groups + 63) >> 6;
-  for (int c = wave; c < chunks; c += kDecWaves) {
-    const int j = 64 * c + lane;
-    const int sz = j < p.num_groups ? max(p.group_sizes[j], 0) : 0;
-    s_size[j] = sz;
-    const unsigned long long mask = __ballot(sz > 0);
-    int rows = sz;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) rows += __shfl_xor(rows, off);
-    if (lane == 0) {
-      s_mask[c] = mask;
-      s_cnt[c] = __popcll(mask);
-      s_rows[c] = rows;
-    }
-  }
-  __syncthreads();
-  // Locate the t-th non-empty group: its 64-group chunk, then its bit inside the chunk's mask.
-  int chunk = -1, cnt_before = 0, rows_before = 0, total_cnt = 0, total_rows = 0;
-  for (int c = 0; c < chunks; ++c) {
-    const int cnt = s_cnt[c], rows = s_rows[c];
-    if (chunk < 0 && total_cnt + cnt > t) {
-      chunk = c;
-      cnt_before = total_cnt;
-      rows_before = total_rows;
-    }
-    total_cnt += cnt;
-    total_rows += rows;
-  }
-  // Rows past the last group belong to no group; the workgroups of the last non-empty group (or
-  // of slot 0 when every group is empty) zero their columns of those rows.
-  const bool zeroes_tail = t == max(total_cnt, 1) - 1;
-  if (chunk < 0 && !zeroes_tail) return;
-  int g = 0, start = 0, size = 0;
-  if (chunk >= 0) {
-    const unsigned long long mask = s_mask[chunk];
-    const int r = t - cnt_before;
-    const bool mine = ((mask >> lane) & 1ull) != 0 && __popcll(mask & ((1ull << lane) - 1ull)) == r;
-    const int bit = __builtin_ctzll(__ballot(mine));
-    g = __builtin_amdgcn_readfirstlane(64 * chunk + bit);
-    int rows = lane < bit ? s_size[64 * chunk + lane] : 0;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) rows += __shfl_xor(rows, off);
-    start = __builtin_amdgcn_readfirstlane(rows_before + rows);
-    size = __builtin_amdgcn_readfirstlane(s_size[g]);
-  }
-  const int end = min(start + size, p.m);
-  const int esz = p.out_dtype == TKX_F32 ? 4 : 2;
+  // Sizes of the groups before this one (for its first row) and its own size are requested first
+  // and used last: the first weight steps go out right behind them, before anything is known
+  // about the group, so that one memory round trip covers both. A workgroup whose group turns out
+  // empty returns with those few loads in flight (32 KB of the group's 1.5 MB, never more).
+  const int first_size = p.group_sizes[min(tid, p.num_groups - 1)];  // unconditional: no wait until it is used
+  const int own_size = max(p.group_sizes[g], 0);
 
   const int kw = p.k / kDecWaves;      // contraction slice of this wave
   const int k_begin = wave * kw;
@@ -161,8 +113,8 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_i8w_kernel(const 
   i32x2 breg[kDecDepth][8];
   i32x4 areg[kDecDepth];
   // Nothing looks at a loaded value before its step comes up, so the only waits are the per-step
-  // vmcnt of the oldest group. (A workgroup without a group gets an empty buffer: its loads read zero.)
-  const __amdgpu_buffer_rsrc_t wbuf = buffer_of(wbase, chunk >= 0 ? (uint32_t)kw * (uint32_t)p.n : 0u);
+  // vmcnt of the oldest group.
+  const __amdgpu_buffer_rsrc_t wbuf = buffer_of(wbase, (uint32_t)kw * (uint32_t)p.n);
   const uint32_t step_bytes = (uint32_t)(kDecKS * p.n);
   auto issue_b = [&](int slot, int step) {
     const uint32_t so = (uint32_t)__builtin_amdgcn_readfirstlane((int)(step * step_bytes));
@@ -180,21 +132,37 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_i8w_kernel(const 
   f32x4_t scale_lo = {1.f, 1.f, 1.f, 1.f}, scale_hi = {1.f, 1.f, 1.f, 1.f};
   {
     const int col = col0 + (tid & 15) * 8;
-    if (p.scale != nullptr && chunk >= 0 && col + 8 <= p.n) {
+    if (p.scale != nullptr && col + 8 <= p.n) {
       const float* sc = p.scale + (int64_t)g * p.n + col;
       scale_lo = *reinterpret_cast<const f32x4_t*>(sc);
       scale_hi = *reinterpret_cast<const f32x4_t*>(sc + 4);
     }
   }
 
-  if (zeroes_tail) {
-    const int tail = min(total_rows, p.m);
+  // Row range of this group.
+  const int size = __builtin_amdgcn_readfirstlane(own_size);
+  if (size == 0 && !last_group) return;
+  int before = tid < g ? max(first_size, 0) : 0;
+  for (int j = tid + kDecThreads; j < g; j += kDecThreads) before += max(p.group_sizes[j], 0);  // G > 256 only
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off);
+  if (lane == 0) s_red[wave] = before;
+  __syncthreads();
+  int start = 0;
+#pragma unroll
+  for (int w = 0; w < kDecWaves; ++w) start += s_red[w];
+  start = __builtin_amdgcn_readfirstlane(start);
+  const int end = min(start + size, p.m);
+  const int esz = p.out_dtype == TKX_F32 ? 4 : 2;
+
+  if (last_group) {
+    // Rows past the last group belong to no group: zero this workgroup's columns of them.
     const int ncol = min(kDecBN, p.n - col0);
     const int pieces = ncol * esz / 16;  // 16-byte pieces per row
     unsigned char* c = reinterpret_cast<unsigned char*>(p.out);
     const i32x4 z = {0, 0, 0, 0};
-    for (int idx = tid; idx < (p.m - tail) * pieces; idx += kDecThreads) {
-      const int r = tail + idx / pieces, ch = idx % pieces;
+    for (int idx = tid; idx < (p.m - end) * pieces; idx += kDecThreads) {
+      const int r = end + idx / pieces, ch = idx % pieces;
       *reinterpret_cast<i32x4*>(c + ((int64_t)r * p.n + col0) * esz + ch * 16) = z;
     }
   }
@@ -315,7 +283,8 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_i8w_kernel(const 
 // Whether the decode kernel can run this problem (else the caller uses the tiled kernel).
 bool decode_i8w_supported(int64_t m, int64_t k, int64_t n, int64_t G) {
   (void)m;
-  if (G > kDecMaxGroups || (k / kDecWaves) * n >= (1LL << 31)) return false;
+  (void)G;
+  if ((k / kDecWaves) * n >= (1LL << 31)) return false;
   return k % (kDecWaves * kDecKS * 8) == 0 && n % 8 == 0 && n >= 8;
 }
 

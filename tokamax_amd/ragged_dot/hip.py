@@ -249,9 +249,8 @@ class HipRaggedDot(base.RaggedDot):
       raise NotImplementedError(f"No hip kernel for dtypes/mode {key}.")
     usable = list(variants)
     if key[2] == _lib.TKX_I8:
-      # The streaming small-m kernel (block_m == 16) needs k % 1024 == 0, n % 8 == 0 and G <= 1024.
-      usable = [v for v in usable
-                if v[0] != 16 or (contraction % 1024 == 0 and cols % 8 == 0 and num_groups <= 1024)]
+      # The streaming small-m kernel (block_m == 16) needs k % 1024 == 0 and n % 8 == 0.
+      usable = [v for v in usable if v[0] != 16 or (contraction % 1024 == 0 and cols % 8 == 0)]
     # Rows per group decide the m-tile: a tile much taller than a group wastes MFMA work on rows
     # that are masked out at the store; a short tile re-reads the weights more often.
     rows_per_group = rows / max(num_groups, 1) if mode != 2 else rows
