@@ -17,6 +17,7 @@ import abc
 import collections
 import contextvars
 import dataclasses
+import functools
 import inspect
 import json
 import logging
@@ -84,12 +85,12 @@ class Op(abc.ABC):
 
   def __call__(self, *args, return_residuals: bool = False, **kwargs):
     ba = self.bind(*args, return_residuals=return_residuals, **kwargs)
-    for device in infer_devices(ba) or {default_device()}:
+    tensors = ba.tensors
+    for device in {t.device for t in tensors} or {default_device()}:
       if not self.supported_on(device):
         raise NotImplementedError(f"Not supported on {device_kind(device) if device.type == 'cuda' else device}.")
     config = ba.default_config
 
-    tensors = [x for x in _leaves(dict(ba.arguments)) if isinstance(x, torch.Tensor)]
     needs_grad = self.vjp is not None and torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
     if not needs_grad:
       out, residuals = self._fwd(*ba.args, config=config, **ba.kwargs)
@@ -147,14 +148,22 @@ class Op(abc.ABC):
 
   @property
   def _fwd_signature(self) -> inspect.Signature:
-    sig = inspect.signature(self._fwd)
-    params = dict(sig.parameters)
-    del params["config"]
-    return sig.replace(parameters=tuple(params.values()))
+    # Per class, not per call: building a Signature costs tens of microseconds and an op call binds
+    # its arguments several times.
+    sig = _FWD_SIGNATURES.get(type(self))
+    if sig is None:
+      full = inspect.signature(type(self)._fwd)
+      params = [p for name, p in full.parameters.items() if name not in ("self", "config")]
+      sig = full.replace(parameters=tuple(params))
+      _FWD_SIGNATURES[type(self)] = sig
+    return sig
 
   def supported_on(self, device: torch.device) -> bool:
     del device
     return True
+
+
+_FWD_SIGNATURES: dict = {}
 
 
 class CacheKey(tuple):
@@ -195,7 +204,12 @@ class BoundArguments:
   def signature(self) -> inspect.Signature:
     return self.op._fwd_signature  # pylint: disable=protected-access
 
-  @property
+  @functools.cached_property
+  def tensors(self) -> tuple:
+    """Every tensor among the arguments (inside containers and quantised arrays too)."""
+    return tuple(x for x in _leaves(dict(self.arguments)) if isinstance(x, torch.Tensor))
+
+  @functools.cached_property
   def _bound_args(self) -> inspect.BoundArguments:
     return inspect.BoundArguments(self.signature, collections.OrderedDict(self.arguments))
 
@@ -236,7 +250,7 @@ class BoundArguments:
   def heuristics_config(self):
     return self.op._get_heuristics_config(self)  # pylint: disable=protected-access
 
-  @property
+  @functools.cached_property
   def autotuning_cache_key(self):
     return self.op._get_autotuning_cache_key(self)  # pylint: disable=protected-access
 
@@ -289,7 +303,9 @@ class BoundArguments:
 
 
 def _leaves(x):
-  if isinstance(x, dict):
+  if isinstance(x, torch.Tensor) or x is None or isinstance(x, (str, int, float, bool)):
+    yield x
+  elif isinstance(x, dict):
     for v in x.values():
       yield from _leaves(v)
   elif isinstance(x, (tuple, list)):
@@ -305,7 +321,7 @@ def _leaves(x):
 
 
 def infer_devices(ba: BoundArguments) -> set:
-  return {x.device for x in _leaves(dict(ba.arguments)) if isinstance(x, torch.Tensor)}
+  return {x.device for x in ba.tensors}
 
 
 def infer_device_kind(ba: BoundArguments) -> DeviceKind | None:

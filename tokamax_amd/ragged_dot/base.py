@@ -13,6 +13,7 @@ path of its own, so its `_fwd` raises `NotImplementedError` and `HipRaggedDot` i
 from __future__ import annotations
 
 import dataclasses
+import functools
 from typing import Any, Callable, Sequence
 
 import numpy as np
@@ -68,8 +69,18 @@ RAGGED_CONTRACTING_DOT_DIM_NUMS = RaggedDotDimensionNumbers((([0], [0]), ([], []
 
 def generate_group_sizes(*, m: int, num_groups: int, p: Sequence[float] | None = None, seed: int = 0) -> tuple[int, ...]:
   """Random group sizes: `m` draws over `num_groups` groups, counted (base.py:171-196)."""
+  if p is None:
+    return _uniform_group_sizes(m, num_groups, seed)
   rng = np.random.default_rng(seed)
   group_ids = rng.choice(num_groups, (m,), p=p, replace=True)
+  return tuple(map(int, np.bincount(group_ids, minlength=num_groups)))
+
+
+@functools.lru_cache(maxsize=256)
+def _uniform_group_sizes(m: int, num_groups: int, seed: int) -> tuple[int, ...]:
+  # Memoised: the abstract form of a GroupSizes argument asks for this on every op call.
+  rng = np.random.default_rng(seed)
+  group_ids = rng.choice(num_groups, (m,), p=None, replace=True)
   return tuple(map(int, np.bincount(group_ids, minlength=num_groups)))
 
 

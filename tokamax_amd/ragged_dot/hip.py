@@ -99,6 +99,12 @@ _MODE_OF_DIMS = {
 }
 
 
+@functools.lru_cache(maxsize=None)
+def _is_gfx950(device: torch.device) -> bool:
+  arch = getattr(torch.cuda.get_device_properties(device), "gcnArchName", "")
+  return arch.split(":")[0] == "gfx950"
+
+
 @dataclasses.dataclass(frozen=True)
 class HipRaggedDot(base.RaggedDot):
   """Hand-written HIP ragged dot for gfx950. Physical layout `mk,gkn->mn`, rhs never transposed."""
@@ -289,5 +295,4 @@ class HipRaggedDot(base.RaggedDot):
       return True
     if device.type != "cuda" or not torch.cuda.is_available() or torch.version.hip is None:
       return False
-    arch = getattr(torch.cuda.get_device_properties(device), "gcnArchName", "")
-    return arch.split(":")[0] == "gfx950"
+    return _is_gfx950(device)
