@@ -589,11 +589,16 @@ struct GemmKernel {
         for (int i = 0; i < TM; ++i) fa[0][i] = fa[1][i] = Frag{};
 #pragma unroll
         for (int j = 0; j < TN; ++j) fb[0][j] = fb[1][j] = Frag{};
-        // Fragment f of an atom: f < TM is the A fragment of row block f, else the B fragment f - TM.
-        auto read_frag = [&](Frag* a, Frag* b, int f, const unsigned char* stage, int kk) {
+        // Read number r of an atom, in the order the atom's MFMAs (row block major) first use the
+        // fragments: A0, B0, B1, ..., then A1, A2, ... Every fragment is then requested at least
+        // TM*TN - 2 MFMAs before its first use. A fragment f < TM is the A fragment of row block f,
+        // else the B fragment f - TM.
+        auto read_frag = [&](Frag* a, Frag* b, int r, const unsigned char* stage, int kk) {
 #if defined(TKX_ABLATE) && (TKX_ABLATE & 2)
           return;
 #endif
+          if (r >= TM + TN) return;
+          const int f = r == 0 ? 0 : r <= TN ? TM + r - 1 : r - TN;
           if (f < TM) {
             if (F || ((rmask >> f) & 1u)) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, wm * WTM + f * 32, kk, lane);
           } else if (f < TM + TN) {
