@@ -61,8 +61,8 @@ typedef struct TkxConfig {
   int32_t block_k;         /* contraction elements per LDS stage */
   int32_t waves_m;         /* wavefronts along m in a workgroup */
   int32_t waves_n;         /* wavefronts along n in a workgroup */
-  int32_t grid_tile_width; /* m-tasks that share an n-panel in launch order (L2 reuse); unused by the
-                              small-m int8 kernel (block_m == 16) */
+  int32_t grid_tile_width; /* most m-tasks (of one group) that share an n-panel in launch order (L2 reuse);
+                              unused by the small-m int8 kernel (block_m == 16) */
   int32_t align_tile;      /* task starts are aligned down to this many rows (reference default 8) */
   int32_t num_stages;      /* LDS stages of block_k contraction elements kept in flight */
 } TkxConfig;
@@ -83,7 +83,10 @@ int64_t tkx_ragged_dot_workspace_bytes(int64_t m, int64_t num_groups, int32_t bl
 /* Word offsets (int32 units) inside the workspace, for callers/tests that read the schedule back:
  * which = 0 num_tasks (1 word), 1 total_rows (1 word), 2 group_offsets (G+1 words),
  * 3..8 = group_id, block_start, actual_start, actual_end, start_within_block, actual_size
- * (tid_size words each). Returns -1 for an unknown `which`. */
+ * (tid_size words each); 9, 10 = span_first, span_width (tid_size words each): the first task and
+ * the number of tasks of the launch-order span a task belongs to (each group's tasks are cut into
+ * spans of at most grid_tile_width tasks; tkx_ragged_dot_schedule itself uses width 1).
+ * Returns -1 for an unknown `which`. */
 int64_t tkx_ragged_dot_workspace_offset(int64_t m, int64_t num_groups, int32_t block_m, int32_t which);
 
 /* Part (1): group-offset prefix sum + tile schedule, one small kernel on `stream`.

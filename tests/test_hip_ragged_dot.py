@@ -54,6 +54,26 @@ def _check(actual, expected, tol, rows=None):
   assert err <= tol, f"rel_l2 {err:.3e} > {tol}"
 
 
+def _check_spans(ws, m, G, block_m, width, gs):
+  """Launch-order spans: consecutive tasks of one group, at most `width` wide, as even as possible."""
+  lib = _lib.load()
+  tid = lib.tkx_ragged_dot_tid_size(m, G, block_m)
+  arr = lambda which: ws[lib.tkx_ragged_dot_workspace_offset(m, G, block_m, which):][:tid].cpu().numpy()
+  num_tasks = int(ws[0].item())
+  gid, first, wid = arr(3)[:num_tasks], arr(9)[:num_tasks], arr(10)[:num_tasks]
+  assert num_tasks == O.group_info_create_aligned(gs, block_m, tid, 8)["num_tasks"]
+  t = 0
+  while t < num_tasks:
+    w = int(wid[t])
+    assert 1 <= w <= width and int(first[t]) == t and t + w <= num_tasks
+    assert (first[t:t + w] == t).all() and (wid[t:t + w] == w).all() and (gid[t:t + w] == gid[t]).all()
+    t += w
+  for g in np.unique(gid):
+    tasks = int((gid == g).sum())
+    widths = wid[gid == g]
+    assert len(np.unique(first[gid == g])) == -(-tasks // width) and widths.max() - widths.min() <= 1
+
+
 # ---- part (1): offsets and tile schedule, bit exact ----------------------------------------------
 with open(os.path.join(GOLDEN, "scheduler_kat.json")) as _f:
   KAT = json.load(_f)
@@ -116,6 +136,22 @@ def test_simple(dtype, device):
   out = tokamax_amd.ragged_dot(a, b, torch.tensor(gs.astype(np.uint32), device=device), preferred_element_type=torch.float32)
   assert out.dtype == torch.float32
   _check(out, _ref(a, b, gs), TOL[dtype])
+
+
+@pytest.mark.parametrize("width", [1, 3, 8, 16])
+def test_launch_order_spans(width, device):
+  rng = np.random.default_rng(width)
+  G, m, k, n = 9, 2048, 128, 256
+  gs = np.array([300, 0, 129, 1, 640, 0, 7, 512, 130], np.int32)
+  a = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  b = torch.tensor(rng.normal(0, 0.1, (G, k, n)).astype(np.float32), device=device).to(torch.bfloat16)
+  for block_m, cfg in ((128, hip_ops.KernelConfig(128, 128, 64, 2, 2, 2, grid_tile_width=width)),
+                       (32, hip_ops.KernelConfig(32, 128, 64, 1, 4, 4, grid_tile_width=width))):
+    got_ws = []
+    out = hip_ops.ragged_dot_fwd(a, b, torch.tensor(gs, device=device), config=cfg, out_dtype=torch.float32,
+                                 workspace_out=got_ws)
+    _check_spans(got_ws[0], m, G, block_m, width, gs)
+    _check(out, _ref(a, b, gs), 1e-5)
 
 
 def test_padded(device):

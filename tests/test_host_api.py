@@ -46,9 +46,9 @@ def test_workspace_layout_queries():
   assert lib.tkx_ragged_dot_tid_size(1024, 8, 128) == 1024 // 128 + 8 - 1
   assert lib.tkx_ragged_dot_tid_size(65536, 256, 128) == 767  # cdiv(m, block_m) + G - 1
   nbytes = lib.tkx_ragged_dot_workspace_bytes(1024, 8, 128)
-  offs = [lib.tkx_ragged_dot_workspace_offset(1024, 8, 128, w) for w in range(9)]
+  offs = [lib.tkx_ragged_dot_workspace_offset(1024, 8, 128, w) for w in range(11)]
   assert offs[0] == 0 and offs[1] == 1 and offs == sorted(offs) and offs[-1] * 4 + 15 * 4 <= nbytes
-  assert lib.tkx_ragged_dot_workspace_offset(1024, 8, 128, 9) == -1
+  assert lib.tkx_ragged_dot_workspace_offset(1024, 8, 128, 11) == -1
   assert lib.tkx_ragged_dot_workspace_bytes(-1, 8, 128) == -1
 
 

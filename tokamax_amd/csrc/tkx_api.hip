@@ -108,7 +108,7 @@ int64_t tkx_ragged_dot_workspace_offset(int64_t m, int64_t num_groups, int32_t b
   if (which == 0) return 0;
   if (which == 1) return 1;
   if (which == 2) return L.offsets;
-  if (which >= 3 && which <= 8) return L.task[which - 3];
+  if (which >= 3 && which <= 10) return L.task[which - 3];
   return -1;
 }
 
@@ -118,7 +118,7 @@ int32_t tkx_ragged_dot_schedule(const int32_t* group_sizes, int64_t num_groups, 
   if (num_groups < 1 || m < 0) return set_error(TKX_ERR_INVALID, "bad sizes m=%lld G=%lld", (long long)m, (long long)num_groups);
   if (block_m < 1 || align_tile < 1) return set_error(TKX_ERR_INVALID, "block_m and align_tile must be positive");
   const WsLayout L = ws_layout(m, num_groups, block_m);
-  return launch_schedule(group_sizes, num_groups, m, block_m, align_tile, static_cast<int32_t*>(workspace), L,
+  return launch_schedule(group_sizes, num_groups, m, block_m, align_tile, 1, static_cast<int32_t*>(workspace), L,
                          static_cast<hipStream_t>(stream));
 }
 
@@ -174,7 +174,8 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   }
 
   const WsLayout L = ws_layout(m, num_groups, c.block_m);
-  int32_t st = launch_schedule(group_sizes, num_groups, m, c.block_m, c.align_tile, static_cast<int32_t*>(workspace), L, stream);
+  int32_t st = launch_schedule(group_sizes, num_groups, m, c.block_m, c.align_tile, c.grid_tile_width,
+                               static_cast<int32_t*>(workspace), L, stream);
   if (st != TKX_OK) return st;
 
   GemmParams p = {};
@@ -205,6 +206,8 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   p.ws_bstart = (int32_t)L.task[1];
   p.ws_astart = (int32_t)L.task[2];
   p.ws_aend = (int32_t)L.task[3];
+  p.ws_span_first = (int32_t)L.task[6];
+  p.ws_span_width = (int32_t)L.task[7];
   if (slots > 0x7fffff00LL) return set_error(TKX_ERR_UNSUPPORTED, "too many tiles");
   // Extra workgroups zero the rows past sum(group_sizes); they exit at once when there are none.
   int64_t zero_wgs = (m * cols * ob + (64 << 10) - 1) / (64 << 10);
@@ -241,7 +244,7 @@ int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* gr
   // so the workspace size depends on (m, G) alone.
   const int32_t sched_bm = 128;
   const WsLayout L = ws_layout(m, num_groups, sched_bm);
-  int32_t st = launch_schedule(group_sizes, num_groups, m, sched_bm, c.align_tile, static_cast<int32_t*>(workspace), L, stream);
+  int32_t st = launch_schedule(group_sizes, num_groups, m, sched_bm, c.align_tile, 1, static_cast<int32_t*>(workspace), L, stream);
   if (st != TKX_OK) return st;
 
   GemmParams p = {};

@@ -9,14 +9,17 @@
 namespace tkx {
 
 // ---- workspace layout (int32 words) -----------------------------------------------------------
-// [0] num_tasks  [1] total_rows  [kWsHeader ..) group_offsets[G+1]  then six task arrays of
+// [0] num_tasks  [1] total_rows  [kWsHeader ..) group_offsets[G+1]  then eight task arrays of
 // tid_size words each (group_id, block_start, actual_start, actual_end, start_within_block,
-// actual_size); every array starts on a 64-word boundary.
+// actual_size, span_first, span_width); every array starts on a 64-word boundary. The last two
+// are not part of the reference's schedule: they cut each group's tasks into spans of at most
+// grid_tile_width tasks (first task and width of the span a task belongs to), which is the unit
+// the GEMM launch order walks n-panel by n-panel.
 constexpr int64_t kWsHeader = 64;
 
 struct WsLayout {
   int64_t offsets;   // word offset of group_offsets
-  int64_t task[6];   // word offsets of the six task arrays
+  int64_t task[8];   // word offsets of the task arrays
   int64_t words;     // total words
   int32_t tid_size;
 };
@@ -30,7 +33,7 @@ inline WsLayout ws_layout(int64_t m, int64_t G, int32_t block_m) {
   int64_t w = kWsHeader;
   L.offsets = w;
   w += round_up64(G + 1);
-  for (int i = 0; i < 6; ++i) {
+  for (int i = 0; i < 8; ++i) {
     L.task[i] = w;
     w += round_up64(L.tid_size);
   }
@@ -50,7 +53,7 @@ int32_t set_error(int32_t code, const char* fmt, ...);
 
 // ---- schedule -------------------------------------------------------------------------------------
 int32_t launch_schedule(const int32_t* group_sizes, int64_t G, int64_t m, int32_t block_m, int32_t align_tile,
-                        int32_t* ws, const WsLayout& L, hipStream_t stream);
+                        int32_t span_width, int32_t* ws, const WsLayout& L, hipStream_t stream);
 
 // ---- grouped GEMM -----------------------------------------------------------------------------
 enum KernelMode { kFwd = 0, kDlhs = 1, kDrhs = 2 };
@@ -71,7 +74,7 @@ struct GemmParams {
   int32_t real_slots;               // fwd/dlhs: workgroups that may own a task tile (multiple of 8)
   int32_t grid_tile_width;
   int32_t out_dtype, activation;
-  int32_t ws_offsets, ws_gid, ws_bstart, ws_astart, ws_aend;  // word offsets into ws
+  int32_t ws_offsets, ws_gid, ws_bstart, ws_astart, ws_aend, ws_span_first, ws_span_width;  // word offsets into ws
 };
 
 struct Variant {

@@ -439,20 +439,21 @@ struct GemmKernel {
         return;
       }
       // XCD-aware order: consecutive workgroup ids land on different XCDs (id % 8), so give XCD x
-      // the x-th contiguous eighth of the tile list; within it, `grid_tile_width` m-tasks share an
-      // n-panel of B back to back, then move to the next n-panel.
+      // the x-th contiguous eighth of the tile list. The list goes span by span (a span = up to
+      // `grid_tile_width` consecutive m-tasks of one group, laid out by the scheduler); inside a span
+      // its m-tasks take an n-panel of the group's weights back to back, then the next n-panel, so
+      // that the workgroups an XCD runs at a time share panels in its L2.
       const int total = num_tasks * p.n_tiles;
       const int per_xcd = (total + 7) >> 3;
       const int idx = b >> 3, xcd = b & 7;
       if (idx >= per_xcd) return;
       const int L = xcd * per_xcd + idx;
       if (L >= total) return;
-      const int W = p.grid_tile_width;
-      const int span = W * p.n_tiles;
-      const int sg = L / span, rem = L - sg * span;
-      const int wcur = min(W, num_tasks - sg * W);
-      const int nt = rem / wcur;
-      const int mt = sg * W + (rem - nt * wcur);
+      const int t0 = L / p.n_tiles;  // some task of the span that holds L (every task owns n_tiles list entries)
+      const int first = ws[p.ws_span_first + t0], width = ws[p.ws_span_width + t0];
+      const int rem = L - first * p.n_tiles;
+      const int nt = rem / width;
+      const int mt = first + (rem - nt * width);
       group = ws[p.ws_gid + mt];
       row0 = ws[p.ws_bstart + mt];
       act_start = ws[p.ws_astart + mt];

@@ -35,9 +35,10 @@ __device__ inline int32_t block_exclusive_scan(int32_t v, int32_t* buf, int32_t*
 
 __global__ __launch_bounds__(kThreads) void schedule_kernel(const int32_t* __restrict__ group_sizes, int32_t G,
                                                              int32_t tile, int32_t tid_size, int32_t align_tile,
-                                                             int32_t* __restrict__ ws, int64_t off_offsets,
-                                                             int64_t off_gid, int64_t off_bstart, int64_t off_astart,
-                                                             int64_t off_aend, int64_t off_swb, int64_t off_asize) {
+                                                             int32_t span_width, int32_t* __restrict__ ws,
+                                                             int64_t off_offsets, int64_t off_gid, int64_t off_bstart,
+                                                             int64_t off_astart, int64_t off_aend, int64_t off_swb,
+                                                             int64_t off_asize, int64_t off_sfirst, int64_t off_swidth) {
   extern __shared__ int32_t smem[];
   int32_t* scan_buf = smem;                         // 2*kThreads
   int32_t* starts = smem + 2 * kThreads;            // G+1 : exclusive cumsum of clamped sizes
@@ -101,19 +102,38 @@ __global__ __launch_bounds__(kThreads) void schedule_kernel(const int32_t* __res
     ws[off_aend + task] = ve;
     ws[off_swb + task] = vs - bs;
     ws[off_asize + task] = max(0, ve - vs);
+    // Span of this task: the group's T tasks are cut into ceil(T / span_width) spans of nearly equal
+    // width, so that the tasks that run side by side on an n-panel all use the same group's weights.
+    int32_t sfirst = task, swidth = 1;
+    const int32_t T = start_tasks[g + 1] - start_tasks[g], idx = task - start_tasks[g];
+    if (task < num_tasks && idx < T) {
+      const int32_t nspans = (T + span_width - 1) / span_width;
+      const int32_t base = T / nspans, extra = T - base * nspans;  // the first `extra` spans are one wider
+      const int32_t wide = extra * (base + 1);
+      if (idx < wide) {
+        swidth = base + 1;
+        sfirst = idx / swidth * swidth;
+      } else {
+        swidth = base;
+        sfirst = wide + (idx - wide) / base * base;
+      }
+      sfirst += start_tasks[g];
+    }
+    ws[off_sfirst + task] = sfirst;
+    ws[off_swidth + task] = swidth;
   }
 }
 
 }  // namespace
 
 int32_t launch_schedule(const int32_t* group_sizes, int64_t G, int64_t m, int32_t block_m, int32_t align_tile,
-                        int32_t* ws, const WsLayout& L, hipStream_t stream) {
+                        int32_t span_width, int32_t* ws, const WsLayout& L, hipStream_t stream) {
   (void)m;
   const size_t smem = sizeof(int32_t) * (size_t)(2 * kThreads + 2 * (G + 1));
   if (smem > 64 * 1024) return set_error(TKX_ERR_UNSUPPORTED, "num_groups=%lld too large for the scheduler", (long long)G);
-  schedule_kernel<<<1, kThreads, smem, stream>>>(group_sizes, (int32_t)G, block_m, L.tid_size, align_tile, ws,
-                                                L.offsets, L.task[0], L.task[1], L.task[2], L.task[3], L.task[4],
-                                                L.task[5]);
+  schedule_kernel<<<1, kThreads, smem, stream>>>(group_sizes, (int32_t)G, block_m, L.tid_size, align_tile,
+                                                span_width < 1 ? 1 : span_width, ws, L.offsets, L.task[0], L.task[1],
+                                                L.task[2], L.task[3], L.task[4], L.task[5], L.task[6], L.task[7]);
   TKX_HIP_CHECK(hipGetLastError());
   return TKX_OK;
 }

@@ -76,7 +76,8 @@ def workspace(m: int, num_groups: int, block_m: int, device) -> torch.Tensor:
 
 
 def schedule(group_sizes: torch.Tensor, m: int, block_m: int, align_tile: int = 8):
-  """Runs the on-device scheduler; returns (dict of the six task arrays + group_offsets, num_tasks)."""
+  """Runs the on-device scheduler; returns a dict of the six task arrays, the launch-order span
+  arrays (`span_first`, `span_width`; spans are one task wide here), group_offsets and the counters."""
   _require_cuda(group_sizes)
   lib = _lib.load()
   gs = _group_sizes_i32(group_sizes)
@@ -88,6 +89,9 @@ def schedule(group_sizes: torch.Tensor, m: int, block_m: int, align_tile: int = 
   for i, name in enumerate(SCHEDULE_FIELDS):
     off = lib.tkx_ragged_dot_workspace_offset(m, G, block_m, 3 + i)
     out[name] = ws[off:off + tid_size]
+  for i, name in enumerate(("span_first", "span_width")):
+    off = lib.tkx_ragged_dot_workspace_offset(m, G, block_m, 9 + i)
+    out[name] = ws[off:off + tid_size]
   off = lib.tkx_ragged_dot_workspace_offset(m, G, block_m, 2)
   out["group_offsets"] = ws[off:off + G + 1]
   out["num_tasks"] = ws[0:1]
@@ -96,8 +100,11 @@ def schedule(group_sizes: torch.Tensor, m: int, block_m: int, align_tile: int = 
 
 
 def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: torch.dtype, trans_rhs: bool = False,
-                   lhs_scale=None, rhs_scale=None, activation: str | None = None) -> torch.Tensor:
-  """out[m,n] = lhs[m,k] . rhs[g,k,n]   (trans_rhs: out[m,k] = lhs[m,n] . rhs[g,k,n]^T)."""
+                   lhs_scale=None, rhs_scale=None, activation: str | None = None,
+                   workspace_out: list | None = None) -> torch.Tensor:
+  """out[m,n] = lhs[m,k] . rhs[g,k,n]   (trans_rhs: out[m,k] = lhs[m,n] . rhs[g,k,n]^T).
+
+  `workspace_out`, if given, receives the int32 workspace the call filled (schedule arrays included)."""
   _require_cuda(lhs, rhs, group_sizes, lhs_scale, rhs_scale)
   lib = _lib.load()
   if lhs.dim() != 2 or rhs.dim() != 3:
@@ -128,6 +135,8 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
         _lib.TKX_MODE_TRANS_RHS if trans_rhs else _lib.TKX_MODE_DEFAULT, _lib.ACTIVATIONS[activation],
         ctypes.byref(cfg), _stream(lhs.device))
   _lib.check(st)
+  if workspace_out is not None:
+    workspace_out.append(ws)
   return out
 
 
