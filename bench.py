@@ -41,8 +41,8 @@ PEAK_HBM_GBS = 8000.0
 # this script, each scaled by what the same counter reads for a copy kernel of known size; None
 # where no counter run has been made for the current kernel.
 MEASURED_TRAFFIC_BYTES = {
-    "mixtral": 4.460e9,  # 256x256x64 kernel: 3.968e9 read + 0.492e9 written (algorithmic: 1.543e9)
-    "decode": 1.803e8,   # streaming int8 kernel: 1.799e8 read + 3.9e5 written (algorithmic: 1.748e8)
+    "mixtral": 5.93e9,  # 256x256x64 kernel: 5.21e9 read + 0.72e9 written past L2 (algorithmic: 1.543e9)
+    "decode": 1.838e8,  # streaming int8 kernel: 1.834e8 read + 3.9e5 written (algorithmic: 1.748e8)
 }
 
 
