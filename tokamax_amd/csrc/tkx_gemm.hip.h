@@ -250,7 +250,16 @@ struct DirectLoader {
   static constexpr int PER = (INSTRS + NWAVES - 1) / NWAVES;
   static_assert(BYTES % 1024 == 0, "tile must be a whole number of wave-wide 16-byte loads");
 
-  uint32_t voff[PER];  // per-lane byte offset from the wave-uniform base pointer of a k-step
+  // Rows between two consecutive instructions of one wave. In the row/column-contiguous layout the
+  // rows are contraction indices (never clamped) and the swizzle repeats every 8 rows, so when this
+  // is a multiple of 8 the per-lane offsets of a wave's instructions differ by a wave-uniform
+  // stride: one per-lane offset is kept and the stride goes into the scalar base pointer.
+  static constexpr int ROWS_PER_INSTR_STEP = NWAVES * 1024 / ROW_BYTES;
+  static constexpr bool STRIDED = LAYOUT == kMC && (NWAVES * 1024) % ROW_BYTES == 0 && ROWS_PER_INSTR_STEP % 8 == 0;
+  static constexpr int NOFF = STRIDED ? 1 : PER;
+
+  uint32_t voff[NOFF];  // per-lane byte offset from the wave-uniform base pointer of a k-step
+  int64_t stride;       // STRIDED: bytes between consecutive instructions of one wave
 
   // Base pointer of the k-step that starts at contraction index kc0 (uniform across the workgroup).
   static __device__ __forceinline__ int64_t step_base(int rc0, int64_t ld, int kc0) {
@@ -263,8 +272,9 @@ struct DirectLoader {
   }
 
   __device__ __forceinline__ void init(int rc0, int rc_ext, int64_t ld, int wave, int lane) {
+    stride = (int64_t)ROWS_PER_INSTR_STEP * ld * ESZ;
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
+    for (int i = 0; i < NOFF; ++i) {
       const int j = i * NWAVES + wave;
       const int off = j * 1024 + lane * 16;
       const int row = off / ROW_BYTES, pc = (off % ROW_BYTES) >> 4;
@@ -291,7 +301,8 @@ struct DirectLoader {
 #endif
     const int j = i * NWAVES + wave;
     if (INSTRS % NWAVES != 0 && j >= INSTRS) return;
-    direct_load_16(base, voff[i], tile_lds + j * 1024);
+    if constexpr (STRIDED) direct_load_16(base + i * stride, voff[0], tile_lds + j * 1024);
+    else direct_load_16(base, voff[i], tile_lds + j * 1024);
   }
   __device__ __forceinline__ void issue(const unsigned char* base, unsigned tile_lds, int wave) const {
 #pragma unroll
@@ -610,8 +621,11 @@ struct GemmKernel {
         constexpr int NM = TM * TN;                      // MFMAs per atom
         constexpr int RPM = (TM + TN + NM - 1) / NM;     // fragment reads threaded after each MFMA
         constexpr int LPM = (NLD + NM - 1) / NM;         // load slots threaded after each MFMA
-        auto atom = [&](const Frag* a, const Frag* b, Frag* na, Frag* nb, const unsigned char* rd_stage, int rd_kk,
-                        bool reads, bool loads, const StepPtrs& sp) {
+        // (`reads` and `loads` are compile-time tags: a run-time test after every MFMA would put two
+        // branches into each MFMA slot.)
+        auto atom = [&](auto reads_tag, auto loads_tag, const Frag* a, const Frag* b, Frag* na, Frag* nb,
+                        const unsigned char* rd_stage, int rd_kk, const StepPtrs& sp) {
+          constexpr bool reads = decltype(reads_tag)::value, loads = decltype(loads_tag)::value;
 #pragma unroll
           for (int t = 0; t < NM; ++t) {
             const int i = t / TN, j = t % TN;
@@ -636,23 +650,31 @@ struct GemmKernel {
         for (int f = 0; f < TM + TN; ++f) read_frag(fa[0], fb[0], f, smem, 0);
         int cur_stage = 0;
         const StepPtrs none = {};
-        for (int kt = 0; kt < nfull; ++kt) {
+        // One k-step. `refill_tag`: the stage it releases is refilled with k-step kt + NS;
+        // `more_tag`: another k-step follows, so the next stage's first fragments are read.
+        auto k_step = [&](auto refill_tag, auto more_tag, int kt) {
           const unsigned char* cur = smem + cur_stage * STAGE_BYTES;
           const int freed = cur_stage;
           cur_stage = cur_stage + 1 == NS ? 0 : cur_stage + 1;
           const unsigned char* nxt = smem + cur_stage * STAGE_BYTES;
           // (Pointers of the refill are computed here, far ahead of the MFMAs they are issued between.)
-          const bool refill = kt + NS < nfull;
-          const StepPtrs sp = refill ? step_ptrs(kt + NS, freed) : none;
+          const StepPtrs sp = decltype(refill_tag)::value ? step_ptrs(kt + NS, freed) : none;
 #pragma unroll
           for (int kk = 0; kk + 1 < KSTEPS; ++kk)
-            atom(fa[kk & 1], fb[kk & 1], fa[(kk + 1) & 1], fb[(kk + 1) & 1], cur, kk + 1, true, false, none);
+            atom(std::true_type{}, std::false_type{}, fa[kk & 1], fb[kk & 1], fa[(kk + 1) & 1], fb[(kk + 1) & 1], cur,
+                 kk + 1, none);
           // All LDS reads of `cur` are issued. After the barrier the next stage is complete and `cur`
           // is free: the last atom's MFMAs cover the first fragment reads of the next stage and the
           // issue of the loads that refill `cur` with k-step kt + NS.
           step_barrier(kt + NS - 1 < nfull);
-          atom(fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1], fa[0], fb[0], nxt, 0, kt + 1 < nfull, refill, sp);
-        }
+          atom(more_tag, refill_tag, fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1], fa[0], fb[0], nxt, 0, sp);
+        };
+        // Steady state first (every step refills), then the last NS steps in loops of their own, so
+        // that the hot loop is one straight-line body.
+        int kt = 0;
+        for (; kt + NS < nfull; ++kt) k_step(std::true_type{}, std::true_type{}, kt);
+        for (; kt + 1 < nfull; ++kt) k_step(std::false_type{}, std::true_type{}, kt);
+        for (; kt < nfull; ++kt) k_step(std::false_type{}, std::false_type{}, kt);
       };
       if (all_rows) k_loop(std::true_type{});
       else k_loop(std::false_type{});
