@@ -431,6 +431,11 @@ struct GemmKernel {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: all that derives from it is uniform
     const int wm = wave / WN, wn = wave % WN;
+    // The wave's TM row blocks (32 rows each) are interleaved with those of the other waves along
+    // m: block i of wave row wm is block i * WM + wm of the tile. A task that owns only part of the
+    // tile's rows (a group boundary) then leaves every wave row about the same number of blocks
+    // with rows to compute, instead of all of them to one wave row.
+    auto row_block = [&](int i) { return i * WM + wm; };
     const int32_t* ws = p.ws;
     const int b = blockIdx.x;
 
@@ -505,7 +510,7 @@ struct GemmKernel {
     uint32_t rmask = 0;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const int r0 = row0 + wm * WTM + i * 32;
+      const int r0 = row0 + row_block(i) * 32;
       if (r0 < act_end && r0 + 32 > act_start) rmask |= 1u << i;
     }
     rmask = __builtin_amdgcn_readfirstlane(rmask);
@@ -517,7 +522,7 @@ struct GemmKernel {
 #pragma unroll
       for (int i = 0; i < TM; ++i)
         if (decltype(full)::value || ((rmask >> i) & 1u))
-          fa[i] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, wm * WTM + i * 32, kk, lane);
+          fa[i] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, row_block(i) * 32, kk, lane);
       if (decltype(full)::value || rmask != 0) {
 #pragma unroll
         for (int j = 0; j < TN; ++j)
@@ -612,7 +617,7 @@ struct GemmKernel {
           if (r >= TM + TN) return;
           const int f = r == 0 ? 0 : r <= TN ? TM + r - 1 : r - TN;
           if (f < TM) {
-            if (F || ((rmask >> f) & 1u)) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, wm * WTM + f * 32, kk, lane);
+            if (F || ((rmask >> f) & 1u)) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, row_block(f) * 32, kk, lane);
           } else if (f < TM + TN) {
             if (F || rmask != 0)
               b[f - TM] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + (f - TM) * 32, kk, lane);
@@ -666,7 +671,7 @@ struct GemmKernel {
           // All LDS reads of `cur` are issued. After the barrier the next stage is complete and `cur`
           // is free: the last atom's MFMAs cover the first fragment reads of the next stage and the
           // issue of the loads that refill `cur` with k-step kt + NS.
-          step_barrier(kt + NS - 1 < nfull);
+          step_barrier(decltype(refill_tag)::value || kt + NS - 1 < nfull);
           atom(more_tag, refill_tag, fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1], fa[0], fb[0], nxt, 0, sp);
         };
         // Steady state first (every step refills), then the last NS steps in loops of their own, so
@@ -709,7 +714,7 @@ struct GemmKernel {
       if (p.a_scale != nullptr) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-          const int row = min(row0 + wm * WTM + i * 32 + (lane & 31), p.m_ext - 1);
+          const int row = min(row0 + row_block(i) * 32 + (lane & 31), p.m_ext - 1);
           const float rs = p.a_scale[row];
 #pragma unroll
           for (int j = 0; j < TN; ++j)
@@ -766,12 +771,13 @@ struct GemmKernel {
         constexpr int CPR = ROW_BYTES / 16;                       // 16-byte chunks per row
         constexpr int RPI = 64 / CPR;                             // rows per store instruction
         static_assert(64 % CPR == 0 && CPR <= 64, "a store instruction must cover whole rows");
+        static_assert(32 % RPI == 0, "a store instruction must stay inside one 32-row block");
         unsigned char* const slice = smem + wave * WAVE_LDS;
         unsigned char* const tile = const_cast<unsigned char*>(uniform_pointer(Cg + ((int64_t)row0 * p.ldc + col0) * ESZ));
         const int rd_row = lane / CPR, rd_chunk = lane % CPR;
         const int gcol = col0 + wn * WTN + rd_chunk * (16 / ESZ);
         const bool col_ok = inside || gcol + 16 / ESZ <= p.n_ext;
-        const uint32_t voff = (uint32_t)(((wm * WTM + rd_row) * (int)p.ldc + wn * WTN + rd_chunk * (16 / ESZ)) * ESZ);
+        const uint32_t voff = (uint32_t)(((wm * 32 + rd_row) * (int)p.ldc + wn * WTN + rd_chunk * (16 / ESZ)) * ESZ);
 #pragma unroll
         for (int i0 = 0; i0 < TM; i0 += AP) {
 #pragma unroll
@@ -805,14 +811,16 @@ struct GemmKernel {
           constexpr int ROWS = AP * 32;
 #pragma unroll
           for (int s_ = 0; s_ < ROWS / RPI; ++s_) {
-            const int lrow = i0 * 32 + s_ * RPI + rd_row;            // row inside the wave's part of the tile
-            if (lrow >= WTM) continue;
-            const int row = row0 + wm * WTM + lrow;
+            const int srow = s_ * RPI;                                // first slice row of this instruction
+            const int i = i0 + srow / 32;                             // the wave's row block it belongs to
+            if (i >= TM) continue;
+            const int trow = i * WM * 32 + srow % 32;                 // tile row, less the lane part in voff
+            const int row = row0 + trow + wm * 32 + rd_row;
             const i32x4 val = *reinterpret_cast<const i32x4*>(slice + (s_ * RPI + rd_row) * PITCH + rd_chunk * 16);
             // (Non-temporal: the output is not read again by this kernel and should not displace
             // the operand panels the other workgroups of the XCD share in L2.)
             if (row >= act_start && row < act_end && col_ok)
-              __builtin_nontemporal_store(val, (__attribute__((address_space(1))) i32x4*)(tile + (size_t)(i0 * 32 + s_ * RPI) * p.ldc * ESZ + voff));
+              __builtin_nontemporal_store(val, (__attribute__((address_space(1))) i32x4*)(tile + (size_t)trow * p.ldc * ESZ + voff));
           }
         }
       };

@@ -267,14 +267,19 @@ class HipRaggedDot(base.RaggedDot):
     def score(v):
       bm, bn, bk, wm, wn, ns = v
       # drhs streams two row-contiguous operands: shallower k-steps with more stages in flight win there.
-      depth = bk if mode == 2 else -bk
-      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), depth, ns)
+      if mode == 2:
+        return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), 0, bk, ns)
+      # One workgroup per CU (8 waves): what hides the latency of the weight stream is the depth of
+      # contraction in flight, (stages - 1) * block_k; beyond 128 more depth buys nothing, and at
+      # equal depth the longer k-step has fewer barriers per flop.
+      in_flight = min((ns - 1) * bk, 128) if wm * wn == 8 else 0
+      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -in_flight, -bk, ns)
 
     bm, bn, bk, wm, wn, ns = min(usable, key=score)
     # grid_tile_width m-tasks run side by side on an n-panel of one group's weights; that only pays
     # when a group has that many tasks, otherwise neighbours belong to different groups.
     tasks_per_group = rows_per_group / bm
-    width = 8 if tasks_per_group >= 3 else 2
+    width = 16 if tasks_per_group >= 6 else 8 if tasks_per_group >= 3 else 2
     if bm == 16 and key[2] == _lib.TKX_I8:
       width = 1  # the small-m int8 kernel has no tile order to tune
     return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns, grid_tile_width=width,
