@@ -271,7 +271,10 @@ struct DirectLoader {
     else return (int64_t)BK * ld * ESZ;
   }
 
-  __device__ __forceinline__ void init(int rc0, int rc_ext, int64_t ld, int wave, int lane) {
+  // `rc_lo`, `rc_hi`: the rows (contraction-contiguous layout) whose data the caller uses. Rows
+  // outside are redirected to the nearest one inside: that keeps every address valid, and the
+  // lanes of a load that fall outside all fetch one row's cache lines instead of one each.
+  __device__ __forceinline__ void init(int rc0, int rc_ext, int64_t ld, int wave, int lane, int rc_lo, int rc_hi) {
     stride = (int64_t)ROWS_PER_INSTR_STEP * ld * ESZ;
 #pragma unroll
     for (int i = 0; i < NOFF; ++i) {
@@ -281,7 +284,8 @@ struct DirectLoader {
       if constexpr (LAYOUT == kKC) {
         const int lc = pc ^ kc_swizzle<ROW_BYTES>(row);
         int grow = rc0 + row;
-        grow = (grow < rc_ext ? grow : rc_ext - 1) - rc0;
+        grow = grow < rc_hi ? grow : rc_hi - 1;
+        grow = (grow > rc_lo ? grow : rc_lo) - rc0;
         voff[i] = (uint32_t)(grow * (int)ld * ESZ + lc * 16);
       } else {
         const int lc = ((((pc >> 1) ^ mc_swizzle<ROW_BYTES, ES>(row))) << 1) | (pc & 1);
@@ -550,8 +554,9 @@ struct GemmKernel {
     if (nfull > 0) {
       DirA da;
       DirB db;
-      da.init(row0, p.m_ext, p.lda, wave, lane);
-      db.init(col0, p.n_ext, p.ldb, wave, lane);
+      const int a_hi = max(min(act_end, p.m_ext), 1), a_lo = min(max(act_start, 0), a_hi - 1);
+      da.init(row0, p.m_ext, p.lda, wave, lane, a_lo, a_hi);
+      db.init(col0, p.n_ext, p.ldb, wave, lane, 0, p.n_ext);
       const unsigned char* const gA0 = Ab + DirA::step_base(row0, p.lda, kc_begin);
       const unsigned char* const gB0 = Bb + DirB::step_base(col0, p.ldb, kc_begin);
       const int64_t stepA = DirA::step_bytes(p.lda), stepB = DirB::step_bytes(p.ldb);
