@@ -62,7 +62,7 @@ typedef struct TkxConfig {
   int32_t waves_m;         /* wavefronts along m in a workgroup */
   int32_t waves_n;         /* wavefronts along n in a workgroup */
   int32_t grid_tile_width; /* most m-tasks (of one group) that share an n-panel in launch order (L2 reuse);
-                              unused by the small-m int8 kernel (block_m == 16) */
+                              unused by the streaming small-m kernel (block_m == 16) */
   int32_t align_tile;      /* task starts are aligned down to this many rows (reference default 8) */
   int32_t num_stages;      /* LDS stages of block_k contraction elements kept in flight */
 } TkxConfig;

@@ -406,6 +406,43 @@ def test_small_m_int8_kernel_edges(case, depth, device):
                                                  out_dtype=torch.float32, rhs_scale=scale))
 
 
+@pytest.mark.parametrize("depth", [2, 4])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", ["ragged", "two_chunks", "all_empty", "one_big_group"])
+def test_small_m_16bit_weight_kernel_edges(case, dtype, depth, device):
+  """The streaming small-m kernel on 16-bit weights (no scales): same edge cases as with int8 weights,
+  and the public entry picks it for groups of at most 16 rows."""
+  rng = np.random.default_rng(len(case) + depth)
+  k, n = 2048, 208
+  if case == "ragged":
+    gs = np.array([3, 0, 0, 17, 1, 0, 16, 2], np.int32)
+  elif case == "two_chunks":
+    gs = rng.integers(0, 4, 70).astype(np.int32)
+    gs[[0, 63, 64, 69]] = [0, 2, 0, 5]
+  elif case == "all_empty":
+    gs = np.zeros(5, np.int32)
+  else:
+    gs = np.array([0, 45, 0], np.int32)
+  G, m = len(gs), int(gs.sum()) + 11
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(dtype)
+  rhs = torch.tensor(rng.normal(0, k ** -0.5, (G, k, n)).astype(np.float32), device=device).to(dtype)
+  gst = torch.tensor(gs, device=device)
+  cfg = hip_ops.KernelConfig(16, 128, 32, 1, 4, depth)
+  out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32)
+  want = O.ragged_dot(_np(lhs), _np(rhs), gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, 1e-5)  # f32 output of exact 16-bit products
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  out16 = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=dtype)
+  assert torch.equal(out16, out.to(dtype))
+  assert torch.equal(out, hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32))
+  if case == "ragged" and depth == 2:
+    op = tokamax_amd.HipRaggedDot()
+    small = np.array([3, 0, 0, 7, 1, 0, 6, 2], np.int32)
+    assert op._get_heuristics_config(op.bind(lhs[:19], rhs, group_sizes=torch.tensor(small, device=device))).block_m == 16
+    _check(op(lhs[:19], rhs, group_sizes=torch.tensor(small, device=device), preferred_element_type=torch.float32),
+           O.ragged_dot(_np(lhs[:19]), _np(rhs), small, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 1e-5)
+
+
 def test_unsupported_inputs_are_declined(device):
   a = torch.zeros(64, 100, dtype=torch.bfloat16, device=device)  # k not a multiple of any block_k
   b = torch.zeros(2, 100, 64, dtype=torch.bfloat16, device=device)

@@ -30,11 +30,13 @@ struct Registry {
     v = variants_f32(&n);  all.insert(all.end(), v, v + n);
     v = variants_f8(&n);   all.insert(all.end(), v, v + n);
     v = variants_i8w(&n);  all.insert(all.end(), v, v + n);
-    // The streaming small-m kernel for int8 weights is not a tile variant of the GEMM template;
-    // it is listed here (fn == nullptr) so that configs can name it.
-    all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, 2, 0, nullptr});
-    all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, 4, 0, nullptr});
-    all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, 8, 0, nullptr});
+    // The streaming small-m kernel is not a tile variant of the GEMM template; it is listed here
+    // (fn == nullptr, num_stages = steps of loads in flight) so that configs can name it.
+    for (int depth : {2, 4, 8})
+      all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
+    for (int dtype : {TKX_BF16, TKX_F16})
+      for (int depth : {2, 4})
+        all.push_back({kFwd, dtype, dtype, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
   }
 };
 
@@ -165,12 +167,14 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   if (v->fn == nullptr) {
     // Streaming decode kernel: one launch, no schedule.
     if (lhs_scale != nullptr) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no lhs scale");
-    if (!decode_i8w_supported(m, k, n, num_groups))
+    if (rhs_scale != nullptr && rhs_dtype != TKX_I8)
+      return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes an rhs scale with int8 weights only");
+    if (!decode_supported(lhs_dtype, rhs_dtype, m, k, n, num_groups))
       return set_error(TKX_ERR_UNSUPPORTED,
                        "decode kernel needs k %% 1024 == 0 and n %% 8 == 0 (k=%lld n=%lld G=%lld)",
                        (long long)k, (long long)n, (long long)num_groups);
-    return launch_decode_i8w(lhs, rhs, rhs_scale, group_sizes, out, m, k, n, num_groups, out_dtype, activation,
-                             c.num_stages, stream);
+    return launch_decode(lhs, rhs, rhs_scale, group_sizes, out, m, k, n, num_groups, rhs_dtype, out_dtype, activation,
+                         c.num_stages, stream);
   }
 
   const WsLayout L = ws_layout(m, num_groups, c.block_m);

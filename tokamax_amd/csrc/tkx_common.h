@@ -85,12 +85,12 @@ struct Variant {
   const void* fn;  // __global__ void (*)(GemmParams)
 };
 
-// ---- decode (small-m, int8 weights) ------------------------------------------------------------
+// ---- decode (small-m streaming kernel; int8 or 16-bit weights) -----------------------------------
 constexpr int32_t kDecodeBlockM = 16, kDecodeBlockN = 128, kDecodeBlockK = 32, kDecodeWaves = 4, kDecodeStages = 4;
-bool decode_i8w_supported(int64_t m, int64_t k, int64_t n, int64_t G);
-int32_t launch_decode_i8w(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
-                          int64_t m, int64_t k, int64_t n, int64_t G, int32_t out_dtype, int32_t activation,
-                          int32_t depth, hipStream_t stream);
+bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k, int64_t n, int64_t G);
+int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
+                      int64_t m, int64_t k, int64_t n, int64_t G, int32_t rhs_dtype, int32_t out_dtype,
+                      int32_t activation, int32_t depth, hipStream_t stream);
 
 // Each dtype family registers its variants from its own translation unit.
 const Variant* variants_bf16(int* count);

@@ -1,4 +1,5 @@
-// Small-m ("decode") ragged dot with int8 weights: bf16 lhs [m,k] x int8 rhs [G,k,n], f32 scales [G,n].
+// Small-m ("decode") ragged dot: bf16 lhs [m,k] x int8 rhs [G,k,n] with f32 scales [G,n], or
+// bf16 x bf16 / f16 x f16 without scales.
 //
 // This regime is bound by HBM: every touched expert's [k,n] weight panel is read once, and a group
 // has a handful of rows. The kernel is built around streaming those panels:
@@ -12,7 +13,8 @@
 //     (i, q) loads 8 bytes (columns 8i..8i+7) from each of the 8 rows 8q..8q+7 of a 32-row step and
 //     feeds MFMA j (j = 0..7) with byte j of those 8 loads, i.e. 8 contraction values of column
 //     8i+j.  MFMA j therefore produces the output columns {8i+j}; the lhs fragment of lane (r, q) is
-//     lhs[r][8q..8q+7] of the same step, one 16-byte load;
+//     lhs[r][8q..8q+7] of the same step, one 16-byte load. (16-bit weights: 16 bytes per row and the
+//     j-th half-word of each, otherwise the same);
 //   * int8 is widened to bf16 exactly and goes through the 16x16x32 bf16 MFMA with f32 accumulation;
 //   * the four partial tiles are added in a fixed order through LDS (deterministic), scaled per
 //     (group, column), and rows past the group's end are never written.
@@ -29,8 +31,8 @@ constexpr int kDecRows = 16;   // lhs rows per pass
 constexpr int kDecThreads = kDecWaves * 64;
 
 struct DecodeParams {
-  const __bf16* lhs;
-  const signed char* rhs;
+  const unsigned char* lhs;  // 16-bit elements
+  const unsigned char* rhs;  // int8, or 16-bit elements of the lhs type
   const float* scale;
   const int32_t* group_sizes;
   void* out;
@@ -54,6 +56,18 @@ __device__ __forceinline__ i32x2 buffer_load_8(__amdgpu_buffer_rsrc_t r, uint32_
 __device__ __forceinline__ i32x4 buffer_load_16(__amdgpu_buffer_rsrc_t r, uint32_t lane_offset, uint32_t uniform_offset) {
   return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_offset, (int)uniform_offset, 0));
 }
+__device__ __forceinline__ i32x4 buffer_load_16_streaming(__amdgpu_buffer_rsrc_t r, uint32_t lane_offset, uint32_t uniform_offset) {
+  return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_offset, (int)uniform_offset, kStreamingLoad));
+}
+
+// What a lane holds of one weight row of a step: its 8 columns.
+template <int EW> struct WeightRow { typedef i32x4 T; static constexpr int ESZ = 2; };
+template <> struct WeightRow<kEI8> { typedef i32x2 T; static constexpr int ESZ = 1; };
+template <int EW>
+__device__ __forceinline__ typename WeightRow<EW>::T load_weight_row(__amdgpu_buffer_rsrc_t r, uint32_t lane_offset, uint32_t uniform_offset) {
+  if constexpr (EW == kEI8) return buffer_load_8(r, lane_offset, uniform_offset);
+  else return buffer_load_16_streaming(r, lane_offset, uniform_offset);
+}
 
 // Sign-extended byte B of a dword -> f32, one SDWA instruction.
 template <int B>
@@ -69,7 +83,7 @@ __device__ __forceinline__ unsigned i8_to_f32_bits(int w) {
 // Byte J of each of 8 loaded 8-byte rows -> bf16 x8 (exact: |v| <= 128 fits the significand). The
 // upper halves of two f32 are the two bf16, packed with one byte permute.
 template <int J>
-__device__ __forceinline__ bf16x8 column_to_bf16x8(const i32x2 (&rows)[8]) {
+__device__ __forceinline__ i32x4 column_fragment(const i32x2 (&rows)[8]) {
   i32x4 out;
 #pragma unroll
   for (int h = 0; h < 4; ++h) {
@@ -78,11 +92,33 @@ __device__ __forceinline__ bf16x8 column_to_bf16x8(const i32x2 (&rows)[8]) {
     // v_perm_b32 picks bytes from {first operand: bytes 7..4, second operand: bytes 3..0}.
     out[h] = (int)__builtin_amdgcn_perm(f1, f0, 0x07060302u);
   }
-  return __builtin_bit_cast(bf16x8, out);
+  return out;
+}
+// 16-bit weights: half-word J of each of 8 loaded 16-byte rows, two rows per byte permute.
+template <int J>
+__device__ __forceinline__ i32x4 column_fragment(const i32x4 (&rows)[8]) {
+  i32x4 out;
+#pragma unroll
+  for (int h = 0; h < 4; ++h)
+    out[h] = (int)__builtin_amdgcn_perm((unsigned)rows[2 * h + 1][J >> 1], (unsigned)rows[2 * h][J >> 1],
+                                        (J & 1) ? 0x07060302u : 0x05040100u);
+  return out;
+}
+// 16x16x32 MFMA on 8 contraction values per lane of either 16-bit type.
+template <int EA>
+__device__ __forceinline__ f32x4_t mma_16x16x32(i32x4 w, i32x4 a, f32x4_t acc) {
+  if constexpr (EA == kEF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, w), __builtin_bit_cast(f16x8, a), acc, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, a), acc, 0, 0, 0);
 }
 
-template <int kDecDepth, int kMinWgs>
-__global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_i8w_kernel(const DecodeParams p) {
+// EW = element kind of the weights; the lhs is bf16 for int8 weights, else of the weights' type.
+template <int EW, int kDecDepth, int kMinWgs>
+__global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const DecodeParams p) {
+  constexpr int EA = EW == kEI8 ? kEBF16 : EW;
+  constexpr int WESZ = WeightRow<EW>::ESZ;
+  typedef typename WeightRow<EW>::T WRow;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   __shared__ int s_red[kDecWaves];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -100,7 +136,7 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_i8w_kernel(const 
   const int kw = p.k / kDecWaves;      // contraction slice of this wave
   const int k_begin = wave * kw;
   const int steps = kw / kDecKS;       // multiple of kDecDepth (checked on the host)
-  const signed char* wbase = p.rhs + ((int64_t)g * p.k + k_begin) * p.n;
+  const unsigned char* wbase = p.rhs + ((int64_t)g * p.k + k_begin) * p.n * WESZ;
   // B loads: lane (i = lane % 16, q = lane / 16) -> rows 8q + e (e = 0..7), columns col0 + 8i .. 8i+7,
   // clamped at the last 8 columns (n is a multiple of 8; clamped lanes feed columns that are never stored).
   const int li = lane & 15, lq = lane >> 4;
@@ -108,18 +144,18 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_i8w_kernel(const 
   colb = colb < p.n - 8 ? colb : p.n - 8;
   uint32_t boff[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) boff[e] = (uint32_t)((8 * lq + e) * p.n + colb);
+  for (int e = 0; e < 8; ++e) boff[e] = (uint32_t)((8 * lq + e) * p.n + colb) * WESZ;
 
-  i32x2 breg[kDecDepth][8];
+  WRow breg[kDecDepth][8];
   i32x4 areg[kDecDepth];
   // Nothing looks at a loaded value before its step comes up, so the only waits are the per-step
   // vmcnt of the oldest group.
-  const __amdgpu_buffer_rsrc_t wbuf = buffer_of(wbase, (uint32_t)kw * (uint32_t)p.n);
-  const uint32_t step_bytes = (uint32_t)(kDecKS * p.n);
+  const __amdgpu_buffer_rsrc_t wbuf = buffer_of(wbase, (uint32_t)kw * (uint32_t)p.n * WESZ);
+  const uint32_t step_bytes = (uint32_t)(kDecKS * p.n) * WESZ;
   auto issue_b = [&](int slot, int step) {
     const uint32_t so = (uint32_t)__builtin_amdgcn_readfirstlane((int)(step * step_bytes));
 #pragma unroll
-    for (int e = 0; e < 8; ++e) breg[slot][e] = buffer_load_8(wbuf, boff[e], so);
+    for (int e = 0; e < 8; ++e) breg[slot][e] = load_weight_row<EW>(wbuf, boff[e], so);
   };
 #pragma unroll
   for (int d = 0; d < kDecDepth; ++d) {
@@ -169,7 +205,7 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_i8w_kernel(const 
   if (end <= start) return;
 
   // lhs rows of this group as one buffer: rows at or past the group's end read as zero.
-  const __amdgpu_buffer_rsrc_t abuf = buffer_of(p.lhs + (int64_t)start * p.k, (uint32_t)(end - start) * (uint32_t)p.k * 2u);
+  const __amdgpu_buffer_rsrc_t abuf = buffer_of(p.lhs + (int64_t)start * p.k * 2, (uint32_t)(end - start) * (uint32_t)p.k * 2u);
 
   for (int rb = start; rb < end; rb += kDecRows) {
     // A fragments: lane (i, q) holds lhs[rb + i][k + 8q .. 8q+7].
@@ -195,20 +231,20 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_i8w_kernel(const 
 #pragma unroll
       for (int d = 0; d < kDecDepth; ++d) {
         const int s = s0 + d;
-        const bf16x8 afrag = __builtin_bit_cast(bf16x8, areg[d]);
+        const i32x4 afrag = areg[d];
         // MFMA j contracts this step's 32 rows for the columns {8i + j}; operands are swapped, so a
         // lane ends up with one lhs row and the weight-column indices 4q..4q+3.
-        bf16x8 lo[4], hi[4];
-        lo[0] = column_to_bf16x8<0>(breg[d]);
-        lo[1] = column_to_bf16x8<1>(breg[d]);
-        lo[2] = column_to_bf16x8<2>(breg[d]);
-        lo[3] = column_to_bf16x8<3>(breg[d]);
+        i32x4 lo[4], hi[4];
+        lo[0] = column_fragment<0>(breg[d]);
+        lo[1] = column_fragment<1>(breg[d]);
+        lo[2] = column_fragment<2>(breg[d]);
+        lo[3] = column_fragment<3>(breg[d]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lo[j], afrag, acc[j], 0, 0, 0);
-        hi[0] = column_to_bf16x8<4>(breg[d]);
-        hi[1] = column_to_bf16x8<5>(breg[d]);
-        hi[2] = column_to_bf16x8<6>(breg[d]);
-        hi[3] = column_to_bf16x8<7>(breg[d]);
+        for (int j = 0; j < 4; ++j) acc[j] = mma_16x16x32<EA>(lo[j], afrag, acc[j]);
+        hi[0] = column_fragment<4>(breg[d]);
+        hi[1] = column_fragment<5>(breg[d]);
+        hi[2] = column_fragment<6>(breg[d]);
+        hi[3] = column_fragment<7>(breg[d]);
         // Refill unconditionally: past the wave's slice the weight buffer reads as zero without
         // touching memory, and a uniform loop body keeps the waits partial. The scheduling fences
         // keep the compiler from sinking the loads to the end of the block, which would collapse
@@ -217,7 +253,7 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_i8w_kernel(const 
         issue_b(d, s + kDecDepth);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi[j], afrag, acc[4 + j], 0, 0, 0);
+        for (int j = 0; j < 4; ++j) acc[4 + j] = mma_16x16x32<EA>(hi[j], afrag, acc[4 + j]);
         // The lhs refill goes into the registers the MFMAs above read, so it follows them.
         __builtin_amdgcn_sched_barrier(0);
         issue_a(d, s + kDecDepth);
@@ -281,19 +317,23 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_i8w_kernel(const 
 }  // namespace
 
 // Whether the decode kernel can run this problem (else the caller uses the tiled kernel).
-bool decode_i8w_supported(int64_t m, int64_t k, int64_t n, int64_t G) {
+bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k, int64_t n, int64_t G) {
   (void)m;
   (void)G;
-  if ((k / kDecWaves) * n >= (1LL << 31)) return false;
+  const bool types = (lhs_dtype == TKX_BF16 && (rhs_dtype == TKX_I8 || rhs_dtype == TKX_BF16)) ||
+                     (lhs_dtype == TKX_F16 && rhs_dtype == TKX_F16);
+  if (!types) return false;
+  const int64_t wesz = rhs_dtype == TKX_I8 ? 1 : 2;
+  if ((k / kDecWaves) * n * wesz >= (1LL << 31)) return false;
   return k % (kDecWaves * kDecKS * 8) == 0 && n % 8 == 0 && n >= 8;
 }
 
-int32_t launch_decode_i8w(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
-                          int64_t m, int64_t k, int64_t n, int64_t G, int32_t out_dtype, int32_t activation,
-                          int32_t depth, hipStream_t stream) {
+int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
+                      int64_t m, int64_t k, int64_t n, int64_t G, int32_t rhs_dtype, int32_t out_dtype,
+                      int32_t activation, int32_t depth, hipStream_t stream) {
   DecodeParams p;
-  p.lhs = static_cast<const __bf16*>(lhs);
-  p.rhs = static_cast<const signed char*>(rhs);
+  p.lhs = static_cast<const unsigned char*>(lhs);
+  p.rhs = static_cast<const unsigned char*>(rhs);
   p.scale = scale;
   p.group_sizes = group_sizes;
   p.out = out;
@@ -309,10 +349,19 @@ int32_t launch_decode_i8w(const void* lhs, const void* rhs, const float* scale, 
   const int64_t grid = G * p.n_tiles;
   if (grid > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "too many workgroups");
   // `depth` = steps of loads in flight per wave; deeper pipelines need more registers and allow
-  // fewer waves per CU.
-  const void* fn = depth <= 2   ? reinterpret_cast<const void*>(&decode_i8w_kernel<2, 4>)
-                   : depth <= 4 ? reinterpret_cast<const void*>(&decode_i8w_kernel<4, 3>)
-                                : reinterpret_cast<const void*>(&decode_i8w_kernel<8, 2>);
+  // fewer waves per CU. A step of 16-bit weights takes twice the registers of an int8 one.
+  const void* fn;
+  if (rhs_dtype == TKX_I8) {
+    fn = depth <= 2   ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 2, 4>)
+         : depth <= 4 ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 4, 3>)
+                      : reinterpret_cast<const void*>(&decode_kernel<kEI8, 8, 2>);
+  } else if (rhs_dtype == TKX_BF16) {
+    fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEBF16, 2, 3>)
+                    : reinterpret_cast<const void*>(&decode_kernel<kEBF16, 4, 2>);
+  } else {
+    fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEF16, 2, 3>)
+                    : reinterpret_cast<const void*>(&decode_kernel<kEF16, 4, 2>);
+  }
   DecodeParams params = p;
   void* args[] = {&params};
   TKX_HIP_CHECK(hipLaunchKernel(fn, dim3((unsigned)grid), dim3(kDecThreads), args, smem, stream));

@@ -253,15 +253,18 @@ class HipRaggedDot(base.RaggedDot):
     variants = _variant_table().get(key)
     if not variants:
       raise NotImplementedError(f"No hip kernel for dtypes/mode {key}.")
-    usable = list(variants)
-    if key[2] == _lib.TKX_I8:
-      # The streaming small-m kernel (block_m == 16) needs k % 1024 == 0 and n % 8 == 0.
-      usable = [v for v in usable if v[0] != 16 or (contraction % 1024 == 0 and cols % 8 == 0)]
+    # The streaming small-m kernel (listed with block_m == 16; forward only) needs k % 1024 == 0 and
+    # n % 8 == 0, and a weight slice (k/4 rows of n) that a 32-bit buffer offset spans.
+    wbytes = 1 if key[2] == _lib.TKX_I8 else 2
+    streaming_ok = (mode == 0 and contraction % 1024 == 0 and cols % 8 == 0
+                    and (contraction // 4) * cols * wbytes < 2**31)
+    usable = [v for v in variants if v[0] != 16 or streaming_ok]
     # Rows per group decide the m-tile: a tile much taller than a group wastes MFMA work on rows
     # that are masked out at the store; a short tile re-reads the weights more often.
     rows_per_group = rows / max(num_groups, 1) if mode != 2 else rows
     want_m = (256 if rows_per_group >= 1024 else 128 if rows_per_group >= 192 else 64 if rows_per_group >= 48
-              else 32 if rows_per_group > 16 else 16)
+              else 32 if rows_per_group > 8 else 16)  # 16 = one pass of the streaming kernel; the mean must
+    # leave room for the largest group, which re-reads its weights for every further 16 rows
     want_n = 256 if cols >= 2048 else 128
 
     def score(v):
@@ -280,8 +283,8 @@ class HipRaggedDot(base.RaggedDot):
     # when a group has that many tasks, otherwise neighbours belong to different groups.
     tasks_per_group = rows_per_group / bm
     width = 16 if tasks_per_group >= 6 else 8 if tasks_per_group >= 3 else 2
-    if bm == 16 and key[2] == _lib.TKX_I8:
-      width = 1  # the small-m int8 kernel has no tile order to tune
+    if bm == 16:
+      width = 1  # the streaming small-m kernel has no tile order to tune
     return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns, grid_tile_width=width,
                   align_tile=8)
 
@@ -289,7 +292,7 @@ class HipRaggedDot(base.RaggedDot):
     mode, key, _, _, _, _ = self._problem(ba)
     configs = set()
     for bm, bn, bk, wm, wn, ns in _variant_table().get(key, []):
-      widths = (1,) if (mode == 2 or (bm == 16 and key[2] == _lib.TKX_I8)) else (1, 2, 4, 8, 16)
+      widths = (1,) if (mode == 2 or bm == 16) else (1, 2, 4, 8, 16)
       for w in widths:
         configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns,
                            grid_tile_width=w))
