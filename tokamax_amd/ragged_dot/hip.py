@@ -279,10 +279,11 @@ class HipRaggedDot(base.RaggedDot):
       return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -in_flight, -bk, ns)
 
     bm, bn, bk, wm, wn, ns = min(usable, key=score)
-    # grid_tile_width m-tasks run side by side on an n-panel of one group's weights; that only pays
-    # when a group has that many tasks, otherwise neighbours belong to different groups.
-    tasks_per_group = rows_per_group / bm
-    width = 16 if tasks_per_group >= 6 else 8 if tasks_per_group >= 3 else 2
+    # grid_tile_width m-tasks of one group run side by side on an n-panel of its weights (a span never
+    # crosses a group, so small groups simply get short spans). With the 32 tiles an XCD runs at a
+    # time, 8 wide x 4 n-panels needs the fewest distinct operand panels in its L2; 16 wide measured
+    # the same speed on the Mixtral shape with 50% more traffic past L2.
+    width = 8
     if bm == 16:
       width = 1  # the streaming small-m kernel has no tile order to tune
     return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns, grid_tile_width=width,
