@@ -200,7 +200,8 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   p.num_groups = (int32_t)num_groups;
   p.n_tiles = (int32_t)((cols + c.block_n - 1) / c.block_n);
   p.m_tiles = 0;
-  const int64_t slots = ((int64_t)L.tid_size * p.n_tiles + 7) / 8 * 8;
+  // Whole chunks for every XCD, so that each list entry has a workgroup (see the launch order in run()).
+  const int64_t slots = ((int64_t)L.tid_size * p.n_tiles + 8 * kXcdChunk - 1) / (8 * kXcdChunk) * (8 * kXcdChunk);
   p.real_slots = (int32_t)slots;
   p.grid_tile_width = c.grid_tile_width;
   p.out_dtype = out_dtype;

@@ -58,6 +58,10 @@ int32_t launch_schedule(const int32_t* group_sizes, int64_t G, int64_t m, int32_
 // ---- grouped GEMM -----------------------------------------------------------------------------
 enum KernelMode { kFwd = 0, kDlhs = 1, kDrhs = 2 };
 
+// fwd/dlhs launch order: the tile list is dealt to the 8 XCDs in chunks of this many consecutive
+// tiles (the number of CUs of an XCD: one chunk is what an XCD runs at a time).
+constexpr int32_t kXcdChunk = 32;
+
 struct GemmParams {
   const void* A;
   const void* B;
@@ -71,7 +75,7 @@ struct GemmParams {
   int32_t m_ext, n_ext, k_ext;      // extents of the C rows, C columns and the contraction
   int32_t num_groups;
   int32_t n_tiles, m_tiles;         // tiles along C columns; along C rows (drhs only)
-  int32_t real_slots;               // fwd/dlhs: workgroups that may own a task tile (multiple of 8)
+  int32_t real_slots;               // fwd/dlhs: workgroups that may own a task tile (multiple of 8 * kXcdChunk)
   int32_t grid_tile_width;
   int32_t out_dtype, activation;
   int32_t ws_offsets, ws_gid, ws_bstart, ws_astart, ws_aend, ws_span_first, ws_span_width;  // word offsets into ws

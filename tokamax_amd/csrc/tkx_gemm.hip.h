@@ -458,16 +458,17 @@ struct GemmKernel {
           *reinterpret_cast<i32x4*>(c + o) = z;
         return;
       }
-      // XCD-aware order: consecutive workgroup ids land on different XCDs (id % 8), so give XCD x
-      // the x-th contiguous eighth of the tile list. The list goes span by span (a span = up to
-      // `grid_tile_width` consecutive m-tasks of one group, laid out by the scheduler); inside a span
-      // its m-tasks take an n-panel of the group's weights back to back, then the next n-panel, so
-      // that the workgroups an XCD runs at a time share panels in its L2.
+      // XCD-aware order: consecutive workgroup ids land on different XCDs (id % 8). The tile list is
+      // dealt out in chunks of kXcdChunk consecutive tiles, chunk c to XCD c % 8, so that the
+      // workgroups an XCD runs at a time are consecutive in the list and the 8 XCDs work on
+      // neighbouring chunks. The list goes span by span (a span = up to `grid_tile_width`
+      // consecutive m-tasks of one group, laid out by the scheduler); inside a span its m-tasks take
+      // an n-panel of the group's weights back to back, then the next n-panel: the tiles of a chunk
+      // share panels in their XCD's L2, and neighbouring chunks share the span's lhs panels in the
+      // memory-side cache.
       const int total = num_tasks * p.n_tiles;
-      const int per_xcd = (total + 7) >> 3;
       const int idx = b >> 3, xcd = b & 7;
-      if (idx >= per_xcd) return;
-      const int L = xcd * per_xcd + idx;
+      const int L = ((idx / kXcdChunk) * 8 + xcd) * kXcdChunk + idx % kXcdChunk;
       if (L >= total) return;
       const int t0 = L / p.n_tiles;  // some task of the span that holds L (every task owns n_tiles list entries)
       const int first = ws[p.ws_span_first + t0], width = ws[p.ws_span_width + t0];
