@@ -837,8 +837,9 @@ struct GemmKernel {
   }
 };
 
+// (4-wave workgroups: at most 256 registers per lane, so that two of them fit a CU when their LDS does.)
 template <class K>
-__global__ __launch_bounds__(K::THREADS) void gemm_entry(const GemmParams p) {
+__global__ __launch_bounds__(K::THREADS, K::THREADS <= 256 ? 2 : 1) void gemm_entry(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char tkx_smem[];
   K::run(p, tkx_smem);
 }

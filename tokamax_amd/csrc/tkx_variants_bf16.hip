@@ -14,6 +14,7 @@ static const Variant kVariants[] = {
     FWD_DLHS(128, 256, 64, 2, 4, 3),
     FWD_DLHS(128, 256, 64, 2, 2, 3),
     FWD_DLHS(128, 256, 32, 2, 4, 5),
+    FWD_DLHS(128, 256, 32, 2, 2, 3),
     FWD_DLHS(128, 128, 64, 2, 2, 4),
     FWD_DLHS(128, 128, 64, 2, 2, 2),
     FWD_DLHS(64, 256, 64, 2, 2, 3),
@@ -23,6 +24,8 @@ static const Variant kVariants[] = {
     DRHS(256, 256, 64, 2, 4, 2),
     DRHS(256, 256, 32, 2, 4, 4),
     DRHS(128, 256, 64, 2, 4, 3),
+    DRHS(128, 256, 32, 2, 2, 3),
+    DRHS(256, 128, 32, 2, 2, 3),
     DRHS(128, 128, 64, 2, 2, 4),
     DRHS(64, 128, 64, 2, 2, 4),
 };

@@ -8,9 +8,12 @@ namespace tkx {
 
 static const Variant kVariants[] = {
     FWD_DLHS(256, 256, 32, 2, 4, 4),
+    FWD_DLHS(128, 256, 64, 2, 4, 3),
     FWD_DLHS(128, 128, 64, 2, 2, 4),
     FWD_DLHS(32, 128, 64, 1, 4, 4),
     DRHS(128, 128, 64, 2, 2, 4),
+    DRHS(256, 128, 32, 2, 2, 3),
+    DRHS(256, 256, 32, 2, 4, 4),
 };
 
 const Variant* variants_f16(int* count) {

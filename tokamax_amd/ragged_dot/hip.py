@@ -271,11 +271,16 @@ class HipRaggedDot(base.RaggedDot):
       bm, bn, bk, wm, wn, ns = v
       # drhs streams two row-contiguous operands: shallower k-steps with more stages in flight win there.
       if mode == 2:
+        # A group's contraction (its rows) is short next to the tile it produces, so the store of a
+        # tile weighs as much as its MFMAs: up to about 1500 rows per group two 4-wave workgroups
+        # per CU (one stores while the other computes) beat one 8-wave workgroup with the larger tile.
+        if contraction / max(num_groups, 1) < 1536:
+          return (abs(bm - 256), abs(bn - 128), abs(wm * wn - 4), 0, bk, ns)
         return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), 0, bk, ns)
       # One workgroup per CU (8 waves): what hides the latency of the weight stream is the depth of
-      # contraction in flight, (stages - 1) * block_k; beyond 128 more depth buys nothing, and at
-      # equal depth the longer k-step has fewer barriers per flop.
-      in_flight = min((ns - 1) * bk, 128) if wm * wn == 8 else 0
+      # contraction in flight, (stages - 1) * block_k; beyond 96 more depth buys nothing (it measured
+      # 1.5% slower), and at equal depth the longer k-step has fewer barriers per flop.
+      in_flight = min((ns - 1) * bk, 96) if wm * wn == 8 else 0
       return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -in_flight, -bk, ns)
 
     bm, bn, bk, wm, wn, ns = min(usable, key=score)
