@@ -277,6 +277,33 @@ def main():
     measure("vjp_drhs_bf16", lambda: op(w.lhs, w.dout, group_sizes=gs, ragged_dot_dimension_numbers=base.RAGGED_CONTRACTING_DOT_DIM_NUMS),
             w.flops, nb, "mfma", "bf16", cfg)
     del w
+
+    # Mixtral FFN-1 with the gate and up projections in one call (weights [G, k, 2n]) and
+    # silu(gate) * up applied in the kernel's epilogue; also the 16-bit-weight small-m kernel.
+    gsz = workloads.router_top2_group_sizes(8192, 8, 0)
+    gs = torch.tensor(gsz, device=device)
+    gen = torch.Generator(device=device).manual_seed(0)
+    m_, k_, n_ = int(gsz.sum()), 4096, 14336
+    lhs = torch.randn(m_, k_, device=device, dtype=torch.bfloat16, generator=gen)
+    rhs = (torch.randn(8, k_, 2 * n_, device=device, dtype=torch.float32, generator=gen) * k_ ** -0.5).to(torch.bfloat16)
+    cfg = op.bind(lhs, rhs, group_sizes=gs, fuse_gateup_activation="silu").default_config
+    nb = (m_ * k_ + 8 * k_ * 2 * n_ + m_ * n_) * 2
+    measure("mixtral_gateup_silu_bf16", lambda: op(lhs, rhs, group_sizes=gs, fuse_gateup_activation="silu"),
+            2 * m_ * k_ * 2 * n_, nb, "mfma", "bf16", cfg)
+    del lhs, rhs
+
+    w = workloads.make("decode", device, seed=0)
+    gs = torch.tensor(w.group_sizes, device=device)
+    copies = [(torch.randn(w.num_groups, w.k, w.n, device=device, dtype=torch.float32, generator=gen) * w.k ** -0.5)
+              .to(torch.bfloat16) for _ in range(3)]
+    cfg = op.bind(w.lhs, copies[0], group_sizes=gs).default_config
+    nb16 = (w.nonempty_groups * w.k * w.n + w.m * w.k + w.m * w.n) * 2
+    m16 = _time_graph([(lambda r=r: op(w.lhs, r, group_sizes=gs)) for r in copies], 24)
+    extras["decode_bf16_weights_cold"] = dict(
+        ms_per_step=round(m16, 5), gbs=round(nb16 / m16 / 1e6, 2), timing="HIP graph of 24 back-to-back launches",
+        roofline=_roofline("hbm", w.flops, nb16, m16, "bf16"),
+        kernel_config=[cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages])
+    del w, copies
     result["extras"] = extras
 
   print(json.dumps(result), flush=True)

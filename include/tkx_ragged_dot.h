@@ -14,6 +14,9 @@
  *                               dispatched by pallas_mosaic_gpu.py:103-244, for
  *                               DEFAULT_RAGGED_DOT_DIM_NUMS (base.py:40-44) and
  *                               TRANS_RHS_RAGGED_DOT_DIM_NUMS (base.py:45-49, the dlhs of base.py:434-446)
+ *   tkx_ragged_dot_fwd_fused    the `rhs_bias` and `fuse_gateup_activation` arguments of RaggedDot
+ *                               (base.py:205-217, :242-245): ragged_dot(lhs, rhs) + rhs_bias, and
+ *                               activate(tmp[:, :n]) * tmp[:, n:] with tmp = ragged_dot(lhs, [gate, up])
  *   tkx_ragged_dot_drhs         RAGGED_CONTRACTING_DOT_DIM_NUMS (base.py:50-54), the drhs of
  *                               base.py:448-461; kernel counterpart pallas_mosaic_gpu_kernel_sm90.py:184-285
  *   TkxConfig                   pallas_mosaic_gpu_common.py:45-73 (Config)
@@ -108,6 +111,19 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
                            int32_t rhs_dtype, int32_t out_dtype, int32_t mode, int32_t activation,
                            const TkxConfig* config, tkx_stream_t stream);
 
+/* Forward (mode DEFAULT) with the fused epilogue terms of base.py:205-217.
+ *   rhs_bias: f32[G,n] added to the scaled accumulator, or NULL.
+ *   gateup = 1: rhs is [G,k,n] with its columns [gate | up] (n/2 each) and out is [m, n/2] =
+ *     act(lhs.gate + bias_gate) * (lhs.up + bias_up), `activation` (not NONE) naming act; needs
+ *     n % 16 == 0, k % block_k == 0 and a variant of mode 3 (see tkx_ragged_dot_variant).
+ *   gateup = 0: as tkx_ragged_dot_fwd plus the bias; `activation` applies to the biased result.
+ * The streaming small-m kernel (block_m == 16) takes neither. */
+int32_t tkx_ragged_dot_fwd_fused(const void* lhs, const void* rhs, const int32_t* group_sizes,
+                                 const float* lhs_scale, const float* rhs_scale, const float* rhs_bias, void* out,
+                                 void* workspace, int64_t m, int64_t k, int64_t n, int64_t num_groups,
+                                 int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype, int32_t activation,
+                                 int32_t gateup, const TkxConfig* config, tkx_stream_t stream);
+
 /* Part (4-drhs): out[G,k,n] = lhs[rows_g, k]^T . dout[rows_g, n], zeros for empty groups.
  * lhs [m,k], dout [m,n] row-major of `dtype` (f32/bf16/f16); out_dtype f32/bf16/f16.
  * Deterministic: one workgroup owns each output tile, no atomics. block_m/block_n of `config`
@@ -118,7 +134,8 @@ int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* gr
 
 /* Enumerates compiled kernel variants, for the autotuner's search space.
  * kind: 0 = fwd/dlhs variants, 1 = drhs variants.  Returns the count; tkx_ragged_dot_variant fills
- * `config` (tile + wave fields) and the dtype pair of variant `index`, returning 0, or TKX_ERR_INVALID. */
+ * `config` (tile + wave fields), the dtype pair and the mode of variant `index` (0 = fwd, 1 = dlhs,
+ * 2 = drhs, 3 = fwd with gate-up fusion), returning 0, or TKX_ERR_INVALID. */
 int32_t tkx_ragged_dot_num_variants(int32_t kind);
 int32_t tkx_ragged_dot_variant(int32_t kind, int32_t index, TkxConfig* config, int32_t* lhs_dtype,
                                int32_t* rhs_dtype, int32_t* mode);

@@ -29,8 +29,17 @@ below therefore cites the reference call site it follows, and says what pins it:
   generate_group_sizes         base.py:171-196                                    invariants of base_test.py:45-51
                                                                                   (len == G, sum == m) + literal restatement
 
+  ragged_dot_fused             base.py:205-217 (docstring of `rhs_bias` and       composition of `ragged_dot` with the
+                               `fuse_gateup_activation`)                          formulas of that docstring; the
+                                                                                  activations against torch's silu /
+                                                                                  gelu(approximate="tanh")
+
 Status of "parity unpinned": `qwix.quantize` (absmax calibration / rounding) is
 NOT restated -- quantised inputs are generated directly as (qvalue, scale) pairs.
+`ragged_dot_fused` follows the docstring's formulas only: the one reference
+backend that computes them (pallas_mosaic_tpu_v2.py:205-250) calls a kernel that
+is not in the tree, so the flavour of "gelu" (taken as jax.nn.gelu's default
+tanh form) and "swigluoai" (not restated) are parity unpinned.
 Everything else above has a pin listed.
 """
 
@@ -242,6 +251,36 @@ def ragged_dot(lhs, rhs, group_sizes, mode: str = DEFAULT, *, acc_dtype=np.float
   else:
     raise ValueError(mode)
   return _round_out(out, out_dtype)
+
+
+def silu(x):
+  return x / (1.0 + np.exp(-x))
+
+
+def gelu_tanh(x):
+  return 0.5 * x * (1.0 + np.tanh(0.7978845608028654 * (x + 0.044715 * x ** 3)))
+
+
+def ragged_dot_fused(lhs, rhs, group_sizes, *, rhs_bias=None, gateup_activation=None, acc_dtype=np.float64,
+                     out_dtype: str = "f64"):
+  """`ragged_dot(lhs, rhs) + rhs_bias`, then `act(tmp[:, :n]) * tmp[:, n:]` (base.py:205-217).
+
+  `rhs_bias` is [G, 1, 2n] (or [G, 2n]): row i gets the bias of its group; rows past the last group
+  stay zero. `gateup_activation` is "silu" or "gelu" (tanh form); None leaves `tmp` as it is.
+  """
+  tmp = np.asarray(ragged_dot(lhs, rhs, group_sizes, DEFAULT, acc_dtype=acc_dtype, out_dtype="f64"), np.float64)
+  off = group_offsets(group_sizes)
+  if rhs_bias is not None:
+    bias = np.asarray(rhs_bias, np.float64).reshape(len(off) - 1, -1)
+    for g in range(len(off) - 1):
+      s, e = int(off[g]), min(int(off[g + 1]), tmp.shape[0])
+      if e > s:
+        tmp[s:e] += bias[g]
+  if gateup_activation is not None:
+    act = {"silu": silu, "gelu": gelu_tanh}[gateup_activation]
+    n = tmp.shape[1] // 2
+    tmp = act(tmp[:, :n]) * tmp[:, n:]
+  return _round_out(tmp, out_dtype)
 
 
 def ragged_dot_bruteforce(lhs, rhs, group_sizes, mode: str = DEFAULT):

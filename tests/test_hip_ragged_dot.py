@@ -339,6 +339,15 @@ def test_every_kernel_variant_through_c_abi(v, device):
                              grid_tile_width=3)
   lt, rt = _TORCH_DTYPE[v["lhs_dtype"]], _TORCH_DTYPE[v["rhs_dtype"]]
   mk = lambda shape, std: torch.tensor(rng.normal(0, std, shape).astype(np.float32), device=device)
+  if v["mode"] == 3:  # forward with gate-up fusion and a bias: rhs [g, k, 2 n'] -> out [m, n']
+    lhs, rhs = mk((m, k), 1.0).to(lt), mk((G, k, n), k ** -0.5).to(rt)
+    bias = mk((G, 1, n), 0.5)
+    out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, rhs_bias=bias, activation="silu",
+                                 gateup=True)
+    want = O.ragged_dot_fused(_np(lhs), _np(rhs), gs, rhs_bias=_np(bias), gateup_activation="silu")
+    _check(out, want, 1e-5)
+    assert out.shape == (m, n // 2) and torch.count_nonzero(out[int(gs.sum()):]) == 0
+    return
   if v["mode"] == 2:
     lhs, dout = mk((m, k), 1.0).to(lt), mk((m, n), 1.0).to(lt)
     out = hip_ops.ragged_dot_drhs(lhs, dout, gst, G, config=cfg, out_dtype=torch.float32)
@@ -441,6 +450,44 @@ def test_small_m_16bit_weight_kernel_edges(case, dtype, depth, device):
     assert op._get_heuristics_config(op.bind(lhs[:19], rhs, group_sizes=torch.tensor(small, device=device))).block_m == 16
     _check(op(lhs[:19], rhs, group_sizes=torch.tensor(small, device=device), preferred_element_type=torch.float32),
            O.ragged_dot(_np(lhs[:19]), _np(rhs), small, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 1e-5)
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("m,k,n2,gs", [
+    (300, 256, 512, [100, 0, 57, 120]),          # ragged groups, an empty one, a tail of 23 rows
+    (64, 128, 144, [5, 7, 0, 40]),               # n' = 72: not a multiple of the tile's 128 output columns
+    (1100, 512, 1024, [1024, 0, 76]),            # a group of several 256-row tasks
+])
+def test_rhs_bias_and_gateup_fusion(m, k, n2, gs, act, device):
+  """`rhs_bias` and `fuse_gateup_activation` through the op (base.py:205-217) against the oracle's
+  composition; bf16 inputs, f32 and bf16 outputs; the bias alone, with and without an activation."""
+  rng = np.random.default_rng(m + n2)
+  gs = np.array(gs, np.int32)
+  G = len(gs)
+  gst = torch.tensor(gs, device=device)
+  mk = lambda shape, std: torch.tensor(rng.normal(0, std, shape).astype(np.float32), device=device)
+  lhs, rhs = mk((m, k), 1.0).to(torch.bfloat16), mk((G, k, n2), k ** -0.5).to(torch.bfloat16)
+  bias = mk((G, 1, n2), 0.7).to(torch.bfloat16)
+  op = tokamax_amd.HipRaggedDot()
+  out = op(lhs, rhs, group_sizes=gst, rhs_bias=bias, fuse_gateup_activation=act, preferred_element_type=torch.float32)
+  want = O.ragged_dot_fused(_np(lhs), _np(rhs), gs, rhs_bias=_np(bias), gateup_activation=act)
+  assert out.shape == (m, n2 // 2)
+  _check(out, want, 1e-5)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  out16 = op(lhs, rhs, group_sizes=gst, rhs_bias=bias, fuse_gateup_activation=act)
+  assert out16.dtype == torch.bfloat16
+  _check(out16, want, 2e-3)
+  # without a bias
+  _check(op(lhs, rhs, group_sizes=gst, fuse_gateup_activation=act, preferred_element_type=torch.float32),
+         O.ragged_dot_fused(_np(lhs), _np(rhs), gs, gateup_activation=act), 1e-5)
+  # the bias alone, and under a fused activation
+  plain = O.ragged_dot_fused(_np(lhs), _np(rhs), gs, rhs_bias=_np(bias))
+  _check(op(lhs, rhs, group_sizes=gst, rhs_bias=bias, preferred_element_type=torch.float32), plain, 1e-5)
+  got = op(lhs, rhs, group_sizes=gst, rhs_bias=bias, activation=torch.nn.functional.silu,
+           preferred_element_type=torch.float32)
+  _check(got, O.silu(plain), 1e-5)
+  with pytest.raises(NotImplementedError):
+    op(lhs, rhs, group_sizes=gst, fuse_gateup_activation="swigluoai")
 
 
 def test_unsupported_inputs_are_declined(device):

@@ -56,7 +56,8 @@ def test_variant_enumeration_matches_config_space():
   fwd = _lib.variants(0)
   drhs = _lib.variants(1)
   assert fwd and drhs
-  assert {v["mode"] for v in fwd} == {0, 1} and {v["mode"] for v in drhs} == {2}
+  assert {v["mode"] for v in fwd} == {0, 1, 3} and {v["mode"] for v in drhs} == {2}  # 3 = fwd with gate-up fusion
+  assert all(v["block_n"] // (32 * v["waves_n"]) % 2 == 0 for v in fwd if v["mode"] == 3)  # gate/up halves pair up
   pairs = {(v["lhs_dtype"], v["rhs_dtype"]) for v in fwd}
   assert {(_lib.TKX_BF16, _lib.TKX_BF16), (_lib.TKX_F32, _lib.TKX_F32), (_lib.TKX_F8E4M3FN, _lib.TKX_F8E4M3FN),
           (_lib.TKX_BF16, _lib.TKX_I8)} <= pairs
@@ -73,6 +74,9 @@ def test_c_abi_argument_errors_without_gpu():
   assert st == _lib.TKX_ERR_INVALID and "null" in _lib.last_error()
   with pytest.raises(ValueError):
     _lib.check(st)
+  st = lib.tkx_ragged_dot_fwd_fused(None, None, None, None, None, None, None, None, 8, 8, 8, 1, 1, 1, 1, 0, 2,
+                                    ctypes.byref(cfg), None)
+  assert st == _lib.TKX_ERR_INVALID and "gateup" in _lib.last_error()
   with pytest.raises(NotImplementedError):
     _lib.check(_lib.TKX_ERR_UNSUPPORTED)
   with pytest.raises(_lib.HipLibraryError):

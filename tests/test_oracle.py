@@ -173,6 +173,27 @@ def test_e4m3fn_matches_torch_exhaustively():
   np.testing.assert_array_equal(O.e4m3fn_decode(enc), O.e4m3fn_decode(tw))
 
 
+def test_fused_epilogue_terms():
+  """rhs_bias and gate-up fusion (base.py:205-217): the activations against torch's, the composition
+  against brute force on a tiny case."""
+  x = np.linspace(-6, 6, 97)
+  np.testing.assert_allclose(O.silu(x), torch.nn.functional.silu(torch.tensor(x)).numpy(), rtol=1e-12, atol=1e-15)
+  np.testing.assert_allclose(O.gelu_tanh(x), torch.nn.functional.gelu(torch.tensor(x), approximate="tanh").numpy(),
+                             rtol=1e-12, atol=1e-15)
+  rng = np.random.default_rng(5)
+  gs = np.array([2, 0, 3], np.int32)
+  lhs, rhs = rng.normal(size=(7, 5)), rng.normal(size=(3, 5, 8))
+  bias = rng.normal(size=(3, 1, 8))
+  tmp = O.ragged_dot_bruteforce(lhs, rhs, gs)
+  for g, (s, e) in enumerate([(0, 2), (2, 2), (2, 5)]):
+    tmp[s:e] += bias[g, 0]
+  np.testing.assert_allclose(O.ragged_dot_fused(lhs, rhs, gs, rhs_bias=bias), tmp, rtol=1e-12, atol=1e-12)
+  assert np.all(O.ragged_dot_fused(lhs, rhs, gs, rhs_bias=bias)[5:] == 0)  # rows of no group get no bias
+  want = torch.nn.functional.silu(torch.tensor(tmp[:, :4])).numpy() * tmp[:, 4:]
+  np.testing.assert_allclose(O.ragged_dot_fused(lhs, rhs, gs, rhs_bias=bias, gateup_activation="silu"), want,
+                             rtol=1e-12, atol=1e-12)
+
+
 def test_dequantize_is_tile_repeat():
   rng = np.random.default_rng(9)
   q = rng.integers(-127, 128, (2, 8, 6)).astype(np.int8)

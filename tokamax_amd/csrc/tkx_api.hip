@@ -124,10 +124,15 @@ int32_t tkx_ragged_dot_schedule(const int32_t* group_sizes, int64_t num_groups, 
                          static_cast<hipStream_t>(stream));
 }
 
-int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* group_sizes, const float* lhs_scale,
-                           const float* rhs_scale, void* out, void* workspace, int64_t m, int64_t k, int64_t n,
-                           int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype, int32_t mode,
-                           int32_t activation, const TkxConfig* config, tkx_stream_t stream_) {
+}  // extern "C"
+
+namespace {
+// Forward / dlhs launcher behind both public forward entry points. `gateup`: rhs is [g, k, n] =
+// [gate | up] and out is [m, n/2] = act(lhs.gate + bias) * (lhs.up + bias), `activation` naming act.
+int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, const float* lhs_scale,
+                 const float* rhs_scale, const float* rhs_bias, void* out, void* workspace, int64_t m, int64_t k,
+                 int64_t n, int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype, int32_t mode,
+                 int32_t activation, bool gateup, const TkxConfig* config, tkx_stream_t stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (!lhs || !rhs || !group_sizes || !out || !workspace || !config)
     return set_error(TKX_ERR_INVALID, "null pointer argument");
@@ -146,12 +151,17 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   if (c.grid_tile_width < 1 || c.align_tile < 1) return set_error(TKX_ERR_INVALID, "grid_tile_width/align_tile must be >= 1");
   const bool dlhs = mode == TKX_MODE_TRANS_RHS;
   if (dlhs && (lhs_scale || rhs_scale)) return set_error(TKX_ERR_UNSUPPORTED, "scales are not supported with TRANS_RHS");
-  const Variant* v = find_variant(dlhs ? kDlhs : kFwd, lhs_dtype, rhs_dtype, c);
+  if (dlhs && (rhs_bias || gateup)) return set_error(TKX_ERR_UNSUPPORTED, "bias and gate-up fusion need the default mode");
+  if (gateup && (n % 16 != 0 || k % c.block_k != 0))
+    return set_error(TKX_ERR_UNSUPPORTED, "gate-up fusion needs n %% 16 == 0 and k %% block_k == 0 (k=%lld n=%lld)",
+                     (long long)k, (long long)n);
+  if (rhs_bias && (uintptr_t)rhs_bias % 16 != 0) return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
+  const Variant* v = find_variant(dlhs ? kDlhs : gateup ? kFwdGlu : kFwd, lhs_dtype, rhs_dtype, c);
   if (v == nullptr)
     return set_error(TKX_ERR_UNSUPPORTED, "no kernel variant for mode=%d dtypes=(%d,%d) tile=%dx%dx%d waves=%dx%d stages=%d",
                      mode, lhs_dtype, rhs_dtype, c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages);
   // In C terms: rows = m; cols = n (fwd) or k (dlhs); contraction = k (fwd) or n (dlhs).
-  const int64_t cols = dlhs ? k : n, contraction = dlhs ? n : k;
+  const int64_t cols = dlhs ? k : gateup ? n / 2 : n, contraction = dlhs ? n : k;
   const int lb = dtype_bytes(lhs_dtype), rb = dtype_bytes(rhs_dtype), ob = dtype_bytes(out_dtype);
   // 16-byte vector accesses: every row of every operand must start 16-byte aligned and the tile
   // loaders move whole 16-byte chunks along the contiguous axis. The contraction size itself need
@@ -167,6 +177,7 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   if (v->fn == nullptr) {
     // Streaming decode kernel: one launch, no schedule.
     if (lhs_scale != nullptr) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no lhs scale");
+    if (rhs_bias != nullptr || gateup) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no bias or gate-up fusion");
     if (rhs_scale != nullptr && rhs_dtype != TKX_I8)
       return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes an rhs scale with int8 weights only");
     if (!decode_supported(lhs_dtype, rhs_dtype, m, k, n, num_groups))
@@ -188,6 +199,7 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   p.C = out;
   p.a_scale = lhs_scale;
   p.b_scale = rhs_scale;
+  p.b_bias = rhs_bias;
   p.ws = static_cast<const int32_t*>(workspace);
   p.lda = dlhs ? n : k;
   p.ldb = n;
@@ -196,9 +208,11 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   p.c_group_stride = 0;
   p.m_ext = (int32_t)m;
   p.n_ext = (int32_t)cols;
+  p.nb_ext = (int32_t)(gateup ? n : cols);
   p.k_ext = (int32_t)contraction;
   p.num_groups = (int32_t)num_groups;
-  p.n_tiles = (int32_t)((cols + c.block_n - 1) / c.block_n);
+  const int64_t out_block_n = gateup ? c.block_n / 2 : c.block_n;  // output columns of a tile
+  p.n_tiles = (int32_t)((cols + out_block_n - 1) / out_block_n);
   p.m_tiles = 0;
   // Whole chunks for every XCD, so that each list entry has a workgroup (see the launch order in run()).
   const int64_t slots = ((int64_t)L.tid_size * p.n_tiles + 8 * kXcdChunk - 1) / (8 * kXcdChunk) * (8 * kXcdChunk);
@@ -219,6 +233,28 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
   if (zero_wgs > 256) zero_wgs = 256;
   if (zero_wgs < 1) zero_wgs = 1;
   return launch(v, p, slots + zero_wgs, stream);
+}
+}  // namespace
+
+extern "C" {
+
+int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* group_sizes, const float* lhs_scale,
+                           const float* rhs_scale, void* out, void* workspace, int64_t m, int64_t k, int64_t n,
+                           int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype, int32_t mode,
+                           int32_t activation, const TkxConfig* config, tkx_stream_t stream) {
+  return fwd_impl(lhs, rhs, group_sizes, lhs_scale, rhs_scale, nullptr, out, workspace, m, k, n, num_groups, lhs_dtype,
+                  rhs_dtype, out_dtype, mode, activation, false, config, stream);
+}
+
+int32_t tkx_ragged_dot_fwd_fused(const void* lhs, const void* rhs, const int32_t* group_sizes, const float* lhs_scale,
+                                 const float* rhs_scale, const float* rhs_bias, void* out, void* workspace, int64_t m,
+                                 int64_t k, int64_t n, int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype,
+                                 int32_t out_dtype, int32_t activation, int32_t gateup, const TkxConfig* config,
+                                 tkx_stream_t stream) {
+  if (gateup != 0 && gateup != 1) return set_error(TKX_ERR_INVALID, "gateup must be 0 or 1");
+  if (gateup && activation == TKX_ACT_NONE) return set_error(TKX_ERR_INVALID, "gate-up fusion needs an activation");
+  return fwd_impl(lhs, rhs, group_sizes, lhs_scale, rhs_scale, rhs_bias, out, workspace, m, k, n, num_groups, lhs_dtype,
+                  rhs_dtype, out_dtype, TKX_MODE_DEFAULT, activation, gateup == 1, config, stream);
 }
 
 int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* group_sizes, void* out, void* workspace,
@@ -263,6 +299,7 @@ int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* gr
   p.c_group_stride = k * n;
   p.m_ext = (int32_t)k;
   p.n_ext = (int32_t)n;
+  p.nb_ext = (int32_t)n;
   p.k_ext = (int32_t)m;
   p.num_groups = (int32_t)num_groups;
   p.n_tiles = (int32_t)((n + c.block_n - 1) / c.block_n);

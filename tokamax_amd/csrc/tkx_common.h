@@ -56,7 +56,8 @@ int32_t launch_schedule(const int32_t* group_sizes, int64_t G, int64_t m, int32_
                         int32_t span_width, int32_t* ws, const WsLayout& L, hipStream_t stream);
 
 // ---- grouped GEMM -----------------------------------------------------------------------------
-enum KernelMode { kFwd = 0, kDlhs = 1, kDrhs = 2 };
+// kFwdGlu = forward over weights [gate | up] ([g, k, 2 n_out]) with the epilogue act(gate) * up.
+enum KernelMode { kFwd = 0, kDlhs = 1, kDrhs = 2, kFwdGlu = 3 };
 
 // fwd/dlhs launch order: the tile list is dealt to the 8 XCDs in chunks of this many consecutive
 // tiles (the number of CUs of an XCD: one chunk is what an XCD runs at a time).
@@ -67,12 +68,14 @@ struct GemmParams {
   const void* B;
   void* C;
   const float* a_scale;  // per A row, or null
-  const float* b_scale;  // per (group, column), or null
+  const float* b_scale;  // per (group, column of B), or null
+  const float* b_bias;   // per (group, column of B), added after the scales, or null
   const int32_t* ws;
   int64_t lda, ldb, ldc;            // leading dimensions, elements
   int64_t b_group_stride;           // elements between consecutive groups of B (fwd/dlhs)
   int64_t c_group_stride;           // elements between consecutive groups of C (drhs)
   int32_t m_ext, n_ext, k_ext;      // extents of the C rows, C columns and the contraction
+  int32_t nb_ext;                   // columns of B (fwd/dlhs): n_ext, or 2 * n_ext for kFwdGlu
   int32_t num_groups;
   int32_t n_tiles, m_tiles;         // tiles along C columns; along C rows (drhs only)
   int32_t real_slots;               // fwd/dlhs: workgroups that may own a task tile (multiple of 8 * kXcdChunk)

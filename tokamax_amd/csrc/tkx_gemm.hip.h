@@ -3,6 +3,7 @@
 //   C[rows, cols] = sum over the contraction of A(row, kc) * B(kc, col)
 //
 //   mode kFwd  : A = lhs  [m,k]  contraction-contiguous   B = rhs[g] [k,n]  column-contiguous
+//   mode kFwdGlu: as kFwd with B = rhs[g] [k, 2 n] = [gate | up] and C[m,n] = act(A.gate) * (A.up)
 //   mode kDlhs : A = dout [m,n]  contraction-contiguous   B = rhs[g] [k,n]  contraction-contiguous
 //                (C[m,k] = dout . rhs[g]^T: rhs is read in place, never transposed in memory)
 //   mode kDrhs : A = lhs  [m,k]  row(k-index)-contiguous  B = dout [m,n]    column-contiguous
@@ -274,7 +275,13 @@ struct DirectLoader {
   // `rc_lo`, `rc_hi`: the rows (contraction-contiguous layout) whose data the caller uses. Rows
   // outside are redirected to the nearest one inside: that keeps every address valid, and the
   // lanes of a load that fall outside all fetch one row's cache lines instead of one each.
-  __device__ __forceinline__ void init(int rc0, int rc_ext, int64_t ld, int wave, int lane, int rc_lo, int rc_hi) {
+  // `glu_tn` > 0 (row/column-contiguous layout only): the tile's columns are [gate | up] pairs. The
+  // tile is cut into blocks of 32 columns, `glu_tn` blocks per wave column; the first half of a wave
+  // column's blocks comes from the gate columns [rc0, rc0 + RC/2) and the second half from the up
+  // columns `glu_up` further on, so that accumulator block j and block j + glu_tn/2 of a lane hold
+  // gate and up of the same output column.
+  __device__ __forceinline__ void init(int rc0, int rc_ext, int64_t ld, int wave, int lane, int rc_lo, int rc_hi,
+                                       int glu_tn = 0, int glu_up = 0) {
     stride = (int64_t)ROWS_PER_INSTR_STEP * ld * ESZ;
 #pragma unroll
     for (int i = 0; i < NOFF; ++i) {
@@ -290,6 +297,11 @@ struct DirectLoader {
       } else {
         const int lc = ((((pc >> 1) ^ mc_swizzle<ROW_BYTES, ES>(row))) << 1) | (pc & 1);
         int colb = rc0 * ESZ + lc * 16;
+        if (glu_tn > 0) {
+          const int c = lc * (16 / ESZ), blk = c >> 5, half = glu_tn >> 1;
+          const int w = blk / glu_tn, j = blk % glu_tn;
+          colb = ((j < half ? rc0 : rc0 + glu_up) + (w * half + j % half) * 32 + (c & 31)) * ESZ;
+        }
         const int lim = rc_ext * ESZ - 16;
         colb = colb < lim ? colb : lim;
         voff[i] = (uint32_t)(row * (int)ld * ESZ + colb);
@@ -414,10 +426,14 @@ struct GemmKernel {
   static constexpr int THREADS = WM * WN * 64;
   static constexpr int LA = (MODE == kDrhs) ? kMC : kKC;
   static constexpr int LB = (MODE == kDlhs) ? kKC : kMC;
+  static constexpr bool GLU = MODE == kFwdGlu;
+  static constexpr int BNO = GLU ? BN / 2 : BN;  // output columns of a tile
   static constexpr int EC = EA;  // MFMA type follows A; B may be stored narrower (int8 weights)
   static constexpr int KA = Mma<EC>::KA;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int TM = WTM / 32, TN = WTN / 32;
+  static_assert(MODE != kFwdGlu || TN % 2 == 0, "gate-up tiles pair the two halves of a wave's column blocks");
+  static constexpr int TNO = MODE == kFwdGlu ? TN / 2 : TN, WTNO = MODE == kFwdGlu ? WTN / 2 : WTN;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % KA == 0, "tile does not split into 32x32 atoms");
   static constexpr int KSTEPS = BK / KA;
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
@@ -479,7 +495,7 @@ struct GemmKernel {
       row0 = ws[p.ws_bstart + mt];
       act_start = ws[p.ws_astart + mt];
       act_end = ws[p.ws_aend + mt];
-      col0 = nt * BN;
+      col0 = nt * BNO;
       kc_begin = 0;
       kc_end = p.k_ext;
     } else {
@@ -557,7 +573,7 @@ struct GemmKernel {
       DirB db;
       const int a_hi = max(min(act_end, p.m_ext), 1), a_lo = min(max(act_start, 0), a_hi - 1);
       da.init(row0, p.m_ext, p.lda, wave, lane, a_lo, a_hi);
-      db.init(col0, p.n_ext, p.ldb, wave, lane, 0, p.n_ext);
+      db.init(col0, p.nb_ext, p.ldb, wave, lane, 0, p.nb_ext, GLU ? TN : 0, GLU ? p.n_ext : 0);
       const unsigned char* const gA0 = Ab + DirA::step_base(row0, p.lda, kc_begin);
       const unsigned char* const gB0 = Bb + DirB::step_base(col0, p.ldb, kc_begin);
       const int64_t stepA = DirA::step_bytes(p.lda), stepB = DirB::step_bytes(p.ldb);
@@ -690,10 +706,10 @@ struct GemmKernel {
       if (all_rows) k_loop(std::true_type{});
       else k_loop(std::false_type{});
     }
-    if (tail) {
+    if (tail && !GLU) {  // (gate-up problems are taken only with whole k-steps)
       const int kc0 = kc_begin + nfull * BK;
       StageA::copy(Ab, p.lda, row0, p.m_ext, kc0, kc_end, smem, tid);
-      StageB::copy(Bb, p.ldb, col0, p.n_ext, kc0, kc_end, smem + StageA::BYTES, tid);
+      StageB::copy(Bb, p.ldb, col0, p.nb_ext, kc0, kc_end, smem + StageA::BYTES, tid);
       __syncthreads();
 #pragma unroll
       for (int kk = 0; kk < KSTEPS; ++kk) {
@@ -715,8 +731,12 @@ struct GemmKernel {
     {
       unsigned char* Cg = reinterpret_cast<unsigned char*>(p.C);
       if constexpr (MODE == kDrhs) Cg += (int64_t)group * p.c_group_stride * (p.out_dtype == TKX_F32 ? 4 : 2);
-      const bool inside = col0 + BN <= p.n_ext;
-      const int lane_col = wn * WTN + 4 * (lane >> 5);
+      const bool inside = col0 + BNO <= p.n_ext;
+      // Column of B (of its scales and bias) behind accumulator block j, element group t of this lane.
+      auto b_col = [&](int j, int t) {
+        const int c = GLU ? (j < TNO ? 0 : p.n_ext) + col0 + wn * WTNO + (j % TNO) * 32 : col0 + wn * WTN + j * 32;
+        return min(c + 4 * (lane >> 5) + 8 * t, p.nb_ext - 4);
+      };
       if (p.a_scale != nullptr) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
@@ -733,12 +753,24 @@ struct GemmKernel {
         for (int j = 0; j < TN; ++j) {
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
-            const int col = min(col0 + lane_col + j * 32 + 8 * t, p.n_ext - 4);
-            const f32x4 cs = *reinterpret_cast<const f32x4*>(p.b_scale + (int64_t)group * p.n_ext + col);
+            const f32x4 cs = *reinterpret_cast<const f32x4*>(p.b_scale + (int64_t)group * p.nb_ext + b_col(j, t));
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
               for (int e = 0; e < 4; ++e) acc[i][j][4 * t + e] *= cs[e];
+          }
+        }
+      }
+      if (p.b_bias != nullptr) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const f32x4 cb = *reinterpret_cast<const f32x4*>(p.b_bias + (int64_t)group * p.nb_ext + b_col(j, t));
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[i][j][4 * t + e] += cb[e];
           }
         }
       }
@@ -747,7 +779,7 @@ struct GemmKernel {
 #pragma unroll
           for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < TNO; ++j)  // (gate-up: the gate blocks only)
 #pragma unroll
               for (int e = 0; e < 16; ++e) acc[i][j][e] = fn(acc[i][j][e]);
         };
@@ -760,6 +792,15 @@ struct GemmKernel {
         else if (p.activation == TKX_ACT_GELU_TANH)
           for_all([&](float x) { return 0.5f * x * (1.f + fast_tanh(0.7978845608028654f * (x + 0.044715f * x * x * x))); });
       }
+      if constexpr (GLU) {
+        // act(gate) * up: block j and block j + TNO of a lane are gate and up of the same output columns.
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TNO; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] *= acc[i][j + TNO][e];
+      }
       // The stores go through LDS (free once the k loop is done): as the MFMA leaves them, a
       // lane's values are 4 columns of one row, so a store straight from registers writes 16-byte
       // pieces of 32 different rows and the memory pipeline takes it apart line by line. Each wave
@@ -769,7 +810,7 @@ struct GemmKernel {
       auto emit = [&](auto out_tag) {
         constexpr int OUT = decltype(out_tag)::value;
         constexpr int ESZ = OUT == TKX_F32 ? 4 : 2;
-        constexpr int ROW_BYTES = WTN * ESZ;
+        constexpr int ROW_BYTES = WTNO * ESZ;
         constexpr int PITCH = ROW_BYTES + 16;                     // keeps 16-byte alignment, staggers banks
         constexpr int WAVE_LDS = (SMEM_BYTES / (WM * WN)) / 16 * 16;
         constexpr int AP = (WAVE_LDS / PITCH) / 32 < TM ? (WAVE_LDS / PITCH) / 32 : TM;  // atoms (32 rows) per pass
@@ -781,9 +822,9 @@ struct GemmKernel {
         unsigned char* const slice = smem + wave * WAVE_LDS;
         unsigned char* const tile = const_cast<unsigned char*>(uniform_pointer(Cg + ((int64_t)row0 * p.ldc + col0) * ESZ));
         const int rd_row = lane / CPR, rd_chunk = lane % CPR;
-        const int gcol = col0 + wn * WTN + rd_chunk * (16 / ESZ);
+        const int gcol = col0 + wn * WTNO + rd_chunk * (16 / ESZ);
         const bool col_ok = inside || gcol + 16 / ESZ <= p.n_ext;
-        const uint32_t voff = (uint32_t)(((wm * 32 + rd_row) * (int)p.ldc + wn * WTN + rd_chunk * (16 / ESZ)) * ESZ);
+        const uint32_t voff = (uint32_t)(((wm * 32 + rd_row) * (int)p.ldc + wn * WTNO + rd_chunk * (16 / ESZ)) * ESZ);
 #pragma unroll
         for (int i0 = 0; i0 < TM; i0 += AP) {
 #pragma unroll
@@ -791,7 +832,7 @@ struct GemmKernel {
             if (i0 + ii >= TM) break;
             const int i = i0 + ii;
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
+            for (int j = 0; j < TNO; ++j) {
 #pragma unroll
               for (int t = 0; t < 4; ++t) {
                 f32x4 v;

@@ -4,6 +4,7 @@
 namespace tkx {
 #define FWD_DLHS(BM, BN, BK, WM, WN, NS) \
   TKX_VARIANT(kFwd, kEBF16, kEBF16, BM, BN, BK, WM, WN, NS), TKX_VARIANT(kDlhs, kEBF16, kEBF16, BM, BN, BK, WM, WN, NS)
+#define GLU(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdGlu, kEBF16, kEBF16, BM, BN, BK, WM, WN, NS)
 #define DRHS(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kDrhs, kEBF16, kEBF16, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
@@ -21,6 +22,10 @@ static const Variant kVariants[] = {
     FWD_DLHS(64, 128, 64, 2, 2, 4),
     FWD_DLHS(32, 256, 64, 1, 4, 3),
     FWD_DLHS(32, 128, 64, 1, 4, 4),
+    GLU(256, 256, 32, 2, 4, 4),
+    GLU(128, 256, 64, 2, 4, 3),
+    GLU(64, 256, 64, 2, 2, 3),
+    GLU(32, 256, 64, 1, 4, 3),
     DRHS(256, 256, 64, 2, 4, 2),
     DRHS(256, 256, 32, 2, 4, 4),
     DRHS(128, 256, 64, 2, 4, 3),

@@ -69,6 +69,10 @@ _ACTIVATION_NAMES = {
 }
 
 
+# `fuse_gateup_activation` names -> in-kernel activation (jax.nn.gelu defaults to the tanh form).
+_GATEUP_ACTIVATIONS = {"silu": "silu", "gelu": "gelu_tanh"}
+
+
 def _fused_activation_name(activation) -> str | None:
   """Name of the in-kernel epilogue for a known activation callable, else None."""
   try:
@@ -142,13 +146,21 @@ class HipRaggedDot(base.RaggedDot):
       rhs_quantization_dtype=None,
   ):
     del manual_axis_type  # sharding annotation only; no meaning on a single device
-    if (group_offset is not None or rhs_scale is not None or rhs_bias is not None or maybe_quantize_lhs
-        or not zero_initialize or fuse_gateup_activation is not None or lhs_quantization_dtype is not None
-        or rhs_quantization_dtype is not None):
+    if (group_offset is not None or rhs_scale is not None or maybe_quantize_lhs or not zero_initialize
+        or lhs_quantization_dtype is not None or rhs_quantization_dtype is not None):
       raise NotImplementedError(
-          "The hip implementation does not support group_offset, rhs_scale, rhs_bias, maybe_quantize_lhs,"
-          " zero_initialize, fuse_gateup_activation, lhs_quantization_dtype, or rhs_quantization_dtype."
+          "The hip implementation does not support group_offset, rhs_scale, maybe_quantize_lhs,"
+          " zero_initialize, lhs_quantization_dtype, or rhs_quantization_dtype."
       )
+    # rhs_bias and fuse_gateup_activation (base.py:205-217) are fused into the forward kernel's epilogue.
+    gateup = None
+    if fuse_gateup_activation is not None:
+      gateup = _GATEUP_ACTIVATIONS.get(fuse_gateup_activation)
+      if gateup is None:
+        raise NotImplementedError(f"fuse_gateup_activation={fuse_gateup_activation!r} is not supported by the hip"
+                                  " implementation (supported: 'silu', 'gelu').")
+      if return_residuals:
+        raise NotImplementedError("return_residuals is not supported with fuse_gateup_activation.")
     if isinstance(lhs, AsQArray) or isinstance(rhs, AsQArray):
       raise NotImplementedError("The hip implementation does not quantise inputs on the fly (AsQArray).")
     mode = _MODE_OF_DIMS.get(ragged_dot_dimension_numbers)
@@ -202,6 +214,22 @@ class HipRaggedDot(base.RaggedDot):
     if activation is not None and not return_residuals:
       fused = _fused_activation_name(activation)
 
+    if (rhs_bias is not None or gateup is not None) and mode != 0:
+      raise NotImplementedError("rhs_bias and fuse_gateup_activation need the default dimension numbers.")
+    if rhs_bias is not None:
+      g, _, n = rhs_v.shape
+      if tuple(rhs_bias.shape) != (g, 1, n):
+        raise NotImplementedError(f"rhs_bias must have shape [g,1,n], got {tuple(rhs_bias.shape)}")
+
+    if gateup is not None:
+      # act(gate) * up in the kernel; an `activation` on top of that is applied to the f32 result.
+      kernel_out = torch.float32 if activation is not None else preferred_element_type
+      dot_out = hip_ops.ragged_dot_fwd(lhs_v, rhs_v, gs, config=kcfg, out_dtype=kernel_out, lhs_scale=lhs_scale,
+                                       rhs_scale=rhs_scale_, rhs_bias=rhs_bias, activation=gateup, gateup=True)
+      if activation is not None:
+        dot_out = activation(dot_out).to(preferred_element_type)
+      return dot_out, None
+
     if mode == 2:
       if isinstance(lhs, QArray) or isinstance(rhs, QArray):
         raise NotImplementedError("Quantised inputs are not supported with ragged contracting dimensions.")
@@ -212,7 +240,7 @@ class HipRaggedDot(base.RaggedDot):
       unfused = activation is not None and not return_residuals and fused is None
       kernel_out = torch.float32 if unfused else preferred_element_type
       dot_out = hip_ops.ragged_dot_fwd(lhs_v, rhs_v, gs, config=kcfg, out_dtype=kernel_out, trans_rhs=(mode == 1),
-                                       lhs_scale=lhs_scale, rhs_scale=rhs_scale_, activation=fused)
+                                       lhs_scale=lhs_scale, rhs_scale=rhs_scale_, activation=fused, rhs_bias=rhs_bias)
       if unfused:
         dot_out = activation(dot_out).to(preferred_element_type)
 
@@ -230,6 +258,8 @@ class HipRaggedDot(base.RaggedDot):
     mode = _MODE_OF_DIMS.get(dims)
     if mode is None:
       raise NotImplementedError("Unsupported ragged dot dimension numbers.")
+    if mode == 0 and ba.kwargs.get("fuse_gateup_activation") is not None:
+      mode = 3  # forward with gate-up fusion: variants of their own
     lhs_shape = tuple(lhs.shape)
     rhs_shape = tuple(rhs.shape)
     if mode == 2:
@@ -256,7 +286,7 @@ class HipRaggedDot(base.RaggedDot):
     # The streaming small-m kernel (listed with block_m == 16; forward only) needs k % 1024 == 0 and
     # n % 8 == 0, and a weight slice (k/4 rows of n) that a 32-bit buffer offset spans.
     wbytes = 1 if key[2] == _lib.TKX_I8 else 2
-    streaming_ok = (mode == 0 and contraction % 1024 == 0 and cols % 8 == 0
+    streaming_ok = (mode == 0 and ba.kwargs.get("rhs_bias") is None and contraction % 1024 == 0 and cols % 8 == 0
                     and (contraction // 4) * cols * wbytes < 2**31)
     usable = [v for v in variants if v[0] != 16 or streaming_ok]
     # Rows per group decide the m-tile: a tile much taller than a group wastes MFMA work on rows

@@ -100,12 +100,14 @@ def schedule(group_sizes: torch.Tensor, m: int, block_m: int, align_tile: int = 
 
 
 def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: torch.dtype, trans_rhs: bool = False,
-                   lhs_scale=None, rhs_scale=None, activation: str | None = None,
-                   workspace_out: list | None = None) -> torch.Tensor:
+                   lhs_scale=None, rhs_scale=None, activation: str | None = None, rhs_bias=None,
+                   gateup: bool = False, workspace_out: list | None = None) -> torch.Tensor:
   """out[m,n] = lhs[m,k] . rhs[g,k,n]   (trans_rhs: out[m,k] = lhs[m,n] . rhs[g,k,n]^T).
 
+  `rhs_bias` ([g,n] or [g,1,n]) is added to the scaled result before the activation. `gateup`: rhs
+  columns are [gate | up] and out[m,n/2] = activation(gate part) * (up part) (base.py:211-217).
   `workspace_out`, if given, receives the int32 workspace the call filled (schedule arrays included)."""
-  _require_cuda(lhs, rhs, group_sizes, lhs_scale, rhs_scale)
+  _require_cuda(lhs, rhs, group_sizes, lhs_scale, rhs_scale, rhs_bias)
   lib = _lib.load()
   if lhs.dim() != 2 or rhs.dim() != 3:
     raise ValueError(f"expected lhs [m,k] and rhs [g,k,n], got {tuple(lhs.shape)} and {tuple(rhs.shape)}")
@@ -117,6 +119,10 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
     raise ValueError(f"group_sizes has {gs.numel()} entries, rhs has {G} groups")
   if lhs.shape[1] != (n if trans_rhs else k):
     raise ValueError("contraction sizes of lhs and rhs differ")
+  if (rhs_bias is not None or gateup) and trans_rhs:
+    raise NotImplementedError("bias and gate-up fusion need the default dimension numbers")
+  if gateup and (activation is None or n % 2):
+    raise ValueError("gate-up fusion needs an activation and an even number of rhs columns")
   if lhs_scale is not None:
     lhs_scale = lhs_scale.to(torch.float32).contiguous().view(-1)
     if lhs_scale.numel() != m:
@@ -125,15 +131,26 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
     rhs_scale = rhs_scale.to(torch.float32).contiguous().view(-1)
     if rhs_scale.numel() != G * n:
       raise NotImplementedError("rhs scale must be one f32 per (group, column)")
-  out = torch.empty((m, k if trans_rhs else n), dtype=out_dtype, device=lhs.device)
+  if rhs_bias is not None:
+    rhs_bias = rhs_bias.to(torch.float32).contiguous().view(-1)
+    if rhs_bias.numel() != G * n:
+      raise NotImplementedError("rhs bias must be one value per (group, column)")
+  out_cols = k if trans_rhs else n // 2 if gateup else n
+  out = torch.empty((m, out_cols), dtype=out_dtype, device=lhs.device)
   ws = workspace(m, G, config.block_m, lhs.device)
   cfg = config.to_c()
   with torch.cuda.device(lhs.device):
-    st = lib.tkx_ragged_dot_fwd(
-        _ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(out), _ptr(ws), m, k, n, G,
-        dtype_code(lhs.dtype), dtype_code(rhs.dtype), dtype_code(out_dtype),
-        _lib.TKX_MODE_TRANS_RHS if trans_rhs else _lib.TKX_MODE_DEFAULT, _lib.ACTIVATIONS[activation],
-        ctypes.byref(cfg), _stream(lhs.device))
+    if rhs_bias is None and not gateup:
+      st = lib.tkx_ragged_dot_fwd(
+          _ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(out), _ptr(ws), m, k, n, G,
+          dtype_code(lhs.dtype), dtype_code(rhs.dtype), dtype_code(out_dtype),
+          _lib.TKX_MODE_TRANS_RHS if trans_rhs else _lib.TKX_MODE_DEFAULT, _lib.ACTIVATIONS[activation],
+          ctypes.byref(cfg), _stream(lhs.device))
+    else:
+      st = lib.tkx_ragged_dot_fwd_fused(
+          _ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(rhs_bias), _ptr(out), _ptr(ws), m, k,
+          n, G, dtype_code(lhs.dtype), dtype_code(rhs.dtype), dtype_code(out_dtype), _lib.ACTIVATIONS[activation],
+          1 if gateup else 0, ctypes.byref(cfg), _stream(lhs.device))
   _lib.check(st)
   if workspace_out is not None:
     workspace_out.append(ws)
