@@ -308,6 +308,23 @@ def test_config_options():
     del os.environ["TOKAMAX_IGNORE_AUTOTUNING_CACHE"]
 
 
+def test_shipped_mi355x_cache_parses_and_names_compiled_variants():
+  """data/autotuning/amd_instinct_mi355x/hip_ragged_dot.json (written by data/autotuning/generate.py on
+  an MI355X): every key binds again, and every timed config is a compiled kernel variant."""
+  op = tokamax_amd.HipRaggedDot()
+  path = cache_lib.cache_file(op.replace(vjp=None), "AMD Instinct MI355X")
+  with open(path, encoding="utf-8") as f:
+    loaded = cache_lib.loads(op, f.read())
+  assert len(loaded) >= 6
+  compiled = {(v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"], v["num_stages"])
+              for kind in (0, 1) for v in _lib.variants(kind)}
+  for key, data in loaded.items():
+    assert len(data) >= 8, key
+    for cfg in data:
+      assert (cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages) in compiled
+    assert data.fastest_config.block_m >= 128  # the tuned workloads are the large prefill / VJP shapes
+
+
 def test_cache_file_name_and_json_round_trip(tmp_path):
   op = hip.HipRaggedDot()
   assert cache_lib.op_file_name(op) == "hip_ragged_dot.json"

@@ -1,0 +1,74 @@
+"""Regenerates the shipped autotuning cache for the device this runs on.
+
+Times every compiled kernel variant x launch-order span width on the benchmark workloads whose
+kernels run long enough for eager timing to separate them (the prefill shapes, the fp8 shape, both
+VJP products and the gate-up fused FFN shape) and writes
+`tokamax_amd/data/autotuning/<device kind>/hip_ragged_dot.json`, the file `Op.get_autotuning_cache`
+reads (layout of the reference's tokamax/data/autotuning/<device>/<op>.json).
+
+  python -m tokamax_amd.data.autotuning.generate [--iterations N]
+"""
+
+from __future__ import annotations
+
+import argparse
+import os
+
+import torch
+
+import tokamax_amd
+from tokamax_amd import op as op_lib
+from tokamax_amd.autotuning import autotuner as autotuner_lib
+from tokamax_amd.autotuning import cache as cache_lib
+from tokamax_amd.ragged_dot import base
+from tokamax_amd.ragged_dot import workloads
+
+
+def bound_arguments(op, device):
+  """Yields (name, BoundArguments) one at a time (each holds its workload's tensors)."""
+  w = workloads.make("mixtral", device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  yield "mixtral", op.bind(w.lhs, w.rhs, group_sizes=gs)
+  n = w.n
+  rhs2 = torch.cat([w.rhs, w.rhs], dim=2)
+  yield "mixtral gate-up", op.bind(w.lhs, rhs2, group_sizes=gs, fuse_gateup_activation="silu")
+  del w, rhs2, n
+  w = workloads.make("deepseek", device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  yield "deepseek", op.bind(w.lhs, w.rhs, group_sizes=gs)
+  del w
+  w = workloads.make("fp8", device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  yield "fp8", op.bind(tokamax_amd.QArray(w.lhs, w.lhs_scale), tokamax_amd.QArray(w.rhs, w.rhs_scale), group_sizes=gs,
+                       preferred_element_type=torch.bfloat16)
+  del w
+  w = workloads.make("vjp", device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  yield "dlhs", op.bind(w.dout, w.rhs, group_sizes=gs, ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS)
+  yield "drhs", op.bind(w.lhs, w.dout, group_sizes=gs,
+                        ragged_dot_dimension_numbers=base.RAGGED_CONTRACTING_DOT_DIM_NUMS)
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--iterations", type=int, default=10)
+  args = ap.parse_args()
+  device = torch.device("cuda:0")
+  op = tokamax_amd.HipRaggedDot()
+  tuner = autotuner_lib.Autotuner(iterations=args.iterations, warmup=2)
+  for name, ba in bound_arguments(op, device):
+    data = ba.autotune(autotuner=tuner, cache_results=True)
+    best = data.fastest_config
+    print(f"{name}: {len(data)} configs, fastest {best} {min(data[best].evaluation_times_ms):.4f} ms", flush=True)
+    del ba, data
+    torch.cuda.empty_cache()
+  kind = op_lib.device_kind()
+  path = cache_lib.cache_file(op.replace(vjp=None), kind)
+  os.makedirs(os.path.dirname(path), exist_ok=True)
+  with open(path, "w", encoding="utf-8") as f:
+    f.write(cache_lib.dumps(op, op.get_autotuning_cache(kind)))
+  print("wrote", path)
+
+
+if __name__ == "__main__":
+  main()

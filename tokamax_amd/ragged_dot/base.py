@@ -267,7 +267,9 @@ class RaggedDot(op.Op):
       if name in out:
         out[name] = serialization.array_spec_from_json(out[name])
     if "group_sizes" in out:
-      out["group_sizes"] = GroupSizes.from_json(out["group_sizes"])
+      # Wrapped in `GroupSizes` only under the default dimension numbers (see `bind`); a plain array otherwise.
+      gs = out["group_sizes"]
+      out["group_sizes"] = serialization.array_spec_from_json(gs) if isinstance(gs, str) else GroupSizes.from_json(gs)
     if out.get("ragged_dot_dimension_numbers") is not None:
       out["ragged_dot_dimension_numbers"] = RaggedDotDimensionNumbers.from_json(out["ragged_dot_dimension_numbers"])
     if isinstance(out.get("precision"), list):
