@@ -490,6 +490,60 @@ def test_rhs_bias_and_gateup_fusion(m, k, n2, gs, act, device):
     op(lhs, rhs, group_sizes=gst, fuse_gateup_activation="swigluoai")
 
 
+def test_hip_graph_replays_follow_new_inputs_and_group_sizes(device):
+  """The entry points allocate nothing, synchronise nothing and schedule on the device, so a captured
+  HIP graph stays valid when the contents of lhs, the weights and even group_sizes change between
+  replays. One graph holds a tiled forward, a streaming small-m forward, a dlhs and a drhs; every
+  replay is checked against the oracle on the inputs of that replay."""
+  rng = np.random.default_rng(11)
+  G, m, k, n = 6, 640, 256, 384
+  f32 = torch.float32
+  mk = lambda shape, std: torch.tensor(rng.normal(0, std, shape).astype(np.float32), device=device).to(torch.bfloat16)
+  lhs, rhs, dout = mk((m, k), 1.0), mk((G, k, n), k ** -0.5), mk((m, n), 1.0)
+  gs = torch.tensor([100, 0, 257, 9, 130, 80], dtype=torch.int32, device=device)
+  small_lhs, small_rhs = mk((40, 1024), 1.0), mk((G, 1024, 256), 1 / 32)
+  small_gs = torch.tensor([3, 0, 16, 1, 7, 2], dtype=torch.int32, device=device)
+  tiled = hip_ops.KernelConfig(128, 128, 64, 2, 2, 4, grid_tile_width=3)
+  stream_cfg = hip_ops.KernelConfig(16, 128, 32, 1, 4, 2)
+  drhs_cfg = hip_ops.KernelConfig(128, 128, 64, 2, 2, 4)
+
+  def run():
+    return (hip_ops.ragged_dot_fwd(lhs, rhs, gs, config=tiled, out_dtype=f32),
+            hip_ops.ragged_dot_fwd(small_lhs, small_rhs, small_gs, config=stream_cfg, out_dtype=f32),
+            hip_ops.ragged_dot_fwd(dout, rhs, gs, config=tiled, out_dtype=f32, trans_rhs=True),
+            hip_ops.ragged_dot_drhs(lhs, dout, gs, G, config=drhs_cfg, out_dtype=f32))
+
+  def check(outs):
+    g, sg = gs.cpu().numpy(), small_gs.cpu().numpy()
+    _check(outs[0], _ref(lhs, rhs, g), 1e-5)
+    assert torch.count_nonzero(outs[0][int(g.sum()):]) == 0
+    _check(outs[1], _ref(small_lhs, small_rhs, sg), 1e-5)
+    assert torch.count_nonzero(outs[1][int(sg.sum()):]) == 0
+    _check(outs[2], _ref(dout, rhs, g, O.TRANS_RHS), 1e-5)
+    _check(outs[3], _ref(lhs, dout, g, O.RAGGED_CONTRACTING), 1e-5)
+
+  side = torch.cuda.Stream()
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.stream(side):
+    run()
+    side.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+      outs = run()
+  torch.cuda.synchronize()
+  new_sizes = [[100, 0, 257, 9, 130, 80], [0, 300, 1, 0, 200, 139], [640, 0, 0, 0, 0, 0]]
+  new_small = [[3, 0, 16, 1, 7, 2], [0, 0, 0, 0, 0, 0], [16, 1, 0, 12, 0, 11]]
+  for sizes, ssizes in zip(new_sizes, new_small):
+    gs.copy_(torch.tensor(sizes, dtype=torch.int32))
+    small_gs.copy_(torch.tensor(ssizes, dtype=torch.int32))
+    lhs.copy_(mk((m, k), 1.0))
+    small_rhs.copy_(mk((G, 1024, 256), 1 / 32))
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    check(outs)
+    check(run())  # eager work between the replays
+
+
 def test_unsupported_inputs_are_declined(device):
   a = torch.zeros(64, 100, dtype=torch.bfloat16, device=device)  # k not a multiple of any block_k
   b = torch.zeros(2, 100, 64, dtype=torch.bfloat16, device=device)
