@@ -19,6 +19,8 @@
  *                               activate(tmp[:, :n]) * tmp[:, n:] with tmp = ragged_dot(lhs, [gate, up])
  *   tkx_ragged_dot_drhs         RAGGED_CONTRACTING_DOT_DIM_NUMS (base.py:50-54), the drhs of
  *                               base.py:448-461; kernel counterpart pallas_mosaic_gpu_kernel_sm90.py:184-285
+ *   tkx_dequantize_weights      quantization.py:80-83 (as_array: qvalue * scale with tile-repeat
+ *                               broadcasting) for int8 weights with sub-channel scales
  *   TkxConfig                   pallas_mosaic_gpu_common.py:45-73 (Config)
  */
 #ifndef TKX_RAGGED_DOT_H_
@@ -131,6 +133,16 @@ int32_t tkx_ragged_dot_fwd_fused(const void* lhs, const void* rhs, const int32_t
 int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* group_sizes, void* out,
                             void* workspace, int64_t m, int64_t k, int64_t n, int64_t num_groups,
                             int32_t dtype, int32_t out_dtype, const TkxConfig* config, tkx_stream_t stream);
+
+/* Weights with several scale blocks along k (the scale tile (1, t_k, 1) with t_k < k of
+ * pallas_mosaic_gpu_kernel_sm90_quant.py:91-97; quantization.py:80-83 for the dequantisation):
+ *   out[g, kk, c] = qvalue[g, kk, c] * scale[g, kk / scale_block_k, c]
+ * qvalue int8 [G,k,n], scale f32 [G, k / scale_block_k, n], out bf16 [G,k,n] (caller-owned); the
+ * result feeds the bf16 kernels. (scale_block_k == k needs no such pass: tkx_ragged_dot_fwd applies
+ * one scale per (group, column) in its epilogue.) One streaming kernel on `stream`. */
+int32_t tkx_dequantize_weights(const void* qvalue, const float* scale, void* out, int64_t num_groups, int64_t k,
+                               int64_t n, int64_t scale_block_k, int32_t q_dtype, int32_t out_dtype,
+                               tkx_stream_t stream);
 
 /* Enumerates compiled kernel variants, for the autotuner's search space.
  * kind: 0 = fwd/dlhs variants, 1 = drhs variants.  Returns the count; tkx_ragged_dot_variant fills

@@ -233,9 +233,10 @@ def test_vjp(m, k, n, activation, device):
   assert O.rel_l2(_np(b_t.grad), b_ref.grad.numpy()) <= 4e-3
 
 
-@pytest.mark.parametrize("b_tile_shape,supported", [((1, 256, 1), True), ((1, 16, 1), False), ((1, 1, 16), False)])
+@pytest.mark.parametrize("b_tile_shape,supported", [((1, 256, 1), True), ((1, 16, 1), True), ((1, 1, 16), False)])
 def test_quantized_int8_weights(b_tile_shape, supported, device):
-  """bf16 x int8: per-(group, column) scales run natively; other scale tilings are declined."""
+  """bf16 x int8: per-(group, column) scales run in the kernels' epilogue, sub-channel scales along k
+  through the widening pass; scale tiles along n are declined."""
   G, m, k, n = 8, 512, 256, 512
   a, _, gs = _inputs("test_quantized", G, m, k, n, torch.bfloat16, device, random_groups=True)
   rng = np.random.default_rng(11)
@@ -488,6 +489,29 @@ def test_rhs_bias_and_gateup_fusion(m, k, n2, gs, act, device):
   _check(got, O.silu(plain), 1e-5)
   with pytest.raises(NotImplementedError):
     op(lhs, rhs, group_sizes=gst, fuse_gateup_activation="swigluoai")
+
+
+@pytest.mark.parametrize("m,blocks", [(300, 4), (24, 8), (1100, 2)])
+def test_int8_weights_with_sub_channel_scales(m, blocks, device):
+  """Scale tile (1, t_k, 1) with t_k < k (pallas_mosaic_gpu_kernel_sm90_quant.py:91-97): the weights are
+  widened to bf16 by `tkx_dequantize_weights` (bit-exact against the oracle's dequantisation rounded to
+  bf16) and the result matches the oracle on the dequantised weights."""
+  rng = np.random.default_rng(m + blocks)
+  G, k, n = 5, 1024, 208
+  gs = rng.multinomial(m - 7, [0.3, 0.0, 0.4, 0.1, 0.2]).astype(np.int32)
+  gst = torch.tensor(gs, device=device)
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  q = torch.tensor(rng.integers(-128, 128, (G, k, n)).astype(np.int8), device=device)
+  scale = torch.tensor((np.abs(rng.normal(0, 0.01, (G, blocks, n))) + 1e-3).astype(np.float32), device=device)
+  deq = O.dequantize(q.cpu().numpy(), _np(scale))
+  wide = hip_ops.dequantize_weights(q, scale)
+  assert wide.dtype == torch.bfloat16 and np.array_equal(_np(wide), O.round_to_bf16(deq.astype(np.float32)))
+  out = tokamax_amd.HipRaggedDot()(lhs, tokamax_amd.QArray(q, scale), group_sizes=gst, preferred_element_type=torch.float32)
+  _check(out, O.ragged_dot(_np(lhs), _np(wide), gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 1e-5)
+  _check(out, O.ragged_dot(_np(lhs), deq, gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 3e-2)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  with pytest.raises(NotImplementedError):  # a scale that does not tile k
+    tokamax_amd.HipRaggedDot()(lhs, tokamax_amd.QArray(q, torch.ones(G, 3, n, device=device)), group_sizes=gst)
 
 
 def test_hip_graph_replays_follow_new_inputs_and_group_sizes(device):

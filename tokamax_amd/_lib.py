@@ -29,6 +29,7 @@ EXPORTED_SYMBOLS = (
     "tkx_ragged_dot_fwd",
     "tkx_ragged_dot_fwd_fused",
     "tkx_ragged_dot_drhs",
+    "tkx_dequantize_weights",
     "tkx_ragged_dot_num_variants",
     "tkx_ragged_dot_variant",
 )
@@ -77,6 +78,8 @@ def _declare(lib):
                                            cfgp, vp]
   lib.tkx_ragged_dot_drhs.restype = i32
   lib.tkx_ragged_dot_drhs.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32, cfgp, vp]
+  lib.tkx_dequantize_weights.restype = i32
+  lib.tkx_dequantize_weights.argtypes = [vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
   lib.tkx_ragged_dot_num_variants.restype = i32
   lib.tkx_ragged_dot_num_variants.argtypes = [i32]
   lib.tkx_ragged_dot_variant.restype = i32

@@ -311,6 +311,23 @@ int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* gr
   return launch(v, p, (int64_t)num_groups * p.m_tiles * p.n_tiles, stream);
 }
 
+int32_t tkx_dequantize_weights(const void* qvalue, const float* scale, void* out, int64_t num_groups, int64_t k,
+                               int64_t n, int64_t scale_block_k, int32_t q_dtype, int32_t out_dtype,
+                               tkx_stream_t stream) {
+  if (!qvalue || !scale || !out) return set_error(TKX_ERR_INVALID, "null pointer argument");
+  if (num_groups < 1 || k < 1 || n < 1 || scale_block_k < 1)
+    return set_error(TKX_ERR_INVALID, "bad sizes G=%lld k=%lld n=%lld block=%lld", (long long)num_groups, (long long)k,
+                     (long long)n, (long long)scale_block_k);
+  if (q_dtype != TKX_I8 || out_dtype != TKX_BF16)
+    return set_error(TKX_ERR_UNSUPPORTED, "dequantisation is int8 -> bf16 only (got %d -> %d)", q_dtype, out_dtype);
+  if (k % scale_block_k != 0) return set_error(TKX_ERR_INVALID, "k=%lld is not a multiple of the scale block %lld",
+                                               (long long)k, (long long)scale_block_k);
+  if (n % 16 != 0) return set_error(TKX_ERR_UNSUPPORTED, "n must be a multiple of 16");
+  if (((uintptr_t)qvalue | (uintptr_t)scale | (uintptr_t)out) % 16 != 0)
+    return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
+  return launch_dequant_i8(qvalue, scale, out, num_groups, k, n, scale_block_k, static_cast<hipStream_t>(stream));
+}
+
 int32_t tkx_ragged_dot_num_variants(int32_t kind) {
   int32_t n = 0;
   for (const Variant& v : registry().all) n += ((v.mode == kDrhs) == (kind == 1));

@@ -99,6 +99,10 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
                       int64_t m, int64_t k, int64_t n, int64_t G, int32_t rhs_dtype, int32_t out_dtype,
                       int32_t activation, int32_t depth, hipStream_t stream);
 
+// ---- dequantisation of int8 weights with sub-channel scales to bf16 ------------------------------
+int32_t launch_dequant_i8(const void* q, const float* scale, void* out, int64_t G, int64_t k, int64_t n, int64_t t_k,
+                          hipStream_t stream);
+
 // Each dtype family registers its variants from its own translation unit.
 const Variant* variants_bf16(int* count);
 const Variant* variants_f16(int* count);

@@ -81,6 +81,16 @@ def _fused_activation_name(activation) -> str | None:
     return None
 
 
+def _scale_blocks_along_k(q: QArray) -> int | None:
+  """Number of scale blocks along k of a quantised rhs [g,k,n] (scale [g, blocks, n]), or None if the
+  scale has another form."""
+  g, k, n = q.qvalue.shape
+  shape = tuple(q.scale.shape)
+  if len(shape) != 3 or shape[0] != g or shape[2] != n or shape[1] < 1 or k % shape[1] != 0:
+    return None
+  return shape[1]
+
+
 def _dtype_of(x) -> torch.dtype:
   return x.qtype if isinstance(x, (QArray, AsQArray)) else x.dtype
 
@@ -181,10 +191,17 @@ class HipRaggedDot(base.RaggedDot):
       if mode != 0 or rhs.zero_point is not None:
         raise NotImplementedError("Quantised rhs: default dimension numbers without zero point only.")
       g, k, n = rhs.qvalue.shape
-      if tuple(rhs.scale.shape) != (g, 1, n):
+      blocks = _scale_blocks_along_k(rhs)
+      if blocks is None:
         raise NotImplementedError(
-            f"rhs scale must have shape [g,1,n] (one per group and column), got {tuple(rhs.scale.shape)}")
-      rhs_scale_, rhs_v = rhs.scale, rhs.qvalue
+            f"rhs scale must have shape [g,1,n] or [g,k/t_k,n] (sub-channel along k), got {tuple(rhs.scale.shape)}")
+      if blocks == 1:
+        rhs_scale_, rhs_v = rhs.scale, rhs.qvalue  # one scale per (group, column): applied in the epilogue
+      else:
+        # Several scale blocks along k: widened to bf16 by a streaming pass, then the bf16 kernels.
+        if isinstance(lhs, QArray) or rhs.qvalue.dtype != torch.int8 or n % 16 != 0:
+          raise NotImplementedError("Sub-channel rhs scales: int8 weights, unquantised lhs and n % 16 == 0 only.")
+        rhs_v = hip_ops.dequantize_weights(rhs.qvalue, rhs.scale)
     else:
       rhs_v = rhs
 
@@ -272,6 +289,8 @@ class HipRaggedDot(base.RaggedDot):
       num_groups = rhs_shape[0]
       rows, cols, contraction = lhs_shape[0], rhs_shape[2], rhs_shape[1]
     lhs_dt, rhs_dt = _dtype_of(lhs), _dtype_of(rhs)
+    if isinstance(rhs, QArray) and (_scale_blocks_along_k(rhs) or 1) > 1:
+      rhs_dt = torch.bfloat16  # sub-channel scales: `_fwd` widens the weights to bf16 first
     if (ba.kwargs.get("precision") == precision_lib.DotAlgorithmPreset.BF16_BF16_F32
         and not isinstance(lhs, (QArray, AsQArray)) and not isinstance(rhs, (QArray, AsQArray))):
       lhs_dt = rhs_dt = torch.bfloat16  # `_fwd` casts both operands for this preset

@@ -157,6 +157,25 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
   return out
 
 
+def dequantize_weights(qvalue: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+  """bf16 [g,k,n] = int8 qvalue [g,k,n] * scale [g, k/t_k, n] repeated t_k times along k (quantization.py:80-83)."""
+  _require_cuda(qvalue, scale)
+  lib = _lib.load()
+  if qvalue.dim() != 3 or scale.dim() != 3 or qvalue.dtype != torch.int8:
+    raise NotImplementedError("expected int8 qvalue [g,k,n] and scale [g, k/t_k, n]")
+  G, k, n = qvalue.shape
+  if scale.shape[0] != G or scale.shape[2] != n or scale.shape[1] < 1 or k % scale.shape[1] != 0:
+    raise NotImplementedError(f"scale shape {tuple(scale.shape)} does not tile qvalue {tuple(qvalue.shape)} along k")
+  qvalue = qvalue.contiguous()
+  scale = scale.to(torch.float32).contiguous()
+  out = torch.empty((G, k, n), dtype=torch.bfloat16, device=qvalue.device)
+  with torch.cuda.device(qvalue.device):
+    st = lib.tkx_dequantize_weights(_ptr(qvalue), _ptr(scale), _ptr(out), G, k, n, k // scale.shape[1],
+                                    _lib.TKX_I8, _lib.TKX_BF16, _stream(qvalue.device))
+  _lib.check(st)
+  return out
+
+
 def ragged_dot_drhs(lhs, dout, group_sizes, num_groups: int, *, config: KernelConfig,
                     out_dtype: torch.dtype) -> torch.Tensor:
   """out[g,k,n] = lhs[rows_g,k]^T . dout[rows_g,n]."""
