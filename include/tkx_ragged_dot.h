@@ -119,12 +119,17 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
  *     act(lhs.gate + bias_gate) * (lhs.up + bias_up), `activation` (not NONE) naming act; needs
  *     n % 16 == 0, k % block_k == 0 and a variant of mode 3 (see tkx_ragged_dot_variant).
  *   gateup = 0: as tkx_ragged_dot_fwd plus the bias; `activation` applies to the biased result.
- * The streaming small-m kernel (block_m == 16) takes neither. */
+ *   rhs_scale_blocks: rhs_scale is f32[G, rhs_scale_blocks, n], block b scaling the k rows
+ *     [b * k/blocks, (b+1) * k/blocks) (scale tile (1, t_k, 1), pallas_mosaic_gpu_kernel_sm90_quant.py:91-97).
+ *     1 = one scale per (group, column). More than 1 is taken by the streaming small-m kernel only
+ *     (int8 weights, k/blocks a power of two >= 32); for the tiled kernels widen the weights with
+ *     tkx_dequantize_weights first.
+ * The streaming small-m kernel (block_m == 16) takes neither a bias nor gate-up fusion. */
 int32_t tkx_ragged_dot_fwd_fused(const void* lhs, const void* rhs, const int32_t* group_sizes,
                                  const float* lhs_scale, const float* rhs_scale, const float* rhs_bias, void* out,
                                  void* workspace, int64_t m, int64_t k, int64_t n, int64_t num_groups,
-                                 int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype, int32_t activation,
-                                 int32_t gateup, const TkxConfig* config, tkx_stream_t stream);
+                                 int64_t rhs_scale_blocks, int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype,
+                                 int32_t activation, int32_t gateup, const TkxConfig* config, tkx_stream_t stream);
 
 /* Part (4-drhs): out[G,k,n] = lhs[rows_g, k]^T . dout[rows_g, n], zeros for empty groups.
  * lhs [m,k], dout [m,n] row-major of `dtype` (f32/bf16/f16); out_dtype f32/bf16/f16.

@@ -514,6 +514,35 @@ def test_int8_weights_with_sub_channel_scales(m, blocks, device):
     tokamax_amd.HipRaggedDot()(lhs, tokamax_amd.QArray(q, torch.ones(G, 3, n, device=device)), group_sizes=gst)
 
 
+@pytest.mark.parametrize("blocks,depth", [(2, 2), (8, 2), (32, 4), (4, 8)])
+def test_small_m_int8_kernel_with_sub_channel_scales(blocks, depth, device):
+  """The streaming small-m kernel scales int8 weights per k-block while it widens them: same result as
+  the oracle on the weights dequantised and rounded to bf16; the op picks this path for small groups."""
+  rng = np.random.default_rng(blocks)
+  k, n = 1024, 208
+  gs = np.array([3, 0, 0, 17, 1, 0, 16, 2], np.int32)
+  G, m = len(gs), int(gs.sum()) + 5
+  gst = torch.tensor(gs, device=device)
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  q = torch.tensor(rng.integers(-128, 128, (G, k, n)).astype(np.int8), device=device)
+  scale = torch.tensor((np.abs(rng.normal(0, 0.01, (G, blocks, n))) + 1e-3).astype(np.float32), device=device)
+  wide = O.round_to_bf16(O.dequantize(q.cpu().numpy(), _np(scale)).astype(np.float32))
+  want = O.ragged_dot(_np(lhs), wide, gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+  cfg = hip_ops.KernelConfig(16, 128, 32, 1, 4, depth)
+  out = hip_ops.ragged_dot_fwd(lhs, q, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale)
+  _check(out, want, 1e-5)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  with pytest.raises(NotImplementedError):  # the tiled kernels take one scale per (group, column)
+    hip_ops.ragged_dot_fwd(lhs, q, gst, config=hip_ops.KernelConfig(32, 128, 64, 1, 4, 4), out_dtype=torch.float32,
+                           rhs_scale=scale)
+  op = tokamax_amd.HipRaggedDot()
+  small = np.array([3, 0, 0, 7, 1, 0, 6, 2], np.int32)
+  sgs = torch.tensor(small, device=device)
+  assert op.bind(lhs[:19], tokamax_amd.QArray(q, scale), group_sizes=sgs).default_config.block_m == 16
+  _check(op(lhs[:19], tokamax_amd.QArray(q, scale), group_sizes=sgs, preferred_element_type=torch.float32),
+         O.ragged_dot(_np(lhs[:19]), wide, small, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 1e-5)
+
+
 def test_hip_graph_replays_follow_new_inputs_and_group_sizes(device):
   """The entry points allocate nothing, synchronise nothing and schedule on the device, so a captured
   HIP graph stays valid when the contents of lhs, the weights and even group_sizes change between

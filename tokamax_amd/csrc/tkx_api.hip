@@ -132,7 +132,8 @@ namespace {
 int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, const float* lhs_scale,
                  const float* rhs_scale, const float* rhs_bias, void* out, void* workspace, int64_t m, int64_t k,
                  int64_t n, int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype, int32_t mode,
-                 int32_t activation, bool gateup, const TkxConfig* config, tkx_stream_t stream_) {
+                 int32_t activation, bool gateup, int64_t rhs_scale_blocks, const TkxConfig* config,
+                 tkx_stream_t stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (!lhs || !rhs || !group_sizes || !out || !workspace || !config)
     return set_error(TKX_ERR_INVALID, "null pointer argument");
@@ -180,13 +181,18 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
     if (rhs_bias != nullptr || gateup) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no bias or gate-up fusion");
     if (rhs_scale != nullptr && rhs_dtype != TKX_I8)
       return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes an rhs scale with int8 weights only");
-    if (!decode_supported(lhs_dtype, rhs_dtype, m, k, n, num_groups))
+    if (!decode_supported(lhs_dtype, rhs_dtype, m, k, n, num_groups, rhs_scale ? rhs_scale_blocks : 1))
       return set_error(TKX_ERR_UNSUPPORTED,
-                       "decode kernel needs k %% 1024 == 0 and n %% 8 == 0 (k=%lld n=%lld G=%lld)",
-                       (long long)k, (long long)n, (long long)num_groups);
+                       "decode kernel needs k %% 1024 == 0, n %% 8 == 0 and scale blocks of a power-of-two multiple of 32"
+                       " rows (k=%lld n=%lld G=%lld scale blocks=%lld)",
+                       (long long)k, (long long)n, (long long)num_groups, (long long)rhs_scale_blocks);
     return launch_decode(lhs, rhs, rhs_scale, group_sizes, out, m, k, n, num_groups, rhs_dtype, out_dtype, activation,
-                         c.num_stages, stream);
+                         c.num_stages, rhs_scale ? rhs_scale_blocks : 1, stream);
   }
+  if (rhs_scale && rhs_scale_blocks != 1)
+    return set_error(TKX_ERR_UNSUPPORTED,
+                     "the tiled kernels take one rhs scale per (group, column); widen weights with %lld scale blocks"
+                     " along k with tkx_dequantize_weights first", (long long)rhs_scale_blocks);
 
   const WsLayout L = ws_layout(m, num_groups, c.block_m);
   int32_t st = launch_schedule(group_sizes, num_groups, m, c.block_m, c.align_tile, c.grid_tile_width,
@@ -243,18 +249,19 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
                            int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype, int32_t mode,
                            int32_t activation, const TkxConfig* config, tkx_stream_t stream) {
   return fwd_impl(lhs, rhs, group_sizes, lhs_scale, rhs_scale, nullptr, out, workspace, m, k, n, num_groups, lhs_dtype,
-                  rhs_dtype, out_dtype, mode, activation, false, config, stream);
+                  rhs_dtype, out_dtype, mode, activation, false, 1, config, stream);
 }
 
 int32_t tkx_ragged_dot_fwd_fused(const void* lhs, const void* rhs, const int32_t* group_sizes, const float* lhs_scale,
                                  const float* rhs_scale, const float* rhs_bias, void* out, void* workspace, int64_t m,
-                                 int64_t k, int64_t n, int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype,
-                                 int32_t out_dtype, int32_t activation, int32_t gateup, const TkxConfig* config,
-                                 tkx_stream_t stream) {
+                                 int64_t k, int64_t n, int64_t num_groups, int64_t rhs_scale_blocks, int32_t lhs_dtype,
+                                 int32_t rhs_dtype, int32_t out_dtype, int32_t activation, int32_t gateup,
+                                 const TkxConfig* config, tkx_stream_t stream) {
   if (gateup != 0 && gateup != 1) return set_error(TKX_ERR_INVALID, "gateup must be 0 or 1");
+  if (rhs_scale_blocks < 1) return set_error(TKX_ERR_INVALID, "rhs_scale_blocks must be >= 1");
   if (gateup && activation == TKX_ACT_NONE) return set_error(TKX_ERR_INVALID, "gate-up fusion needs an activation");
   return fwd_impl(lhs, rhs, group_sizes, lhs_scale, rhs_scale, rhs_bias, out, workspace, m, k, n, num_groups, lhs_dtype,
-                  rhs_dtype, out_dtype, TKX_MODE_DEFAULT, activation, gateup == 1, config, stream);
+                  rhs_dtype, out_dtype, TKX_MODE_DEFAULT, activation, gateup == 1, rhs_scale_blocks, config, stream);
 }
 
 int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* group_sizes, void* out, void* workspace,

@@ -37,6 +37,8 @@ struct DecodeParams {
   const int32_t* group_sizes;
   void* out;
   int32_t m, k, n, num_groups, n_tiles, out_dtype, activation;
+  int32_t scale_blocks;     // scale blocks along k: scale is [G, scale_blocks, n]
+  int32_t log2_block_rows;  // scale_blocks > 1: log2 of the contraction rows per scale block
 };
 
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
@@ -94,6 +96,16 @@ __device__ __forceinline__ i32x4 column_fragment(const i32x2 (&rows)[8]) {
   }
   return out;
 }
+// Sub-channel scales: the same column, each value multiplied by the column's scale of the current
+// k-block and rounded to bf16 (nearest even).
+template <int J>
+__device__ __forceinline__ i32x4 column_fragment_scaled(const i32x2 (&rows)[8], float scale) {
+  bf16x8 out;
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    out[e] = (__bf16)(__builtin_bit_cast(float, i8_to_f32_bits<(J & 3)>(rows[e][J >> 2])) * scale);
+  return __builtin_bit_cast(i32x4, out);
+}
 // 16-bit weights: half-word J of each of 8 loaded 16-byte rows, two rows per byte permute.
 template <int J>
 __device__ __forceinline__ i32x4 column_fragment(const i32x4 (&rows)[8]) {
@@ -114,8 +126,13 @@ __device__ __forceinline__ f32x4_t mma_16x16x32(i32x4 w, i32x4 a, f32x4_t acc) {
 }
 
 // EW = element kind of the weights; the lhs is bf16 for int8 weights, else of the weights' type.
-template <int EW, int kDecDepth, int kMinWgs>
+// SUB (int8 weights): the scale has several blocks along k; every step fetches the 8 scales of its
+// lane's columns for its k-block alongside the weights (the same unconditional pipeline; they come
+// from L2, a scale row serves all the weight rows of its block) and the weights are scaled while
+// they are widened, instead of one multiply per output in the epilogue.
+template <int EW, int kDecDepth, int kMinWgs, bool SUB = false>
 __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const DecodeParams p) {
+  static_assert(!SUB || EW == kEI8, "sub-channel scales belong to int8 weights");
   constexpr int EA = EW == kEI8 ? kEBF16 : EW;
   constexpr int WESZ = WeightRow<EW>::ESZ;
   typedef typename WeightRow<EW>::T WRow;
@@ -148,6 +165,10 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
 
   WRow breg[kDecDepth][8];
   i32x4 areg[kDecDepth];
+  i32x4 sreg[SUB ? kDecDepth : 1][2];  // SUB: f32 scales of columns 8i..8i+7 for the step's k-block
+  const __amdgpu_buffer_rsrc_t sbuf = buffer_of(SUB ? p.scale + (int64_t)g * p.scale_blocks * p.n : nullptr,
+                                                SUB ? (uint32_t)p.scale_blocks * (uint32_t)p.n * 4u : 0u);
+  const uint32_t soff = (uint32_t)colb * 4u;
   // Nothing looks at a loaded value before its step comes up, so the only waits are the per-step
   // vmcnt of the oldest group.
   const __amdgpu_buffer_rsrc_t wbuf = buffer_of(wbase, (uint32_t)kw * (uint32_t)p.n * WESZ);
@@ -156,6 +177,13 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
     const uint32_t so = (uint32_t)__builtin_amdgcn_readfirstlane((int)(step * step_bytes));
 #pragma unroll
     for (int e = 0; e < 8; ++e) breg[slot][e] = load_weight_row<EW>(wbuf, boff[e], so);
+    if constexpr (SUB) {
+      // (Past the wave's slice the block index runs past the buffer and the loads return zero.)
+      const uint32_t kb = (uint32_t)(k_begin + step * kDecKS) >> p.log2_block_rows;
+      const uint32_t ro = (uint32_t)__builtin_amdgcn_readfirstlane((int)(kb * (uint32_t)p.n * 4u));
+      sreg[slot][0] = buffer_load_16(sbuf, soff, ro);
+      sreg[slot][1] = buffer_load_16(sbuf, soff + 16u, ro);
+    }
   };
 #pragma unroll
   for (int d = 0; d < kDecDepth; ++d) {
@@ -168,7 +196,7 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
   f32x4_t scale_lo = {1.f, 1.f, 1.f, 1.f}, scale_hi = {1.f, 1.f, 1.f, 1.f};
   {
     const int col = col0 + (tid & 15) * 8;
-    if (p.scale != nullptr && col + 8 <= p.n) {
+    if (!SUB && p.scale != nullptr && col + 8 <= p.n) {
       const float* sc = p.scale + (int64_t)g * p.n + col;
       scale_lo = *reinterpret_cast<const f32x4_t*>(sc);
       scale_hi = *reinterpret_cast<const f32x4_t*>(sc + 4);
@@ -235,16 +263,27 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
         // MFMA j contracts this step's 32 rows for the columns {8i + j}; operands are swapped, so a
         // lane ends up with one lhs row and the weight-column indices 4q..4q+3.
         i32x4 lo[4], hi[4];
-        lo[0] = column_fragment<0>(breg[d]);
-        lo[1] = column_fragment<1>(breg[d]);
-        lo[2] = column_fragment<2>(breg[d]);
-        lo[3] = column_fragment<3>(breg[d]);
+        float col_scale[8];  // SUB: scales of the lane's 8 columns for this step's k-block
+        if constexpr (SUB) {
+          const f32x4_t s_lo = __builtin_bit_cast(f32x4_t, sreg[d][0]), s_hi = __builtin_bit_cast(f32x4_t, sreg[d][1]);
+          col_scale[0] = s_lo[0]; col_scale[1] = s_lo[1]; col_scale[2] = s_lo[2]; col_scale[3] = s_lo[3];
+          col_scale[4] = s_hi[0]; col_scale[5] = s_hi[1]; col_scale[6] = s_hi[2]; col_scale[7] = s_hi[3];
+        }
+        auto column = [&](auto j_tag) {
+          constexpr int J = decltype(j_tag)::value;
+          if constexpr (SUB) return column_fragment_scaled<J>(breg[d], col_scale[J]);
+          else return column_fragment<J>(breg[d]);
+        };
+        lo[0] = column(std::integral_constant<int, 0>{});
+        lo[1] = column(std::integral_constant<int, 1>{});
+        lo[2] = column(std::integral_constant<int, 2>{});
+        lo[3] = column(std::integral_constant<int, 3>{});
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] = mma_16x16x32<EA>(lo[j], afrag, acc[j]);
-        hi[0] = column_fragment<4>(breg[d]);
-        hi[1] = column_fragment<5>(breg[d]);
-        hi[2] = column_fragment<6>(breg[d]);
-        hi[3] = column_fragment<7>(breg[d]);
+        hi[0] = column(std::integral_constant<int, 4>{});
+        hi[1] = column(std::integral_constant<int, 5>{});
+        hi[2] = column(std::integral_constant<int, 6>{});
+        hi[3] = column(std::integral_constant<int, 7>{});
         // Refill unconditionally: past the wave's slice the weight buffer reads as zero without
         // touching memory, and a uniform loop body keeps the waits partial. The scheduling fences
         // keep the compiler from sinking the loads to the end of the block, which would collapse
@@ -317,9 +356,16 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
 }  // namespace
 
 // Whether the decode kernel can run this problem (else the caller uses the tiled kernel).
-bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k, int64_t n, int64_t G) {
+bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k, int64_t n, int64_t G,
+                      int64_t scale_blocks) {
   (void)m;
   (void)G;
+  if (scale_blocks != 1) {
+    // Sub-channel scales: int8 weights, blocks of a power-of-two number of rows that whole steps fit.
+    if (rhs_dtype != TKX_I8 || scale_blocks < 1 || k % scale_blocks != 0) return false;
+    const int64_t rows = k / scale_blocks;
+    if (rows % kDecKS != 0 || (rows & (rows - 1)) != 0 || scale_blocks * n * 4 >= (1LL << 31)) return false;
+  }
   const bool types = (lhs_dtype == TKX_BF16 && (rhs_dtype == TKX_I8 || rhs_dtype == TKX_BF16)) ||
                      (lhs_dtype == TKX_F16 && rhs_dtype == TKX_F16);
   if (!types) return false;
@@ -330,8 +376,12 @@ bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k
 
 int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
                       int64_t m, int64_t k, int64_t n, int64_t G, int32_t rhs_dtype, int32_t out_dtype,
-                      int32_t activation, int32_t depth, hipStream_t stream) {
+                      int32_t activation, int32_t depth, int64_t scale_blocks, hipStream_t stream) {
   DecodeParams p;
+  p.scale_blocks = (int32_t)scale_blocks;
+  p.log2_block_rows = 0;
+  for (int64_t rows = k / scale_blocks; rows > 1; rows >>= 1) ++p.log2_block_rows;
+  const bool sub = scale_blocks > 1 && scale != nullptr;
   p.lhs = static_cast<const unsigned char*>(lhs);
   p.rhs = static_cast<const unsigned char*>(rhs);
   p.scale = scale;
@@ -351,7 +401,10 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
   // `depth` = steps of loads in flight per wave; deeper pipelines need more registers and allow
   // fewer waves per CU. A step of 16-bit weights takes twice the registers of an int8 one.
   const void* fn;
-  if (rhs_dtype == TKX_I8) {
+  if (sub) {
+    fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 2, 3, true>)
+                    : reinterpret_cast<const void*>(&decode_kernel<kEI8, 4, 2, true>);  // (8 deep would spill)
+  } else if (rhs_dtype == TKX_I8) {
     fn = depth <= 2   ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 2, 4>)
          : depth <= 4 ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 4, 3>)
                       : reinterpret_cast<const void*>(&decode_kernel<kEI8, 8, 2>);

@@ -201,7 +201,13 @@ class HipRaggedDot(base.RaggedDot):
         # Several scale blocks along k: widened to bf16 by a streaming pass, then the bf16 kernels.
         if isinstance(lhs, QArray) or rhs.qvalue.dtype != torch.int8 or n % 16 != 0:
           raise NotImplementedError("Sub-channel rhs scales: int8 weights, unquantised lhs and n % 16 == 0 only.")
-        rhs_v = hip_ops.dequantize_weights(rhs.qvalue, rhs.scale)
+        rows = k // blocks
+        if (config.block_m == 16 and rows % 32 == 0 and rows & (rows - 1) == 0 and rhs_bias is None
+            and fuse_gateup_activation is None):
+          # The streaming small-m kernel scales the weights per k-block while it widens them.
+          rhs_scale_, rhs_v = rhs.scale, rhs.qvalue
+        else:
+          rhs_v = hip_ops.dequantize_weights(rhs.qvalue, rhs.scale)
     else:
       rhs_v = rhs
 

@@ -104,7 +104,8 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
                    gateup: bool = False, workspace_out: list | None = None) -> torch.Tensor:
   """out[m,n] = lhs[m,k] . rhs[g,k,n]   (trans_rhs: out[m,k] = lhs[m,n] . rhs[g,k,n]^T).
 
-  `rhs_bias` ([g,n] or [g,1,n]) is added to the scaled result before the activation. `gateup`: rhs
+  `rhs_scale` is [g,n] / [g,1,n], or [g,blocks,n] with `blocks` scale blocks along k (streaming small-m
+  kernel only). `rhs_bias` ([g,n] or [g,1,n]) is added to the scaled result before the activation. `gateup`: rhs
   columns are [gate | up] and out[m,n/2] = activation(gate part) * (up part) (base.py:211-217).
   `workspace_out`, if given, receives the int32 workspace the call filled (schedule arrays included)."""
   _require_cuda(lhs, rhs, group_sizes, lhs_scale, rhs_scale, rhs_bias)
@@ -127,10 +128,13 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
     lhs_scale = lhs_scale.to(torch.float32).contiguous().view(-1)
     if lhs_scale.numel() != m:
       raise NotImplementedError("lhs scale must be one f32 per row")
+  scale_blocks = 1
   if rhs_scale is not None:
+    if rhs_scale.dim() == 3 and rhs_scale.shape[1] > 1:
+      scale_blocks = int(rhs_scale.shape[1])
     rhs_scale = rhs_scale.to(torch.float32).contiguous().view(-1)
-    if rhs_scale.numel() != G * n:
-      raise NotImplementedError("rhs scale must be one f32 per (group, column)")
+    if rhs_scale.numel() != G * scale_blocks * n or k % scale_blocks:
+      raise NotImplementedError("rhs scale must be one f32 per (group, column) or per (group, k-block, column)")
   if rhs_bias is not None:
     rhs_bias = rhs_bias.to(torch.float32).contiguous().view(-1)
     if rhs_bias.numel() != G * n:
@@ -140,7 +144,7 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
   ws = workspace(m, G, config.block_m, lhs.device)
   cfg = config.to_c()
   with torch.cuda.device(lhs.device):
-    if rhs_bias is None and not gateup:
+    if rhs_bias is None and not gateup and scale_blocks == 1:
       st = lib.tkx_ragged_dot_fwd(
           _ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(out), _ptr(ws), m, k, n, G,
           dtype_code(lhs.dtype), dtype_code(rhs.dtype), dtype_code(out_dtype),
@@ -149,7 +153,7 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
     else:
       st = lib.tkx_ragged_dot_fwd_fused(
           _ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(rhs_bias), _ptr(out), _ptr(ws), m, k,
-          n, G, dtype_code(lhs.dtype), dtype_code(rhs.dtype), dtype_code(out_dtype), _lib.ACTIVATIONS[activation],
+          n, G, scale_blocks, dtype_code(lhs.dtype), dtype_code(rhs.dtype), dtype_code(out_dtype), _lib.ACTIVATIONS[activation],
           1 if gateup else 0, ctypes.byref(cfg), _stream(lhs.device))
   _lib.check(st)
   if workspace_out is not None:
