@@ -380,7 +380,8 @@ def test_every_kernel_variant_through_c_abi(v, device):
 
 
 @pytest.mark.parametrize("depth", [2, 4, 8])
-@pytest.mark.parametrize("case", ["ragged", "two_chunks", "all_empty", "one_big_group", "first_and_last_empty"])
+@pytest.mark.parametrize("case", ["ragged", "two_chunks", "all_empty", "one_big_group", "first_and_last_empty",
+                                  "many_groups"])
 def test_small_m_int8_kernel_edges(case, depth, device):
   """The streaming small-m kernel: empty groups anywhere, more than 64 groups, groups taller than one
   16-row pass, a column count that is not a multiple of its 128-column tile, and a zero tail."""
@@ -395,6 +396,8 @@ def test_small_m_int8_kernel_edges(case, depth, device):
     gs = np.zeros(5, np.int32)
   elif case == "one_big_group":
     gs = np.array([0, 45, 0], np.int32)
+  elif case == "many_groups":  # more groups than the workgroup has threads: the row-offset sum loops
+    gs = rng.integers(0, 3, 600).astype(np.int32)
   else:
     gs = np.array([0, 4, 9, 0], np.int32)
   G, m = len(gs), int(gs.sum()) + 11
