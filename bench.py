@@ -266,6 +266,18 @@ def main():
             w.algorithmic_bytes(), "mfma", "fp8", cfg)
     del w, ql, qr
 
+    # the Mixtral shape with int8 weights (one f32 scale per (group, column)): the weight stream into LDS is half of bf16's
+    w = workloads.make("mixtral", device, seed=0)
+    gs = torch.tensor(w.group_sizes, device=device)
+    gen8 = torch.Generator(device=device).manual_seed(1)
+    q8 = tokamax_amd.QArray(torch.randint(-127, 128, tuple(w.rhs.shape), device=device, dtype=torch.int8, generator=gen8),
+                            (torch.rand(w.num_groups, 1, w.n, device=device, generator=gen8) + 0.5) / (127 * w.k ** 0.5))
+    cfg = op.bind(w.lhs, q8, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    nb = w.m * w.k * 2 + w.nonempty_groups * w.k * w.n + w.m * w.n * 2
+    measure("mixtral_prefill_int8_weights", lambda: op(w.lhs, q8, group_sizes=gs, preferred_element_type=torch.bfloat16),
+            w.flops, nb, "mfma", "bf16", cfg)
+    del w, q8
+
     w = workloads.make("vjp", device, seed=0)
     gs = torch.tensor(w.group_sizes, device=device)
     cfg = op.bind(w.dout, w.rhs, group_sizes=gs, ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS).default_config

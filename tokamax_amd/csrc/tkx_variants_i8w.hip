@@ -6,6 +6,10 @@ namespace tkx {
 #define FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEBF16, kEI8, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
+    FWD(256, 256, 32, 2, 4, 4),
+    FWD(256, 256, 64, 2, 4, 2),
+    FWD(256, 256, 64, 2, 4, 3),
+    FWD(128, 256, 64, 2, 4, 3),
     FWD(128, 128, 64, 2, 2, 4),
     FWD(64, 128, 64, 2, 2, 4),
     FWD(32, 128, 64, 1, 4, 4),
