@@ -26,18 +26,23 @@ __global__ __launch_bounds__(kDqThreads) void dequant_i8_kernel(const signed cha
     const int c0 = (int)(idx - row * chunks) * 16;
     const int64_t g = row / k;
     const int kk = (int)(row - g * k);
-    const i32x4 w = *reinterpret_cast<const i32x4*>(q + row * n + c0);
-    const float* s = scale + ((int64_t)g * kb_per_group + kk / t_k) * n + c0;
+    const i32x4 w = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(q + row * n + c0));
+    const f32x4* s = reinterpret_cast<const f32x4*>(scale + ((int64_t)g * kb_per_group + kk / t_k) * n + c0);
     bf16x8 lo, hi;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const float v = (float)(signed char)((w[e >> 2] >> (8 * (e & 3))) & 0xff) * s[e];
-      if (e < 8) lo[e] = (__bf16)v;
-      else hi[e - 8] = (__bf16)v;
+    for (int d = 0; d < 4; ++d) {
+      const f32x4 sc = s[d];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const float v = (float)(signed char)((w[d] >> (8 * b)) & 0xff) * sc[b];
+        const int e = 4 * d + b;
+        if (e < 8) lo[e] = (__bf16)v;
+        else hi[e - 8] = (__bf16)v;
+      }
     }
     __bf16* o = out + row * n + c0;
-    *reinterpret_cast<bf16x8*>(o) = lo;
-    *reinterpret_cast<bf16x8*>(o + 8) = hi;
+    __builtin_nontemporal_store(lo, reinterpret_cast<bf16x8*>(o));
+    __builtin_nontemporal_store(hi, reinterpret_cast<bf16x8*>(o + 8));
   }
 }
 
