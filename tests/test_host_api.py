@@ -319,7 +319,7 @@ def test_shipped_mi355x_cache_parses_and_names_compiled_variants():
   compiled = {(v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"], v["num_stages"])
               for kind in (0, 1) for v in _lib.variants(kind)}
   for key, data in loaded.items():
-    assert len(data) >= 8, key
+    assert len(data) >= 4, key
     for cfg in data:
       assert (cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages) in compiled
     assert data.fastest_config.block_m >= 128  # the tuned workloads are the large prefill / VJP shapes
