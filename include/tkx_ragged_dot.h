@@ -55,7 +55,8 @@ enum TkxMode {
   TKX_MODE_TRANS_RHS = 1 /* out[m,k] = lhs[m,n] . rhs[g,k,n]^T  (dlhs)    (base.py:45-49) */
 };
 
-enum TkxActivation { TKX_ACT_NONE = 0, TKX_ACT_RELU = 1, TKX_ACT_TANH = 2, TKX_ACT_SILU = 3, TKX_ACT_GELU_TANH = 4 };
+enum TkxActivation { TKX_ACT_NONE = 0, TKX_ACT_RELU = 1, TKX_ACT_TANH = 2, TKX_ACT_SILU = 3, TKX_ACT_GELU_TANH = 4,
+                     TKX_ACT_SIGMOID = 5 };
 
 /* Tunables; the gfx950 counterpart of the reference's Config (pallas_mosaic_gpu_common.py:45-73).
  * (block_m, block_n, block_k, waves_m, waves_n, num_stages) must name a compiled kernel variant
@@ -116,7 +117,7 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
 /* Forward (mode DEFAULT) with the fused epilogue terms of base.py:205-217.
  *   rhs_bias: f32[G,n] added to the scaled accumulator, or NULL.
  *   gateup = 1: rhs is [G,k,n] with its columns [gate | up] (n/2 each) and out is [m, n/2] =
- *     act(lhs.gate + bias_gate) * (lhs.up + bias_up), `activation` (not NONE) naming act; needs
+ *     act(lhs.gate + bias_gate) * (lhs.up + bias_up), `activation` naming act (NONE: the plain product); needs
  *     n % 16 == 0, k % block_k == 0 and a variant of mode 3 (see tkx_ragged_dot_variant).
  *   gateup = 0: as tkx_ragged_dot_fwd plus the bias; `activation` applies to the biased result.
  *   rhs_scale_blocks: rhs_scale is f32[G, rhs_scale_blocks, n], block b scaling the k rows

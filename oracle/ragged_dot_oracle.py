@@ -34,6 +34,9 @@ below therefore cites the reference call site it follows, and says what pins it:
                                                                                   activations against torch's silu /
                                                                                   gelu(approximate="tanh")
 
+  gated_linear_unit            gated_linear_unit/base.py:60-120                   torch matmul + torch activations on
+                                                                                  f64 (library routines)
+
 Status of "parity unpinned": `qwix.quantize` (absmax calibration / rounding) is
 NOT restated -- quantised inputs are generated directly as (qvalue, scale) pairs.
 `ragged_dot_fused` follows the docstring's formulas only: the one reference
@@ -281,6 +284,15 @@ def ragged_dot_fused(lhs, rhs, group_sizes, *, rhs_bias=None, gateup_activation=
     n = tmp.shape[1] // 2
     tmp = act(tmp[:, :n]) * tmp[:, n:]
   return _round_out(tmp, out_dtype)
+
+
+def gated_linear_unit(x, weights, activation=None):
+  """`activation(x @ weights[:, 0]) * (x @ weights[:, 1])` in float64 (gated_linear_unit/base.py:60-120);
+  `weights` is [K, 2, N], `activation` a NumPy callable or None."""
+  x = np.asarray(x, np.float64)
+  w = np.asarray(weights, np.float64)
+  gate, up = x @ w[:, 0, :], x @ w[:, 1, :]
+  return (gate if activation is None else activation(gate)) * up
 
 
 def ragged_dot_bruteforce(lhs, rhs, group_sizes, mode: str = DEFAULT):

@@ -546,6 +546,29 @@ def test_small_m_int8_kernel_with_sub_channel_scales(blocks, depth, device):
          O.ragged_dot(_np(lhs[:19]), wide, small, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 1e-5)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16])
+@pytest.mark.parametrize("shape", [((3, 70), 256, 192), ((1100,), 512, 1024), ((2, 2, 9), 128, 72)])
+def test_gated_linear_unit(shape, dtype, device):
+  """`gated_linear_unit` (gated_linear_unit/base.py:60-120) = the gate-up fused kernel with one group:
+  fused and unfused weights, the in-kernel activations, no activation, and a callable with no
+  in-kernel twin."""
+  lead, k, n = shape
+  rng = np.random.default_rng(k + n)
+  x = torch.tensor(rng.normal(0, 1, (*lead, k)).astype(np.float32), device=device).to(dtype)
+  w = torch.tensor(rng.normal(0, k ** -0.5, (k, 2, n)).astype(np.float32), device=device).to(dtype)
+  F = torch.nn.functional
+  acts = [(F.silu, O.silu), (torch.sigmoid, lambda v: 1 / (1 + np.exp(-v))), (torch.relu, lambda v: np.maximum(v, 0)),
+          (torch.tanh, np.tanh), (None, None), (F.softplus, lambda v: np.log1p(np.exp(v)))]
+  for act, ref_act in acts:
+    out = tokamax_amd.gated_linear_unit(x, w, activation=act)
+    assert out.shape == (*lead, n) and out.dtype == dtype
+    _check(out, O.gated_linear_unit(_np(x), _np(w), ref_act), 3e-3)
+  pair = (w[:, 0].contiguous(), w[:, 1].contiguous())
+  assert torch.equal(tokamax_amd.gated_linear_unit(x, pair, activation=F.silu), tokamax_amd.gated_linear_unit(x, w, activation=F.silu))
+  with pytest.raises(NotImplementedError):
+    tokamax_amd.gated_linear_unit(x, w.float(), activation=F.silu)
+
+
 def test_hip_graph_replays_follow_new_inputs_and_group_sizes(device):
   """The entry points allocate nothing, synchronise nothing and schedule on the device, so a captured
   HIP graph stays valid when the contents of lhs, the weights and even group_sizes change between

@@ -194,6 +194,18 @@ def test_fused_epilogue_terms():
                              rtol=1e-12, atol=1e-12)
 
 
+def test_gated_linear_unit_matches_torch():
+  rng = np.random.default_rng(3)
+  x, w = rng.normal(size=(2, 5, 7)), rng.normal(size=(7, 2, 4))
+  xt, wt = torch.tensor(x), torch.tensor(w)
+  want = torch.nn.functional.silu(xt @ wt[:, 0]) * (xt @ wt[:, 1])
+  np.testing.assert_allclose(O.gated_linear_unit(x, w, O.silu), want.numpy(), rtol=1e-12, atol=1e-12)
+  np.testing.assert_allclose(O.gated_linear_unit(x, w), ((xt @ wt[:, 0]) * (xt @ wt[:, 1])).numpy(), rtol=1e-12, atol=1e-12)
+  # one group that owns every row of the fused gate-up ragged dot is the same thing
+  np.testing.assert_allclose(O.ragged_dot_fused(x.reshape(10, 7), w.reshape(1, 7, 8), [10], gateup_activation="silu"),
+                             want.numpy().reshape(10, 4), rtol=1e-12, atol=1e-12)
+
+
 def test_dequantize_is_tile_repeat():
   rng = np.random.default_rng(9)
   q = rng.integers(-127, 128, (2, 8, 6)).astype(np.int8)

@@ -9,6 +9,8 @@ from tokamax_amd import config
 from tokamax_amd.autotuning.api import AutotuningResult, autotune
 from tokamax_amd.op import AUTO, BoundArguments, NullConfig, Op
 from tokamax_amd.quantization import AsQArray, QArray
+from tokamax_amd.gated_linear_unit.api import gated_linear_unit
+from tokamax_amd.gated_linear_unit.hip import HipGatedLinearUnit
 from tokamax_amd.ragged_dot.api import IMPLEMENTATIONS as RAGGED_DOT_IMPLEMENTATIONS
 from tokamax_amd.ragged_dot.api import ragged_dot, ragged_dot_general
 from tokamax_amd.ragged_dot.base import (
@@ -23,9 +25,10 @@ from tokamax_amd.ragged_dot.hip import Config as HipRaggedDotConfig
 from tokamax_amd.ragged_dot.hip import HipRaggedDot
 
 __all__ = [
-    "AUTO", "AsQArray", "AutotuningResult", "BoundArguments", "DEFAULT_RAGGED_DOT_DIM_NUMS", "HipRaggedDot",
+    "AUTO", "AsQArray", "AutotuningResult", "BoundArguments", "DEFAULT_RAGGED_DOT_DIM_NUMS", "HipGatedLinearUnit",
+    "HipRaggedDot",
     "HipRaggedDotConfig", "NullConfig", "Op", "QArray", "RAGGED_CONTRACTING_DOT_DIM_NUMS",
     "RAGGED_DOT_IMPLEMENTATIONS", "RaggedDotDimensionNumbers", "RaggedDotGroupSizes",
-    "TRANS_RHS_RAGGED_DOT_DIM_NUMS", "autotune", "config", "generate_group_sizes", "ragged_dot",
+    "TRANS_RHS_RAGGED_DOT_DIM_NUMS", "autotune", "config", "gated_linear_unit", "generate_group_sizes", "ragged_dot",
     "ragged_dot_general",
 ]

@@ -142,7 +142,7 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
                      (long long)n, (long long)num_groups);
   if (mode != TKX_MODE_DEFAULT && mode != TKX_MODE_TRANS_RHS) return set_error(TKX_ERR_INVALID, "bad mode %d", mode);
   if (!valid_out_dtype(out_dtype)) return set_error(TKX_ERR_UNSUPPORTED, "out dtype %d not supported", out_dtype);
-  if (activation < TKX_ACT_NONE || activation > TKX_ACT_GELU_TANH)
+  if (activation < TKX_ACT_NONE || activation > TKX_ACT_SIGMOID)
     return set_error(TKX_ERR_INVALID, "bad activation %d", activation);
   // Per-lane byte offsets inside a tile are 32-bit: (256 rows) x (row bytes) must stay below 2^31.
   if (m > 0x7fffffffLL / 2 || k >= (1 << 21) || n >= (1 << 21))
@@ -259,7 +259,6 @@ int32_t tkx_ragged_dot_fwd_fused(const void* lhs, const void* rhs, const int32_t
                                  const TkxConfig* config, tkx_stream_t stream) {
   if (gateup != 0 && gateup != 1) return set_error(TKX_ERR_INVALID, "gateup must be 0 or 1");
   if (rhs_scale_blocks < 1) return set_error(TKX_ERR_INVALID, "rhs_scale_blocks must be >= 1");
-  if (gateup && activation == TKX_ACT_NONE) return set_error(TKX_ERR_INVALID, "gate-up fusion needs an activation");
   return fwd_impl(lhs, rhs, group_sizes, lhs_scale, rhs_scale, rhs_bias, out, workspace, m, k, n, num_groups, lhs_dtype,
                   rhs_dtype, out_dtype, TKX_MODE_DEFAULT, activation, gateup == 1, rhs_scale_blocks, config, stream);
 }

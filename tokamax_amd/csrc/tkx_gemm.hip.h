@@ -376,6 +376,7 @@ __device__ __forceinline__ float apply_activation(float x, int act) {
     case TKX_ACT_RELU: return x > 0.f ? x : 0.f;
     case TKX_ACT_TANH: return tanhf(x);
     case TKX_ACT_SILU: return x / (1.f + __expf(-x));
+    case TKX_ACT_SIGMOID: return 1.f / (1.f + __expf(-x));
     case TKX_ACT_GELU_TANH: {
       const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
       return 0.5f * x * (1.f + tanhf(u));
@@ -789,6 +790,7 @@ struct GemmKernel {
         if (p.activation == TKX_ACT_RELU) for_all([](float x) { return x > 0.f ? x : 0.f; });
         else if (p.activation == TKX_ACT_TANH) for_all(fast_tanh);
         else if (p.activation == TKX_ACT_SILU) for_all([](float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-x)); });
+        else if (p.activation == TKX_ACT_SIGMOID) for_all([](float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); });
         else if (p.activation == TKX_ACT_GELU_TANH)
           for_all([&](float x) { return 0.5f * x * (1.f + fast_tanh(0.7978845608028654f * (x + 0.044715f * x * x * x))); });
       }

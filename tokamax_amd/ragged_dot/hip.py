@@ -66,6 +66,8 @@ _ACTIVATION_NAMES = {
     torch.tanh: "tanh",
     torch.nn.functional.tanh: "tanh",
     torch.nn.functional.silu: "silu",
+    torch.sigmoid: "sigmoid",
+    torch.nn.functional.sigmoid: "sigmoid",
 }
 
 

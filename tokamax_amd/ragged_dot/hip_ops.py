@@ -122,8 +122,8 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
     raise ValueError("contraction sizes of lhs and rhs differ")
   if (rhs_bias is not None or gateup) and trans_rhs:
     raise NotImplementedError("bias and gate-up fusion need the default dimension numbers")
-  if gateup and (activation is None or n % 2):
-    raise ValueError("gate-up fusion needs an activation and an even number of rhs columns")
+  if gateup and n % 2:
+    raise ValueError("gate-up fusion needs an even number of rhs columns")
   if lhs_scale is not None:
     lhs_scale = lhs_scale.to(torch.float32).contiguous().view(-1)
     if lhs_scale.numel() != m:
