@@ -150,6 +150,19 @@ int32_t tkx_dequantize_weights(const void* qvalue, const float* scale, void* out
                                int64_t n, int64_t scale_block_k, int32_t q_dtype, int32_t out_dtype,
                                tkx_stream_t stream);
 
+/* The token permute / un-permute steps either side of the ragged dot in an MoE layer, one kernel:
+ *   out[j, :] = sum over r < reduce_group_size of keep(g) * weights[g] * x[indices[g], :],  g = j * reduce_group_size + r
+ * keep(g) = (start == NULL or start[0] <= indices[g] < end[0]) and (valid == NULL or valid[g] != 0).
+ *   ragged_gather         (tokamax/_src/ops/ragged_gather/base.py:25-32): weights = valid = start = end = NULL, reduce 1
+ *   ragged_scatter        (ragged_scatter/base.py:26-38): start/end given (device int32 scalars), reduce 1
+ *   ragged_gather_reduce  (ragged_gather_reduce/base.py:26-40): weights f32[out_rows * reduce], valid bytes, reduce = R;
+ *                         products and sums in f32, one rounding to `dtype`
+ * x [in_rows, hidden], out [out_rows, hidden] of `dtype` (f32/bf16/f16), rows a multiple of 16 bytes;
+ * indices int32[out_rows * reduce_group_size] (clamped into [0, in_rows)). */
+int32_t tkx_ragged_gather_rows(const void* x, const int32_t* indices, const float* weights, const uint8_t* valid,
+                               const int32_t* start, const int32_t* end, void* out, int64_t in_rows, int64_t out_rows,
+                               int64_t hidden, int64_t reduce_group_size, int32_t dtype, tkx_stream_t stream);
+
 /* Enumerates compiled kernel variants, for the autotuner's search space.
  * kind: 0 = fwd/dlhs variants, 1 = drhs variants.  Returns the count; tkx_ragged_dot_variant fills
  * `config` (tile + wave fields), the dtype pair and the mode of variant `index` (0 = fwd, 1 = dlhs,

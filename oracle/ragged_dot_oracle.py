@@ -37,6 +37,9 @@ below therefore cites the reference call site it follows, and says what pins it:
   gated_linear_unit            gated_linear_unit/base.py:60-120                   torch matmul + torch activations on
                                                                                   f64 (library routines)
 
+  ragged_gather / _scatter /   ragged_gather/base.py:25-32, ragged_scatter/        NumPy fancy indexing (library
+    _gather_reduce             base.py:26-38, ragged_gather_reduce/base.py:26-40    routine) + loops on a tiny case
+
 Status of "parity unpinned": `qwix.quantize` (absmax calibration / rounding) is
 NOT restated -- quantised inputs are generated directly as (qvalue, scale) pairs.
 `ragged_dot_fused` follows the docstring's formulas only: the one reference
@@ -293,6 +296,26 @@ def gated_linear_unit(x, weights, activation=None):
   w = np.asarray(weights, np.float64)
   gate, up = x @ w[:, 0, :], x @ w[:, 1, :]
   return (gate if activation is None else activation(gate)) * up
+
+
+def ragged_gather(x, indices):
+  """`x[indices]` (ragged_gather/base.py:25-32)."""
+  return np.asarray(x)[np.asarray(indices)]
+
+
+def ragged_scatter(x, indices, start: int, end: int):
+  """`where(start <= indices < end, x[indices], 0)` (ragged_scatter/base.py:26-38)."""
+  idx = np.asarray(indices)
+  out = np.asarray(x)[np.clip(idx, 0, len(x) - 1)]
+  return np.where(((idx >= start) & (idx < end))[:, None], out, 0).astype(out.dtype)
+
+
+def ragged_gather_reduce(x, indices, topk_weights, valid_rows_mask, reduce_group_size: int):
+  """f32 `sum over groups of R rows of valid * weight * x[index]` (ragged_gather_reduce/base.py:26-40),
+  returned as float32 (the caller rounds to the input type)."""
+  out = np.asarray(x, np.float32)[np.asarray(indices)] * np.asarray(topk_weights, np.float32)[:, None]
+  out = np.where(np.asarray(valid_rows_mask, bool)[:, None], out, np.float32(0))
+  return out.reshape(-1, reduce_group_size, out.shape[-1]).sum(axis=1, dtype=np.float32)
 
 
 def ragged_dot_bruteforce(lhs, rhs, group_sizes, mode: str = DEFAULT):

@@ -569,6 +569,52 @@ def test_gated_linear_unit(shape, dtype, device):
     tokamax_amd.gated_linear_unit(x, w.float(), activation=F.silu)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_row_movement_ops(dtype, device):
+  """ragged_gather, ragged_scatter (bit-exact copies / zeros) and ragged_gather_reduce (f32 sums, one
+  rounding) against the oracle; the token permute -> ragged dot -> weighted un-permute round trip."""
+  rng = np.random.default_rng(21)
+  rows, hidden, n_out, R = 300, 264, 1040, 4
+  x = torch.tensor(rng.normal(0, 1, (rows, hidden)).astype(np.float32), device=device).to(dtype)
+  idx = torch.tensor(rng.integers(0, rows, n_out).astype(np.int32), device=device)
+  got = tokamax_amd.ragged_gather(x, idx, torch.tensor([0], device=device), torch.tensor([rows], device=device))
+  assert torch.equal(got, x[idx.long()])
+  start, end = 40, 211
+  got = tokamax_amd.ragged_scatter(x, idx, torch.tensor([start], device=device), torch.tensor(end, device=device))
+  want = O.ragged_scatter(_np(x), idx.cpu().numpy(), start, end)
+  assert np.array_equal(_np(got), want)
+  w = torch.tensor(rng.uniform(0, 1, n_out).astype(np.float32), device=device)
+  valid = torch.tensor(rng.integers(0, 4, n_out) > 0, device=device)
+  got = tokamax_amd.ragged_gather_reduce(x, idx, w, valid, R)
+  want = O.ragged_gather_reduce(_np(x), idx.cpu().numpy(), _np(w), valid.cpu().numpy(), R)
+  assert got.shape == (n_out // R, hidden) and got.dtype == dtype
+  _check(got, want, 1e-6 if dtype == torch.float32 else 3e-3)
+  got = tokamax_amd.ragged_gather_reduce(x, idx, w, valid, 13)  # more rows per output row than the kernel keeps in registers
+  _check(got, O.ragged_gather_reduce(_np(x), idx.cpu().numpy(), _np(w), valid.cpu().numpy(), 13),
+         1e-6 if dtype == torch.float32 else 3e-3)
+  if dtype == torch.float32:
+    return
+  # MoE round trip: sort tokens by expert, ragged dot, weighted top-2 combine
+  tokens, k, n, G = 64, 128, 256, 4
+  h = torch.tensor(rng.normal(0, 1, (tokens, k)).astype(np.float32), device=device).to(dtype)
+  wts = torch.tensor(rng.normal(0, k ** -0.5, (G, k, n)).astype(np.float32), device=device).to(dtype)
+  expert = torch.tensor(np.stack([rng.permutation(G)[:2] for _ in range(tokens)]).astype(np.int64), device=device)
+  flat = expert.reshape(-1)
+  order = torch.argsort(flat, stable=True)
+  gs = torch.bincount(flat, minlength=G).to(torch.int32)
+  permuted = tokamax_amd.ragged_gather(h, (order // 2).to(torch.int32), 0, tokens)
+  y = tokamax_amd.HipRaggedDot()(permuted, wts, group_sizes=gs)
+  gate = torch.tensor(rng.uniform(0, 1, tokens * 2).astype(np.float32), device=device)
+  inverse = torch.argsort(order).to(torch.int32)
+  combined = tokamax_amd.ragged_gather_reduce(y, inverse, gate, torch.ones(tokens * 2, dtype=torch.bool, device=device), 2)
+  want = np.zeros((tokens, n), np.float64)
+  hn, wn, gn, en = _np(h).astype(np.float64), _np(wts).astype(np.float64), _np(gate), expert.cpu().numpy()
+  for t in range(tokens):
+    for s in range(2):
+      want[t] += gn[2 * t + s] * (hn[t] @ wn[en[t, s]])
+  _check(combined, want, 6e-3)
+
+
 def test_hip_graph_replays_follow_new_inputs_and_group_sizes(device):
   """The entry points allocate nothing, synchronise nothing and schedule on the device, so a captured
   HIP graph stays valid when the contents of lhs, the weights and even group_sizes change between

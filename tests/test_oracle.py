@@ -206,6 +206,22 @@ def test_gated_linear_unit_matches_torch():
                              want.numpy().reshape(10, 4), rtol=1e-12, atol=1e-12)
 
 
+def test_row_movement_ops_against_loops():
+  rng = np.random.default_rng(9)
+  x = rng.normal(size=(6, 3)).astype(np.float32)
+  idx = np.array([5, 0, 0, 3, 2, 4, 1, 1], np.int32)
+  w = rng.normal(size=8).astype(np.float32)
+  valid = np.array([1, 0, 1, 1, 1, 1, 0, 1], bool)
+  assert np.array_equal(O.ragged_gather(x, idx), np.stack([x[i] for i in idx]))
+  want = np.stack([x[i] if 1 <= i < 4 else np.zeros(3, np.float32) for i in idx])
+  assert np.array_equal(O.ragged_scatter(x, idx, 1, 4), want)
+  want = np.zeros((4, 3), np.float32)
+  for g in range(8):
+    if valid[g]:
+      want[g // 2] += w[g] * x[idx[g]]
+  np.testing.assert_allclose(O.ragged_gather_reduce(x, idx, w, valid, 2), want, rtol=1e-6, atol=1e-7)
+
+
 def test_dequantize_is_tile_repeat():
   rng = np.random.default_rng(9)
   q = rng.integers(-127, 128, (2, 8, 6)).astype(np.int8)

@@ -11,6 +11,7 @@ from tokamax_amd.op import AUTO, BoundArguments, NullConfig, Op
 from tokamax_amd.quantization import AsQArray, QArray
 from tokamax_amd.gated_linear_unit.api import gated_linear_unit
 from tokamax_amd.gated_linear_unit.hip import HipGatedLinearUnit
+from tokamax_amd.ragged_gather import ragged_gather, ragged_gather_reduce, ragged_scatter
 from tokamax_amd.ragged_dot.api import IMPLEMENTATIONS as RAGGED_DOT_IMPLEMENTATIONS
 from tokamax_amd.ragged_dot.api import ragged_dot, ragged_dot_general
 from tokamax_amd.ragged_dot.base import (
@@ -30,5 +31,5 @@ __all__ = [
     "HipRaggedDotConfig", "NullConfig", "Op", "QArray", "RAGGED_CONTRACTING_DOT_DIM_NUMS",
     "RAGGED_DOT_IMPLEMENTATIONS", "RaggedDotDimensionNumbers", "RaggedDotGroupSizes",
     "TRANS_RHS_RAGGED_DOT_DIM_NUMS", "autotune", "config", "gated_linear_unit", "generate_group_sizes", "ragged_dot",
-    "ragged_dot_general",
+    "ragged_dot_general", "ragged_gather", "ragged_gather_reduce", "ragged_scatter",
 ]

@@ -30,6 +30,7 @@ EXPORTED_SYMBOLS = (
     "tkx_ragged_dot_fwd_fused",
     "tkx_ragged_dot_drhs",
     "tkx_dequantize_weights",
+    "tkx_ragged_gather_rows",
     "tkx_ragged_dot_num_variants",
     "tkx_ragged_dot_variant",
 )
@@ -80,6 +81,8 @@ def _declare(lib):
   lib.tkx_ragged_dot_drhs.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32, cfgp, vp]
   lib.tkx_dequantize_weights.restype = i32
   lib.tkx_dequantize_weights.argtypes = [vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
+  lib.tkx_ragged_gather_rows.restype = i32
+  lib.tkx_ragged_gather_rows.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]
   lib.tkx_ragged_dot_num_variants.restype = i32
   lib.tkx_ragged_dot_num_variants.argtypes = [i32]
   lib.tkx_ragged_dot_variant.restype = i32

@@ -334,6 +334,24 @@ int32_t tkx_dequantize_weights(const void* qvalue, const float* scale, void* out
   return launch_dequant_i8(qvalue, scale, out, num_groups, k, n, scale_block_k, static_cast<hipStream_t>(stream));
 }
 
+int32_t tkx_ragged_gather_rows(const void* x, const int32_t* indices, const float* weights, const uint8_t* valid,
+                               const int32_t* start, const int32_t* end, void* out, int64_t in_rows, int64_t out_rows,
+                               int64_t hidden, int64_t reduce_group_size, int32_t dtype, tkx_stream_t stream) {
+  if (!x || !indices || !out) return set_error(TKX_ERR_INVALID, "null pointer argument");
+  if (in_rows < 1 || out_rows < 0 || hidden < 1 || reduce_group_size < 1)
+    return set_error(TKX_ERR_INVALID, "bad sizes in_rows=%lld out_rows=%lld hidden=%lld reduce=%lld", (long long)in_rows,
+                     (long long)out_rows, (long long)hidden, (long long)reduce_group_size);
+  if ((start == nullptr) != (end == nullptr)) return set_error(TKX_ERR_INVALID, "start and end go together");
+  if (dtype != TKX_F32 && dtype != TKX_BF16 && dtype != TKX_F16)
+    return set_error(TKX_ERR_UNSUPPORTED, "dtype %d not supported", dtype);
+  const int64_t esz = dtype_bytes(dtype);
+  if ((hidden * esz) % 16 != 0 || ((uintptr_t)x | (uintptr_t)out) % 16 != 0)
+    return set_error(TKX_ERR_UNSUPPORTED, "rows must be a multiple of 16 bytes and 16-byte aligned");
+  if (hidden >= (1LL << 31) || reduce_group_size >= (1LL << 31)) return set_error(TKX_ERR_UNSUPPORTED, "dimension too large");
+  return launch_gather_rows(x, indices, weights, valid, start, end, out, in_rows, out_rows, hidden, reduce_group_size,
+                            dtype, static_cast<hipStream_t>(stream));
+}
+
 int32_t tkx_ragged_dot_num_variants(int32_t kind) {
   int32_t n = 0;
   for (const Variant& v : registry().all) n += ((v.mode == kDrhs) == (kind == 1));

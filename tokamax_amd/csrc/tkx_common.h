@@ -105,6 +105,11 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
 int32_t launch_dequant_i8(const void* q, const float* scale, void* out, int64_t G, int64_t k, int64_t n, int64_t t_k,
                           hipStream_t stream);
 
+// ---- row gather with optional mask, weight and reduction (token permute / un-permute) -------------
+int32_t launch_gather_rows(const void* x, const int32_t* indices, const float* weights, const unsigned char* valid,
+                           const int32_t* start, const int32_t* end, void* out, int64_t in_rows, int64_t out_rows,
+                           int64_t hidden, int64_t reduce, int32_t dtype, hipStream_t stream);
+
 // Each dtype family registers its variants from its own translation unit.
 const Variant* variants_bf16(int* count);
 const Variant* variants_f16(int* count);
