@@ -257,6 +257,42 @@ def test_config_resolution_order():
   assert ba.default_config == _FakeConfig(42)
 
 
+def test_config_memo_is_dropped_when_its_inputs_change():
+  """`default_config` of identical calls is answered from a per-op memo; a new shape, a config option, an
+  overlay or newly cached autotuning data each lead to a fresh resolution."""
+  calls = []
+
+  class _Counting(_FakeOp):
+    def _get_heuristics_config(self, ba):
+      calls.append(1)
+      return _FakeConfig(42)
+
+  op = _Counting()
+  x, y = torch.zeros(3), torch.zeros(4)
+  assert op.bind(x, x).default_config == _FakeConfig(42) and len(calls) == 1
+  assert op.bind(torch.ones(3), torch.ones(3)).default_config == _FakeConfig(42) and len(calls) == 1  # same shapes: memo
+  assert op.bind(y, y).default_config == _FakeConfig(42) and len(calls) == 2                          # new shape
+  ba = op.bind(x, x)
+  data = autotuner_lib.AutotuningData({_FakeConfig(1): _bench(3.0), _FakeConfig(2): _bench(1.0)})
+  with tokamax_amd.AutotuningResult(op_lib.device_kind(), ((ba, data),)):
+    assert op.bind(x, x).default_config == _FakeConfig(2)
+    with config_lib.ignore_autotuning_cache(True):
+      assert op.bind(x, x).default_config == _FakeConfig(42)
+  assert op.bind(x, x).default_config == _FakeConfig(42)
+  with config_lib.autotuning_cache_miss_fallback("error"):
+    with pytest.raises(ValueError, match="No config found"):
+      _ = op.bind(x, x).default_config
+  # data written to the op's cache (what `autotune(cache_results=True)` does) is seen by the next call
+  op.get_autotuning_cache()[ba.autotuning_cache_key] = data
+  op_lib.bump_config_epoch()
+  try:
+    assert op.bind(x, x).default_config == _FakeConfig(2)
+  finally:
+    del op.get_autotuning_cache()[ba.autotuning_cache_key]
+    op_lib.bump_config_epoch()
+  assert op.bind(x, x).default_config == _FakeConfig(42)
+
+
 def test_autotuner_records_failures_and_picks_fastest():
   x = torch.zeros(3)
   ba = _FakeOp().bind(x, x)

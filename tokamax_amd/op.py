@@ -57,7 +57,13 @@ def device_kind(device=None) -> DeviceKind:
   """The key autotuning caches are filed under (the role of `jax.Device.device_kind`)."""
   if not torch.cuda.is_available():
     return "cpu"
-  props = torch.cuda.get_device_properties(device)
+  index = device.index if isinstance(device, torch.device) else device
+  return _device_kind_of(torch.cuda.current_device() if index is None else int(index))
+
+
+@functools.lru_cache(maxsize=None)
+def _device_kind_of(index: int) -> DeviceKind:
+  props = torch.cuda.get_device_properties(index)
   arch = getattr(props, "gcnArchName", "").split(":")[0]
   if arch in _ARCH_DEVICE_KINDS:
     return _ARCH_DEVICE_KINDS[arch]
@@ -177,6 +183,41 @@ class CacheKey(tuple):
 
 
 _AUTOTUNING_CACHE: dict = {}
+
+# Config memo. Resolving a config walks the overlay stack and the JSON cache with a key built from
+# every argument; an eager caller repeats that for identical shapes on every call. The result is
+# kept per op instance under a cheap structural signature of the arguments plus everything else the
+# answer depends on: this counter (bumped whenever cached autotuning data changes), the two config
+# options, and the identity of the overlay stack.
+_CONFIG_EPOCH = [0]
+
+
+def bump_config_epoch() -> None:
+  _CONFIG_EPOCH[0] += 1
+
+
+class _Unhashable(Exception):
+  pass
+
+
+def _fast_signature(v):
+  """A cheap hashable stand-in for one argument: shapes, dtypes and devices of arrays, values of the rest."""
+  if isinstance(v, torch.Tensor):
+    return (v.shape, v.dtype, v.device)
+  if v is None or isinstance(v, (bool, int, float, str, torch.dtype)):
+    return v
+  sig = getattr(v, "_fast_signature", None)
+  if sig is not None:
+    return sig()
+  if isinstance(v, (tuple, list)):
+    return tuple(_fast_signature(x) for x in v)
+  if callable(v) and not dataclasses.is_dataclass(v):
+    return ("callable", id(v))
+  try:
+    hash(v)
+  except TypeError:
+    raise _Unhashable from None
+  return v
 # Stack of {op: {device_kind: {key: AutotuningData}}} overlays pushed by `AutotuningResult`.
 AUTOTUNING_CACHE_OVERLAY_STACK: contextvars.ContextVar[tuple] = contextvars.ContextVar(
     "AUTOTUNING_CACHE_OVERLAY_STACK", default=()
@@ -225,10 +266,28 @@ class BoundArguments:
   def default_config(self):
     """`op.config`, else cache, else autotune / heuristics / error by the cache-miss option."""
     fallback = config_lib.autotuning_cache_miss_fallback.value
-    return self.get_config(
+    memo_key = None
+    if fallback != "autotune":  # (autotuning has side effects: never answered from the memo)
+      try:
+        memo_key = (tuple((k, _fast_signature(v)) for k, v in self.arguments.items()), _CONFIG_EPOCH[0], fallback,
+                    config_lib.ignore_autotuning_cache.value, id(AUTOTUNING_CACHE_OVERLAY_STACK.get()))
+      except _Unhashable:
+        memo_key = None
+    memo = self.op.__dict__.get("_config_memo")
+    if memo_key is not None and memo is not None and memo_key in memo:
+      return memo[memo_key]
+    config = self.get_config(
         autotune_configs=AUTO if fallback == "autotune" else None,
         allow_heuristics=fallback != "error",
     )
+    if memo_key is not None:
+      if memo is None or len(memo) > 256:
+        memo = {}
+        object.__setattr__(self.op, "_config_memo", memo)
+      # The overlay stack tuple is kept alive with the entry, so its id cannot be reused meanwhile.
+      memo[memo_key] = config
+      memo.setdefault("_keepalive", []).append(AUTOTUNING_CACHE_OVERLAY_STACK.get())
+    return config
 
   def get_config(self, check_autotuning_cache: bool = True, autotune_configs=None,
                  cache_autotuning_results: bool = True, allow_heuristics: bool = True):
@@ -287,6 +346,7 @@ class BoundArguments:
     data = autotuner.autotune(op_fn, configs, *self.args, timeout=timeout, **self.kwargs)
     if cache_results:
       self.op.get_autotuning_cache()[self.autotuning_cache_key] = data
+      bump_config_epoch()
     return data
 
   def to_json_dict(self) -> dict:

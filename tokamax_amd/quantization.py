@@ -27,6 +27,11 @@ class QArray:
     if self.qtype is None:
       object.__setattr__(self, "qtype", self.qvalue.dtype)
 
+  def _fast_signature(self):
+    """Structural stand-in used by the op's config memo (shapes, dtypes, devices)."""
+    sig = lambda t: None if t is None else (tuple(t.shape), t.dtype, getattr(t, "device", None))
+    return ("QArray", sig(self.qvalue), sig(self.scale), sig(self.zero_point), self.qtype)
+
   shape = property(lambda self: tuple(self.qvalue.shape))
   dtype = property(lambda self: self.scale.dtype)  # the dtype it dequantises to
   ndim = property(lambda self: len(self.qvalue.shape))

@@ -5,8 +5,10 @@ PyTorch is used for device memory and streams only; all arithmetic happens in th
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import dataclasses
+import functools
 
 import torch
 
@@ -44,8 +46,29 @@ class KernelConfig:
   align_tile: int = 8
 
   def to_c(self) -> _lib.TkxConfig:
-    return _lib.TkxConfig(self.block_m, self.block_n, self.block_k, self.waves_m, self.waves_n,
-                          self.grid_tile_width, self.align_tile, self.num_stages)
+    return _config_struct(self)
+
+
+@functools.lru_cache(maxsize=256)
+def _config_struct(c: "KernelConfig") -> _lib.TkxConfig:
+  """The C struct of a config (built once per distinct config; the library only reads it)."""
+  return _lib.TkxConfig(c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.grid_tile_width, c.align_tile,
+                        c.num_stages)
+
+
+@functools.lru_cache(maxsize=1024)
+def _workspace_words(m: int, num_groups: int, block_m: int) -> int:
+  nbytes = _lib.load().tkx_ragged_dot_workspace_bytes(m, num_groups, block_m)
+  if nbytes < 0:
+    raise ValueError(f"bad sizes m={m} G={num_groups} block_m={block_m}")
+  return nbytes // 4
+
+
+def _on_device(device):
+  """Context that makes `device` current for the launch; free when it already is."""
+  if device.index is None or torch.cuda.current_device() == device.index:
+    return contextlib.nullcontext()
+  return torch.cuda.device(device)
 
 
 def _require_cuda(*tensors):
@@ -69,10 +92,7 @@ def _group_sizes_i32(group_sizes: torch.Tensor) -> torch.Tensor:
 
 
 def workspace(m: int, num_groups: int, block_m: int, device) -> torch.Tensor:
-  nbytes = _lib.load().tkx_ragged_dot_workspace_bytes(m, num_groups, block_m)
-  if nbytes < 0:
-    raise ValueError(f"bad sizes m={m} G={num_groups} block_m={block_m}")
-  return torch.empty(nbytes // 4, dtype=torch.int32, device=device)
+  return torch.empty(_workspace_words(m, num_groups, block_m), dtype=torch.int32, device=device)
 
 
 def schedule(group_sizes: torch.Tensor, m: int, block_m: int, align_tile: int = 8):
@@ -143,7 +163,7 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
   out = torch.empty((m, out_cols), dtype=out_dtype, device=lhs.device)
   ws = workspace(m, G, config.block_m, lhs.device)
   cfg = config.to_c()
-  with torch.cuda.device(lhs.device):
+  with _on_device(lhs.device):
     if rhs_bias is None and not gateup and scale_blocks == 1:
       st = lib.tkx_ragged_dot_fwd(
           _ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(out), _ptr(ws), m, k, n, G,
@@ -173,7 +193,7 @@ def dequantize_weights(qvalue: torch.Tensor, scale: torch.Tensor) -> torch.Tenso
   qvalue = qvalue.contiguous()
   scale = scale.to(torch.float32).contiguous()
   out = torch.empty((G, k, n), dtype=torch.bfloat16, device=qvalue.device)
-  with torch.cuda.device(qvalue.device):
+  with _on_device(qvalue.device):
     st = lib.tkx_dequantize_weights(_ptr(qvalue), _ptr(scale), _ptr(out), G, k, n, k // scale.shape[1],
                                     _lib.TKX_I8, _lib.TKX_BF16, _stream(qvalue.device))
   _lib.check(st)
@@ -198,7 +218,7 @@ def ragged_dot_drhs(lhs, dout, group_sizes, num_groups: int, *, config: KernelCo
   out = torch.empty((num_groups, k, n), dtype=out_dtype, device=lhs.device)
   ws = workspace(m, num_groups, 128, lhs.device)
   cfg = config.to_c()
-  with torch.cuda.device(lhs.device):
+  with _on_device(lhs.device):
     st = lib.tkx_ragged_dot_drhs(_ptr(lhs), _ptr(dout), _ptr(gs), _ptr(out), _ptr(ws), m, k, n, num_groups,
                                  dtype_code(lhs.dtype), dtype_code(out_dtype), ctypes.byref(cfg), _stream(lhs.device))
   _lib.check(st)
