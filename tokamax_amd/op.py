@@ -248,7 +248,10 @@ class BoundArguments:
   @functools.cached_property
   def tensors(self) -> tuple:
     """Every tensor among the arguments (inside containers and quantised arrays too)."""
-    return tuple(x for x in _leaves(dict(self.arguments)) if isinstance(x, torch.Tensor))
+    out: list = []
+    for v in self.arguments.values():
+      _collect_tensors(v, out)
+    return tuple(out)
 
   @functools.cached_property
   def _bound_args(self) -> inspect.BoundArguments:
@@ -362,22 +365,27 @@ class BoundArguments:
     return dataclasses.replace(self, **kwargs)
 
 
-def _leaves(x):
-  if isinstance(x, torch.Tensor) or x is None or isinstance(x, (str, int, float, bool)):
-    yield x
+_SCALARS = (str, int, float, bool, torch.dtype)
+
+
+def _collect_tensors(x, out: list) -> None:
+  """Appends every tensor inside `x` to `out` (through containers, dataclasses and objects with a `_leaves()` method; common cases first)."""
+  if isinstance(x, torch.Tensor):
+    out.append(x)
+  elif x is None or isinstance(x, _SCALARS):
+    return
   elif isinstance(x, dict):
     for v in x.values():
-      yield from _leaves(v)
+      _collect_tensors(v, out)
   elif isinstance(x, (tuple, list)):
     for v in x:
-      yield from _leaves(v)
+      _collect_tensors(v, out)
+  elif hasattr(x, "_leaves"):
+    for v in x._leaves():  # pylint: disable=protected-access
+      _collect_tensors(v, out)
   elif dataclasses.is_dataclass(x) and not isinstance(x, type):
     for f in dataclasses.fields(x):
-      yield from _leaves(getattr(x, f.name))
-  elif hasattr(x, "_leaves"):
-    yield from x._leaves()  # pylint: disable=protected-access
-  else:
-    yield x
+      _collect_tensors(getattr(x, f.name), out)
 
 
 def infer_devices(ba: BoundArguments) -> set:
