@@ -9,13 +9,15 @@
 //   mode kDrhs : A = lhs  [m,k]  row(k-index)-contiguous  B = dout [m,n]    column-contiguous
 //                (C[g][k,n] = lhs[rows_g]^T . dout[rows_g]; contraction = the group's row range)
 //
-// A workgroup owns one BM x BN tile of C. k-steps of BK contraction elements are staged through
-// two LDS buffers with direct-to-LDS loads (global_load_lds_dwordx4): the next step's loads are in
-// flight during the MFMAs of the current one, and fragments are double-buffered in registers. Operands that are contraction-contiguous are read from LDS with
-// ds_read_b128; operands that are contiguous along the other axis are read with the gfx950
-// transposing LDS loads (ds_read_b64_tr_b16 / _tr_b8), so no operand is ever transposed in memory.
-// The 32x32 MFMA is issued with its operands swapped (B-fragment first) so that each lane ends up
-// holding runs of 4 consecutive C columns of one C row: the epilogue stores 8/16-byte vectors.
+// A workgroup owns one BM x BN tile of C. k-steps of BK contraction elements are staged through a
+// ring of NS LDS stages with direct-to-LDS loads (global_load_lds_dwordx4), all stages in flight: a
+// stage is refilled right after the barrier that releases it, between the MFMAs of the step's last
+// k-atom, and fragments are double-buffered in registers. Operands that are contraction-contiguous
+// are read from LDS with ds_read_b128; operands that are contiguous along the other axis are read
+// with the gfx950 transposing LDS loads (ds_read_b64_tr_b16 / _tr_b8), so no operand is ever
+// transposed in memory. The 32x32 MFMA is issued with its operands swapped (B-fragment first) so
+// that each lane ends up holding runs of 4 consecutive C columns of one C row; the epilogue applies
+// scales, bias and activation in registers and writes whole row segments through LDS.
 #pragma once
 
 #include <type_traits>
