@@ -379,14 +379,15 @@ def test_every_kernel_variant_through_c_abi(v, device):
   assert torch.count_nonzero(out[int(gs.sum()):]) == 0
 
 
-@pytest.mark.parametrize("depth", [2, 4, 8])
+@pytest.mark.parametrize("block_n,depth", [(128, 2), (128, 4), (128, 8), (256, 2), (256, 4)])
 @pytest.mark.parametrize("case", ["ragged", "two_chunks", "all_empty", "one_big_group", "first_and_last_empty",
                                   "many_groups"])
-def test_small_m_int8_kernel_edges(case, depth, device):
-  """The streaming small-m kernel: empty groups anywhere, more than 64 groups, groups taller than one
-  16-row pass, a column count that is not a multiple of its 128-column tile, and a zero tail."""
+def test_small_m_int8_kernel_edges(case, block_n, depth, device):
+  """The streaming small-m kernel (128 columns per workgroup, and the wide one with 256): empty groups
+  anywhere, more than 64 groups, groups taller than one 16-row pass, a column count that is not a
+  multiple of its column tile, and a zero tail."""
   rng = np.random.default_rng(len(case) + depth)
-  k, n = 1024, 208
+  k, n = 1024, 208 if block_n == 128 else 464  # one partial tile; a whole and a partial tile
   if case == "ragged":
     gs = np.array([3, 0, 0, 17, 1, 0, 16, 2], np.int32)
   elif case == "two_chunks":
@@ -404,7 +405,7 @@ def test_small_m_int8_kernel_edges(case, depth, device):
   lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
   rhs = torch.tensor(rng.integers(-128, 128, (G, k, n)).astype(np.int8), device=device)
   scale = torch.tensor((np.abs(rng.normal(0, 0.01, (G, 1, n))) + 1e-3).astype(np.float32), device=device)
-  cfg = hip_ops.KernelConfig(16, 128, 32, 1, 4, depth)
+  cfg = hip_ops.KernelConfig(16, block_n, 32, 1, 4, depth)
   out = hip_ops.ragged_dot_fwd(lhs, rhs, torch.tensor(gs, device=device), config=cfg, out_dtype=torch.float32,
                                rhs_scale=scale)
   want = O.ragged_dot(_np(lhs), O.dequantize(rhs.cpu().numpy(), _np(scale)), gs, O.DEFAULT, acc_dtype=np.float64,
@@ -417,6 +418,33 @@ def test_small_m_int8_kernel_edges(case, depth, device):
   assert torch.equal(out16, out.to(torch.bfloat16))
   assert torch.equal(out, hip_ops.ragged_dot_fwd(lhs, rhs, torch.tensor(gs, device=device), config=cfg,
                                                  out_dtype=torch.float32, rhs_scale=scale))
+
+
+def test_public_op_picks_the_wide_small_m_kernel_when_it_fills_the_chip(device):
+  """64 groups x 2048 columns = 512 workgroups of 256 columns (two per CU): the heuristics name the wide
+  streaming kernel, and the public entry's result on it matches the oracle."""
+  rng = np.random.default_rng(5)
+  G, k, n = 64, 1024, 2048
+  gs = rng.integers(0, 5, G).astype(np.int32)
+  m = int(gs.sum()) + 3
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  q = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+  scale = torch.tensor((rng.uniform(0.5, 1.5, (G, 1, n)) / 127 * 0.1).astype(np.float32), device=device)
+  rhs = tokamax_amd.QArray(q, scale)
+  gst = torch.tensor(gs, device=device)
+  op = tokamax_amd.HipRaggedDot()
+  cfg = op._get_heuristics_config(op.bind(lhs, rhs, group_sizes=gst))
+  assert (cfg.block_m, cfg.block_n) == (16, 256)
+  out = op(lhs, rhs, group_sizes=gst, preferred_element_type=torch.float32)
+  want = np.zeros((m, n))
+  start = 0
+  for g in range(G):  # group by group: the widened weights of all groups at once would take 1 GB
+    w = O.dequantize(q[g:g + 1].cpu().numpy(), _np(scale[g:g + 1]))
+    rows = slice(start, start + int(gs[g]))
+    want[rows] = O.ragged_dot(_np(lhs[rows]), w, gs[g:g + 1], O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+    start += int(gs[g])
+  _check(out, want, 1e-5)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
 
 
 @pytest.mark.parametrize("depth", [2, 4])

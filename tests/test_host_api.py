@@ -431,6 +431,10 @@ def test_hip_config_validation_and_heuristics():
   q = tokamax_amd.QArray(ShapeDtype((128, 2048, 768), torch.int8), ShapeDtype((128, 1, 768), torch.float32))
   ba = op.bind(ShapeDtype((256, 2048), torch.bfloat16), q, group_sizes=base.GroupSizes(ShapeDtype((128,), torch.int32), 256))
   assert ba.heuristics_config.block_m == 16  # the streaming small-m kernel
+  assert ba.heuristics_config.block_n == 128  # 128 x 3 wide workgroups would fill 256 CUs unevenly
+  q = tokamax_amd.QArray(ShapeDtype((128, 2048, 1024), torch.int8), ShapeDtype((128, 1, 1024), torch.float32))
+  ba = op.bind(ShapeDtype((256, 2048), torch.bfloat16), q, group_sizes=base.GroupSizes(ShapeDtype((128,), torch.int32), 256))
+  assert (ba.heuristics_config.block_m, ba.heuristics_config.block_n) == (16, 256)  # 512 wide workgroups: two per CU
   with pytest.raises(NotImplementedError):
     _ = op.bind(ShapeDtype((256, 2048), torch.float64), ShapeDtype((8, 2048, 768), torch.float64),
                 group_sizes=base.GroupSizes(ShapeDtype((8,), torch.int32), 256)).heuristics_config

@@ -34,6 +34,8 @@ struct Registry {
     // (fn == nullptr, num_stages = steps of loads in flight) so that configs can name it.
     for (int depth : {2, 4, 8})
       all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
+    for (int depth : {2, 4})
+      all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeWideBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
     for (int dtype : {TKX_BF16, TKX_F16})
       for (int depth : {2, 4})
         all.push_back({kFwd, dtype, dtype, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
@@ -181,13 +183,13 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
     if (rhs_bias != nullptr || gateup) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no bias or gate-up fusion");
     if (rhs_scale != nullptr && rhs_dtype != TKX_I8)
       return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes an rhs scale with int8 weights only");
-    if (!decode_supported(lhs_dtype, rhs_dtype, m, k, n, num_groups, rhs_scale ? rhs_scale_blocks : 1))
+    if (!decode_supported(lhs_dtype, rhs_dtype, m, k, n, num_groups, rhs_scale ? rhs_scale_blocks : 1, c.block_n))
       return set_error(TKX_ERR_UNSUPPORTED,
-                       "decode kernel needs k %% 1024 == 0, n %% 8 == 0 and scale blocks of a power-of-two multiple of 32"
-                       " rows (k=%lld n=%lld G=%lld scale blocks=%lld)",
+                       "decode kernel needs k %% 1024 == 0, n %% 8 == 0 (n %% 16 == 0 and one scale block at block_n 256)"
+                       " and scale blocks of a power-of-two multiple of 32 rows (k=%lld n=%lld G=%lld scale blocks=%lld)",
                        (long long)k, (long long)n, (long long)num_groups, (long long)rhs_scale_blocks);
     return launch_decode(lhs, rhs, rhs_scale, group_sizes, out, m, k, n, num_groups, rhs_dtype, out_dtype, activation,
-                         c.num_stages, rhs_scale ? rhs_scale_blocks : 1, stream);
+                         c.num_stages, rhs_scale ? rhs_scale_blocks : 1, c.block_n, stream);
   }
   if (rhs_scale && rhs_scale_blocks != 1)
     return set_error(TKX_ERR_UNSUPPORTED,

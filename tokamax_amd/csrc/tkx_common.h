@@ -94,12 +94,14 @@ struct Variant {
 
 // ---- decode (small-m streaming kernel; int8 or 16-bit weights) -----------------------------------
 constexpr int32_t kDecodeBlockM = 16, kDecodeBlockN = 128, kDecodeBlockK = 32, kDecodeWaves = 4, kDecodeStages = 4;
+constexpr int32_t kDecodeWideBlockN = 256;  // int8 weights with per-column scales only
 // `scale_blocks`: the scale is [G, scale_blocks, n]; 1 = one scale per (group, column).
+// `block_n`: output columns per workgroup, kDecodeBlockN or kDecodeWideBlockN.
 bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k, int64_t n, int64_t G,
-                      int64_t scale_blocks);
+                      int64_t scale_blocks, int32_t block_n);
 int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
                       int64_t m, int64_t k, int64_t n, int64_t G, int32_t rhs_dtype, int32_t out_dtype,
-                      int32_t activation, int32_t depth, int64_t scale_blocks, hipStream_t stream);
+                      int32_t activation, int32_t depth, int64_t scale_blocks, int32_t block_n, hipStream_t stream);
 
 // ---- dequantisation of int8 weights with sub-channel scales to bf16 ------------------------------
 int32_t launch_dequant_i8(const void* q, const float* scale, void* out, int64_t G, int64_t k, int64_t n, int64_t t_k,

@@ -14,17 +14,22 @@
 //     feeds MFMA j (j = 0..7) with byte j of those 8 loads, i.e. 8 contraction values of column
 //     8i+j.  MFMA j therefore produces the output columns {8i+j}; the lhs fragment of lane (r, q) is
 //     lhs[r][8q..8q+7] of the same step, one 16-byte load. (16-bit weights: 16 bytes per row and the
-//     j-th half-word of each, otherwise the same);
+//     j-th half-word of each, otherwise the same; int8 weights also come with 16 columns per lane,
+//     256 per workgroup: 16-byte loads and 16 MFMAs per step);
 //   * int8 is widened to bf16 exactly and goes through the 16x16x32 bf16 MFMA with f32 accumulation;
 //   * the four partial tiles are added in a fixed order through LDS (deterministic), scaled per
 //     (group, column), and rows past the group's end are never written.
 #include "tkx_common.h"
 #include "tkx_gemm.hip.h"
 
+#include <mutex>
+#include <utility>
+#include <vector>
+
 namespace tkx {
 namespace {
 
-constexpr int kDecBN = 128;    // output columns per workgroup
+constexpr int kDecBN = 128;    // output columns per workgroup (256 for the wide int8 kernel)
 constexpr int kDecWaves = 4;   // waves per workgroup; each takes k / 4 of the contraction
 constexpr int kDecKS = 32;     // contraction elements per step (one 16x16x32 MFMA deep)
 constexpr int kDecRows = 16;   // lhs rows per pass
@@ -62,12 +67,13 @@ __device__ __forceinline__ i32x4 buffer_load_16_streaming(__amdgpu_buffer_rsrc_t
   return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_offset, (int)uniform_offset, kStreamingLoad));
 }
 
-// What a lane holds of one weight row of a step: its 8 columns.
-template <int EW> struct WeightRow { typedef i32x4 T; static constexpr int ESZ = 2; };
-template <> struct WeightRow<kEI8> { typedef i32x2 T; static constexpr int ESZ = 1; };
-template <int EW>
-__device__ __forceinline__ typename WeightRow<EW>::T load_weight_row(__amdgpu_buffer_rsrc_t r, uint32_t lane_offset, uint32_t uniform_offset) {
-  if constexpr (EW == kEI8) return buffer_load_8(r, lane_offset, uniform_offset);
+// What a lane holds of one weight row of a step: its CPL columns (8, or 16 of int8).
+template <int EW, int CPL> struct WeightRow { typedef i32x4 T; static constexpr int ESZ = 2; };
+template <> struct WeightRow<kEI8, 8> { typedef i32x2 T; static constexpr int ESZ = 1; };
+template <> struct WeightRow<kEI8, 16> { typedef i32x4 T; static constexpr int ESZ = 1; };
+template <int EW, int CPL>
+__device__ __forceinline__ typename WeightRow<EW, CPL>::T load_weight_row(__amdgpu_buffer_rsrc_t r, uint32_t lane_offset, uint32_t uniform_offset) {
+  if constexpr (EW == kEI8 && CPL == 8) return buffer_load_8(r, lane_offset, uniform_offset);
   else return buffer_load_16_streaming(r, lane_offset, uniform_offset);
 }
 
@@ -82,10 +88,10 @@ __device__ __forceinline__ unsigned i8_to_f32_bits(int w) {
   return f;
 }
 
-// Byte J of each of 8 loaded 8-byte rows -> bf16 x8 (exact: |v| <= 128 fits the significand). The
-// upper halves of two f32 are the two bf16, packed with one byte permute.
-template <int J>
-__device__ __forceinline__ i32x4 column_fragment(const i32x2 (&rows)[8]) {
+// Byte J of each of 8 loaded 8- or 16-byte rows -> bf16 x8 (exact: |v| <= 128 fits the significand).
+// The upper halves of two f32 are the two bf16, packed with one byte permute.
+template <int J, typename Row>
+__device__ __forceinline__ i32x4 column_fragment_i8(const Row (&rows)[8]) {
   i32x4 out;
 #pragma unroll
   for (int h = 0; h < 4; ++h) {
@@ -108,7 +114,7 @@ __device__ __forceinline__ i32x4 column_fragment_scaled(const i32x2 (&rows)[8], 
 }
 // 16-bit weights: half-word J of each of 8 loaded 16-byte rows, two rows per byte permute.
 template <int J>
-__device__ __forceinline__ i32x4 column_fragment(const i32x4 (&rows)[8]) {
+__device__ __forceinline__ i32x4 column_fragment_16bit(const i32x4 (&rows)[8]) {
   i32x4 out;
 #pragma unroll
   for (int h = 0; h < 4; ++h)
@@ -130,17 +136,21 @@ __device__ __forceinline__ f32x4_t mma_16x16x32(i32x4 w, i32x4 a, f32x4_t acc) {
 // lane's columns for its k-block alongside the weights (the same unconditional pipeline; they come
 // from L2, a scale row serves all the weight rows of its block) and the weights are scaled while
 // they are widened, instead of one multiply per output in the epilogue.
-template <int EW, int kDecDepth, int kMinWgs, bool SUB = false>
+// CPL = columns per lane; a workgroup covers BN = 16 CPL columns. 16 (int8 only) makes the loads 16
+// bytes per lane and the rows a wave reads 256 bytes long, the shape 16-bit weights have at CPL 8.
+template <int EW, int kDecDepth, int kMinWgs, bool SUB = false, int CPL = 8>
 __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const DecodeParams p) {
   static_assert(!SUB || EW == kEI8, "sub-channel scales belong to int8 weights");
+  static_assert(CPL == 8 || (CPL == 16 && EW == kEI8 && !SUB), "16 columns per lane: int8 weights with per-column scales");
   constexpr int EA = EW == kEI8 ? kEBF16 : EW;
-  constexpr int WESZ = WeightRow<EW>::ESZ;
-  typedef typename WeightRow<EW>::T WRow;
+  constexpr int WESZ = WeightRow<EW, CPL>::ESZ;
+  constexpr int BN = 16 * CPL;
+  typedef typename WeightRow<EW, CPL>::T WRow;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   __shared__ int s_red[kDecWaves];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = blockIdx.x / p.n_tiles, nt = blockIdx.x - g * p.n_tiles;
-  const int col0 = nt * kDecBN;
+  const int col0 = nt * BN;
   const bool last_group = g == p.num_groups - 1;
 
   // Sizes of the groups before this one (for its first row) and its own size are requested first
@@ -154,11 +164,11 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
   const int k_begin = wave * kw;
   const int steps = kw / kDecKS;       // multiple of kDecDepth (checked on the host)
   const unsigned char* wbase = p.rhs + ((int64_t)g * p.k + k_begin) * p.n * WESZ;
-  // B loads: lane (i = lane % 16, q = lane / 16) -> rows 8q + e (e = 0..7), columns col0 + 8i .. 8i+7,
-  // clamped at the last 8 columns (n is a multiple of 8; clamped lanes feed columns that are never stored).
+  // B loads: lane (i = lane % 16, q = lane / 16) -> rows 8q + e (e = 0..7), columns col0 + CPL i .. + CPL - 1,
+  // clamped at the last CPL columns (n is a multiple of CPL; clamped lanes feed columns that are never stored).
   const int li = lane & 15, lq = lane >> 4;
-  int colb = col0 + li * 8;
-  colb = colb < p.n - 8 ? colb : p.n - 8;
+  int colb = col0 + li * CPL;
+  colb = colb < p.n - CPL ? colb : p.n - CPL;
   uint32_t boff[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) boff[e] = (uint32_t)((8 * lq + e) * p.n + colb) * WESZ;
@@ -176,7 +186,7 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
   auto issue_b = [&](int slot, int step) {
     const uint32_t so = (uint32_t)__builtin_amdgcn_readfirstlane((int)(step * step_bytes));
 #pragma unroll
-    for (int e = 0; e < 8; ++e) breg[slot][e] = load_weight_row<EW>(wbuf, boff[e], so);
+    for (int e = 0; e < 8; ++e) breg[slot][e] = load_weight_row<EW, CPL>(wbuf, boff[e], so);
     if constexpr (SUB) {
       // (Past the wave's slice the block index runs past the buffer and the loads return zero.)
       const uint32_t kb = (uint32_t)(k_begin + step * kDecKS) >> p.log2_block_rows;
@@ -191,15 +201,17 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
     __builtin_amdgcn_sched_barrier(0);
   }
 
-  // Per-column scales of this thread's 8 epilogue columns, fetched now so that the epilogue does
+  // Per-column scales of this thread's CPL epilogue columns, fetched now so that the epilogue does
   // not end on a dependent memory round trip.
-  f32x4_t scale_lo = {1.f, 1.f, 1.f, 1.f}, scale_hi = {1.f, 1.f, 1.f, 1.f};
+  f32x4_t col_scales[CPL / 4];
+#pragma unroll
+  for (int t = 0; t < CPL / 4; ++t) col_scales[t] = (f32x4_t){1.f, 1.f, 1.f, 1.f};
   {
-    const int col = col0 + (tid & 15) * 8;
-    if (!SUB && p.scale != nullptr && col + 8 <= p.n) {
+    const int col = col0 + (tid & 15) * CPL;
+    if (!SUB && p.scale != nullptr && col + CPL <= p.n) {
       const float* sc = p.scale + (int64_t)g * p.n + col;
-      scale_lo = *reinterpret_cast<const f32x4_t*>(sc);
-      scale_hi = *reinterpret_cast<const f32x4_t*>(sc + 4);
+#pragma unroll
+      for (int t = 0; t < CPL / 4; ++t) col_scales[t] = *reinterpret_cast<const f32x4_t*>(sc + 4 * t);
     }
   }
 
@@ -221,7 +233,7 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
 
   if (last_group) {
     // Rows past the last group belong to no group: zero this workgroup's columns of them.
-    const int ncol = min(kDecBN, p.n - col0);
+    const int ncol = min(BN, p.n - col0);
     const int pieces = ncol * esz / 16;  // 16-byte pieces per row
     unsigned char* c = reinterpret_cast<unsigned char*>(p.out);
     const i32x4 z = {0, 0, 0, 0};
@@ -240,9 +252,9 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
     const uint32_t aoff = (uint32_t)((rb + li - start) * p.k + k_begin + 8 * lq) * 2u;
     auto issue_a = [&](int slot, int step) { areg[slot] = buffer_load_16(abuf, aoff, (uint32_t)(step * (kDecKS * 2))); };
 
-    f32x4_t acc[8];
+    f32x4_t acc[CPL];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < CPL; ++j) acc[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll
     for (int d = 0; d < kDecDepth; ++d) {
@@ -260,9 +272,8 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
       for (int d = 0; d < kDecDepth; ++d) {
         const int s = s0 + d;
         const i32x4 afrag = areg[d];
-        // MFMA j contracts this step's 32 rows for the columns {8i + j}; operands are swapped, so a
+        // MFMA j contracts this step's 32 rows for the columns {CPL i + j}; operands are swapped, so a
         // lane ends up with one lhs row and the weight-column indices 4q..4q+3.
-        i32x4 lo[4], hi[4];
         float col_scale[8];  // SUB: scales of the lane's 8 columns for this step's k-block
         if constexpr (SUB) {
           const f32x4_t s_lo = __builtin_bit_cast(f32x4_t, sreg[d][0]), s_hi = __builtin_bit_cast(f32x4_t, sreg[d][1]);
@@ -272,27 +283,38 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
         auto column = [&](auto j_tag) {
           constexpr int J = decltype(j_tag)::value;
           if constexpr (SUB) return column_fragment_scaled<J>(breg[d], col_scale[J]);
-          else return column_fragment<J>(breg[d]);
+          else if constexpr (EW == kEI8) return column_fragment_i8<J>(breg[d]);
+          else return column_fragment_16bit<J>(breg[d]);
         };
-        lo[0] = column(std::integral_constant<int, 0>{});
-        lo[1] = column(std::integral_constant<int, 1>{});
-        lo[2] = column(std::integral_constant<int, 2>{});
-        lo[3] = column(std::integral_constant<int, 3>{});
+        // Four columns at a time: widen, then their MFMAs.
+        auto quad = [&](auto q_tag, auto before_mfma) {
+          constexpr int Q = decltype(q_tag)::value;
+          i32x4 frag[4];
+          frag[0] = column(std::integral_constant<int, 4 * Q + 0>{});
+          frag[1] = column(std::integral_constant<int, 4 * Q + 1>{});
+          frag[2] = column(std::integral_constant<int, 4 * Q + 2>{});
+          frag[3] = column(std::integral_constant<int, 4 * Q + 3>{});
+          before_mfma();
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = mma_16x16x32<EA>(lo[j], afrag, acc[j]);
-        hi[0] = column(std::integral_constant<int, 4>{});
-        hi[1] = column(std::integral_constant<int, 5>{});
-        hi[2] = column(std::integral_constant<int, 6>{});
-        hi[3] = column(std::integral_constant<int, 7>{});
+          for (int j = 0; j < 4; ++j) acc[4 * Q + j] = mma_16x16x32<EA>(frag[j], afrag, acc[4 * Q + j]);
+        };
+        auto nothing = [] {};
         // Refill unconditionally: past the wave's slice the weight buffer reads as zero without
-        // touching memory, and a uniform loop body keeps the waits partial. The scheduling fences
-        // keep the compiler from sinking the loads to the end of the block, which would collapse
-        // the pipeline to a single step in flight.
-        __builtin_amdgcn_sched_barrier(0);
-        issue_b(d, s + kDecDepth);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[4 + j] = mma_16x16x32<EA>(hi[j], afrag, acc[4 + j]);
+        // touching memory, and a uniform loop body keeps the waits partial. The refill goes out once
+        // the last of the slot's registers have been widened; the scheduling fences keep the compiler
+        // from sinking the loads to the end of the block, which would collapse the pipeline to a
+        // single step in flight.
+        auto refill = [&] {
+          __builtin_amdgcn_sched_barrier(0);
+          issue_b(d, s + kDecDepth);
+          __builtin_amdgcn_sched_barrier(0);
+        };
+        quad(std::integral_constant<int, 0>{}, nothing);
+        if constexpr (CPL == 16) {
+          quad(std::integral_constant<int, 1>{}, nothing);
+          quad(std::integral_constant<int, 2>{}, nothing);
+        }
+        quad(std::integral_constant<int, CPL / 4 - 1>{}, refill);
         // The lhs refill goes into the registers the MFMAs above read, so it follows them.
         __builtin_amdgcn_sched_barrier(0);
         issue_a(d, s + kDecDepth);
@@ -303,42 +325,33 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
 #pragma unroll 1
     for (int s0 = kDecDepth; s0 < steps; s0 += kDecDepth) block(s0);
 
-    // Cross-wave reduction in a fixed order. acc[j][r] of lane (i, q) is row i, column 32 q + 8 r + j.
-    float* part = reinterpret_cast<float*>(smem) + wave * (kDecRows * kDecBN);
+    // Cross-wave reduction in a fixed order. acc[j][r] of lane (i, q) is row i, column CPL (4 q + r) + j.
+    float* part = reinterpret_cast<float*>(smem) + wave * (kDecRows * BN);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      float* dst = part + li * kDecBN + 32 * lq + 8 * r;
-      *reinterpret_cast<f32x4_t*>(dst) = (f32x4_t){acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-      *reinterpret_cast<f32x4_t*>(dst + 4) = (f32x4_t){acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
+      float* dst = part + li * BN + CPL * (4 * lq + r);
+#pragma unroll
+      for (int t = 0; t < CPL / 4; ++t)
+        *reinterpret_cast<f32x4_t*>(dst + 4 * t) = (f32x4_t){acc[4 * t][r], acc[4 * t + 1][r], acc[4 * t + 2][r], acc[4 * t + 3][r]};
     }
     __syncthreads();
     {
-      const int r = tid >> 4, c8 = (tid & 15) * 8;  // 16 rows x 16 column octets = 256 threads
-      const int row = rb + r, col = col0 + c8;
-      if (row < end && col + 8 <= p.n) {
-        float v[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = 0.f;
-#pragma unroll
-        for (int w = 0; w < kDecWaves; ++w) {
-          const float* src = reinterpret_cast<const float*>(smem) + w * (kDecRows * kDecBN) + r * kDecBN + c8;
-          const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(src), hi = *reinterpret_cast<const f32x4_t*>(src + 4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            v[e] += lo[e];
-            v[4 + e] += hi[e];
-          }
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          v[e] *= scale_lo[e];
-          v[4 + e] *= scale_hi[e];
-        }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = apply_activation(v[e], p.activation);
+      const int r = tid >> 4, c0 = (tid & 15) * CPL;  // 16 rows x 16 runs of CPL columns = 256 threads
+      const int row = rb + r, col = col0 + c0;
+      if (row < end && col + CPL <= p.n) {
         const int64_t idx = (int64_t)row * p.n + col;
-        store4(p.out, idx, (f32x4){v[0], v[1], v[2], v[3]}, p.out_dtype);
-        store4(p.out, idx + 4, (f32x4){v[4], v[5], v[6], v[7]}, p.out_dtype);
+#pragma unroll
+        for (int t = 0; t < CPL / 4; ++t) {
+          f32x4_t v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int w = 0; w < kDecWaves; ++w)
+            v += *reinterpret_cast<const f32x4_t*>(reinterpret_cast<const float*>(smem) + w * (kDecRows * BN) + r * BN + c0 + 4 * t);
+          v *= col_scales[t];
+          store4(p.out, idx + 4 * t,
+                 (f32x4){apply_activation(v[0], p.activation), apply_activation(v[1], p.activation),
+                         apply_activation(v[2], p.activation), apply_activation(v[3], p.activation)},
+                 p.out_dtype);
+        }
       }
     }
     __syncthreads();  // partials are consumed before the next pass overwrites them
@@ -357,9 +370,13 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
 
 // Whether the decode kernel can run this problem (else the caller uses the tiled kernel).
 bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k, int64_t n, int64_t G,
-                      int64_t scale_blocks) {
+                      int64_t scale_blocks, int32_t block_n) {
   (void)m;
   (void)G;
+  if (block_n != kDecBN) {
+    // The wide kernel: int8 weights with per-column scales, 16 columns per lane.
+    if (block_n != 2 * kDecBN || rhs_dtype != TKX_I8 || scale_blocks != 1 || n % 16 != 0) return false;
+  }
   if (scale_blocks != 1) {
     // Sub-channel scales: int8 weights, blocks of a power-of-two number of rows that whole steps fit.
     if (rhs_dtype != TKX_I8 || scale_blocks < 1 || k % scale_blocks != 0) return false;
@@ -376,7 +393,7 @@ bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k
 
 int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
                       int64_t m, int64_t k, int64_t n, int64_t G, int32_t rhs_dtype, int32_t out_dtype,
-                      int32_t activation, int32_t depth, int64_t scale_blocks, hipStream_t stream) {
+                      int32_t activation, int32_t depth, int64_t scale_blocks, int32_t block_n, hipStream_t stream) {
   DecodeParams p;
   p.scale_blocks = (int32_t)scale_blocks;
   p.log2_block_rows = 0;
@@ -391,11 +408,12 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
   p.k = (int32_t)k;
   p.n = (int32_t)n;
   p.num_groups = (int32_t)G;
-  p.n_tiles = (int32_t)((n + kDecBN - 1) / kDecBN);
+  p.n_tiles = (int32_t)((n + block_n - 1) / block_n);
   p.out_dtype = out_dtype;
   p.activation = activation;
-  // Dynamic LDS holds only the four partial tiles of the cross-wave reduction (4 x 16 x 128 f32 = 32 KB).
-  const size_t smem = kDecWaves * kDecRows * kDecBN * 4;
+  // Dynamic LDS holds only the four partial tiles of the cross-wave reduction (4 x 16 x 128 f32 = 32 KB;
+  // 64 KB for the wide kernel).
+  const size_t smem = (size_t)kDecWaves * kDecRows * block_n * 4;
   const int64_t grid = G * p.n_tiles;
   if (grid > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "too many workgroups");
   // `depth` = steps of loads in flight per wave; deeper pipelines need more registers and allow
@@ -404,6 +422,9 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
   if (sub) {
     fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 2, 3, true>)
                     : reinterpret_cast<const void*>(&decode_kernel<kEI8, 4, 2, true>);  // (8 deep would spill)
+  } else if (rhs_dtype == TKX_I8 && block_n == 2 * kDecBN) {
+    fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 2, 2, false, 16>)
+                    : reinterpret_cast<const void*>(&decode_kernel<kEI8, 4, 1, false, 16>);  // (2 workgroups per CU would spill)
   } else if (rhs_dtype == TKX_I8) {
     fn = depth <= 2   ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 2, 4>)
          : depth <= 4 ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 4, 3>)
@@ -414,6 +435,20 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
   } else {
     fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEF16, 2, 3>)
                     : reinterpret_cast<const void*>(&decode_kernel<kEF16, 4, 2>);
+  }
+  if (smem + 64 > 64 * 1024) {
+    // Past the default limit of dynamic LDS: raised once per (device, kernel).
+    static std::mutex mu;
+    static std::vector<std::pair<int, const void*>> raised;
+    int dev = 0;
+    TKX_HIP_CHECK(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(mu);
+    bool found = false;
+    for (auto& r : raised) found = found || (r.first == dev && r.second == fn);
+    if (!found) {
+      TKX_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+      raised.emplace_back(dev, fn);
+    }
   }
   DecodeParams params = p;
   void* args[] = {&params};

@@ -323,9 +323,16 @@ class HipRaggedDot(base.RaggedDot):
               else 32 if rows_per_group > 8 else 16)  # 16 = one pass of the streaming kernel; the mean must
     # leave room for the largest group, which re-reads its weights for every further 16 rows
     want_n = 256 if cols >= 2048 else 128
+    # The streaming kernel on int8 weights has a wide form (256 columns per workgroup, two workgroups
+    # per CU) that streams 7-9% faster when its workgroups fill the chip evenly, and slower than the
+    # 128-column form when they do not (measured: 384 workgroups on 256 CUs lose 10%).
+    wide_wgs = num_groups * -(-cols // 256)
+    stream_n = 256 if cols % 16 == 0 and wide_wgs / (-(-wide_wgs // 512) * 512) >= 0.9 else 128
 
     def score(v):
       bm, bn, bk, wm, wn, ns = v
+      if bm == 16:
+        return (abs(bm - want_m), abs(bn - stream_n), 0, 0, 0, ns)
       # drhs streams two row-contiguous operands: shallower k-steps with more stages in flight win there.
       if mode == 2:
         # A group's contraction (its rows) is short next to the tile it produces, so the store of a
