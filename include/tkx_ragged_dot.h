@@ -56,7 +56,11 @@ enum TkxMode {
 };
 
 enum TkxActivation { TKX_ACT_NONE = 0, TKX_ACT_RELU = 1, TKX_ACT_TANH = 2, TKX_ACT_SILU = 3, TKX_ACT_GELU_TANH = 4,
-                     TKX_ACT_SIGMOID = 5 };
+                     TKX_ACT_SIGMOID = 5,
+                     /* Gate-up fusion only (experimental/gmm_v2/gmm_v2.py:29-50): both clip gate from above and up
+                      * from both sides at a limit first. SWIGLU_OAI (limit 7): (up + 1) * gate * sigmoid(1.702 gate);
+                      * SILU_CLAMP (limit 10): silu(gate) * up. */
+                     TKX_ACT_SWIGLU_OAI = 6, TKX_ACT_SILU_CLAMP = 7 };
 
 /* Tunables; the gfx950 counterpart of the reference's Config (pallas_mosaic_gpu_common.py:45-73).
  * (block_m, block_n, block_k, waves_m, waves_n, num_stages) must name a compiled kernel variant
@@ -119,7 +123,8 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
  *   gateup = 1: rhs is [G,k,n] with its columns [gate | up] (n/2 each) and out is [m, n/2] =
  *     act(lhs.gate + bias_gate) * (lhs.up + bias_up), `activation` naming act (NONE: the plain product); needs
  *     n % 16 == 0, k % block_k == 0 and a variant of mode 3 (see tkx_ragged_dot_variant).
- *   gateup = 0: as tkx_ragged_dot_fwd plus the bias; `activation` applies to the biased result.
+ *   gateup = 0: as tkx_ragged_dot_fwd plus the bias; `activation` applies to the biased result
+ *   (TKX_ACT_SWIGLU_OAI and TKX_ACT_SILU_CLAMP need gateup = 1: TKX_ERR_INVALID otherwise).
  *   rhs_scale_blocks: rhs_scale is f32[G, rhs_scale_blocks, n], block b scaling the k rows
  *     [b * k/blocks, (b+1) * k/blocks) (scale tile (1, t_k, 1), pallas_mosaic_gpu_kernel_sm90_quant.py:91-97).
  *     1 = one scale per (group, column). More than 1 is taken by the streaming small-m kernel only

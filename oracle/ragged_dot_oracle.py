@@ -29,10 +29,12 @@ below therefore cites the reference call site it follows, and says what pins it:
   generate_group_sizes         base.py:171-196                                    invariants of base_test.py:45-51
                                                                                   (len == G, sum == m) + literal restatement
 
-  ragged_dot_fused             base.py:205-217 (docstring of `rhs_bias` and       composition of `ragged_dot` with the
-                               `fuse_gateup_activation`)                          formulas of that docstring; the
-                                                                                  activations against torch's silu /
-                                                                                  gelu(approximate="tanh")
+  ragged_dot_fused / gateup    base.py:205-217 (docstring of `rhs_bias` and       composition of `ragged_dot` with the
+                               `fuse_gateup_activation`); the gate-up forms of    formulas of that docstring; the gate-up
+                               experimental/gmm_v2/gmm_v2.py:29-50,96-107 (bias    forms against torch's silu / sigmoid /
+                               joins the accumulator before them, :662-663)       gelu(approximate="tanh") / clamp
+                                                                                  (library routines) and hand-computed
+                                                                                  values at and past the clipping limits
 
   gated_linear_unit            gated_linear_unit/base.py:60-120                   torch matmul + torch activations on
                                                                                   f64 (library routines)
@@ -42,11 +44,9 @@ below therefore cites the reference call site it follows, and says what pins it:
 
 Status of "parity unpinned": `qwix.quantize` (absmax calibration / rounding) is
 NOT restated -- quantised inputs are generated directly as (qvalue, scale) pairs.
-`ragged_dot_fused` follows the docstring's formulas only: the one reference
-backend that computes them (pallas_mosaic_tpu_v2.py:205-250) calls a kernel that
-is not in the tree, so the flavour of "gelu" (taken as jax.nn.gelu's default
-tanh form) and "swigluoai" (not restated) are parity unpinned.
-Everything else above has a pin listed.
+"gelu" in the gate-up forms is `jax.nn.gelu(gate)` (gmm_v2.py:99-100); JAX is not
+in the tree, and its documented default (`approximate=True`, the tanh form) is
+taken. Everything else above has a pin listed.
 """
 
 from __future__ import annotations
@@ -267,12 +267,34 @@ def gelu_tanh(x):
   return 0.5 * x * (1.0 + np.tanh(0.7978845608028654 * (x + 0.044715 * x ** 3)))
 
 
+def gateup(gate, up, name: str):
+  """The fused gate-up forms of experimental/gmm_v2/gmm_v2.py:96-107 on f64 arrays.
+
+  "silu": silu(gate) * up; "gelu" (`jax.nn.gelu`, whose default is the tanh form) and "gelu_tanh":
+  gelu_tanh(gate) * up; "swigluoai" (gmm_v2.py:29-38): gate clipped from above at 7, up clipped to
+  [-7, 7], (up + 1) * gate * sigmoid(1.702 gate); "silu_and_mul_with_clamp" (gmm_v2.py:41-50): the
+  same clipping at 10, silu(gate) * up.
+  """
+  gate, up = np.asarray(gate, np.float64), np.asarray(up, np.float64)
+  if name == "silu":
+    return silu(gate) * up
+  if name in ("gelu", "gelu_tanh"):
+    return gelu_tanh(gate) * up
+  if name == "swigluoai":
+    gate, up = np.minimum(gate, 7.0), np.clip(up, -7.0, 7.0)
+    return (up + 1.0) * (gate / (1.0 + np.exp(-1.702 * gate)))
+  if name == "silu_and_mul_with_clamp":
+    gate, up = np.minimum(gate, 10.0), np.clip(up, -10.0, 10.0)
+    return silu(gate) * up
+  raise NotImplementedError(name)
+
+
 def ragged_dot_fused(lhs, rhs, group_sizes, *, rhs_bias=None, gateup_activation=None, acc_dtype=np.float64,
                      out_dtype: str = "f64"):
   """`ragged_dot(lhs, rhs) + rhs_bias`, then `act(tmp[:, :n]) * tmp[:, n:]` (base.py:205-217).
 
   `rhs_bias` is [G, 1, 2n] (or [G, 2n]): row i gets the bias of its group; rows past the last group
-  stay zero. `gateup_activation` is "silu" or "gelu" (tanh form); None leaves `tmp` as it is.
+  stay zero. `gateup_activation` is a name `gateup` knows; None leaves `tmp` as it is.
   """
   tmp = np.asarray(ragged_dot(lhs, rhs, group_sizes, DEFAULT, acc_dtype=acc_dtype, out_dtype="f64"), np.float64)
   off = group_offsets(group_sizes)
@@ -283,9 +305,8 @@ def ragged_dot_fused(lhs, rhs, group_sizes, *, rhs_bias=None, gateup_activation=
       if e > s:
         tmp[s:e] += bias[g]
   if gateup_activation is not None:
-    act = {"silu": silu, "gelu": gelu_tanh}[gateup_activation]
     n = tmp.shape[1] // 2
-    tmp = act(tmp[:, :n]) * tmp[:, n:]
+    tmp = gateup(tmp[:, :n], tmp[:, n:], gateup_activation)
   return _round_out(tmp, out_dtype)
 
 

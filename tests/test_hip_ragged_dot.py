@@ -519,7 +519,35 @@ def test_rhs_bias_and_gateup_fusion(m, k, n2, gs, act, device):
            preferred_element_type=torch.float32)
   _check(got, O.silu(plain), 1e-5)
   with pytest.raises(NotImplementedError):
-    op(lhs, rhs, group_sizes=gst, fuse_gateup_activation="swigluoai")
+    op(lhs, rhs, group_sizes=gst, fuse_gateup_activation="relu")
+
+
+@pytest.mark.parametrize("act", ["swigluoai", "silu_and_mul_with_clamp", "gelu_tanh"])
+def test_clamped_gateup_forms(act, device):
+  """The clamped gate-up forms (experimental/gmm_v2/gmm_v2.py:29-50) through the op, on products wide
+  enough (standard deviation 6) that a good part of the gates and ups lies past the limits of 7 and 10;
+  the C ABI declines them outside gate-up fusion."""
+  rng = np.random.default_rng(17)
+  m, k, n2 = 300, 256, 512
+  gs = np.array([100, 0, 57, 120], np.int32)
+  G = len(gs)
+  gst = torch.tensor(gs, device=device)
+  mk = lambda shape, std: torch.tensor(rng.normal(0, std, shape).astype(np.float32), device=device)
+  lhs, rhs = mk((m, k), 1.0).to(torch.bfloat16), mk((G, k, n2), 6.0 * k ** -0.5).to(torch.bfloat16)
+  bias = mk((G, 1, n2), 2.0).to(torch.bfloat16)
+  op = tokamax_amd.HipRaggedDot()
+  tmp = O.ragged_dot_fused(_np(lhs), _np(rhs), gs, rhs_bias=_np(bias))[:int(gs.sum())]
+  assert (np.abs(tmp) > 10).mean() > 0.05 and (np.abs(tmp) < 7).mean() > 0.5  # both sides of the limits are hit
+  want = O.ragged_dot_fused(_np(lhs), _np(rhs), gs, rhs_bias=_np(bias), gateup_activation=act)
+  out = op(lhs, rhs, group_sizes=gst, rhs_bias=bias, fuse_gateup_activation=act, preferred_element_type=torch.float32)
+  _check(out, want, 1e-5)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  _check(op(lhs, rhs, group_sizes=gst, rhs_bias=bias, fuse_gateup_activation=act), want, 2e-3)
+  if act != "gelu_tanh":
+    cfg = op._get_heuristics_config(op.bind(lhs, rhs, group_sizes=gst))
+    kc = hip_ops.KernelConfig(cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages)
+    with pytest.raises(ValueError, match="gate-up"):
+      hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=kc, out_dtype=torch.float32, activation=act, rhs_bias=bias.float())
 
 
 @pytest.mark.parametrize("m,blocks", [(300, 4), (24, 8), (1100, 2)])

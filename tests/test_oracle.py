@@ -194,6 +194,35 @@ def test_fused_epilogue_terms():
                              rtol=1e-12, atol=1e-12)
 
 
+def test_clamped_gateup_forms():
+  """"swigluoai" and "silu_and_mul_with_clamp" (experimental/gmm_v2/gmm_v2.py:29-50): against torch's clamp /
+  sigmoid / silu, and values worked by hand where the clipping acts: the gate is clipped from above
+  only, the up part on both sides, and "swigluoai" multiplies by up + 1."""
+  rng = np.random.default_rng(2)
+  gate, up = rng.normal(0, 6, 400), rng.normal(0, 6, 400)
+  g, u = torch.tensor(gate), torch.tensor(up)
+  gc, uc = g.clamp(max=7.0), u.clamp(-7.0, 7.0)
+  np.testing.assert_allclose(O.gateup(gate, up, "swigluoai"), ((uc + 1) * gc * torch.sigmoid(1.702 * gc)).numpy(),
+                             rtol=1e-12, atol=1e-12)
+  gc, uc = g.clamp(max=10.0), u.clamp(-10.0, 10.0)
+  np.testing.assert_allclose(O.gateup(gate, up, "silu_and_mul_with_clamp"),
+                             (torch.nn.functional.silu(gc) * uc).numpy(), rtol=1e-12, atol=1e-12)
+  # gate 9 -> 7 and up 9 -> 7: 8 * 7 * sigmoid(11.914) = 56 / (1 + e^-11.914) = 56 / 1.0000066967 = 55.999625
+  np.testing.assert_allclose(O.gateup([9.0], [9.0], "swigluoai"), [55.999625], rtol=2e-8)
+  # up -9 -> -7: (-7 + 1) * 7 * sigmoid(11.914) = -41.999719; a zero gate gives zero; gate -> -inf gives 0 (not clipped below)
+  np.testing.assert_allclose(O.gateup([7.0], [-9.0], "swigluoai"), [-41.999719], rtol=2e-8)
+  assert O.gateup([0.0], [3.0], "swigluoai")[0] == 0.0
+  assert abs(O.gateup([-40.0], [3.0], "swigluoai")[0]) < 1e-25
+  # up = -1 cancels "swigluoai" and not the clamped silu; silu(1) = 1 / (1 + 1/e) = 0.7310585786
+  assert O.gateup([1.0], [-1.0], "swigluoai")[0] == 0.0
+  np.testing.assert_allclose(O.gateup([1.0], [-1.0], "silu_and_mul_with_clamp"), [-0.7310585786], rtol=1e-9)
+  # gate 12 -> 10, up 12 -> 10: silu(10) * 10 = 100 / (1 + e^-10) = 99.995460
+  np.testing.assert_allclose(O.gateup([12.0], [12.0], "silu_and_mul_with_clamp"), [99.995460], rtol=2e-8)
+  np.testing.assert_allclose(O.gateup(gate, up, "gelu"), O.gateup(gate, up, "gelu_tanh"))
+  with pytest.raises(NotImplementedError):
+    O.gateup(gate, up, "relu")
+
+
 def test_gated_linear_unit_matches_torch():
   rng = np.random.default_rng(3)
   x, w = rng.normal(size=(2, 5, 7)), rng.normal(size=(7, 2, 4))

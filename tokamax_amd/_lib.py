@@ -16,7 +16,8 @@ LIB_PATH = os.path.join(_HERE, "lib", "libtkx_ragged_dot.so")
 TKX_OK, TKX_ERR_INVALID, TKX_ERR_UNSUPPORTED, TKX_ERR_RUNTIME = 0, 1, 2, 3
 TKX_F32, TKX_BF16, TKX_F16, TKX_F8E4M3FN, TKX_I8 = 0, 1, 2, 3, 4
 TKX_MODE_DEFAULT, TKX_MODE_TRANS_RHS = 0, 1
-ACTIVATIONS = {None: 0, "relu": 1, "tanh": 2, "silu": 3, "gelu_tanh": 4, "sigmoid": 5}
+ACTIVATIONS = {None: 0, "relu": 1, "tanh": 2, "silu": 3, "gelu_tanh": 4, "sigmoid": 5,
+               "swigluoai": 6, "silu_and_mul_with_clamp": 7}  # the last two: gate-up fusion only
 
 # Names of every symbol include/tkx_ragged_dot.h declares.
 EXPORTED_SYMBOLS = (

@@ -144,8 +144,10 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
                      (long long)n, (long long)num_groups);
   if (mode != TKX_MODE_DEFAULT && mode != TKX_MODE_TRANS_RHS) return set_error(TKX_ERR_INVALID, "bad mode %d", mode);
   if (!valid_out_dtype(out_dtype)) return set_error(TKX_ERR_UNSUPPORTED, "out dtype %d not supported", out_dtype);
-  if (activation < TKX_ACT_NONE || activation > TKX_ACT_SIGMOID)
+  if (activation < TKX_ACT_NONE || activation > TKX_ACT_SILU_CLAMP)
     return set_error(TKX_ERR_INVALID, "bad activation %d", activation);
+  if (activation > TKX_ACT_SIGMOID && !gateup)
+    return set_error(TKX_ERR_INVALID, "activation %d belongs to gate-up fusion", activation);
   // Per-lane byte offsets inside a tile are 32-bit: (256 rows) x (row bytes) must stay below 2^31.
   if (m > 0x7fffffffLL / 2 || k >= (1 << 21) || n >= (1 << 21))
     return set_error(TKX_ERR_UNSUPPORTED, "dimension too large");

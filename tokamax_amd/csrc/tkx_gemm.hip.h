@@ -777,6 +777,23 @@ struct GemmKernel {
           }
         }
       }
+      if constexpr (GLU) {
+        // The clamped gate-up forms clip the gate from above and the up part from both sides first;
+        // "swigluoai" multiplies by up + 1.
+        if (p.activation == TKX_ACT_SWIGLU_OAI || p.activation == TKX_ACT_SILU_CLAMP) {
+          const float limit = p.activation == TKX_ACT_SWIGLU_OAI ? 7.f : 10.f;
+          const float shift = p.activation == TKX_ACT_SWIGLU_OAI ? 1.f : 0.f;
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TNO; ++j)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) {
+                acc[i][j][e] = fminf(acc[i][j][e], limit);
+                acc[i][j + TNO][e] = fminf(fmaxf(acc[i][j + TNO][e], -limit), limit) + shift;
+              }
+        }
+      }
       if (p.activation != TKX_ACT_NONE) {
         auto for_all = [&](auto fn) {
 #pragma unroll
@@ -791,7 +808,10 @@ struct GemmKernel {
         auto fast_tanh = [](float x) { return 1.f - 2.f * __builtin_amdgcn_rcpf(__expf(2.f * x) + 1.f); };
         if (p.activation == TKX_ACT_RELU) for_all([](float x) { return x > 0.f ? x : 0.f; });
         else if (p.activation == TKX_ACT_TANH) for_all(fast_tanh);
-        else if (p.activation == TKX_ACT_SILU) for_all([](float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-x)); });
+        else if (p.activation == TKX_ACT_SILU || p.activation == TKX_ACT_SILU_CLAMP)
+          for_all([](float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-x)); });
+        else if (p.activation == TKX_ACT_SWIGLU_OAI)
+          for_all([](float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-1.702f * x)); });
         else if (p.activation == TKX_ACT_SIGMOID) for_all([](float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); });
         else if (p.activation == TKX_ACT_GELU_TANH)
           for_all([&](float x) { return 0.5f * x * (1.f + fast_tanh(0.7978845608028654f * (x + 0.044715f * x * x * x))); });

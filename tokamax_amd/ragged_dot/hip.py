@@ -71,8 +71,10 @@ _ACTIVATION_NAMES = {
 }
 
 
-# `fuse_gateup_activation` names -> in-kernel activation (jax.nn.gelu defaults to the tanh form).
-_GATEUP_ACTIVATIONS = {"silu": "silu", "gelu": "gelu_tanh"}
+# `fuse_gateup_activation` names (experimental/gmm_v2/gmm_v2.py:96-107) -> in-kernel activation.
+# "gelu" is `jax.nn.gelu(gate)`, whose default is the tanh form.
+_GATEUP_ACTIVATIONS = {"silu": "silu", "gelu": "gelu_tanh", "gelu_tanh": "gelu_tanh", "swigluoai": "swigluoai",
+                       "silu_and_mul_with_clamp": "silu_and_mul_with_clamp"}
 
 
 def _fused_activation_name(activation) -> str | None:
@@ -170,7 +172,7 @@ class HipRaggedDot(base.RaggedDot):
       gateup = _GATEUP_ACTIVATIONS.get(fuse_gateup_activation)
       if gateup is None:
         raise NotImplementedError(f"fuse_gateup_activation={fuse_gateup_activation!r} is not supported by the hip"
-                                  " implementation (supported: 'silu', 'gelu').")
+                                  f" implementation (supported: {sorted(_GATEUP_ACTIVATIONS)}).")
       if return_residuals:
         raise NotImplementedError("return_residuals is not supported with fuse_gateup_activation.")
     if isinstance(lhs, AsQArray) or isinstance(rhs, AsQArray):
