@@ -130,12 +130,18 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
  *     1 = one scale per (group, column). More than 1 is taken by the streaming small-m kernel only
  *     (int8 weights, k/blocks a power of two >= 32); for the tiled kernels widen the weights with
  *     tkx_dequantize_weights first.
+ *   group_offset: device int32[1] or NULL (the `group_offset` argument of RaggedDot, base.py:238; semantics of
+ *     experimental/gmm_v2/gmm_v2_test.py:44-101): `group_sizes` then has `num_group_sizes` entries, the
+ *     `num_groups` groups of rhs are its entries [offset, offset + num_groups) (entries outside the array count
+ *     as empty), and the rows of every other entry come out zero: the call of one expert-parallel shard. Read on
+ *     the device, so the offset can change between replays of a captured graph. NULL: `num_group_sizes` is ignored.
  * The streaming small-m kernel (block_m == 16) takes neither a bias nor gate-up fusion. */
 int32_t tkx_ragged_dot_fwd_fused(const void* lhs, const void* rhs, const int32_t* group_sizes,
-                                 const float* lhs_scale, const float* rhs_scale, const float* rhs_bias, void* out,
-                                 void* workspace, int64_t m, int64_t k, int64_t n, int64_t num_groups,
-                                 int64_t rhs_scale_blocks, int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype,
-                                 int32_t activation, int32_t gateup, const TkxConfig* config, tkx_stream_t stream);
+                                 const int32_t* group_offset, const float* lhs_scale, const float* rhs_scale,
+                                 const float* rhs_bias, void* out, void* workspace, int64_t m, int64_t k, int64_t n,
+                                 int64_t num_groups, int64_t num_group_sizes, int64_t rhs_scale_blocks,
+                                 int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype, int32_t activation,
+                                 int32_t gateup, const TkxConfig* config, tkx_stream_t stream);
 
 /* Part (4-drhs): out[G,k,n] = lhs[rows_g, k]^T . dout[rows_g, n], zeros for empty groups.
  * lhs [m,k], dout [m,n] row-major of `dtype` (f32/bf16/f16); out_dtype f32/bf16/f16.

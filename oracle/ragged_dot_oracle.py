@@ -289,21 +289,35 @@ def gateup(gate, up, name: str):
   raise NotImplementedError(name)
 
 
-def ragged_dot_fused(lhs, rhs, group_sizes, *, rhs_bias=None, gateup_activation=None, acc_dtype=np.float64,
-                     out_dtype: str = "f64"):
+def ragged_dot_fused(lhs, rhs, group_sizes, *, rhs_bias=None, gateup_activation=None, group_offset=None,
+                     acc_dtype=np.float64, out_dtype: str = "f64"):
   """`ragged_dot(lhs, rhs) + rhs_bias`, then `act(tmp[:, :n]) * tmp[:, n:]` (base.py:205-217).
 
   `rhs_bias` is [G, 1, 2n] (or [G, 2n]): row i gets the bias of its group; rows past the last group
   stay zero. `gateup_activation` is a name `gateup` knows; None leaves `tmp` as it is.
+  `group_offset` (experimental/gmm_v2/gmm_v2_test.py:44-101): `group_sizes` lists every group of the
+  job, `rhs` and `rhs_bias` hold the groups [offset, offset + G) of them, and the rows of all other
+  groups are zero (before the gate-up form, which maps zeros to zero).
   """
-  tmp = np.asarray(ragged_dot(lhs, rhs, group_sizes, DEFAULT, acc_dtype=acc_dtype, out_dtype="f64"), np.float64)
+  lhs_, rhs_ = np.asarray(lhs), np.asarray(rhs)
+  G = rhs_.shape[0]
+  goff = 0 if group_offset is None else int(np.asarray(group_offset).reshape(-1)[0])
   off = group_offsets(group_sizes)
+  if group_offset is None:
+    tmp = np.asarray(ragged_dot(lhs_, rhs_, group_sizes, DEFAULT, acc_dtype=acc_dtype, out_dtype="f64"), np.float64)
+  else:
+    tmp = np.zeros((lhs_.shape[0], rhs_.shape[2]), np.float64)
+    for j in range(len(off) - 1):
+      s, e = int(off[j]), min(int(off[j + 1]), tmp.shape[0])
+      if 0 <= j - goff < G and e > s:
+        tmp[s:e] = ragged_dot(lhs_[s:e], rhs_[j - goff:j - goff + 1], [e - s], DEFAULT, acc_dtype=acc_dtype,
+                              out_dtype="f64")
   if rhs_bias is not None:
-    bias = np.asarray(rhs_bias, np.float64).reshape(len(off) - 1, -1)
-    for g in range(len(off) - 1):
-      s, e = int(off[g]), min(int(off[g + 1]), tmp.shape[0])
-      if e > s:
-        tmp[s:e] += bias[g]
+    bias = np.asarray(rhs_bias, np.float64).reshape(G, -1)
+    for j in range(len(off) - 1):
+      s, e = int(off[j]), min(int(off[j + 1]), tmp.shape[0])
+      if 0 <= j - goff < G and e > s:
+        tmp[s:e] += bias[j - goff]
   if gateup_activation is not None:
     n = tmp.shape[1] // 2
     tmp = gateup(tmp[:, :n], tmp[:, n:], gateup_activation)

@@ -550,6 +550,104 @@ def test_clamped_gateup_forms(act, device):
       hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=kc, out_dtype=torch.float32, activation=act, rhs_bias=bias.float())
 
 
+@pytest.mark.parametrize("offset,local", [(0, 6), (2, 3), (4, 2), (5, 3), (-1, 3), (7, 2)])
+def test_group_offset_tiled_kernels(offset, local, device):
+  """`group_offset` (experimental/gmm_v2/gmm_v2_test.py:44-101) through the op on the tiled kernels: rhs and
+  rhs_bias hold `local` of the 6 groups, starting at `offset` (also past either end of the sizes); the rows
+  of the other groups and the rows of no group are zero; with and without gate-up fusion."""
+  rng = np.random.default_rng(40 + offset)
+  gs = np.array([100, 0, 57, 120, 3, 260], np.int32)
+  m, k, n2 = int(gs.sum()) + 20, 256, 512
+  gst = torch.tensor(gs, device=device)
+  mk = lambda shape, std: torch.tensor(rng.normal(0, std, shape).astype(np.float32), device=device)
+  lhs, rhs = mk((m, k), 1.0).to(torch.bfloat16), mk((local, k, n2), k ** -0.5).to(torch.bfloat16)
+  bias = mk((local, 1, n2), 0.7).to(torch.bfloat16)
+  goff = torch.tensor([offset], dtype=torch.int32, device=device)
+  op = tokamax_amd.HipRaggedDot()
+  for act in (None, "silu"):
+    want = O.ragged_dot_fused(_np(lhs), _np(rhs), gs, rhs_bias=_np(bias), gateup_activation=act, group_offset=[offset])
+    out = op(lhs, rhs, group_sizes=gst, rhs_bias=bias, fuse_gateup_activation=act, group_offset=goff,
+             preferred_element_type=torch.float32)
+    if np.any(want):
+      _check(out, want, 1e-5)
+    assert torch.equal(out == 0, torch.tensor(want == 0, device=device))  # the same rows are exactly zero
+  # without a bias, bf16 out, and the offset as a plain int
+  want = O.ragged_dot_fused(_np(lhs), _np(rhs), gs, group_offset=[offset])
+  out = op(lhs, rhs, group_sizes=gst, group_offset=offset)
+  if np.any(want):
+    _check(out, want, 2e-3)
+  assert torch.count_nonzero(out[torch.tensor(~want.any(axis=1), device=device)]) == 0
+  with pytest.raises(NotImplementedError):  # the public entry declines it, as api.py:183-184 does
+    tokamax_amd.ragged_dot(lhs, rhs, gst, group_offset=goff)
+
+
+def test_group_offset_shards_add_up_and_follow_the_device_value(device):
+  """Four expert-parallel shards of 8 experts (2 each) of one job add up to the unsharded result, bit for bit
+  in f32 (every row is computed by exactly one shard, by the same kernel); the offset is read on the device, so
+  one tensor updated in place serves all four calls."""
+  rng = np.random.default_rng(8)
+  G, k, n = 8, 512, 1024
+  gs = rng.multinomial(1500, [1 / G] * G).astype(np.int32)
+  m = int(gs.sum()) + 36
+  gst = torch.tensor(gs, device=device)
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  rhs = torch.tensor(rng.normal(0, k ** -0.5, (G, k, n)).astype(np.float32), device=device).to(torch.bfloat16)
+  op = tokamax_amd.HipRaggedDot()
+  full = op(lhs, rhs, group_sizes=gst, preferred_element_type=torch.float32)
+  goff = torch.zeros(1, dtype=torch.int32, device=device)
+  total = torch.zeros_like(full)
+  for shard in range(4):
+    goff.fill_(2 * shard)
+    part = op(lhs, rhs[2 * shard:2 * shard + 2], group_sizes=gst, group_offset=goff, preferred_element_type=torch.float32)
+    rows = slice(int(gs[:2 * shard].sum()), int(gs[:2 * shard + 2].sum()))
+    assert torch.count_nonzero(part[:rows.start]) == 0 and torch.count_nonzero(part[rows.stop:]) == 0
+    total += part
+  assert torch.equal(total, full)
+
+
+@pytest.mark.parametrize("block_n", [128, 256])
+@pytest.mark.parametrize("offset,local", [(0, 9), (3, 4), (7, 4), (-2, 5)])
+def test_group_offset_small_m_kernel(offset, local, block_n, device):
+  """`group_offset` in the streaming small-m kernel (int8 weights): the kernel derives its row ranges
+  from the job's sizes and the device-side offset; rows of other groups are zero."""
+  rng = np.random.default_rng(60 + offset)
+  gs = np.array([3, 0, 5, 17, 1, 0, 16, 2, 4], np.int32)
+  k, n = 1024, 464
+  m = int(gs.sum()) + 5
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  rhs = torch.tensor(rng.integers(-128, 128, (local, k, n)).astype(np.int8), device=device)
+  scale = torch.tensor((np.abs(rng.normal(0, 0.01, (local, 1, n))) + 1e-3).astype(np.float32), device=device)
+  cfg = hip_ops.KernelConfig(16, block_n, 32, 1, 4, 2)
+  goff = torch.tensor([offset], dtype=torch.int32, device=device)
+  out = hip_ops.ragged_dot_fwd(lhs, rhs, torch.tensor(gs, device=device), config=cfg, out_dtype=torch.float32,
+                               rhs_scale=scale, group_offset=goff)
+  want = O.ragged_dot_fused(_np(lhs), O.dequantize(rhs.cpu().numpy(), _np(scale)), gs, group_offset=[offset])
+  _check(out, want, 1e-5)
+  assert torch.equal(out == 0, torch.tensor(want == 0, device=device))
+
+
+def test_raw_rhs_scale_argument(device):
+  """The `rhs_scale` argument of RaggedDot (base.py:208; shape [g, k-blocks, 1, n] with raw int8 weights,
+  experimental/gmm_v2/gmm_v2.py:1193-1199) gives what the same weights give as a QArray; the result defaults
+  to lhs.dtype."""
+  rng = np.random.default_rng(12)
+  G, m, k, n = 4, 300, 256, 512
+  gs = np.array([100, 0, 80, 110], np.int32)
+  gst = torch.tensor(gs, device=device)
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  q = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+  op = tokamax_amd.HipRaggedDot()
+  for blocks in (1, 4):
+    scale = torch.tensor((rng.uniform(0.5, 1.5, (G, blocks, n)) / 127 * 0.1).astype(np.float32), device=device)
+    out = op(lhs, q, group_sizes=gst, rhs_scale=scale.reshape(G, blocks, 1, n))
+    assert out.dtype == torch.bfloat16
+    assert torch.equal(out, op(lhs, tokamax_amd.QArray(q, scale), group_sizes=gst, preferred_element_type=torch.bfloat16))
+    _check(out, O.ragged_dot(_np(lhs), O.dequantize(q.cpu().numpy(), _np(scale)), gs, acc_dtype=np.float64, out_dtype="f64"),
+           3e-3)
+  with pytest.raises(NotImplementedError):
+    op(lhs, q, group_sizes=gst, rhs_scale=scale)  # not [g, blocks, 1, n]
+
+
 @pytest.mark.parametrize("m,blocks", [(300, 4), (24, 8), (1100, 2)])
 def test_int8_weights_with_sub_channel_scales(m, blocks, device):
   """Scale tile (1, t_k, 1) with t_k < k (pallas_mosaic_gpu_kernel_sm90_quant.py:91-97): the weights are

@@ -74,8 +74,8 @@ def test_c_abi_argument_errors_without_gpu():
   assert st == _lib.TKX_ERR_INVALID and "null" in _lib.last_error()
   with pytest.raises(ValueError):
     _lib.check(st)
-  st = lib.tkx_ragged_dot_fwd_fused(None, None, None, None, None, None, None, None, 8, 8, 8, 1, 1, 1, 1, 1, 0, 2,
-                                    ctypes.byref(cfg), None)
+  st = lib.tkx_ragged_dot_fwd_fused(None, None, None, None, None, None, None, None, None, 8, 8, 8, 1, 1, 1, 1, 1, 1, 0,
+                                    2, ctypes.byref(cfg), None)
   assert st == _lib.TKX_ERR_INVALID and "gateup" in _lib.last_error()
   with pytest.raises(NotImplementedError):
     _lib.check(_lib.TKX_ERR_UNSUPPORTED)

@@ -223,6 +223,36 @@ def test_clamped_gateup_forms():
     O.gateup(gate, up, "relu")
 
 
+def test_group_offset_shards():
+  """`group_offset` (experimental/gmm_v2/gmm_v2_test.py:44-101): rhs holds the groups [offset, offset + G)
+  of the job's group sizes and every other group's rows are zero. Pinned by explicit loops on a tiny
+  case and by the identity it exists for: the shards' outputs add up to the unsharded result."""
+  rng = np.random.default_rng(4)
+  gs = np.array([2, 0, 3, 1, 4], np.int32)  # 10 rows, then 2 rows of no group
+  lhs, rhs = rng.normal(size=(12, 5)), rng.normal(size=(5, 5, 6))
+  bias = rng.normal(size=(5, 1, 6))
+  full = O.ragged_dot_fused(lhs, rhs, gs, rhs_bias=bias)
+  np.testing.assert_array_equal(O.ragged_dot_fused(lhs, rhs, gs, rhs_bias=bias, group_offset=[0]), full)
+  # groups 2 and 3 (rows 2..5) as a shard of two groups
+  want = np.zeros((12, 6))
+  for i in range(2, 5):
+    want[i] = lhs[i] @ rhs[2] + bias[2, 0]
+  want[5] = lhs[5] @ rhs[3] + bias[3, 0]
+  got = O.ragged_dot_fused(lhs, rhs[2:4], gs, rhs_bias=bias[2:4], group_offset=np.array([2]))
+  np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-12)
+  parts = [O.ragged_dot_fused(lhs, rhs[o:o + c], gs, rhs_bias=bias[o:o + c], group_offset=[o]) for o, c in ((0, 2), (2, 2), (4, 1))]
+  np.testing.assert_allclose(sum(parts), full, rtol=1e-12, atol=1e-12)
+  # a shard past the last group, and one that starts before the first: entries outside the sizes are empty
+  assert not O.ragged_dot_fused(lhs, rhs[:2], gs, group_offset=[5]).any()
+  got = O.ragged_dot_fused(lhs, rhs[:3], gs, group_offset=[-2])  # local group 2 is global group 0
+  want = np.zeros((12, 6))
+  want[:2] = lhs[:2] @ rhs[2]
+  np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-12)
+  # the gate-up form keeps the other groups' rows at zero
+  glu = O.ragged_dot_fused(lhs, rhs[2:4], gs, rhs_bias=bias[2:4], group_offset=[2], gateup_activation="swigluoai")
+  assert glu.shape == (12, 3) and not glu[:2].any() and not glu[6:].any() and glu[2:6].all()
+
+
 def test_gated_linear_unit_matches_torch():
   rng = np.random.default_rng(3)
   x, w = rng.normal(size=(2, 5, 7)), rng.normal(size=(7, 2, 4))

@@ -76,8 +76,8 @@ def _declare(lib):
   lib.tkx_ragged_dot_fwd.restype = i32
   lib.tkx_ragged_dot_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32, i32, i32, i32, cfgp, vp]
   lib.tkx_ragged_dot_fwd_fused.restype = i32
-  lib.tkx_ragged_dot_fwd_fused.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, i32, i32, i32,
-                                           i32, cfgp, vp]
+  lib.tkx_ragged_dot_fwd_fused.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, i32,
+                                           i32, i32, i32, cfgp, vp]
   lib.tkx_ragged_dot_drhs.restype = i32
   lib.tkx_ragged_dot_drhs.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32, cfgp, vp]
   lib.tkx_dequantize_weights.restype = i32

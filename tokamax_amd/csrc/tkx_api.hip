@@ -122,8 +122,8 @@ int32_t tkx_ragged_dot_schedule(const int32_t* group_sizes, int64_t num_groups, 
   if (num_groups < 1 || m < 0) return set_error(TKX_ERR_INVALID, "bad sizes m=%lld G=%lld", (long long)m, (long long)num_groups);
   if (block_m < 1 || align_tile < 1) return set_error(TKX_ERR_INVALID, "block_m and align_tile must be positive");
   const WsLayout L = ws_layout(m, num_groups, block_m);
-  return launch_schedule(group_sizes, num_groups, m, block_m, align_tile, 1, static_cast<int32_t*>(workspace), L,
-                         static_cast<hipStream_t>(stream));
+  return launch_schedule(group_sizes, num_groups, nullptr, num_groups, m, block_m, align_tile, 1,
+                         static_cast<int32_t*>(workspace), L, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"
@@ -131,14 +131,19 @@ int32_t tkx_ragged_dot_schedule(const int32_t* group_sizes, int64_t num_groups, 
 namespace {
 // Forward / dlhs launcher behind both public forward entry points. `gateup`: rhs is [g, k, n] =
 // [gate | up] and out is [m, n/2] = act(lhs.gate + bias) * (lhs.up + bias), `activation` naming act.
-int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, const float* lhs_scale,
-                 const float* rhs_scale, const float* rhs_bias, void* out, void* workspace, int64_t m, int64_t k,
-                 int64_t n, int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype, int32_t mode,
-                 int32_t activation, bool gateup, int64_t rhs_scale_blocks, const TkxConfig* config,
-                 tkx_stream_t stream_) {
+// `group_offset` (device, one int32, or null) and `num_group_sizes`: the num_groups groups of rhs are
+// entries [offset, offset + num_groups) of the num_group_sizes group sizes.
+int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, const int32_t* group_offset,
+                 const float* lhs_scale, const float* rhs_scale, const float* rhs_bias, void* out, void* workspace,
+                 int64_t m, int64_t k, int64_t n, int64_t num_groups, int64_t num_group_sizes, int32_t lhs_dtype,
+                 int32_t rhs_dtype, int32_t out_dtype, int32_t mode, int32_t activation, bool gateup,
+                 int64_t rhs_scale_blocks, const TkxConfig* config, tkx_stream_t stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (!lhs || !rhs || !group_sizes || !out || !workspace || !config)
     return set_error(TKX_ERR_INVALID, "null pointer argument");
+  if (group_offset == nullptr) num_group_sizes = num_groups;
+  if (num_group_sizes < 1 || num_group_sizes > 0x7fffffffLL)
+    return set_error(TKX_ERR_INVALID, "bad number of group sizes %lld", (long long)num_group_sizes);
   if (m < 1 || k < 1 || n < 1 || num_groups < 1)
     return set_error(TKX_ERR_INVALID, "bad sizes m=%lld k=%lld n=%lld G=%lld", (long long)m, (long long)k,
                      (long long)n, (long long)num_groups);
@@ -191,7 +196,7 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
                        " and scale blocks of a power-of-two multiple of 32 rows (k=%lld n=%lld G=%lld scale blocks=%lld)",
                        (long long)k, (long long)n, (long long)num_groups, (long long)rhs_scale_blocks);
     return launch_decode(lhs, rhs, rhs_scale, group_sizes, out, m, k, n, num_groups, rhs_dtype, out_dtype, activation,
-                         c.num_stages, rhs_scale ? rhs_scale_blocks : 1, c.block_n, stream);
+                         c.num_stages, rhs_scale ? rhs_scale_blocks : 1, c.block_n, group_offset, num_group_sizes, stream);
   }
   if (rhs_scale && rhs_scale_blocks != 1)
     return set_error(TKX_ERR_UNSUPPORTED,
@@ -199,8 +204,8 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
                      " along k with tkx_dequantize_weights first", (long long)rhs_scale_blocks);
 
   const WsLayout L = ws_layout(m, num_groups, c.block_m);
-  int32_t st = launch_schedule(group_sizes, num_groups, m, c.block_m, c.align_tile, c.grid_tile_width,
-                               static_cast<int32_t*>(workspace), L, stream);
+  int32_t st = launch_schedule(group_sizes, num_groups, group_offset, num_group_sizes, m, c.block_m, c.align_tile,
+                               c.grid_tile_width, static_cast<int32_t*>(workspace), L, stream);
   if (st != TKX_OK) return st;
 
   GemmParams p = {};
@@ -238,7 +243,8 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
   p.ws_span_first = (int32_t)L.task[6];
   p.ws_span_width = (int32_t)L.task[7];
   if (slots > 0x7fffff00LL) return set_error(TKX_ERR_UNSUPPORTED, "too many tiles");
-  // Extra workgroups zero the rows past sum(group_sizes); they exit at once when there are none.
+  // Extra workgroups zero the rows past the last group (and before the first, with a group offset);
+  // they exit at once when there are none.
   int64_t zero_wgs = (m * cols * ob + (64 << 10) - 1) / (64 << 10);
   if (zero_wgs > 256) zero_wgs = 256;
   if (zero_wgs < 1) zero_wgs = 1;
@@ -252,19 +258,23 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
                            const float* rhs_scale, void* out, void* workspace, int64_t m, int64_t k, int64_t n,
                            int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype, int32_t out_dtype, int32_t mode,
                            int32_t activation, const TkxConfig* config, tkx_stream_t stream) {
-  return fwd_impl(lhs, rhs, group_sizes, lhs_scale, rhs_scale, nullptr, out, workspace, m, k, n, num_groups, lhs_dtype,
-                  rhs_dtype, out_dtype, mode, activation, false, 1, config, stream);
+  return fwd_impl(lhs, rhs, group_sizes, nullptr, lhs_scale, rhs_scale, nullptr, out, workspace, m, k, n, num_groups,
+                  num_groups, lhs_dtype, rhs_dtype, out_dtype, mode, activation, false, 1, config, stream);
 }
 
-int32_t tkx_ragged_dot_fwd_fused(const void* lhs, const void* rhs, const int32_t* group_sizes, const float* lhs_scale,
-                                 const float* rhs_scale, const float* rhs_bias, void* out, void* workspace, int64_t m,
-                                 int64_t k, int64_t n, int64_t num_groups, int64_t rhs_scale_blocks, int32_t lhs_dtype,
-                                 int32_t rhs_dtype, int32_t out_dtype, int32_t activation, int32_t gateup,
-                                 const TkxConfig* config, tkx_stream_t stream) {
+int32_t tkx_ragged_dot_fwd_fused(const void* lhs, const void* rhs, const int32_t* group_sizes, const int32_t* group_offset,
+                                 const float* lhs_scale, const float* rhs_scale, const float* rhs_bias, void* out,
+                                 void* workspace, int64_t m, int64_t k, int64_t n, int64_t num_groups,
+                                 int64_t num_group_sizes, int64_t rhs_scale_blocks, int32_t lhs_dtype, int32_t rhs_dtype,
+                                 int32_t out_dtype, int32_t activation, int32_t gateup, const TkxConfig* config,
+                                 tkx_stream_t stream) {
   if (gateup != 0 && gateup != 1) return set_error(TKX_ERR_INVALID, "gateup must be 0 or 1");
   if (rhs_scale_blocks < 1) return set_error(TKX_ERR_INVALID, "rhs_scale_blocks must be >= 1");
-  return fwd_impl(lhs, rhs, group_sizes, lhs_scale, rhs_scale, rhs_bias, out, workspace, m, k, n, num_groups, lhs_dtype,
-                  rhs_dtype, out_dtype, TKX_MODE_DEFAULT, activation, gateup == 1, rhs_scale_blocks, config, stream);
+  if (group_offset != nullptr && (uintptr_t)group_offset % 4 != 0)
+    return set_error(TKX_ERR_INVALID, "group_offset must be 4-byte aligned");
+  return fwd_impl(lhs, rhs, group_sizes, group_offset, lhs_scale, rhs_scale, rhs_bias, out, workspace, m, k, n, num_groups,
+                  num_group_sizes, lhs_dtype, rhs_dtype, out_dtype, TKX_MODE_DEFAULT, activation, gateup == 1,
+                  rhs_scale_blocks, config, stream);
 }
 
 int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* group_sizes, void* out, void* workspace,
@@ -295,7 +305,8 @@ int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* gr
   // so the workspace size depends on (m, G) alone.
   const int32_t sched_bm = 128;
   const WsLayout L = ws_layout(m, num_groups, sched_bm);
-  int32_t st = launch_schedule(group_sizes, num_groups, m, sched_bm, c.align_tile, 1, static_cast<int32_t*>(workspace), L, stream);
+  int32_t st = launch_schedule(group_sizes, num_groups, nullptr, num_groups, m, sched_bm, c.align_tile, 1,
+                               static_cast<int32_t*>(workspace), L, stream);
   if (st != TKX_OK) return st;
 
   GemmParams p = {};

@@ -9,7 +9,7 @@
 namespace tkx {
 
 // ---- workspace layout (int32 words) -----------------------------------------------------------
-// [0] num_tasks  [1] total_rows  [kWsHeader ..) group_offsets[G+1]  then eight task arrays of
+// [0] num_tasks  [1] total_rows (end of the last group)  [2] rows before the first group  [kWsHeader ..) group_offsets[G+1]  then eight task arrays of
 // tid_size words each (group_id, block_start, actual_start, actual_end, start_within_block,
 // actual_size, span_first, span_width); every array starts on a 64-word boundary. The last two
 // are not part of the reference's schedule: they cut each group's tasks into spans of at most
@@ -52,8 +52,11 @@ int32_t set_error(int32_t code, const char* fmt, ...);
   } while (0)
 
 // ---- schedule -------------------------------------------------------------------------------------
-int32_t launch_schedule(const int32_t* group_sizes, int64_t G, int64_t m, int32_t block_m, int32_t align_tile,
-                        int32_t span_width, int32_t* ws, const WsLayout& L, hipStream_t stream);
+// `group_offset` (device, one int32; null = 0): the G groups are entries [offset, offset + G) of the
+// `num_global` group sizes.
+int32_t launch_schedule(const int32_t* group_sizes, int64_t G, const int32_t* group_offset, int64_t num_global, int64_t m,
+                        int32_t block_m, int32_t align_tile, int32_t span_width, int32_t* ws, const WsLayout& L,
+                        hipStream_t stream);
 
 // ---- grouped GEMM -----------------------------------------------------------------------------
 // kFwdGlu = forward over weights [gate | up] ([g, k, 2 n_out]) with the epilogue act(gate) * up.
@@ -101,7 +104,8 @@ bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k
                       int64_t scale_blocks, int32_t block_n);
 int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
                       int64_t m, int64_t k, int64_t n, int64_t G, int32_t rhs_dtype, int32_t out_dtype,
-                      int32_t activation, int32_t depth, int64_t scale_blocks, int32_t block_n, hipStream_t stream);
+                      int32_t activation, int32_t depth, int64_t scale_blocks, int32_t block_n,
+                      const int32_t* group_offset, int64_t num_global, hipStream_t stream);
 
 // ---- dequantisation of int8 weights with sub-channel scales to bf16 ------------------------------
 int32_t launch_dequant_i8(const void* q, const float* scale, void* out, int64_t G, int64_t k, int64_t n, int64_t t_k,

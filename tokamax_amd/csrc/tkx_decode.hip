@@ -42,6 +42,8 @@ struct DecodeParams {
   const int32_t* group_sizes;
   void* out;
   int32_t m, k, n, num_groups, n_tiles, out_dtype, activation;
+  const int32_t* group_offset;  // device, one int32, or null: group g is entry offset + g of group_sizes
+  int32_t num_global;           // entries of group_sizes (num_groups without an offset)
   int32_t scale_blocks;     // scale blocks along k: scale is [G, scale_blocks, n]
   int32_t log2_block_rows;  // scale_blocks > 1: log2 of the contraction rows per scale block
 };
@@ -157,8 +159,13 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
   // and used last: the first weight steps go out right behind them, before anything is known
   // about the group, so that one memory round trip covers both. A workgroup whose group turns out
   // empty returns with those few loads in flight (32 KB of the group's 1.5 MB, never more).
-  const int first_size = p.group_sizes[min(tid, p.num_groups - 1)];  // unconditional: no wait until it is used
-  const int own_size = max(p.group_sizes[g], 0);
+  // With a group offset the group is entry offset + g of the sizes (entries outside the array count
+  // as empty) and the rows of the entries before `offset` are skipped; that costs one more dependent
+  // load ahead of the sizes, which the weight loads below overlap as well.
+  const int gg = g + (p.group_offset != nullptr ? __builtin_amdgcn_readfirstlane(p.group_offset[0]) : 0);
+  const int first_size = p.group_sizes[min(tid, p.num_global - 1)];  // unconditional: no wait until it is used
+  const int own_size = gg >= 0 && gg < p.num_global ? max(p.group_sizes[min(max(gg, 0), p.num_global - 1)], 0) : 0;
+  const int preceding = min(max(gg, 0), p.num_global);  // entries whose rows come before this group's
 
   const int kw = p.k / kDecWaves;      // contraction slice of this wave
   const int k_begin = wave * kw;
@@ -217,9 +224,10 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
 
   // Row range of this group.
   const int size = __builtin_amdgcn_readfirstlane(own_size);
-  if (size == 0 && !last_group) return;
-  int before = tid < g ? max(first_size, 0) : 0;
-  for (int j = tid + kDecThreads; j < g; j += kDecThreads) before += max(p.group_sizes[j], 0);  // G > 256 only
+  const bool first_of_shard = g == 0 && p.group_offset != nullptr;
+  if (size == 0 && !last_group && !first_of_shard) return;
+  int before = tid < preceding ? max(first_size, 0) : 0;
+  for (int j = tid + kDecThreads; j < preceding; j += kDecThreads) before += max(p.group_sizes[j], 0);  // G > 256 only
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off);
   if (lane == 0) s_red[wave] = before;
@@ -231,16 +239,21 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
   const int end = min(start + size, p.m);
   const int esz = p.out_dtype == TKX_F32 ? 4 : 2;
 
-  if (last_group) {
-    // Rows past the last group belong to no group: zero this workgroup's columns of them.
+  if (last_group || first_of_shard) {
+    // Rows past the last group, and with a group offset the rows before the first, belong to no
+    // group of this call: zero this workgroup's columns of them.
     const int ncol = min(BN, p.n - col0);
     const int pieces = ncol * esz / 16;  // 16-byte pieces per row
     unsigned char* c = reinterpret_cast<unsigned char*>(p.out);
     const i32x4 z = {0, 0, 0, 0};
-    for (int idx = tid; idx < (p.m - end) * pieces; idx += kDecThreads) {
-      const int r = end + idx / pieces, ch = idx % pieces;
-      *reinterpret_cast<i32x4*>(c + ((int64_t)r * p.n + col0) * esz + ch * 16) = z;
-    }
+    auto zero_rows = [&](int r0, int r1) {
+      for (int idx = tid; idx < (r1 - r0) * pieces; idx += kDecThreads) {
+        const int r = r0 + idx / pieces, ch = idx % pieces;
+        *reinterpret_cast<i32x4*>(c + ((int64_t)r * p.n + col0) * esz + ch * 16) = z;
+      }
+    };
+    if (last_group) zero_rows(end, p.m);
+    if (first_of_shard) zero_rows(0, min(start, p.m));
   }
   if (end <= start) return;
 
@@ -393,8 +406,11 @@ bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k
 
 int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
                       int64_t m, int64_t k, int64_t n, int64_t G, int32_t rhs_dtype, int32_t out_dtype,
-                      int32_t activation, int32_t depth, int64_t scale_blocks, int32_t block_n, hipStream_t stream) {
+                      int32_t activation, int32_t depth, int64_t scale_blocks, int32_t block_n,
+                      const int32_t* group_offset, int64_t num_global, hipStream_t stream) {
   DecodeParams p;
+  p.group_offset = group_offset;
+  p.num_global = (int32_t)num_global;
   p.scale_blocks = (int32_t)scale_blocks;
   p.log2_block_rows = 0;
   for (int64_t rows = k / scale_blocks; rows > 1; rows >>= 1) ++p.log2_block_rows;

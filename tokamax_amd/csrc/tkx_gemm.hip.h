@@ -466,15 +466,18 @@ struct GemmKernel {
     if constexpr (MODE != kDrhs) {
       const int num_tasks = ws[0];
       if (b >= p.real_slots) {
-        // Tail duty: rows [total_rows, m_ext) belong to no group and are defined to be zero.
-        const int total_rows = min(ws[1], p.m_ext);
+        // Tail duty: rows [total_rows, m_ext), and with a group offset the rows before the first
+        // group, belong to no group of this call and are defined to be zero.
+        const int total_rows = min(ws[1], p.m_ext), lead_rows = min(ws[2], p.m_ext);
         const int64_t esz = p.out_dtype == TKX_F32 ? 4 : 2;
         const int64_t lo = (int64_t)total_rows * p.ldc * esz, hi = (int64_t)p.m_ext * p.ldc * esz;
         unsigned char* c = reinterpret_cast<unsigned char*>(p.C);
         const int64_t nzb = gridDim.x - p.real_slots;
         const i32x4 z = {0, 0, 0, 0};
-        for (int64_t o = lo + ((int64_t)(b - p.real_slots) * THREADS + tid) * 16; o < hi; o += nzb * THREADS * 16)
-          *reinterpret_cast<i32x4*>(c + o) = z;
+        const int64_t first = ((int64_t)(b - p.real_slots) * THREADS + tid) * 16;
+        for (int64_t o = lo + first; o < hi; o += nzb * THREADS * 16) *reinterpret_cast<i32x4*>(c + o) = z;
+        const int64_t lead_bytes = (int64_t)lead_rows * p.ldc * esz;
+        for (int64_t o = first; o < lead_bytes; o += nzb * THREADS * 16) *reinterpret_cast<i32x4*>(c + o) = z;
         return;
       }
       // XCD-aware order: consecutive workgroup ids land on different XCDs (id % 8). The tile list is

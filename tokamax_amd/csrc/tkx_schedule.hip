@@ -33,7 +33,12 @@ __device__ inline int32_t block_exclusive_scan(int32_t v, int32_t* buf, int32_t*
   return incl - v;
 }
 
+// `group_offset` (device pointer to one int32, or null for 0) and `num_global`: group_sizes has
+// num_global entries and the G groups scheduled here are its entries [offset, offset + G) (the
+// expert-parallel shard of experimental/gmm_v2/gmm_v2_test.py:44-101); entries outside
+// [0, num_global) count as empty, and the rows of the groups before `offset` are skipped.
 __global__ __launch_bounds__(kThreads) void schedule_kernel(const int32_t* __restrict__ group_sizes, int32_t G,
+                                                             const int32_t* __restrict__ group_offset, int32_t num_global,
                                                              int32_t tile, int32_t tid_size, int32_t align_tile,
                                                              int32_t span_width, int32_t* __restrict__ ws,
                                                              int64_t off_offsets, int64_t off_gid, int64_t off_bstart,
@@ -47,21 +52,34 @@ __global__ __launch_bounds__(kThreads) void schedule_kernel(const int32_t* __res
   const int per = (G + kThreads - 1) / kThreads;
   const int lo = min(t * per, G), hi = min(lo + per, G);
 
-  // pass 1: group starts
+  const int32_t goff = group_offset != nullptr ? group_offset[0] : 0;
+  auto size_of = [&](int g) -> int32_t {
+    const int64_t j = (int64_t)goff + g;
+    return j >= 0 && j < num_global ? max(group_sizes[j], 0) : 0;
+  };
+  // pass 0: rows of the groups before the first one of this shard
   int32_t local = 0;
-  for (int g = lo; g < hi; ++g) local += max(group_sizes[g], 0);
+  const int32_t before = min(max(goff, 0), num_global);
+  for (int j = t; j < before; j += kThreads) local += max(group_sizes[j], 0);
+  int32_t lead;
+  block_exclusive_scan(local, scan_buf, &lead);
+
+  // pass 1: group starts
+  local = 0;
+  for (int g = lo; g < hi; ++g) local += size_of(g);
   int32_t total_rows;
-  int32_t run = block_exclusive_scan(local, scan_buf, &total_rows);
+  int32_t run = lead + block_exclusive_scan(local, scan_buf, &total_rows);
+  total_rows += lead;
   for (int g = lo; g < hi; ++g) {
     starts[g] = run;
-    run += max(group_sizes[g], 0);
+    run += size_of(g);
   }
   if (t == 0) starts[G] = total_rows;
   __syncthreads();
 
   // pass 2: blocks per group -> first task of each group
   auto blocks_of = [&](int g) -> int32_t {
-    int32_t sz = max(group_sizes[g], 0);
+    int32_t sz = size_of(g);
     int32_t aligned = (starts[g] / align_tile) * align_tile;
     return sz == 0 ? 0 : (starts[g] + sz - aligned + tile - 1) / tile;
   };
@@ -77,6 +95,7 @@ __global__ __launch_bounds__(kThreads) void schedule_kernel(const int32_t* __res
     start_tasks[G] = num_tasks;
     ws[0] = num_tasks;
     ws[1] = total_rows;
+    ws[2] = lead;
   }
   __syncthreads();
 
@@ -90,7 +109,7 @@ __global__ __launch_bounds__(kThreads) void schedule_kernel(const int32_t* __res
       if (start_tasks[mid + 1] <= task) l = mid + 1; else h = mid;
     }
     const int g = l;
-    const int32_t sz = max(group_sizes[g], 0);
+    const int32_t sz = size_of(g);
     const int32_t aligned = (starts[g] / align_tile) * align_tile;
     const int32_t end = starts[g] + sz;
     const int32_t bs = aligned + tile * (task - start_tasks[g]);
@@ -126,12 +145,14 @@ __global__ __launch_bounds__(kThreads) void schedule_kernel(const int32_t* __res
 
 }  // namespace
 
-int32_t launch_schedule(const int32_t* group_sizes, int64_t G, int64_t m, int32_t block_m, int32_t align_tile,
-                        int32_t span_width, int32_t* ws, const WsLayout& L, hipStream_t stream) {
+int32_t launch_schedule(const int32_t* group_sizes, int64_t G, const int32_t* group_offset, int64_t num_global, int64_t m,
+                        int32_t block_m, int32_t align_tile, int32_t span_width, int32_t* ws, const WsLayout& L,
+                        hipStream_t stream) {
   (void)m;
   const size_t smem = sizeof(int32_t) * (size_t)(2 * kThreads + 2 * (G + 1));
   if (smem > 64 * 1024) return set_error(TKX_ERR_UNSUPPORTED, "num_groups=%lld too large for the scheduler", (long long)G);
-  schedule_kernel<<<1, kThreads, smem, stream>>>(group_sizes, (int32_t)G, block_m, L.tid_size, align_tile,
+  if (num_global < 0 || num_global > 0x7fffffffLL) return set_error(TKX_ERR_INVALID, "bad number of group sizes");
+  schedule_kernel<<<1, kThreads, smem, stream>>>(group_sizes, (int32_t)G, group_offset, (int32_t)num_global, block_m, L.tid_size, align_tile,
                                                 span_width < 1 ? 1 : span_width, ws, L.offsets, L.task[0], L.task[1],
                                                 L.task[2], L.task[3], L.task[4], L.task[5], L.task[6], L.task[7]);
   TKX_HIP_CHECK(hipGetLastError());

@@ -160,12 +160,25 @@ class HipRaggedDot(base.RaggedDot):
       rhs_quantization_dtype=None,
   ):
     del manual_axis_type  # sharding annotation only; no meaning on a single device
-    if (group_offset is not None or rhs_scale is not None or maybe_quantize_lhs or not zero_initialize
-        or lhs_quantization_dtype is not None or rhs_quantization_dtype is not None):
+    if (maybe_quantize_lhs or not zero_initialize or lhs_quantization_dtype is not None
+        or rhs_quantization_dtype is not None):
       raise NotImplementedError(
-          "The hip implementation does not support group_offset, rhs_scale, maybe_quantize_lhs,"
-          " zero_initialize, lhs_quantization_dtype, or rhs_quantization_dtype."
+          "The hip implementation does not support maybe_quantize_lhs, zero_initialize,"
+          " lhs_quantization_dtype, or rhs_quantization_dtype."
       )
+    if rhs_scale is not None:
+      # The raw-array form of quantised weights (experimental/gmm_v2/gmm_v2.py:1193-1199): rhs holds the
+      # quantised values and rhs_scale is [g, k-blocks, 1, n]; the result defaults to lhs.dtype (:1369-1370).
+      if isinstance(lhs, (QArray, AsQArray)) or isinstance(rhs, (QArray, AsQArray)):
+        raise NotImplementedError("rhs_scale comes with raw arrays, not QArrays.")
+      g, k, n = rhs.shape
+      if rhs_scale.dim() != 4 or tuple(rhs_scale.shape[::2]) != (g, 1) or rhs_scale.shape[3] != n:
+        raise NotImplementedError(f"rhs_scale must have shape [g, k-blocks, 1, n], got {tuple(rhs_scale.shape)}")
+      rhs = QArray(rhs, rhs_scale.reshape(g, rhs_scale.shape[1], n))
+      if preferred_element_type is None:
+        preferred_element_type = lhs.dtype
+    if group_offset is not None and ragged_dot_dimension_numbers != base.DEFAULT_RAGGED_DOT_DIM_NUMS:
+      raise NotImplementedError("group_offset needs the default dimension numbers.")
     # rhs_bias and fuse_gateup_activation (base.py:205-217) are fused into the forward kernel's epilogue.
     gateup = None
     if fuse_gateup_activation is not None:
@@ -236,6 +249,12 @@ class HipRaggedDot(base.RaggedDot):
     if not isinstance(gs, torch.Tensor):
       gs = torch.as_tensor(gs, dtype=torch.int32, device=device)
 
+    if group_offset is not None:
+      # One int32 on the device: the kernels read it there, so nothing synchronises with the host.
+      group_offset = torch.as_tensor(group_offset, device=device).to(torch.int32).reshape(-1)
+      if group_offset.numel() != 1:
+        raise ValueError("group_offset must hold one element")
+
     kcfg = config.to_kernel_config()
     fused = None
     if activation is not None and not return_residuals:
@@ -252,7 +271,8 @@ class HipRaggedDot(base.RaggedDot):
       # act(gate) * up in the kernel; an `activation` on top of that is applied to the f32 result.
       kernel_out = torch.float32 if activation is not None else preferred_element_type
       dot_out = hip_ops.ragged_dot_fwd(lhs_v, rhs_v, gs, config=kcfg, out_dtype=kernel_out, lhs_scale=lhs_scale,
-                                       rhs_scale=rhs_scale_, rhs_bias=rhs_bias, activation=gateup, gateup=True)
+                                       rhs_scale=rhs_scale_, rhs_bias=rhs_bias, activation=gateup, gateup=True,
+                                       group_offset=group_offset)
       if activation is not None:
         dot_out = activation(dot_out).to(preferred_element_type)
       return dot_out, None
@@ -267,7 +287,8 @@ class HipRaggedDot(base.RaggedDot):
       unfused = activation is not None and not return_residuals and fused is None
       kernel_out = torch.float32 if unfused else preferred_element_type
       dot_out = hip_ops.ragged_dot_fwd(lhs_v, rhs_v, gs, config=kcfg, out_dtype=kernel_out, trans_rhs=(mode == 1),
-                                       lhs_scale=lhs_scale, rhs_scale=rhs_scale_, activation=fused, rhs_bias=rhs_bias)
+                                       lhs_scale=lhs_scale, rhs_scale=rhs_scale_, activation=fused, rhs_bias=rhs_bias,
+                                       group_offset=group_offset)
       if unfused:
         dot_out = activation(dot_out).to(preferred_element_type)
 
@@ -299,7 +320,9 @@ class HipRaggedDot(base.RaggedDot):
       num_groups = rhs_shape[0]
       rows, cols, contraction = lhs_shape[0], rhs_shape[2], rhs_shape[1]
     lhs_dt, rhs_dt = _dtype_of(lhs), _dtype_of(rhs)
-    if isinstance(rhs, QArray) and (_scale_blocks_along_k(rhs) or 1) > 1:
+    raw_scale = ba.kwargs.get("rhs_scale")
+    if ((isinstance(rhs, QArray) and (_scale_blocks_along_k(rhs) or 1) > 1)
+        or (raw_scale is not None and len(raw_scale.shape) == 4 and raw_scale.shape[1] > 1)):
       rhs_dt = torch.bfloat16  # sub-channel scales: `_fwd` widens the weights to bf16 first
     if (ba.kwargs.get("precision") == precision_lib.DotAlgorithmPreset.BF16_BF16_F32
         and not isinstance(lhs, (QArray, AsQArray)) and not isinstance(rhs, (QArray, AsQArray))):

@@ -121,14 +121,17 @@ def schedule(group_sizes: torch.Tensor, m: int, block_m: int, align_tile: int = 
 
 def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: torch.dtype, trans_rhs: bool = False,
                    lhs_scale=None, rhs_scale=None, activation: str | None = None, rhs_bias=None,
-                   gateup: bool = False, workspace_out: list | None = None) -> torch.Tensor:
+                   gateup: bool = False, group_offset=None, workspace_out: list | None = None) -> torch.Tensor:
   """out[m,n] = lhs[m,k] . rhs[g,k,n]   (trans_rhs: out[m,k] = lhs[m,n] . rhs[g,k,n]^T).
 
   `rhs_scale` is [g,n] / [g,1,n], or [g,blocks,n] with `blocks` scale blocks along k (streaming small-m
   kernel only). `rhs_bias` ([g,n] or [g,1,n]) is added to the scaled result before the activation. `gateup`: rhs
   columns are [gate | up] and out[m,n/2] = activation(gate part) * (up part) (base.py:211-217).
+  `group_offset` (device int32 tensor of one element): `group_sizes` covers every group of the job, rhs holds the
+  groups [offset, offset + g) of them, and the rows of all other groups come out zero (the call of one
+  expert-parallel shard, experimental/gmm_v2/gmm_v2_test.py:44-101).
   `workspace_out`, if given, receives the int32 workspace the call filled (schedule arrays included)."""
-  _require_cuda(lhs, rhs, group_sizes, lhs_scale, rhs_scale, rhs_bias)
+  _require_cuda(lhs, rhs, group_sizes, lhs_scale, rhs_scale, rhs_bias, group_offset)
   lib = _lib.load()
   if lhs.dim() != 2 or rhs.dim() != 3:
     raise ValueError(f"expected lhs [m,k] and rhs [g,k,n], got {tuple(lhs.shape)} and {tuple(rhs.shape)}")
@@ -136,8 +139,17 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
   gs = _group_sizes_i32(group_sizes)
   G, k, n = rhs.shape
   m = lhs.shape[0]
-  if gs.numel() != G:
-    raise ValueError(f"group_sizes has {gs.numel()} entries, rhs has {G} groups")
+  if group_offset is None:
+    if gs.numel() != G:
+      raise ValueError(f"group_sizes has {gs.numel()} entries, rhs has {G} groups")
+  else:
+    if trans_rhs:
+      raise NotImplementedError("group_offset needs the default dimension numbers")
+    if group_offset.numel() != 1 or gs.numel() < 1:
+      raise ValueError("group_offset must hold one element and group_sizes at least one")
+    if group_offset.dtype != torch.int32:
+      group_offset = group_offset.to(torch.int32)
+    group_offset = group_offset.contiguous()
   if lhs.shape[1] != (n if trans_rhs else k):
     raise ValueError("contraction sizes of lhs and rhs differ")
   if (rhs_bias is not None or gateup) and trans_rhs:
@@ -164,7 +176,7 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
   ws = workspace(m, G, config.block_m, lhs.device)
   cfg = config.to_c()
   with _on_device(lhs.device):
-    if rhs_bias is None and not gateup and scale_blocks == 1:
+    if rhs_bias is None and not gateup and scale_blocks == 1 and group_offset is None:
       st = lib.tkx_ragged_dot_fwd(
           _ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(out), _ptr(ws), m, k, n, G,
           dtype_code(lhs.dtype), dtype_code(rhs.dtype), dtype_code(out_dtype),
@@ -172,9 +184,9 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
           ctypes.byref(cfg), _stream(lhs.device))
     else:
       st = lib.tkx_ragged_dot_fwd_fused(
-          _ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(rhs_bias), _ptr(out), _ptr(ws), m, k,
-          n, G, scale_blocks, dtype_code(lhs.dtype), dtype_code(rhs.dtype), dtype_code(out_dtype), _lib.ACTIVATIONS[activation],
-          1 if gateup else 0, ctypes.byref(cfg), _stream(lhs.device))
+          _ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(group_offset), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(rhs_bias), _ptr(out),
+          _ptr(ws), m, k, n, G, gs.numel(), scale_blocks, dtype_code(lhs.dtype), dtype_code(rhs.dtype),
+          dtype_code(out_dtype), _lib.ACTIVATIONS[activation], 1 if gateup else 0, ctypes.byref(cfg), _stream(lhs.device))
   _lib.check(st)
   if workspace_out is not None:
     workspace_out.append(ws)
