@@ -19,8 +19,8 @@
  *                               activate(tmp[:, :n]) * tmp[:, n:] with tmp = ragged_dot(lhs, [gate, up])
  *   tkx_ragged_dot_drhs         RAGGED_CONTRACTING_DOT_DIM_NUMS (base.py:50-54), the drhs of
  *                               base.py:448-461; kernel counterpart pallas_mosaic_gpu_kernel_sm90.py:184-285
- *   tkx_dequantize_weights      quantization.py:80-83 (as_array: qvalue * scale with tile-repeat
- *                               broadcasting) for int8 weights with sub-channel scales
+ *   tkx_dequantize_weights,     quantization.py:80-83 (as_array: qvalue * scale with tile-repeat
+ *   tkx_dequantize              broadcasting) for int8 / fp8 operands with sub-channel scales
  *   TkxConfig                   pallas_mosaic_gpu_common.py:45-73 (Config)
  */
 #ifndef TKX_RAGGED_DOT_H_
@@ -154,12 +154,22 @@ int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* gr
 /* Weights with several scale blocks along k (the scale tile (1, t_k, 1) with t_k < k of
  * pallas_mosaic_gpu_kernel_sm90_quant.py:91-97; quantization.py:80-83 for the dequantisation):
  *   out[g, kk, c] = qvalue[g, kk, c] * scale[g, kk / scale_block_k, c]
- * qvalue int8 [G,k,n], scale f32 [G, k / scale_block_k, n], out bf16 [G,k,n] (caller-owned); the
- * result feeds the bf16 kernels. (scale_block_k == k needs no such pass: tkx_ragged_dot_fwd applies
+ * qvalue int8 or fp8 (e4m3fn) [G,k,n], scale f32 [G, k / scale_block_k, n], out bf16 [G,k,n] (caller-owned);
+ * the result feeds the bf16 kernels. (scale_block_k == k needs no such pass: tkx_ragged_dot_fwd applies
  * one scale per (group, column) in its epilogue.) One streaming kernel on `stream`. */
 int32_t tkx_dequantize_weights(const void* qvalue, const float* scale, void* out, int64_t num_groups, int64_t k,
                                int64_t n, int64_t scale_block_k, int32_t q_dtype, int32_t out_dtype,
                                tkx_stream_t stream);
+
+/* The same pass for any row-major quantised operand with block scales (quantization.py:80-83; the
+ * k-subchannel scales xs[row, k_sub] and ws[g, k_sub, n] of pallas_mosaic_gpu_kernel_sm100_i8_quant.py:51-102):
+ *   out[r, c] = qvalue[r, c] * scale[r / scale_block_rows, c / scale_block_cols]
+ * qvalue int8 or fp8 (e4m3fn) [rows, cols], scale f32 [rows / scale_block_rows, cols / scale_block_cols], out bf16.
+ * An lhs [m,k] with scale [m, k/t] is (rows, cols, blocks) = (m, k, 1 x t); weights [G,k,n] with scale
+ * [G, k/t_k, n/t_n] are (G*k, n, t_k x t_n). cols % 16 == 0; scale_block_cols is 1 or a multiple of 16. */
+int32_t tkx_dequantize(const void* qvalue, const float* scale, void* out, int64_t rows, int64_t cols,
+                       int64_t scale_block_rows, int64_t scale_block_cols, int32_t q_dtype, int32_t out_dtype,
+                       tkx_stream_t stream);
 
 /* The token permute / un-permute steps either side of the ragged dot in an MoE layer, one kernel:
  *   out[j, :] = sum over r < reduce_group_size of keep(g) * weights[g] * x[indices[g], :],  g = j * reduce_group_size + r

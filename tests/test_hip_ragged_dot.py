@@ -233,10 +233,12 @@ def test_vjp(m, k, n, activation, device):
   assert O.rel_l2(_np(b_t.grad), b_ref.grad.numpy()) <= 4e-3
 
 
-@pytest.mark.parametrize("b_tile_shape,supported", [((1, 256, 1), True), ((1, 16, 1), True), ((1, 1, 16), False)])
+@pytest.mark.parametrize("b_tile_shape,supported", [((1, 256, 1), True), ((1, 16, 1), True), ((1, 1, 16), True),
+                                                    ((1, 64, 32), True), ((1, 1, 8), False), ((2, 1, 1), False)])
 def test_quantized_int8_weights(b_tile_shape, supported, device):
-  """bf16 x int8: per-(group, column) scales run in the kernels' epilogue, sub-channel scales along k
-  through the widening pass; scale tiles along n are declined."""
+  """bf16 x int8: per-(group, column) scales run in the kernels' epilogue, sub-channel scales along k and
+  scale tiles of a multiple of 16 columns along n through the widening pass; narrower tiles along n and
+  scales shared between groups are declined."""
   G, m, k, n = 8, 512, 256, 512
   a, _, gs = _inputs("test_quantized", G, m, k, n, torch.bfloat16, device, random_groups=True)
   rng = np.random.default_rng(11)
@@ -646,6 +648,71 @@ def test_raw_rhs_scale_argument(device):
            3e-3)
   with pytest.raises(NotImplementedError):
     op(lhs, q, group_sizes=gst, rhs_scale=scale)  # not [g, blocks, 1, n]
+  # permissions the kernels do not use: lhs stays unquantised, rows of no group are zeroed anyway
+  again = op(lhs, q, group_sizes=gst, rhs_scale=scale.reshape(G, blocks, 1, n), maybe_quantize_lhs=True, zero_initialize=False)
+  assert torch.equal(again, out)
+  with pytest.raises(NotImplementedError):
+    op(lhs, q, group_sizes=gst, rhs_scale=scale.reshape(G, blocks, 1, n), lhs_quantization_dtype=torch.int8)
+
+
+@pytest.mark.parametrize("qdtype", [torch.int8, torch.float8_e4m3fn])
+@pytest.mark.parametrize("rows,cols,t_r,t_c", [(96, 256, 1, 128), (96, 256, 1, 256), (512, 128, 64, 1), (512, 256, 128, 128),
+                                               (40, 48, 8, 16)])
+def test_dequantize_kernel_bit_exact(rows, cols, t_r, t_c, qdtype, device):
+  """`tkx_dequantize`: int8 / fp8 values times block scales, rounded to bf16 -- bit for bit the oracle's
+  dequantisation (quantization.py:80-83) rounded to bf16 (one f32 multiply, one rounding)."""
+  rng = np.random.default_rng(rows + t_c)
+  if qdtype == torch.int8:
+    q = torch.tensor(rng.integers(-128, 128, (rows, cols)).astype(np.int8), device=device)
+    qf = q.cpu().numpy()
+  else:
+    q = torch.tensor(rng.integers(0, 256, (rows, cols)).astype(np.uint8), device=device)
+    q = torch.where((q & 0x7f) == 0x7f, torch.zeros_like(q), q).view(torch.float8_e4m3fn)  # no NaN codes
+    qf = O.e4m3fn_decode(q.view(torch.uint8).cpu().numpy())
+  scale = torch.tensor(rng.uniform(0.01, 2.0, (rows // t_r, cols // t_c)).astype(np.float32), device=device)
+  got = hip_ops.dequantize(q, scale)
+  want = O.round_to_bf16(O.dequantize(qf, _np(scale)))
+  np.testing.assert_array_equal(_np(got), want)
+  # weights [g, k, n] with scale [g, k/t_k, n/t_n] are the same pass over g * k rows
+  if rows % (2 * t_r) == 0:
+    got3 = hip_ops.dequantize(q.view(2, rows // 2, cols), scale.view(2, -1, cols // t_c))
+    np.testing.assert_array_equal(_np(got3).reshape(rows, cols), want)
+
+
+@pytest.mark.parametrize("case", ["fp8_blocks_128", "fp8_row_x_k_blocks", "int8_k_sub", "int8_row_col"])
+def test_k_subchannel_scales_through_widening(case, device):
+  """Scales that change along the contraction on both operands -- the fp8 recipe with [m, k/128] and
+  [g, k/128, n/128] scales, and the int8 activation form acc += (x_q . w_q) xs[row, k_sub] ws[g, k_sub, n]
+  (pallas_mosaic_gpu_kernel_sm100_i8_quant.py:51-102) -- go through the widening pass and the bf16 (or
+  bf16 x int8) kernels; the oracle contracts the dequantised operands in f64."""
+  rng = np.random.default_rng(len(case))
+  G, m, k, n = 4, 300, 512, 256
+  gs = np.array([100, 0, 80, 110], np.int32)
+  gst = torch.tensor(gs, device=device)
+  def quantised(shape, qdtype, scale_shape, spread):
+    if qdtype == torch.int8:
+      q = torch.tensor(rng.integers(-127, 128, shape).astype(np.int8), device=device)
+      qf = q.cpu().numpy().astype(np.float64)
+    else:
+      q = torch.tensor(rng.normal(0, 1.0, shape).astype(np.float32), device=device).to(torch.float8_e4m3fn)
+      qf = O.e4m3fn_decode(q.view(torch.uint8).cpu().numpy()).astype(np.float64)
+    scale = torch.tensor((rng.uniform(0.5, 1.5, scale_shape) * spread).astype(np.float32), device=device)
+    return tokamax_amd.QArray(q, scale), O.dequantize(qf, _np(scale))
+  f8, i8 = torch.float8_e4m3fn, torch.int8
+  lhs_spec, rhs_spec = {
+      "fp8_blocks_128": (((m, k), f8, (m, k // 128), 1.0), ((G, k, n), f8, (G, k // 128, n // 128), k ** -0.5)),
+      "fp8_row_x_k_blocks": (((m, k), f8, (m, 1), 1.0), ((G, k, n), f8, (G, k // 128, n), k ** -0.5)),
+      "int8_k_sub": (((m, k), i8, (m, k // 64), 1 / 127), ((G, k, n), i8, (G, k // 64, n), k ** -0.5 / 127)),
+      "int8_row_col": (((m, k), i8, (m, 1), 1 / 127), ((G, k, n), i8, (G, 1, n), k ** -0.5 / 127)),
+  }[case]
+  lhs, lhs_f = quantised(*lhs_spec)
+  rhs, rhs_f = quantised(*rhs_spec)
+  out = tokamax_amd.ragged_dot(lhs, rhs, gst, preferred_element_type=torch.float32)
+  want = O.ragged_dot(lhs_f, rhs_f, gs, acc_dtype=np.float64, out_dtype="f64")
+  count = int(gs.sum())
+  _check(out, want, TOL["fp8"], rows=count)
+  assert O.rel_l2(_np(out)[:count], want[:count]) < 6e-3  # two operands rounded to bf16, f32 accumulation
+  assert torch.count_nonzero(out[count:]) == 0
 
 
 @pytest.mark.parametrize("m,blocks", [(300, 4), (24, 8), (1100, 2)])

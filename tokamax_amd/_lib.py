@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "tkx_ragged_dot_fwd_fused",
     "tkx_ragged_dot_drhs",
     "tkx_dequantize_weights",
+    "tkx_dequantize",
     "tkx_ragged_gather_rows",
     "tkx_ragged_dot_num_variants",
     "tkx_ragged_dot_variant",
@@ -82,6 +83,8 @@ def _declare(lib):
   lib.tkx_ragged_dot_drhs.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32, cfgp, vp]
   lib.tkx_dequantize_weights.restype = i32
   lib.tkx_dequantize_weights.argtypes = [vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
+  lib.tkx_dequantize.restype = i32
+  lib.tkx_dequantize.argtypes = [vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
   lib.tkx_ragged_gather_rows.restype = i32
   lib.tkx_ragged_gather_rows.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]
   lib.tkx_ragged_dot_num_variants.restype = i32

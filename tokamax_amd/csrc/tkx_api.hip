@@ -339,14 +339,32 @@ int32_t tkx_dequantize_weights(const void* qvalue, const float* scale, void* out
   if (num_groups < 1 || k < 1 || n < 1 || scale_block_k < 1)
     return set_error(TKX_ERR_INVALID, "bad sizes G=%lld k=%lld n=%lld block=%lld", (long long)num_groups, (long long)k,
                      (long long)n, (long long)scale_block_k);
-  if (q_dtype != TKX_I8 || out_dtype != TKX_BF16)
-    return set_error(TKX_ERR_UNSUPPORTED, "dequantisation is int8 -> bf16 only (got %d -> %d)", q_dtype, out_dtype);
   if (k % scale_block_k != 0) return set_error(TKX_ERR_INVALID, "k=%lld is not a multiple of the scale block %lld",
                                                (long long)k, (long long)scale_block_k);
-  if (n % 16 != 0) return set_error(TKX_ERR_UNSUPPORTED, "n must be a multiple of 16");
-  if (((uintptr_t)qvalue | (uintptr_t)scale | (uintptr_t)out) % 16 != 0)
+  // Weights [G, k, n] as G * k rows: a block of scale_block_k rows never straddles two groups.
+  return tkx_dequantize(qvalue, scale, out, num_groups * k, n, scale_block_k, 1, q_dtype, out_dtype, stream);
+}
+
+int32_t tkx_dequantize(const void* qvalue, const float* scale, void* out, int64_t rows, int64_t cols,
+                       int64_t scale_block_rows, int64_t scale_block_cols, int32_t q_dtype, int32_t out_dtype,
+                       tkx_stream_t stream) {
+  if (!qvalue || !scale || !out) return set_error(TKX_ERR_INVALID, "null pointer argument");
+  if (rows < 1 || cols < 1 || scale_block_rows < 1 || scale_block_cols < 1)
+    return set_error(TKX_ERR_INVALID, "bad sizes rows=%lld cols=%lld block=%lldx%lld", (long long)rows, (long long)cols,
+                     (long long)scale_block_rows, (long long)scale_block_cols);
+  if ((q_dtype != TKX_I8 && q_dtype != TKX_F8E4M3FN) || out_dtype != TKX_BF16)
+    return set_error(TKX_ERR_UNSUPPORTED, "dequantisation is int8 or fp8 -> bf16 only (got %d -> %d)", q_dtype, out_dtype);
+  if (rows % scale_block_rows != 0 || cols % scale_block_cols != 0)
+    return set_error(TKX_ERR_INVALID, "scale blocks %lldx%lld do not tile %lldx%lld", (long long)scale_block_rows,
+                     (long long)scale_block_cols, (long long)rows, (long long)cols);
+  if (cols % 16 != 0 || cols > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "cols must be a multiple of 16");
+  if (scale_block_cols != 1 && scale_block_cols % 16 != 0)
+    return set_error(TKX_ERR_UNSUPPORTED, "scale blocks along the columns must be 1 or a multiple of 16 wide");
+  if (scale_block_rows > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "scale block too tall");
+  if (((uintptr_t)qvalue | (uintptr_t)out) % 16 != 0 || (uintptr_t)scale % (scale_block_cols == 1 ? 16 : 4) != 0)
     return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
-  return launch_dequant_i8(qvalue, scale, out, num_groups, k, n, scale_block_k, static_cast<hipStream_t>(stream));
+  return launch_dequant(qvalue, scale, out, rows, cols, scale_block_rows, scale_block_cols, q_dtype,
+                        static_cast<hipStream_t>(stream));
 }
 
 int32_t tkx_ragged_gather_rows(const void* x, const int32_t* indices, const float* weights, const uint8_t* valid,

@@ -108,8 +108,9 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
                       const int32_t* group_offset, int64_t num_global, hipStream_t stream);
 
 // ---- dequantisation of int8 weights with sub-channel scales to bf16 ------------------------------
-int32_t launch_dequant_i8(const void* q, const float* scale, void* out, int64_t G, int64_t k, int64_t n, int64_t t_k,
-                          hipStream_t stream);
+// out[r, c] = q[r, c] * scale[r / t_r, c / t_c]; q int8 or fp8 (e4m3fn), out bf16; t_c is 1 or a multiple of 16.
+int32_t launch_dequant(const void* q, const float* scale, void* out, int64_t rows, int64_t n, int64_t t_r, int64_t t_c,
+                       int32_t q_dtype, hipStream_t stream);
 
 // ---- row gather with optional mask, weight and reduction (token permute / un-permute) -------------
 int32_t launch_gather_rows(const void* x, const int32_t* indices, const float* weights, const unsigned char* valid,

@@ -1,10 +1,12 @@
-// Weight dequantisation with sub-channel scales: out[g, kk, c] = q[g, kk, c] * scale[g, kk / t_k, c].
+// Dequantisation with block scales: out[r, c] = q[r, c] * scale[r / t_r, c / t_c], q int8 or fp8
+// (e4m3fn), out bf16.
 //
-// The tiled kernels apply one scale per (group, column) in their epilogue, which covers scales that
-// span the whole contraction (t_k == k). Weights with several scale blocks along k (t_k < k, scale
-// [G, k / t_k, n]) are widened to bf16 by this streaming pass and then take the bf16 kernels; the
+// The tiled kernels apply one scale per lhs row and one per (group, column) in their epilogue, which
+// covers scales that span the whole contraction. Operands whose scales change along the contraction
+// (weights [G, k, n] with scale [G, k / t_k, n / t_n], viewed as G * k rows; an lhs [m, k] with scale
+// [m, k / t]) are widened to bf16 by this streaming pass and then take the bf16 kernels; the
 // reference's "xla" path does the same as a separate elementwise step (base.py:332). The pass is
-// bound by HBM: it reads 1 byte and writes 2 per weight.
+// bound by HBM: it reads 1 byte and writes 2 per element.
 #include "tkx_common.h"
 #include "tkx_gemm.hip.h"
 
@@ -13,31 +15,48 @@ namespace {
 
 constexpr int kDqThreads = 256;
 
-// One thread converts 16 consecutive columns of one k-row: a 16-byte load of int8, two 16-byte
-// scale loads per 8 columns (L2-resident: a scale row serves t_k weight rows), two 16-byte stores.
-__global__ __launch_bounds__(kDqThreads) void dequant_i8_kernel(const signed char* __restrict__ q,
-                                                               const float* __restrict__ scale, __bf16* __restrict__ out,
-                                                               int64_t rows /* G * k */, int32_t k, int32_t n, int32_t t_k) {
+// Byte B of a dword as f32: a sign-extended int8, or an OCP e4m3fn value (the hardware conversion).
+template <int EQ, int B>
+__device__ __forceinline__ float widen_byte(int w) {
+  if constexpr (EQ == kEI8) return (float)(signed char)((w >> (8 * B)) & 0xff);
+  else return __builtin_amdgcn_cvt_f32_fp8(w, B);
+}
+
+// One thread converts 16 consecutive columns of one row: a 16-byte load, the scales of those columns
+// (four 16-byte loads when every column has its own, t_c == 1; one value when a scale block spans
+// them, t_c % 16 == 0; L2-resident either way: a scale row serves t_r rows), two 16-byte stores.
+template <int EQ>
+__global__ __launch_bounds__(kDqThreads) void dequant_kernel(const unsigned char* __restrict__ q,
+                                                            const float* __restrict__ scale, __bf16* __restrict__ out,
+                                                            int64_t rows, int32_t n, int32_t t_r, int32_t t_c) {
   const int chunks = n / 16;  // n % 16 == 0 (checked on the host)
   const int64_t total = rows * chunks;
-  const int kb_per_group = k / t_k;
+  const int scale_cols = n / t_c;
   for (int64_t idx = (int64_t)blockIdx.x * kDqThreads + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * kDqThreads) {
     const int64_t row = idx / chunks;
     const int c0 = (int)(idx - row * chunks) * 16;
-    const int64_t g = row / k;
-    const int kk = (int)(row - g * k);
     const i32x4 w = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(q + row * n + c0));
-    const f32x4* s = reinterpret_cast<const f32x4*>(scale + ((int64_t)g * kb_per_group + kk / t_k) * n + c0);
+    const float* srow = scale + (row / t_r) * scale_cols;
+    f32x4 sc[4];
+    if (t_c == 1) {
+#pragma unroll
+      for (int d = 0; d < 4; ++d) sc[d] = *reinterpret_cast<const f32x4*>(srow + c0 + 4 * d);
+    } else {
+      const float one = srow[c0 / t_c];
+#pragma unroll
+      for (int d = 0; d < 4; ++d) sc[d] = (f32x4){one, one, one, one};
+    }
     bf16x8 lo, hi;
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-      const f32x4 sc = s[d];
+      const int word = w[d];
+      const float v[4] = {widen_byte<EQ, 0>(word) * sc[d][0], widen_byte<EQ, 1>(word) * sc[d][1],
+                          widen_byte<EQ, 2>(word) * sc[d][2], widen_byte<EQ, 3>(word) * sc[d][3]};
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
-        const float v = (float)(signed char)((w[d] >> (8 * b)) & 0xff) * sc[b];
         const int e = 4 * d + b;
-        if (e < 8) lo[e] = (__bf16)v;
-        else hi[e - 8] = (__bf16)v;
+        if (e < 8) lo[e] = (__bf16)v[b];
+        else hi[e - 8] = (__bf16)v[b];
       }
     }
     __bf16* o = out + row * n + c0;
@@ -48,13 +67,19 @@ __global__ __launch_bounds__(kDqThreads) void dequant_i8_kernel(const signed cha
 
 }  // namespace
 
-int32_t launch_dequant_i8(const void* q, const float* scale, void* out, int64_t G, int64_t k, int64_t n, int64_t t_k,
-                          hipStream_t stream) {
-  const int64_t total = G * k * (n / 16);
+int32_t launch_dequant(const void* q, const float* scale, void* out, int64_t rows, int64_t n, int64_t t_r, int64_t t_c,
+                       int32_t q_dtype, hipStream_t stream) {
+  const int64_t total = rows * (n / 16);
   int64_t grid = (total + kDqThreads - 1) / kDqThreads;
   if (grid > 256 * 16) grid = 256 * 16;  // 16 workgroups per CU, grid-stride beyond that
-  dequant_i8_kernel<<<dim3((unsigned)grid), dim3(kDqThreads), 0, stream>>>(
-      static_cast<const signed char*>(q), scale, static_cast<__bf16*>(out), G * k, (int32_t)k, (int32_t)n, (int32_t)t_k);
+  if (grid < 1) grid = 1;
+  const auto* qb = static_cast<const unsigned char*>(q);
+  if (q_dtype == TKX_I8)
+    dequant_kernel<kEI8><<<dim3((unsigned)grid), dim3(kDqThreads), 0, stream>>>(qb, scale, static_cast<__bf16*>(out), rows,
+                                                                               (int32_t)n, (int32_t)t_r, (int32_t)t_c);
+  else
+    dequant_kernel<kEF8><<<dim3((unsigned)grid), dim3(kDqThreads), 0, stream>>>(qb, scale, static_cast<__bf16*>(out), rows,
+                                                                               (int32_t)n, (int32_t)t_r, (int32_t)t_c);
   TKX_HIP_CHECK(hipGetLastError());
   return TKX_OK;
 }

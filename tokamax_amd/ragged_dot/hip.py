@@ -95,6 +95,56 @@ def _scale_blocks_along_k(q: QArray) -> int | None:
   return shape[1]
 
 
+def _rhs_scale_tiles(q: QArray) -> bool:
+  """Scale [g, k/t_k, n/t_n] with t_n a multiple of 16 (block scales along both k and n)."""
+  g, k, n = q.qvalue.shape
+  shape = tuple(q.scale.shape)
+  return (len(shape) == 3 and shape[0] == g and shape[1] >= 1 and shape[2] >= 1 and k % shape[1] == 0
+          and n % shape[2] == 0 and (n // shape[2]) % 16 == 0)
+
+
+def _lhs_scale_blocks(q: QArray) -> int | None:
+  """Number of scale blocks along k of a quantised lhs [m,k] (scale [m, blocks], blocks of a multiple of 16
+  columns), or None if the scale has another form."""
+  m, k = q.qvalue.shape
+  shape = tuple(q.scale.shape)
+  if shape == (m, 1):
+    return 1
+  if len(shape) != 2 or shape[0] != m or shape[1] < 1 or k % shape[1] != 0 or (k // shape[1]) % 16 != 0:
+    return None
+  return shape[1]
+
+
+def _widening_plan(lhs, rhs) -> tuple[bool, bool]:
+  """(widen lhs, widen rhs): which quantised operands are dequantised to bf16 before the kernels.
+
+  The kernels apply one scale per lhs row and one per (group, column) in their epilogue. Scales that change
+  along the contraction (the k-subchannel scales of pallas_mosaic_gpu_kernel_sm100_i8_quant.py:51-102, the scale
+  tile (1, t_k, 1) of pallas_mosaic_gpu_kernel_sm90_quant.py:91-97) or along n in blocks are multiplied in by a
+  widening pass instead; an fp8 operand whose partner was widened is widened too (there is no bf16 x fp8 kernel)."""
+  lhs_q, rhs_q = isinstance(lhs, QArray), isinstance(rhs, QArray)
+  widen_lhs = widen_rhs = False
+  if lhs_q:
+    blocks = _lhs_scale_blocks(lhs)
+    if blocks is None:
+      raise NotImplementedError(f"lhs scale must have shape [m,1] or [m, k/t] with 16 | t, got {tuple(lhs.scale.shape)}")
+    widen_lhs = blocks > 1 or _dtype_of(lhs) == torch.int8  # (no kernel contracts int8 activations directly)
+  if rhs_q:
+    blocks = _scale_blocks_along_k(rhs)
+    if blocks is None and not _rhs_scale_tiles(rhs):
+      raise NotImplementedError("rhs scale must have shape [g,1,n], [g,k/t_k,n] or [g,k/t_k,n/t_n] with 16 | t_n, got"
+                                f" {tuple(rhs.scale.shape)}")
+    widen_rhs = blocks is None or blocks > 1
+  eight_bit_float = lambda x: _dtype_of(x) == torch.float8_e4m3fn
+  if widen_rhs and lhs_q and eight_bit_float(lhs):
+    widen_lhs = True
+  if widen_lhs and rhs_q and eight_bit_float(rhs):
+    widen_rhs = True
+  if (widen_lhs and not rhs_q and eight_bit_float(rhs)) or (widen_rhs and not lhs_q and eight_bit_float(lhs)):
+    raise NotImplementedError("A raw fp8 operand cannot meet a widened (bf16) one.")
+  return widen_lhs, widen_rhs
+
+
 def _dtype_of(x) -> torch.dtype:
   return x.qtype if isinstance(x, (QArray, AsQArray)) else x.dtype
 
@@ -160,11 +210,14 @@ class HipRaggedDot(base.RaggedDot):
       rhs_quantization_dtype=None,
   ):
     del manual_axis_type  # sharding annotation only; no meaning on a single device
-    if (maybe_quantize_lhs or not zero_initialize or lhs_quantization_dtype is not None
-        or rhs_quantization_dtype is not None):
+    # `maybe_quantize_lhs` permits quantising lhs when rhs is quantised (base.py:208); the lhs stays as it is
+    # here (16-bit lhs x int8 weights, the more exact of the two choices). `zero_initialize=False` only
+    # releases the rows of no group from being zero (base.py:209-210); they are zeroed all the same.
+    del maybe_quantize_lhs, zero_initialize
+    if lhs_quantization_dtype is not None or rhs_quantization_dtype is not None:
       raise NotImplementedError(
-          "The hip implementation does not support maybe_quantize_lhs, zero_initialize,"
-          " lhs_quantization_dtype, or rhs_quantization_dtype."
+          "The hip implementation does not quantise inputs on the fly (lhs_quantization_dtype,"
+          " rhs_quantization_dtype)."
       )
     if rhs_scale is not None:
       # The raw-array form of quantised weights (experimental/gmm_v2/gmm_v2.py:1193-1199): rhs holds the
@@ -195,36 +248,36 @@ class HipRaggedDot(base.RaggedDot):
       raise NotImplementedError("Unsupported ragged dot dimension numbers.")
 
     lhs_scale = rhs_scale_ = None
+    for name, x in (("lhs", lhs), ("rhs", rhs)):
+      if isinstance(x, QArray) and (mode != 0 or x.zero_point is not None):
+        raise NotImplementedError(f"Quantised {name}: default dimension numbers without zero point only.")
+    widen_lhs, widen_rhs = _widening_plan(lhs, rhs)
     if isinstance(lhs, QArray):
-      if mode != 0 or lhs.zero_point is not None:
-        raise NotImplementedError("Quantised lhs: default dimension numbers without zero point only.")
-      m, k = lhs.qvalue.shape
-      if tuple(lhs.scale.shape) != (m, 1):
-        raise NotImplementedError(f"lhs scale must have shape [m,1] (one per row), got {tuple(lhs.scale.shape)}")
-      lhs_scale, lhs_v = lhs.scale, lhs.qvalue
+      if widen_lhs:
+        if lhs.qvalue.shape[1] % 16 != 0:
+          raise NotImplementedError("Widening a quantised lhs needs k % 16 == 0.")
+        lhs_v = hip_ops.dequantize(lhs.qvalue, lhs.scale)
+      else:
+        lhs_scale, lhs_v = lhs.scale, lhs.qvalue  # one scale per row: applied in the epilogue
     else:
       lhs_v = lhs
     if isinstance(rhs, QArray):
-      if mode != 0 or rhs.zero_point is not None:
-        raise NotImplementedError("Quantised rhs: default dimension numbers without zero point only.")
       g, k, n = rhs.qvalue.shape
-      blocks = _scale_blocks_along_k(rhs)
-      if blocks is None:
-        raise NotImplementedError(
-            f"rhs scale must have shape [g,1,n] or [g,k/t_k,n] (sub-channel along k), got {tuple(rhs.scale.shape)}")
-      if blocks == 1:
+      if not widen_rhs:
         rhs_scale_, rhs_v = rhs.scale, rhs.qvalue  # one scale per (group, column): applied in the epilogue
       else:
-        # Several scale blocks along k: widened to bf16 by a streaming pass, then the bf16 kernels.
-        if isinstance(lhs, QArray) or rhs.qvalue.dtype != torch.int8 or n % 16 != 0:
-          raise NotImplementedError("Sub-channel rhs scales: int8 weights, unquantised lhs and n % 16 == 0 only.")
-        rows = k // blocks
-        if (config.block_m == 16 and rows % 32 == 0 and rows & (rows - 1) == 0 and rhs_bias is None
-            and fuse_gateup_activation is None):
-          # The streaming small-m kernel scales the weights per k-block while it widens them.
+        # Scales that change along k (or in blocks along n): widened to bf16 by a streaming pass, then the
+        # bf16 kernels.
+        if n % 16 != 0:
+          raise NotImplementedError("Widening quantised weights needs n % 16 == 0.")
+        blocks = _scale_blocks_along_k(rhs)
+        rows = k // blocks if blocks else 0
+        if (blocks and config.block_m == 16 and rhs.qvalue.dtype == torch.int8 and not isinstance(lhs, QArray)
+            and rows % 32 == 0 and rows & (rows - 1) == 0 and rhs_bias is None and fuse_gateup_activation is None):
+          # The streaming small-m kernel scales int8 weights per k-block while it widens them.
           rhs_scale_, rhs_v = rhs.scale, rhs.qvalue
         else:
-          rhs_v = hip_ops.dequantize_weights(rhs.qvalue, rhs.scale)
+          rhs_v = hip_ops.dequantize(rhs.qvalue, rhs.scale)
     else:
       rhs_v = rhs
 
@@ -321,9 +374,12 @@ class HipRaggedDot(base.RaggedDot):
       rows, cols, contraction = lhs_shape[0], rhs_shape[2], rhs_shape[1]
     lhs_dt, rhs_dt = _dtype_of(lhs), _dtype_of(rhs)
     raw_scale = ba.kwargs.get("rhs_scale")
-    if ((isinstance(rhs, QArray) and (_scale_blocks_along_k(rhs) or 1) > 1)
-        or (raw_scale is not None and len(raw_scale.shape) == 4 and raw_scale.shape[1] > 1)):
+    if raw_scale is not None and len(raw_scale.shape) == 4 and raw_scale.shape[1] > 1:
       rhs_dt = torch.bfloat16  # sub-channel scales: `_fwd` widens the weights to bf16 first
+    if mode in (0, 3):
+      widen_lhs, widen_rhs = _widening_plan(lhs, rhs)
+      lhs_dt = torch.bfloat16 if widen_lhs else lhs_dt
+      rhs_dt = torch.bfloat16 if widen_rhs else rhs_dt
     if (ba.kwargs.get("precision") == precision_lib.DotAlgorithmPreset.BF16_BF16_F32
         and not isinstance(lhs, (QArray, AsQArray)) and not isinstance(rhs, (QArray, AsQArray))):
       lhs_dt = rhs_dt = torch.bfloat16  # `_fwd` casts both operands for this preset

@@ -212,6 +212,34 @@ def dequantize_weights(qvalue: torch.Tensor, scale: torch.Tensor) -> torch.Tenso
   return out
 
 
+def dequantize(qvalue: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+  """bf16 = qvalue * scale with each scale entry repeated over its tile (quantization.py:80-83).
+
+  qvalue int8 or fp8 (e4m3fn): [rows, cols] with scale [rows/t_r, cols/t_c], or weights [g,k,n] with scale
+  [g, k/t_k, n/t_n]; t_c / t_n is 1 or a multiple of 16."""
+  _require_cuda(qvalue, scale)
+  lib = _lib.load()
+  if qvalue.dtype not in (torch.int8, torch.float8_e4m3fn) or qvalue.dim() not in (2, 3) or scale.dim() != qvalue.dim():
+    raise NotImplementedError("expected an int8 or fp8 qvalue of 2 or 3 dimensions and a scale of as many")
+  if any(s < 1 or q % s for q, s in zip(qvalue.shape, scale.shape)):
+    raise NotImplementedError(f"scale shape {tuple(scale.shape)} does not tile qvalue {tuple(qvalue.shape)}")
+  if qvalue.dim() == 3:
+    if scale.shape[0] != qvalue.shape[0]:
+      raise NotImplementedError("one scale set per group expected")
+    rows, cols = qvalue.shape[0] * qvalue.shape[1], qvalue.shape[2]
+  else:
+    rows, cols = qvalue.shape
+  t_r, t_c = qvalue.shape[-2] // scale.shape[-2], qvalue.shape[-1] // scale.shape[-1]
+  qvalue = qvalue.contiguous()
+  scale = scale.to(torch.float32).contiguous()
+  out = torch.empty(qvalue.shape, dtype=torch.bfloat16, device=qvalue.device)
+  with _on_device(qvalue.device):
+    st = lib.tkx_dequantize(_ptr(qvalue), _ptr(scale), _ptr(out), rows, cols, t_r, t_c, dtype_code(qvalue.dtype),
+                            _lib.TKX_BF16, _stream(qvalue.device))
+  _lib.check(st)
+  return out
+
+
 def ragged_dot_drhs(lhs, dout, group_sizes, num_groups: int, *, config: KernelConfig,
                     out_dtype: torch.dtype) -> torch.Tensor:
   """out[g,k,n] = lhs[rows_g,k]^T . dout[rows_g,n]."""
