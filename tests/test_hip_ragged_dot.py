@@ -715,6 +715,28 @@ def test_k_subchannel_scales_through_widening(case, device):
   assert torch.count_nonzero(out[count:]) == 0
 
 
+def test_int4_values_in_int8_storage(device):
+  """fp8 x int4 with scale tile (1, 128, 1) (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:266-350) and bf16 x int4:
+  torch holds int4 values in int8 storage (qtype says int4); they run as int8."""
+  rng = np.random.default_rng(3)
+  G, m, k, n = 4, 300, 512, 256
+  gs = np.array([100, 0, 80, 110], np.int32)
+  gst = torch.tensor(gs, device=device)
+  q = torch.tensor(rng.integers(-8, 8, (G, k, n)).astype(np.int8), device=device)
+  scale = torch.tensor((rng.uniform(0.5, 1.5, (G, k // 128, n)) * k ** -0.5 / 7).astype(np.float32), device=device)
+  rhs = tokamax_amd.QArray(q, scale, qtype=torch.int4)
+  rhs_f = O.dequantize(q.cpu().numpy().astype(np.float64), _np(scale))
+  count = int(gs.sum())
+  a16 = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  out = tokamax_amd.ragged_dot(a16, rhs, gst, preferred_element_type=torch.float32)
+  _check(out, O.ragged_dot(_np(a16), rhs_f, gs, acc_dtype=np.float64, out_dtype="f64"), TOL["int8"], rows=count)
+  a8 = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.float8_e4m3fn)
+  a_scale = torch.tensor(rng.uniform(0.5, 1.5, (m, 1)).astype(np.float32), device=device)
+  lhs_f = O.dequantize(O.e4m3fn_decode(a8.view(torch.uint8).cpu().numpy()).astype(np.float64), _np(a_scale))
+  out = tokamax_amd.ragged_dot(tokamax_amd.QArray(a8, a_scale), rhs, gst, preferred_element_type=torch.float32)
+  _check(out, O.ragged_dot(lhs_f, rhs_f, gs, acc_dtype=np.float64, out_dtype="f64"), TOL["fp8"], rows=count)
+
+
 @pytest.mark.parametrize("m,blocks", [(300, 4), (24, 8), (1100, 2)])
 def test_int8_weights_with_sub_channel_scales(m, blocks, device):
   """Scale tile (1, t_k, 1) with t_k < k (pallas_mosaic_gpu_kernel_sm90_quant.py:91-97): the weights are

@@ -145,7 +145,14 @@ def _widening_plan(lhs, rhs) -> tuple[bool, bool]:
   return widen_lhs, widen_rhs
 
 
+_SUB_BYTE_INTS = tuple(getattr(torch, f"int{b}") for b in range(1, 8) if hasattr(torch, f"int{b}"))
+
+
 def _dtype_of(x) -> torch.dtype:
+  """The element type the kernels see. torch has no packed sub-byte tensors: a QArray whose qtype is int4
+  (or another sub-byte integer) holds its values in int8 storage and runs as int8."""
+  if isinstance(x, QArray) and x.qtype in _SUB_BYTE_INTS and x.qvalue.dtype == torch.int8:
+    return torch.int8
   return x.qtype if isinstance(x, (QArray, AsQArray)) else x.dtype
 
 
