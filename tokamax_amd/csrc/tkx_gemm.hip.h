@@ -82,11 +82,15 @@ __device__ __forceinline__ f32x16 mma_atom(const typename Mma<EA>::Frag& first, 
 
 // ---- LDS tile addressing ------------------------------------------------------------------------
 // Contraction-contiguous tile: [rows][ROW_BYTES], 16-byte chunks XOR-swizzled by the row so that the
-// 16/32 lanes of one ds_read_b128 phase touch distinct banks.
+// 16 lanes of one ds_read_b128 phase (16 consecutive rows, one chunk each: 256 bytes, every bank
+// once) touch distinct banks. A row covers CPR of the 16 chunk slots of a 256-byte bank line, so
+// the swizzle has to tell apart the 16 / CPR rows that start on the same slot: with 4 chunks per
+// row those are rows r, r + 4, r + 8, r + 12 (row bits 2 and 3), with 8 chunks per row r, r + 2, ...
 template <int ROW_BYTES>
 __device__ __forceinline__ int kc_swizzle(int row) {
   constexpr int CPR = ROW_BYTES / 16;
-  return ((row & 7) ^ ((row >> 3) & 1)) & (CPR - 1);
+  if constexpr (CPR == 4) return (row >> 2) & 3;
+  else return ((row & 7) ^ ((row >> 3) & 1)) & (CPR - 1);
 }
 template <int ROW_BYTES>
 __device__ __forceinline__ int kc_offset(int row, int chunk) {
