@@ -127,9 +127,10 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
  *   (TKX_ACT_SWIGLU_OAI and TKX_ACT_SILU_CLAMP need gateup = 1: TKX_ERR_INVALID otherwise).
  *   rhs_scale_blocks: rhs_scale is f32[G, rhs_scale_blocks, n], block b scaling the k rows
  *     [b * k/blocks, (b+1) * k/blocks) (scale tile (1, t_k, 1), pallas_mosaic_gpu_kernel_sm90_quant.py:91-97).
- *     1 = one scale per (group, column). More than 1 is taken by the streaming small-m kernel only
- *     (int8 weights, k/blocks a power of two >= 32); for the tiled kernels widen the weights with
- *     tkx_dequantize_weights first.
+ *     1 = one scale per (group, column). More than 1 (int8 weights, k/blocks a power of two): taken by the
+ *     streaming small-m kernel (k/blocks >= 32) and by the tiled variants of mode 4 (block_k divides k/blocks;
+ *     256-column tiles), which multiply each k-block's scales in while they widen the weights, to the same bits
+ *     as tkx_dequantize_weights followed by the bf16 kernels; for other block sizes widen the weights first.
  *   group_offset: device int32[1] or NULL (the `group_offset` argument of RaggedDot, base.py:238; semantics of
  *     experimental/gmm_v2/gmm_v2_test.py:44-101): `group_sizes` then has `num_group_sizes` entries, the
  *     `num_groups` groups of rhs are its entries [offset, offset + num_groups) (entries outside the array count
@@ -187,7 +188,8 @@ int32_t tkx_ragged_gather_rows(const void* x, const int32_t* indices, const floa
 /* Enumerates compiled kernel variants, for the autotuner's search space.
  * kind: 0 = fwd/dlhs variants, 1 = drhs variants.  Returns the count; tkx_ragged_dot_variant fills
  * `config` (tile + wave fields), the dtype pair and the mode of variant `index` (0 = fwd, 1 = dlhs,
- * 2 = drhs, 3 = fwd with gate-up fusion), returning 0, or TKX_ERR_INVALID. */
+ * 2 = drhs, 3 = fwd with gate-up fusion, 4 = fwd over int8 weights with per-k-block scales), returning 0, or
+ * TKX_ERR_INVALID. */
 int32_t tkx_ragged_dot_num_variants(int32_t kind);
 int32_t tkx_ragged_dot_variant(int32_t kind, int32_t index, TkxConfig* config, int32_t* lhs_dtype,
                                int32_t* rhs_dtype, int32_t* mode);

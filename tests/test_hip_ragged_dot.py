@@ -351,6 +351,18 @@ def test_every_kernel_variant_through_c_abi(v, device):
     _check(out, want, 1e-5)
     assert out.shape == (m, n // 2) and torch.count_nonzero(out[int(gs.sum()):]) == 0
     return
+  if v["mode"] == 4:  # forward over int8 weights with per-k-block scales (4 blocks of 64 rows) and a bias
+    lhs = mk((m, k), 1.0).to(lt)
+    rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+    scale = mk((G, 4, n), 0.01).abs() + 1e-3
+    bias = mk((G, 1, n), 0.5)
+    out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale, rhs_bias=bias)
+    # the kernel rounds weight x scale to bf16 (as the widening pass does): the oracle contracts those values
+    rhs_f = O.round_to_bf16(O.dequantize(rhs.cpu().numpy(), _np(scale)))
+    want = O.ragged_dot_fused(_np(lhs), rhs_f, gs, rhs_bias=_np(bias))
+    _check(out, want, 1e-5)
+    assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+    return
   if v["mode"] == 2:
     lhs, dout = mk((m, k), 1.0).to(lt), mk((m, n), 1.0).to(lt)
     out = hip_ops.ragged_dot_drhs(lhs, dout, gst, G, config=cfg, out_dtype=torch.float32)

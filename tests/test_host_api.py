@@ -56,7 +56,7 @@ def test_variant_enumeration_matches_config_space():
   fwd = _lib.variants(0)
   drhs = _lib.variants(1)
   assert fwd and drhs
-  assert {v["mode"] for v in fwd} == {0, 1, 3} and {v["mode"] for v in drhs} == {2}  # 3 = fwd with gate-up fusion
+  assert {v["mode"] for v in fwd} == {0, 1, 3, 4} and {v["mode"] for v in drhs} == {2}  # 3 = gate-up fusion, 4 = k-block scales
   assert all(v["block_n"] // (32 * v["waves_n"]) % 2 == 0 for v in fwd if v["mode"] == 3)  # gate/up halves pair up
   pairs = {(v["lhs_dtype"], v["rhs_dtype"]) for v in fwd}
   assert {(_lib.TKX_BF16, _lib.TKX_BF16), (_lib.TKX_F32, _lib.TKX_F32), (_lib.TKX_F8E4M3FN, _lib.TKX_F8E4M3FN),

@@ -166,7 +166,23 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
     return set_error(TKX_ERR_UNSUPPORTED, "gate-up fusion needs n %% 16 == 0 and k %% block_k == 0 (k=%lld n=%lld)",
                      (long long)k, (long long)n);
   if (rhs_bias && (uintptr_t)rhs_bias % 16 != 0) return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
-  const Variant* v = find_variant(dlhs ? kDlhs : gateup ? kFwdGlu : kFwd, lhs_dtype, rhs_dtype, c);
+  // Scales that change along k: the streaming small-m kernel (block_m == 16) takes them itself; the tiled
+  // kernels have variants of their own (kFwdSubK) that carry the scale rows through LDS.
+  const bool subk = rhs_scale != nullptr && rhs_scale_blocks != 1 && !dlhs && c.block_m != kDecodeBlockM;
+  int32_t log2_block_rows = 0;
+  if (subk) {
+    if (gateup) return set_error(TKX_ERR_UNSUPPORTED, "gate-up fusion takes one rhs scale per (group, column)");
+    if (k % rhs_scale_blocks != 0) return set_error(TKX_ERR_INVALID, "k=%lld is not a multiple of the %lld scale blocks",
+                                                    (long long)k, (long long)rhs_scale_blocks);
+    const int64_t rows = k / rhs_scale_blocks;
+    while ((1LL << log2_block_rows) < rows) ++log2_block_rows;
+    if ((1LL << log2_block_rows) != rows || rows % c.block_k != 0 || k % c.block_k != 0)
+      return set_error(TKX_ERR_UNSUPPORTED,
+                       "the tiled kernels take scale blocks of a power-of-two number of k rows that block_k divides"
+                       " (k=%lld blocks=%lld block_k=%d); widen the weights with tkx_dequantize_weights otherwise",
+                       (long long)k, (long long)rhs_scale_blocks, c.block_k);
+  }
+  const Variant* v = find_variant(dlhs ? kDlhs : gateup ? kFwdGlu : subk ? kFwdSubK : kFwd, lhs_dtype, rhs_dtype, c);
   if (v == nullptr)
     return set_error(TKX_ERR_UNSUPPORTED, "no kernel variant for mode=%d dtypes=(%d,%d) tile=%dx%dx%d waves=%dx%d stages=%d",
                      mode, lhs_dtype, rhs_dtype, c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages);
@@ -198,10 +214,6 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
     return launch_decode(lhs, rhs, rhs_scale, group_sizes, out, m, k, n, num_groups, rhs_dtype, out_dtype, activation,
                          c.num_stages, rhs_scale ? rhs_scale_blocks : 1, c.block_n, group_offset, num_group_sizes, stream);
   }
-  if (rhs_scale && rhs_scale_blocks != 1)
-    return set_error(TKX_ERR_UNSUPPORTED,
-                     "the tiled kernels take one rhs scale per (group, column); widen weights with %lld scale blocks"
-                     " along k with tkx_dequantize_weights first", (long long)rhs_scale_blocks);
 
   const WsLayout L = ws_layout(m, num_groups, c.block_m);
   int32_t st = launch_schedule(group_sizes, num_groups, group_offset, num_group_sizes, m, c.block_m, c.align_tile,
@@ -235,6 +247,8 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
   p.grid_tile_width = c.grid_tile_width;
   p.out_dtype = out_dtype;
   p.activation = activation;
+  p.scale_blocks = subk ? (int32_t)rhs_scale_blocks : 1;
+  p.log2_block_rows = log2_block_rows;
   p.ws_offsets = (int32_t)L.offsets;
   p.ws_gid = (int32_t)L.task[0];
   p.ws_bstart = (int32_t)L.task[1];

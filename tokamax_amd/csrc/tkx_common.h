@@ -60,7 +60,9 @@ int32_t launch_schedule(const int32_t* group_sizes, int64_t G, const int32_t* gr
 
 // ---- grouped GEMM -----------------------------------------------------------------------------
 // kFwdGlu = forward over weights [gate | up] ([g, k, 2 n_out]) with the epilogue act(gate) * up.
-enum KernelMode { kFwd = 0, kDlhs = 1, kDrhs = 2, kFwdGlu = 3 };
+// kFwdSubK = forward over int8 weights whose scales change along k ([g, k / t_k, n]): the scale row of a
+// k-step's block travels into LDS with the step and the weights are scaled while they are widened.
+enum KernelMode { kFwd = 0, kDlhs = 1, kDrhs = 2, kFwdGlu = 3, kFwdSubK = 4 };
 
 // fwd/dlhs launch order: the tile list is dealt to the 8 XCDs in chunks of this many consecutive
 // tiles (the number of CUs of an XCD: one chunk is what an XCD runs at a time).
@@ -84,6 +86,7 @@ struct GemmParams {
   int32_t real_slots;               // fwd/dlhs: workgroups that may own a task tile (multiple of 8 * kXcdChunk)
   int32_t grid_tile_width;
   int32_t out_dtype, activation;
+  int32_t scale_blocks, log2_block_rows;  // kFwdSubK: b_scale is [g, scale_blocks, n]; rows of k per block = 1 << log2
   int32_t ws_offsets, ws_gid, ws_bstart, ws_astart, ws_aend, ws_span_first, ws_span_width;  // word offsets into ws
 };
 

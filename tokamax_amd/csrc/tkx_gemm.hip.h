@@ -204,6 +204,20 @@ __device__ __forceinline__ typename Mma<EC>::Frag load_frag(const unsigned char*
   }
 }
 
+// The same 8 int8 values times one scale (the column's scale for the current k-block), rounded to bf16.
+__device__ __forceinline__ i32x4 i8x8_to_bf16x8_scaled(i32x2 v, float scale) {
+  bf16x8 out;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int w = v[h];
+    out[4 * h + 0] = (__bf16)((float)(signed char)(w & 0xff) * scale);
+    out[4 * h + 1] = (__bf16)((float)(signed char)((w >> 8) & 0xff) * scale);
+    out[4 * h + 2] = (__bf16)((float)(signed char)((w >> 16) & 0xff) * scale);
+    out[4 * h + 3] = (__bf16)((float)(signed char)((w >> 24) & 0xff) * scale);
+  }
+  return __builtin_bit_cast(i32x4, out);
+}
+
 // ---- global -> LDS, fast path: direct-to-LDS loads -------------------------------------------
 // global_load_lds_dwordx4 moves 16 bytes per lane straight into LDS; one wave instruction fills
 // 1024 contiguous LDS bytes (lane l lands at base + 16*l). The LDS swizzle is therefore applied
@@ -434,6 +448,8 @@ struct GemmKernel {
   static constexpr int LA = (MODE == kDrhs) ? kMC : kKC;
   static constexpr int LB = (MODE == kDlhs) ? kKC : kMC;
   static constexpr bool GLU = MODE == kFwdGlu;
+  static constexpr bool SUBK = MODE == kFwdSubK;
+  static_assert(!SUBK || (EB == kEI8 && BN == 256), "per-k-block scales: int8 weights, one 1 KB scale row per k-step");
   static constexpr int BNO = GLU ? BN / 2 : BN;  // output columns of a tile
   static constexpr int EC = EA;  // MFMA type follows A; B may be stored narrower (int8 weights)
   static constexpr int KA = Mma<EC>::KA;
@@ -450,7 +466,8 @@ struct GemmKernel {
   static constexpr int NLOAD = WM * WN;
   typedef DirectLoader<LA, EA, BM, BK, NLOAD> DirA;
   typedef DirectLoader<LB, EB, BN, BK, NLOAD> DirB;
-  static constexpr int STAGE_BYTES = StageA::BYTES + StageB::BYTES;
+  static constexpr int SCALE_BYTES = SUBK ? BN * 4 : 0;  // kFwdSubK: the k-step's scale row behind its two tiles
+  static constexpr int STAGE_BYTES = StageA::BYTES + StageB::BYTES + SCALE_BYTES;
   static constexpr int SMEM_BYTES = NS * STAGE_BYTES;
   static_assert(NS >= 2 && SMEM_BYTES <= 160 * 1024, "stages must fit the 160 KB LDS");
 
@@ -546,6 +563,21 @@ struct GemmKernel {
     }
     rmask = __builtin_amdgcn_readfirstlane(rmask);
     const bool all_rows = rmask == (1u << TM) - 1u;
+    // B fragment j of k-atom kk of a stage. kFwdSubK: the int8 values of the lane's column (lane % 32 of the
+    // block) are multiplied by that column's scale for the stage's k-block, which lies behind the tiles.
+    auto load_b_frag = [&](const unsigned char* stage, int j, int kk) -> Frag {
+      if constexpr (SUBK) {
+        const int blk = lane >> 4, s_ = lane & 15;
+        const int col = wn * WTN + j * 32 + 16 * (blk & 1) + 8 * (s_ & 1);
+        const int krow = kk * KA + 8 * (blk >> 1) + (s_ >> 1);
+        const i32x2 v = lds_read_tr8(stage + StageA::BYTES + mc_offset<StageB::ROW_BYTES, EB>(krow, col));
+        const float scale = *reinterpret_cast<const float*>(stage + StageA::BYTES + StageB::BYTES +
+                                                            4 * (wn * WTN + j * 32 + (lane & 31)));
+        return i8x8_to_bf16x8_scaled(v, scale);
+      } else {
+        return load_frag<LB, EB, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + j * 32, kk, lane);
+      }
+    };
     auto load_frags = [&](auto full, Frag* fa, Frag* fb, const unsigned char* stage, int kk) {
 #if defined(TKX_ABLATE) && (TKX_ABLATE & 2)
       return;
@@ -556,8 +588,7 @@ struct GemmKernel {
           fa[i] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, row_block(i) * 32, kk, lane);
       if (decltype(full)::value || rmask != 0) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          fb[j] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + j * 32, kk, lane);
+        for (int j = 0; j < TN; ++j) fb[j] = load_b_frag(stage, j, kk);
       }
     };
     auto mma_all = [&](auto full, const Frag* fa, const Frag* fb) {
@@ -591,23 +622,33 @@ struct GemmKernel {
       // A load wave may leave the loads of the NS-2 k-steps after the needed one in flight; that
       // count is only known at compile time when the tile splits evenly over the load waves.
       constexpr bool kExact = DirA::INSTRS % NLOAD == 0 && DirB::INSTRS % NLOAD == 0;
-      constexpr int kInFlight = kExact ? (NS - 2) * (DirA::PER + DirB::PER) : 0;
-      static_assert(kInFlight < 64, "too many direct loads in flight for vmcnt");
-
       // One k-step of loads is a list of NLD per-wave instructions; slot q of the list can be issued
-      // on its own, so that the list can be threaded between MFMAs.
-      constexpr int NLD = DirA::PER + DirB::PER;
-      struct StepPtrs { const unsigned char *a, *b; unsigned lds; };
+      // on its own, so that the list can be threaded between MFMAs. kFwdSubK adds one: every wave
+      // fetches the 1 KB scale row of the step's k-block (the same bytes to the same place, so that
+      // all waves count the same number of loads).
+      constexpr int NLD = DirA::PER + DirB::PER + (SUBK ? 1 : 0);
+      constexpr int kInFlight = kExact ? (NS - 2) * NLD : 0;
+      static_assert(kInFlight < 64 && (NS - 1) * NLD < 64, "too many direct loads in flight for vmcnt");
+      struct StepPtrs { const unsigned char *a, *b, *s; unsigned lds; };
+      // (kFwdSubK) scales of this tile's columns: row `block` of the group's [scale_blocks, n] table; lanes past
+      // the last column re-read the last four (their products are never stored).
+      const unsigned char* const gS0 =
+          SUBK ? reinterpret_cast<const unsigned char*>(p.b_scale + (int64_t)group * p.scale_blocks * p.nb_ext) : nullptr;
+      const uint32_t scale_voff = SUBK ? (uint32_t)min(col0 + 4 * lane, p.nb_ext - 4) * 4u : 0u;
       auto step_ptrs = [&](int step, int stage) {
         StepPtrs sp;
         sp.a = uniform_pointer(gA0 + step * stepA);
         sp.b = uniform_pointer(gB0 + step * stepB);
+        sp.s = nullptr;
+        if constexpr (SUBK)
+          sp.s = uniform_pointer(gS0 + (int64_t)((kc_begin + step * BK) >> p.log2_block_rows) * p.nb_ext * 4);
         sp.lds = smem_lds + stage * STAGE_BYTES;
         return sp;
       };
       auto issue_slot = [&](int q, const StepPtrs& sp) {
         if (q < DirA::PER) da.issue_one(q, sp.a, sp.lds, wave);
         else if (q < DirA::PER + DirB::PER) db.issue_one(q - DirA::PER, sp.b, sp.lds + StageA::BYTES, wave);
+        else if (SUBK && q == DirA::PER + DirB::PER) direct_load_16(sp.s, scale_voff, sp.lds + StageA::BYTES + StageB::BYTES);
       };
       // Every wave drains the loads the next k-step needs before it arrives at a barrier.
       auto step_barrier = [&](bool partial) {
@@ -624,7 +665,7 @@ struct GemmKernel {
           for (int q = 0; q < NLD; ++q) issue_slot(q, sp);
         }
       }
-      if (kExact && nfull >= NS) barrier_after_direct_loads<(NS - 1) * (DirA::PER + DirB::PER)>();
+      if (kExact && nfull >= NS) barrier_after_direct_loads<(NS - 1) * NLD>();
       else barrier_after_direct_loads<0>();
 
       // The k loop. Each 32-wide (KA-deep) atom is a run of TM*TN MFMAs; the LDS reads of the next
@@ -651,8 +692,7 @@ struct GemmKernel {
           if (f < TM) {
             if (F || ((rmask >> f) & 1u)) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, row_block(f) * 32, kk, lane);
           } else if (f < TM + TN) {
-            if (F || rmask != 0)
-              b[f - TM] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + (f - TM) * 32, kk, lane);
+            if (F || rmask != 0) b[f - TM] = load_b_frag(stage, f - TM, kk);
           }
         };
         constexpr int NM = TM * TN;                      // MFMAs per atom
@@ -716,7 +756,7 @@ struct GemmKernel {
       if (all_rows) k_loop(std::true_type{});
       else k_loop(std::false_type{});
     }
-    if (tail && !GLU) {  // (gate-up problems are taken only with whole k-steps)
+    if (tail && !GLU && !SUBK) {  // (gate-up and per-k-block-scale problems are taken only with whole k-steps)
       const int kc0 = kc_begin + nfull * BK;
       StageA::copy(Ab, p.lda, row0, p.m_ext, kc0, kc_end, smem, tid);
       StageB::copy(Bb, p.ldb, col0, p.nb_ext, kc0, kc_end, smem + StageA::BYTES, tid);
@@ -758,7 +798,7 @@ struct GemmKernel {
             for (int e = 0; e < 16; ++e) acc[i][j][e] *= rs;
         }
       }
-      if (p.b_scale != nullptr) {
+      if (!SUBK && p.b_scale != nullptr) {  // (kFwdSubK: applied to the weights on their way into the MFMAs)
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
 #pragma unroll

@@ -1,9 +1,11 @@
 // bf16 activations x int8 weights forward variants (weights converted to bf16 on the way from LDS
-// to the MFMA; per-(group, column) scales in the epilogue).
+// to the MFMA; per-(group, column) scales in the epilogue, or per-(group, k-block, column) scales
+// multiplied in during that conversion: kFwdSubK, 256-column tiles).
 #include "tkx_gemm.hip.h"
 
 namespace tkx {
 #define FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEBF16, kEI8, BM, BN, BK, WM, WN, NS)
+#define SUBK(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdSubK, kEBF16, kEI8, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
     FWD(256, 256, 32, 2, 4, 4),
@@ -16,6 +18,10 @@ static const Variant kVariants[] = {
     FWD(32, 256, 64, 1, 4, 4),
     FWD(32, 128, 128, 1, 4, 4),
     FWD(32, 128, 128, 1, 4, 2),
+    SUBK(256, 256, 64, 2, 4, 3),
+    SUBK(256, 256, 32, 2, 4, 4),
+    SUBK(128, 256, 64, 2, 4, 3),
+    SUBK(32, 256, 64, 1, 4, 4),
 };
 
 const Variant* variants_i8w(int* count) {

@@ -21,6 +21,7 @@ from tokamax_amd import _lib
 from tokamax_amd import config as config_lib
 from tokamax_amd import op
 from tokamax_amd import precision as precision_lib
+from tokamax_amd.serialization import ShapeDtype
 from tokamax_amd.ragged_dot import base
 from tokamax_amd.ragged_dot import hip_ops
 
@@ -115,8 +116,11 @@ def _lhs_scale_blocks(q: QArray) -> int | None:
   return shape[1]
 
 
-def _widening_plan(lhs, rhs) -> tuple[bool, bool]:
-  """(widen lhs, widen rhs): which quantised operands are dequantised to bf16 before the kernels.
+def _widening_plan(lhs, rhs, allow_native: bool = True) -> tuple[bool, bool, bool]:
+  """(widen lhs, widen rhs, native k-blocks): which quantised operands are dequantised to bf16 before the
+  kernels, and whether int8 weights with scales [g, k/t_k, n] keep them (t_k a power of two that 64 divides,
+  bf16 on the other side, `allow_native`: no gate-up fusion): kernels of their own multiply each k-block's
+  scales in while they widen the weights.
 
   The kernels apply one scale per lhs row and one per (group, column) in their epilogue. Scales that change
   along the contraction (the k-subchannel scales of pallas_mosaic_gpu_kernel_sm100_i8_quant.py:51-102, the scale
@@ -135,6 +139,12 @@ def _widening_plan(lhs, rhs) -> tuple[bool, bool]:
       raise NotImplementedError("rhs scale must have shape [g,1,n], [g,k/t_k,n] or [g,k/t_k,n/t_n] with 16 | t_n, got"
                                 f" {tuple(rhs.scale.shape)}")
     widen_rhs = blocks is None or blocks > 1
+    if allow_native and blocks is not None and blocks > 1 and rhs.qvalue.dtype == torch.int8:
+      _, k, n = rhs.qvalue.shape
+      rows = k // blocks
+      lhs_is_bf16 = _dtype_of(lhs) == torch.int8 if lhs_q else lhs.dtype == torch.bfloat16  # (int8 lhs: widened)
+      if rows % 64 == 0 and rows & (rows - 1) == 0 and n % 16 == 0 and lhs_is_bf16:
+        return widen_lhs, False, True
   eight_bit_float = lambda x: _dtype_of(x) == torch.float8_e4m3fn
   if widen_rhs and lhs_q and eight_bit_float(lhs):
     widen_lhs = True
@@ -142,7 +152,7 @@ def _widening_plan(lhs, rhs) -> tuple[bool, bool]:
     widen_rhs = True
   if (widen_lhs and not rhs_q and eight_bit_float(rhs)) or (widen_rhs and not lhs_q and eight_bit_float(lhs)):
     raise NotImplementedError("A raw fp8 operand cannot meet a widened (bf16) one.")
-  return widen_lhs, widen_rhs
+  return widen_lhs, widen_rhs, False
 
 
 _SUB_BYTE_INTS = tuple(getattr(torch, f"int{b}") for b in range(1, 8) if hasattr(torch, f"int{b}"))
@@ -258,7 +268,7 @@ class HipRaggedDot(base.RaggedDot):
     for name, x in (("lhs", lhs), ("rhs", rhs)):
       if isinstance(x, QArray) and (mode != 0 or x.zero_point is not None):
         raise NotImplementedError(f"Quantised {name}: default dimension numbers without zero point only.")
-    widen_lhs, widen_rhs = _widening_plan(lhs, rhs)
+    widen_lhs, widen_rhs, native_k_blocks = _widening_plan(lhs, rhs, allow_native=gateup is None)
     if isinstance(lhs, QArray):
       if widen_lhs:
         if lhs.qvalue.shape[1] % 16 != 0:
@@ -271,7 +281,8 @@ class HipRaggedDot(base.RaggedDot):
     if isinstance(rhs, QArray):
       g, k, n = rhs.qvalue.shape
       if not widen_rhs:
-        rhs_scale_, rhs_v = rhs.scale, rhs.qvalue  # one scale per (group, column): applied in the epilogue
+        # One scale per (group, column): applied in the epilogue. Native k-blocks: [g, k/t_k, n] goes as it is.
+        rhs_scale_, rhs_v = rhs.scale, rhs.qvalue
       else:
         # Scales that change along k (or in blocks along n): widened to bf16 by a streaming pass, then the
         # bf16 kernels.
@@ -381,12 +392,16 @@ class HipRaggedDot(base.RaggedDot):
       rows, cols, contraction = lhs_shape[0], rhs_shape[2], rhs_shape[1]
     lhs_dt, rhs_dt = _dtype_of(lhs), _dtype_of(rhs)
     raw_scale = ba.kwargs.get("rhs_scale")
-    if raw_scale is not None and len(raw_scale.shape) == 4 and raw_scale.shape[1] > 1:
-      rhs_dt = torch.bfloat16  # sub-channel scales: `_fwd` widens the weights to bf16 first
+    if raw_scale is not None and len(raw_scale.shape) == 4 and not isinstance(rhs, (QArray, AsQArray)):
+      # (the raw form of quantised weights: `_fwd` makes the same QArray of it)
+      g_, blocks_, _, n_ = raw_scale.shape
+      rhs = QArray(rhs, ShapeDtype((g_, blocks_, n_), raw_scale.dtype))
     if mode in (0, 3):
-      widen_lhs, widen_rhs = _widening_plan(lhs, rhs)
+      widen_lhs, widen_rhs, native_k_blocks = _widening_plan(lhs, rhs, allow_native=mode == 0)
       lhs_dt = torch.bfloat16 if widen_lhs else lhs_dt
       rhs_dt = torch.bfloat16 if widen_rhs else rhs_dt
+      if native_k_blocks:
+        mode = 4  # forward with per-k-block weight scales: variants of their own
     if (ba.kwargs.get("precision") == precision_lib.DotAlgorithmPreset.BF16_BF16_F32
         and not isinstance(lhs, (QArray, AsQArray)) and not isinstance(rhs, (QArray, AsQArray))):
       lhs_dt = rhs_dt = torch.bfloat16  # `_fwd` casts both operands for this preset
@@ -398,10 +413,14 @@ class HipRaggedDot(base.RaggedDot):
     variants = _variant_table().get(key)
     if not variants:
       raise NotImplementedError(f"No hip kernel for dtypes/mode {key}.")
+    if mode == 4:
+      # The streaming small-m kernel takes per-k-block scales in its 128-column form (listed with the
+      # plain forward variants).
+      variants = variants + [v for v in _variant_table().get((0, key[1], key[2]), []) if v[0] == 16 and v[1] == 128]
     # The streaming small-m kernel (listed with block_m == 16; forward only) needs k % 1024 == 0 and
     # n % 8 == 0, and a weight slice (k/4 rows of n) that a 32-bit buffer offset spans.
     wbytes = 1 if key[2] == _lib.TKX_I8 else 2
-    streaming_ok = (mode == 0 and ba.kwargs.get("rhs_bias") is None and contraction % 1024 == 0 and cols % 8 == 0
+    streaming_ok = (mode in (0, 4) and ba.kwargs.get("rhs_bias") is None and contraction % 1024 == 0 and cols % 8 == 0
                     and (contraction // 4) * cols * wbytes < 2**31)
     usable = [v for v in variants if v[0] != 16 or streaming_ok]
     # Rows per group decide the m-tile: a tile much taller than a group wastes MFMA work on rows
@@ -415,7 +434,7 @@ class HipRaggedDot(base.RaggedDot):
     # per CU) that streams 7-9% faster when its workgroups fill the chip evenly, and slower than the
     # 128-column form when they do not (measured: 384 workgroups on 256 CUs lose 10%).
     wide_wgs = num_groups * -(-cols // 256)
-    stream_n = 256 if cols % 16 == 0 and wide_wgs / (-(-wide_wgs // 512) * 512) >= 0.9 else 128
+    stream_n = 256 if mode == 0 and cols % 16 == 0 and wide_wgs / (-(-wide_wgs // 512) * 512) >= 0.9 else 128
 
     def score(v):
       bm, bn, bk, wm, wn, ns = v
@@ -433,7 +452,8 @@ class HipRaggedDot(base.RaggedDot):
       # contraction in flight, (stages - 1) * block_k; beyond 96 more depth buys nothing (it measured
       # 1.5% slower), and at equal depth the longer k-step has fewer barriers per flop.
       in_flight = min((ns - 1) * bk, 96) if wm * wn == 8 else 0
-      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -in_flight, -bk, ns)
+      # (With per-k-block scales the shorter k-step measured 3 % faster at equal depth: 991 against 961 TFLOP/s.)
+      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -in_flight, bk if mode == 4 else -bk, ns)
 
     bm, bn, bk, wm, wn, ns = min(usable, key=score)
     # grid_tile_width m-tasks of one group run side by side on an n-panel of its weights (a span never
