@@ -41,7 +41,7 @@ PEAK_HBM_GBS = 8000.0
 # this script, each scaled by what the same counter reads for a copy kernel of known size; None
 # where no counter run has been made for the current kernel.
 MEASURED_TRAFFIC_BYTES = {
-    "mixtral": 4.26e9,  # 256x256x32 kernel: 3.67e9 read + 0.60e9 written past L2 (algorithmic: 1.543e9)
+    "mixtral": 4.21e9,  # 256x256x32 kernel: 3.62e9 read + 0.60e9 written past L2 (algorithmic: 1.543e9)
     "decode": 1.838e8,  # streaming int8 kernel: 1.834e8 read + 3.9e5 written (algorithmic: 1.748e8)
 }
 
@@ -276,7 +276,13 @@ def main():
     nb = w.m * w.k * 2 + w.nonempty_groups * w.k * w.n + w.m * w.n * 2
     measure("mixtral_prefill_int8_weights", lambda: op(w.lhs, q8, group_sizes=gs, preferred_element_type=torch.bfloat16),
             w.flops, nb, "mfma", "bf16", cfg)
-    del w, q8
+    # the same weights with a scale per (group, block of 128 k rows, column): scaled while widened, in the kernel
+    q8k = tokamax_amd.QArray(q8.qvalue, (torch.rand(w.num_groups, w.k // 128, w.n, device=device, generator=gen8) + 0.5)
+                             / (127 * w.k ** 0.5))
+    cfg = op.bind(w.lhs, q8k, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_prefill_int8_weights_k_block_scales", lambda: op(w.lhs, q8k, group_sizes=gs, preferred_element_type=torch.bfloat16),
+            w.flops, nb + w.nonempty_groups * (w.k // 128) * w.n * 4, "mfma", "bf16", cfg)
+    del w, q8, q8k
 
     w = workloads.make("vjp", device, seed=0)
     gs = torch.tensor(w.group_sizes, device=device)
