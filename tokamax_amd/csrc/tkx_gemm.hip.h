@@ -623,9 +623,9 @@ struct GemmKernel {
       // count is only known at compile time when the tile splits evenly over the load waves.
       constexpr bool kExact = DirA::INSTRS % NLOAD == 0 && DirB::INSTRS % NLOAD == 0;
       // One k-step of loads is a list of NLD per-wave instructions; slot q of the list can be issued
-      // on its own, so that the list can be threaded between MFMAs. kFwdSubK adds one: every wave
-      // fetches the 1 KB scale row of the step's k-block (the same bytes to the same place, so that
-      // all waves count the same number of loads).
+      // on its own, so that the list can be threaded between MFMAs. kFwdSubK adds one: the 1 KB scale
+      // row of the step's k-block, of which every wave fetches its 1/NLOAD with that many of its lanes
+      // (so that all waves count the same number of loads).
       constexpr int NLD = DirA::PER + DirB::PER + (SUBK ? 1 : 0);
       constexpr int kInFlight = kExact ? (NS - 2) * NLD : 0;
       static_assert(kInFlight < 64 && (NS - 1) * NLD < 64, "too many direct loads in flight for vmcnt");
@@ -634,7 +634,8 @@ struct GemmKernel {
       // the last column re-read the last four (their products are never stored).
       const unsigned char* const gS0 =
           SUBK ? reinterpret_cast<const unsigned char*>(p.b_scale + (int64_t)group * p.scale_blocks * p.nb_ext) : nullptr;
-      const uint32_t scale_voff = SUBK ? (uint32_t)min(col0 + 4 * lane, p.nb_ext - 4) * 4u : 0u;
+      constexpr int SCALE_LANES = 64 / NLOAD;  // lanes of a wave that fetch 16 bytes of the scale row each
+      const uint32_t scale_voff = SUBK ? (uint32_t)min(col0 + 4 * (wave * SCALE_LANES + lane), p.nb_ext - 4) * 4u : 0u;
       auto step_ptrs = [&](int step, int stage) {
         StepPtrs sp;
         sp.a = uniform_pointer(gA0 + step * stepA);
@@ -648,7 +649,10 @@ struct GemmKernel {
       auto issue_slot = [&](int q, const StepPtrs& sp) {
         if (q < DirA::PER) da.issue_one(q, sp.a, sp.lds, wave);
         else if (q < DirA::PER + DirB::PER) db.issue_one(q - DirA::PER, sp.b, sp.lds + StageA::BYTES, wave);
-        else if (SUBK && q == DirA::PER + DirB::PER) direct_load_16(sp.s, scale_voff, sp.lds + StageA::BYTES + StageB::BYTES);
+        else if (SUBK && q == DirA::PER + DirB::PER) {
+          if (lane < SCALE_LANES)
+            direct_load_16(sp.s, scale_voff, sp.lds + StageA::BYTES + StageB::BYTES + wave * (SCALE_LANES * 16));
+        }
       };
       // Every wave drains the loads the next k-step needs before it arrives at a barrier.
       auto step_barrier = [&](bool partial) {
