@@ -351,14 +351,19 @@ def test_every_kernel_variant_through_c_abi(v, device):
     _check(out, want, 1e-5)
     assert out.shape == (m, n // 2) and torch.count_nonzero(out[int(gs.sum()):]) == 0
     return
-  if v["mode"] == 4:  # forward over int8 weights with per-k-block scales (4 blocks of 64 rows) and a bias
+  if v["mode"] == 4:  # forward over int8 / fp8 weights with per-k-block scales (4 blocks of 64 rows) and a bias
     lhs = mk((m, k), 1.0).to(lt)
-    rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+    if rt == torch.int8:
+      rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+      rhs_values = rhs.cpu().numpy()
+    else:
+      rhs = mk((G, k, n), 1.0).to(rt)
+      rhs_values = O.e4m3fn_decode(rhs.view(torch.uint8).cpu().numpy())
     scale = mk((G, 4, n), 0.01).abs() + 1e-3
     bias = mk((G, 1, n), 0.5)
     out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale, rhs_bias=bias)
     # the kernel rounds weight x scale to bf16 (as the widening pass does): the oracle contracts those values
-    rhs_f = O.round_to_bf16(O.dequantize(rhs.cpu().numpy(), _np(scale)))
+    rhs_f = O.round_to_bf16(O.dequantize(rhs_values, _np(scale)))
     want = O.ragged_dot_fused(_np(lhs), rhs_f, gs, rhs_bias=_np(bias))
     _check(out, want, 1e-5)
     assert torch.count_nonzero(out[int(gs.sum()):]) == 0
@@ -725,6 +730,34 @@ def test_k_subchannel_scales_through_widening(case, device):
   _check(out, want, TOL["fp8"], rows=count)
   assert O.rel_l2(_np(out)[:count], want[:count]) < 6e-3  # two operands rounded to bf16, f32 accumulation
   assert torch.count_nonzero(out[count:]) == 0
+
+
+def test_bf16_activations_fp8_weights(device):
+  """bf16 x fp8 (e4m3fn) weights with one scale per (group, column) or per (group, 128 k rows, column): the kernels
+  that scale the weights while they widen them; an fp8 lhs with row scales is widened first for them."""
+  rng = np.random.default_rng(21)
+  G, m, k, n = 4, 300, 512, 256
+  gs = np.array([100, 0, 80, 110], np.int32)
+  gst = torch.tensor(gs, device=device)
+  count = int(gs.sum())
+  a16 = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  q = torch.tensor(rng.normal(0, 1, (G, k, n)).astype(np.float32), device=device).to(torch.float8_e4m3fn)
+  qf = O.e4m3fn_decode(q.view(torch.uint8).cpu().numpy()).astype(np.float64)
+  op = tokamax_amd.HipRaggedDot()
+  for blocks in (1, k // 128):
+    scale = torch.tensor((rng.uniform(0.5, 1.5, (G, blocks, n)) * k ** -0.5).astype(np.float32), device=device)
+    rhs = tokamax_amd.QArray(q, scale)
+    cfg = op._get_heuristics_config(op.bind(a16, rhs, group_sizes=gst))
+    assert cfg.block_n == 256 and cfg.block_m != 16
+    out = tokamax_amd.ragged_dot(a16, rhs, gst, preferred_element_type=torch.float32)
+    want = O.ragged_dot(_np(a16), O.dequantize(qf, _np(scale)), gs, acc_dtype=np.float64, out_dtype="f64")
+    _check(out, want, 4e-3, rows=count)  # weight x scale rounded to bf16
+    assert torch.count_nonzero(out[count:]) == 0
+  a8 = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.float8_e4m3fn)
+  a_scale = torch.tensor(rng.uniform(0.5, 1.5, (m, 1)).astype(np.float32), device=device)
+  lhs_f = O.dequantize(O.e4m3fn_decode(a8.view(torch.uint8).cpu().numpy()).astype(np.float64), _np(a_scale))
+  out = tokamax_amd.ragged_dot(tokamax_amd.QArray(a8, a_scale), rhs, gst, preferred_element_type=torch.float32)
+  _check(out, O.ragged_dot(lhs_f, O.dequantize(qf, _np(scale)), gs, acc_dtype=np.float64, out_dtype="f64"), 6e-3, rows=count)
 
 
 def test_int4_values_in_int8_storage(device):

@@ -168,9 +168,15 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
   if (rhs_bias && (uintptr_t)rhs_bias % 16 != 0) return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
   // Scales that change along k: the streaming small-m kernel (block_m == 16) takes them itself; the tiled
   // kernels have variants of their own (kFwdSubK) that carry the scale rows through LDS.
-  const bool subk = rhs_scale != nullptr && rhs_scale_blocks != 1 && !dlhs && c.block_m != kDecodeBlockM;
+  // bf16 activations x fp8 weights exist in that form only, also with a single scale block.
+  const bool a16w8f = lhs_dtype == TKX_BF16 && rhs_dtype == TKX_F8E4M3FN;
+  if (a16w8f && (rhs_scale == nullptr || dlhs))
+    return set_error(TKX_ERR_UNSUPPORTED, "bf16 x fp8 weights: default mode with an rhs scale only");
+  const bool subk = rhs_scale != nullptr && (rhs_scale_blocks != 1 || a16w8f) && !dlhs && c.block_m != kDecodeBlockM;
   int32_t log2_block_rows = 0;
-  if (subk) {
+  if (subk && rhs_scale_blocks == 1) {
+    log2_block_rows = 30;  // every k-step falls into block 0
+  } else if (subk) {
     if (gateup) return set_error(TKX_ERR_UNSUPPORTED, "gate-up fusion takes one rhs scale per (group, column)");
     if (k % rhs_scale_blocks != 0) return set_error(TKX_ERR_INVALID, "k=%lld is not a multiple of the %lld scale blocks",
                                                     (long long)k, (long long)rhs_scale_blocks);

@@ -218,6 +218,20 @@ __device__ __forceinline__ i32x4 i8x8_to_bf16x8_scaled(i32x2 v, float scale) {
   return __builtin_bit_cast(i32x4, out);
 }
 
+// 8 fp8 (e4m3fn) values times one scale, rounded to bf16.
+__device__ __forceinline__ i32x4 f8x8_to_bf16x8_scaled(i32x2 v, float scale) {
+  bf16x8 out;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int w = v[h];
+    out[4 * h + 0] = (__bf16)(__builtin_amdgcn_cvt_f32_fp8(w, 0) * scale);
+    out[4 * h + 1] = (__bf16)(__builtin_amdgcn_cvt_f32_fp8(w, 1) * scale);
+    out[4 * h + 2] = (__bf16)(__builtin_amdgcn_cvt_f32_fp8(w, 2) * scale);
+    out[4 * h + 3] = (__bf16)(__builtin_amdgcn_cvt_f32_fp8(w, 3) * scale);
+  }
+  return __builtin_bit_cast(i32x4, out);
+}
+
 // ---- global -> LDS, fast path: direct-to-LDS loads -------------------------------------------
 // global_load_lds_dwordx4 moves 16 bytes per lane straight into LDS; one wave instruction fills
 // 1024 contiguous LDS bytes (lane l lands at base + 16*l). The LDS swizzle is therefore applied
@@ -449,7 +463,8 @@ struct GemmKernel {
   static constexpr int LB = (MODE == kDlhs) ? kKC : kMC;
   static constexpr bool GLU = MODE == kFwdGlu;
   static constexpr bool SUBK = MODE == kFwdSubK;
-  static_assert(!SUBK || (EB == kEI8 && BN == 256), "per-k-block scales: int8 weights, one 1 KB scale row per k-step");
+  static_assert(!SUBK || ((EB == kEI8 || EB == kEF8) && EA == kEBF16 && BN == 256),
+                "per-k-block scales: bf16 lhs, int8 or fp8 weights, one 1 KB scale row per k-step");
   static constexpr int BNO = GLU ? BN / 2 : BN;  // output columns of a tile
   static constexpr int EC = EA;  // MFMA type follows A; B may be stored narrower (int8 weights)
   static constexpr int KA = Mma<EC>::KA;
@@ -573,7 +588,8 @@ struct GemmKernel {
         const i32x2 v = lds_read_tr8(stage + StageA::BYTES + mc_offset<StageB::ROW_BYTES, EB>(krow, col));
         const float scale = *reinterpret_cast<const float*>(stage + StageA::BYTES + StageB::BYTES +
                                                             4 * (wn * WTN + j * 32 + (lane & 31)));
-        return i8x8_to_bf16x8_scaled(v, scale);
+        if constexpr (EB == kEI8) return i8x8_to_bf16x8_scaled(v, scale);
+        else return f8x8_to_bf16x8_scaled(v, scale);
       } else {
         return load_frag<LB, EB, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + j * 32, kk, lane);
       }

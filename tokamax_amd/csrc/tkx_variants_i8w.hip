@@ -6,6 +6,9 @@
 namespace tkx {
 #define FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEBF16, kEI8, BM, BN, BK, WM, WN, NS)
 #define SUBK(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdSubK, kEBF16, kEI8, BM, BN, BK, WM, WN, NS)
+// The same with fp8 (e4m3fn) weights: bf16 activations x fp8 weights exist in this form only (one scale block
+// covers the case of one scale per (group, column)).
+#define SUBK_F8(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdSubK, kEBF16, kEF8, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
     FWD(256, 256, 32, 2, 4, 4),
@@ -22,6 +25,10 @@ static const Variant kVariants[] = {
     SUBK(256, 256, 32, 2, 4, 4),
     SUBK(128, 256, 64, 2, 4, 3),
     SUBK(32, 256, 64, 1, 4, 4),
+    SUBK_F8(256, 256, 64, 2, 4, 3),
+    SUBK_F8(256, 256, 32, 2, 4, 4),
+    SUBK_F8(128, 256, 64, 2, 4, 3),
+    SUBK_F8(32, 256, 64, 1, 4, 4),
 };
 
 const Variant* variants_i8w(int* count) {

@@ -139,13 +139,18 @@ def _widening_plan(lhs, rhs, allow_native: bool = True) -> tuple[bool, bool, boo
       raise NotImplementedError("rhs scale must have shape [g,1,n], [g,k/t_k,n] or [g,k/t_k,n/t_n] with 16 | t_n, got"
                                 f" {tuple(rhs.scale.shape)}")
     widen_rhs = blocks is None or blocks > 1
-    if allow_native and blocks is not None and blocks > 1 and rhs.qvalue.dtype == torch.int8:
-      _, k, n = rhs.qvalue.shape
-      rows = k // blocks
-      lhs_is_bf16 = _dtype_of(lhs) == torch.int8 if lhs_q else lhs.dtype == torch.bfloat16  # (int8 lhs: widened)
-      if rows % 64 == 0 and rows & (rows - 1) == 0 and n % 16 == 0 and lhs_is_bf16:
-        return widen_lhs, False, True
   eight_bit_float = lambda x: _dtype_of(x) == torch.float8_e4m3fn
+  if rhs_q and allow_native and blocks is not None and rhs.qvalue.dtype in (torch.int8, torch.float8_e4m3fn):
+    # Kernels of their own (bf16 lhs; 256-column tiles) for int8 weights with several scale blocks along k and
+    # for fp8 weights with any number of them, unless fp8 meets fp8 with one scale each (the fp8 MFMA kernels).
+    _, k, n = rhs.qvalue.shape
+    rows = k // blocks
+    shape_ok = n % 16 == 0 and k % 64 == 0 and (blocks == 1 or (rows % 64 == 0 and rows & (rows - 1) == 0))
+    fp8_pair = lhs_q and eight_bit_float(lhs) and not widen_lhs and blocks == 1
+    wanted = blocks > 1 or (eight_bit_float(rhs) and not fp8_pair)
+    lhs_becomes_bf16 = lhs_q or lhs.dtype == torch.bfloat16  # (a quantised lhs is widened for it)
+    if shape_ok and wanted and lhs_becomes_bf16:
+      return lhs_q, False, True
   if widen_rhs and lhs_q and eight_bit_float(lhs):
     widen_lhs = True
   if widen_lhs and rhs_q and eight_bit_float(rhs):
