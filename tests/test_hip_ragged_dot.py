@@ -732,6 +732,40 @@ def test_k_subchannel_scales_through_widening(case, device):
   assert torch.count_nonzero(out[count:]) == 0
 
 
+@pytest.mark.parametrize("blocks", [1, 4])
+@pytest.mark.parametrize("depth", [2, 4])
+def test_small_m_kernel_fp8_weights(blocks, depth, device):
+  """The streaming small-m kernel on fp8 (e4m3fn) weights: one scale per (group, column) in the epilogue (an fp8
+  value is a bf16 value exactly, so the f32 result is exact up to accumulation order), or per k-block while the
+  weights are widened; the public entry picks it for groups of a few rows."""
+  rng = np.random.default_rng(30 + blocks + depth)
+  gs = np.array([3, 0, 0, 17, 1, 0, 16, 2], np.int32)
+  G, k, n = len(gs), 1024, 208
+  m = int(gs.sum()) + 11
+  gst = torch.tensor(gs, device=device)
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  q = torch.tensor(rng.normal(0, 1, (G, k, n)).astype(np.float32), device=device).to(torch.float8_e4m3fn)
+  qf = O.e4m3fn_decode(q.view(torch.uint8).cpu().numpy()).astype(np.float64)
+  scale = torch.tensor((rng.uniform(0.5, 1.5, (G, blocks, n)) * k ** -0.5).astype(np.float32), device=device)
+  cfg = hip_ops.KernelConfig(16, 128, 32, 1, 4, depth)
+  out = hip_ops.ragged_dot_fwd(lhs, q, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale)
+  if blocks == 1:
+    want = O.ragged_dot(_np(lhs), O.dequantize(qf, _np(scale)), gs, acc_dtype=np.float64, out_dtype="f64")
+    _check(out, want, 1e-5)
+  else:  # weight x scale rounded to bf16
+    want = O.ragged_dot(_np(lhs), O.round_to_bf16(O.dequantize(qf, _np(scale))), gs, acc_dtype=np.float64, out_dtype="f64")
+    _check(out, want, 1e-5)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  if depth == 2:
+    op = tokamax_amd.HipRaggedDot()
+    small = np.array([3, 0, 0, 7, 1, 0, 6, 2], np.int32)
+    rhs = tokamax_amd.QArray(q, scale)
+    sgt = torch.tensor(small, device=device)
+    assert op._get_heuristics_config(op.bind(lhs[:19], rhs, group_sizes=sgt)).block_m == 16
+    got = op(lhs[:19], rhs, group_sizes=sgt, preferred_element_type=torch.float32)
+    _check(got, O.ragged_dot(_np(lhs[:19]), O.dequantize(qf, _np(scale)), small, acc_dtype=np.float64, out_dtype="f64"), 4e-3)
+
+
 def test_bf16_activations_fp8_weights(device):
   """bf16 x fp8 (e4m3fn) weights with one scale per (group, column) or per (group, 128 k rows, column): the kernels
   that scale the weights while they widen them; an fp8 lhs with row scales is widened first for them."""

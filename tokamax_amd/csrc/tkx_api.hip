@@ -36,6 +36,8 @@ struct Registry {
       all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
     for (int depth : {2, 4})
       all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeWideBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
+    for (int depth : {2, 4})
+      all.push_back({kFwd, TKX_BF16, TKX_F8E4M3FN, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
     for (int dtype : {TKX_BF16, TKX_F16})
       for (int depth : {2, 4})
         all.push_back({kFwd, dtype, dtype, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
@@ -210,8 +212,8 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
     // Streaming decode kernel: one launch, no schedule.
     if (lhs_scale != nullptr) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no lhs scale");
     if (rhs_bias != nullptr || gateup) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no bias or gate-up fusion");
-    if (rhs_scale != nullptr && rhs_dtype != TKX_I8)
-      return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes an rhs scale with int8 weights only");
+    if (rhs_scale != nullptr && rhs_dtype != TKX_I8 && rhs_dtype != TKX_F8E4M3FN)
+      return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes an rhs scale with int8 or fp8 weights only");
     if (!decode_supported(lhs_dtype, rhs_dtype, m, k, n, num_groups, rhs_scale ? rhs_scale_blocks : 1, c.block_n))
       return set_error(TKX_ERR_UNSUPPORTED,
                        "decode kernel needs k %% 1024 == 0, n %% 8 == 0 (n %% 16 == 0 and one scale block at block_n 256)"

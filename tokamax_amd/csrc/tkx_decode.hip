@@ -1,5 +1,5 @@
-// Small-m ("decode") ragged dot: bf16 lhs [m,k] x int8 rhs [G,k,n] with f32 scales [G,n], or
-// bf16 x bf16 / f16 x f16 without scales.
+// Small-m ("decode") ragged dot: bf16 lhs [m,k] x int8 or fp8 (e4m3fn) rhs [G,k,n] with f32 scales [G,n],
+// or bf16 x bf16 / f16 x f16 without scales.
 //
 // This regime is bound by HBM: every touched expert's [k,n] weight panel is read once, and a group
 // has a handful of rows. The kernel is built around streaming those panels:
@@ -72,10 +72,11 @@ __device__ __forceinline__ i32x4 buffer_load_16_streaming(__amdgpu_buffer_rsrc_t
 // What a lane holds of one weight row of a step: its CPL columns (8, or 16 of int8).
 template <int EW, int CPL> struct WeightRow { typedef i32x4 T; static constexpr int ESZ = 2; };
 template <> struct WeightRow<kEI8, 8> { typedef i32x2 T; static constexpr int ESZ = 1; };
+template <> struct WeightRow<kEF8, 8> { typedef i32x2 T; static constexpr int ESZ = 1; };
 template <> struct WeightRow<kEI8, 16> { typedef i32x4 T; static constexpr int ESZ = 1; };
 template <int EW, int CPL>
 __device__ __forceinline__ typename WeightRow<EW, CPL>::T load_weight_row(__amdgpu_buffer_rsrc_t r, uint32_t lane_offset, uint32_t uniform_offset) {
-  if constexpr (EW == kEI8 && CPL == 8) return buffer_load_8(r, lane_offset, uniform_offset);
+  if constexpr ((EW == kEI8 || EW == kEF8) && CPL == 8) return buffer_load_8(r, lane_offset, uniform_offset);
   else return buffer_load_16_streaming(r, lane_offset, uniform_offset);
 }
 
@@ -104,14 +105,31 @@ __device__ __forceinline__ i32x4 column_fragment_i8(const Row (&rows)[8]) {
   }
   return out;
 }
+// fp8 (e4m3fn) weights: byte J of each row through the hardware conversion; an e4m3 value has 3
+// significand bits, so the upper half of its f32 is its bf16 exactly.
+template <int J>
+__device__ __forceinline__ i32x4 column_fragment_f8(const i32x2 (&rows)[8]) {
+  i32x4 out;
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    const unsigned f0 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_f32_fp8(rows[2 * h][J >> 2], J & 3));
+    const unsigned f1 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_f32_fp8(rows[2 * h + 1][J >> 2], J & 3));
+    out[h] = (int)__builtin_amdgcn_perm(f1, f0, 0x07060302u);
+  }
+  return out;
+}
 // Sub-channel scales: the same column, each value multiplied by the column's scale of the current
 // k-block and rounded to bf16 (nearest even).
-template <int J>
+template <int EW, int J>
 __device__ __forceinline__ i32x4 column_fragment_scaled(const i32x2 (&rows)[8], float scale) {
   bf16x8 out;
 #pragma unroll
-  for (int e = 0; e < 8; ++e)
-    out[e] = (__bf16)(__builtin_bit_cast(float, i8_to_f32_bits<(J & 3)>(rows[e][J >> 2])) * scale);
+  for (int e = 0; e < 8; ++e) {
+    float v;
+    if constexpr (EW == kEI8) v = __builtin_bit_cast(float, i8_to_f32_bits<(J & 3)>(rows[e][J >> 2]));
+    else v = __builtin_amdgcn_cvt_f32_fp8(rows[e][J >> 2], J & 3);
+    out[e] = (__bf16)(v * scale);
+  }
   return __builtin_bit_cast(i32x4, out);
 }
 // 16-bit weights: half-word J of each of 8 loaded 16-byte rows, two rows per byte permute.
@@ -142,9 +160,9 @@ __device__ __forceinline__ f32x4_t mma_16x16x32(i32x4 w, i32x4 a, f32x4_t acc) {
 // bytes per lane and the rows a wave reads 256 bytes long, the shape 16-bit weights have at CPL 8.
 template <int EW, int kDecDepth, int kMinWgs, bool SUB = false, int CPL = 8>
 __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const DecodeParams p) {
-  static_assert(!SUB || EW == kEI8, "sub-channel scales belong to int8 weights");
+  static_assert(!SUB || EW == kEI8 || EW == kEF8, "sub-channel scales belong to int8 or fp8 weights");
   static_assert(CPL == 8 || (CPL == 16 && EW == kEI8 && !SUB), "16 columns per lane: int8 weights with per-column scales");
-  constexpr int EA = EW == kEI8 ? kEBF16 : EW;
+  constexpr int EA = (EW == kEI8 || EW == kEF8) ? kEBF16 : EW;
   constexpr int WESZ = WeightRow<EW, CPL>::ESZ;
   constexpr int BN = 16 * CPL;
   typedef typename WeightRow<EW, CPL>::T WRow;
@@ -295,8 +313,9 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
         }
         auto column = [&](auto j_tag) {
           constexpr int J = decltype(j_tag)::value;
-          if constexpr (SUB) return column_fragment_scaled<J>(breg[d], col_scale[J]);
+          if constexpr (SUB) return column_fragment_scaled<EW, J>(breg[d], col_scale[J]);
           else if constexpr (EW == kEI8) return column_fragment_i8<J>(breg[d]);
+          else if constexpr (EW == kEF8) return column_fragment_f8<J>(breg[d]);
           else return column_fragment_16bit<J>(breg[d]);
         };
         // Four columns at a time: widen, then their MFMAs.
@@ -392,14 +411,14 @@ bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k
   }
   if (scale_blocks != 1) {
     // Sub-channel scales: int8 weights, blocks of a power-of-two number of rows that whole steps fit.
-    if (rhs_dtype != TKX_I8 || scale_blocks < 1 || k % scale_blocks != 0) return false;
+    if ((rhs_dtype != TKX_I8 && rhs_dtype != TKX_F8E4M3FN) || scale_blocks < 1 || k % scale_blocks != 0) return false;
     const int64_t rows = k / scale_blocks;
     if (rows % kDecKS != 0 || (rows & (rows - 1)) != 0 || scale_blocks * n * 4 >= (1LL << 31)) return false;
   }
-  const bool types = (lhs_dtype == TKX_BF16 && (rhs_dtype == TKX_I8 || rhs_dtype == TKX_BF16)) ||
+  const bool types = (lhs_dtype == TKX_BF16 && (rhs_dtype == TKX_I8 || rhs_dtype == TKX_F8E4M3FN || rhs_dtype == TKX_BF16)) ||
                      (lhs_dtype == TKX_F16 && rhs_dtype == TKX_F16);
   if (!types) return false;
-  const int64_t wesz = rhs_dtype == TKX_I8 ? 1 : 2;
+  const int64_t wesz = (rhs_dtype == TKX_I8 || rhs_dtype == TKX_F8E4M3FN) ? 1 : 2;
   if ((k / kDecWaves) * n * wesz >= (1LL << 31)) return false;
   return k % (kDecWaves * kDecKS * 8) == 0 && n % 8 == 0 && n >= 8;
 }
@@ -435,7 +454,13 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
   // `depth` = steps of loads in flight per wave; deeper pipelines need more registers and allow
   // fewer waves per CU. A step of 16-bit weights takes twice the registers of an int8 one.
   const void* fn;
-  if (sub) {
+  if (sub && rhs_dtype == TKX_F8E4M3FN) {
+    fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEF8, 2, 3, true>)
+                    : reinterpret_cast<const void*>(&decode_kernel<kEF8, 4, 2, true>);
+  } else if (rhs_dtype == TKX_F8E4M3FN) {
+    fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEF8, 2, 4>)
+                    : reinterpret_cast<const void*>(&decode_kernel<kEF8, 4, 3>);
+  } else if (sub) {
     fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 2, 3, true>)
                     : reinterpret_cast<const void*>(&decode_kernel<kEI8, 4, 2, true>);  // (8 deep would spill)
   } else if (rhs_dtype == TKX_I8 && block_n == 2 * kDecBN) {
