@@ -343,11 +343,19 @@ def test_every_kernel_variant_through_c_abi(v, device):
   lt, rt = _TORCH_DTYPE[v["lhs_dtype"]], _TORCH_DTYPE[v["rhs_dtype"]]
   mk = lambda shape, std: torch.tensor(rng.normal(0, std, shape).astype(np.float32), device=device)
   if v["mode"] == 3:  # forward with gate-up fusion and a bias: rhs [g, k, 2 n'] -> out [m, n']
-    lhs, rhs = mk((m, k), 1.0).to(lt), mk((G, k, n), k ** -0.5).to(rt)
+    lhs = mk((m, k), 1.0).to(lt)
     bias = mk((G, 1, n), 0.5)
+    scale = None
+    if rt == torch.int8:  # int8 weights with one scale per (group, column)
+      rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+      scale = mk((G, 1, n), 0.005).abs() + 1e-3
+      rhs_f = O.dequantize(rhs.cpu().numpy(), _np(scale))
+    else:
+      rhs = mk((G, k, n), k ** -0.5).to(rt)
+      rhs_f = _np(rhs)
     out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, rhs_bias=bias, activation="silu",
-                                 gateup=True)
-    want = O.ragged_dot_fused(_np(lhs), _np(rhs), gs, rhs_bias=_np(bias), gateup_activation="silu")
+                                 gateup=True, rhs_scale=scale)
+    want = O.ragged_dot_fused(_np(lhs), rhs_f, gs, rhs_bias=_np(bias), gateup_activation="silu")
     _check(out, want, 1e-5)
     assert out.shape == (m, n // 2) and torch.count_nonzero(out[int(gs.sum()):]) == 0
     return
@@ -539,6 +547,34 @@ def test_rhs_bias_and_gateup_fusion(m, k, n2, gs, act, device):
   _check(got, O.silu(plain), 1e-5)
   with pytest.raises(NotImplementedError):
     op(lhs, rhs, group_sizes=gst, fuse_gateup_activation="relu")
+
+
+@pytest.mark.parametrize("blocks", [1, 4])
+def test_gateup_fusion_over_int8_weights(blocks, device):
+  """Gate-up fusion with quantised weights (the reference's gmm_v2 test crosses `fuse_act` with `use_weight_scale`,
+  experimental/gmm_v2/gmm_v2_test.py:1158-1166): one scale per (group, column) runs on gate-up variants of the
+  int8-weight kernels; scales per k-block go through the widening pass and the bf16 gate-up kernels."""
+  rng = np.random.default_rng(13 + blocks)
+  m, k, n2 = 300, 256, 512
+  gs = np.array([100, 0, 57, 120], np.int32)
+  G = len(gs)
+  gst = torch.tensor(gs, device=device)
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  q = torch.tensor(rng.integers(-127, 128, (G, k, n2)).astype(np.int8), device=device)
+  scale = torch.tensor((rng.uniform(0.5, 1.5, (G, blocks, n2)) * k ** -0.5 / 127 * 2).astype(np.float32), device=device)
+  bias = torch.tensor(rng.normal(0, 0.7, (G, 1, n2)).astype(np.float32), device=device).to(torch.bfloat16)
+  rhs = tokamax_amd.QArray(q, scale)
+  op = tokamax_amd.HipRaggedDot()
+  want = O.ragged_dot_fused(_np(lhs), O.dequantize(q.cpu().numpy(), _np(scale)), gs, rhs_bias=_np(bias),
+                            gateup_activation="silu")
+  out = op(lhs, rhs, group_sizes=gst, rhs_bias=bias, fuse_gateup_activation="silu", preferred_element_type=torch.float32)
+  assert out.shape == (m, n2 // 2)
+  _check(out, want, 1e-5 if blocks == 1 else 4e-3)  # (widened weights are rounded to bf16)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  # the raw-array form of the same call
+  out2 = op(lhs, q, group_sizes=gst, rhs_scale=scale.reshape(G, blocks, 1, n2), rhs_bias=bias, fuse_gateup_activation="silu",
+            preferred_element_type=torch.float32)
+  assert torch.equal(out, out2)
 
 
 @pytest.mark.parametrize("act", ["swigluoai", "silu_and_mul_with_clamp", "gelu_tanh"])

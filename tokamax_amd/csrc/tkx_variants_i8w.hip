@@ -5,6 +5,8 @@
 
 namespace tkx {
 #define FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEBF16, kEI8, BM, BN, BK, WM, WN, NS)
+// Gate-up fusion over int8 weights [gate | up] with one scale per (group, column).
+#define GLU(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdGlu, kEBF16, kEI8, BM, BN, BK, WM, WN, NS)
 #define SUBK(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdSubK, kEBF16, kEI8, BM, BN, BK, WM, WN, NS)
 // The same with fp8 (e4m3fn) weights: bf16 activations x fp8 weights exist in this form only (one scale block
 // covers the case of one scale per (group, column)).
@@ -21,6 +23,9 @@ static const Variant kVariants[] = {
     FWD(32, 256, 64, 1, 4, 4),
     FWD(32, 128, 128, 1, 4, 4),
     FWD(32, 128, 128, 1, 4, 2),
+    GLU(256, 256, 64, 2, 4, 3),
+    GLU(128, 256, 64, 2, 4, 3),
+    GLU(32, 256, 64, 1, 4, 4),
     SUBK(256, 256, 64, 2, 4, 3),
     SUBK(256, 256, 32, 2, 4, 4),
     SUBK(128, 256, 64, 2, 4, 3),
