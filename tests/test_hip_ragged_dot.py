@@ -389,6 +389,13 @@ def test_every_kernel_variant_through_c_abi(v, device):
     lhs = mk((m, k), 1.0).to(lt)
     lhs_f = _np(lhs)
     tol = 1e-5
+  elif rt == torch.float8_e4m3fn and lt == torch.bfloat16:  # the streaming small-m kernel on fp8 weights
+    rhs = mk((G, k, n), 1.0).to(rt)
+    rhs_scale = mk((G, 1, n), 0.01).abs() + 1e-3
+    rhs_f = O.dequantize(O.e4m3fn_decode(rhs.view(torch.uint8).cpu().numpy()), _np(rhs_scale))
+    lhs = mk((m, k), 1.0).to(lt)
+    lhs_f = _np(lhs)
+    tol = 1e-5
   elif lt == torch.float8_e4m3fn:
     lhs, rhs = mk((m, k), 1.0).to(lt), mk((G, k, n), 1.0).to(rt)
     lhs_scale, rhs_scale = mk((m, 1), 0.1).abs() + 0.05, mk((G, 1, n), 0.1).abs() + 0.05
