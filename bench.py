@@ -285,7 +285,15 @@ def main():
     cfg = op.bind(ql, qr, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
     measure("mixtral_prefill_fp8", lambda: op(ql, qr, group_sizes=gs, preferred_element_type=torch.bfloat16), w.flops,
             w.algorithmic_bytes(), "mfma", "fp8", cfg)
-    del w, ql, qr
+    # the same operands with one scale per (row, 128 k) and per (group, 128 k, column): folded in after every k-block
+    genk = torch.Generator(device=device).manual_seed(2)
+    kb = w.k // 128
+    qlk = tokamax_amd.QArray(w.lhs, torch.rand(w.m, kb, device=device, generator=genk) + 0.5)
+    qrk = tokamax_amd.QArray(w.rhs, (torch.rand(w.num_groups, kb, w.n, device=device, generator=genk) + 0.5) / w.k ** 0.5)
+    cfg = op.bind(qlk, qrk, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_prefill_fp8_k_block_scales", lambda: op(qlk, qrk, group_sizes=gs, preferred_element_type=torch.bfloat16),
+            w.flops, w.algorithmic_bytes() + (w.m * kb + w.nonempty_groups * kb * w.n) * 4, "mfma", "fp8", cfg)
+    del w, ql, qr, qlk, qrk
 
     # the Mixtral shape with int8 weights (one f32 scale per (group, column)): the weight stream into LDS is half of bf16's
     w = workloads.make("mixtral", device, seed=0)

@@ -129,7 +129,9 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
  *   (TKX_ACT_SWIGLU_OAI and TKX_ACT_SILU_CLAMP need gateup = 1: TKX_ERR_INVALID otherwise).
  *   rhs_scale_blocks: rhs_scale is f32[G, rhs_scale_blocks, n], block b scaling the k rows
  *     [b * k/blocks, (b+1) * k/blocks) (scale tile (1, t_k, 1), pallas_mosaic_gpu_kernel_sm90_quant.py:91-97).
- *     1 = one scale per (group, column). bf16 x fp8 weights run on the variants of mode 4 only, with any number
+ *     1 = one scale per (group, column). fp8 x fp8 with more than 1: lhs_scale is then f32[rhs_scale_blocks, m]
+ *     (one scale per k-block and row), both operands' scales are folded in after every k-block (mode 4; m % 4 == 0).
+ *     bf16 x fp8 weights run on the variants of mode 4 only, with any number
  *     of blocks. More than 1 (int8 or fp8 weights, k/blocks a power of two): taken by the
  *     streaming small-m kernel (k/blocks >= 32) and by the tiled variants of mode 4 (block_k divides k/blocks;
  *     256-column tiles), which multiply each k-block's scales in while they widen the weights, to the same bits

@@ -359,6 +359,16 @@ def test_every_kernel_variant_through_c_abi(v, device):
     _check(out, want, 1e-5)
     assert out.shape == (m, n // 2) and torch.count_nonzero(out[int(gs.sum()):]) == 0
     return
+  if v["mode"] == 4 and lt == torch.float8_e4m3fn:  # fp8 x fp8, scales per block of 128 k rows on both sides, a bias
+    lhs, rhs = mk((m, k), 1.0).to(lt), mk((G, k, n), 1.0).to(rt)
+    xs, ws_ = mk((m, 2), 0.1).abs() + 0.05, mk((G, 2, n), 0.1).abs() + 0.05
+    bias = mk((G, 1, n), 0.5)
+    out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs, rhs_scale=ws_, rhs_bias=bias)
+    lhs_f = O.dequantize(O.e4m3fn_decode(lhs.view(torch.uint8).cpu().numpy()).astype(np.float64), _np(xs))
+    rhs_f = O.dequantize(O.e4m3fn_decode(rhs.view(torch.uint8).cpu().numpy()).astype(np.float64), _np(ws_))
+    _check(out, O.ragged_dot_fused(lhs_f, rhs_f, gs, rhs_bias=_np(bias)), 1e-4)
+    assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+    return
   if v["mode"] == 4:  # forward over int8 / fp8 weights with per-k-block scales (4 blocks of 64 rows) and a bias
     lhs = mk((m, k), 1.0).to(lt)
     if rt == torch.int8:
@@ -739,7 +749,7 @@ def test_dequantize_kernel_bit_exact(rows, cols, t_r, t_c, qdtype, device):
     np.testing.assert_array_equal(_np(got3).reshape(rows, cols), want)
 
 
-@pytest.mark.parametrize("case", ["fp8_blocks_128", "fp8_row_x_k_blocks", "int8_k_sub", "int8_row_col"])
+@pytest.mark.parametrize("case", ["fp8_blocks_128", "fp8_row_x_k_blocks", "fp8_k_sub", "int8_k_sub", "int8_row_col"])
 def test_k_subchannel_scales_through_widening(case, device):
   """Scales that change along the contraction on both operands -- the fp8 recipe with [m, k/128] and
   [g, k/128, n/128] scales, and the int8 activation form acc += (x_q . w_q) xs[row, k_sub] ws[g, k_sub, n]
@@ -762,6 +772,8 @@ def test_k_subchannel_scales_through_widening(case, device):
   lhs_spec, rhs_spec = {
       "fp8_blocks_128": (((m, k), f8, (m, k // 128), 1.0), ((G, k, n), f8, (G, k // 128, n // 128), k ** -0.5)),
       "fp8_row_x_k_blocks": (((m, k), f8, (m, 1), 1.0), ((G, k, n), f8, (G, k // 128, n), k ** -0.5)),
+      # (the same k-blocks on both sides: the fp8 MFMA kernel that folds the scales in after every k-block)
+      "fp8_k_sub": (((m, k), f8, (m, k // 128), 1.0), ((G, k, n), f8, (G, k // 128, n), k ** -0.5)),
       "int8_k_sub": (((m, k), i8, (m, k // 64), 1 / 127), ((G, k, n), i8, (G, k // 64, n), k ** -0.5 / 127)),
       "int8_row_col": (((m, k), i8, (m, 1), 1 / 127), ((G, k, n), i8, (G, 1, n), k ** -0.5 / 127)),
   }[case]

@@ -190,6 +190,12 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
                        " (k=%lld blocks=%lld block_k=%d); widen the weights with tkx_dequantize_weights otherwise",
                        (long long)k, (long long)rhs_scale_blocks, c.block_k);
   }
+  if (subk && lhs_dtype == TKX_F8E4M3FN) {
+    // fp8 x fp8: the lhs scales come per k-block too, as f32[rhs_scale_blocks, m].
+    if (lhs_scale == nullptr || m % 4 != 0 || c.align_tile % 4 != 0 || (uintptr_t)lhs_scale % 16 != 0)
+      return set_error(TKX_ERR_UNSUPPORTED,
+                       "fp8 x fp8 with scale blocks along k needs lhs scales f32[blocks, m], m %% 4 == 0 and align_tile %% 4 == 0");
+  }
   const Variant* v = find_variant(dlhs ? kDlhs : gateup ? kFwdGlu : subk ? kFwdSubK : kFwd, lhs_dtype, rhs_dtype, c);
   if (v == nullptr)
     return set_error(TKX_ERR_UNSUPPORTED, "no kernel variant for mode=%d dtypes=(%d,%d) tile=%dx%dx%d waves=%dx%d stages=%d",

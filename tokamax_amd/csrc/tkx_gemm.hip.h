@@ -463,8 +463,12 @@ struct GemmKernel {
   static constexpr int LB = (MODE == kDlhs) ? kKC : kMC;
   static constexpr bool GLU = MODE == kFwdGlu;
   static constexpr bool SUBK = MODE == kFwdSubK;
-  static_assert(!SUBK || ((EB == kEI8 || EB == kEF8) && EA == kEBF16 && BN == 256),
-                "per-k-block scales: bf16 lhs, int8 or fp8 weights, one 1 KB scale row per k-step");
+  // fp8 x fp8 with scales per k-block on both sides (xs[row, k_sub] ws[g, k_sub, n],
+  // pallas_mosaic_gpu_kernel_sm100_i8_quant.py:51-102): the MFMAs of a k-step (= one k-block or a part of one)
+  // accumulate into partial accumulators, which are folded into the result with the block's scales.
+  static constexpr bool SUBP = SUBK && EA == kEF8;
+  static_assert(!SUBK || ((EB == kEI8 || EB == kEF8) && (EA == kEBF16 || (SUBP && EB == kEF8)) && BN == 256),
+                "per-k-block scales: bf16 lhs with int8 or fp8 weights, or fp8 x fp8; one 1 KB scale row per k-step");
   static constexpr int BNO = GLU ? BN / 2 : BN;  // output columns of a tile
   static constexpr int EC = EA;  // MFMA type follows A; B may be stored narrower (int8 weights)
   static constexpr int KA = Mma<EC>::KA;
@@ -481,9 +485,12 @@ struct GemmKernel {
   static constexpr int NLOAD = WM * WN;
   typedef DirectLoader<LA, EA, BM, BK, NLOAD> DirA;
   typedef DirectLoader<LB, EB, BN, BK, NLOAD> DirB;
-  static constexpr int SCALE_BYTES = SUBK ? BN * 4 : 0;  // kFwdSubK: the k-step's scale row behind its two tiles
+  static constexpr int SCALE_BYTES = (SUBK && !SUBP) ? BN * 4 : 0;  // kFwdSubK: the k-step's scale row behind its two tiles
   static constexpr int STAGE_BYTES = StageA::BYTES + StageB::BYTES + SCALE_BYTES;
-  static constexpr int SMEM_BYTES = NS * STAGE_BYTES;
+  // fp8 x fp8: the scales of a k-step (BN weight-column scales, then BM lhs-row scales) are still needed when its
+  // stage is already being refilled, so they live in a ring of NS + 1 slots behind the stages.
+  static constexpr int RING_SLOT = SUBP ? (BN + BM) * 4 : 0;
+  static constexpr int SMEM_BYTES = NS * STAGE_BYTES + (NS + 1) * RING_SLOT;
   static_assert(NS >= 2 && SMEM_BYTES <= 160 * 1024, "stages must fit the 160 KB LDS");
 
   static __device__ __forceinline__ void run(const GemmParams& p, unsigned char* smem) {
@@ -565,6 +572,7 @@ struct GemmKernel {
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
+    f32x16 pacc[SUBP ? TM : 1][SUBP ? TN : 1];  // (fp8 x fp8 with k-block scales) the current k-step's products
     typedef typename Mma<EC>::Frag Frag;
     // Row blocks (32 rows) of this wave that hold at least one row the task stores. A task at a
     // group boundary can have only a few such rows; the blocks without any skip their LDS reads and
@@ -581,7 +589,7 @@ struct GemmKernel {
     // B fragment j of k-atom kk of a stage. kFwdSubK: the int8 values of the lane's column (lane % 32 of the
     // block) are multiplied by that column's scale for the stage's k-block, which lies behind the tiles.
     auto load_b_frag = [&](const unsigned char* stage, int j, int kk) -> Frag {
-      if constexpr (SUBK) {
+      if constexpr (SUBK && !SUBP) {
         const int blk = lane >> 4, s_ = lane & 15;
         const int col = wn * WTN + j * 32 + 16 * (blk & 1) + 8 * (s_ & 1);
         const int krow = kk * KA + 8 * (blk >> 1) + (s_ >> 1);
@@ -642,23 +650,35 @@ struct GemmKernel {
       // on its own, so that the list can be threaded between MFMAs. kFwdSubK adds one: the 1 KB scale
       // row of the step's k-block, of which every wave fetches its 1/NLOAD with that many of its lanes
       // (so that all waves count the same number of loads).
-      constexpr int NLD = DirA::PER + DirB::PER + (SUBK ? 1 : 0);
+      constexpr int NLD = DirA::PER + DirB::PER + (SUBP ? 2 : SUBK ? 1 : 0);
       constexpr int kInFlight = kExact ? (NS - 2) * NLD : 0;
       static_assert(kInFlight < 64 && (NS - 1) * NLD < 64, "too many direct loads in flight for vmcnt");
-      struct StepPtrs { const unsigned char *a, *b, *s; unsigned lds; };
+      struct StepPtrs { const unsigned char *a, *b, *s, *x; unsigned lds, ring; };
       // (kFwdSubK) scales of this tile's columns: row `block` of the group's [scale_blocks, n] table; lanes past
       // the last column re-read the last four (their products are never stored).
       const unsigned char* const gS0 =
           SUBK ? reinterpret_cast<const unsigned char*>(p.b_scale + (int64_t)group * p.scale_blocks * p.nb_ext) : nullptr;
       constexpr int SCALE_LANES = 64 / NLOAD;  // lanes of a wave that fetch 16 bytes of the scale row each
       const uint32_t scale_voff = SUBK ? (uint32_t)min(col0 + 4 * (wave * SCALE_LANES + lane), p.nb_ext - 4) * 4u : 0u;
+      // (fp8 x fp8) lhs scales [scale_blocks, m]: the BM rows of the tile, 4 per lane; chunks past the last row
+      // re-read the last four (m and row0 are multiples of 4, so a chunk is all inside or all outside).
+      constexpr int XS_LANES = BM / 4 / NLOAD;
+      static_assert(!SUBP || BM / 4 % NLOAD == 0, "the lhs scales of a tile split evenly over the load waves");
+      const uint32_t xs_voff = SUBP ? (uint32_t)min(row0 + 4 * (wave * XS_LANES + lane), p.m_ext - 4) * 4u : 0u;
       auto step_ptrs = [&](int step, int stage) {
         StepPtrs sp;
         sp.a = uniform_pointer(gA0 + step * stepA);
         sp.b = uniform_pointer(gB0 + step * stepB);
-        sp.s = nullptr;
-        if constexpr (SUBK)
-          sp.s = uniform_pointer(gS0 + (int64_t)((kc_begin + step * BK) >> p.log2_block_rows) * p.nb_ext * 4);
+        sp.s = sp.x = nullptr;
+        sp.ring = 0;
+        if constexpr (SUBK) {
+          const int64_t block = (kc_begin + step * BK) >> p.log2_block_rows;
+          sp.s = uniform_pointer(gS0 + block * p.nb_ext * 4);
+          if constexpr (SUBP) {
+            sp.x = uniform_pointer(reinterpret_cast<const unsigned char*>(p.a_scale) + block * p.m_ext * 4);
+            sp.ring = smem_lds + NS * STAGE_BYTES + (step % (NS + 1)) * RING_SLOT;
+          }
+        }
         sp.lds = smem_lds + stage * STAGE_BYTES;
         return sp;
       };
@@ -666,8 +686,10 @@ struct GemmKernel {
         if (q < DirA::PER) da.issue_one(q, sp.a, sp.lds, wave);
         else if (q < DirA::PER + DirB::PER) db.issue_one(q - DirA::PER, sp.b, sp.lds + StageA::BYTES, wave);
         else if (SUBK && q == DirA::PER + DirB::PER) {
-          if (lane < SCALE_LANES)
-            direct_load_16(sp.s, scale_voff, sp.lds + StageA::BYTES + StageB::BYTES + wave * (SCALE_LANES * 16));
+          const unsigned dst = SUBP ? sp.ring : sp.lds + StageA::BYTES + StageB::BYTES;
+          if (lane < SCALE_LANES) direct_load_16(sp.s, scale_voff, dst + wave * (SCALE_LANES * 16));
+        } else if (SUBP && q == DirA::PER + DirB::PER + 1) {
+          if (lane < XS_LANES) direct_load_16(sp.x, xs_voff, sp.ring + BN * 4 + wave * (XS_LANES * 16));
         }
       };
       // Every wave drains the loads the next k-step needs before it arrives at a barrier.
@@ -721,15 +743,27 @@ struct GemmKernel {
         // (`reads` and `loads` are compile-time tags: a run-time test after every MFMA would put two
         // branches into each MFMA slot.)
         auto atom = [&](auto reads_tag, auto loads_tag, const Frag* a, const Frag* b, Frag* na, Frag* nb,
-                        const unsigned char* rd_stage, int rd_kk, const StepPtrs& sp) {
+                        const unsigned char* rd_stage, int rd_kk, const StepPtrs& sp, auto first_tag) {
           constexpr bool reads = decltype(reads_tag)::value, loads = decltype(loads_tag)::value;
+          constexpr bool first_of_step = decltype(first_tag)::value;  // (SUBP) the partial accumulators start at zero
 #pragma unroll
           for (int t = 0; t < NM; ++t) {
             const int i = t / TN, j = t % TN;
 #if defined(TKX_ABLATE) && (TKX_ABLATE & 4)
             asm volatile("" ::"v"(a[i]), "v"(b[j]));
 #else
-            if (F || ((rmask >> i) & 1u)) acc[i][j] = mma_atom<EC>(b[j], a[i], acc[i][j]);
+            if (F || ((rmask >> i) & 1u)) {
+              if constexpr (SUBP) {
+                f32x16 c = pacc[i][j];
+                if constexpr (first_of_step) {
+#pragma unroll
+                  for (int e = 0; e < 16; ++e) c[e] = 0.f;
+                }
+                pacc[i][j] = mma_atom<EC>(b[j], a[i], c);
+              } else {
+                acc[i][j] = mma_atom<EC>(b[j], a[i], acc[i][j]);
+              }
+            }
 #endif
             if (reads) {
 #pragma unroll
@@ -756,15 +790,38 @@ struct GemmKernel {
           const unsigned char* nxt = smem + cur_stage * STAGE_BYTES;
           // (Pointers of the refill are computed here, far ahead of the MFMAs they are issued between.)
           const StepPtrs sp = decltype(refill_tag)::value ? step_ptrs(kt + NS, freed) : none;
+          static_assert(!SUBP || KSTEPS == 2, "the partial accumulators restart with the first of two atoms");
+          atom(std::true_type{}, std::false_type{}, fa[0], fb[0], fa[1], fb[1], cur, 1, none, std::true_type{});
 #pragma unroll
-          for (int kk = 0; kk + 1 < KSTEPS; ++kk)
+          for (int kk = 1; kk + 1 < KSTEPS; ++kk)
             atom(std::true_type{}, std::false_type{}, fa[kk & 1], fb[kk & 1], fa[(kk + 1) & 1], fb[(kk + 1) & 1], cur,
-                 kk + 1, none);
+                 kk + 1, none, std::false_type{});
           // All LDS reads of `cur` are issued. After the barrier the next stage is complete and `cur`
           // is free: the last atom's MFMAs cover the first fragment reads of the next stage and the
           // issue of the loads that refill `cur` with k-step kt + NS.
           step_barrier(decltype(refill_tag)::value || kt + NS - 1 < nfull);
-          atom(more_tag, refill_tag, fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1], fa[0], fb[0], nxt, 0, sp);
+          atom(more_tag, refill_tag, fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1], fa[0], fb[0], nxt, 0, sp, std::false_type{});
+          if constexpr (SUBP) {
+            // Fold the k-step's products into the result with the scales of its k-block: lane l holds row l % 32
+            // and, for t = 0..3, columns 8 t + 4 (l / 32) + {0..3} of every 32 x 32 block.
+            const unsigned char* slot = smem + NS * STAGE_BYTES + (kt % (NS + 1)) * RING_SLOT;
+            float xs[TM];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+              xs[i] = *reinterpret_cast<const float*>(slot + BN * 4 + 4 * (row_block(i) * 32 + (lane & 31)));
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                const f32x4 wsc = *reinterpret_cast<const f32x4*>(slot + 4 * (wn * WTN + j * 32 + 8 * t + 4 * (lane >> 5)));
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                  if (F || ((rmask >> i) & 1u)) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][j][4 * t + e] += pacc[i][j][4 * t + e] * (xs[i] * wsc[e]);
+                  }
+              }
+          }
         };
         // Steady state first (every step refills), then the last NS steps in loops of their own, so
         // that the hot loop is one straight-line body.
@@ -807,7 +864,7 @@ struct GemmKernel {
         const int c = GLU ? (j < TNO ? 0 : p.n_ext) + col0 + wn * WTNO + (j % TNO) * 32 : col0 + wn * WTN + j * 32;
         return min(c + 4 * (lane >> 5) + 8 * t, p.nb_ext - 4);
       };
-      if (p.a_scale != nullptr) {
+      if (!SUBP && p.a_scale != nullptr) {  // (SUBP: folded in per k-block)
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
           const int row = min(row0 + row_block(i) * 32 + (lane & 31), p.m_ext - 1);

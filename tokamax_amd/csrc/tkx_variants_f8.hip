@@ -1,4 +1,5 @@
-// OCP fp8 (e4m3fn) x fp8 forward variants; per-row / per-(group, column) scales in the epilogue.
+// OCP fp8 (e4m3fn) x fp8 forward variants; per-row / per-(group, column) scales in the epilogue, or
+// (kFwdSubK) scales per k-block on both operands folded in after every k-step.
 #include "tkx_gemm.hip.h"
 
 namespace tkx {
@@ -11,6 +12,7 @@ static const Variant kVariants[] = {
     FWD(128, 128, 128, 2, 2, 4),
     FWD(64, 128, 128, 2, 2, 4),
     FWD(32, 128, 128, 1, 4, 4),
+    TKX_VARIANT(kFwdSubK, kEF8, kEF8, 128, 256, 128, 2, 4, 3),
 };
 
 const Variant* variants_f8(int* count) {

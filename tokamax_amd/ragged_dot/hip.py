@@ -140,6 +140,13 @@ def _widening_plan(lhs, rhs, allow_native: bool = True) -> tuple[bool, bool, boo
                                 f" {tuple(rhs.scale.shape)}")
     widen_rhs = blocks is None or blocks > 1
   eight_bit_float = lambda x: _dtype_of(x) == torch.float8_e4m3fn
+  if (lhs_q and rhs_q and allow_native and eight_bit_float(lhs) and eight_bit_float(rhs) and blocks is not None
+      and blocks > 1 and _lhs_scale_blocks(lhs) == blocks):
+    # fp8 x fp8 with the same k-blocks on both sides: the fp8 MFMA kernel that folds the scales in per k-block.
+    m, k = lhs.qvalue.shape
+    rows = k // blocks
+    if rows % 128 == 0 and rows & (rows - 1) == 0 and m % 4 == 0 and rhs.qvalue.shape[2] % 16 == 0:
+      return False, False, True
   if rhs_q and allow_native and blocks is not None and rhs.qvalue.dtype in (torch.int8, torch.float8_e4m3fn):
     # Kernels of their own (bf16 lhs; 256-column tiles) for int8 weights with several scale blocks along k and
     # for fp8 weights with any number of them, unless fp8 meets fp8 with one scale each (the fp8 MFMA kernels).

@@ -156,10 +156,16 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
     raise NotImplementedError("bias and gate-up fusion need the default dimension numbers")
   if gateup and n % 2:
     raise ValueError("gate-up fusion needs an even number of rhs columns")
+  lhs_scale_blocks = 1
   if lhs_scale is not None:
-    lhs_scale = lhs_scale.to(torch.float32).contiguous().view(-1)
-    if lhs_scale.numel() != m:
-      raise NotImplementedError("lhs scale must be one f32 per row")
+    if lhs_scale.dim() == 2 and lhs_scale.shape[1] > 1:
+      # One scale per (row, k-block): the kernels take them as [k-blocks, m].
+      lhs_scale_blocks = int(lhs_scale.shape[1])
+      lhs_scale = lhs_scale.to(torch.float32).t().contiguous().view(-1)
+    else:
+      lhs_scale = lhs_scale.to(torch.float32).contiguous().view(-1)
+    if lhs_scale.numel() != m * lhs_scale_blocks:
+      raise NotImplementedError("lhs scale must be one f32 per row (or per row and k-block)")
   scale_blocks = 1
   if rhs_scale is not None:
     if rhs_scale.dim() == 3 and rhs_scale.shape[1] > 1:
@@ -167,6 +173,8 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
     rhs_scale = rhs_scale.to(torch.float32).contiguous().view(-1)
     if rhs_scale.numel() != G * scale_blocks * n or k % scale_blocks:
       raise NotImplementedError("rhs scale must be one f32 per (group, column) or per (group, k-block, column)")
+  if lhs_scale_blocks != 1 and lhs_scale_blocks != scale_blocks:
+    raise NotImplementedError("lhs and rhs scales must have the same number of blocks along k")
   if rhs_bias is not None:
     rhs_bias = rhs_bias.to(torch.float32).contiguous().view(-1)
     if rhs_bias.numel() != G * n:
