@@ -234,11 +234,10 @@ def test_vjp(m, k, n, activation, device):
 
 
 @pytest.mark.parametrize("b_tile_shape,supported", [((1, 256, 1), True), ((1, 16, 1), True), ((1, 1, 16), True),
-                                                    ((1, 64, 32), True), ((1, 1, 8), False), ((2, 1, 1), False)])
+                                                    ((1, 64, 32), True), ((1, 1, 8), True), ((2, 1, 1), False)])
 def test_quantized_int8_weights(b_tile_shape, supported, device):
   """bf16 x int8: per-(group, column) scales run in the kernels' epilogue, sub-channel scales along k and
-  scale tiles of a multiple of 16 columns along n through the widening pass; narrower tiles along n and
-  scales shared between groups are declined."""
+  scale tiles along n are repeated over their columns first; scales shared between groups are declined."""
   G, m, k, n = 8, 512, 256, 512
   a, _, gs = _inputs("test_quantized", G, m, k, n, torch.bfloat16, device, random_groups=True)
   rng = np.random.default_rng(11)

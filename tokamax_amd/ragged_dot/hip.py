@@ -104,6 +104,21 @@ def _rhs_scale_tiles(q: QArray) -> bool:
           and n % shape[2] == 0 and (n // shape[2]) % 16 == 0)
 
 
+def _per_column_rhs_scale(rhs):
+  """A quantised rhs whose scale is tiled along n ([g, k/t_k, n/t_n], e.g. 128 x 128 blocks) with every scale
+  repeated over its t_n columns ([g, k/t_k, n]): the form the kernels take. Works on tensors and on shapes."""
+  if not isinstance(rhs, QArray) or len(rhs.scale.shape) != 3 or len(rhs.qvalue.shape) != 3:
+    return rhs
+  n, nt = rhs.qvalue.shape[2], rhs.scale.shape[2]
+  if nt == n or nt < 1 or n % nt != 0 or rhs.scale.shape[0] != rhs.qvalue.shape[0]:
+    return rhs
+  if isinstance(rhs.scale, torch.Tensor):
+    scale = rhs.scale.repeat_interleave(n // nt, dim=2)
+  else:
+    scale = ShapeDtype((rhs.scale.shape[0], rhs.scale.shape[1], n), rhs.scale.dtype)
+  return QArray(rhs.qvalue, scale, rhs.zero_point, rhs.qtype)
+
+
 def _lhs_scale_blocks(q: QArray) -> int | None:
   """Number of scale blocks along k of a quantised lhs [m,k] (scale [m, blocks], blocks of a multiple of 16
   columns), or None if the scale has another form."""
@@ -259,6 +274,7 @@ class HipRaggedDot(base.RaggedDot):
       rhs = QArray(rhs, rhs_scale.reshape(g, rhs_scale.shape[1], n))
       if preferred_element_type is None:
         preferred_element_type = lhs.dtype
+    rhs = _per_column_rhs_scale(rhs)
     if group_offset is not None and ragged_dot_dimension_numbers != base.DEFAULT_RAGGED_DOT_DIM_NUMS:
       raise NotImplementedError("group_offset needs the default dimension numbers.")
     # rhs_bias and fuse_gateup_activation (base.py:205-217) are fused into the forward kernel's epilogue.
@@ -409,6 +425,7 @@ class HipRaggedDot(base.RaggedDot):
       g_, blocks_, _, n_ = raw_scale.shape
       rhs = QArray(rhs, ShapeDtype((g_, blocks_, n_), raw_scale.dtype))
     if mode in (0, 3):
+      rhs = _per_column_rhs_scale(rhs)
       widen_lhs, widen_rhs, native_k_blocks = _widening_plan(lhs, rhs, allow_native=mode == 0)
       lhs_dt = torch.bfloat16 if widen_lhs else lhs_dt
       rhs_dt = torch.bfloat16 if widen_rhs else rhs_dt
