@@ -818,6 +818,16 @@ def test_small_m_kernel_fp8_weights(blocks, depth, device):
     assert op._get_heuristics_config(op.bind(lhs[:19], rhs, group_sizes=sgt)).block_m == 16
     got = op(lhs[:19], rhs, group_sizes=sgt, preferred_element_type=torch.float32)
     _check(got, O.ragged_dot(_np(lhs[:19]), O.dequantize(qf, _np(scale)), small, acc_dtype=np.float64, out_dtype="f64"), 4e-3)
+    # an fp8 lhs with scales per (row, k-block) is widened for the same kernel (20 rows: a multiple of 4)
+    a8 = torch.tensor(rng.normal(0, 1, (20, k)).astype(np.float32), device=device).to(torch.float8_e4m3fn)
+    xs = torch.tensor(rng.uniform(0.5, 1.5, (20, blocks)).astype(np.float32), device=device)
+    lq = tokamax_amd.QArray(a8, xs)
+    # (with one scale per row and per column the pair stays on the fp8 MFMA kernels)
+    assert (op._get_heuristics_config(op.bind(lq, rhs, group_sizes=sgt)).block_m == 16) == (blocks > 1)
+    got = op(lq, rhs, group_sizes=sgt, preferred_element_type=torch.float32)
+    lhs_f = O.dequantize(O.e4m3fn_decode(a8.view(torch.uint8).cpu().numpy()).astype(np.float64), _np(xs))
+    _check(got, O.ragged_dot(lhs_f, O.dequantize(qf, _np(scale)), small, acc_dtype=np.float64, out_dtype="f64"), 6e-3,
+           rows=int(small.sum()))
 
 
 def test_bf16_activations_fp8_weights(device):

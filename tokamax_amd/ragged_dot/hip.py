@@ -160,7 +160,9 @@ def _widening_plan(lhs, rhs, allow_native: bool = True) -> tuple[bool, bool, boo
     # fp8 x fp8 with the same k-blocks on both sides: the fp8 MFMA kernel that folds the scales in per k-block.
     m, k = lhs.qvalue.shape
     rows = k // blocks
-    if rows % 128 == 0 and rows & (rows - 1) == 0 and m % 4 == 0 and rhs.qvalue.shape[2] % 16 == 0:
+    # (Groups of a few rows are better off with a widened lhs and the streaming small-m kernel, below.)
+    if (rows % 128 == 0 and rows & (rows - 1) == 0 and m % 4 == 0 and rhs.qvalue.shape[2] % 16 == 0
+        and m > 8 * rhs.qvalue.shape[0]):
       return False, False, True
   if rhs_q and allow_native and blocks is not None and rhs.qvalue.dtype in (torch.int8, torch.float8_e4m3fn):
     # Kernels of their own (bf16 lhs; 256-column tiles) for int8 weights with several scale blocks along k and
