@@ -13,6 +13,8 @@ static const Variant kVariants[] = {
     FWD(64, 128, 128, 2, 2, 4),
     FWD(32, 128, 128, 1, 4, 4),
     TKX_VARIANT(kFwdSubK, kEF8, kEF8, 128, 256, 128, 2, 4, 3),
+    TKX_VARIANT(kFwdSubK, kEF8, kEF8, 64, 256, 128, 2, 2, 3),
+    TKX_VARIANT(kFwdSubK, kEF8, kEF8, 32, 256, 128, 1, 4, 3),
 };
 
 const Variant* variants_f8(int* count) {
