@@ -669,15 +669,13 @@ struct GemmKernel {
         StepPtrs sp;
         sp.a = uniform_pointer(gA0 + step * stepA);
         sp.b = uniform_pointer(gB0 + step * stepB);
-        sp.s = sp.x = nullptr;
-        sp.ring = 0;
-        if constexpr (SUBK) {
+        sp.s = nullptr;
+        if constexpr (SUBK)
+          sp.s = uniform_pointer(gS0 + (int64_t)((kc_begin + step * BK) >> p.log2_block_rows) * p.nb_ext * 4);
+        if constexpr (SUBP) {
           const int64_t block = (kc_begin + step * BK) >> p.log2_block_rows;
-          sp.s = uniform_pointer(gS0 + block * p.nb_ext * 4);
-          if constexpr (SUBP) {
-            sp.x = uniform_pointer(reinterpret_cast<const unsigned char*>(p.a_scale) + block * p.m_ext * 4);
-            sp.ring = smem_lds + NS * STAGE_BYTES + (step % (NS + 1)) * RING_SLOT;
-          }
+          sp.x = uniform_pointer(reinterpret_cast<const unsigned char*>(p.a_scale) + block * p.m_ext * 4);
+          sp.ring = smem_lds + NS * STAGE_BYTES + (step % (NS + 1)) * RING_SLOT;
         }
         sp.lds = smem_lds + stage * STAGE_BYTES;
         return sp;
@@ -752,17 +750,17 @@ struct GemmKernel {
 #if defined(TKX_ABLATE) && (TKX_ABLATE & 4)
             asm volatile("" ::"v"(a[i]), "v"(b[j]));
 #else
-            if (F || ((rmask >> i) & 1u)) {
-              if constexpr (SUBP) {
+            if constexpr (SUBP) {
+              if (F || ((rmask >> i) & 1u)) {
                 f32x16 c = pacc[i][j];
                 if constexpr (first_of_step) {
 #pragma unroll
                   for (int e = 0; e < 16; ++e) c[e] = 0.f;
                 }
                 pacc[i][j] = mma_atom<EC>(b[j], a[i], c);
-              } else {
-                acc[i][j] = mma_atom<EC>(b[j], a[i], acc[i][j]);
               }
+            } else {
+              if (F || ((rmask >> i) & 1u)) acc[i][j] = mma_atom<EC>(b[j], a[i], acc[i][j]);
             }
 #endif
             if (reads) {
@@ -791,11 +789,14 @@ struct GemmKernel {
           // (Pointers of the refill are computed here, far ahead of the MFMAs they are issued between.)
           const StepPtrs sp = decltype(refill_tag)::value ? step_ptrs(kt + NS, freed) : none;
           static_assert(!SUBP || KSTEPS == 2, "the partial accumulators restart with the first of two atoms");
-          atom(std::true_type{}, std::false_type{}, fa[0], fb[0], fa[1], fb[1], cur, 1, none, std::true_type{});
+          if constexpr (SUBP) {
+            atom(std::true_type{}, std::false_type{}, fa[0], fb[0], fa[1], fb[1], cur, 1, none, std::true_type{});
+          } else {
 #pragma unroll
-          for (int kk = 1; kk + 1 < KSTEPS; ++kk)
-            atom(std::true_type{}, std::false_type{}, fa[kk & 1], fb[kk & 1], fa[(kk + 1) & 1], fb[(kk + 1) & 1], cur,
-                 kk + 1, none, std::false_type{});
+            for (int kk = 0; kk + 1 < KSTEPS; ++kk)
+              atom(std::true_type{}, std::false_type{}, fa[kk & 1], fb[kk & 1], fa[(kk + 1) & 1], fb[(kk + 1) & 1], cur,
+                   kk + 1, none, std::false_type{});
+          }
           // All LDS reads of `cur` are issued. After the barrier the next stage is complete and `cur`
           // is free: the last atom's MFMAs cover the first fragment reads of the next stage and the
           // issue of the loads that refill `cur` with k-step kt + NS.
