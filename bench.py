@@ -41,8 +41,8 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script, each scaled by what the same counter reads for a copy kernel of known size; None
 # where no counter run has been made for the current kernel.
+MEASURED_TRAFFIC_BYTES = {
     "mixtral": 4.19e9,  # 256x256x32 kernel: 3.60e9 read + 0.60e9 written past L2 (algorithmic: 1.543e9)
-    "mixtral": 4.21e9,  # 256x256x32 kernel: 3.62e9 read + 0.60e9 written past L2 (algorithmic: 1.543e9)
     "decode": 1.838e8,  # streaming int8 kernel: 1.834e8 read + 3.9e5 written (algorithmic: 1.748e8)
 }
 
