@@ -110,7 +110,7 @@ int32_t tkx_ragged_dot_schedule(const int32_t* group_sizes, int64_t num_groups, 
  * lhs_scale: f32[m] per-row scale or NULL; rhs_scale: f32[G,n] per-(group, column) scale or NULL
  * (both applied to the f32 accumulator in the epilogue; DEFAULT mode only).
  * Supported (lhs_dtype, rhs_dtype): (f32,f32) (bf16,bf16) (f16,f16) (f8e4m3fn,f8e4m3fn) (bf16,i8), and
- * (bf16,f8e4m3fn) with an rhs scale in DEFAULT mode.
+ * (bf16,f8e4m3fn) with an rhs scale and (i8,i8) with both scales, in DEFAULT mode.
  * out_dtype: f32, bf16 or f16. Rows >= sum(group_sizes) of `out` are set to zero.
  * Runs the schedule kernel itself (workspace must hold tkx_ragged_dot_workspace_bytes bytes). */
 int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* group_sizes,
@@ -129,7 +129,8 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
  *   (TKX_ACT_SWIGLU_OAI and TKX_ACT_SILU_CLAMP need gateup = 1: TKX_ERR_INVALID otherwise).
  *   rhs_scale_blocks: rhs_scale is f32[G, rhs_scale_blocks, n], block b scaling the k rows
  *     [b * k/blocks, (b+1) * k/blocks) (scale tile (1, t_k, 1), pallas_mosaic_gpu_kernel_sm90_quant.py:91-97).
- *     1 = one scale per (group, column). fp8 x fp8 with more than 1: lhs_scale is then f32[rhs_scale_blocks, m]
+ *     1 = one scale per (group, column). int8 x int8 (any number of blocks; m % 4 == 0) and fp8 x fp8 with more
+ *     than 1: lhs_scale is then f32[rhs_scale_blocks, m]
  *     (one scale per k-block and row), both operands' scales are folded in after every k-block (mode 4; m % 4 == 0).
  *     bf16 x fp8 weights run on the variants of mode 4 only, with any number
  *     of blocks. More than 1 (int8 or fp8 weights, k/blocks a power of two): taken by the

@@ -368,6 +368,18 @@ def test_every_kernel_variant_through_c_abi(v, device):
     _check(out, O.ragged_dot_fused(lhs_f, rhs_f, gs, rhs_bias=_np(bias)), 1e-4)
     assert torch.count_nonzero(out[int(gs.sum()):]) == 0
     return
+  if v["mode"] == 4 and lt == torch.int8:  # int8 x int8 on the int8 MFMAs, scales per block of 64 k rows on both sides
+    lhs = torch.tensor(rng.integers(-127, 128, (m, k)).astype(np.int8), device=device)
+    rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+    for blocks in (k // v["block_k"], 1):  # scale blocks of one k-step (128 or 64 rows), and one block
+      xs, ws_ = mk((m, blocks), 0.01).abs() + 0.005, mk((G, blocks, n), 0.01).abs() + 0.005
+      bias = mk((G, 1, n), 0.5)
+      out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs, rhs_scale=ws_, rhs_bias=bias)
+      lhs_f = O.dequantize(lhs.cpu().numpy().astype(np.float64), _np(xs))
+      rhs_f = O.dequantize(rhs.cpu().numpy().astype(np.float64), _np(ws_))
+      _check(out, O.ragged_dot_fused(lhs_f, rhs_f, gs, rhs_bias=_np(bias)), 1e-5)  # int32 sums are exact
+      assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+    return
   if v["mode"] == 4:  # forward over int8 / fp8 weights with per-k-block scales (4 blocks of 64 rows) and a bias
     lhs = mk((m, k), 1.0).to(lt)
     if rt == torch.int8:

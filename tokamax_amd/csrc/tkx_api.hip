@@ -174,7 +174,11 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
   const bool a16w8f = lhs_dtype == TKX_BF16 && rhs_dtype == TKX_F8E4M3FN;
   if (a16w8f && (rhs_scale == nullptr || dlhs))
     return set_error(TKX_ERR_UNSUPPORTED, "bf16 x fp8 weights: default mode with an rhs scale only");
-  const bool subk = rhs_scale != nullptr && (rhs_scale_blocks != 1 || a16w8f) && !dlhs && c.block_m != kDecodeBlockM;
+  // int8 x int8 likewise (the int8 MFMA kernels fold both operands' scales in per k-block).
+  const bool a8w8 = lhs_dtype == TKX_I8 && rhs_dtype == TKX_I8;
+  if (a8w8 && (rhs_scale == nullptr || lhs_scale == nullptr || dlhs))
+    return set_error(TKX_ERR_UNSUPPORTED, "int8 x int8: default mode with lhs and rhs scales only");
+  const bool subk = rhs_scale != nullptr && (rhs_scale_blocks != 1 || a16w8f || a8w8) && !dlhs && c.block_m != kDecodeBlockM;
   int32_t log2_block_rows = 0;
   if (subk && rhs_scale_blocks == 1) {
     log2_block_rows = 30;  // every k-step falls into block 0
@@ -190,8 +194,8 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
                        " (k=%lld blocks=%lld block_k=%d); widen the weights with tkx_dequantize_weights otherwise",
                        (long long)k, (long long)rhs_scale_blocks, c.block_k);
   }
-  if (subk && lhs_dtype == TKX_F8E4M3FN) {
-    // fp8 x fp8: the lhs scales come per k-block too, as f32[rhs_scale_blocks, m].
+  if (subk && (lhs_dtype == TKX_F8E4M3FN || lhs_dtype == TKX_I8)) {
+    // fp8 x fp8, int8 x int8: the lhs scales come per k-block too, as f32[rhs_scale_blocks, m].
     if (lhs_scale == nullptr || m % 4 != 0 || c.align_tile % 4 != 0 || (uintptr_t)lhs_scale % 16 != 0)
       return set_error(TKX_ERR_UNSUPPORTED,
                        "fp8 x fp8 with scale blocks along k needs lhs scales f32[blocks, m], m %% 4 == 0 and align_tile %% 4 == 0");

@@ -60,6 +60,8 @@ template <> struct Mma<kEBF16> { static constexpr int KA = 16; typedef i32x4 Fra
 template <> struct Mma<kEF16> { static constexpr int KA = 16; typedef i32x4 Frag; };
 template <> struct Mma<kEF32> { static constexpr int KA = 8; typedef i32x4 Frag; };
 template <> struct Mma<kEF8> { static constexpr int KA = 64; typedef i32x8 Frag; };
+// int8 x int8 -> int32: the accumulator registers hold int32 bits (kept in the f32x16 type the kernel uses).
+template <> struct Mma<kEI8> { static constexpr int KA = 32; typedef i32x4 Frag; };
 
 template <int EA>
 __device__ __forceinline__ f32x16 mma_atom(const typename Mma<EA>::Frag& first, const typename Mma<EA>::Frag& second,
@@ -70,6 +72,9 @@ __device__ __forceinline__ f32x16 mma_atom(const typename Mma<EA>::Frag& first, 
   } else if constexpr (EA == kEF16) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, first),
                                                   __builtin_bit_cast(f16x8, second), acc, 0, 0, 0);
+  } else if constexpr (EA == kEI8) {
+    typedef int i32x16_t __attribute__((ext_vector_type(16)));
+    return __builtin_bit_cast(f32x16, __builtin_amdgcn_mfma_i32_32x32x32_i8(first, second, __builtin_bit_cast(i32x16_t, acc), 0, 0, 0));
   } else if constexpr (EA == kEF32) {
     f32x4 a = __builtin_bit_cast(f32x4, first), b = __builtin_bit_cast(f32x4, second);
 #pragma unroll
@@ -194,8 +199,16 @@ __device__ __forceinline__ typename Mma<EC>::Frag load_frag(const unsigned char*
           f[2 * j + 1] = v[1];
         }
         return f;
+      } else if constexpr (EC == kEI8) {
+        // 16 contraction values per lane: k rows 16 (l / 32) .. + 15 of the atom.
+        const int krow = kb + 16 * (blk >> 1) + (s >> 1);
+        const i32x2 lo = lds_read_tr8(tile + mc_offset<ROW_BYTES, ES>(krow, col));
+        const i32x2 hi = lds_read_tr8(tile + mc_offset<ROW_BYTES, ES>(krow + 8, col));
+        Frag f;
+        f[0] = lo[0]; f[1] = lo[1]; f[2] = hi[0]; f[3] = hi[1];
+        return f;
       } else {
-        static_assert(EC == kEBF16 && ES == kEI8, "1-byte storage feeds fp8 or bf16(int8) MFMAs only");
+        static_assert(EC == kEBF16 && ES == kEI8, "1-byte storage feeds fp8, int8 or bf16(int8) MFMAs only");
         const int krow = kb + 8 * (blk >> 1) + (s >> 1);
         const i32x2 v = lds_read_tr8(tile + mc_offset<ROW_BYTES, ES>(krow, col));
         return i8x8_to_bf16x8(v);
@@ -466,9 +479,10 @@ struct GemmKernel {
   // fp8 x fp8 with scales per k-block on both sides (xs[row, k_sub] ws[g, k_sub, n],
   // pallas_mosaic_gpu_kernel_sm100_i8_quant.py:51-102): the MFMAs of a k-step (= one k-block or a part of one)
   // accumulate into partial accumulators, which are folded into the result with the block's scales.
-  static constexpr bool SUBP = SUBK && EA == kEF8;
-  static_assert(!SUBK || ((EB == kEI8 || EB == kEF8) && (EA == kEBF16 || (SUBP && EB == kEF8)) && BN == 256),
-                "per-k-block scales: bf16 lhs with int8 or fp8 weights, or fp8 x fp8; one 1 KB scale row per k-step");
+  // int8 x int8 runs the same way on the int8 MFMAs (int32 partial sums, exact), also with one block.
+  static constexpr bool SUBP = SUBK && (EA == kEF8 || EA == kEI8);
+  static_assert(!SUBK || ((EB == kEI8 || EB == kEF8) && (EA == kEBF16 || (SUBP && EB == EA)) && BN == 256),
+                "per-k-block scales: bf16 lhs with int8 or fp8 weights, fp8 x fp8 or int8 x int8; one 1 KB scale row per k-step");
   static constexpr int BNO = GLU ? BN / 2 : BN;  // output columns of a tile
   static constexpr int EC = EA;  // MFMA type follows A; B may be stored narrower (int8 weights)
   static constexpr int KA = Mma<EC>::KA;
@@ -788,8 +802,27 @@ struct GemmKernel {
           const unsigned char* nxt = smem + cur_stage * STAGE_BYTES;
           // (Pointers of the refill are computed here, far ahead of the MFMAs they are issued between.)
           const StepPtrs sp = decltype(refill_tag)::value ? step_ptrs(kt + NS, freed) : none;
-          static_assert(!SUBP || KSTEPS == 2, "the partial accumulators restart with the first of two atoms");
-          if constexpr (SUBP) {
+          static_assert(!(SUBP && EC == kEF8) || KSTEPS == 2, "the partial accumulators restart with the first of two atoms");
+          // int8: the int32 sums stay exact over a whole k-block, so they are folded in at the end of the block
+          // only (a fold costs as much vector work as three k-steps of int8 MFMAs); fp8: after every k-step.
+          [[maybe_unused]] bool block_end = true;
+          if constexpr (SUBP && EC == kEI8) {
+            const int mask = (1 << p.log2_block_rows) - 1;
+            const int k0 = kc_begin + kt * BK;
+            block_end = ((k0 + BK) & mask) == 0 || kt + 1 == nfull;
+            if ((k0 & mask) == 0) {
+#pragma unroll
+              for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                  for (int e = 0; e < 16; ++e) pacc[i][j][e] = 0.f;
+            }
+#pragma unroll
+            for (int kk = 0; kk + 1 < KSTEPS; ++kk)
+              atom(std::true_type{}, std::false_type{}, fa[kk & 1], fb[kk & 1], fa[(kk + 1) & 1], fb[(kk + 1) & 1], cur,
+                   kk + 1, none, std::false_type{});
+          } else if constexpr (SUBP) {
             atom(std::true_type{}, std::false_type{}, fa[0], fb[0], fa[1], fb[1], cur, 1, none, std::true_type{});
           } else {
 #pragma unroll
@@ -802,8 +835,8 @@ struct GemmKernel {
           // issue of the loads that refill `cur` with k-step kt + NS.
           step_barrier(decltype(refill_tag)::value || kt + NS - 1 < nfull);
           atom(more_tag, refill_tag, fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1], fa[0], fb[0], nxt, 0, sp, std::false_type{});
-          if constexpr (SUBP) {
-            // Fold the k-step's products into the result with the scales of its k-block: lane l holds row l % 32
+          if constexpr (SUBP) if (block_end) {
+            // Fold the products into the result with the scales of their k-block: lane l holds row l % 32
             // and, for t = 0..3, columns 8 t + 4 (l / 32) + {0..3} of every 32 x 32 block.
             const unsigned char* slot = smem + NS * STAGE_BYTES + (kt % (NS + 1)) * RING_SLOT;
             float xs[TM];
@@ -819,7 +852,11 @@ struct GemmKernel {
                 for (int i = 0; i < TM; ++i)
                   if (F || ((rmask >> i) & 1u)) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[i][j][4 * t + e] += pacc[i][j][4 * t + e] * (xs[i] * wsc[e]);
+                    for (int e = 0; e < 4; ++e) {
+                      float part = pacc[i][j][4 * t + e];
+                      if constexpr (EC == kEI8) part = (float)__builtin_bit_cast(int, part);  // int32 partial sums
+                      acc[i][j][4 * t + e] += part * (xs[i] * wsc[e]);
+                    }
                   }
               }
           }

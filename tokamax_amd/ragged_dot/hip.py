@@ -143,11 +143,12 @@ def _widening_plan(lhs, rhs, allow_native: bool = True) -> tuple[bool, bool, boo
   widening pass instead; an fp8 operand whose partner was widened is widened too (there is no bf16 x fp8 kernel)."""
   lhs_q, rhs_q = isinstance(lhs, QArray), isinstance(rhs, QArray)
   widen_lhs = widen_rhs = False
+  blocks = None  # (scale blocks along k of a quantised rhs)
   if lhs_q:
-    blocks = _lhs_scale_blocks(lhs)
-    if blocks is None:
+    lhs_blocks = _lhs_scale_blocks(lhs)
+    if lhs_blocks is None:
       raise NotImplementedError(f"lhs scale must have shape [m,1] or [m, k/t] with 16 | t, got {tuple(lhs.scale.shape)}")
-    widen_lhs = blocks > 1 or _dtype_of(lhs) == torch.int8  # (no kernel contracts int8 activations directly)
+    widen_lhs = lhs_blocks > 1 or _dtype_of(lhs) == torch.int8  # (unless int8 meets int8 below)
   if rhs_q:
     blocks = _scale_blocks_along_k(rhs)
     if blocks is None and not _rhs_scale_tiles(rhs):
@@ -155,14 +156,19 @@ def _widening_plan(lhs, rhs, allow_native: bool = True) -> tuple[bool, bool, boo
                                 f" {tuple(rhs.scale.shape)}")
     widen_rhs = blocks is None or blocks > 1
   eight_bit_float = lambda x: _dtype_of(x) == torch.float8_e4m3fn
-  if (lhs_q and rhs_q and allow_native and eight_bit_float(lhs) and eight_bit_float(rhs) and blocks is not None
-      and blocks > 1 and _lhs_scale_blocks(lhs) == blocks):
-    # fp8 x fp8 with the same k-blocks on both sides: the fp8 MFMA kernel that folds the scales in per k-block.
+  both_int8 = (lhs_q and rhs_q and _dtype_of(lhs) == torch.int8 and _dtype_of(rhs) == torch.int8
+               and lhs.qvalue.dtype == torch.int8 and rhs.qvalue.dtype == torch.int8)
+  both_fp8 = lhs_q and rhs_q and eight_bit_float(lhs) and eight_bit_float(rhs)
+  if (allow_native and (both_fp8 or both_int8) and blocks is not None and (blocks > 1 or both_int8)
+      and _lhs_scale_blocks(lhs) == blocks):
+    # The same k-blocks on both sides: the fp8 (int8) MFMA kernels that fold the scales in per k-block; int8 x int8
+    # also with a single block (there is no other kernel that contracts int8 activations).
     m, k = lhs.qvalue.shape
     rows = k // blocks
+    step = 128 if both_fp8 else 64
+    shape_ok = k % step == 0 and (blocks == 1 or (rows % step == 0 and rows & (rows - 1) == 0))
     # (Groups of a few rows are better off with a widened lhs and the streaming small-m kernel, below.)
-    if (rows % 128 == 0 and rows & (rows - 1) == 0 and m % 4 == 0 and rhs.qvalue.shape[2] % 16 == 0
-        and m > 8 * rhs.qvalue.shape[0]):
+    if shape_ok and m % 4 == 0 and rhs.qvalue.shape[2] % 16 == 0 and m > 8 * rhs.qvalue.shape[0]:
       return False, False, True
   if rhs_q and allow_native and blocks is not None and rhs.qvalue.dtype in (torch.int8, torch.float8_e4m3fn):
     # Kernels of their own (bf16 lhs; 256-column tiles) for int8 weights with several scale blocks along k and
@@ -454,6 +460,15 @@ class HipRaggedDot(base.RaggedDot):
     streaming_ok = (mode in (0, 4) and ba.kwargs.get("rhs_bias") is None and contraction % 1024 == 0 and cols % 8 == 0
                     and (contraction // 4) * cols * wbytes < 2**31)
     usable = [v for v in variants if v[0] != 16 or streaming_ok]
+    if mode == 4:
+      # The k-step of a tiled variant has to divide the rows of a scale block (and the contraction).
+      rhs_ = _per_column_rhs_scale(ba.args[1])
+      raw_scale = ba.kwargs.get("rhs_scale")
+      blocks = raw_scale.shape[1] if raw_scale is not None else rhs_.scale.shape[1]
+      step = contraction // blocks if blocks > 1 else contraction
+      usable = [v for v in usable if v[0] == 16 or step % v[2] == 0]
+      if not usable:
+        raise NotImplementedError(f"No hip kernel variant whose k-step divides {step} rows.")
     # Rows per group decide the m-tile: a tile much taller than a group wastes MFMA work on rows
     # that are masked out at the store; a short tile re-reads the weights more often.
     rows_per_group = rows / max(num_groups, 1) if mode != 2 else rows
@@ -484,7 +499,9 @@ class HipRaggedDot(base.RaggedDot):
       # 1.5% slower), and at equal depth the longer k-step has fewer barriers per flop.
       in_flight = min((ns - 1) * bk, 96) if wm * wn == 8 else 0
       # (With per-k-block scales the shorter k-step measured 3 % faster at equal depth: 991 against 961 TFLOP/s.)
-      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -in_flight, bk if mode == 4 else -bk, ns)
+      # Integer or fp8 MFMAs on both sides: the longer k-step again.
+      short_k = mode == 4 and key[1] == _lib.TKX_BF16
+      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -in_flight, bk if short_k else -bk, ns)
 
     bm, bn, bk, wm, wn, ns = min(usable, key=score)
     # grid_tile_width m-tasks of one group run side by side on an n-panel of its weights (a span never
