@@ -371,7 +371,7 @@ def test_every_kernel_variant_through_c_abi(v, device):
   if v["mode"] == 4 and lt == torch.int8:  # int8 x int8 on the int8 MFMAs, scales per block of 64 k rows on both sides
     lhs = torch.tensor(rng.integers(-127, 128, (m, k)).astype(np.int8), device=device)
     rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
-    for blocks in (k // v["block_k"], 1):  # scale blocks of one k-step (128 or 64 rows), and one block
+    for blocks in (k // v["block_k"],):  # scale blocks of one k-step (128 or 64 rows); one block runs the mode-0 variants
       xs, ws_ = mk((m, blocks), 0.01).abs() + 0.005, mk((G, blocks, n), 0.01).abs() + 0.005
       bias = mk((G, 1, n), 0.5)
       out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs, rhs_scale=ws_, rhs_bias=bias)
@@ -403,7 +403,14 @@ def test_every_kernel_variant_through_c_abi(v, device):
     _check(out, _ref(lhs, dout, gs, O.RAGGED_CONTRACTING), TOL[lt])
     return
   lhs_scale = rhs_scale = None
-  if rt == torch.int8:
+  if rt == torch.int8 and lt == torch.int8:  # int8 x int8, one scale per row and per (group, column)
+    lhs = torch.tensor(rng.integers(-127, 128, (m, k)).astype(np.int8), device=device)
+    rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+    lhs_scale, rhs_scale = mk((m, 1), 0.01).abs() + 0.005, mk((G, 1, n), 0.01).abs() + 0.005
+    lhs_f = O.dequantize(lhs.cpu().numpy().astype(np.float64), _np(lhs_scale))
+    rhs_f = O.dequantize(rhs.cpu().numpy().astype(np.float64), _np(rhs_scale))
+    tol = 1e-5  # the int32 sums are exact
+  elif rt == torch.int8:
     rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
     rhs_scale = mk((G, 1, n), 0.01).abs() + 1e-3
     rhs_f = O.dequantize(rhs.cpu().numpy(), _np(rhs_scale))

@@ -178,7 +178,7 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
   const bool a8w8 = lhs_dtype == TKX_I8 && rhs_dtype == TKX_I8;
   if (a8w8 && (rhs_scale == nullptr || lhs_scale == nullptr || dlhs))
     return set_error(TKX_ERR_UNSUPPORTED, "int8 x int8: default mode with lhs and rhs scales only");
-  const bool subk = rhs_scale != nullptr && (rhs_scale_blocks != 1 || a16w8f || a8w8) && !dlhs && c.block_m != kDecodeBlockM;
+  const bool subk = rhs_scale != nullptr && (rhs_scale_blocks != 1 || a16w8f) && !dlhs && c.block_m != kDecodeBlockM;
   int32_t log2_block_rows = 0;
   if (subk && rhs_scale_blocks == 1) {
     log2_block_rows = 30;  // every k-step falls into block 0

@@ -896,6 +896,18 @@ struct GemmKernel {
     {
       unsigned char* Cg = reinterpret_cast<unsigned char*>(p.C);
       if constexpr (MODE == kDrhs) Cg += (int64_t)group * p.c_group_stride * (p.out_dtype == TKX_F32 ? 4 : 2);
+      if constexpr (EC == kEI8 && !SUBP) {
+        // int8 x int8 with one scale per row and per column: the accumulators hold the exact int32 sums.
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+              const float bits = acc[i][j][e];  // (a scalar copy first: a bit cast straight from a vector element misreads)
+              acc[i][j][e] = (float)__builtin_bit_cast(int, bits);
+            }
+      }
       const bool inside = col0 + BNO <= p.n_ext;
       // Column of B (of its scales and bias) behind accumulator block j, element group t of this lane.
       auto b_col = [&](int j, int t) {

@@ -32,6 +32,11 @@ static const Variant kVariants[] = {
     SUBK(32, 256, 64, 1, 4, 4),
     // int8 activations x int8 weights on the int8 MFMAs: int32 sums of a k-step, folded into the f32 result with
     // the scales of its k-block (one block = one scale per row and per (group, column)).
+    // (one scale per row and per (group, column): plain forward variants, the scales in the epilogue)
+    TKX_VARIANT(kFwd, kEI8, kEI8, 256, 256, 128, 2, 4, 2),
+    TKX_VARIANT(kFwd, kEI8, kEI8, 128, 256, 128, 2, 4, 3),
+    TKX_VARIANT(kFwd, kEI8, kEI8, 64, 128, 128, 2, 2, 4),
+    TKX_VARIANT(kFwd, kEI8, kEI8, 32, 128, 128, 1, 4, 4),
     TKX_VARIANT(kFwdSubK, kEI8, kEI8, 128, 256, 128, 2, 4, 3),
     TKX_VARIANT(kFwdSubK, kEI8, kEI8, 128, 256, 64, 2, 4, 3),
     TKX_VARIANT(kFwdSubK, kEI8, kEI8, 64, 256, 64, 2, 2, 4),

@@ -168,6 +168,8 @@ def _widening_plan(lhs, rhs, allow_native: bool = True) -> tuple[bool, bool, boo
     step = 128 if both_fp8 else 64
     shape_ok = k % step == 0 and (blocks == 1 or (rows % step == 0 and rows & (rows - 1) == 0))
     # (Groups of a few rows are better off with a widened lhs and the streaming small-m kernel, below.)
+    if both_int8 and blocks == 1 and k % 16 == 0:
+      return False, False, False  # one scale per row and per column: the plain int8 MFMA variants, scales in the epilogue
     if shape_ok and m % 4 == 0 and rhs.qvalue.shape[2] % 16 == 0 and m > 8 * rhs.qvalue.shape[0]:
       return False, False, True
   if rhs_q and allow_native and blocks is not None and rhs.qvalue.dtype in (torch.int8, torch.float8_e4m3fn):
