@@ -35,7 +35,7 @@ if ROOT not in sys.path:
   sys.path.insert(0, ROOT)
 
 # MI355X published peaks (dense).
-PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "f32": 157.3}
+PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "f32": 157.3}  # (int8: TOP/s)
 PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
@@ -311,7 +311,13 @@ def main():
     cfg = op.bind(w.lhs, q8k, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
     measure("mixtral_prefill_int8_weights_k_block_scales", lambda: op(w.lhs, q8k, group_sizes=gs, preferred_element_type=torch.bfloat16),
             w.flops, nb + w.nonempty_groups * (w.k // 128) * w.n * 4, "mfma", "bf16", cfg)
-    del w, q8, q8k
+    # int8 activations x the same int8 weights, one scale per row and per (group, column): the int8 MFMAs
+    a8 = tokamax_amd.QArray(torch.randint(-127, 128, (w.m, w.k), device=device, dtype=torch.int8, generator=gen8),
+                            (torch.rand(w.m, 1, device=device, generator=gen8) + 0.5) / 127)
+    cfg = op.bind(a8, q8, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_prefill_int8_int8", lambda: op(a8, q8, group_sizes=gs, preferred_element_type=torch.bfloat16),
+            w.flops, w.m * w.k + w.nonempty_groups * w.k * w.n + w.m * w.n * 2, "mfma", "int8", cfg)
+    del w, q8, q8k, a8
 
     w = workloads.make("vjp", device, seed=0)
     gs = torch.tensor(w.group_sizes, device=device)
