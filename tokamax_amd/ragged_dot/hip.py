@@ -132,15 +132,19 @@ def _lhs_scale_blocks(q: QArray) -> int | None:
 
 
 def _widening_plan(lhs, rhs, allow_native: bool = True) -> tuple[bool, bool, bool]:
-  """(widen lhs, widen rhs, native k-blocks): which quantised operands are dequantised to bf16 before the
-  kernels, and whether int8 weights with scales [g, k/t_k, n] keep them (t_k a power of two that 64 divides,
-  bf16 on the other side, `allow_native`: no gate-up fusion): kernels of their own multiply each k-block's
-  scales in while they widen the weights.
+  """(widen lhs, widen rhs, native k-blocks): how a pair of (possibly quantised) operands reaches the kernels.
 
-  The kernels apply one scale per lhs row and one per (group, column) in their epilogue. Scales that change
-  along the contraction (the k-subchannel scales of pallas_mosaic_gpu_kernel_sm100_i8_quant.py:51-102, the scale
-  tile (1, t_k, 1) of pallas_mosaic_gpu_kernel_sm90_quant.py:91-97) or along n in blocks are multiplied in by a
-  widening pass instead; an fp8 operand whose partner was widened is widened too (there is no bf16 x fp8 kernel)."""
+  * One scale per lhs row and one per (group, column): applied in the kernels' epilogue (bf16 x int8, fp8 x fp8,
+    int8 x int8), nothing is widened.
+  * "native k-blocks" (`allow_native`: no gate-up fusion): scales [g, k/t_k, n] go to the kernels as they are, to
+    - fp8 x fp8 and int8 x int8 with the same k-blocks on both sides (xs[row, k_sub] ws[g, k_sub, n],
+      pallas_mosaic_gpu_kernel_sm100_i8_quant.py:51-102): MFMA kernels that fold the scales in per k-block;
+    - int8 or fp8 weights under a bf16 lhs (the scale tile (1, t_k, 1) of pallas_mosaic_gpu_kernel_sm90_quant.py:91-97;
+      fp8 weights also with a single block): kernels that scale the weights while they widen them; a quantised lhs
+      is widened to bf16 for them.
+    t_k is a power of two that the kernels' k-step divides.
+  * Everything else that is quantised is dequantised to bf16 by a widening pass first; an fp8 operand whose partner
+    was widened is widened too (there is no bf16 x fp8 kernel outside the native ones)."""
   lhs_q, rhs_q = isinstance(lhs, QArray), isinstance(rhs, QArray)
   widen_lhs = widen_rhs = False
   blocks = None  # (scale blocks along k of a quantised rhs)
