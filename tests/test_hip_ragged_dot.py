@@ -877,6 +877,33 @@ def test_bf16_activations_fp8_weights(device):
   _check(out, O.ragged_dot(lhs_f, O.dequantize(qf, _np(scale)), gs, acc_dtype=np.float64, out_dtype="f64"), 6e-3, rows=count)
 
 
+@pytest.mark.parametrize("qdtype", [torch.float8_e4m3fn, torch.int8])
+def test_per_tensor_scales(qdtype, device):
+  """One scale per tensor on both operands (scale shapes [1,1] and [1,1,1]), the plainest fp8 / int8 recipe: the
+  scales are repeated per row and per (group, column) and the pair runs on the fp8 / int8 MFMA kernels."""
+  rng = np.random.default_rng(31)
+  G, m, k, n = 4, 300, 512, 256
+  gs = np.array([100, 0, 80, 110], np.int32)
+  gst = torch.tensor(gs, device=device)
+  if qdtype == torch.int8:
+    a = torch.tensor(rng.integers(-127, 128, (m, k)).astype(np.int8), device=device)
+    b = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+    af, bf = a.cpu().numpy().astype(np.float64), b.cpu().numpy().astype(np.float64)
+  else:
+    a = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(qdtype)
+    b = torch.tensor(rng.normal(0, 1, (G, k, n)).astype(np.float32), device=device).to(qdtype)
+    af = O.e4m3fn_decode(a.view(torch.uint8).cpu().numpy()).astype(np.float64)
+    bf = O.e4m3fn_decode(b.view(torch.uint8).cpu().numpy()).astype(np.float64)
+  sa, sb = torch.full((1, 1), 0.037, device=device), torch.full((1, 1, 1), 0.0021, device=device)
+  op = tokamax_amd.HipRaggedDot()
+  lhs, rhs = tokamax_amd.QArray(a, sa), tokamax_amd.QArray(b, sb)
+  key = op._problem(op.bind(lhs, rhs, group_sizes=gst))[1]
+  assert key[1] == key[2] == hip_ops.dtype_code(qdtype)  # nothing is widened
+  out = op(lhs, rhs, group_sizes=gst, preferred_element_type=torch.float32)
+  want = O.ragged_dot(af * 0.037, bf * 0.0021, gs, acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, 1e-4, rows=int(gs.sum()))
+
+
 def test_int4_values_in_int8_storage(device):
   """fp8 x int4 with scale tile (1, 128, 1) (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:266-350) and bf16 x int4:
   torch holds int4 values in int8 storage (qtype says int4); they run as int8."""

@@ -109,14 +109,31 @@ def _per_column_rhs_scale(rhs):
   repeated over its t_n columns ([g, k/t_k, n]): the form the kernels take. Works on tensors and on shapes."""
   if not isinstance(rhs, QArray) or len(rhs.scale.shape) != 3 or len(rhs.qvalue.shape) != 3:
     return rhs
-  n, nt = rhs.qvalue.shape[2], rhs.scale.shape[2]
-  if nt == n or nt < 1 or n % nt != 0 or rhs.scale.shape[0] != rhs.qvalue.shape[0]:
+  g, n = rhs.qvalue.shape[0], rhs.qvalue.shape[2]
+  gs, nt = rhs.scale.shape[0], rhs.scale.shape[2]
+  if (nt == n and gs == g) or nt < 1 or n % nt != 0 or gs not in (1, g):
     return rhs
   if isinstance(rhs.scale, torch.Tensor):
-    scale = rhs.scale.repeat_interleave(n // nt, dim=2)
+    scale = rhs.scale.expand(g, -1, -1) if gs != g else rhs.scale  # (one scale set shared by all groups)
+    scale = scale.repeat_interleave(n // nt, dim=2) if nt != n else scale.contiguous()
   else:
-    scale = ShapeDtype((rhs.scale.shape[0], rhs.scale.shape[1], n), rhs.scale.dtype)
+    scale = ShapeDtype((g, rhs.scale.shape[1], n), rhs.scale.dtype)
   return QArray(rhs.qvalue, scale, rhs.zero_point, rhs.qtype)
+
+
+def _per_row_lhs_scale(lhs):
+  """A quantised lhs [m, k] whose scale has one row ([1, blocks]: shared by all rows, e.g. one scale per tensor)
+  with that row repeated for every lhs row. Works on tensors and on shapes."""
+  if not isinstance(lhs, QArray) or len(lhs.scale.shape) != 2 or len(lhs.qvalue.shape) != 2:
+    return lhs
+  m = lhs.qvalue.shape[0]
+  if lhs.scale.shape[0] != 1 or m == 1:
+    return lhs
+  if isinstance(lhs.scale, torch.Tensor):
+    scale = lhs.scale.expand(m, -1)
+  else:
+    scale = ShapeDtype((m, lhs.scale.shape[1]), lhs.scale.dtype)
+  return QArray(lhs.qvalue, scale, lhs.zero_point, lhs.qtype)
 
 
 def _lhs_scale_blocks(q: QArray) -> int | None:
@@ -288,7 +305,7 @@ class HipRaggedDot(base.RaggedDot):
       rhs = QArray(rhs, rhs_scale.reshape(g, rhs_scale.shape[1], n))
       if preferred_element_type is None:
         preferred_element_type = lhs.dtype
-    rhs = _per_column_rhs_scale(rhs)
+    lhs, rhs = _per_row_lhs_scale(lhs), _per_column_rhs_scale(rhs)
     if group_offset is not None and ragged_dot_dimension_numbers != base.DEFAULT_RAGGED_DOT_DIM_NUMS:
       raise NotImplementedError("group_offset needs the default dimension numbers.")
     # rhs_bias and fuse_gateup_activation (base.py:205-217) are fused into the forward kernel's epilogue.
@@ -439,7 +456,7 @@ class HipRaggedDot(base.RaggedDot):
       g_, blocks_, _, n_ = raw_scale.shape
       rhs = QArray(rhs, ShapeDtype((g_, blocks_, n_), raw_scale.dtype))
     if mode in (0, 3):
-      rhs = _per_column_rhs_scale(rhs)
+      lhs, rhs = _per_row_lhs_scale(lhs), _per_column_rhs_scale(rhs)
       widen_lhs, widen_rhs, native_k_blocks = _widening_plan(lhs, rhs, allow_native=mode == 0)
       lhs_dt = torch.bfloat16 if widen_lhs else lhs_dt
       rhs_dt = torch.bfloat16 if widen_rhs else rhs_dt
