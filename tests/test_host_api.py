@@ -440,6 +440,37 @@ def test_hip_config_validation_and_heuristics():
                 group_sizes=base.GroupSizes(ShapeDtype((8,), torch.int32), 256)).heuristics_config
 
 
+def test_quantised_operand_routes():
+  """Which kernels a pair of quantised operands takes (mode, lhs kind, rhs kind of the variant key), decided on
+  shapes alone: epilogue scales, scales folded in per k-block, weights scaled while widened, or the widening pass."""
+  op = hip.HipRaggedDot()
+  f8, i8, bf, f32 = torch.float8_e4m3fn, torch.int8, torch.bfloat16, torch.float32
+  F8, I8, BF = _lib.TKX_F8E4M3FN, _lib.TKX_I8, _lib.TKX_BF16
+  m, k, n, G = 4096, 1024, 512, 8
+  q = lambda shape, dt, sshape: tokamax_amd.QArray(ShapeDtype(shape, dt), ShapeDtype(sshape, f32))
+  gsz = base.GroupSizes(ShapeDtype((G,), torch.int32), m)
+  def key(lhs, rhs):
+    return op._problem(op.bind(lhs, rhs, group_sizes=gsz))[1]
+  lhs16 = ShapeDtype((m, k), bf)
+  assert key(q((m, k), f8, (m, 1)), q((G, k, n), f8, (G, 1, n))) == (0, F8, F8)              # epilogue scales
+  assert key(q((m, k), f8, (1, 1)), q((G, k, n), f8, (1, 1, 1))) == (0, F8, F8)              # one scale per tensor
+  assert key(q((m, k), f8, (m, k // 128)), q((G, k, n), f8, (G, k // 128, n))) == (4, F8, F8)        # folded per k-block
+  assert key(q((m, k), f8, (m, k // 128)), q((G, k, n), f8, (G, k // 128, n // 128))) == (4, F8, F8)  # 128 x 128 blocks
+  assert key(q((m, k), i8, (m, 1)), q((G, k, n), i8, (G, 1, n))) == (0, I8, I8)              # int8 MFMAs, epilogue scales
+  assert key(q((m, k), i8, (m, k // 64)), q((G, k, n), i8, (G, k // 64, n))) == (4, I8, I8)
+  assert key(lhs16, q((G, k, n), i8, (G, 1, n))) == (0, BF, I8)
+  assert key(lhs16, q((G, k, n), i8, (G, k // 128, n))) == (4, BF, I8)                       # scaled while widened
+  assert key(lhs16, q((G, k, n), f8, (G, 1, n))) == (4, BF, F8)
+  assert key(q((m, k), f8, (m, 1)), q((G, k, n), f8, (G, k // 128, n))) == (4, BF, F8)       # lhs widened for it
+  assert key(lhs16, q((G, k, n), i8, (G, k // 32, n))) == (0, BF, BF)                        # t_k = 32: the widening pass
+  assert key(q((m, k), f8, (m, k // 32)), q((G, k, n), f8, (G, k // 32, n))) == (0, BF, BF)
+  with pytest.raises(NotImplementedError):
+    key(lhs16, q((G, k, n), i8, (G // 2, 1, n)))                                              # scales shared by pairs of groups
+  # the k-step of the chosen variant divides the rows of a scale block
+  ba = op.bind(q((m, k), i8, (m, k // 64)), q((G, k, n), i8, (G, k // 64, n)), group_sizes=gsz)
+  assert 64 % ba.heuristics_config.block_k == 0
+
+
 def test_arg_specs_and_flops():
   names = {s.full_name for s in arg_specs.ARG_SPECS}
   assert {"compute_bound", "memory_bound", "mixtral_8x7b"} <= names
