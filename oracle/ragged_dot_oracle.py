@@ -26,8 +26,13 @@ below therefore cites the reference call site it follows, and says what pins it:
                                ..._sm100_fp8_quant_test.py:229-232                q.astype(f32)*repeat(scale, tile)
   round_to_bf16 / e4m3fn       base.py:342-354 (.astype(out_dtype))               torch's bf16 / float8_e4m3fn casts
                                                                                   (library routine), exhaustive for fp8
-  generate_group_sizes         base.py:171-196                                    invariants of base_test.py:45-51
-                                                                                  (len == G, sum == m) + literal restatement
+  generate_group_sizes         base.py:171-196                                    what the definition fixes: the three
+                                                                                  cases of base_test.py:45-51 (incl.
+                                                                                  G > m), a one-hot p, counts within 4
+                                                                                  sigma of p*m at m = 1e6, m = 1 / G = 1,
+                                                                                  seed selects the draw; the exact values
+                                                                                  per seed are NumPy's (no stored vector
+                                                                                  in the reference to compare with)
 
   ragged_dot_fused / gateup    base.py:205-217 (docstring of `rhs_bias` and       composition of `ragged_dot` with the
                                `fuse_gateup_activation`); the gate-up forms of    formulas of that docstring; the gate-up

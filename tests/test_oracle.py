@@ -71,10 +71,62 @@ def test_scheduler_invariants_and_c_agrees(seed):
   assert np.all(a["actual_size"][nt:] == 0)
 
 
-def test_generate_group_sizes():
-  gs = O.generate_group_sizes(m=1024, num_groups=8)
-  assert len(gs) == 8 and sum(gs) == 1024  # base_test.py:45-51
-  assert gs == tuple(np.bincount(np.random.default_rng(0).choice(8, (1024,)), minlength=8))
+# What the mathematics fixes of `generate_group_sizes` (base.py:171-196: `m` draws with replacement over the
+# groups with probabilities `p`, counted per group). The reference stores no sizes for any seed, so the exact
+# values are compared between the oracle and the product twin only; each property below fails for a plausible
+# mistake (ignoring `p`, dropping `minlength`, a fixed generator, counting something other than the draws).
+@pytest.mark.parametrize("m,num_groups,p", [(256, 4, None), (16, 64, None), (256, 4, (0.1, 0.2, 0.3, 0.4))])
+def test_generate_group_sizes_reference_cases(m, num_groups, p):
+  # The three parametrisations of base_test.py:45-51; (16, 64) has more groups than rows, so the trailing
+  # groups nobody drew must still be listed (with 16 draws over 64 groups some always are empty).
+  gs = O.generate_group_sizes(m=m, num_groups=num_groups, p=p)
+  assert isinstance(gs, tuple) and all(isinstance(v, int) for v in gs)
+  assert len(gs) == num_groups and sum(gs) == m and min(gs) >= 0
+  from tokamax_amd.ragged_dot import base
+  assert base.generate_group_sizes(m=m, num_groups=num_groups, p=p) == gs
+
+
+def test_generate_group_sizes_one_hot_p_puts_every_row_in_that_group():
+  for hot in (0, 2, 4):
+    p = [0.0] * 5
+    p[hot] = 1.0
+    want = [0] * 5
+    want[hot] = 1000
+    assert O.generate_group_sizes(m=1000, num_groups=5, p=p) == tuple(want)
+
+
+def test_generate_group_sizes_frequencies_follow_p():
+  from tokamax_amd.ragged_dot import base
+  m = 10 ** 6
+  p = np.array((0.1, 0.2, 0.3, 0.4))
+  for seed in (0, 7):
+    gs = np.array(O.generate_group_sizes(m=m, num_groups=4, p=tuple(p), seed=seed))
+    sigma = np.sqrt(m * p * (1 - p))  # each count is binomial(m, p_i)
+    assert np.all(np.abs(gs - m * p) <= 4 * sigma), (gs, m * p, sigma)
+    assert base.generate_group_sizes(m=m, num_groups=4, p=tuple(p), seed=seed) == tuple(gs)
+  # p=None is the uniform distribution: the same test with p_i = 1/G, and no group anywhere near p's pattern.
+  gs = np.array(O.generate_group_sizes(m=m, num_groups=8))
+  assert np.all(np.abs(gs - m / 8) <= 4 * np.sqrt(m * (1 / 8) * (7 / 8)))
+
+
+def test_generate_group_sizes_seed_selects_the_draw():
+  from tokamax_amd.ragged_dot import base
+  a = O.generate_group_sizes(m=4096, num_groups=16, seed=3)
+  assert a == O.generate_group_sizes(m=4096, num_groups=16, seed=3)   # a function of its arguments only
+  assert a != O.generate_group_sizes(m=4096, num_groups=16, seed=4)   # and the seed is used
+  assert a != O.generate_group_sizes(m=4096, num_groups=16)           # default seed is 0, not 3
+  assert O.generate_group_sizes(m=4096, num_groups=16) == O.generate_group_sizes(m=4096, num_groups=16, seed=0)
+  for seed in (0, 3, 4):
+    assert base.generate_group_sizes(m=4096, num_groups=16, seed=seed) == O.generate_group_sizes(m=4096, num_groups=16, seed=seed)
+
+
+def test_generate_group_sizes_counts_the_draws():
+  # With m = 1 exactly one group holds the row; with G = 1 every row lands in it.
+  for seed in range(5):
+    gs = O.generate_group_sizes(m=1, num_groups=7, seed=seed)
+    assert sorted(gs) == [0] * 6 + [1]
+  assert O.generate_group_sizes(m=123, num_groups=1) == (123,)
+  assert O.generate_group_sizes(m=0, num_groups=3) == (0, 0, 0)
 
 
 @pytest.mark.parametrize("mode", [O.DEFAULT, O.TRANS_RHS, O.RAGGED_CONTRACTING])
