@@ -1,7 +1,6 @@
 """Benchmark of the hip ragged dot on one MI355X.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--calibration-copy]
-                  [--decode-group-sweep]
 
 Prints ONE JSON line. A step is one pass of the hot path (scheduler kernel + grouped-GEMM kernel)
 over one seeded synthetic batch that is already resident in HBM. The headline workload is the
@@ -140,8 +139,6 @@ def main():
   ap.add_argument("--warmup", type=int, default=5)
   ap.add_argument("--no-extras", action="store_true", help="headline workload only")
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-  ap.add_argument("--decode-group-sweep", action="store_true",
-                  help="also time the decode launch with other sets of non-empty groups (extras.decode_int8_group_sweep)")
   ap.add_argument("--calibration-copy", action="store_true",
                   help="also run one elementwise copy of 1 GiB (reads 1 GiB, writes 1 GiB), the known-size kernel "
                        "that hardware byte counters are scaled by")
@@ -259,24 +256,6 @@ def main():
     extras["decode_int8_cold"]["eager_wall_ms_per_call"] = round(wall / steps, 5)  # host dispatch included
     extras["decode_int8_cold"]["algorithmic_bytes"] = int(w.algorithmic_bytes())
     extras["decode_int8_cold"]["touched_experts"] = w.nonempty_groups
-    if args.decode_group_sweep:
-      # The same launch with other sets of non-empty groups: time follows the workgroups a CU holds, not the bytes.
-      import numpy as np
-      G_ = w.num_groups
-      sweep = {"all_groups_2_rows": np.full(G_, 2, np.int32)}
-      for name, idx in (("first_110_groups_2_rows", slice(0, 110)), ("every_second_group_4_rows", slice(0, G_, 2)),
-                        ("first_64_groups_4_rows", slice(0, 64))):
-        sizes = np.zeros(G_, np.int32)
-        sizes[idx] = 4 if "4_rows" in name else 2
-        sweep[name] = sizes
-      rows = {}
-      for name, sizes in sweep.items():
-        gs_ = torch.tensor(sizes, device=device)
-        m_ = _time_graph([(lambda q=q: op(w.lhs, q, group_sizes=gs_, preferred_element_type=torch.bfloat16)) for q in copies], 24)
-        nb = int((sizes > 0).sum()) * (w.k * w.n + w.n * 4) + w.m * w.k * 2 + w.m * w.n * 2
-        rows[name] = dict(non_empty_groups=int((sizes > 0).sum()), us_per_launch=round(m_ * 1e3, 2), gbs=round(nb / m_ / 1e6, 1),
-                          frac_of_hbm_peak=round(nb / m_ / 1e6 / (PEAK_HBM_GBS), 4))
-      extras["decode_int8_group_sweep"] = rows
     del w, copies
 
     w = workloads.make("fp8", device, seed=0)

@@ -186,7 +186,7 @@ int32_t tkx_dequantize(const void* qvalue, const float* scale, void* out, int64_
  *   ragged_gather_reduce  (ragged_gather_reduce/base.py:26-40): weights f32[out_rows * reduce], valid bytes, reduce = R;
  *                         products and sums in f32, one rounding to `dtype`
  * x [in_rows, hidden], out [out_rows, hidden] of `dtype` (f32/bf16/f16), rows a multiple of 16 bytes;
- * indices int32[out_rows * reduce_group_size] (clamped into [0, in_rows)). */
+ * indices int32[out_rows * reduce_group_size] (negative ones count from the end; what is then still outside [0, in_rows) is clamped). */
 int32_t tkx_ragged_gather_rows(const void* x, const int32_t* indices, const float* weights, const uint8_t* valid,
                                const int32_t* start, const int32_t* end, void* out, int64_t in_rows, int64_t out_rows,
                                int64_t hidden, int64_t reduce_group_size, int32_t dtype, tkx_stream_t stream);

@@ -338,22 +338,32 @@ def gated_linear_unit(x, weights, activation=None):
   return (gate if activation is None else activation(gate)) * up
 
 
+def _jax_take_rows(x, indices):
+  """Row lookup `x[indices]` with JAX's indexing rules, which differ from NumPy's for indices outside the array:
+  a negative index counts from the end (i -> i + len(x)), and what is then still outside [0, len(x)) is clamped
+  to the nearest row instead of raising (JAX documents gathers through indexing as clamped)."""
+  x = np.asarray(x)
+  idx = np.asarray(indices).astype(np.int64)
+  idx = np.where(idx < 0, idx + len(x), idx)
+  return x[np.clip(idx, 0, len(x) - 1)]
+
+
 def ragged_gather(x, indices):
   """`x[indices]` (ragged_gather/base.py:25-32)."""
-  return np.asarray(x)[np.asarray(indices)]
+  return _jax_take_rows(x, indices)
 
 
 def ragged_scatter(x, indices, start: int, end: int):
   """`where(start <= indices < end, x[indices], 0)` (ragged_scatter/base.py:26-38)."""
   idx = np.asarray(indices)
-  out = np.asarray(x)[np.clip(idx, 0, len(x) - 1)]
+  out = _jax_take_rows(x, idx)
   return np.where(((idx >= start) & (idx < end))[:, None], out, 0).astype(out.dtype)
 
 
 def ragged_gather_reduce(x, indices, topk_weights, valid_rows_mask, reduce_group_size: int):
   """f32 `sum over groups of R rows of valid * weight * x[index]` (ragged_gather_reduce/base.py:26-40),
   returned as float32 (the caller rounds to the input type)."""
-  out = np.asarray(x, np.float32)[np.asarray(indices)] * np.asarray(topk_weights, np.float32)[:, None]
+  out = _jax_take_rows(np.asarray(x, np.float32), indices) * np.asarray(topk_weights, np.float32)[:, None]
   out = np.where(np.asarray(valid_rows_mask, bool)[:, None], out, np.float32(0))
   return out.reshape(-1, reduce_group_size, out.shape[-1]).sum(axis=1, dtype=np.float32)
 

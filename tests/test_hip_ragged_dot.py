@@ -1047,6 +1047,61 @@ def test_row_movement_ops(dtype, device):
   _check(combined, want, 6e-3)
 
 
+def test_row_lookup_outside_the_array(device):
+  """Indices outside [0, rows): negative ones count from the end, the rest is clamped (the reference's `x[indices]`)."""
+  rows, hidden = 37, 64
+  rng = np.random.default_rng(5)
+  x = torch.tensor(rng.normal(0, 1, (rows, hidden)).astype(np.float32), device=device).to(torch.bfloat16)
+  idx_np = np.array([-1, -37, -38, -1000, 36, 37, 5000, 0, -2, 3, 2 ** 31 - 1, -2 ** 31], np.int64).astype(np.int32)
+  idx = torch.tensor(idx_np, device=device)
+  got = tokamax_amd.ragged_gather(x, idx, 0, rows)
+  assert np.array_equal(_np(got), O.ragged_gather(_np(x), idx_np))
+  got = tokamax_amd.ragged_scatter(x, idx, torch.tensor([0], device=device), torch.tensor([rows], device=device))
+  assert np.array_equal(_np(got), O.ragged_scatter(_np(x), idx_np, 0, rows))
+  w = torch.tensor(rng.uniform(0, 1, 12).astype(np.float32), device=device)
+  got = tokamax_amd.ragged_gather_reduce(x, idx, w, torch.ones(12, dtype=torch.bool, device=device), 3)
+  _check(got, O.ragged_gather_reduce(_np(x), idx_np, _np(w), np.ones(12, bool), 3), 3e-3)
+
+
+@pytest.mark.parametrize("cfg", [hip_ops.KernelConfig(128, 128, 64, 2, 2, 4, grid_tile_width=4),
+                                 hip_ops.KernelConfig(256, 256, 32, 2, 4, 4, grid_tile_width=8),
+                                 hip_ops.KernelConfig(32, 128, 64, 1, 4, 4, grid_tile_width=2),
+                                 hip_ops.KernelConfig(16, 128, 32, 1, 4, 2)])
+@pytest.mark.parametrize("gs", [(300, 300, 300, 300), (5, 2000, 7, 1), (0, 0, 5000, 0), (129, 129, 129, 300)])
+def test_group_sizes_that_add_up_to_more_than_m(cfg, gs, device):
+  """Unchecked group sizes (checkify is off by default, base.py:223) whose sum exceeds m: the rows below m match
+  the oracle, nothing is written past the output (guard rows around it stay as they were) and the call returns."""
+  G, m, k, n = 4, 520, 1024, 256
+  rng = np.random.default_rng(sum(gs))
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  rhs = torch.tensor(rng.normal(0, k ** -0.5, (G, k, n)).astype(np.float32), device=device).to(torch.bfloat16)
+  gs_t = torch.tensor(gs, dtype=torch.int32, device=device)
+  lib = _lib.load()
+  guard = 64
+  buf = torch.full((m + 2 * guard, n), 7.0, dtype=torch.bfloat16, device=device)
+  out = buf[guard:guard + m]
+  ws = hip_ops.workspace(m, G, cfg.block_m, device)
+  ws_guarded = torch.full((ws.numel() + 512,), -12345, dtype=torch.int32, device=device)
+  c = cfg.to_c()
+  import ctypes
+  for mode, a, b_, cols in ((0, lhs, rhs, n), (1, torch.tensor(rng.normal(0, 1, (m, n)).astype(np.float32), device=device).to(torch.bfloat16), rhs, k)):
+    if mode == 1 and cfg.block_m == 16:
+      continue
+    obuf = torch.full((m + 2 * guard, cols), 7.0, dtype=torch.bfloat16, device=device)
+    o = obuf[guard:guard + m]
+    st = lib.tkx_ragged_dot_fwd(a.data_ptr(), b_.data_ptr(), gs_t.data_ptr(), None, None, o.data_ptr(),
+                                ws_guarded[256:].data_ptr(), m, k, n, G, _lib.TKX_BF16, _lib.TKX_BF16, _lib.TKX_BF16, mode, 0,
+                                ctypes.byref(c), torch.cuda.current_stream().cuda_stream)
+    _lib.check(st)
+    torch.cuda.synchronize()
+    assert (obuf[:guard] == 7.0).all() and (obuf[guard + m:] == 7.0).all()
+    assert (ws_guarded[:256] == -12345).all() and (ws_guarded[256 + ws.numel():] == -12345).all()
+    want = O.ragged_dot(_np(a), _np(rhs), np.array(gs), O.DEFAULT if mode == 0 else O.TRANS_RHS, acc_dtype=np.float64,
+                        out_dtype="f64")
+    _check(o, want, 2e-3)
+  del buf, out
+
+
 def test_hip_graph_replays_follow_new_inputs_and_group_sizes(device):
   """The entry points allocate nothing, synchronise nothing and schedule on the device, so a captured
   HIP graph stays valid when the contents of lhs, the weights and even group_sizes change between

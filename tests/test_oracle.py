@@ -333,6 +333,46 @@ def test_row_movement_ops_against_loops():
   np.testing.assert_allclose(O.ragged_gather_reduce(x, idx, w, valid, 2), want, rtol=1e-6, atol=1e-7)
 
 
+def test_row_lookup_outside_the_array_wraps_then_clamps():
+  """`x[indices]` in the reference is JAX indexing: -1 is the last row, and what is still outside is clamped."""
+  x = np.arange(12, dtype=np.float32).reshape(4, 3)
+  idx = np.array([-1, -4, -5, -100, 3, 4, 99, 0], np.int32)
+  want = np.stack([x[3], x[0], x[0], x[0], x[3], x[3], x[3], x[0]])  # by hand
+  assert np.array_equal(O.ragged_gather(x, idx), want)
+  # the scatter mask tests the index as given: -1 lies outside [0, 4) although it reads the last row
+  assert np.array_equal(O.ragged_scatter(x, idx, 0, 4), np.where(((idx >= 0) & (idx < 4))[:, None], want, 0))
+  got = O.ragged_gather_reduce(x, idx, np.ones(8, np.float32), np.ones(8, bool), 2)
+  assert np.array_equal(got, want.reshape(4, 2, 3).sum(1))
+
+
+@pytest.mark.parametrize("gs,m,tile", [([300, 300, 300], 512, 128), ([5, 1000, 7], 256, 64), ([0, 2000], 130, 32),
+                                        ([129, 129, 129, 129, 129, 129, 129, 129], 520, 128), ([4000], 8, 16)])
+def test_group_sizes_beyond_m_keep_every_row_below_m_inside_the_task_slots(gs, m, tile):
+  """Group sizes are unchecked device data (checkify is off by default, base.py:223): they may add up to more
+  than m. The task arrays have tid_size = cdiv(m, tile) + G - 1 slots; the claim the kernels rely on is that
+  every task that stores a row below m has an index below tid_size, so dropping the tasks past the slots and
+  cutting the stored rows at m loses nothing below m and never indexes past the arrays."""
+  G = len(gs)
+  tid_size = -(-m // tile) + G - 1
+  big = O.group_info_create_aligned(np.array(gs, np.int32), tile, 4 * (sum(gs) // tile + G + 1), 8)
+  nt = big["num_tasks"]
+  assert nt > tid_size or sum(gs) <= m + tile * G  # (the cases are meant to overflow the slots)
+  covered = np.zeros(m, bool)
+  for t in range(nt):
+    lo, hi = int(big["actual_start"][t]), int(big["actual_end"][t])
+    if lo < m:
+      assert t < tid_size, (t, tid_size, lo)
+      hi = min(hi, m)            # what the kernel stores after its clamp
+      assert not covered[lo:hi].any()
+      covered[lo:hi] = True
+  assert covered[:min(m, sum(gs))].all()
+  # the slots the kernel does read hold the same tasks as the unbounded schedule
+  small = O.group_info_create_aligned(np.array(gs, np.int32), tile, tid_size, 8)
+  for name in ("group_id", "block_start", "actual_start", "actual_end"):
+    keep = min(nt, tid_size)
+    assert np.array_equal(small[name][:keep], big[name][:keep])
+
+
 def test_dequantize_is_tile_repeat():
   rng = np.random.default_rng(9)
   q = rng.integers(-127, 128, (2, 8, 6)).astype(np.int8)

@@ -84,6 +84,7 @@ struct GemmParams {
   int32_t num_groups;
   int32_t n_tiles, m_tiles;         // tiles along C columns; along C rows (drhs only)
   int32_t real_slots;               // fwd/dlhs: workgroups that may own a task tile (multiple of 8 * kXcdChunk)
+  int32_t tid_size;                 // fwd/dlhs: slots of the schedule's task arrays
   int32_t grid_tile_width;
   int32_t out_dtype, activation;
   int32_t scale_blocks, log2_block_rows;  // kFwdSubK: b_scale is [g, scale_blocks, n]; rows of k per block = 1 << log2
@@ -96,6 +97,7 @@ struct Variant {
   int32_t block_m, block_n, block_k, waves_m, waves_n, num_stages;
   int32_t smem_bytes;
   const void* fn;  // __global__ void (*)(GemmParams)
+  int32_t split_b; // > 0: the split pipeline (B stages of block_k / 2); whole A stages of contraction only
 };
 
 // ---- decode (small-m streaming kernel; int8 or 16-bit weights) -----------------------------------

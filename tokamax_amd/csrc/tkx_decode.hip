@@ -403,8 +403,9 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
 // Whether the decode kernel can run this problem (else the caller uses the tiled kernel).
 bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k, int64_t n, int64_t G,
                       int64_t scale_blocks, int32_t block_n) {
-  (void)m;
   (void)G;
+  // The lhs rows of a group are addressed through one buffer with 32-bit byte offsets (a group may hold all m rows).
+  if (m * k * 2 >= (1LL << 32)) return false;
   if (block_n != kDecBN) {
     // The wide kernel: int8 weights with per-column scales, 16 columns per lane.
     if (block_n != 2 * kDecBN || rhs_dtype != TKX_I8 || scale_blocks != 1 || n % 16 != 0) return false;

@@ -31,14 +31,18 @@ template <int ESZ>
 __global__ __launch_bounds__(kGatherThreads) void gather_rows_kernel(const GatherParams p) {
   constexpr int PER = 16 / ESZ;  // elements per 16-byte access
   const int chunks = p.hidden / PER;
-  const int lo = p.start ? p.start[0] : INT32_MIN, hi = p.end ? p.end[0] : INT32_MAX;
+  const bool ranged = p.start != nullptr;
+  const int lo = ranged ? p.start[0] : 0, hi = ranged ? p.end[0] : 0;
   constexpr int RMAX = 8;  // gathered rows per output row whose index, mask and weight are read once per row
   for (int64_t j = blockIdx.x; j < p.out_rows; j += gridDim.x) {
     // Source row (-1: dropped) and weight of gathered row g.
     auto source = [&](int64_t g, int64_t& row, float& w) {
       const int idx = p.indices[g];
-      const bool keep = idx >= lo && idx < hi && !(p.valid && p.valid[g] == 0);
-      row = !keep ? -1 : idx < 0 ? 0 : idx >= p.in_rows ? p.in_rows - 1 : idx;
+      const bool keep = (!ranged || (idx >= lo && idx < hi)) && !(p.valid && p.valid[g] == 0);
+      // x[indices] as the reference's indexing reads it: a negative index counts from the end, and what is
+      // still outside the array after that is clamped to the nearest row.
+      const int64_t wrapped = idx < 0 ? (int64_t)idx + p.in_rows : (int64_t)idx;
+      row = !keep ? -1 : wrapped < 0 ? 0 : wrapped >= p.in_rows ? p.in_rows - 1 : wrapped;
       w = p.weights ? p.weights[g] : 1.f;
     };
     int64_t rows[RMAX];

@@ -282,9 +282,6 @@ __device__ __forceinline__ void barrier_after_direct_loads() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
   // s_waitcnt immediate: vmcnt = bits [3:0] and [15:14], expcnt = [6:4] (7: no wait), lgkmcnt = [11:8] (0: all).
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4));
-#if defined(TKX_ABLATE) && (TKX_ABLATE & 8)
-  return;
-#endif
   __syncthreads();
 }
 
@@ -359,9 +356,6 @@ struct DirectLoader {
   // Instruction i (0 <= i < PER) of this wave's share: `base` = wave-uniform pointer of the k-step,
   // `tile_lds` = LDS byte address of the destination tile (wave-uniform).
   __device__ __forceinline__ void issue_one(int i, const unsigned char* base, unsigned tile_lds, int wave) const {
-#if defined(TKX_ABLATE) && (TKX_ABLATE & 1)
-    return;
-#endif
     const int j = i * NWAVES + wave;
     if (INSTRS % NWAVES != 0 && j >= INSTRS) return;
     if constexpr (STRIDED) direct_load_16(base + i * stride, voff[0], tile_lds + j * 1024);
@@ -469,8 +463,40 @@ __device__ __forceinline__ void store4_as(unsigned char* ptr, f32x4 v) {
 }
 
 // ---- the kernel ---------------------------------------------------------------------------------
-template <int MODE, int EA, int EB, int BM, int BN, int BK, int WM, int WN, int NS>
+// How many of the most recently issued direct loads a wave may leave in flight at the barrier of compute step
+// `kt` of the split pipeline (GemmKernel with HB > 0). Loads go out in a fixed order: step t issues, if t is odd,
+// the PA loads of A double-step (t - 1) / 2 + NS and then the PB loads of B step t + HB (negative t: the
+// prologue, which follows the same order from t = -max(HB, 2 NS) on). The barrier of step kt needs B step kt + 1
+// and A double-step (kt + 1) / 2 complete; loads complete in issue order, so everything issued after the later of
+// the two may stay in flight. kt = -1 is the barrier before the first step.
+constexpr int split_loads_in_flight(int kt, int NS, int HB, int PA, int PB) {
+  const int look = HB > 2 * NS ? HB : 2 * NS;
+  int after_a = -1, after_b = -1, count = 0;
+  for (int t = kt - 1; t >= -look; --t) {  // backwards: within a step the B loads were issued last
+    const int s = t + HB;
+    if (s >= 0) {
+      if (s == kt + 1) after_b = count;
+      count += PB;
+    }
+    if (t & 1) {
+      const int j = (t - 1) / 2 + NS;
+      if (j >= 0) {
+        if (j == (kt + 1) / 2) after_a = count;
+        count += PA;
+      }
+    }
+  }
+  return after_a < after_b ? after_a : after_b;
+}
+
+// HB > 0 ("split pipeline", forward with a contraction-contiguous A): BK is the depth of an A stage and half of it
+// the depth of a compute step and of a B stage; NS A stages and HB B stages. A row of an A stage is then a whole
+// 128-byte line for 16-bit elements at BK = 64, where a stage as deep as a compute step holds half a line per row
+// and every line of A is requested from L2 twice, once by each of two consecutive steps.
+template <int MODE, int EA, int EB, int BM, int BN, int BK, int WM, int WN, int NS, int HB = 0>
 struct GemmKernel {
+  static constexpr bool SPLIT = HB > 0;
+  static constexpr int BKC = SPLIT ? BK / 2 : BK;  // contraction elements per compute step
   static constexpr int THREADS = WM * WN * 64;
   static constexpr int LA = (MODE == kDrhs) ? kMC : kKC;
   static constexpr int LB = (MODE == kDlhs) ? kKC : kMC;
@@ -491,20 +517,21 @@ struct GemmKernel {
   static_assert(MODE != kFwdGlu || TN % 2 == 0, "gate-up tiles pair the two halves of a wave's column blocks");
   static constexpr int TNO = MODE == kFwdGlu ? TN / 2 : TN, WTNO = MODE == kFwdGlu ? WTN / 2 : WTN;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % KA == 0, "tile does not split into 32x32 atoms");
-  static constexpr int KSTEPS = BK / KA;
+  static constexpr int KSTEPS = BKC / KA;
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
+  static_assert(!SPLIT || (MODE == kFwd && EA == EB && BK % 2 == 0), "split pipeline: plain forward, operands of one type");
   typedef TileStage<LA, EA, BM, BK, THREADS> StageA;
-  typedef TileStage<LB, EB, BN, BK, THREADS> StageB;
+  typedef TileStage<LB, EB, BN, BKC, THREADS> StageB;
   // Every wave takes an equal share of a k-step's direct-to-LDS loads.
   static constexpr int NLOAD = WM * WN;
   typedef DirectLoader<LA, EA, BM, BK, NLOAD> DirA;
-  typedef DirectLoader<LB, EB, BN, BK, NLOAD> DirB;
+  typedef DirectLoader<LB, EB, BN, BKC, NLOAD> DirB;
   static constexpr int SCALE_BYTES = (SUBK && !SUBP) ? BN * 4 : 0;  // kFwdSubK: the k-step's scale row behind its two tiles
   static constexpr int STAGE_BYTES = StageA::BYTES + StageB::BYTES + SCALE_BYTES;
   // fp8 x fp8: the scales of a k-step (BN weight-column scales, then BM lhs-row scales) are still needed when its
   // stage is already being refilled, so they live in a ring of NS + 1 slots behind the stages.
   static constexpr int RING_SLOT = SUBP ? (BN + BM) * 4 : 0;
-  static constexpr int SMEM_BYTES = NS * STAGE_BYTES + (NS + 1) * RING_SLOT;
+  static constexpr int SMEM_BYTES = SPLIT ? NS * StageA::BYTES + HB * StageB::BYTES : NS * STAGE_BYTES + (NS + 1) * RING_SLOT;
   static_assert(NS >= 2 && SMEM_BYTES <= 160 * 1024, "stages must fit the 160 KB LDS");
 
   static __device__ __forceinline__ void run(const GemmParams& p, unsigned char* smem) {
@@ -521,7 +548,10 @@ struct GemmKernel {
 
     int group, row0, act_start, act_end, col0, kc_begin, kc_end;
     if constexpr (MODE != kDrhs) {
-      const int num_tasks = ws[0];
+      // (Group sizes are device data nobody has checked: when they add up to more than m_ext rows the schedule
+      // holds more tasks than its arrays have slots for. Every task with a row below m_ext has a slot, so the rest
+      // are dropped here, and the tasks kept store no row at or past m_ext.)
+      const int num_tasks = min(ws[0], p.tid_size);
       if (b >= p.real_slots) {
         // Tail duty: rows [total_rows, m_ext), and with a group offset the rows before the first
         // group, belong to no group of this call and are defined to be zero.
@@ -554,10 +584,12 @@ struct GemmKernel {
       const int rem = L - first * p.n_tiles;
       const int nt = rem / width;
       const int mt = first + (rem - nt * width);
+      if (mt >= p.tid_size) return;  // (a span that runs past the last slot: rows past m_ext only)
       group = ws[p.ws_gid + mt];
       row0 = ws[p.ws_bstart + mt];
-      act_start = ws[p.ws_astart + mt];
-      act_end = ws[p.ws_aend + mt];
+      act_end = min(ws[p.ws_aend + mt], p.m_ext);
+      act_start = min(ws[p.ws_astart + mt], act_end);
+      if (act_start >= act_end) return;  // (every row of the task lies at or past m_ext)
       col0 = nt * BNO;
       kc_begin = 0;
       kc_end = p.k_ext;
@@ -617,9 +649,6 @@ struct GemmKernel {
       }
     };
     auto load_frags = [&](auto full, Frag* fa, Frag* fb, const unsigned char* stage, int kk) {
-#if defined(TKX_ABLATE) && (TKX_ABLATE & 2)
-      return;
-#endif
 #pragma unroll
       for (int i = 0; i < TM; ++i)
         if (decltype(full)::value || ((rmask >> i) & 1u))
@@ -630,11 +659,6 @@ struct GemmKernel {
       }
     };
     auto mma_all = [&](auto full, const Frag* fa, const Frag* fb) {
-#if defined(TKX_ABLATE) && (TKX_ABLATE & 4)
-      for (int i = 0; i < TM; ++i) asm volatile("" ::"v"(fa[i]));
-      for (int j = 0; j < TN; ++j) asm volatile("" ::"v"(fb[j]));
-      return;
-#endif
 #pragma unroll
       for (int i = 0; i < TM; ++i)
         if (decltype(full)::value || ((rmask >> i) & 1u)) {
@@ -644,10 +668,157 @@ struct GemmKernel {
     };
 
     const int span = kc_end - kc_begin;
-    const int nfull = span > 0 ? span / BK : 0;  // whole k-steps: direct-to-LDS, software pipelined
-    const bool tail = span > nfull * BK;         // partial last k-step: zero-filled through registers
+    const int nfull = span > 0 ? span / BKC : 0;  // whole k-steps: direct-to-LDS, software pipelined
+    const bool tail = span > nfull * BKC;         // partial last k-step: zero-filled through registers
 
-    if (nfull > 0) {
+    if constexpr (SPLIT) {
+      // The launcher takes this variant only when the contraction is a whole number of A stages, so nfull is even
+      // and there is no partial step.
+      DirA da;
+      DirB db;
+      const int a_hi = max(min(act_end, p.m_ext), 1), a_lo = min(max(act_start, 0), a_hi - 1);
+      da.init(row0, p.m_ext, p.lda, wave, lane, a_lo, a_hi);
+      db.init(col0, p.nb_ext, p.ldb, wave, lane, 0, p.nb_ext);
+      const unsigned char* const gA0 = Ab + DirA::step_base(row0, p.lda, kc_begin);
+      const unsigned char* const gB0 = Bb + DirB::step_base(col0, p.ldb, kc_begin);
+      const int64_t stepA = DirA::step_bytes(p.lda), stepB = DirB::step_bytes(p.ldb);
+      const unsigned smem_lds = lds_address32(smem);
+      constexpr int A_BYTES = StageA::BYTES, B_BYTES = StageB::BYTES, B_REGION = NS * A_BYTES;
+      constexpr int PA = DirA::PER, PB = DirB::PER;
+      static_assert(DirA::INSTRS % NLOAD == 0 && DirB::INSTRS % NLOAD == 0, "split pipeline: the loads split evenly over the waves");
+      constexpr int LOOK = HB > 2 * NS ? HB : 2 * NS;  // steps between the issue of a load and the last step that may need it
+      constexpr int kFirst = split_loads_in_flight(-1, NS, HB, PA, PB);
+      constexpr int kEven = split_loads_in_flight(4 * LOOK, NS, HB, PA, PB), kOdd = split_loads_in_flight(4 * LOOK + 1, NS, HB, PA, PB);
+      static_assert(kFirst >= 0 && kEven >= 0 && kOdd >= 0 && kFirst < 64, "split pipeline: load order does not cover a needed step");
+      const int ndouble = nfull / 2;
+      auto issue_a = [&](int q, int dstep, int stage) {
+        da.issue_one(q, uniform_pointer(gA0 + dstep * stepA), smem_lds + stage * A_BYTES, wave);
+      };
+      auto issue_b = [&](int q, int step, int stage) {
+        db.issue_one(q, uniform_pointer(gB0 + step * stepB), smem_lds + B_REGION + stage * B_BYTES, wave);
+      };
+      // Prologue, in the order of the steady state (steps -LOOK .. -1).
+#pragma unroll
+      for (int t = -LOOK; t < 0; ++t) {
+        if (t & 1) {
+          const int j = (t - 1) / 2 + NS;
+          if (j >= 0 && j < ndouble) {
+#pragma unroll
+            for (int q = 0; q < PA; ++q) issue_a(q, j, j);
+          }
+        }
+        const int s_ = t + HB;
+        if (s_ >= 0 && s_ < nfull) {
+#pragma unroll
+          for (int q = 0; q < PB; ++q) issue_b(q, s_, s_);
+        }
+      }
+      if (nfull >= LOOK) barrier_after_direct_loads<kFirst>();
+      else barrier_after_direct_loads<0>();
+
+      auto k_loop = [&](auto full) {
+        constexpr bool F = decltype(full)::value;
+        Frag fa[2][TM], fb[2][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[0][i] = fa[1][i] = Frag{};
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[0][j] = fb[1][j] = Frag{};
+        // Read number r of an atom, in the order its MFMAs (row block major) first use the fragments.
+        auto read_frag = [&](Frag* a, Frag* b, int r, const unsigned char* atile, int akk, const unsigned char* btile, int bkk) {
+          if (r >= TM + TN) return;
+          const int f = r == 0 ? 0 : r <= TN ? TM + r - 1 : r - TN;
+          if (f < TM) {
+            if (F || ((rmask >> f) & 1u)) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(atile, row_block(f) * 32, akk, lane);
+          } else {
+            if (F || rmask != 0) b[f - TM] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(btile, wn * WTN + (f - TM) * 32, bkk, lane);
+          }
+        };
+        constexpr int NM = TM * TN;
+        constexpr int RPM = (TM + TN + NM - 1) / NM;
+        // One atom: its MFMAs with, threaded between them, the reads of the next atom's fragments and (`NL` > 0) load
+        // slots 0 .. NL - 1 of `issue`.
+        auto atom = [&](auto nl_tag, const Frag* a, const Frag* b, Frag* na, Frag* nb, const unsigned char* atile, int akk,
+                        const unsigned char* btile, int bkk, auto issue) {
+          constexpr int NL = decltype(nl_tag)::value;
+          constexpr int LPM = (NL + NM - 1) / NM;
+#pragma unroll
+          for (int t = 0; t < NM; ++t) {
+            const int i = t / TN, j = t % TN;
+            if (F || ((rmask >> i) & 1u)) acc[i][j] = mma_atom<EC>(b[j], a[i], acc[i][j]);
+#pragma unroll
+            for (int r = 0; r < RPM; ++r) read_frag(na, nb, t * RPM + r, atile, akk, btile, bkk);
+#pragma unroll
+            for (int q = 0; q < LPM; ++q)
+              if (t * LPM + q < NL) issue(t * LPM + q);
+            if (F) __builtin_amdgcn_sched_barrier(0);
+          }
+        };
+        auto no_loads = [](int) {};
+#pragma unroll
+        for (int f = 0; f < TM + TN; ++f) read_frag(fa[0], fb[0], f, smem, 0, smem + B_REGION, 0);
+        int a_idx = 0, b_idx = 0;  // stages of the current step
+        // One compute step. ODD: second half of its A stage, which it releases. STEADY: every load this step and the
+        // LOOK steps before it could issue exists, so the loads in flight are known at compile time; the other steps
+        // (the last few of a tile) issue what is left in one piece and wait for everything.
+        auto k_step = [&](auto odd_tag, auto steady_tag, int kt) {
+          constexpr bool ODD = decltype(odd_tag)::value, STEADY = decltype(steady_tag)::value;
+          const unsigned char* const a_cur = smem + a_idx * A_BYTES;
+          const unsigned char* const b_cur = smem + B_REGION + b_idx * B_BYTES;
+          constexpr int akk0 = ODD ? KSTEPS : 0;
+          const int a_freed = a_idx, b_freed = b_idx;
+          if (ODD) a_idx = a_idx + 1 == NS ? 0 : a_idx + 1;
+          b_idx = b_idx + 1 == HB ? 0 : b_idx + 1;
+          const unsigned char* const a_nxt = smem + a_idx * A_BYTES;
+          const unsigned char* const b_nxt = smem + B_REGION + b_idx * B_BYTES;
+          constexpr int nkk0 = ODD ? 0 : KSTEPS;
+          // (Pointers of the refills are computed here, far ahead of the MFMAs they are issued between.)
+          const unsigned char* const src_b = uniform_pointer(gB0 + (int64_t)(kt + HB) * stepB);
+          const unsigned char* const src_a = uniform_pointer(gA0 + (int64_t)((kt - 1) / 2 + NS) * stepA);
+          const unsigned dst_b = smem_lds + B_REGION + b_freed * B_BYTES, dst_a = smem_lds + a_freed * A_BYTES;
+#pragma unroll
+          for (int kk = 0; kk + 1 < KSTEPS; ++kk)
+            atom(std::integral_constant<int, 0>{}, fa[kk & 1], fb[kk & 1], fa[(kk + 1) & 1], fb[(kk + 1) & 1], a_cur,
+                 akk0 + kk + 1, b_cur, kk + 1, no_loads);
+          // All LDS reads of this step are issued. After the barrier the next step's operands are complete and this
+          // step's B stage (and, after an odd step, its A stage) is free.
+          if constexpr (STEADY) {
+            barrier_after_direct_loads<(ODD ? kOdd : kEven)>();
+            auto issue = [&](int q) {
+              if (ODD && q < PA) da.issue_one(q, src_a, dst_a, wave);
+              else db.issue_one(q - (ODD ? PA : 0), src_b, dst_b, wave);
+            };
+            atom(std::integral_constant<int, (ODD ? PA : 0) + PB>{}, fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1], fa[0], fb[0],
+                 a_nxt, nkk0, b_nxt, 0, issue);
+          } else {
+            barrier_after_direct_loads<0>();
+            if (ODD && (kt - 1) / 2 + NS < ndouble) {
+#pragma unroll
+              for (int q = 0; q < PA; ++q) da.issue_one(q, src_a, dst_a, wave);
+            }
+            if (kt + HB < nfull) {
+#pragma unroll
+              for (int q = 0; q < PB; ++q) db.issue_one(q, src_b, dst_b, wave);
+            }
+            // (After the last step the reads below fetch fragments nobody uses, from LDS that is there.)
+            atom(std::integral_constant<int, 0>{}, fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1], fa[0], fb[0], a_nxt, nkk0,
+                 b_nxt, 0, no_loads);
+          }
+        };
+        int kt = 0;
+        for (; kt + 2 + LOOK <= nfull; kt += 2) {
+          k_step(std::false_type{}, std::true_type{}, kt);
+          k_step(std::true_type{}, std::true_type{}, kt + 1);
+        }
+        for (; kt < nfull; kt += 2) {
+          k_step(std::false_type{}, std::false_type{}, kt);
+          k_step(std::true_type{}, std::false_type{}, kt + 1);
+        }
+      };
+      if (nfull > 0) {
+        if (all_rows) k_loop(std::true_type{});
+        else k_loop(std::false_type{});
+      }
+    } else if (nfull > 0) {
       DirA da;
       DirB db;
       const int a_hi = max(min(act_end, p.m_ext), 1), a_lo = min(max(act_start, 0), a_hi - 1);
@@ -738,9 +909,6 @@ struct GemmKernel {
         // TM*TN - 2 MFMAs before its first use. A fragment f < TM is the A fragment of row block f,
         // else the B fragment f - TM.
         auto read_frag = [&](Frag* a, Frag* b, int r, const unsigned char* stage, int kk) {
-#if defined(TKX_ABLATE) && (TKX_ABLATE & 2)
-          return;
-#endif
           if (r >= TM + TN) return;
           const int f = r == 0 ? 0 : r <= TN ? TM + r - 1 : r - TN;
           if (f < TM) {
@@ -761,9 +929,6 @@ struct GemmKernel {
 #pragma unroll
           for (int t = 0; t < NM; ++t) {
             const int i = t / TN, j = t % TN;
-#if defined(TKX_ABLATE) && (TKX_ABLATE & 4)
-            asm volatile("" ::"v"(a[i]), "v"(b[j]));
-#else
             if constexpr (SUBP) {
               if (F || ((rmask >> i) & 1u)) {
                 f32x16 c = pacc[i][j];
@@ -776,7 +941,6 @@ struct GemmKernel {
             } else {
               if (F || ((rmask >> i) & 1u)) acc[i][j] = mma_atom<EC>(b[j], a[i], acc[i][j]);
             }
-#endif
             if (reads) {
 #pragma unroll
               for (int r = 0; r < RPM; ++r) read_frag(na, nb, t * RPM + r, rd_stage, rd_kk);
@@ -871,7 +1035,7 @@ struct GemmKernel {
       if (all_rows) k_loop(std::true_type{});
       else k_loop(std::false_type{});
     }
-    if (tail && !GLU && !SUBK) {  // (gate-up and per-k-block-scale problems are taken only with whole k-steps)
+    if (tail && !GLU && !SUBK && !SPLIT) {  // (gate-up, per-k-block-scale and split-pipeline problems are taken only with whole k-steps)
       const int kc0 = kc_begin + nfull * BK;
       StageA::copy(Ab, p.lda, row0, p.m_ext, kc0, kc_end, smem, tid);
       StageB::copy(Bb, p.ldb, col0, p.nb_ext, kc0, kc_end, smem + StageA::BYTES, tid);
@@ -1082,6 +1246,12 @@ __global__ __launch_bounds__(K::THREADS, K::THREADS <= 256 ? 2 : 1) void gemm_en
   extern __shared__ __attribute__((aligned(1024))) unsigned char tkx_smem[];
   K::run(p, tkx_smem);
 }
+
+#define TKX_VARIANT_SPLIT(MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB)                                           \
+  {                                                                                                            \
+    MODE, EA, EB, BM, BN, BK, WM, WN, NS, ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>::SMEM_BYTES, \
+        reinterpret_cast<const void*>(&::tkx::gemm_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>>), HB \
+  }
 
 #define TKX_VARIANT(MODE, EA, EB, BM, BN, BK, WM, WN, NS)                                            \
   {                                                                                                  \

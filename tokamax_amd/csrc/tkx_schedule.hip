@@ -124,7 +124,9 @@ __global__ __launch_bounds__(kThreads) void schedule_kernel(const int32_t* __res
     // Span of this task: the group's T tasks are cut into ceil(T / span_width) spans of nearly equal
     // width, so that the tasks that run side by side on an n-panel all use the same group's weights.
     int32_t sfirst = task, swidth = 1;
-    const int32_t T = start_tasks[g + 1] - start_tasks[g], idx = task - start_tasks[g];
+    // (Sizes that add up to more than m rows make more tasks than slots: spans end with the slots, so that the
+    // launch order, which walks whole spans, stays inside the arrays.)
+    const int32_t T = min(start_tasks[g + 1], tid_size) - start_tasks[g], idx = task - start_tasks[g];
     if (task < num_tasks && idx < T) {
       const int32_t nspans = (T + span_width - 1) / span_width;
       const int32_t base = T / nspans, extra = T - base * nspans;  // the first `extra` spans are one wider

@@ -8,6 +8,8 @@ namespace tkx {
 #define DRHS(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kDrhs, kEBF16, kEBF16, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
+    // split pipeline: A stages of 64 (whole 128-byte lines), B stages of 32; (A stages, B stages) = (3, 4): 160 KB
+    TKX_VARIANT_SPLIT(kFwd, kEBF16, kEBF16, 256, 256, 64, 2, 4, 3, 4),
     FWD_DLHS(256, 256, 64, 2, 4, 2),
     FWD_DLHS(256, 256, 32, 2, 4, 4),
     FWD_DLHS(256, 256, 32, 2, 4, 5),

@@ -421,7 +421,11 @@ def _call_with_vjp(op: Op, ba: BoundArguments, config, return_residuals: bool):
       kwargs = dict(bound.kwargs)
       kwargs["return_residuals"] = True
       out, residuals = op._fwd(*bound.args, config=config, **kwargs)  # pylint: disable=protected-access
-      ctx.bound, ctx.out, ctx.residuals = bound, out, residuals
+      # Inputs and residuals go through save_for_backward, and the output is not kept at all (`vjp` does not use
+      # it): a tensor this function returns, held as a plain attribute of ctx, would close the cycle
+      # out -> grad_fn -> ctx -> out, and the activations would live until the cyclic collector runs.
+      ctx.has_residuals = residuals is not None
+      ctx.save_for_backward(*ts, *([residuals] if residuals is not None else []))
       if return_residuals:
         ctx.mark_non_differentiable(residuals)
         return out, residuals
@@ -429,11 +433,15 @@ def _call_with_vjp(op: Op, ba: BoundArguments, config, return_residuals: bool):
 
     @staticmethod
     def backward(ctx, dout, *unused):
-      bound = ctx.bound
+      saved = ctx.saved_tensors
+      ts, residuals = (saved[:-1], saved[-1]) if ctx.has_residuals else (saved, None)
+      full = dict(arguments)
+      full.update(zip(names, ts))
+      bound = BoundArguments(op, full)
       kwargs = dict(bound.kwargs)
       kwargs.pop("return_residuals")
       with torch.no_grad():
-        grads = op.vjp(ctx.residuals, ctx.out, dout, *bound.args, **kwargs)
+        grads = op.vjp(residuals, None, dout, *bound.args, **kwargs)
       by_name = dict(grads) if isinstance(grads, dict) else dict(zip(pos_names, grads))
       return tuple(by_name.get(n) for n in names)
 

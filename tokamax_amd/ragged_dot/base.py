@@ -330,40 +330,30 @@ def vjp(
       a = activation(r)
     (dout,) = torch.autograd.grad(a, r, dout.to(a.dtype))
 
-  dot_dim_nums = ragged_dot_dimension_numbers.dot_dimension_numbers
-  lhs_ragged = ragged_dot_dimension_numbers.lhs_ragged_dimensions
-  rhs_group = ragged_dot_dimension_numbers.rhs_group_dimensions
-  (lhs_contract, rhs_contract), (lhs_batch, rhs_batch) = dot_dim_nums
-  lhs_not_kept = (*lhs_batch, *lhs_contract)
-  rhs_not_kept = (*rhs_batch, *rhs_contract, *rhs_group)
-  lhs_kept = [i for i in range(lhs.ndim) if i not in lhs_not_kept]
-  rhs_kept = [i for i in range(rhs.ndim) if i not in rhs_not_kept]
-
-  assert len(lhs_batch) == len(rhs_batch)
-  assert dout.ndim == len(lhs_batch) + len(lhs_kept) + len(rhs_kept)
-  dout_batch = list(range(len(lhs_batch)))
-  dout_lhs_kept = list(range(len(lhs_batch), len(lhs_batch) + len(lhs_kept)))
-  dout_rhs_kept = list(range(len(lhs_batch) + len(lhs_kept), dout.ndim))
-
-  dlhs_dims = ((dout_rhs_kept, rhs_kept), (dout_batch, rhs_batch))
-  dout_ragged = [(len(dout_batch) + lhs_kept.index(d)) for d in lhs_ragged]
-
-  dlhs = dlhs_ragged_dot(
-      dout,
-      rhs,
-      group_sizes=group_sizes,
-      ragged_dot_dimension_numbers=RaggedDotDimensionNumbers(dlhs_dims, dout_ragged, rhs_group),
-      precision=precision,
-      preferred_element_type=lhs.dtype,
-  )
-
-  drhs_dims = ((lhs_kept, dout_lhs_kept), (lhs_batch, dout_batch))
-  drhs = drhs_ragged_dot(
-      lhs,
-      dout,
-      group_sizes=group_sizes,
-      ragged_dot_dimension_numbers=RaggedDotDimensionNumbers(drhs_dims, lhs_ragged, []),
-      precision=precision,
-      preferred_element_type=rhs.dtype,
-  )
+  # The two cotangents are ragged dots again (base.py:416-461 derives their dimension numbers from the forward's
+  # in general). The kernels here know three layouts, so the derivation is a table: for each forward layout, the
+  # operands and the layout of the product that yields each cotangent.
+  try:
+    (dlhs_a, dlhs_b, dlhs_dims), (drhs_a, drhs_b, drhs_dims) = _COTANGENT_PRODUCTS[ragged_dot_dimension_numbers]
+  except KeyError:
+    raise NotImplementedError("Unsupported ragged dot dimension numbers on the backward path.") from None
+  operands = {"lhs": lhs, "rhs": rhs, "dout": dout}
+  dlhs = dlhs_ragged_dot(operands[dlhs_a], operands[dlhs_b], group_sizes=group_sizes,
+                         ragged_dot_dimension_numbers=dlhs_dims, precision=precision, preferred_element_type=lhs.dtype)
+  drhs = drhs_ragged_dot(operands[drhs_a], operands[drhs_b], group_sizes=group_sizes,
+                         ragged_dot_dimension_numbers=drhs_dims, precision=precision, preferred_element_type=rhs.dtype)
   return dlhs, drhs
+
+
+# forward layout -> ((first operand, second operand, layout) for d lhs, the same for d rhs)
+_COTANGENT_PRODUCTS = {
+    # out[m,n] = lhs[m,k] . rhs[g,k,n]:  dlhs[m,k] = dout[m,n] . rhs[g,k,n]^T,  drhs[g,k,n] = lhs[rows_g]^T . dout[rows_g]
+    DEFAULT_RAGGED_DOT_DIM_NUMS: (("dout", "rhs", TRANS_RHS_RAGGED_DOT_DIM_NUMS),
+                                  ("lhs", "dout", RAGGED_CONTRACTING_DOT_DIM_NUMS)),
+    # out[m,k] = lhs[m,n] . rhs[g,k,n]^T:  dlhs[m,n] = dout[m,k] . rhs[g,k,n],  drhs[g,k,n] = dout[rows_g]^T . lhs[rows_g]
+    TRANS_RHS_RAGGED_DOT_DIM_NUMS: (("dout", "rhs", DEFAULT_RAGGED_DOT_DIM_NUMS),
+                                    ("dout", "lhs", RAGGED_CONTRACTING_DOT_DIM_NUMS)),
+    # out[g,k,n] = lhs[rows_g,k]^T . rhs[rows_g,n]:  dlhs[m,k] = rhs[m,n] . dout[g,k,n]^T,  drhs[m,n] = lhs[m,k] . dout[g,k,n]
+    RAGGED_CONTRACTING_DOT_DIM_NUMS: (("rhs", "dout", TRANS_RHS_RAGGED_DOT_DIM_NUMS),
+                                      ("lhs", "dout", DEFAULT_RAGGED_DOT_DIM_NUMS)),
+}
