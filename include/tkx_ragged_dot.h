@@ -119,6 +119,20 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
                            int32_t rhs_dtype, int32_t out_dtype, int32_t mode, int32_t activation,
                            const TkxConfig* config, tkx_stream_t stream);
 
+/* tkx_ragged_dot_fwd for callers that cannot hand over a workspace they allocated: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference (XLA owns every buffer
+ * there). Same arguments and results as tkx_ragged_dot_fwd, without `workspace`: the schedule arrays live in a
+ * 256 KiB device array inside the library (one copy per GPU, held until the process ends), which limits
+ * tkx_ragged_dot_workspace_bytes(m, num_groups, block_m) to 262144, i.e. about cdiv(m, block_m) + num_groups <= 8100;
+ * larger problems return TKX_ERR_UNSUPPORTED. The call allocates and frees nothing. All calls on one GPU share that
+ * array: two of them that overlap in time (different streams or threads) race; calls on one stream are ordered.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress) and should be made outside capture. */
+int32_t tkx_ragged_dot_fwd_static_workspace(const void* lhs, const void* rhs, const int32_t* group_sizes,
+                                            const float* lhs_scale, const float* rhs_scale, void* out, int64_t m,
+                                            int64_t k, int64_t n, int64_t num_groups, int32_t lhs_dtype,
+                                            int32_t rhs_dtype, int32_t out_dtype, int32_t mode, int32_t activation,
+                                            const TkxConfig* config, tkx_stream_t stream);
+
 /* Forward (mode DEFAULT) with the fused epilogue terms of base.py:205-217.
  *   rhs_bias: f32[G,n] added to the scaled accumulator, or NULL.
  *   gateup = 1: rhs is [G,k,n] with its columns [gate | up] (n/2 each) and out is [m, n/2] =

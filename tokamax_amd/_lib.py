@@ -28,6 +28,7 @@ EXPORTED_SYMBOLS = (
     "tkx_ragged_dot_workspace_offset",
     "tkx_ragged_dot_schedule",
     "tkx_ragged_dot_fwd",
+    "tkx_ragged_dot_fwd_static_workspace",
     "tkx_ragged_dot_fwd_fused",
     "tkx_ragged_dot_drhs",
     "tkx_dequantize_weights",
@@ -76,6 +77,8 @@ def _declare(lib):
   lib.tkx_ragged_dot_schedule.argtypes = [vp, i64, i64, i32, i32, vp, vp]
   lib.tkx_ragged_dot_fwd.restype = i32
   lib.tkx_ragged_dot_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32, i32, i32, i32, cfgp, vp]
+  lib.tkx_ragged_dot_fwd_static_workspace.restype = i32
+  lib.tkx_ragged_dot_fwd_static_workspace.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32, i32, i32, i32, cfgp, vp]
   lib.tkx_ragged_dot_fwd_fused.restype = i32
   lib.tkx_ragged_dot_fwd_fused.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, i32,
                                            i32, i32, i32, cfgp, vp]

@@ -6,6 +6,12 @@
 
 #include "tkx_common.h"
 
+// Schedule workspace of tkx_ragged_dot_fwd_static_workspace: one copy per GPU the library runs on, held until the
+// process ends. In host code this name is only a handle for hipGetSymbolAddress; the device address it yields
+// (one per device) is what kernels and copies take.
+constexpr int64_t kScratchWords = 64 * 1024;  // 256 KiB of int32
+static __device__ __align__(256) int32_t scratch[kScratchWords];
+
 namespace tkx {
 
 static thread_local char g_err[512] = "";
@@ -70,7 +76,7 @@ int32_t prepare(const Variant* v) {
   for (auto& d : done)
     if (d.first == dev && d.second == v->fn) return TKX_OK;
   TKX_HIP_CHECK(hipFuncSetAttribute(v->fn, hipFuncAttributeMaxDynamicSharedMemorySize, v->smem_bytes));
-  done.emplace_back(dev, v->fn);
+  done.emplace_back(dev, v->fn);  // (host memory, once per kernel and device)
   return TKX_OK;
 }
 
@@ -86,6 +92,26 @@ int32_t launch(const Variant* v, const GemmParams& p, int64_t grid, hipStream_t 
 }
 
 bool valid_out_dtype(int d) { return d == TKX_F32 || d == TKX_BF16 || d == TKX_F16; }
+
+// Device address of `scratch` on the current device, looked up once per device (each GPU holds its own copy of
+// the array at its own address). Fixed-size table: nothing here allocates.
+int32_t scratch_address(int32_t** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static int32_t* address[kMaxDevices] = {};
+  int dev = 0;
+  TKX_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return set_error(TKX_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (address[dev] == nullptr) {
+    void* ptr = nullptr;
+    TKX_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) return set_error(TKX_ERR_RUNTIME, "hipGetSymbolAddress returned a null address");
+    address[dev] = static_cast<int32_t*>(ptr);
+  }
+  *out = address[dev];
+  return TKX_OK;
+}
 
 }  // namespace
 }  // namespace tkx
@@ -295,6 +321,28 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
                            int32_t activation, const TkxConfig* config, tkx_stream_t stream) {
   return fwd_impl(lhs, rhs, group_sizes, nullptr, lhs_scale, rhs_scale, nullptr, out, workspace, m, k, n, num_groups,
                   num_groups, lhs_dtype, rhs_dtype, out_dtype, mode, activation, false, 1, config, stream);
+}
+
+int32_t tkx_ragged_dot_fwd_static_workspace(const void* lhs, const void* rhs, const int32_t* group_sizes,
+                                            const float* lhs_scale, const float* rhs_scale, void* out, int64_t m, int64_t k,
+                                            int64_t n, int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype,
+                                            int32_t out_dtype, int32_t mode, int32_t activation, const TkxConfig* config,
+                                            tkx_stream_t stream) {
+  if (config == nullptr) return set_error(TKX_ERR_INVALID, "null pointer argument");
+  if (m < 1 || num_groups < 1 || config->block_m < 1)
+    return set_error(TKX_ERR_INVALID, "bad sizes m=%lld G=%lld block_m=%d", (long long)m, (long long)num_groups, config->block_m);
+  const int64_t words = ws_layout(m, num_groups, config->block_m).words;
+  if (words > kScratchWords)
+    return set_error(TKX_ERR_UNSUPPORTED,
+                     "the schedule of m=%lld, G=%lld, block_m=%d needs %lld bytes; the built-in workspace holds %lld"
+                     " (use tkx_ragged_dot_fwd with a workspace of your own)",
+                     (long long)m, (long long)num_groups, config->block_m, (long long)(words * 4), (long long)(kScratchWords * 4));
+  int32_t* ws = nullptr;
+  const int32_t st = scratch_address(&ws);
+  if (st != TKX_OK) return st;
+  // The scheduler kernel writes every word the GEMM kernel reads, so nothing of the last call's contents matters.
+  return fwd_impl(lhs, rhs, group_sizes, nullptr, lhs_scale, rhs_scale, nullptr, out, ws, m, k, n, num_groups, num_groups,
+                  lhs_dtype, rhs_dtype, out_dtype, mode, activation, false, 1, config, stream);
 }
 
 int32_t tkx_ragged_dot_fwd_fused(const void* lhs, const void* rhs, const int32_t* group_sizes, const int32_t* group_offset,
