@@ -441,6 +441,33 @@ def test_every_kernel_variant_through_c_abi(v, device):
   assert torch.count_nonzero(out[int(gs.sum()):]) == 0
 
 
+def _plain_tiled_variants():
+  """Forward and dlhs tile variants whose operands share one unquantised type."""
+  return [v for v in _variant_cases() if v.values[0]["mode"] in (0, 1) and v.values[0]["block_m"] != 16
+          and v.values[0]["lhs_dtype"] == v.values[0]["rhs_dtype"] and v.values[0]["lhs_dtype"] in (_lib.TKX_F32, _lib.TKX_BF16, _lib.TKX_F16)]
+
+
+@pytest.mark.parametrize("contraction", [40, 104, 200])
+@pytest.mark.parametrize("v", _plain_tiled_variants())
+def test_contraction_lengths_that_are_not_whole_steps(v, contraction, device):
+  """Any contraction length whose rows are 16-byte multiples is taken: what the pipelined k-steps leave over (a
+  partial step; for the split-pipeline variants up to two) goes through a zero-filled masked path."""
+  rng = np.random.default_rng(contraction + v["block_k"])
+  G, m, other = 3, 200, 136
+  gs = np.array([90, 0, 97], np.int32)
+  dt = _TORCH_DTYPE[v["lhs_dtype"]]
+  trans = v["mode"] == 1
+  k, n = (other, contraction) if trans else (contraction, other)
+  mk = lambda shape, std: torch.tensor(rng.normal(0, std, shape).astype(np.float32), device=device).to(dt)
+  lhs, rhs = mk((m, contraction), 1.0), mk((G, k, n), contraction ** -0.5)
+  cfg = hip_ops.KernelConfig(v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"], v["num_stages"],
+                             grid_tile_width=2)
+  out = hip_ops.ragged_dot_fwd(lhs, rhs, torch.tensor(gs, device=device), config=cfg, out_dtype=torch.float32, trans_rhs=trans)
+  want = O.ragged_dot(_np(lhs), _np(rhs), gs, O.TRANS_RHS if trans else O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, 1e-5)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+
+
 @pytest.mark.parametrize("block_n,depth", [(128, 2), (128, 4), (128, 8), (256, 2), (256, 4)])
 @pytest.mark.parametrize("case", ["ragged", "two_chunks", "all_empty", "one_big_group", "first_and_last_empty",
                                   "many_groups"])

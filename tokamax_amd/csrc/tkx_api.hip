@@ -232,9 +232,7 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
                      mode, lhs_dtype, rhs_dtype, c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages);
   // In C terms: rows = m; cols = n (fwd) or k (dlhs); contraction = k (fwd) or n (dlhs).
   const int64_t cols = dlhs ? k : gateup ? n / 2 : n, contraction = dlhs ? n : k;
-  if (v->split_b > 0 && contraction % v->block_k != 0)
-    return set_error(TKX_ERR_UNSUPPORTED, "this variant needs the contraction (%lld) to be a multiple of block_k=%d",
-                     (long long)contraction, v->block_k);
+
   const int lb = dtype_bytes(lhs_dtype), rb = dtype_bytes(rhs_dtype), ob = dtype_bytes(out_dtype);
   // 16-byte vector accesses: every row of every operand must start 16-byte aligned and the tile
   // loaders move whole 16-byte chunks along the contiguous axis. The contraction size itself need

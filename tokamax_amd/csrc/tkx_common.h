@@ -97,7 +97,7 @@ struct Variant {
   int32_t block_m, block_n, block_k, waves_m, waves_n, num_stages;
   int32_t smem_bytes;
   const void* fn;  // __global__ void (*)(GemmParams)
-  int32_t split_b; // > 0: the split pipeline (B stages of block_k / 2); whole A stages of contraction only
+  int32_t split_b; // > 0: the split pipeline (that many B stages of block_k / 2; num_stages A stages of block_k)
 };
 
 // ---- decode (small-m streaming kernel; int8 or 16-bit weights) -----------------------------------

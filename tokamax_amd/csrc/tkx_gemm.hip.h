@@ -463,6 +463,17 @@ __device__ __forceinline__ void store4_as(unsigned char* ptr, f32x4 v) {
 }
 
 // ---- the kernel ---------------------------------------------------------------------------------
+// Calls f(integral_constant<int, sel>) for a run-time sel in [I, N].
+template <int I, int N, class Fn>
+__device__ __forceinline__ void dispatch_upto(int sel, Fn&& f) {
+  if constexpr (I < N) {
+    if (sel == I) f(std::integral_constant<int, I>{});
+    else dispatch_upto<I + 1, N>(sel, f);
+  } else {
+    f(std::integral_constant<int, N>{});
+  }
+}
+
 // How many of the most recently issued direct loads a wave may leave in flight at the barrier of compute step
 // `kt` of the split pipeline (GemmKernel with HB > 0). Loads go out in a fixed order: step t issues, if t is odd,
 // the PA loads of A double-step (t - 1) / 2 + NS and then the PB loads of B step t + HB (negative t: the
@@ -631,7 +642,11 @@ struct GemmKernel {
       if (r0 < act_end && r0 + 32 > act_start) rmask |= 1u << i;
     }
     rmask = __builtin_amdgcn_readfirstlane(rmask);
-    const bool all_rows = rmask == (1u << TM) - 1u;
+    // The blocks with rows are the first `nv` of the wave (a task's rows start in the tile's first 8 rows and the
+    // blocks of a wave ascend through the tile), so the k loop is compiled once per count: straight-line code for
+    // whole and partial tiles alike, no test around an MFMA. (Any other pattern computes every block.)
+    const int nv_count = __builtin_popcount(rmask);
+    const int nv_sel = rmask == (1u << nv_count) - 1u ? nv_count : TM;
     // B fragment j of k-atom kk of a stage. kFwdSubK: the int8 values of the lane's column (lane % 32 of the
     // block) are multiplied by that column's scale for the stage's k-block, which lies behind the tiles.
     auto load_b_frag = [&](const unsigned char* stage, int j, int kk) -> Frag {
@@ -648,32 +663,16 @@ struct GemmKernel {
         return load_frag<LB, EB, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + j * 32, kk, lane);
       }
     };
-    auto load_frags = [&](auto full, Frag* fa, Frag* fb, const unsigned char* stage, int kk) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        if (decltype(full)::value || ((rmask >> i) & 1u))
-          fa[i] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, row_block(i) * 32, kk, lane);
-      if (decltype(full)::value || rmask != 0) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j) fb[j] = load_b_frag(stage, j, kk);
-      }
-    };
-    auto mma_all = [&](auto full, const Frag* fa, const Frag* fb) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        if (decltype(full)::value || ((rmask >> i) & 1u)) {
-#pragma unroll
-          for (int j = 0; j < TN; ++j) acc[i][j] = mma_atom<EC>(fb[j], fa[i], acc[i][j]);
-        }
-    };
-
     const int span = kc_end - kc_begin;
     const int nfull = span > 0 ? span / BKC : 0;  // whole k-steps: direct-to-LDS, software pipelined
-    const bool tail = span > nfull * BKC;         // partial last k-step: zero-filled through registers
+    // (split pipeline: whole A stages, i.e. an even number of compute steps)
+    const int nmain = SPLIT ? (span > 0 ? span / BK * 2 : 0) : nfull;
+    const bool tail = span > nmain * BKC;         // the rest of the contraction: zero-filled steps through registers
 
     if constexpr (SPLIT) {
-      // The launcher takes this variant only when the contraction is a whole number of A stages, so nfull is even
-      // and there is no partial step.
+      // The pipelined loop takes whole A stages (pairs of compute steps); what is left of the contraction, less than
+      // one A stage, goes through the masked path below.
+      const int nfull = nmain;
       DirA da;
       DirB db;
       const int a_hi = max(min(act_end, p.m_ext), 1), a_lo = min(max(act_start, 0), a_hi - 1);
@@ -716,8 +715,8 @@ struct GemmKernel {
       if (nfull >= LOOK) barrier_after_direct_loads<kFirst>();
       else barrier_after_direct_loads<0>();
 
-      auto k_loop = [&](auto full) {
-        constexpr bool F = decltype(full)::value;
+      auto k_loop = [&](auto nv_tag) {
+        constexpr int NV = decltype(nv_tag)::value;  // row blocks of this wave that hold rows of the task
         Frag fa[2][TM], fb[2][TN];
 #pragma unroll
         for (int i = 0; i < TM; ++i) fa[0][i] = fa[1][i] = Frag{};
@@ -728,9 +727,9 @@ struct GemmKernel {
           if (r >= TM + TN) return;
           const int f = r == 0 ? 0 : r <= TN ? TM + r - 1 : r - TN;
           if (f < TM) {
-            if (F || ((rmask >> f) & 1u)) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(atile, row_block(f) * 32, akk, lane);
+            if (f < NV) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(atile, row_block(f) * 32, akk, lane);
           } else {
-            if (F || rmask != 0) b[f - TM] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(btile, wn * WTN + (f - TM) * 32, bkk, lane);
+            if (NV > 0) b[f - TM] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(btile, wn * WTN + (f - TM) * 32, bkk, lane);
           }
         };
         constexpr int NM = TM * TN;
@@ -744,13 +743,13 @@ struct GemmKernel {
 #pragma unroll
           for (int t = 0; t < NM; ++t) {
             const int i = t / TN, j = t % TN;
-            if (F || ((rmask >> i) & 1u)) acc[i][j] = mma_atom<EC>(b[j], a[i], acc[i][j]);
+            if (i < NV) acc[i][j] = mma_atom<EC>(b[j], a[i], acc[i][j]);
 #pragma unroll
             for (int r = 0; r < RPM; ++r) read_frag(na, nb, t * RPM + r, atile, akk, btile, bkk);
 #pragma unroll
             for (int q = 0; q < LPM; ++q)
               if (t * LPM + q < NL) issue(t * LPM + q);
-            if (F) __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_sched_barrier(0);
           }
         };
         auto no_loads = [](int) {};
@@ -814,10 +813,7 @@ struct GemmKernel {
           k_step(std::true_type{}, std::false_type{}, kt + 1);
         }
       };
-      if (nfull > 0) {
-        if (all_rows) k_loop(std::true_type{});
-        else k_loop(std::false_type{});
-      }
+      if (nfull > 0) dispatch_upto<0, TM>(nv_sel, k_loop);
     } else if (nfull > 0) {
       DirA da;
       DirB db;
@@ -897,8 +893,8 @@ struct GemmKernel {
       // atom's fragments and, in the last atom of a k-step, the global loads that refill the stage
       // just released are threaded between those MFMAs one by one, so that the matrix pipe is
       // never left waiting behind a block of memory instructions.
-      auto k_loop = [&](auto full) {
-        constexpr bool F = decltype(full)::value;
+      auto k_loop = [&](auto nv_tag) {
+        constexpr int NV = decltype(nv_tag)::value;  // row blocks of this wave that hold rows of the task
         Frag fa[2][TM], fb[2][TN];
 #pragma unroll
         for (int i = 0; i < TM; ++i) fa[0][i] = fa[1][i] = Frag{};
@@ -912,9 +908,9 @@ struct GemmKernel {
           if (r >= TM + TN) return;
           const int f = r == 0 ? 0 : r <= TN ? TM + r - 1 : r - TN;
           if (f < TM) {
-            if (F || ((rmask >> f) & 1u)) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, row_block(f) * 32, kk, lane);
+            if (f < NV) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, row_block(f) * 32, kk, lane);
           } else if (f < TM + TN) {
-            if (F || rmask != 0) b[f - TM] = load_b_frag(stage, f - TM, kk);
+            if (NV > 0) b[f - TM] = load_b_frag(stage, f - TM, kk);
           }
         };
         constexpr int NM = TM * TN;                      // MFMAs per atom
@@ -930,7 +926,7 @@ struct GemmKernel {
           for (int t = 0; t < NM; ++t) {
             const int i = t / TN, j = t % TN;
             if constexpr (SUBP) {
-              if (F || ((rmask >> i) & 1u)) {
+              if (i < NV) {
                 f32x16 c = pacc[i][j];
                 if constexpr (first_of_step) {
 #pragma unroll
@@ -939,7 +935,7 @@ struct GemmKernel {
                 pacc[i][j] = mma_atom<EC>(b[j], a[i], c);
               }
             } else {
-              if (F || ((rmask >> i) & 1u)) acc[i][j] = mma_atom<EC>(b[j], a[i], acc[i][j]);
+              if (i < NV) acc[i][j] = mma_atom<EC>(b[j], a[i], acc[i][j]);
             }
             if (reads) {
 #pragma unroll
@@ -949,7 +945,7 @@ struct GemmKernel {
 #pragma unroll
               for (int q = 0; q < LPM; ++q) issue_slot(t * LPM + q, sp);
             }
-            if (F) __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_sched_barrier(0);
           }
         };
 
@@ -1014,7 +1010,7 @@ struct GemmKernel {
                 const f32x4 wsc = *reinterpret_cast<const f32x4*>(slot + 4 * (wn * WTN + j * 32 + 8 * t + 4 * (lane >> 5)));
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
-                  if (F || ((rmask >> i) & 1u)) {
+                  if (i < NV) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                       float part = pacc[i][j][4 * t + e];
@@ -1032,23 +1028,37 @@ struct GemmKernel {
         for (; kt + 1 < nfull; ++kt) k_step(std::false_type{}, std::true_type{}, kt);
         for (; kt < nfull; ++kt) k_step(std::false_type{}, std::false_type{}, kt);
       };
-      if (all_rows) k_loop(std::true_type{});
-      else k_loop(std::false_type{});
+      dispatch_upto<0, TM>(nv_sel, k_loop);
     }
-    if (tail && !GLU && !SUBK && !SPLIT) {  // (gate-up, per-k-block-scale and split-pipeline problems are taken only with whole k-steps)
-      const int kc0 = kc_begin + nfull * BK;
-      StageA::copy(Ab, p.lda, row0, p.m_ext, kc0, kc_end, smem, tid);
-      StageB::copy(Bb, p.ldb, col0, p.nb_ext, kc0, kc_end, smem + StageA::BYTES, tid);
-      __syncthreads();
+    if constexpr (!GLU && !SUBK) if (tail) {  // (gate-up and per-k-block-scale problems are taken only with whole k-steps)
+      typedef TileStage<LA, EA, BM, BKC, THREADS> TailA;  // (an A tile as deep as a compute step)
+      for (int kc0 = kc_begin + nmain * BKC; kc0 < kc_end; kc0 += BKC) {
+        if (kc0 > kc_begin) __syncthreads();  // the tile's last reads of the LDS written below are done
+        TailA::copy(Ab, p.lda, row0, p.m_ext, kc0, kc_end, smem, tid);
+        StageB::copy(Bb, p.ldb, col0, p.nb_ext, kc0, kc_end, smem + TailA::BYTES, tid);
+        __syncthreads();
 #pragma unroll
-      for (int kk = 0; kk < KSTEPS; ++kk) {
-        Frag fa[TM], fb[TN];
+        for (int kk = 0; kk < KSTEPS; ++kk) {
+          Frag fa[TM], fb[TN];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[i] = Frag{};
+          for (int i = 0; i < TM; ++i) fa[i] = Frag{};
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fb[j] = Frag{};
-        load_frags(std::false_type{}, fa, fb, smem, kk);
-        mma_all(std::false_type{}, fa, fb);
+          for (int j = 0; j < TN; ++j) fb[j] = Frag{};
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            if ((rmask >> i) & 1u) fa[i] = load_frag<LA, EA, EC, TailA::ROW_BYTES>(smem, row_block(i) * 32, kk, lane);
+          if (rmask != 0) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+              fb[j] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(smem + TailA::BYTES, wn * WTN + j * 32, kk, lane);
+          }
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            if ((rmask >> i) & 1u) {
+#pragma unroll
+              for (int j = 0; j < TN; ++j) acc[i][j] = mma_atom<EC>(fb[j], fa[i], acc[i][j]);
+            }
+        }
       }
     }
 

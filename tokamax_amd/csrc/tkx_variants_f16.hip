@@ -7,6 +7,7 @@ namespace tkx {
 #define DRHS(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kDrhs, kEF16, kEF16, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
+    TKX_VARIANT_SPLIT(kFwd, kEF16, kEF16, 256, 256, 64, 2, 4, 3, 4),  // A stages of 64 (whole lines), B stages of 32
     FWD_DLHS(256, 256, 32, 2, 4, 4),
     FWD_DLHS(128, 256, 64, 2, 4, 3),
     FWD_DLHS(128, 128, 64, 2, 2, 4),
