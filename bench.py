@@ -324,6 +324,53 @@ def main():
             2 * m_ * k_ * 2 * n_, nb, "mfma", "bf16", cfg)
     del lhs, rhs
 
+    # The reference's own benchmark shapes with published timings on other hardware (tokamax/_src/ops/ragged_dot/
+    # arg_specs.py:23-60; standard-normal inputs and representative group sizes as its benchmarks make them):
+    # `8x7b` (B200: 0.734 ms Triton, 1.050 ms Mosaic), `compute_bound` (B200: 0.105 ms Triton) and `memory_bound`
+    # (one row per group over 268 MB of bf16 weights; B200: 0.0418 ms Triton), the last timed as a graph.
+    from tokamax_amd.ragged_dot import arg_specs
+    for spec in arg_specs.ARG_SPECS:
+      if spec.name not in ("8x7b", "compute_bound", "memory_bound"):
+        continue
+      kw = arg_specs.random_initialize(spec.args, device)
+      lhs_, rhs_, gs_ = kw["lhs"], kw["rhs"], kw["group_sizes"]
+      sizes = spec.args["group_sizes"].representative_value
+      rows_, touched = int(sum(sizes)), sum(1 for x in sizes if x > 0)
+      cfg = op.bind(lhs_, rhs_, group_sizes=gs_).default_config
+      fl = arg_specs.flops(**spec.args)
+      nb = (rows_ * rhs_.shape[1] + touched * rhs_.shape[1] * rhs_.shape[2] + lhs_.shape[0] * rhs_.shape[2]) * 2
+      key = "arg_spec_" + spec.full_name
+      if spec.name == "memory_bound":
+        copies_ = [rhs_] + [rhs_.clone() for _ in range(2)]  # 3 x 268 MB defeat the 256 MB last-level cache
+        m_ = _time_graph([(lambda r=r: op(lhs_, r, group_sizes=gs_)) for r in copies_], 24)
+        extras[key] = dict(ms_per_step=round(m_, 5), gbs=round(nb / m_ / 1e6, 2), timing="HIP graph of 24 back-to-back launches",
+                           roofline=_roofline("hbm", fl, nb, m_, "bf16"),
+                           kernel_config=[cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages])
+        del copies_
+      else:
+        measure(key, lambda: op(lhs_, rhs_, group_sizes=gs_), fl, nb, "mfma", "bf16", cfg)
+      del kw, lhs_, rhs_, gs_
+
+    # Stated ceilings of this box, same run, same kind of data (context for the fractions above, not product code):
+    # the vendor library's dense bf16 GEMM on one expert's worth of the Mixtral shape in the layout the forward pass
+    # has (NN: weights [k, n]) and in the transposed one (NT), and an elementwise copy of 1 GiB.
+    a_ = torch.randn(16384, 4096, device=device, dtype=torch.bfloat16, generator=gen)
+    b_nn = (torch.randn(4096, 14336, device=device, dtype=torch.float32, generator=gen) * 4096 ** -0.5).to(torch.bfloat16)
+    b_nt = b_nn.t().contiguous()
+    c_ = torch.empty(16384, 14336, device=device, dtype=torch.bfloat16)
+    dense_flops = 2 * 16384 * 4096 * 14336
+    t_nn, _, _ = _time_steps(lambda: torch.matmul(a_, b_nn, out=c_), steps, warm, stream)
+    t_nt, _, _ = _time_steps(lambda: torch.matmul(a_, b_nt.t(), out=c_), steps, warm, stream)
+    src_ = torch.zeros(1 << 28, dtype=torch.int32, device=device)
+    dst_ = torch.empty_like(src_)
+    t_cp, _, _ = _time_steps(lambda: dst_.copy_(src_), steps, warm, stream)
+    extras["ceilings_same_box"] = dict(
+        dense_bf16_matmul_nn_tflops=round(dense_flops / (t_nn / steps) / 1e9, 1),
+        dense_bf16_matmul_nt_tflops=round(dense_flops / (t_nt / steps) / 1e9, 1),
+        copy_1gib_read_plus_write_gbs=round(2 * (1 << 30) / (t_cp / steps) / 1e6, 1),
+        note="torch.matmul [16384,4096] x [4096,14336] bf16 (random normal data) and torch copy_ of 1 GiB, HIP-event timed")
+    del a_, b_nn, b_nt, c_, src_, dst_
+
     w = workloads.make("decode", device, seed=0)
     gs = torch.tensor(w.group_sizes, device=device)
     copies = [(torch.randn(w.num_groups, w.k, w.n, device=device, dtype=torch.float32, generator=gen) * w.k ** -0.5)

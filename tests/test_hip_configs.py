@@ -12,7 +12,7 @@ import torch
 
 import tokamax_amd
 from oracle import ragged_dot_oracle as O
-from tokamax_amd.ragged_dot import base, workloads
+from tokamax_amd.ragged_dot import arg_specs, base, workloads
 
 pytestmark = pytest.mark.gpu
 
@@ -131,3 +131,27 @@ def test_vjp_config(device):
   out.backward(w.dout[:512])
   want_dlhs = tokamax_amd.ragged_dot_general(w.dout[:512], w.rhs, torch.tensor(small, device=device), base.TRANS_RHS_RAGGED_DOT_DIM_NUMS)
   assert torch.equal(lhs.grad, want_dlhs)
+
+
+@pytest.mark.parametrize("spec", [s for s in arg_specs.ARG_SPECS if "ci_tests" in s.tags], ids=lambda s: s.full_name)
+def test_bench_arg_specs(spec, device):
+  """The reference's `test_bench` (test_base.py:316-344) over its `ci_tests` arg specs (arg_specs.py:23-60:
+  compute_bound, memory_bound, mixtral 8x7b): standard-normal inputs, representative group sizes, the first
+  sum(group_sizes) rows against the reference definition within atol=0.01, rtol=0.005 (the 8x7b shape on sampled
+  rows of every group, the other two in full)."""
+  kwargs = arg_specs.random_initialize(spec.args, device)
+  lhs, rhs, gs = kwargs["lhs"], kwargs["rhs"], kwargs["group_sizes"]
+  sizes = np.array(spec.args["group_sizes"].representative_value, np.int32)
+  count = int(sizes.sum())
+  assert count <= lhs.shape[0] and tuple(gs.shape) == (rhs.shape[0],)
+  out = tokamax_amd.ragged_dot(lhs, rhs, gs)
+  assert out.dtype == torch.bfloat16 and tuple(out.shape) == (lhs.shape[0], rhs.shape[2])
+  if lhs.shape[0] * rhs.shape[1] * rhs.shape[2] <= 2 ** 37:
+    want = O.ragged_dot(_np(lhs), _np(rhs), sizes, acc_dtype=np.float32, out_dtype="f32")
+    np.testing.assert_allclose(_np(out)[:count], want[:count], atol=0.01, rtol=0.005)
+    assert O.rel_l2(_np(out)[:count], want[:count]) <= 2e-3
+  else:
+    rows, groups = _sample_rows(sizes, 24, 5)
+    lhs_f = _np(lhs[torch.as_tensor(rows, device=device)])
+    _check_rows(out, lhs_f, lambda g: _np(rhs[g]), rows, groups, 2e-3)
+  assert arg_specs.flops(**spec.args) == 2 * count * rhs.shape[1] * rhs.shape[2]

@@ -1209,3 +1209,33 @@ def test_autotune_on_device(device):
   with res:
     assert ba.default_config == best
   assert tokamax_amd.op.device_kind() == "AMD Instinct MI355X"
+
+
+def test_autotune_of_a_function_on_device(device):
+  """`tokamax_amd.autotune(f, *args)` (autotuning/api.py:322-418) on a function that calls the ragged dot twice with
+  different shapes and once through `jax.grad`'s counterpart: each distinct call is found, tuned on the device and
+  served from the result when it is used as an overlay."""
+  a, b, gs = _inputs("test_autotune_fn", 8, 1024, 128, 256, torch.bfloat16, device)
+  gst = torch.tensor(gs, device=device)
+  a2, b2 = a[:512, :64].contiguous(), b[:, :64, :128].contiguous()
+  gs2 = torch.tensor(gs // 2, device=device)
+
+  def layer(x, w, x2, w2):
+    y = tokamax_amd.ragged_dot(x, w, gst)
+    y2 = tokamax_amd.ragged_dot(x2, w2, gs2)
+    return y, y2, tokamax_amd.ragged_dot(x, w, gst)  # (a repeated call: one entry)
+
+  found = tokamax_amd.get_bound_args(layer, a, b, a2, b2)
+  assert [tuple(ba.arguments["lhs"].shape) for ba in found] == [(1024, 128), (512, 64)]
+  res = tokamax_amd.autotune(layer, a, b, a2, b2, autotuner=tokamax_amd.autotuning.autotuner.Autotuner(iterations=2, warmup=1))
+  assert res.device_kind == "AMD Instinct MI355X" and len(res.data) == 2
+  want = layer(a, b, a2, b2)
+  with res:
+    for ba, data in res.data:
+      assert ba.default_config == data.fastest_config
+      assert data[data.fastest_config].median_evaluation_time_ms > 0
+    got = layer(a, b, a2, b2)
+  for g, w_ in zip(got, want):
+    _check(g, _np(w_), 2e-3)
+  back = tokamax_amd.AutotuningResult.loads(res.dumps(), {"HipRaggedDot": OP})
+  assert [d.fastest_config for _, d in back.data] == [d.fastest_config for _, d in res.data]

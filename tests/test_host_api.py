@@ -399,6 +399,65 @@ def test_cache_file_name_and_json_round_trip(tmp_path):
         assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages) in tiles
 
 
+def test_autotune_discovers_the_ops_a_function_calls():
+  """`get_bound_args(f, *args, **kwargs)` and `autotune(f, *args)` (autotuning/api.py:202-239, :322-418; test pattern of
+  autotuning/api_test.py:42-60): the ops a function calls are found by running it, unique by (op, cache key), in call
+  order, without the config of the call; a list of bound arguments is taken as it is."""
+  class _Timer(autotuner_lib.Autotuner):
+    def autotune(self, fn_factory, configs, *args, timeout=None, **kwargs):
+      out = {}
+      for c in configs:
+        try:
+          fn_factory(c)(*args, **kwargs)
+          out[c] = _bench(float(c.foo))
+        except Exception as e:  # pylint: disable=broad-exception-caught
+          out[c] = e
+      return autotuner_lib.AutotuningData(out)
+
+  op = _FakeOp()
+
+  def f(x, y, scale=1.0):
+    a = op(x, y)                               # [3] + [3]
+    b = _FakeOp(config=_FakeConfig(7))(a, a)   # the same op and shapes again, with an explicit config: one entry
+    c = op(torch.zeros(5), torch.zeros(5))     # another shape: a second entry
+    return b * scale, c
+
+  x = torch.zeros(3)
+  found = tokamax_amd.get_bound_args(f, x, x, scale=2.0)
+  assert [tuple(ba.arguments["x"].shape) for ba in found] == [(3,), (5,)]
+  assert all(ba.op.config is None for ba in found)
+  assert op_lib.OP_CALL_RECORDER.get() is None  # nothing is recorded outside
+  assert tokamax_amd.get_bound_args(list(found)) == found
+  with pytest.raises(ValueError, match="only supported if `f` is callable"):
+    tokamax_amd.get_bound_args(list(found), x)
+  with pytest.raises(TypeError):
+    tokamax_amd.get_bound_args(3)
+
+  res = tokamax_amd.autotune(f, x, x, autotuner=_Timer())
+  assert isinstance(res, tokamax_amd.AutotuningResult) and len(res.data) == 2
+  assert res.device_kind == op_lib.device_kind()
+  for ba, data in res.data:
+    assert data.fastest_config == _FakeConfig(1) and isinstance(data[_FakeConfig(13)], RuntimeError)
+  assert [ba for ba, _ in res.data] == list(found)
+  with res:  # the result works as an overlay: the next call of `f` runs with the tuned config
+    assert op.bind(x, x).default_config == _FakeConfig(1)
+  assert op.bind(x, x).default_config == _FakeConfig(42)
+  # from a list of bound arguments; ops that already have cached data are skipped unless ignore_cache
+  assert len(tokamax_amd.autotune(list(found), autotuner=_Timer()).data) == 2
+  with res:
+    assert len(tokamax_amd.autotune(f, x, x, autotuner=_Timer()).data) == 0
+    assert len(tokamax_amd.autotune(f, x, x, autotuner=_Timer(), ignore_cache=True).data) == 2
+
+  # an op that cannot be tuned is logged and left out, the others still come back (api.py:403-416)
+  class _Broken(autotuner_lib.Autotuner):
+    def autotune(self, fn_factory, configs, *args, timeout=None, **kwargs):
+      if args[0].shape == (5,):
+        raise RuntimeError("no timer")
+      return _Timer().autotune(fn_factory, configs, *args, timeout=timeout, **kwargs)
+
+  assert [tuple(ba.arguments["x"].shape) for ba, _ in tokamax_amd.autotune(f, x, x, autotuner=_Broken()).data] == [(3,)]
+
+
 def test_bound_args_and_autotuning_result_round_trip():
   op = hip.HipRaggedDot()
   for spec in arg_specs.ARG_SPECS:  # ops/op_test.py:201-237 does this over all arg specs
@@ -476,3 +535,22 @@ def test_arg_specs_and_flops():
   assert {"compute_bound", "memory_bound", "mixtral_8x7b"} <= names
   s = next(s for s in arg_specs.ARG_SPECS if s.name == "8x7b")
   assert arg_specs.flops(**s.args) == 2 * 8192 * 4096 * 14336  # bench.py:52-56
+
+
+def test_ffi_shim_compiles_to_its_stub_without_the_xla_header(tmp_path):
+  """tokamax_amd/csrc/ffi_shim.cc holds the XLA FFI handlers behind `__has_include("xla/ffi/api/ffi.h")`; without the
+  header (this image has no jaxlib) it must still compile, to a stub that says so."""
+  import shutil
+  import subprocess
+  cxx = shutil.which("g++") or shutil.which("c++")
+  if cxx is None:
+    pytest.skip("no host C++ compiler")
+  src = os.path.join(ROOT, "tokamax_amd", "csrc", "ffi_shim.cc")
+  out = tmp_path / "libshim.so"
+  subprocess.check_call([cxx, "-std=c++17", "-shared", "-fPIC", "-I", os.path.join(ROOT, "include"), src, "-o", str(out)])
+  lib = ctypes.CDLL(str(out))
+  lib.tkx_ffi_shim_available.restype = ctypes.c_int32
+  assert lib.tkx_ffi_shim_available() == 0
+  text = open(src).read()
+  for symbol in ("TkxRaggedDotFwd", "TkxRaggedDotFwdFused", "TkxRaggedDotDrhs"):
+    assert f"XLA_FFI_DEFINE_HANDLER_SYMBOL({symbol}," in text

@@ -6,7 +6,7 @@ Public names follow tokamax/__init__.py:18-41 for this operator: `ragged_dot`,
 """
 
 from tokamax_amd import config
-from tokamax_amd.autotuning.api import AutotuningResult, autotune
+from tokamax_amd.autotuning.api import AutotuningResult, autotune, get_bound_args
 from tokamax_amd.op import AUTO, BoundArguments, NullConfig, Op
 from tokamax_amd.quantization import AsQArray, QArray
 from tokamax_amd.gated_linear_unit.api import gated_linear_unit
@@ -30,6 +30,6 @@ __all__ = [
     "HipRaggedDot",
     "HipRaggedDotConfig", "NullConfig", "Op", "QArray", "RAGGED_CONTRACTING_DOT_DIM_NUMS",
     "RAGGED_DOT_IMPLEMENTATIONS", "RaggedDotDimensionNumbers", "RaggedDotGroupSizes",
-    "TRANS_RHS_RAGGED_DOT_DIM_NUMS", "autotune", "config", "gated_linear_unit", "generate_group_sizes", "ragged_dot",
+    "TRANS_RHS_RAGGED_DOT_DIM_NUMS", "autotune", "get_bound_args", "config", "gated_linear_unit", "generate_group_sizes", "ragged_dot",
     "ragged_dot_general", "ragged_gather", "ragged_gather_reduce", "ragged_scatter",
 ]

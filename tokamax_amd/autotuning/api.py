@@ -1,16 +1,19 @@
-"""`autotune` and `AutotuningResult`.
+"""`autotune`, `get_bound_args` and `AutotuningResult`.
 
 Counterpart of tokamax/_src/autotuning/api.py: `AutotuningResult` (:70-199) is a serialisable set
 of (bound arguments -> timings) that can be pushed as an overlay over the shipped cache with a
-`with` block (:151-167); `autotune` (:322-418) tunes a list of bound arguments. The reference can
-also discover the ops inside a jitted function from its HLO; without a tracing compiler there is
-nothing to walk, so this `autotune` takes the bound arguments directly.
+`with` block (:151-167); `get_bound_args(f, *args, **kwargs)` (:202-239) lists the unique op calls a
+function makes; `autotune(f, *args)` (:322-418) tunes them, or a list of bound arguments. The
+reference finds the calls by lowering `f` and walking its HLO for the payload every op leaves there
+(hlo_utils.py:263-286); here `f` is run once, eagerly, while every `Op.__call__` records its bound
+arguments.
 """
 
 from __future__ import annotations
 
 import dataclasses
 import json
+import logging
 from typing import Iterable, Sequence
 
 from tokamax_amd import benchmarking
@@ -69,21 +72,59 @@ class AutotuningResult:
     return cls(raw["device_kind"], tuple(data))
 
 
-def autotune(bound_args: Iterable[op_lib.BoundArguments], *, ignore_cache: bool = False,
-             all_implementations: bool = False,
-             autotuner: autotuner_lib.Autotuner = autotuner_lib.Autotuner()) -> AutotuningResult:
-  """Autotunes each of `bound_args`; already cached ones are skipped unless `ignore_cache`."""
-  del all_implementations  # one implementation per op in this package
+def get_bound_args(f, *args, **kwargs) -> tuple:
+  """The unique `BoundArguments` of all ops `f(*args, **kwargs)` calls (api.py:202-239).
+
+  `f` is run once; ops are unique by (op class, autotuning cache key), in call order, and carry no config (the
+  one a call was made with is not part of what gets tuned). A sequence of `BoundArguments` is returned as it is."""
+  if isinstance(f, (list, tuple)) and all(isinstance(b, op_lib.BoundArguments) for b in f):
+    if args or kwargs:
+      raise ValueError("`args` / `kwargs` are only supported if `f` is callable.")
+    return tuple(f)
+  if not callable(f):
+    raise TypeError(f"expected a callable or a sequence of BoundArguments, got {type(f).__name__}")
+  calls: list = []
+  token = op_lib.OP_CALL_RECORDER.set(calls)
+  try:
+    f(*args, **kwargs)
+  finally:
+    op_lib.OP_CALL_RECORDER.reset(token)
+  seen, unique = set(), []
+  for ba in calls:
+    ba = op_lib.BoundArguments(ba.op.replace(config=None), ba.arguments)
+    key = (type(ba.op).__name__, ba.autotuning_cache_key)
+    if key not in seen:
+      seen.add(key)
+      unique.append(ba)
+  return tuple(unique)
+
+
+def autotune(f, *args, ignore_cache: bool = False, all_implementations: bool = False, progress_bar: bool = False,
+             timeout: float | None = 600.0, max_workers: int | None = None,
+             autotuner: autotuner_lib.Autotuner | None = None) -> AutotuningResult:
+  """Autotunes all ops `f(*args)` calls (api.py:322-418).
+
+  `f` is a callable or a sequence of `BoundArguments`; to tune a callable with keyword arguments pass
+  `get_bound_args(f, *args, **kwargs)`. Ops already in the autotuning cache are skipped unless `ignore_cache`. A
+  failure to tune one op is logged and leaves that op out of the result. `all_implementations` and `max_workers`
+  are accepted for the reference's signature: each op here has one implementation, and its kernel variants are
+  precompiled, so there is no compilation to spread over workers."""
+  del all_implementations, max_workers, progress_bar
+  bound_args = get_bound_args(f, *args)
+  if not ignore_cache:
+    bound_args = [ba for ba in bound_args if ba.cached_autotuning_data is None]
+  kinds = {k for k in map(op_lib.infer_device_kind, bound_args) if k is not None and k != "cpu"}
+  if len(kinds) > 1:
+    raise ValueError(f"Multiple device kinds found: {kinds}")
+  device_kind = kinds.pop() if kinds else op_lib.device_kind()
+  autotuner = autotuner if autotuner is not None else autotuner_lib.Autotuner()
   results = []
-  seen = set()
   for ba in bound_args:
-    if ba in seen:
-      continue
-    seen.add(ba)
-    if not ignore_cache and ba.cached_autotuning_data is not None:
-      continue
-    results.append((ba, ba.autotune(autotuner=autotuner, cache_results=False)))
-  return AutotuningResult(op_lib.device_kind(), tuple(results))
+    try:
+      results.append((ba, ba.autotune(autotuner=autotuner, cache_results=False, timeout=timeout)))
+    except Exception:  # pylint: disable=broad-exception-caught
+      logging.getLogger(__name__).exception("Failed to autotune for op %s", ba.op)
+  return AutotuningResult(device_kind, tuple(results))
 
 
 def save_cache_file(ops_results: Sequence[tuple], path: str) -> None:

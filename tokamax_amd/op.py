@@ -91,6 +91,9 @@ class Op(abc.ABC):
 
   def __call__(self, *args, return_residuals: bool = False, **kwargs):
     ba = self.bind(*args, return_residuals=return_residuals, **kwargs)
+    recorder = OP_CALL_RECORDER.get()
+    if recorder is not None:
+      recorder.append(ba)
     tensors = ba.tensors
     for device in {t.device for t in tensors} or {default_device()}:
       if not self.supported_on(device):
@@ -219,6 +222,11 @@ def _fast_signature(v):
     raise _Unhashable from None
   return v
 # Stack of {op: {device_kind: {key: AutotuningData}}} overlays pushed by `AutotuningResult`.
+# While a list is installed here, every `Op.__call__` appends its bound arguments to it: how `autotune(f, *args)`
+# finds the ops a function runs. (The reference walks the function's lowered HLO for the payloads its ops leave
+# there, tokamax/_src/hlo_utils.py:263-286; eager calls leave the same record here.)
+OP_CALL_RECORDER: contextvars.ContextVar[list | None] = contextvars.ContextVar("OP_CALL_RECORDER", default=None)
+
 AUTOTUNING_CACHE_OVERLAY_STACK: contextvars.ContextVar[tuple] = contextvars.ContextVar(
     "AUTOTUNING_CACHE_OVERLAY_STACK", default=()
 )

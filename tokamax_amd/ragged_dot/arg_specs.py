@@ -52,16 +52,42 @@ SPEC_SHAPES = {
     "8x7b": (8, 8192, 14336, 4096, _BF16, _BF16, None, "mixtral", ("primary", "ci_tests")),
 }
 
-ARG_SPECS = (
-    _make_maxtext_spec("deepseek-v3", 256, m=131072, n=1024, k=7168, tags=("primary",)),
-    _make_maxtext_spec("deepseek-v3", 256, m=131072, n=7168, k=1024, tags=("primary",)),
-    _make_maxtext_spec("deepseek-v3", 256, m=131072, n=512, k=7168, tags=("primary",)),
-    _make_maxtext_spec("deepseek-v3", 256, m=131072, n=7168, k=512, tags=("primary",)),
-    _make_maxtext_spec("deepseek-v3", 256, m=262144, n=2048, k=7168, tags=("primary",)),
-    _make_maxtext_spec("gpt-oss", 128, m=131072, n=768, k=2048),
-    _make_maxtext_spec("gpt-oss", 128, m=131072, n=1536, k=4096),
-    _make_maxtext_spec("gpt-oss", 256, m=65536, n=2048, k=7168),
-    _make_maxtext_spec("gpt-oss", 256, m=131072, n=2048, k=7168),
+# (project prefix, groups, m, n, k[, tags]) of the MaxText shapes, arg_specs.py:91-155.
+_MAXTEXT_SHAPES = (
+    ("deepseek-v3", 256, 131072, 1024, 7168, ("primary",)),
+    ("deepseek-v3", 256, 131072, 7168, 1024, ("primary",)),
+    ("deepseek-v3", 256, 131072, 512, 7168, ("primary",)),
+    ("deepseek-v3", 256, 131072, 7168, 512, ("primary",)),
+    ("deepseek-v3", 256, 262144, 512, 7168, ("primary",)),
+    ("deepseek-v3", 256, 262144, 7168, 256, ("primary",)),
+    ("deepseek-v3", 256, 262144, 7168, 1024, ("primary",)),
+    ("deepseek-v3", 256, 262144, 1024, 7168, ("primary",)),
+    ("deepseek-v3", 256, 262144, 2048, 7168, ("primary",)),
+    ("gpt-oss", 128, 327680, 2880, 2880, ()),
+    ("gpt-oss", 128, 393216, 768, 2048, ()),
+    ("gpt-oss", 128, 393216, 2048, 768, ()),
+    ("gpt-oss", 128, 524288, 1536, 4096, ()),
+    ("gpt-oss", 128, 524288, 4096, 1536, ()),
+    ("gpt-oss", 256, 524288, 2048, 7168, ()),
+    ("gpt-oss", 128, 262144, 1536, 4096, ()),
+    ("gpt-oss", 128, 262144, 4096, 1536, ()),
+    ("gpt-oss", 128, 131072, 2048, 7168, ()),
+    ("gpt-oss", 128, 131072, 768, 2048, ()),
+    ("gpt-oss", 128, 131072, 1536, 4096, ()),
+    ("gpt-oss", 128, 131072, 4096, 1536, ()),
+    ("gpt-oss", 256, 131072, 2048, 7168, ()),
+    ("gpt-oss", 256, 65536, 2048, 7168, ()),
+    ("gpt-oss", 256, 131072, 512, 7168, ()),
+    ("gpt-oss", 256, 131072, 7168, 512, ()),
+    ("gpt-oss", 256, 262144, 7168, 512, ()),
+    ("gpt-oss", 256, 262144, 512, 7168, ()),
+    ("gpt-oss", 256, 262144, 7168, 256, ()),
+    ("gpt-oss", 256, 262144, 7168, 1024, ()),
+    ("gpt-oss", 256, 262144, 1024, 7168, ()),
+)
+
+ARG_SPECS = tuple(
+    _make_maxtext_spec(prefix, groups, m=m, n=n, k=k, tags=tags) for prefix, groups, m, n, k, tags in _MAXTEXT_SHAPES
 ) + tuple(_make_spec(name, *args) for name, args in SPEC_SHAPES.items())
 
 
@@ -71,3 +97,22 @@ def flops(lhs, rhs, *, group_sizes) -> int:
   _, k, n = rhs.shape
   gs = group_sizes.representative_value if isinstance(group_sizes, base.GroupSizes) else group_sizes
   return 2 * int(sum(int(x) for x in gs)) * int(k) * int(n)
+
+
+def random_initialize(spec_args: dict, device, seed: int = 0) -> dict:
+  """Concrete arguments for an arg spec, as the reference's benchmarks and `test_bench` make them
+  (tokamax/_src/numerics.py:179-264 and base.py:99-106): abstract arrays become standard-normal values cast to their
+  type, drawn on the device; a `GroupSizes` spec becomes its representative sizes (an int32 device tensor)."""
+  gen = torch.Generator(device=device)
+  gen.manual_seed(seed)
+  out = {}
+  for name, x in spec_args.items():
+    if isinstance(x, base.GroupSizes):
+      out[name] = torch.tensor(x.representative_value, dtype=torch.int32, device=device)
+    elif isinstance(x, ShapeDtype):
+      t = torch.empty(tuple(x.shape), dtype=torch.float32 if x.dtype == torch.float32 else torch.bfloat16, device=device)
+      t.normal_(0.0, 1.0, generator=gen)
+      out[name] = t.to(x.dtype)
+    else:
+      out[name] = x
+  return out
