@@ -21,6 +21,8 @@
  *                               base.py:448-461; kernel counterpart pallas_mosaic_gpu_kernel_sm90.py:184-285
  *   tkx_dequantize_weights,     quantization.py:80-83 (as_array: qvalue * scale with tile-repeat
  *   tkx_dequantize              broadcasting) for int8 / fp8 operands with sub-channel scales
+ *   tkx_dequantize_zero_point   quantization.py:85-93 (operands with a zero point are dequantised first)
+ *   tkx_quantize                quantization.py:65-78 (AsQArray.as_qarray: absmax quantisation on the fly)
  *   TkxConfig                   pallas_mosaic_gpu_common.py:45-73 (Config)
  */
 #ifndef TKX_RAGGED_DOT_H_
@@ -191,6 +193,27 @@ int32_t tkx_dequantize_weights(const void* qvalue, const float* scale, void* out
 int32_t tkx_dequantize(const void* qvalue, const float* scale, void* out, int64_t rows, int64_t cols,
                        int64_t scale_block_rows, int64_t scale_block_cols, int32_t q_dtype, int32_t out_dtype,
                        tkx_stream_t stream);
+
+/* tkx_dequantize with a zero point (quantization.py:85-93 dequantises such operands before the kernels, which take
+ * none): out[r, c] = (qvalue[r, c] - zero_point[R, C]) * scale[R, C], zero_point f32 shaped like the scale. */
+int32_t tkx_dequantize_zero_point(const void* qvalue, const float* scale, const float* zero_point, void* out, int64_t rows,
+                                  int64_t cols, int64_t scale_block_rows, int64_t scale_block_cols, int32_t q_dtype,
+                                  int32_t out_dtype, tkx_stream_t stream);
+
+/* Quantisation on the fly (AsQArray.as_qarray, quantization.py:65-78: qwix.quantize with the "absmax" calibration), the
+ * inverse of tkx_dequantize:
+ *   scale[R, C] = max |x[r, c]| over the tile (R, C) / qmax   (1 where the tile is all zero)
+ *   qvalue[r, c] = convert(x[r, c] / scale[r / scale_block_rows, c / scale_block_cols])
+ * `qmax`: the largest quantised magnitude, at most 127 (int8) or 448 (fp8 e4m3fn); 0 means that maximum (7 gives int4
+ * values in int8 storage). convert rounds to nearest even and saturates at +-qmax (the form the reference gives the
+ * same calibration in pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:802-822).
+ * x f32, bf16 or f16 [rows, cols] row-major; qvalue int8 or fp8 [rows, cols]; scale f32
+ * [rows / scale_block_rows, cols / scale_block_cols]. Tiles: one row tall and a multiple of 8 columns wide (an lhs with
+ * one scale per row, scale_block_cols = cols, or per (row, k-block)); or several rows tall and 1, 8, 16, ... or 256
+ * columns wide (weights [g, k, n] as g * k rows: (k, 1) is one scale per (group, column), (t_k, 1) the scale tile
+ * (1, t_k, 1), (128, 128) square blocks). cols % 8 == 0. */
+int32_t tkx_quantize(const void* x, void* qvalue, float* scale, int64_t rows, int64_t cols, int64_t scale_block_rows,
+                     int64_t scale_block_cols, int32_t x_dtype, int32_t q_dtype, float qmax, tkx_stream_t stream);
 
 /* The token permute / un-permute steps either side of the ragged dot in an MoE layer, one kernel:
  *   out[j, :] = sum over r < reduce_group_size of keep(g) * weights[g] * x[indices[g], :],  g = j * reduce_group_size + r

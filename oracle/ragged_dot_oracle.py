@@ -47,8 +47,18 @@ below therefore cites the reference call site it follows, and says what pins it:
   ragged_gather / _scatter /   ragged_gather/base.py:25-32, ragged_scatter/        NumPy fancy indexing (library
     _gather_reduce             base.py:26-38, ragged_gather_reduce/base.py:26-40    routine) + loops on a tiny case
 
-Status of "parity unpinned": `qwix.quantize` (absmax calibration / rounding) is
-NOT restated -- quantised inputs are generated directly as (qvalue, scale) pairs.
+  quantize_absmax              quantization.py:65-78 (the call of qwix.quantize)  the reference's own statement of the
+                               pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:802-   calibration (absmax / qmax, clip) for
+                               822 (the same calibration, in the tree)            fp8; max |q| == qmax per tile; error
+                                                                                  <= scale / 2; exact powers of two;
+                                                                                  torch's float8_e4m3fn cast; zero tile
+  dequantize_zero_point        quantization.py:85-93                              hand-computed values
+
+Status of "parity unpinned": `qwix.quantize` itself (qwix>=0.1.2, pyproject.toml:27) is not in the tree.
+`quantize_absmax` follows the form of its absmax calibration that the reference writes out for fp8; for the integer
+types the bound qwix divides by (127 against 127.5 for int8) is NOT fixed by anything in the tree: parity unpinned.
+Quantising and dequantising with one and the same rule, as every test of the reference does
+(test_base.py:36-62, :187-242), keeps that choice out of the results compared.
 "gelu" in the gate-up forms is `jax.nn.gelu(gate)` (gmm_v2.py:99-100); JAX is not
 in the tree, and its documented default (`approximate=True`, the tanh form) is
 taken. Everything else above has a pin listed.
@@ -202,6 +212,48 @@ def dequantize(qvalue, scale) -> np.ndarray:
     assert q.shape[ax] % s.shape[ax] == 0, (q.shape, s.shape)
     s = np.repeat(s, q.shape[ax] // s.shape[ax], axis=ax)
   return q * s
+
+
+def dequantize_zero_point(qvalue, scale, zero_point) -> np.ndarray:
+  """`(qvalue - zero_point) * scale`, scale and zero point repeated over their tiles: the asymmetric form of
+  `qwix.dequantize` that quantization.py:85-93 applies before any kernel sees the operand."""
+  q = np.asarray(qvalue, np.float32)
+  s, z = np.asarray(scale, np.float32), np.asarray(zero_point, np.float32)
+  assert q.ndim == s.ndim and s.shape == z.shape, (q.shape, s.shape, z.shape)
+  for ax in range(q.ndim):
+    rep = q.shape[ax] // s.shape[ax]
+    s, z = np.repeat(s, rep, axis=ax), np.repeat(z, rep, axis=ax)
+  return (q - z) * s
+
+
+QMAX = {"int8": 127.0, "int4": 7.0, "fp8": 448.0}
+
+
+def quantize_absmax(x, qtype: str, tile_shape):
+  """Symmetric absmax quantisation with one f32 scale per tile: what `AsQArray.as_qarray` asks of
+  `qwix.quantize(x, qtype, tiled_axes=dict(enumerate(tile_shape)))` (quantization.py:65-78), stated the way the
+  reference states the same calibration itself (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:802-822):
+    scale = absmax(tile) / qmax, 1 where the tile is all zero;  q = x / scale, rounded to nearest even, clipped to +-qmax
+  with qmax the largest finite value of the type (127, 7, 448). Returns (q, scale): q int8 for the integer types, the
+  uint8 e4m3fn codes for "fp8"; scale float32 of shape x.shape / tile_shape. All arithmetic in float32."""
+  x = np.asarray(x, np.float32)
+  qmax = np.float32(QMAX[qtype])
+  tile_shape = tuple(int(t) for t in tile_shape)
+  assert x.ndim == len(tile_shape) and all(d % t == 0 for d, t in zip(x.shape, tile_shape)), (x.shape, tile_shape)
+  split = []
+  for d, t in zip(x.shape, tile_shape):
+    split += [d // t, t]
+  tiles = x.reshape(split)
+  inner = tuple(range(1, 2 * x.ndim, 2))
+  absmax = np.abs(tiles).max(axis=inner)
+  scale = np.where(absmax == 0, np.float32(1), absmax / qmax).astype(np.float32)
+  full = scale
+  for ax, t in enumerate(tile_shape):
+    full = np.repeat(full, t, axis=ax)
+  q = np.clip((x / full).astype(np.float32), -qmax, qmax)
+  if qtype == "fp8":
+    return e4m3fn_encode(q), scale
+  return np.rint(q).astype(np.int8), scale
 
 
 # ----------------------------------------------------------------------------

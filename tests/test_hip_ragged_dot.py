@@ -1239,3 +1239,125 @@ def test_autotune_of_a_function_on_device(device):
     _check(g, _np(w_), 2e-3)
   back = tokamax_amd.AutotuningResult.loads(res.dumps(), {"HipRaggedDot": OP})
   assert [d.fastest_config for _, d in back.data] == [d.fastest_config for _, d in res.data]
+
+
+# ---- quantisation on the fly (AsQArray), zero points, fp8 output -----------------------------------
+_QNAME = {torch.int8: "int8", torch.int4: "int4", torch.float8_e4m3fn: "fp8"}
+
+
+def _oracle_qarray(x, qtype, tile):
+  """`QArray` holding what the oracle's absmax quantisation makes of `x`."""
+  q, s = O.quantize_absmax(_np(x), _QNAME[qtype], tile)
+  qv = torch.tensor(q, device=x.device)
+  if qtype == torch.float8_e4m3fn:
+    qv = qv.view(torch.float8_e4m3fn)
+  return tokamax_amd.QArray(qv, torch.tensor(s, device=x.device), None, qtype)
+
+
+def _dequantized(q):
+  vals = q.qvalue.view(torch.uint8).cpu().numpy() if q.qvalue.dtype == torch.float8_e4m3fn else q.qvalue.cpu().numpy()
+  vals = O.e4m3fn_decode(vals) if q.qvalue.dtype == torch.float8_e4m3fn else vals
+  return O.dequantize(vals, _np(q.scale))
+
+
+@pytest.mark.parametrize("xdtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("qtype", [torch.int8, torch.int4, torch.float8_e4m3fn])
+@pytest.mark.parametrize("shape,tile", [((96, 256), (1, 128)), ((96, 256), (1, 16)), ((96, 256), (1, 256)), ((300, 4096), (1, 4096)),
+                                        ((512, 256), (256, 1)), ((512, 256), (16, 1)), ((256, 384), (128, 128)),
+                                        ((8, 256, 512), (1, 256, 1)), ((8, 256, 512), (1, 16, 1)), ((8, 256, 512), (1, 1, 16)),
+                                        ((3, 128, 264), (1, 128, 8)), ((40, 2880), (1, 2880)), ((64, 8), (1, 8))])
+def test_quantize_kernel_bit_exact(shape, tile, qtype, xdtype, device):
+  """`tkx_quantize` against the oracle's absmax quantisation: the same values and the same scales, bit for bit, for the
+  tile shapes of the reference's quantised tests (test_base.py:187-192) and a few more; an all-zero tile included."""
+  rng = np.random.default_rng(sum(shape) * 3 + sum(tile))
+  x = rng.normal(0, 0.1, shape).astype(np.float32)
+  x[tuple(slice(0, t) for t in tile)] = 0.0  # the first tile is all zero: scale 1, values 0
+  xt = torch.tensor(x, device=device).to(xdtype)
+  qv, scale = hip_ops.quantize(xt, qtype, tile)
+  want_q, want_s = O.quantize_absmax(_np(xt), _QNAME[qtype], tile)
+  assert scale.dtype == torch.float32 and tuple(scale.shape) == want_s.shape
+  assert np.array_equal(scale.cpu().numpy(), want_s)
+  got_q = qv.view(torch.uint8).cpu().numpy() if qtype == torch.float8_e4m3fn else qv.cpu().numpy()
+  assert np.array_equal(got_q, want_q)
+  as_q = tokamax_amd.AsQArray(xt, qtype, tiled_axes=dict(enumerate(tile))).as_qarray()
+  assert torch.equal(as_q.scale, scale) and as_q.qtype == qtype and as_q.zero_point is None
+  assert torch.equal(as_q.qvalue.view(torch.uint8), qv.view(torch.uint8))
+
+
+@pytest.mark.parametrize("activation", [None, torch.relu, torch.tanh])
+@pytest.mark.parametrize("use_as_qarray", [True, False])
+@pytest.mark.parametrize("b_tile_shape", [(1, 1, 16), (1, 1, 128), (1, 256, 1), (1, 16, 1)])
+@pytest.mark.parametrize("a_tile_shape", [None, (1, 128), (1, 16), (256, 1), (16, 1)])
+@pytest.mark.parametrize("qtype", [torch.int8, torch.int4])
+def test_quantized(qtype, a_tile_shape, b_tile_shape, use_as_qarray, activation, device):
+  """The reference's `test_quantized` (test_base.py:187-242), parametrised as there: both operands quantised with the
+  given tile shapes, handed over as `AsQArray` (quantised on the fly) or as `QArray`; the expected value contracts
+  the dequantised operands in f32; atol 0.01, rtol 0.005 on the first sum(group_sizes) rows."""
+  G, m, k, n = 8, 512, 256, 512
+  a, b, gs = _inputs("test_quantized", G, m, k, n, torch.bfloat16, device, random_groups=True)
+  if use_as_qarray:
+    wrap = lambda x, t: tokamax_amd.AsQArray(x, qtype, tiled_axes=dict(enumerate(t)))
+  else:
+    wrap = lambda x, t: _oracle_qarray(x, qtype, t)
+  a_in = a if a_tile_shape is None else wrap(a, a_tile_shape)
+  b_in = wrap(b, b_tile_shape)
+  a_f = _np(a) if a_tile_shape is None else _dequantized(_oracle_qarray(a, qtype, a_tile_shape))
+  b_f = _dequantized(_oracle_qarray(b, qtype, b_tile_shape))
+  want = O.ragged_dot(a_f, b_f, gs, acc_dtype=np.float32, out_dtype="f32")
+  if activation is not None:
+    want = activation(torch.tensor(want)).numpy()
+  got = OP(a_in, b_in, group_sizes=torch.tensor(gs, device=device), activation=activation)
+  count = int(gs.sum())
+  np.testing.assert_allclose(_np(got)[:count], want[:count], atol=0.01, rtol=0.005)
+
+
+@pytest.mark.parametrize("side", ["rhs", "lhs", "both"])
+def test_operands_with_a_zero_point(side, device):
+  """Quantised operands that carry a zero point are dequantised first, `(q - zero_point) * scale`
+  (quantization.py:85-93), and then take the bf16 kernels."""
+  rng = np.random.default_rng(31)
+  G, m, k, n = 4, 200, 128, 256
+  gs = np.array([60, 0, 90, 40], np.int32)
+  mk = lambda shape, std: torch.tensor(rng.normal(0, std, shape).astype(np.float32), device=device)
+  lhs, rhs = mk((m, k), 1.0).to(torch.bfloat16), mk((G, k, n), k ** -0.5).to(torch.bfloat16)
+  lhs_f, rhs_f = _np(lhs), _np(rhs)
+  if side in ("rhs", "both"):
+    q = torch.tensor(rng.integers(-128, 128, (G, k, n)).astype(np.int8), device=device)
+    scale, zp = mk((G, 4, n), 0.01).abs() + 1e-3, torch.tensor(rng.integers(-20, 20, (G, 4, n)).astype(np.float32), device=device)
+    rhs = tokamax_amd.QArray(q, scale, zp)
+    rhs_f = O.round_to_bf16(O.dequantize_zero_point(q.cpu().numpy(), _np(scale), _np(zp)))
+  if side in ("lhs", "both"):
+    q = torch.tensor(rng.integers(-128, 128, (m, k)).astype(np.int8), device=device)
+    scale, zp = mk((m, 1), 0.02).abs() + 1e-3, torch.tensor(rng.integers(-9, 9, (m, 1)).astype(np.float32), device=device)
+    lhs = tokamax_amd.QArray(q, scale, zp)
+    lhs_f = O.round_to_bf16(O.dequantize_zero_point(q.cpu().numpy(), _np(scale), _np(zp)))
+  got = OP(lhs, rhs, group_sizes=torch.tensor(gs, device=device), preferred_element_type=torch.float32)
+  _check(got, O.ragged_dot(lhs_f, rhs_f, gs, acc_dtype=np.float64, out_dtype="f64"), 1e-5)
+  assert torch.count_nonzero(got[int(gs.sum()):]) == 0
+
+
+@pytest.mark.parametrize("activation", [None, torch.relu, torch.nn.functional.silu])
+def test_fp8_output_quantisation(activation, device):
+  """`enable_fused_epilogue_quant` with an fp8 `preferred_element_type` returns the result quantised per (row, 128
+  columns) as a QArray (pallas_mosaic_gpu_common.py:63-68; test of pallas_mosaic_gpu_kernel_sm100_fp8_quant_test.py:
+  237-279: dequantised result within atol 0.06, rtol 0.1 of the reference, second run bit-identical). Without the
+  switch the fp8 request is widened to the weights' type (pallas_mosaic_gpu.py:197-205)."""
+  G, m, k, n = 8, 512, 256, 512
+  a, b, gs = _inputs("test_epilogue_quant", G, m, k, n, torch.bfloat16, device, random_groups=True)
+  gst = torch.tensor(gs, device=device)
+  op_q = hip.HipRaggedDot(enable_fused_epilogue_quant=True)
+  out = op_q(a, b, group_sizes=gst, preferred_element_type=torch.float8_e4m3fn, activation=activation)
+  assert isinstance(out, tokamax_amd.QArray) and out.qvalue.dtype == torch.float8_e4m3fn
+  assert tuple(out.qvalue.shape) == (m, n) and tuple(out.scale.shape) == (m, n // 128)
+  want = O.ragged_dot(_np(a), _np(b), gs, acc_dtype=np.float32, out_dtype="f32")
+  if activation is not None:
+    want = activation(torch.tensor(want)).numpy()
+  count = int(gs.sum())
+  np.testing.assert_allclose(_dequantized(out)[:count], want[:count], atol=0.06, rtol=0.1)
+  # exactly the absmax quantisation of the f32 result of the same call
+  dense = OP(a, b, group_sizes=gst, preferred_element_type=torch.float32, activation=activation)
+  q, s = O.quantize_absmax(_np(dense), "fp8", (1, 128))
+  assert np.array_equal(out.qvalue.view(torch.uint8).cpu().numpy(), q) and np.array_equal(_np(out.scale), s)
+  again = op_q(a, b, group_sizes=gst, preferred_element_type=torch.float8_e4m3fn, activation=activation)
+  assert torch.equal(again.qvalue.view(torch.uint8), out.qvalue.view(torch.uint8)) and torch.equal(again.scale, out.scale)
+  assert OP(a, b, group_sizes=gst, preferred_element_type=torch.float8_e4m3fn).dtype == torch.bfloat16

@@ -399,3 +399,66 @@ def test_golden_fixtures_match_oracle():
   np.testing.assert_allclose(f(z["lhs"], O.dequantize(z["q8"], z["q8_scale"]), gs), z["fwd_q8"], rtol=1e-12, atol=1e-12)
   # the brute-force loops agree with the stored vectors too (small enough to run here)
   np.testing.assert_allclose(O.ragged_dot_bruteforce(z["lhs"][:40], z["rhs"], [23, 0, 17, 0]), z["fwd"][:40], rtol=1e-10, atol=1e-10)
+
+
+# ---- absmax quantisation (AsQArray.as_qarray) -----------------------------------------------------
+@pytest.mark.parametrize("qtype", ["int8", "int4", "fp8"])
+@pytest.mark.parametrize("shape,tile", [((6, 32), (1, 8)), ((6, 32), (1, 32)), ((8, 16), (4, 1)), ((8, 16), (8, 8)),
+                                        ((2, 8, 16), (1, 8, 1)), ((2, 8, 16), (1, 4, 8))])
+def test_quantize_absmax_properties(qtype, shape, tile):
+  """What the definition fixes: the largest entry of every tile maps to +-qmax, no entry lies further than half a
+  quantisation step from its dequantised value, an all-zero tile gets scale 1, scale shapes are shape / tile."""
+  rng = np.random.default_rng(sum(shape) + sum(tile))
+  x = rng.normal(0, 3, shape).astype(np.float32)
+  x[(0,) * len(shape)] = 0.0
+  q, scale = O.quantize_absmax(x, qtype, tile)
+  qmax = O.QMAX[qtype]
+  assert scale.shape == tuple(d // t for d, t in zip(shape, tile)) and scale.dtype == np.float32
+  qf = O.e4m3fn_decode(q) if qtype == "fp8" else q.astype(np.float32)
+  split = []
+  for d, t in zip(shape, tile):
+    split += [d // t, t]
+  inner = tuple(range(1, 2 * len(shape), 2))
+  assert np.all(np.abs(qf).reshape(split).max(axis=inner) == qmax)
+  absmax = np.abs(x).reshape(split).max(axis=inner)
+  np.testing.assert_allclose(scale, absmax / np.float32(qmax), rtol=1e-6)
+  back = O.dequantize(qf, scale)
+  full = O.dequantize(np.ones(shape, np.float32), scale)
+  if qtype == "fp8":  # e4m3: 3 mantissa bits -> relative step 2^-3, half of it plus the subnormal floor
+    assert np.all(np.abs(back - x) <= np.maximum(np.abs(x) * 2.0 ** -4, full * 2.0 ** -10) * 1.0001)
+  else:
+    assert np.all(np.abs(back - x) <= full * 0.5 * 1.0001)
+  z, zs = O.quantize_absmax(np.zeros(shape, np.float32), qtype, tile)
+  assert np.all(zs == 1) and np.all(z == 0)
+
+
+def test_quantize_absmax_exact_cases():
+  # powers of two: absmax = 127 / 4 -> scale = 1/4 exactly, every multiple of 1/4 is its own code
+  x = np.array([[31.75, -0.25, 0.5, 10.0, -31.75, 0.0, 1.25, -7.5]], np.float32)
+  q, s = O.quantize_absmax(x, "int8", (1, 8))
+  assert s[0, 0] == 0.25 and q.tolist() == [[127, -1, 2, 40, -127, 0, 5, -30]]
+  # ties go to the even code: with scale 1, x.5 rounds to the even neighbour
+  x = np.array([[127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.49]], np.float32)
+  q, s = O.quantize_absmax(x, "int8", (1, 8))
+  assert s[0, 0] == 1.0 and q.tolist() == [[127, 0, 2, 2, 0, -2, -2, 3]]
+  # int4: qmax 7
+  q, s = O.quantize_absmax(np.array([[3.5, -1.0, 0.24, 0.26]], np.float32), "int4", (1, 4))
+  assert s[0, 0] == 0.5 and q.tolist() == [[7, -2, 0, 1]]
+  # fp8: x / scale rounded the way torch casts to float8_e4m3fn (library routine), for every tile
+  rng = np.random.default_rng(1)
+  x = rng.normal(0, 1, (16, 64)).astype(np.float32)
+  q, s = O.quantize_absmax(x, "fp8", (1, 16))
+  want = (torch.tensor(x) / torch.tensor(np.repeat(s, 16, axis=1))).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+  assert np.array_equal(q, want)
+  # the per-column form: a tile (k, 1) of weights [k, n] gives one scale per column
+  w = rng.normal(0, 1, (8, 4)).astype(np.float32)
+  q, s = O.quantize_absmax(w, "int8", (8, 1))
+  assert s.shape == (1, 4) and np.allclose(s[0], np.abs(w).max(axis=0) / 127)
+  for c in range(4):
+    assert np.array_equal(q[:, c], np.rint(w[:, c] / s[0, c]).astype(np.int8))
+
+
+def test_dequantize_zero_point_by_hand():
+  q = np.array([[10, -3, 0, 7]], np.int8)
+  got = O.dequantize_zero_point(q, np.array([[0.5, 2.0]], np.float32), np.array([[2.0, -1.0]], np.float32))
+  assert got.tolist() == [[4.0, -2.5, 2.0, 16.0]]  # (10 - 2) / 2, (-3 - 2) / 2, (0 + 1) * 2, (7 + 1) * 2

@@ -33,6 +33,8 @@ EXPORTED_SYMBOLS = (
     "tkx_ragged_dot_drhs",
     "tkx_dequantize_weights",
     "tkx_dequantize",
+    "tkx_dequantize_zero_point",
+    "tkx_quantize",
     "tkx_ragged_gather_rows",
     "tkx_ragged_dot_num_variants",
     "tkx_ragged_dot_variant",
@@ -88,6 +90,10 @@ def _declare(lib):
   lib.tkx_dequantize_weights.argtypes = [vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
   lib.tkx_dequantize.restype = i32
   lib.tkx_dequantize.argtypes = [vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
+  lib.tkx_dequantize_zero_point.restype = i32
+  lib.tkx_dequantize_zero_point.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
+  lib.tkx_quantize.restype = i32
+  lib.tkx_quantize.argtypes = [vp, vp, vp, i64, i64, i64, i64, i32, i32, ctypes.c_float, vp]
   lib.tkx_ragged_gather_rows.restype = i32
   lib.tkx_ragged_gather_rows.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]
   lib.tkx_ragged_dot_num_variants.restype = i32

@@ -444,8 +444,66 @@ int32_t tkx_dequantize(const void* qvalue, const float* scale, void* out, int64_
   if (scale_block_rows > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "scale block too tall");
   if (((uintptr_t)qvalue | (uintptr_t)out) % 16 != 0 || (uintptr_t)scale % (scale_block_cols == 1 ? 16 : 4) != 0)
     return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
-  return launch_dequant(qvalue, scale, out, rows, cols, scale_block_rows, scale_block_cols, q_dtype,
+  return launch_dequant(qvalue, scale, nullptr, out, rows, cols, scale_block_rows, scale_block_cols, q_dtype,
                         static_cast<hipStream_t>(stream));
+}
+
+int32_t tkx_dequantize_zero_point(const void* qvalue, const float* scale, const float* zero_point, void* out, int64_t rows,
+                                  int64_t cols, int64_t scale_block_rows, int64_t scale_block_cols, int32_t q_dtype,
+                                  int32_t out_dtype, tkx_stream_t stream) {
+  if (!zero_point) return set_error(TKX_ERR_INVALID, "null pointer argument");
+  // (the checks of tkx_dequantize, which launches nothing when one fails)
+  if (!qvalue || !scale || !out) return set_error(TKX_ERR_INVALID, "null pointer argument");
+  if (rows < 1 || cols < 1 || scale_block_rows < 1 || scale_block_cols < 1)
+    return set_error(TKX_ERR_INVALID, "bad sizes rows=%lld cols=%lld block=%lldx%lld", (long long)rows, (long long)cols,
+                     (long long)scale_block_rows, (long long)scale_block_cols);
+  if ((q_dtype != TKX_I8 && q_dtype != TKX_F8E4M3FN) || out_dtype != TKX_BF16)
+    return set_error(TKX_ERR_UNSUPPORTED, "dequantisation is int8 or fp8 -> bf16 only (got %d -> %d)", q_dtype, out_dtype);
+  if (rows % scale_block_rows != 0 || cols % scale_block_cols != 0)
+    return set_error(TKX_ERR_INVALID, "scale blocks %lldx%lld do not tile %lldx%lld", (long long)scale_block_rows,
+                     (long long)scale_block_cols, (long long)rows, (long long)cols);
+  if (cols % 16 != 0 || cols > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "cols must be a multiple of 16");
+  if (scale_block_cols != 1 && scale_block_cols % 16 != 0)
+    return set_error(TKX_ERR_UNSUPPORTED, "scale blocks along the columns must be 1 or a multiple of 16 wide");
+  if (scale_block_rows > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "scale block too tall");
+  const uintptr_t table_align = scale_block_cols == 1 ? 16 : 4;
+  if (((uintptr_t)qvalue | (uintptr_t)out) % 16 != 0 || (uintptr_t)scale % table_align != 0 || (uintptr_t)zero_point % table_align != 0)
+    return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
+  return launch_dequant(qvalue, scale, zero_point, out, rows, cols, scale_block_rows, scale_block_cols, q_dtype,
+                        static_cast<hipStream_t>(stream));
+}
+
+int32_t tkx_quantize(const void* x, void* qvalue, float* scale, int64_t rows, int64_t cols, int64_t scale_block_rows,
+                     int64_t scale_block_cols, int32_t x_dtype, int32_t q_dtype, float qmax, tkx_stream_t stream) {
+  if (!x || !qvalue || !scale) return set_error(TKX_ERR_INVALID, "null pointer argument");
+  if (rows < 1 || cols < 1 || scale_block_rows < 1 || scale_block_cols < 1)
+    return set_error(TKX_ERR_INVALID, "bad sizes rows=%lld cols=%lld block=%lldx%lld", (long long)rows, (long long)cols,
+                     (long long)scale_block_rows, (long long)scale_block_cols);
+  if (x_dtype != TKX_F32 && x_dtype != TKX_BF16 && x_dtype != TKX_F16)
+    return set_error(TKX_ERR_UNSUPPORTED, "quantisation reads f32, bf16 or f16 (got %d)", x_dtype);
+  if (q_dtype != TKX_I8 && q_dtype != TKX_F8E4M3FN)
+    return set_error(TKX_ERR_UNSUPPORTED, "quantisation writes int8 or fp8 e4m3fn (got %d)", q_dtype);
+  if (rows % scale_block_rows != 0 || cols % scale_block_cols != 0)
+    return set_error(TKX_ERR_INVALID, "scale blocks %lldx%lld do not tile %lldx%lld", (long long)scale_block_rows,
+                     (long long)scale_block_cols, (long long)rows, (long long)cols);
+  if (cols % 8 != 0 || cols > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "cols must be a multiple of 8");
+  const bool pow2 = (scale_block_cols & (scale_block_cols - 1)) == 0;
+  if (scale_block_rows == 1) {
+    if (scale_block_cols % 8 != 0) return set_error(TKX_ERR_UNSUPPORTED, "tiles one row tall must be a multiple of 8 columns wide");
+  } else {
+    if (scale_block_rows > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "scale block too tall");
+    if (scale_block_cols != 1 && !(pow2 && scale_block_cols >= 8 && scale_block_cols <= 256))
+      return set_error(TKX_ERR_UNSUPPORTED, "tiles several rows tall must be 1, 8, 16, ... or 256 columns wide (got %lld)",
+                       (long long)scale_block_cols);
+    if (scale_block_cols == 1 && cols % 4 != 0) return set_error(TKX_ERR_UNSUPPORTED, "cols must be a multiple of 4");
+  }
+  if ((uintptr_t)x % 16 != 0 || (uintptr_t)qvalue % 8 != 0 || (uintptr_t)scale % 16 != 0)
+    return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
+  const float type_max = q_dtype == TKX_I8 ? 127.f : 448.f;
+  if (qmax == 0.f) qmax = type_max;
+  if (!(qmax > 0.f) || qmax > type_max) return set_error(TKX_ERR_INVALID, "qmax must lie in (0, %g]", (double)type_max);
+  return launch_quantize(x, qvalue, scale, rows, cols, scale_block_rows, scale_block_cols, x_dtype, q_dtype, qmax,
+                         static_cast<hipStream_t>(stream));
 }
 
 int32_t tkx_ragged_gather_rows(const void* x, const int32_t* indices, const float* weights, const uint8_t* valid,

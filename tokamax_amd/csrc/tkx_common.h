@@ -114,8 +114,14 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
 
 // ---- dequantisation of int8 weights with sub-channel scales to bf16 ------------------------------
 // out[r, c] = q[r, c] * scale[r / t_r, c / t_c]; q int8 or fp8 (e4m3fn), out bf16; t_c is 1 or a multiple of 16.
-int32_t launch_dequant(const void* q, const float* scale, void* out, int64_t rows, int64_t n, int64_t t_r, int64_t t_c,
-                       int32_t q_dtype, hipStream_t stream);
+// `zero_point` (f32, shaped like the scale, or null): out = (q - zero_point) * scale.
+int32_t launch_dequant(const void* q, const float* scale, const float* zero_point, void* out, int64_t rows, int64_t n,
+                       int64_t t_r, int64_t t_c, int32_t q_dtype, hipStream_t stream);
+
+// ---- absmax quantisation to int8 / fp8 with block scales (the inverse pass) -------------------------
+// scale[R, C] = absmax of tile (R, C) / qmax (1 for an all-zero tile); q = convert(x / scale). x f32, bf16 or f16.
+int32_t launch_quantize(const void* x, void* q, float* scale, int64_t rows, int64_t cols, int64_t t_r, int64_t t_c,
+                        int32_t x_dtype, int32_t q_dtype, float qmax, hipStream_t stream);
 
 // ---- row gather with optional mask, weight and reduction (token permute / un-permute) -------------
 int32_t launch_gather_rows(const void* x, const int32_t* indices, const float* weights, const unsigned char* valid,

@@ -1,5 +1,5 @@
-// Dequantisation with block scales: out[r, c] = q[r, c] * scale[r / t_r, c / t_c], q int8 or fp8
-// (e4m3fn), out bf16.
+// Dequantisation with block scales: out[r, c] = (q[r, c] - zero_point[R, C]) * scale[R, C] with
+// (R, C) = (r / t_r, c / t_c), q int8 or fp8 (e4m3fn), out bf16; the zero point (f32, shaped like the scale) is optional.
 //
 // The tiled kernels apply one scale per lhs row and one per (group, column) in their epilogue, which
 // covers scales that span the whole contraction. Operands whose scales change along the contraction
@@ -25,9 +25,10 @@ __device__ __forceinline__ float widen_byte(int w) {
 // One thread converts 16 consecutive columns of one row: a 16-byte load, the scales of those columns
 // (four 16-byte loads when every column has its own, t_c == 1; one value when a scale block spans
 // them, t_c % 16 == 0; L2-resident either way: a scale row serves t_r rows), two 16-byte stores.
-template <int EQ>
+template <int EQ, bool ZP>
 __global__ __launch_bounds__(kDqThreads) void dequant_kernel(const unsigned char* __restrict__ q,
-                                                            const float* __restrict__ scale, __bf16* __restrict__ out,
+                                                            const float* __restrict__ scale,
+                                                            const float* __restrict__ zero_point, __bf16* __restrict__ out,
                                                             int64_t rows, int32_t n, int32_t t_r, int32_t t_c) {
   const int chunks = n / 16;  // n % 16 == 0 (checked on the host)
   const int64_t total = rows * chunks;
@@ -37,7 +38,7 @@ __global__ __launch_bounds__(kDqThreads) void dequant_kernel(const unsigned char
     const int c0 = (int)(idx - row * chunks) * 16;
     const i32x4 w = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(q + row * n + c0));
     const float* srow = scale + (row / t_r) * scale_cols;
-    f32x4 sc[4];
+    f32x4 sc[4], zp[4];
     if (t_c == 1) {
 #pragma unroll
       for (int d = 0; d < 4; ++d) sc[d] = *reinterpret_cast<const f32x4*>(srow + c0 + 4 * d);
@@ -46,12 +47,27 @@ __global__ __launch_bounds__(kDqThreads) void dequant_kernel(const unsigned char
 #pragma unroll
       for (int d = 0; d < 4; ++d) sc[d] = (f32x4){one, one, one, one};
     }
+    if constexpr (ZP) {
+      const float* zrow = zero_point + (row / t_r) * scale_cols;
+      if (t_c == 1) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) zp[d] = *reinterpret_cast<const f32x4*>(zrow + c0 + 4 * d);
+      } else {
+        const float one = zrow[c0 / t_c];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) zp[d] = (f32x4){one, one, one, one};
+      }
+    }
     bf16x8 lo, hi;
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       const int word = w[d];
-      const float v[4] = {widen_byte<EQ, 0>(word) * sc[d][0], widen_byte<EQ, 1>(word) * sc[d][1],
-                          widen_byte<EQ, 2>(word) * sc[d][2], widen_byte<EQ, 3>(word) * sc[d][3]};
+      float v[4] = {widen_byte<EQ, 0>(word), widen_byte<EQ, 1>(word), widen_byte<EQ, 2>(word), widen_byte<EQ, 3>(word)};
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        if constexpr (ZP) v[b] -= zp[d][b];
+        v[b] *= sc[d][b];
+      }
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         const int e = 4 * d + b;
@@ -67,19 +83,20 @@ __global__ __launch_bounds__(kDqThreads) void dequant_kernel(const unsigned char
 
 }  // namespace
 
-int32_t launch_dequant(const void* q, const float* scale, void* out, int64_t rows, int64_t n, int64_t t_r, int64_t t_c,
-                       int32_t q_dtype, hipStream_t stream) {
+int32_t launch_dequant(const void* q, const float* scale, const float* zero_point, void* out, int64_t rows, int64_t n,
+                       int64_t t_r, int64_t t_c, int32_t q_dtype, hipStream_t stream) {
   const int64_t total = rows * (n / 16);
   int64_t grid = (total + kDqThreads - 1) / kDqThreads;
   if (grid > 256 * 16) grid = 256 * 16;  // 16 workgroups per CU, grid-stride beyond that
   if (grid < 1) grid = 1;
   const auto* qb = static_cast<const unsigned char*>(q);
-  if (q_dtype == TKX_I8)
-    dequant_kernel<kEI8><<<dim3((unsigned)grid), dim3(kDqThreads), 0, stream>>>(qb, scale, static_cast<__bf16*>(out), rows,
-                                                                               (int32_t)n, (int32_t)t_r, (int32_t)t_c);
-  else
-    dequant_kernel<kEF8><<<dim3((unsigned)grid), dim3(kDqThreads), 0, stream>>>(qb, scale, static_cast<__bf16*>(out), rows,
-                                                                               (int32_t)n, (int32_t)t_r, (int32_t)t_c);
+  auto* ob = static_cast<__bf16*>(out);
+  const dim3 g((unsigned)grid), b(kDqThreads);
+  const int32_t n32 = (int32_t)n, tr = (int32_t)t_r, tc = (int32_t)t_c;
+  if (q_dtype == TKX_I8 && zero_point) dequant_kernel<kEI8, true><<<g, b, 0, stream>>>(qb, scale, zero_point, ob, rows, n32, tr, tc);
+  else if (q_dtype == TKX_I8) dequant_kernel<kEI8, false><<<g, b, 0, stream>>>(qb, scale, nullptr, ob, rows, n32, tr, tc);
+  else if (zero_point) dequant_kernel<kEF8, true><<<g, b, 0, stream>>>(qb, scale, zero_point, ob, rows, n32, tr, tc);
+  else dequant_kernel<kEF8, false><<<g, b, 0, stream>>>(qb, scale, nullptr, ob, rows, n32, tr, tc);
   TKX_HIP_CHECK(hipGetLastError());
   return TKX_OK;
 }

@@ -21,6 +21,7 @@ from tokamax_amd import _lib
 from tokamax_amd import config as config_lib
 from tokamax_amd import op
 from tokamax_amd import precision as precision_lib
+from tokamax_amd import quantization
 from tokamax_amd.serialization import ShapeDtype
 from tokamax_amd.ragged_dot import base
 from tokamax_amd.ragged_dot import hip_ops
@@ -148,6 +149,20 @@ def _lhs_scale_blocks(q: QArray) -> int | None:
   return shape[1]
 
 
+def _widening_pass_takes(q: QArray) -> bool:
+  """Whether `tkx_dequantize` takes this operand: the scale tiles the values, in blocks 1 or a multiple of 16 columns
+  wide (the last axis), over row-major values whose rows are a multiple of 16 entries."""
+  shape, sshape = tuple(q.qvalue.shape), tuple(q.scale.shape)
+  if len(shape) != len(sshape) or len(shape) not in (2, 3) or shape[-1] % 16:
+    return False
+  if any(s < 1 or d % s for d, s in zip(shape, sshape)):
+    return False
+  if len(shape) == 3 and sshape[0] != shape[0]:
+    return False
+  t_c = shape[-1] // sshape[-1]
+  return t_c == 1 or t_c % 16 == 0
+
+
 def _widening_plan(lhs, rhs, allow_native: bool = True) -> tuple[bool, bool, bool]:
   """(widen lhs, widen rhs, native k-blocks): how a pair of (possibly quantised) operands reaches the kernels.
 
@@ -164,15 +179,20 @@ def _widening_plan(lhs, rhs, allow_native: bool = True) -> tuple[bool, bool, boo
     was widened is widened too (there is no bf16 x fp8 kernel outside the native ones)."""
   lhs_q, rhs_q = isinstance(lhs, QArray), isinstance(rhs, QArray)
   widen_lhs = widen_rhs = False
-  blocks = None  # (scale blocks along k of a quantised rhs)
+  blocks = lhs_blocks = None  # (scale blocks along k of a quantised rhs / lhs)
   if lhs_q:
     lhs_blocks = _lhs_scale_blocks(lhs)
     if lhs_blocks is None:
-      raise NotImplementedError(f"lhs scale must have shape [m,1] or [m, k/t] with 16 | t, got {tuple(lhs.scale.shape)}")
-    widen_lhs = lhs_blocks > 1 or _dtype_of(lhs) == torch.int8  # (unless int8 meets int8 below)
+      # Any other tiling (row blocks, one scale per column, 2-d blocks) goes through the widening pass, as the
+      # reference's sm90 path dequantises a quantised lhs first (pallas_mosaic_gpu.py:152-154).
+      if not _widening_pass_takes(lhs):
+        raise NotImplementedError("lhs scale must tile lhs [m,k] in blocks 1 or a multiple of 16 columns wide, got"
+                                  f" {tuple(lhs.scale.shape)}")
+      lhs_blocks = 0
+    widen_lhs = lhs_blocks != 1 or _dtype_of(lhs) == torch.int8  # (unless int8 meets int8 below)
   if rhs_q:
     blocks = _scale_blocks_along_k(rhs)
-    if blocks is None and not _rhs_scale_tiles(rhs):
+    if blocks is None and not _rhs_scale_tiles(rhs) and not _widening_pass_takes(rhs):
       raise NotImplementedError("rhs scale must have shape [g,1,n], [g,k/t_k,n] or [g,k/t_k,n/t_n] with 16 | t_n, got"
                                 f" {tuple(rhs.scale.shape)}")
     widen_rhs = blocks is None or blocks > 1
@@ -181,7 +201,7 @@ def _widening_plan(lhs, rhs, allow_native: bool = True) -> tuple[bool, bool, boo
                and lhs.qvalue.dtype == torch.int8 and rhs.qvalue.dtype == torch.int8)
   both_fp8 = lhs_q and rhs_q and eight_bit_float(lhs) and eight_bit_float(rhs)
   if (allow_native and (both_fp8 or both_int8) and blocks is not None and (blocks > 1 or both_int8)
-      and _lhs_scale_blocks(lhs) == blocks):
+      and lhs_blocks == blocks):
     # The same k-blocks on both sides: the fp8 (int8) MFMA kernels that fold the scales in per k-block; int8 x int8
     # also with a single block (there is no other kernel that contracts int8 activations).
     m, k = lhs.qvalue.shape
@@ -249,11 +269,103 @@ def _is_gfx950(device: torch.device) -> bool:
 
 
 @dataclasses.dataclass(frozen=True)
+class _Route:
+  """How one call reaches the kernels; computed from shapes and types only, so that the forward pass (on arrays) and
+  the choice of a config (on abstract arguments) cannot disagree."""
+
+  mode: int          # variant-table mode: 0 forward, 1 dlhs, 2 drhs, 3 forward with gate-up fusion, 4 k-block scales
+  lhs: object        # operands in the form the plan was made for (shared scales repeated, raw rhs_scale folded in)
+  rhs: object
+  lhs_dtype: torch.dtype  # element types the kernel sees
+  rhs_dtype: torch.dtype
+  widen_lhs: bool    # the operand goes through the widening pass (tkx_dequantize) first
+  widen_rhs: bool
+  native_k_blocks: bool
+  cast_bf16: bool    # the BF16_BF16_F32 preset: both (unquantised) operands are cast to bf16
+  preferred_element_type: object
+
+  @property
+  def key(self):
+    return (self.mode, hip_ops.dtype_code(self.lhs_dtype), hip_ops.dtype_code(self.rhs_dtype))
+
+
+def _route(lhs, rhs, *, dims, precision, rhs_scale, fuse_gateup_activation, preferred_element_type) -> _Route:
+  """Plans a call. `lhs` / `rhs` are arrays, `QArray`s or their abstract forms (an `AsQArray` has been turned into the
+  `QArray` it quantises to, an operand with a zero point into the bf16 array it dequantises to)."""
+  mode = _MODE_OF_DIMS.get(dims)
+  if mode is None:
+    raise NotImplementedError("Unsupported ragged dot dimension numbers.")
+  if rhs_scale is not None:
+    # The raw-array form of quantised weights (experimental/gmm_v2/gmm_v2.py:1193-1199): rhs holds the quantised values
+    # and rhs_scale is [g, k-blocks, 1, n]; the result defaults to lhs.dtype (:1369-1370).
+    if isinstance(lhs, QArray) or isinstance(rhs, QArray):
+      raise NotImplementedError("rhs_scale comes with raw arrays, not QArrays.")
+    g, k, n = rhs.shape
+    if len(rhs_scale.shape) != 4 or tuple(rhs_scale.shape[::2]) != (g, 1) or rhs_scale.shape[3] != n:
+      raise NotImplementedError(f"rhs_scale must have shape [g, k-blocks, 1, n], got {tuple(rhs_scale.shape)}")
+    scale = (rhs_scale.reshape(g, rhs_scale.shape[1], n) if isinstance(rhs_scale, torch.Tensor)
+             else ShapeDtype((g, rhs_scale.shape[1], n), rhs_scale.dtype))
+    rhs = QArray(rhs, scale)
+    if preferred_element_type is None:
+      preferred_element_type = lhs.dtype
+  gateup = fuse_gateup_activation is not None
+  if (gateup or rhs_scale is not None) and mode != 0:
+    raise NotImplementedError("rhs_scale and fuse_gateup_activation need the default dimension numbers.")
+  lhs_dt, rhs_dt = _dtype_of(lhs), _dtype_of(rhs)
+  widen_lhs = widen_rhs = native = False
+  if mode == 0:
+    lhs, rhs = _per_row_lhs_scale(lhs), _per_column_rhs_scale(rhs)
+    widen_lhs, widen_rhs, native = _widening_plan(lhs, rhs, allow_native=not gateup)
+  else:
+    # dlhs / drhs contract unquantised operands (base.py:395-410 rejects quantised ones on the backward path); a
+    # quantised operand in a direct call is widened first, as pallas_mosaic_gpu.py:170 does for the drhs product.
+    for x in (lhs, rhs):
+      if isinstance(x, QArray) and not _widening_pass_takes(x):
+        raise NotImplementedError(f"cannot dequantise an operand with scale {tuple(x.scale.shape)} for this product")
+    widen_lhs, widen_rhs = isinstance(lhs, QArray), isinstance(rhs, QArray)
+  lhs_dt = torch.bfloat16 if widen_lhs else lhs_dt
+  rhs_dt = torch.bfloat16 if widen_rhs else rhs_dt
+  in_dtype = lhs.dtype if isinstance(lhs, QArray) else lhs_dt   # (a QArray's dtype: what it dequantises to)
+  w_dtype = rhs.dtype if isinstance(rhs, QArray) else rhs_dt
+  cast_bf16 = False
+  if not precision_lib.is_default(in_dtype, w_dtype, precision):
+    if (precision == precision_lib.DotAlgorithmPreset.BF16_BF16_F32 and not isinstance(lhs, QArray)
+        and not isinstance(rhs, QArray)):
+      cast_bf16 = True
+      lhs_dt = rhs_dt = torch.bfloat16
+    else:
+      raise NotImplementedError(f"{precision=} not supported.")
+  if preferred_element_type is None:
+    preferred_element_type = torch.promote_types(in_dtype, w_dtype)
+  if mode == 0:
+    mode = 3 if gateup else 4 if native else 0
+  return _Route(mode, lhs, rhs, lhs_dt, rhs_dt, widen_lhs, widen_rhs, native, cast_bf16, preferred_element_type)
+
+
+def _abstract_operand(x):
+  """The abstract form of what `_concrete_operand` returns."""
+  if isinstance(x, AsQArray):
+    return x.abstract_qarray()
+  if isinstance(x, QArray) and x.zero_point is not None:
+    return ShapeDtype(tuple(x.qvalue.shape), torch.bfloat16)
+  return x
+
+
+def _concrete_operand(x):
+  """An `AsQArray` quantised on the device; an operand with a zero point dequantised to bf16 (quantization.py:85-93:
+  none of the kernels takes a zero point)."""
+  return quantization.as_array_or_qarray_without_zero_point(x)
+
+
+@dataclasses.dataclass(frozen=True)
 class HipRaggedDot(base.RaggedDot):
   """Hand-written HIP ragged dot for gfx950. Physical layout `mk,gkn->mn`, rhs never transposed."""
 
   config_cls: ClassVar[type] = Config
   supports_symbolic_shapes: ClassVar[bool] = False
+  # With `preferred_element_type` fp8 (e4m3fn): return the result quantised per (row, 128 columns) as a QArray instead
+  # of widening it (pallas_mosaic_gpu.py:93, :316-318).
+  enable_fused_epilogue_quant: bool = False
 
   def __post_init__(self):
     if self.vjp is None:
@@ -290,25 +402,10 @@ class HipRaggedDot(base.RaggedDot):
     # releases the rows of no group from being zero (base.py:209-210); they are zeroed all the same.
     del maybe_quantize_lhs, zero_initialize
     if lhs_quantization_dtype is not None or rhs_quantization_dtype is not None:
-      raise NotImplementedError(
-          "The hip implementation does not quantise inputs on the fly (lhs_quantization_dtype,"
-          " rhs_quantization_dtype)."
-      )
-    if rhs_scale is not None:
-      # The raw-array form of quantised weights (experimental/gmm_v2/gmm_v2.py:1193-1199): rhs holds the
-      # quantised values and rhs_scale is [g, k-blocks, 1, n]; the result defaults to lhs.dtype (:1369-1370).
-      if isinstance(lhs, (QArray, AsQArray)) or isinstance(rhs, (QArray, AsQArray)):
-        raise NotImplementedError("rhs_scale comes with raw arrays, not QArrays.")
-      g, k, n = rhs.shape
-      if rhs_scale.dim() != 4 or tuple(rhs_scale.shape[::2]) != (g, 1) or rhs_scale.shape[3] != n:
-        raise NotImplementedError(f"rhs_scale must have shape [g, k-blocks, 1, n], got {tuple(rhs_scale.shape)}")
-      rhs = QArray(rhs, rhs_scale.reshape(g, rhs_scale.shape[1], n))
-      if preferred_element_type is None:
-        preferred_element_type = lhs.dtype
-    lhs, rhs = _per_row_lhs_scale(lhs), _per_column_rhs_scale(rhs)
-    if group_offset is not None and ragged_dot_dimension_numbers != base.DEFAULT_RAGGED_DOT_DIM_NUMS:
-      raise NotImplementedError("group_offset needs the default dimension numbers.")
-    # rhs_bias and fuse_gateup_activation (base.py:205-217) are fused into the forward kernel's epilogue.
+      # (gmm_v2's own arguments: quantise an operand to that type inside the TPU kernel. Callers here say the same
+      # with an `AsQArray` operand.)
+      raise NotImplementedError("lhs_quantization_dtype / rhs_quantization_dtype are not supported by the hip"
+                                " implementation; pass an AsQArray operand instead.")
     gateup = None
     if fuse_gateup_activation is not None:
       gateup = _GATEUP_ACTIVATIONS.get(fuse_gateup_activation)
@@ -317,60 +414,55 @@ class HipRaggedDot(base.RaggedDot):
                                   f" implementation (supported: {sorted(_GATEUP_ACTIVATIONS)}).")
       if return_residuals:
         raise NotImplementedError("return_residuals is not supported with fuse_gateup_activation.")
-    if isinstance(lhs, AsQArray) or isinstance(rhs, AsQArray):
-      raise NotImplementedError("The hip implementation does not quantise inputs on the fly (AsQArray).")
-    mode = _MODE_OF_DIMS.get(ragged_dot_dimension_numbers)
-    if mode is None:
-      raise NotImplementedError("Unsupported ragged dot dimension numbers.")
+    if group_offset is not None and ragged_dot_dimension_numbers != base.DEFAULT_RAGGED_DOT_DIM_NUMS:
+      raise NotImplementedError("group_offset needs the default dimension numbers.")
+
+    # Quantise / dequantise what the kernels cannot take as it is, then plan the call on shapes and types.
+    route = _route(_concrete_operand(lhs), _concrete_operand(rhs), dims=ragged_dot_dimension_numbers, precision=precision,
+                   rhs_scale=rhs_scale, fuse_gateup_activation=fuse_gateup_activation,
+                   preferred_element_type=preferred_element_type)
+    lhs, rhs, preferred_element_type = route.lhs, route.rhs, route.preferred_element_type
+    mode = _MODE_OF_DIMS[ragged_dot_dimension_numbers]
 
     lhs_scale = rhs_scale_ = None
-    for name, x in (("lhs", lhs), ("rhs", rhs)):
-      if isinstance(x, QArray) and (mode != 0 or x.zero_point is not None):
-        raise NotImplementedError(f"Quantised {name}: default dimension numbers without zero point only.")
-    widen_lhs, widen_rhs, native_k_blocks = _widening_plan(lhs, rhs, allow_native=gateup is None)
     if isinstance(lhs, QArray):
-      if widen_lhs:
-        if lhs.qvalue.shape[1] % 16 != 0:
-          raise NotImplementedError("Widening a quantised lhs needs k % 16 == 0.")
+      if route.widen_lhs:
         lhs_v = hip_ops.dequantize(lhs.qvalue, lhs.scale)
       else:
-        lhs_scale, lhs_v = lhs.scale, lhs.qvalue  # one scale per row: applied in the epilogue
+        lhs_scale, lhs_v = lhs.scale, lhs.qvalue  # one scale per row (or the kernels' own k-blocks)
     else:
       lhs_v = lhs
     if isinstance(rhs, QArray):
       g, k, n = rhs.qvalue.shape
-      if not widen_rhs:
+      if not route.widen_rhs:
         # One scale per (group, column): applied in the epilogue. Native k-blocks: [g, k/t_k, n] goes as it is.
         rhs_scale_, rhs_v = rhs.scale, rhs.qvalue
       else:
-        # Scales that change along k (or in blocks along n): widened to bf16 by a streaming pass, then the
-        # bf16 kernels.
-        if n % 16 != 0:
-          raise NotImplementedError("Widening quantised weights needs n % 16 == 0.")
-        blocks = _scale_blocks_along_k(rhs)
+        blocks = _scale_blocks_along_k(rhs) if mode == 0 else None
         rows = k // blocks if blocks else 0
         if (blocks and config.block_m == 16 and rhs.qvalue.dtype == torch.int8 and not isinstance(lhs, QArray)
             and rows % 32 == 0 and rows & (rows - 1) == 0 and rhs_bias is None and fuse_gateup_activation is None):
           # The streaming small-m kernel scales int8 weights per k-block while it widens them.
           rhs_scale_, rhs_v = rhs.scale, rhs.qvalue
         else:
+          # Scales that change along k (or in blocks along n): widened to bf16 by a streaming pass, then the
+          # bf16 kernels.
           rhs_v = hip_ops.dequantize(rhs.qvalue, rhs.scale)
     else:
       rhs_v = rhs
+    if route.cast_bf16:
+      lhs_v, rhs_v = lhs_v.to(torch.bfloat16), rhs_v.to(torch.bfloat16)
 
-    in_dtype = lhs.dtype if isinstance(lhs, QArray) else lhs_v.dtype
-    w_dtype = rhs.dtype if isinstance(rhs, QArray) else rhs_v.dtype
-    if not precision_lib.is_default(in_dtype, w_dtype, precision):
-      if precision == precision_lib.DotAlgorithmPreset.BF16_BF16_F32 and not isinstance(lhs, QArray) \
-          and not isinstance(rhs, QArray):
-        lhs_v, rhs_v = lhs_v.to(torch.bfloat16), rhs_v.to(torch.bfloat16)
-      else:
-        raise NotImplementedError(f"{precision=} not supported.")
-
-    if preferred_element_type is None:
-      preferred_element_type = torch.promote_types(in_dtype, w_dtype)
+    # fp8 output: widened to the weights' type by default (pallas_mosaic_gpu.py:197-205); with
+    # `enable_fused_epilogue_quant` the result is quantised to fp8 per (row, 128 columns) and returned as a QArray
+    # (pallas_mosaic_gpu_common.py:63-68, pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:797-824).
+    quantize_out = False
     if preferred_element_type == torch.float8_e4m3fn:
-      preferred_element_type = w_dtype  # widened, as pallas_mosaic_gpu.py:197-205
+      if self.enable_fused_epilogue_quant and mode == 0 and gateup is None and not return_residuals:
+        quantize_out = True
+        preferred_element_type = torch.float32  # the accumulator's type is what gets quantised
+      else:
+        preferred_element_type = rhs.dtype if isinstance(rhs, QArray) else rhs_v.dtype
     if preferred_element_type not in (torch.float32, torch.bfloat16, torch.float16):
       raise NotImplementedError(f"Output dtype {preferred_element_type} not supported.")
 
@@ -408,8 +500,6 @@ class HipRaggedDot(base.RaggedDot):
       return dot_out, None
 
     if mode == 2:
-      if isinstance(lhs, QArray) or isinstance(rhs, QArray):
-        raise NotImplementedError("Quantised inputs are not supported with ragged contracting dimensions.")
       dot_out = hip_ops.ragged_dot_drhs(lhs_v, rhs_v, gs, gs.numel(), config=kcfg, out_dtype=preferred_element_type)
     else:
       # A callable with no in-kernel twin is applied to an f32 result, i.e. still in the accumulator
@@ -421,6 +511,12 @@ class HipRaggedDot(base.RaggedDot):
                                        group_offset=group_offset)
       if unfused:
         dot_out = activation(dot_out).to(preferred_element_type)
+    if quantize_out:
+      # (a pass of its own over the f32 result, not yet part of the GEMM's epilogue)
+      n_out = dot_out.shape[1]
+      sub = 128 if n_out % 128 == 0 else n_out
+      qvalue, scale = hip_ops.quantize(dot_out, torch.float8_e4m3fn, (1, sub))
+      return QArray(qvalue, scale, None, torch.float8_e4m3fn), None
 
     residuals = dot_out
     if activation is not None and return_residuals:
@@ -432,44 +528,24 @@ class HipRaggedDot(base.RaggedDot):
   # -- configs ---------------------------------------------------------------------------------
   def _problem(self, ba: op.BoundArguments):
     lhs, rhs = ba.args[:2]
-    dims = ba.kwargs["ragged_dot_dimension_numbers"]
-    mode = _MODE_OF_DIMS.get(dims)
-    if mode is None:
-      raise NotImplementedError("Unsupported ragged dot dimension numbers.")
-    if mode == 0 and ba.kwargs.get("fuse_gateup_activation") is not None:
-      mode = 3  # forward with gate-up fusion: variants of their own
-    lhs_shape = tuple(lhs.shape)
-    rhs_shape = tuple(rhs.shape)
-    if mode == 2:
+    route = _route(_abstract_operand(lhs), _abstract_operand(rhs), dims=ba.kwargs["ragged_dot_dimension_numbers"],
+                   precision=ba.kwargs.get("precision"), rhs_scale=ba.kwargs.get("rhs_scale"),
+                   fuse_gateup_activation=ba.kwargs.get("fuse_gateup_activation"),
+                   preferred_element_type=ba.kwargs.get("preferred_element_type"))
+    lhs_shape, rhs_shape = tuple(lhs.shape), tuple(rhs.shape)
+    if route.mode == 2:
       num_groups = int(ba.kwargs["group_sizes"].shape[0])
       rows, cols, contraction = lhs_shape[1], rhs_shape[1], lhs_shape[0]
-    elif mode == 1:
+    elif route.mode == 1:
       num_groups = rhs_shape[0]
       rows, cols, contraction = lhs_shape[0], rhs_shape[1], rhs_shape[2]
     else:
       num_groups = rhs_shape[0]
       rows, cols, contraction = lhs_shape[0], rhs_shape[2], rhs_shape[1]
-    lhs_dt, rhs_dt = _dtype_of(lhs), _dtype_of(rhs)
-    raw_scale = ba.kwargs.get("rhs_scale")
-    if raw_scale is not None and len(raw_scale.shape) == 4 and not isinstance(rhs, (QArray, AsQArray)):
-      # (the raw form of quantised weights: `_fwd` makes the same QArray of it)
-      g_, blocks_, _, n_ = raw_scale.shape
-      rhs = QArray(rhs, ShapeDtype((g_, blocks_, n_), raw_scale.dtype))
-    if mode in (0, 3):
-      lhs, rhs = _per_row_lhs_scale(lhs), _per_column_rhs_scale(rhs)
-      widen_lhs, widen_rhs, native_k_blocks = _widening_plan(lhs, rhs, allow_native=mode == 0)
-      lhs_dt = torch.bfloat16 if widen_lhs else lhs_dt
-      rhs_dt = torch.bfloat16 if widen_rhs else rhs_dt
-      if native_k_blocks:
-        mode = 4  # forward with per-k-block weight scales: variants of their own
-    if (ba.kwargs.get("precision") == precision_lib.DotAlgorithmPreset.BF16_BF16_F32
-        and not isinstance(lhs, (QArray, AsQArray)) and not isinstance(rhs, (QArray, AsQArray))):
-      lhs_dt = rhs_dt = torch.bfloat16  # `_fwd` casts both operands for this preset
-    key = (mode, hip_ops.dtype_code(lhs_dt), hip_ops.dtype_code(rhs_dt))
-    return mode, key, num_groups, rows, cols, contraction
+    return route.mode, route.key, num_groups, rows, cols, contraction, route
 
   def _get_heuristics_config(self, ba: op.BoundArguments) -> Config:
-    mode, key, num_groups, rows, cols, contraction = self._problem(ba)
+    mode, key, num_groups, rows, cols, contraction, route = self._problem(ba)
     variants = _variant_table().get(key)
     if not variants:
       raise NotImplementedError(f"No hip kernel for dtypes/mode {key}.")
@@ -485,9 +561,7 @@ class HipRaggedDot(base.RaggedDot):
     usable = [v for v in variants if v[0] != 16 or streaming_ok]
     if mode == 4:
       # The k-step of a tiled variant has to divide the rows of a scale block (and the contraction).
-      rhs_ = _per_column_rhs_scale(ba.args[1])
-      raw_scale = ba.kwargs.get("rhs_scale")
-      blocks = raw_scale.shape[1] if raw_scale is not None else rhs_.scale.shape[1]
+      blocks = route.rhs.scale.shape[1]
       step = contraction // blocks if blocks > 1 else contraction
       usable = [v for v in usable if v[0] == 16 or step % v[2] == 0]
       if not usable:
@@ -538,7 +612,7 @@ class HipRaggedDot(base.RaggedDot):
                   align_tile=8)
 
   def _get_autotuning_configs(self, ba: op.BoundArguments) -> set[Config]:
-    mode, key, _, _, _, _ = self._problem(ba)
+    mode, key = self._problem(ba)[:2]
     configs = set()
     for bm, bn, bk, wm, wn, ns in _variant_table().get(key, []):
       widths = (1,) if (mode == 2 or bm == 16) else (1, 2, 4, 8, 16)

@@ -220,12 +220,54 @@ def dequantize_weights(qvalue: torch.Tensor, scale: torch.Tensor) -> torch.Tenso
   return out
 
 
-def dequantize(qvalue: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
-  """bf16 = qvalue * scale with each scale entry repeated over its tile (quantization.py:80-83).
+_QMAX = {torch.int8: 127.0, torch.float8_e4m3fn: 448.0}
+for _bits in range(2, 8):
+  if hasattr(torch, f"int{_bits}"):
+    _QMAX[getattr(torch, f"int{_bits}")] = float(2 ** (_bits - 1) - 1)  # sub-byte integers live in int8 storage
+
+
+def quantize(x: torch.Tensor, qtype: torch.dtype, tile_shape) -> tuple[torch.Tensor, torch.Tensor]:
+  """(qvalue, scale) of the absmax quantisation of `x` with one scale per tile of `tile_shape`
+  (`qwix.quantize(x, qtype, tiled_axes=dict(enumerate(tile_shape)))`, quantization.py:65-78):
+  scale = absmax(tile) / qmax (1 for an all-zero tile), qvalue = round_to_nearest_even(x / scale), saturated at qmax.
+
+  x f32, bf16 or f16: [rows, cols] with tiles one row tall and a multiple of 8 columns wide, or several rows tall and
+  1, 8, 16, ... or 256 columns wide; or weights [g, k, n] with a tile (1, t_k, t_n) (taken as g * k rows). qtype int8,
+  fp8 (e4m3fn) or a sub-byte integer (int4: values in [-7, 7], kept in int8 storage)."""
+  _require_cuda(x)
+  lib = _lib.load()
+  if qtype not in _QMAX:
+    raise NotImplementedError(f"quantisation to {qtype} is not supported by the hip implementation")
+  if x.dim() not in (2, 3) or len(tile_shape) != x.dim():
+    raise NotImplementedError("expected an array of 2 or 3 dimensions and a tile shape of as many")
+  tile_shape = tuple(int(t) for t in tile_shape)
+  if any(t < 1 or d % t for d, t in zip(x.shape, tile_shape)):
+    raise NotImplementedError(f"tile shape {tile_shape} does not tile {tuple(x.shape)}")
+  if x.dim() == 3:
+    if tile_shape[0] != 1:
+      raise NotImplementedError("weights are quantised per group: the tile must be (1, t_k, t_n)")
+    rows, cols = x.shape[0] * x.shape[1], x.shape[2]
+  else:
+    rows, cols = x.shape
+  t_r, t_c = tile_shape[-2], tile_shape[-1]
+  x = x.contiguous()
+  storage = torch.float8_e4m3fn if qtype == torch.float8_e4m3fn else torch.int8
+  qvalue = torch.empty(x.shape, dtype=storage, device=x.device)
+  scale = torch.empty(tuple(d // t for d, t in zip(x.shape, tile_shape)), dtype=torch.float32, device=x.device)
+  with _on_device(x.device):
+    st = lib.tkx_quantize(_ptr(x), _ptr(qvalue), _ptr(scale), rows, cols, t_r, t_c, dtype_code(x.dtype), dtype_code(storage),
+                          ctypes.c_float(_QMAX[qtype]), _stream(x.device))
+  _lib.check(st)
+  return qvalue, scale
+
+
+def dequantize(qvalue: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tensor | None = None) -> torch.Tensor:
+  """bf16 = (qvalue - zero_point) * scale with each scale (and zero point) entry repeated over its tile
+  (quantization.py:80-93).
 
   qvalue int8 or fp8 (e4m3fn): [rows, cols] with scale [rows/t_r, cols/t_c], or weights [g,k,n] with scale
-  [g, k/t_k, n/t_n]; t_c / t_n is 1 or a multiple of 16."""
-  _require_cuda(qvalue, scale)
+  [g, k/t_k, n/t_n]; t_c / t_n is 1 or a multiple of 16. `zero_point`, if given, has the scale's shape."""
+  _require_cuda(qvalue, scale, zero_point)
   lib = _lib.load()
   if qvalue.dtype not in (torch.int8, torch.float8_e4m3fn) or qvalue.dim() not in (2, 3) or scale.dim() != qvalue.dim():
     raise NotImplementedError("expected an int8 or fp8 qvalue of 2 or 3 dimensions and a scale of as many")
@@ -242,8 +284,15 @@ def dequantize(qvalue: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
   scale = scale.to(torch.float32).contiguous()
   out = torch.empty(qvalue.shape, dtype=torch.bfloat16, device=qvalue.device)
   with _on_device(qvalue.device):
-    st = lib.tkx_dequantize(_ptr(qvalue), _ptr(scale), _ptr(out), rows, cols, t_r, t_c, dtype_code(qvalue.dtype),
-                            _lib.TKX_BF16, _stream(qvalue.device))
+    if zero_point is None:
+      st = lib.tkx_dequantize(_ptr(qvalue), _ptr(scale), _ptr(out), rows, cols, t_r, t_c, dtype_code(qvalue.dtype),
+                              _lib.TKX_BF16, _stream(qvalue.device))
+    else:
+      if tuple(zero_point.shape) != tuple(scale.shape):
+        raise NotImplementedError("the zero point must have the scale's shape")
+      zero_point = zero_point.to(torch.float32).contiguous()
+      st = lib.tkx_dequantize_zero_point(_ptr(qvalue), _ptr(scale), _ptr(zero_point), _ptr(out), rows, cols, t_r, t_c,
+                                         dtype_code(qvalue.dtype), _lib.TKX_BF16, _stream(qvalue.device))
   _lib.check(st)
   return out
 
