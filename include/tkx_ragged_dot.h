@@ -49,7 +49,11 @@ enum TkxDtype {
   TKX_BF16 = 1,
   TKX_F16 = 2,
   TKX_F8E4M3FN = 3, /* OCP float8_e4m3fn */
-  TKX_I8 = 4
+  TKX_I8 = 4,
+  TKX_I4X2 = 5 /* signed 4-bit integers, two to a byte along the contraction axis: byte [g, kk, c] of an rhs
+                  [G, k/2, n] holds k = 2 kk in bits 0-3 and k = 2 kk + 1 in bits 4-7 (two's complement). Taken as the
+                  rhs of the streaming small-m kernel (block_m == 16, block_n == 128) only; tkx_unpack_int4 turns it
+                  into TKX_I8 for every other kernel. The reference defines no packed layout (its int4 is jnp.int4). */
 };
 
 enum TkxMode {
@@ -77,13 +81,29 @@ typedef struct TkxConfig {
                               unused by the streaming small-m kernel (block_m == 16) */
   int32_t align_tile;      /* task starts are aligned down to this many rows (reference default 8) */
   int32_t num_stages;      /* LDS stages of block_k contraction elements kept in flight */
+  int32_t split_k;         /* workgroups that share the contraction of one output tile (the reference's split_k,
+                              pallas_mosaic_gpu_common.py:53). 0 and 1: no split. Above 1: the streaming small-m kernel
+                              only (block_m == 16, block_n == 128, num_stages <= 4, k a multiple of
+                              128 * split_k * num_stages), and `workspace` then is
+                              tkx_ragged_dot_decode_workspace_bytes long with its first
+                              tkx_ragged_dot_decode_counter_bytes ZERO on entry; the call leaves them zero, so a caller
+                              that keeps one workspace per stream clears it once. */
 } TkxConfig;
 
-/* Library / ABI version (major*1000 + minor). */
+/* Library / ABI version (major*1000 + minor). 1001: TkxConfig gained split_k (a trailing field). */
 int32_t tkx_version(void);
 
 /* Thread-local message for the last non-zero status returned on this thread. */
 const char* tkx_last_error(void);
+
+/* Workspace of the streaming small-m kernel with the contraction split over split_k workgroups per output tile:
+ * arrival counters (one int32 per (group, column tile); the counter bytes come first and must be zero on entry),
+ * then the partial sums f32[split_k, m, n]. Both are 0 for split_k <= 1. The counters take 256 KiB whatever the
+ * shapes (so calls of any shapes can share a workspace that was cleared once), which limits
+ * num_groups * cdiv(n, 128) to 65536. The partial sums are added in the order of the split index whichever
+ * workgroup arrives last, so results are reproducible run to run. */
+int64_t tkx_ragged_dot_decode_workspace_bytes(int64_t m, int64_t n, int32_t split_k);
+int64_t tkx_ragged_dot_decode_counter_bytes(int32_t split_k);
 
 /* Number of task slots the schedule uses for (m, G, block_m): cdiv(m, block_m) + G - 1
  * (pallas_mosaic_gpu_kernel_sm90.py:54). */
@@ -199,6 +219,14 @@ int32_t tkx_dequantize(const void* qvalue, const float* scale, void* out, int64_
 int32_t tkx_dequantize_zero_point(const void* qvalue, const float* scale, const float* zero_point, void* out, int64_t rows,
                                   int64_t cols, int64_t scale_block_rows, int64_t scale_block_cols, int32_t q_dtype,
                                   int32_t out_dtype, tkx_stream_t stream);
+
+/* Packed int4 (TKX_I4X2) to int8 storage and back, for [.., rows, cols] arrays viewed as 2-D: `packed` has
+ * packed_rows rows of `cols` bytes, the int8 side 2 * packed_rows rows of `cols` values; value row 2 r sits in bits 0-3
+ * of packed row r, value row 2 r + 1 in bits 4-7 (for an rhs [G, k, n] with even k: packed_rows = G * k / 2, cols = n).
+ * tkx_pack_int4 keeps the low four bits of each value (values in [-8, 7] survive unchanged). cols % 16 == 0,
+ * 16-byte aligned pointers. No counterpart in the reference, which holds int4 as jnp.int4 arrays. */
+int32_t tkx_unpack_int4(const void* packed, void* out, int64_t packed_rows, int64_t cols, tkx_stream_t stream);
+int32_t tkx_pack_int4(const void* values, void* packed, int64_t packed_rows, int64_t cols, tkx_stream_t stream);
 
 /* Quantisation on the fly (AsQArray.as_qarray, quantization.py:65-78: qwix.quantize with the "absmax" calibration), the
  * inverse of tkx_dequantize:

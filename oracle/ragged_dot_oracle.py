@@ -53,6 +53,8 @@ below therefore cites the reference call site it follows, and says what pins it:
                                                                                   <= scale / 2; exact powers of two;
                                                                                   torch's float8_e4m3fn cast; zero tile
   dequantize_zero_point        quantization.py:85-93                              hand-computed values
+  pack_int4 / unpack_int4      no counterpart (the reference holds int4 as        hand-computed bytes for all 16 values
+                               jnp.int4 arrays; the layout is this library's)     on either side; round trip
 
 Status of "parity unpinned": `qwix.quantize` itself (qwix>=0.1.2, pyproject.toml:27) is not in the tree.
 `quantize_absmax` follows the form of its absmax calibration that the reference writes out for fp8; for the integer
@@ -224,6 +226,23 @@ def dequantize_zero_point(qvalue, scale, zero_point) -> np.ndarray:
     rep = q.shape[ax] // s.shape[ax]
     s, z = np.repeat(s, rep, axis=ax), np.repeat(z, rep, axis=ax)
   return (q - z) * s
+
+
+def pack_int4(values) -> np.ndarray:
+  """uint8 [.., r/2, c] from int values in [-8, 7] [.., r, c]: entry 2 i of the second-to-last axis in bits 0-3 of byte
+  i, entry 2 i + 1 in bits 4-7 (two's complement). The packed layout of the HIP library (TKX_I4X2); the reference has no
+  packed layout of its own."""
+  v = np.asarray(values).astype(np.int64)
+  lo, hi = v[..., 0::2, :] & 0xF, v[..., 1::2, :] & 0xF
+  return (lo | (hi << 4)).astype(np.uint8)
+
+
+def unpack_int4(packed) -> np.ndarray:
+  """The inverse of `pack_int4`: int8 [.., 2 r, c]."""
+  p = np.asarray(packed).astype(np.int64)
+  nib = np.stack([p & 0xF, (p >> 4) & 0xF], axis=-2)  # [.., r, 2, c]
+  nib = np.where(nib >= 8, nib - 16, nib)
+  return nib.reshape(*p.shape[:-2], 2 * p.shape[-2], p.shape[-1]).astype(np.int8)
 
 
 QMAX = {"int8": 127.0, "int4": 7.0, "fp8": 448.0}

@@ -509,6 +509,153 @@ def test_small_m_int8_kernel_edges(case, block_n, depth, device):
                                                  out_dtype=torch.float32, rhs_scale=scale))
 
 
+@pytest.mark.parametrize("split_k,depth", [(2, 2), (2, 4), (4, 2), (8, 2), (4, 4)])
+@pytest.mark.parametrize("case", ["ragged", "two_chunks", "all_empty", "one_big_group", "first_and_last_empty",
+                                  "beyond_m"])
+@pytest.mark.parametrize("weights", ["int8", "bf16", "int8_blocks"])
+def test_small_m_kernel_with_the_contraction_split_over_workgroups(case, split_k, depth, weights, device):
+  """split_k workgroups per (group, column tile): partial sums through the workspace, added by the last to arrive in
+  the order of the split index. Same edges as the unsplit kernel, group sizes that add up to more than m, the same
+  bits on a second run, and the arrival counters back at zero afterwards (the next call relies on it)."""
+  rng = np.random.default_rng(len(case) + depth + split_k)
+  k, n = 128 * split_k * depth * (2 if case == "ragged" else 1), 208
+  if case == "ragged":
+    gs = np.array([3, 0, 0, 17, 1, 0, 16, 2], np.int32)
+  elif case == "two_chunks":
+    gs = rng.integers(0, 4, 70).astype(np.int32)
+    gs[[0, 63, 64, 69]] = [0, 2, 0, 5]
+  elif case == "all_empty":
+    gs = np.zeros(5, np.int32)
+  elif case == "one_big_group":
+    gs = np.array([0, 45, 0], np.int32)
+  elif case == "beyond_m":
+    gs = np.array([5, 9, 7, 4], np.int32)
+  else:
+    gs = np.array([0, 4, 9, 0], np.int32)
+  G = len(gs)
+  m = 17 if case == "beyond_m" else int(gs.sum()) + 11
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  scale = None
+  if weights == "bf16":
+    rhs = torch.tensor(rng.normal(0, k ** -0.5, (G, k, n)).astype(np.float32), device=device).to(torch.bfloat16)
+    dense = _np(rhs)
+  else:
+    blocks = 1 if weights == "int8" else k // 64
+    rhs = torch.tensor(rng.integers(-128, 128, (G, k, n)).astype(np.int8), device=device)
+    scale = torch.tensor((np.abs(rng.normal(0, 0.01, (G, blocks, n))) + 1e-3).astype(np.float32), device=device)
+    dense = O.dequantize(rhs.cpu().numpy(), _np(scale))
+  cfg = hip_ops.KernelConfig(16, 128, 32, 1, 4, depth, split_k=split_k)
+  gst = torch.tensor(gs, device=device)
+  out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale)
+  clipped = np.diff(np.minimum(np.concatenate([[0], np.cumsum(gs)]), m)).astype(np.int32)
+  want = O.ragged_dot(_np(lhs), dense, clipped, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, 2e-3 if weights == "int8_blocks" else 1e-5)
+  assert torch.count_nonzero(out[int(clipped.sum()):]) == 0
+  ws = hip_ops.split_workspace(m, n, split_k, device)
+  counter_words = _lib.load().tkx_ragged_dot_decode_counter_bytes(split_k) // 4
+  assert counter_words >= G * 2 and torch.count_nonzero(ws[:counter_words]) == 0
+  again = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale)
+  assert torch.equal(out, again)
+  out16 = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.bfloat16, rhs_scale=scale)
+  assert torch.equal(out16, out.to(torch.bfloat16))
+
+
+def test_public_op_splits_the_contraction_when_a_launch_has_few_tiles(device):
+  """8 groups x 512 columns = 32 (group, column tile) pairs: the heuristics split the contraction 8 ways (256
+  workgroups), the autotuning search space offers the splits that divide k, and the result matches the oracle."""
+  rng = np.random.default_rng(11)
+  G, k, n = 8, 4096, 512
+  gs = np.array([2, 0, 1, 3, 0, 1, 2, 1], np.int32)
+  m = int(gs.sum()) + 2
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  q = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+  scale = torch.tensor((rng.uniform(0.5, 1.5, (G, 1, n)) / 127 * 0.1).astype(np.float32), device=device)
+  rhs = tokamax_amd.QArray(q, scale)
+  gst = torch.tensor(gs, device=device)
+  op = tokamax_amd.HipRaggedDot()
+  ba = op.bind(lhs, rhs, group_sizes=gst)
+  cfg = op._get_heuristics_config(ba)
+  assert (cfg.block_m, cfg.block_n, cfg.split_k) == (16, 128, 8)
+  splits = {c.split_k for c in op._get_autotuning_configs(ba) if c.block_m == 16}
+  assert splits == {1, 2, 4, 8}
+  out = op(lhs, rhs, group_sizes=gst, preferred_element_type=torch.float32)
+  want = O.ragged_dot(_np(lhs), O.dequantize(q.cpu().numpy(), _np(scale)), gs, O.DEFAULT, acc_dtype=np.float64,
+                      out_dtype="f64")
+  _check(out, want, 1e-5)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+
+
+def test_int4_pack_and_unpack_kernels(device):
+  """tkx_pack_int4 / tkx_unpack_int4 against the oracle's bytes, bit for bit, and the round trip."""
+  rng = np.random.default_rng(3)
+  q = rng.integers(-8, 8, (3, 64, 48)).astype(np.int8)
+  packed = hip_ops.pack_int4(torch.tensor(q, device=device))
+  assert packed.dtype == torch.uint8 and tuple(packed.shape) == (3, 32, 48)
+  assert np.array_equal(packed.cpu().numpy(), O.pack_int4(q))
+  assert np.array_equal(hip_ops.unpack_int4(packed).cpu().numpy(), q)
+  every_byte = torch.arange(256, dtype=torch.uint8, device=device).reshape(1, 16, 16)
+  assert np.array_equal(hip_ops.unpack_int4(every_byte).cpu().numpy(), O.unpack_int4(every_byte.cpu().numpy()))
+
+
+@pytest.mark.parametrize("depth,split_k", [(2, 1), (4, 1), (8, 1), (2, 2), (4, 2)])
+@pytest.mark.parametrize("scales", ["per_column", "k_blocks"])
+@pytest.mark.parametrize("case", ["ragged", "one_big_group", "first_and_last_empty"])
+def test_small_m_kernel_on_packed_int4_weights(case, scales, depth, split_k, device):
+  """Two int4 per byte along k: the streaming kernel's result matches the oracle on the unpacked values, and is the
+  int8 kernel's result on them bit for bit (same contraction order; only the loads and the widening differ)."""
+  if depth == 8 and scales == "k_blocks":
+    pytest.skip("no 8-deep variant with k-block scales")
+  rng = np.random.default_rng(len(case) + depth)
+  k, n = 2048, 208
+  gs = {"ragged": np.array([3, 0, 0, 17, 1, 0, 16, 2], np.int32), "one_big_group": np.array([0, 45, 0], np.int32),
+        "first_and_last_empty": np.array([0, 4, 9, 0], np.int32)}[case]
+  G, m = len(gs), int(gs.sum()) + 5
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  q = rng.integers(-8, 8, (G, k, n)).astype(np.int8)
+  blocks = 1 if scales == "per_column" else k // 128
+  scale = torch.tensor((np.abs(rng.normal(0, 0.05, (G, blocks, n))) + 1e-2).astype(np.float32), device=device)
+  packed = torch.tensor(O.pack_int4(q), device=device)
+  gst = torch.tensor(gs, device=device)
+  cfg = hip_ops.KernelConfig(16, 128, 32, 1, 4, depth, split_k=split_k)
+  out = hip_ops.ragged_dot_fwd(lhs, packed, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale)
+  want = O.ragged_dot(_np(lhs), O.dequantize(q, _np(scale)), gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, 2e-3 if scales == "k_blocks" else 1e-5)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  cfg8 = hip_ops.KernelConfig(16, 128, 32, 1, 4, min(depth, 4), split_k=split_k)
+  same = hip_ops.ragged_dot_fwd(lhs, torch.tensor(q, device=device), gst, config=cfg8, out_dtype=torch.float32, rhs_scale=scale)
+  assert torch.equal(out, same)
+
+
+def test_public_op_on_packed_int4_weights(device):
+  """`pack_int4` of a quantised rhs: with a few rows per group the op keeps it packed (streaming kernel, heuristics
+  name it); with many rows per group, a bias or another lhs type it unpacks to int8 first. Same results as the
+  unpacked QArray either way."""
+  rng = np.random.default_rng(8)
+  G, k, n = 16, 1024, 256
+  q = torch.tensor(rng.integers(-7, 8, (G, k, n)).astype(np.int8), device=device)
+  scale = torch.tensor((rng.uniform(0.5, 1.5, (G, 1, n)) / 7 * 0.1).astype(np.float32), device=device)
+  int4 = getattr(torch, "int4", torch.int8)
+  plain = tokamax_amd.QArray(q, scale, None, int4)
+  packed = tokamax_amd.pack_int4(plain)
+  assert packed.packed and packed.shape == (G, k, n) and tuple(packed.qvalue.shape) == (G, k // 2, n)
+  op = tokamax_amd.HipRaggedDot()
+  for rows in (2, 40):
+    gs = torch.full((G,), rows, dtype=torch.int32, device=device)
+    lhs = torch.tensor(rng.normal(0, 1, (G * rows, k)).astype(np.float32), device=device).to(torch.bfloat16)
+    cfg = op._get_heuristics_config(op.bind(lhs, packed, group_sizes=gs))
+    assert (cfg.block_m == 16) == (rows == 2)
+    out = op(lhs, packed, group_sizes=gs, preferred_element_type=torch.float32)
+    ref = op(lhs, plain, group_sizes=gs, preferred_element_type=torch.float32)
+    want = O.ragged_dot(_np(lhs), O.dequantize(q.cpu().numpy(), _np(scale)), np.full(G, rows, np.int32), O.DEFAULT,
+                        acc_dtype=np.float64, out_dtype="f64")
+    _check(out, want, 1e-5)
+    assert torch.equal(out, ref)
+  bias = torch.tensor(rng.normal(0, 1, (G, 1, n)).astype(np.float32), device=device)
+  gs = torch.full((G,), 2, dtype=torch.int32, device=device)
+  lhs = torch.tensor(rng.normal(0, 1, (G * 2, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  assert torch.equal(op(lhs, packed, group_sizes=gs, rhs_bias=bias), op(lhs, plain, group_sizes=gs, rhs_bias=bias))
+
+
 def test_public_op_picks_the_wide_small_m_kernel_when_it_fills_the_chip(device):
   """64 groups x 2048 columns = 512 workgroups of 256 columns (two per CU): the heuristics name the wide
   streaming kernel, and the public entry's result on it matches the oracle."""

@@ -38,7 +38,7 @@ def test_library_loads_and_exports_every_declared_symbol():
   lib = ctypes.CDLL(_lib.LIB_PATH)
   for name in declared:
     assert hasattr(lib, name), name
-  assert _lib.load().tkx_version() == 1000
+  assert _lib.load().tkx_version() == 1001  # 1001: TkxConfig.split_k
 
 
 def test_workspace_layout_queries():

@@ -462,3 +462,22 @@ def test_dequantize_zero_point_by_hand():
   q = np.array([[10, -3, 0, 7]], np.int8)
   got = O.dequantize_zero_point(q, np.array([[0.5, 2.0]], np.float32), np.array([[2.0, -1.0]], np.float32))
   assert got.tolist() == [[4.0, -2.5, 2.0, 16.0]]  # (10 - 2) / 2, (-3 - 2) / 2, (0 + 1) * 2, (7 + 1) * 2
+
+
+def test_int4_packing_by_hand():
+  """All 16 values in the low and in the high half of a byte, written out by hand: -8..-1 are 0x8..0xF, 0..7 are 0x0..0x7;
+  the even entry of a pair sits in bits 0-3."""
+  values = np.arange(-8, 8)
+  low = np.stack([values, np.zeros(16, int)], 0).T.reshape(32, 1)    # pairs (v, 0): byte = v's nibble
+  high = np.stack([np.zeros(16, int), values], 0).T.reshape(32, 1)   # pairs (0, v): byte = v's nibble << 4
+  nibbles = np.array([8, 9, 10, 11, 12, 13, 14, 15, 0, 1, 2, 3, 4, 5, 6, 7])
+  assert O.pack_int4(low)[:, 0].tolist() == nibbles.tolist()
+  assert O.pack_int4(high)[:, 0].tolist() == (nibbles * 16).tolist()
+  assert O.pack_int4(np.array([[-8], [7]])).tolist() == [[0x78]]
+  assert O.pack_int4(np.array([[1], [-1]])).tolist() == [[0xF1]]
+  assert O.unpack_int4(np.array([[0x78, 0xF1]], np.uint8)).tolist() == [[-8, 1], [7, -1]]
+  rng = np.random.default_rng(0)
+  q = rng.integers(-8, 8, (3, 10, 16)).astype(np.int8)
+  packed = O.pack_int4(q)
+  assert packed.shape == (3, 5, 16) and packed.dtype == np.uint8
+  assert np.array_equal(O.unpack_int4(packed), q)

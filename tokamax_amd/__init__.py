@@ -8,7 +8,7 @@ Public names follow tokamax/__init__.py:18-41 for this operator: `ragged_dot`,
 from tokamax_amd import config
 from tokamax_amd.autotuning.api import AutotuningResult, autotune, get_bound_args
 from tokamax_amd.op import AUTO, BoundArguments, NullConfig, Op
-from tokamax_amd.quantization import AsQArray, QArray
+from tokamax_amd.quantization import AsQArray, QArray, pack_int4
 from tokamax_amd.gated_linear_unit.api import gated_linear_unit
 from tokamax_amd.gated_linear_unit.hip import HipGatedLinearUnit
 from tokamax_amd.ragged_gather import ragged_gather, ragged_gather_reduce, ragged_scatter
@@ -28,7 +28,7 @@ from tokamax_amd.ragged_dot.hip import HipRaggedDot
 __all__ = [
     "AUTO", "AsQArray", "AutotuningResult", "BoundArguments", "DEFAULT_RAGGED_DOT_DIM_NUMS", "HipGatedLinearUnit",
     "HipRaggedDot",
-    "HipRaggedDotConfig", "NullConfig", "Op", "QArray", "RAGGED_CONTRACTING_DOT_DIM_NUMS",
+    "HipRaggedDotConfig", "NullConfig", "Op", "QArray", "RAGGED_CONTRACTING_DOT_DIM_NUMS", "pack_int4",
     "RAGGED_DOT_IMPLEMENTATIONS", "RaggedDotDimensionNumbers", "RaggedDotGroupSizes",
     "TRANS_RHS_RAGGED_DOT_DIM_NUMS", "autotune", "get_bound_args", "config", "gated_linear_unit", "generate_group_sizes", "ragged_dot",
     "ragged_dot_general", "ragged_gather", "ragged_gather_reduce", "ragged_scatter",

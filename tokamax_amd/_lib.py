@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libtkx_ragged_dot.so")
 
 TKX_OK, TKX_ERR_INVALID, TKX_ERR_UNSUPPORTED, TKX_ERR_RUNTIME = 0, 1, 2, 3
-TKX_F32, TKX_BF16, TKX_F16, TKX_F8E4M3FN, TKX_I8 = 0, 1, 2, 3, 4
+TKX_F32, TKX_BF16, TKX_F16, TKX_F8E4M3FN, TKX_I8, TKX_I4X2 = 0, 1, 2, 3, 4, 5
 TKX_MODE_DEFAULT, TKX_MODE_TRANS_RHS = 0, 1
 ACTIVATIONS = {None: 0, "relu": 1, "tanh": 2, "silu": 3, "gelu_tanh": 4, "sigmoid": 5,
                "swigluoai": 6, "silu_and_mul_with_clamp": 7}  # the last two: gate-up fusion only
@@ -38,6 +38,10 @@ EXPORTED_SYMBOLS = (
     "tkx_ragged_gather_rows",
     "tkx_ragged_dot_num_variants",
     "tkx_ragged_dot_variant",
+    "tkx_ragged_dot_decode_workspace_bytes",
+    "tkx_ragged_dot_decode_counter_bytes",
+    "tkx_unpack_int4",
+    "tkx_pack_int4",
 )
 
 
@@ -55,6 +59,7 @@ class TkxConfig(ctypes.Structure):
       ("grid_tile_width", ctypes.c_int32),
       ("align_tile", ctypes.c_int32),
       ("num_stages", ctypes.c_int32),
+      ("split_k", ctypes.c_int32),
   ]
 
 
@@ -67,6 +72,13 @@ def _declare(lib):
   cfgp = ctypes.POINTER(TkxConfig)
   lib.tkx_version.restype = i32
   lib.tkx_version.argtypes = []
+  lib.tkx_ragged_dot_decode_workspace_bytes.restype = i64
+  lib.tkx_ragged_dot_decode_workspace_bytes.argtypes = [i64, i64, i32]
+  lib.tkx_ragged_dot_decode_counter_bytes.restype = i64
+  lib.tkx_ragged_dot_decode_counter_bytes.argtypes = [i32]
+  for fn in (lib.tkx_unpack_int4, lib.tkx_pack_int4):
+    fn.restype = i32
+    fn.argtypes = [vp, vp, i64, i64, vp]
   lib.tkx_last_error.restype = ctypes.c_char_p
   lib.tkx_last_error.argtypes = []
   lib.tkx_ragged_dot_tid_size.restype = i64

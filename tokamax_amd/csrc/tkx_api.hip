@@ -47,6 +47,8 @@ struct Registry {
     for (int dtype : {TKX_BF16, TKX_F16})
       for (int depth : {2, 4})
         all.push_back({kFwd, dtype, dtype, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
+    for (int depth : {2, 4, 8})  // packed int4 weights: the streaming kernel is their only kernel
+      all.push_back({kFwd, TKX_BF16, TKX_I4X2, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
   }
 };
 
@@ -120,9 +122,18 @@ using namespace tkx;
 
 extern "C" {
 
-int32_t tkx_version(void) { return 1000; }
+int32_t tkx_version(void) { return 1001; }
 
 const char* tkx_last_error(void) { return g_err; }
+
+int64_t tkx_ragged_dot_decode_workspace_bytes(int64_t m, int64_t n, int32_t split_k) {
+  if (m < 0 || n < 1) return -1;
+  return decode_split_workspace_words(m, n, split_k) * 4;
+}
+
+int64_t tkx_ragged_dot_decode_counter_bytes(int32_t split_k) {
+  return split_k > 1 ? decode_split_counter_words() * 4 : 0;
+}
 
 int64_t tkx_ragged_dot_tid_size(int64_t m, int64_t num_groups, int32_t block_m) {
   if (m < 0 || num_groups < 1 || block_m < 1) return -1;
@@ -248,15 +259,19 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
     // Streaming decode kernel: one launch, no schedule.
     if (lhs_scale != nullptr) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no lhs scale");
     if (rhs_bias != nullptr || gateup) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no bias or gate-up fusion");
-    if (rhs_scale != nullptr && rhs_dtype != TKX_I8 && rhs_dtype != TKX_F8E4M3FN)
-      return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes an rhs scale with int8 or fp8 weights only");
-    if (!decode_supported(lhs_dtype, rhs_dtype, m, k, n, num_groups, rhs_scale ? rhs_scale_blocks : 1, c.block_n))
+    if (rhs_scale != nullptr && rhs_dtype != TKX_I8 && rhs_dtype != TKX_F8E4M3FN && rhs_dtype != TKX_I4X2)
+      return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes an rhs scale with int8, packed int4 or fp8 weights only");
+    const int32_t split_k = c.split_k > 1 ? c.split_k : 1;  // (0, from a caller that never heard of the field, is 1)
+    if (!decode_supported(lhs_dtype, rhs_dtype, m, k, n, num_groups, rhs_scale ? rhs_scale_blocks : 1, c.block_n,
+                          c.num_stages, split_k))
       return set_error(TKX_ERR_UNSUPPORTED,
-                       "decode kernel needs k %% 1024 == 0, n %% 8 == 0 (n %% 16 == 0 and one scale block at block_n 256)"
-                       " and scale blocks of a power-of-two multiple of 32 rows (k=%lld n=%lld G=%lld scale blocks=%lld)",
-                       (long long)k, (long long)n, (long long)num_groups, (long long)rhs_scale_blocks);
+                       "decode kernel needs k %% 1024 == 0 (split: k %% (128 * split_k * min(num_stages, 4)) == 0, split_k <= 16,"
+                       " num_stages <= 4, block_n 128), n %% 8 == 0 (n %% 16 == 0 and one scale block at block_n 256)"
+                       " and scale blocks of a power-of-two multiple of 32 rows (k=%lld n=%lld G=%lld scale blocks=%lld split_k=%d)",
+                       (long long)k, (long long)n, (long long)num_groups, (long long)rhs_scale_blocks, split_k);
     return launch_decode(lhs, rhs, rhs_scale, group_sizes, out, m, k, n, num_groups, rhs_dtype, out_dtype, activation,
-                         c.num_stages, rhs_scale ? rhs_scale_blocks : 1, c.block_n, group_offset, num_group_sizes, stream);
+                         c.num_stages, rhs_scale ? rhs_scale_blocks : 1, c.block_n, group_offset, num_group_sizes,
+                         split_k, static_cast<int32_t*>(workspace), stream);
   }
 
   const WsLayout L = ws_layout(m, num_groups, c.block_m);
@@ -473,6 +488,24 @@ int32_t tkx_dequantize_zero_point(const void* qvalue, const float* scale, const 
                         static_cast<hipStream_t>(stream));
 }
 
+namespace {
+int32_t int4_repack(const void* in, void* out, int64_t packed_rows, int64_t cols, bool unpack, tkx_stream_t stream) {
+  if (!in || !out) return set_error(TKX_ERR_INVALID, "null pointer argument");
+  if (packed_rows < 1 || cols < 1) return set_error(TKX_ERR_INVALID, "bad sizes rows=%lld cols=%lld", (long long)packed_rows, (long long)cols);
+  if (cols % 16 != 0 || cols > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "cols must be a multiple of 16");
+  if (((uintptr_t)in | (uintptr_t)out) % 16 != 0) return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
+  return launch_int4_repack(in, out, packed_rows, cols, unpack, static_cast<hipStream_t>(stream));
+}
+}  // namespace
+
+int32_t tkx_unpack_int4(const void* packed, void* out, int64_t packed_rows, int64_t cols, tkx_stream_t stream) {
+  return int4_repack(packed, out, packed_rows, cols, true, stream);
+}
+
+int32_t tkx_pack_int4(const void* values, void* packed, int64_t packed_rows, int64_t cols, tkx_stream_t stream) {
+  return int4_repack(values, packed, packed_rows, cols, false, stream);
+}
+
 int32_t tkx_quantize(const void* x, void* qvalue, float* scale, int64_t rows, int64_t cols, int64_t scale_block_rows,
                      int64_t scale_block_cols, int32_t x_dtype, int32_t q_dtype, float qmax, tkx_stream_t stream) {
   if (!x || !qvalue || !scale) return set_error(TKX_ERR_INVALID, "null pointer argument");
@@ -545,6 +578,7 @@ int32_t tkx_ragged_dot_variant(int32_t kind, int32_t index, TkxConfig* config, i
     config->grid_tile_width = 1;
     config->align_tile = 8;
     config->num_stages = v.num_stages;
+    config->split_k = 1;
     *lhs_dtype = v.a_dtype;
     *rhs_dtype = v.b_dtype;
     *mode = v.mode;

@@ -1,4 +1,5 @@
 // Small-m ("decode") ragged dot: bf16 lhs [m,k] x int8 or fp8 (e4m3fn) rhs [G,k,n] with f32 scales [G,n],
+// or x int4 rhs packed two to a byte along k ([G,k/2,n] bytes: k = 2 kk in bits 0-3, k = 2 kk + 1 in bits 4-7),
 // or bf16 x bf16 / f16 x f16 without scales.
 //
 // This regime is bound by HBM: every touched expert's [k,n] weight panel is read once, and a group
@@ -46,6 +47,11 @@ struct DecodeParams {
   int32_t num_global;           // entries of group_sizes (num_groups without an offset)
   int32_t scale_blocks;     // scale blocks along k: scale is [G, scale_blocks, n]
   int32_t log2_block_rows;  // scale_blocks > 1: log2 of the contraction rows per scale block
+  // Contraction split over workgroups (SK kernels): split_k workgroups per (group, column tile), each with
+  // k / split_k of the contraction; f32 partial sums [split_k, m, n] and one arrival counter per tile.
+  int32_t split_k;
+  float* partials;
+  int32_t* counters;  // [G * n_tiles], zero on entry; the last workgroup to arrive at a tile resets its counter
 };
 
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
@@ -69,14 +75,17 @@ __device__ __forceinline__ i32x4 buffer_load_16_streaming(__amdgpu_buffer_rsrc_t
   return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_offset, (int)uniform_offset, kStreamingLoad));
 }
 
+constexpr int kEI4 = TKX_I4X2;  // packed int4 weights: a stored row holds two contraction rows
+
 // What a lane holds of one weight row of a step: its CPL columns (8, or 16 of int8).
 template <int EW, int CPL> struct WeightRow { typedef i32x4 T; static constexpr int ESZ = 2; };
+template <> struct WeightRow<kEI4, 8> { typedef i32x2 T; static constexpr int ESZ = 1; };
 template <> struct WeightRow<kEI8, 8> { typedef i32x2 T; static constexpr int ESZ = 1; };
 template <> struct WeightRow<kEF8, 8> { typedef i32x2 T; static constexpr int ESZ = 1; };
 template <> struct WeightRow<kEI8, 16> { typedef i32x4 T; static constexpr int ESZ = 1; };
 template <int EW, int CPL>
 __device__ __forceinline__ typename WeightRow<EW, CPL>::T load_weight_row(__amdgpu_buffer_rsrc_t r, uint32_t lane_offset, uint32_t uniform_offset) {
-  if constexpr ((EW == kEI8 || EW == kEF8) && CPL == 8) return buffer_load_8(r, lane_offset, uniform_offset);
+  if constexpr ((EW == kEI8 || EW == kEF8 || EW == kEI4) && CPL == 8) return buffer_load_8(r, lane_offset, uniform_offset);
   else return buffer_load_16_streaming(r, lane_offset, uniform_offset);
 }
 
@@ -104,6 +113,32 @@ __device__ __forceinline__ i32x4 column_fragment_i8(const Row (&rows)[8]) {
     out[h] = (int)__builtin_amdgcn_perm(f1, f0, 0x07060302u);
   }
   return out;
+}
+// Packed int4 weights: byte J of each of 4 loaded rows holds two consecutive contraction values of column J (low
+// nibble first); each is sign-extended out of its bit field, converted, and the pair packed as above.
+// (The bit-field builtin is declared with an unsigned result; the value is the sign-extended field.)
+__device__ __forceinline__ float int4_field(int w, unsigned offset) { return (float)(int)__builtin_amdgcn_sbfe(w, offset, 4); }
+template <int J>
+__device__ __forceinline__ i32x4 column_fragment_i4(const i32x2 (&rows)[4]) {
+  i32x4 out;
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    const int w = rows[h][J >> 2];
+    const float lo = int4_field(w, 8 * (J & 3)), hi = int4_field(w, 8 * (J & 3) + 4);
+    out[h] = (int)__builtin_amdgcn_perm(__builtin_bit_cast(unsigned, hi), __builtin_bit_cast(unsigned, lo), 0x07060302u);
+  }
+  return out;
+}
+template <int J>
+__device__ __forceinline__ i32x4 column_fragment_i4_scaled(const i32x2 (&rows)[4], float scale) {
+  bf16x8 out;
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    const int w = rows[h][J >> 2];
+    out[2 * h] = (__bf16)(int4_field(w, 8 * (J & 3)) * scale);
+    out[2 * h + 1] = (__bf16)(int4_field(w, 8 * (J & 3) + 4) * scale);
+  }
+  return __builtin_bit_cast(i32x4, out);
 }
 // fp8 (e4m3fn) weights: byte J of each row through the hardware conversion; an e4m3 value has 3
 // significand bits, so the upper half of its f32 is its bf16 exactly.
@@ -158,18 +193,30 @@ __device__ __forceinline__ f32x4_t mma_16x16x32(i32x4 w, i32x4 a, f32x4_t acc) {
 // they are widened, instead of one multiply per output in the epilogue.
 // CPL = columns per lane; a workgroup covers BN = 16 CPL columns. 16 (int8 only) makes the loads 16
 // bytes per lane and the rows a wave reads 256 bytes long, the shape 16-bit weights have at CPL 8.
-template <int EW, int kDecDepth, int kMinWgs, bool SUB = false, int CPL = 8>
+// SK: the contraction of a (group, column tile) is split over p.split_k workgroups (the finer work items even out
+// what each CU streams when a launch has only two or three of the unsplit ones per CU). Each writes its f32
+// partial sums to p.partials and announces itself on the tile's counter; the last one to arrive adds the partials
+// in the order of the split index (so the result does not depend on who that is), scales and stores. These
+// workgroups wait for their group's size before they load any weights: a workgroup's slice is a few steps long,
+// and loading ahead of the size would read most of an empty group's weights.
+template <int EW, int kDecDepth, int kMinWgs, bool SUB = false, int CPL = 8, bool SK = false>
 __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const DecodeParams p) {
-  static_assert(!SUB || EW == kEI8 || EW == kEF8, "sub-channel scales belong to int8 or fp8 weights");
+  static_assert(!SUB || EW == kEI8 || EW == kEF8 || EW == kEI4, "sub-channel scales belong to int8, int4 or fp8 weights");
   static_assert(CPL == 8 || (CPL == 16 && EW == kEI8 && !SUB), "16 columns per lane: int8 weights with per-column scales");
-  constexpr int EA = (EW == kEI8 || EW == kEF8) ? kEBF16 : EW;
+  constexpr int EA = (EW == kEI8 || EW == kEF8 || EW == kEI4) ? kEBF16 : EW;
+  constexpr int KPR = EW == kEI4 ? 2 : 1;  // contraction rows per stored weight row
+  constexpr int RPS = 8 / KPR;             // stored rows a lane loads per step
   constexpr int WESZ = WeightRow<EW, CPL>::ESZ;
   constexpr int BN = 16 * CPL;
   typedef typename WeightRow<EW, CPL>::T WRow;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   __shared__ int s_red[kDecWaves];
+  __shared__ int s_last;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int g = blockIdx.x / p.n_tiles, nt = blockIdx.x - g * p.n_tiles;
+  const int splits = SK ? p.split_k : 1;
+  const int tile = SK ? (int)blockIdx.x / splits : (int)blockIdx.x;
+  const int split = SK ? (int)blockIdx.x - tile * splits : 0;
+  const int g = tile / p.n_tiles, nt = tile - g * p.n_tiles;
   const int col0 = nt * BN;
   const bool last_group = g == p.num_groups - 1;
 
@@ -185,20 +232,26 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
   const int own_size = gg >= 0 && gg < p.num_global ? max(p.group_sizes[min(max(gg, 0), p.num_global - 1)], 0) : 0;
   const int preceding = min(max(gg, 0), p.num_global);  // entries whose rows come before this group's
 
-  const int kw = p.k / kDecWaves;      // contraction slice of this wave
-  const int k_begin = wave * kw;
+  const bool first_of_shard = g == 0 && p.group_offset != nullptr;
+  const bool zeroes_rows = split == 0 && (last_group || first_of_shard);  // rows of no group are this workgroup's
+  if constexpr (SK) {
+    if (__builtin_amdgcn_readfirstlane(own_size) == 0 && !zeroes_rows) return;
+  }
+
+  const int kw = p.k / (kDecWaves * splits);  // contraction slice of this wave
+  const int k_begin = (split * kDecWaves + wave) * kw;
   const int steps = kw / kDecKS;       // multiple of kDecDepth (checked on the host)
-  const unsigned char* wbase = p.rhs + ((int64_t)g * p.k + k_begin) * p.n * WESZ;
+  const unsigned char* wbase = p.rhs + ((int64_t)g * (p.k / KPR) + k_begin / KPR) * p.n * WESZ;
   // B loads: lane (i = lane % 16, q = lane / 16) -> rows 8q + e (e = 0..7), columns col0 + CPL i .. + CPL - 1,
   // clamped at the last CPL columns (n is a multiple of CPL; clamped lanes feed columns that are never stored).
   const int li = lane & 15, lq = lane >> 4;
   int colb = col0 + li * CPL;
   colb = colb < p.n - CPL ? colb : p.n - CPL;
-  uint32_t boff[8];
+  uint32_t boff[RPS];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) boff[e] = (uint32_t)((8 * lq + e) * p.n + colb) * WESZ;
+  for (int e = 0; e < RPS; ++e) boff[e] = (uint32_t)((RPS * lq + e) * p.n + colb) * WESZ;
 
-  WRow breg[kDecDepth][8];
+  WRow breg[kDecDepth][RPS];
   i32x4 areg[kDecDepth];
   i32x4 sreg[SUB ? kDecDepth : 1][2];  // SUB: f32 scales of columns 8i..8i+7 for the step's k-block
   const __amdgpu_buffer_rsrc_t sbuf = buffer_of(SUB ? p.scale + (int64_t)g * p.scale_blocks * p.n : nullptr,
@@ -206,12 +259,12 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
   const uint32_t soff = (uint32_t)colb * 4u;
   // Nothing looks at a loaded value before its step comes up, so the only waits are the per-step
   // vmcnt of the oldest group.
-  const __amdgpu_buffer_rsrc_t wbuf = buffer_of(wbase, (uint32_t)kw * (uint32_t)p.n * WESZ);
-  const uint32_t step_bytes = (uint32_t)(kDecKS * p.n) * WESZ;
+  const __amdgpu_buffer_rsrc_t wbuf = buffer_of(wbase, (uint32_t)(kw / KPR) * (uint32_t)p.n * WESZ);
+  const uint32_t step_bytes = (uint32_t)(kDecKS / KPR * p.n) * WESZ;
   auto issue_b = [&](int slot, int step) {
     const uint32_t so = (uint32_t)__builtin_amdgcn_readfirstlane((int)(step * step_bytes));
 #pragma unroll
-    for (int e = 0; e < 8; ++e) breg[slot][e] = load_weight_row<EW, CPL>(wbuf, boff[e], so);
+    for (int e = 0; e < RPS; ++e) breg[slot][e] = load_weight_row<EW, CPL>(wbuf, boff[e], so);
     if constexpr (SUB) {
       // (Past the wave's slice the block index runs past the buffer and the loads return zero.)
       const uint32_t kb = (uint32_t)(k_begin + step * kDecKS) >> p.log2_block_rows;
@@ -242,7 +295,6 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
 
   // Row range of this group.
   const int size = __builtin_amdgcn_readfirstlane(own_size);
-  const bool first_of_shard = g == 0 && p.group_offset != nullptr;
   if (size == 0 && !last_group && !first_of_shard) return;
   int before = tid < preceding ? max(first_size, 0) : 0;
   for (int j = tid + kDecThreads; j < preceding; j += kDecThreads) before += max(p.group_sizes[j], 0);  // G > 256 only
@@ -257,7 +309,7 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
   const int end = min(start + size, p.m);
   const int esz = p.out_dtype == TKX_F32 ? 4 : 2;
 
-  if (last_group || first_of_shard) {
+  if (zeroes_rows) {
     // Rows past the last group, and with a group offset the rows before the first, belong to no
     // group of this call: zero this workgroup's columns of them.
     const int ncol = min(BN, p.n - col0);
@@ -273,7 +325,7 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
     if (last_group) zero_rows(end, p.m);
     if (first_of_shard) zero_rows(0, min(start, p.m));
   }
-  if (end <= start) return;
+  if (end <= start) return;  // (every split of a tile takes this exit or none does)
 
   // lhs rows of this group as one buffer: rows at or past the group's end read as zero.
   const __amdgpu_buffer_rsrc_t abuf = buffer_of(p.lhs + (int64_t)start * p.k * 2, (uint32_t)(end - start) * (uint32_t)p.k * 2u);
@@ -313,7 +365,9 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
         }
         auto column = [&](auto j_tag) {
           constexpr int J = decltype(j_tag)::value;
-          if constexpr (SUB) return column_fragment_scaled<EW, J>(breg[d], col_scale[J]);
+          if constexpr (SUB && EW == kEI4) return column_fragment_i4_scaled<J>(breg[d], col_scale[J]);
+          else if constexpr (SUB) return column_fragment_scaled<EW, J>(breg[d], col_scale[J]);
+          else if constexpr (EW == kEI4) return column_fragment_i4<J>(breg[d]);
           else if constexpr (EW == kEI8) return column_fragment_i8<J>(breg[d]);
           else if constexpr (EW == kEF8) return column_fragment_f8<J>(breg[d]);
           else return column_fragment_16bit<J>(breg[d]);
@@ -378,6 +432,14 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
 #pragma unroll
           for (int w = 0; w < kDecWaves; ++w)
             v += *reinterpret_cast<const f32x4_t*>(reinterpret_cast<const float*>(smem) + w * (kDecRows * BN) + r * BN + c0 + 4 * t);
+          if constexpr (SK) {
+            // Stores of device scope: they go through to memory instead of staying in this XCD's L2, so that no
+            // write-back of the whole L2 is needed before the arrival below.
+            float* dst = p.partials + ((int64_t)split * p.m * p.n + idx + 4 * t);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) __hip_atomic_store(dst + i, v[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            continue;
+          }
           v *= col_scales[t];
           store4(p.out, idx + 4 * t,
                  (f32x4){apply_activation(v[0], p.activation), apply_activation(v[1], p.activation),
@@ -396,38 +458,99 @@ __global__ __launch_bounds__(kDecThreads, kMinWgs) void decode_kernel(const Deco
       }
     }
   }
+
+  if constexpr (SK) {
+    // Arrival: every thread waits for its partial sums to be written (a fence of workgroup scope is that wait and
+    // nothing else; the stores themselves were of device scope) before thread 0 counts this workgroup in.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (tid == 0) {
+      int32_t* counter = p.counters + tile;
+      const int arrived = atomicAdd(counter, 1);
+      s_last = arrived == splits - 1;
+      if (arrived == splits - 1) atomicExch(counter, 0);  // nobody else touches it any more in this launch
+    }
+    __syncthreads();
+    if (!s_last) return;
+    // The partial sums are read with loads of device scope, which do not take a line this XCD's L2 may hold.
+    const int c0 = (tid & 15) * CPL, col = col0 + c0;
+    if (col + CPL > p.n) return;
+    for (int row = start + (tid >> 4); row < end; row += kDecRows) {
+      const int64_t idx = (int64_t)row * p.n + col;
+#pragma unroll
+      for (int t = 0; t < CPL / 4; ++t) {
+        f32x4_t v = {0.f, 0.f, 0.f, 0.f};
+        for (int sp = 0; sp < splits; ++sp) {
+          const float* src = p.partials + ((int64_t)sp * p.m * p.n + idx + 4 * t);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] += __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        v *= col_scales[t];
+        store4(p.out, idx + 4 * t,
+               (f32x4){apply_activation(v[0], p.activation), apply_activation(v[1], p.activation),
+                       apply_activation(v[2], p.activation), apply_activation(v[3], p.activation)},
+               p.out_dtype);
+      }
+    }
+  }
 }
 
 }  // namespace
 
-// Whether the decode kernel can run this problem (else the caller uses the tiled kernel).
+constexpr int64_t kDecCounterWords = 64 * 1024;  // arrival counters of the split form: a fixed share of its workspace
+
+// Whether the decode kernel can run this problem (else the caller uses the tiled kernel). `depth` steps of loads in
+// flight per wave, `split_k` workgroups per (group, column tile).
 bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k, int64_t n, int64_t G,
-                      int64_t scale_blocks, int32_t block_n) {
-  (void)G;
+                      int64_t scale_blocks, int32_t block_n, int32_t depth, int32_t split_k) {
   // The lhs rows of a group are addressed through one buffer with 32-bit byte offsets (a group may hold all m rows).
   if (m * k * 2 >= (1LL << 32)) return false;
+  if (split_k < 1 || split_k > 16 || depth < 1) return false;
   if (block_n != kDecBN) {
-    // The wide kernel: int8 weights with per-column scales, 16 columns per lane.
-    if (block_n != 2 * kDecBN || rhs_dtype != TKX_I8 || scale_blocks != 1 || n % 16 != 0) return false;
+    // The wide kernel: int8 weights with per-column scales, 16 columns per lane, no split.
+    if (block_n != 2 * kDecBN || rhs_dtype != TKX_I8 || scale_blocks != 1 || n % 16 != 0 || split_k != 1) return false;
   }
+  if (split_k > 1 && (depth > 4 || G * ((n + block_n - 1) / block_n) > kDecCounterWords)) return false;
   if (scale_blocks != 1) {
     // Sub-channel scales: int8 weights, blocks of a power-of-two number of rows that whole steps fit.
-    if ((rhs_dtype != TKX_I8 && rhs_dtype != TKX_F8E4M3FN) || scale_blocks < 1 || k % scale_blocks != 0) return false;
+    if ((rhs_dtype != TKX_I8 && rhs_dtype != TKX_F8E4M3FN && rhs_dtype != TKX_I4X2) || scale_blocks < 1 || k % scale_blocks != 0) return false;
     const int64_t rows = k / scale_blocks;
     if (rows % kDecKS != 0 || (rows & (rows - 1)) != 0 || scale_blocks * n * 4 >= (1LL << 31)) return false;
   }
-  const bool types = (lhs_dtype == TKX_BF16 && (rhs_dtype == TKX_I8 || rhs_dtype == TKX_F8E4M3FN || rhs_dtype == TKX_BF16)) ||
+  const bool types = (lhs_dtype == TKX_BF16 && (rhs_dtype == TKX_I8 || rhs_dtype == TKX_F8E4M3FN || rhs_dtype == TKX_BF16 ||
+                                                rhs_dtype == TKX_I4X2)) ||
                      (lhs_dtype == TKX_F16 && rhs_dtype == TKX_F16);
   if (!types) return false;
-  const int64_t wesz = (rhs_dtype == TKX_I8 || rhs_dtype == TKX_F8E4M3FN) ? 1 : 2;
+  if (rhs_dtype == TKX_I4X2 && (block_n != kDecBN || (split_k > 1 && depth > 4))) return false;
+  const int64_t wesz = (rhs_dtype == TKX_BF16 || rhs_dtype == TKX_F16) ? 2 : 1;
   if ((k / kDecWaves) * n * wesz >= (1LL << 31)) return false;
-  return k % (kDecWaves * kDecKS * 8) == 0 && n % 8 == 0 && n >= 8;
+  // Every wave's slice is a whole number of pipeline rounds. (Unsplit: 1024, whatever the depth, as it always was.)
+  const int64_t round = split_k == 1 ? kDecWaves * kDecKS * 8 : (int64_t)kDecWaves * split_k * kDecKS * (depth <= 2 ? 2 : 4);
+  return k % round == 0 && n % 8 == 0 && n >= 8;
 }
+
+// Words of workspace the split form needs: the tiles' arrival counters, then the partial sums. The counters take
+// the same number of words whatever the shapes, so that calls of different shapes can share one workspace without
+// one call's partial sums landing where another expects zeroed counters.
+int64_t decode_split_counter_words() { return kDecCounterWords; }
+int64_t decode_split_workspace_words(int64_t m, int64_t n, int32_t split_k) {
+  if (split_k <= 1) return 0;
+  return kDecCounterWords + (int64_t)split_k * m * n;
+}
+
+namespace {
+template <int EW, int D, int W, bool SUB = false>
+const void* decode_fn(bool split) {
+  return split ? reinterpret_cast<const void*>(&decode_kernel<EW, D, W, SUB, 8, true>)
+               : reinterpret_cast<const void*>(&decode_kernel<EW, D, W, SUB, 8, false>);
+}
+}  // namespace
 
 int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
                       int64_t m, int64_t k, int64_t n, int64_t G, int32_t rhs_dtype, int32_t out_dtype,
                       int32_t activation, int32_t depth, int64_t scale_blocks, int32_t block_n,
-                      const int32_t* group_offset, int64_t num_global, hipStream_t stream) {
+                      const int32_t* group_offset, int64_t num_global, int32_t split_k, int32_t* split_workspace,
+                      hipStream_t stream) {
   DecodeParams p;
   p.group_offset = group_offset;
   p.num_global = (int32_t)num_global;
@@ -435,6 +558,7 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
   p.log2_block_rows = 0;
   for (int64_t rows = k / scale_blocks; rows > 1; rows >>= 1) ++p.log2_block_rows;
   const bool sub = scale_blocks > 1 && scale != nullptr;
+  const bool sk = split_k > 1;
   p.lhs = static_cast<const unsigned char*>(lhs);
   p.rhs = static_cast<const unsigned char*>(rhs);
   p.scale = scale;
@@ -447,36 +571,42 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
   p.n_tiles = (int32_t)((n + block_n - 1) / block_n);
   p.out_dtype = out_dtype;
   p.activation = activation;
+  p.split_k = sk ? split_k : 1;
+  p.counters = sk ? split_workspace : nullptr;
+  p.partials = sk ? reinterpret_cast<float*>(split_workspace + kDecCounterWords) : nullptr;
+  if (sk && split_workspace == nullptr) return set_error(TKX_ERR_INVALID, "a split contraction needs its workspace");
   // Dynamic LDS holds only the four partial tiles of the cross-wave reduction (4 x 16 x 128 f32 = 32 KB;
   // 64 KB for the wide kernel).
   const size_t smem = (size_t)kDecWaves * kDecRows * block_n * 4;
-  const int64_t grid = G * p.n_tiles;
+  const int64_t grid = G * p.n_tiles * p.split_k;
   if (grid > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "too many workgroups");
   // `depth` = steps of loads in flight per wave; deeper pipelines need more registers and allow
   // fewer waves per CU. A step of 16-bit weights takes twice the registers of an int8 one.
   const void* fn;
-  if (sub && rhs_dtype == TKX_F8E4M3FN) {
-    fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEF8, 2, 3, true>)
-                    : reinterpret_cast<const void*>(&decode_kernel<kEF8, 4, 2, true>);
+  if (rhs_dtype == TKX_I4X2 && sub) {
+    fn = depth <= 2 ? decode_fn<kEI4, 2, 4, true>(sk) : decode_fn<kEI4, 4, 3, true>(sk);
+  } else if (rhs_dtype == TKX_I4X2) {
+    // Half the registers of int8 per step in flight: the same occupancy one depth further.
+    fn = depth <= 2   ? decode_fn<kEI4, 2, 4>(sk)
+         : depth <= 4 ? decode_fn<kEI4, 4, 4>(sk)
+                      : reinterpret_cast<const void*>(&decode_kernel<kEI4, 8, 3>);
+  } else if (sub && rhs_dtype == TKX_F8E4M3FN) {
+    fn = depth <= 2 ? decode_fn<kEF8, 2, 3, true>(sk) : decode_fn<kEF8, 4, 2, true>(sk);
   } else if (rhs_dtype == TKX_F8E4M3FN) {
-    fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEF8, 2, 4>)
-                    : reinterpret_cast<const void*>(&decode_kernel<kEF8, 4, 3>);
+    fn = depth <= 2 ? decode_fn<kEF8, 2, 4>(sk) : decode_fn<kEF8, 4, 3>(sk);
   } else if (sub) {
-    fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 2, 3, true>)
-                    : reinterpret_cast<const void*>(&decode_kernel<kEI8, 4, 2, true>);  // (8 deep would spill)
+    fn = depth <= 2 ? decode_fn<kEI8, 2, 3, true>(sk) : decode_fn<kEI8, 4, 2, true>(sk);  // (8 deep would spill)
   } else if (rhs_dtype == TKX_I8 && block_n == 2 * kDecBN) {
     fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 2, 2, false, 16>)
                     : reinterpret_cast<const void*>(&decode_kernel<kEI8, 4, 1, false, 16>);  // (2 workgroups per CU would spill)
   } else if (rhs_dtype == TKX_I8) {
-    fn = depth <= 2   ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 2, 4>)
-         : depth <= 4 ? reinterpret_cast<const void*>(&decode_kernel<kEI8, 4, 3>)
+    fn = depth <= 2   ? decode_fn<kEI8, 2, 4>(sk)
+         : depth <= 4 ? decode_fn<kEI8, 4, 3>(sk)
                       : reinterpret_cast<const void*>(&decode_kernel<kEI8, 8, 2>);
   } else if (rhs_dtype == TKX_BF16) {
-    fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEBF16, 2, 3>)
-                    : reinterpret_cast<const void*>(&decode_kernel<kEBF16, 4, 2>);
+    fn = depth <= 2 ? decode_fn<kEBF16, 2, 3>(sk) : decode_fn<kEBF16, 4, 2>(sk);
   } else {
-    fn = depth <= 2 ? reinterpret_cast<const void*>(&decode_kernel<kEF16, 2, 3>)
-                    : reinterpret_cast<const void*>(&decode_kernel<kEF16, 4, 2>);
+    fn = depth <= 2 ? decode_fn<kEF16, 2, 3>(sk) : decode_fn<kEF16, 4, 2>(sk);
   }
   if (smem + 64 > 64 * 1024) {
     // Past the default limit of dynamic LDS: raised once per (device, kernel).

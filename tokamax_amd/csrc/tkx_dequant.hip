@@ -81,7 +81,65 @@ __global__ __launch_bounds__(kDqThreads) void dequant_kernel(const unsigned char
   }
 }
 
+// Packed int4 <-> int8. A packed row holds two value rows: byte [rr, c] = value [2 rr, c] in bits 0-3 and value
+// [2 rr + 1, c] in bits 4-7. One thread takes 16 columns of one packed row (16 bytes in, two rows of 16 out, or back).
+__global__ __launch_bounds__(kDqThreads) void unpack_int4_kernel(const unsigned char* __restrict__ packed,
+                                                                signed char* __restrict__ out, int64_t packed_rows, int32_t n) {
+  const int chunks = n / 16;
+  const int64_t total = packed_rows * chunks;
+  for (int64_t idx = (int64_t)blockIdx.x * kDqThreads + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * kDqThreads) {
+    const int64_t row = idx / chunks;
+    const int c0 = (int)(idx - row * chunks) * 16;
+    const i32x4 w = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(packed + row * n + c0));
+    i32x4 lo, hi;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      // Per byte: sign-extend bits 0-3 (shift the nibble to the byte's top, arithmetic shift back) and bits 4-7.
+      unsigned l = 0, h = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        l |= ((unsigned)__builtin_amdgcn_sbfe(w[d], 8 * b, 4) & 0xffu) << (8 * b);
+        h |= ((unsigned)__builtin_amdgcn_sbfe(w[d], 8 * b + 4, 4) & 0xffu) << (8 * b);
+      }
+      lo[d] = (int)l;
+      hi[d] = (int)h;
+    }
+    *reinterpret_cast<i32x4*>(out + (2 * row) * n + c0) = lo;
+    *reinterpret_cast<i32x4*>(out + (2 * row + 1) * n + c0) = hi;
+  }
+}
+__global__ __launch_bounds__(kDqThreads) void pack_int4_kernel(const signed char* __restrict__ q, unsigned char* __restrict__ packed,
+                                                              int64_t packed_rows, int32_t n) {
+  const int chunks = n / 16;
+  const int64_t total = packed_rows * chunks;
+  for (int64_t idx = (int64_t)blockIdx.x * kDqThreads + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * kDqThreads) {
+    const int64_t row = idx / chunks;
+    const int c0 = (int)(idx - row * chunks) * 16;
+    const i32x4 lo = *reinterpret_cast<const i32x4*>(q + (2 * row) * n + c0);
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(q + (2 * row + 1) * n + c0);
+    i32x4 w;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) w[d] = (int)(((unsigned)lo[d] & 0x0f0f0f0fu) | (((unsigned)hi[d] & 0x0f0f0f0fu) << 4));
+    *reinterpret_cast<i32x4*>(packed + row * n + c0) = w;
+  }
+}
+
 }  // namespace
+
+int32_t launch_int4_repack(const void* in, void* out, int64_t packed_rows, int64_t n, bool unpack, hipStream_t stream) {
+  const int64_t total = packed_rows * (n / 16);
+  int64_t grid = (total + kDqThreads - 1) / kDqThreads;
+  if (grid > 256 * 16) grid = 256 * 16;
+  if (grid < 1) grid = 1;
+  if (unpack)
+    unpack_int4_kernel<<<dim3((unsigned)grid), dim3(kDqThreads), 0, stream>>>(static_cast<const unsigned char*>(in),
+                                                                              static_cast<signed char*>(out), packed_rows, (int32_t)n);
+  else
+    pack_int4_kernel<<<dim3((unsigned)grid), dim3(kDqThreads), 0, stream>>>(static_cast<const signed char*>(in),
+                                                                            static_cast<unsigned char*>(out), packed_rows, (int32_t)n);
+  TKX_HIP_CHECK(hipGetLastError());
+  return TKX_OK;
+}
 
 int32_t launch_dequant(const void* q, const float* scale, const float* zero_point, void* out, int64_t rows, int64_t n,
                        int64_t t_r, int64_t t_c, int32_t q_dtype, hipStream_t stream) {

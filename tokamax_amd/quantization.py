@@ -4,6 +4,10 @@
 `scale`, `zero_point`, `qtype`; tokamax/_src/quantization.py:25, and its use in
 tokamax/_src/ops/ragged_dot/pallas_mosaic_gpu.py:45-75). `scale.shape[i]` divides
 `qvalue.shape[i]`; each scale entry covers a tile of `qvalue.shape[i] // scale.shape[i]` entries.
+A `QArray` whose `qvalue` is uint8 with `qtype` int4 holds two values per byte along its second-to-last axis (entry
+2 i in bits 0-3, entry 2 i + 1 in bits 4-7); its `shape` is the shape of the values, not of the bytes. `pack_int4`
+makes one from int4 values in int8 storage. (The reference holds int4 as `jnp.int4` arrays and leaves the packing to
+XLA; this is the layout the streaming small-m kernel reads.)
 `AsQArray` (quantization.py:39-78) asks for quantisation on the fly: `as_qarray` runs the absmax
 quantisation kernel of the HIP library; `as_array_or_qarray_without_zero_point` (:85-93) dequantises
 operands that carry a zero point, which no kernel takes.
@@ -33,13 +37,32 @@ class QArray:
     sig = lambda t: None if t is None else (tuple(t.shape), t.dtype, getattr(t, "device", None))
     return ("QArray", sig(self.qvalue), sig(self.scale), sig(self.zero_point), self.qtype)
 
-  shape = property(lambda self: tuple(self.qvalue.shape))
+  @property
+  def packed(self) -> bool:
+    """Two int4 values per byte of `qvalue` along its second-to-last axis."""
+    return self.qvalue.dtype == torch.uint8
+
+  @property
+  def shape(self) -> tuple[int, ...]:
+    """The shape of the values (for packed int4: twice the bytes along the second-to-last axis)."""
+    shape = tuple(self.qvalue.shape)
+    return shape[:-2] + (2 * shape[-2], shape[-1]) if self.packed else shape
+
   dtype = property(lambda self: self.scale.dtype)  # the dtype it dequantises to
   ndim = property(lambda self: len(self.qvalue.shape))
 
   @property
   def scale_tile_shape(self) -> tuple[int, ...]:
-    return tuple(q // s for q, s in zip(self.qvalue.shape, self.scale.shape))
+    return tuple(q // s for q, s in zip(self.shape, self.scale.shape))
+
+  def unpacked(self) -> "QArray":
+    """The same values in int8 storage (on arrays: the unpacking kernel; on shapes: the shape it returns)."""
+    if not self.packed:
+      return self
+    if isinstance(self.qvalue, torch.Tensor):
+      from tokamax_amd.ragged_dot import hip_ops  # pylint: disable=g-import-not-at-top
+      return QArray(hip_ops.unpack_int4(self.qvalue), self.scale, self.zero_point, self.qtype)
+    return QArray(type(self.qvalue)(self.shape, torch.int8), self.scale, self.zero_point, self.qtype)
 
 
 @dataclasses.dataclass(frozen=True, eq=False)
@@ -107,6 +130,18 @@ class AsQArray:
     from tokamax_amd.ragged_dot import hip_ops  # pylint: disable=g-import-not-at-top
     qvalue, scale = hip_ops.quantize(self.value, self.qtype, self.tile_shape)
     return QArray(qvalue, scale, None, self.qtype)
+
+
+def pack_int4(q: QArray) -> QArray:
+  """`q` (int4 values in int8 storage, an even number of entries along the second-to-last axis) with two values per
+  byte along that axis."""
+  if q.packed:
+    return q
+  if q.qvalue.dtype != torch.int8 or q.zero_point is not None:
+    raise NotImplementedError("pack_int4 takes int4 values in int8 storage without a zero point")
+  from tokamax_amd.ragged_dot import hip_ops  # pylint: disable=g-import-not-at-top
+  int4 = getattr(torch, "int4", None)
+  return QArray(hip_ops.pack_int4(q.qvalue), q.scale, None, int4 if int4 is not None else q.qtype)
 
 
 def as_array_or_qarray(x):

@@ -37,7 +37,9 @@ class Config:
 
   (block_m, block_n, block_k, waves_m, waves_n, num_stages) selects a precompiled kernel variant;
   `grid_tile_width` m-tasks share one n-panel of rhs in launch order (L2 reuse);
-  `align_tile` is the row alignment of task starts (the reference's `align_tile`, default 8).
+  `align_tile` is the row alignment of task starts (the reference's `align_tile`, default 8);
+  `split_k` workgroups share the contraction of one output tile (the reference's field of that name; here the
+  streaming small-m kernel, block_m == 16, is the one that takes values above 1).
   """
 
   block_m: int
@@ -48,6 +50,7 @@ class Config:
   num_stages: int = 2
   grid_tile_width: int = 8
   align_tile: int = 8
+  split_k: int = 1
 
   def __post_init__(self):
     for f in dataclasses.fields(self):
@@ -59,7 +62,20 @@ class Config:
 
   def to_kernel_config(self) -> hip_ops.KernelConfig:
     return hip_ops.KernelConfig(self.block_m, self.block_n, self.block_k, self.waves_m, self.waves_n,
-                                self.num_stages, self.grid_tile_width, self.align_tile)
+                                self.num_stages, self.grid_tile_width, self.align_tile, self.split_k)
+
+
+def _streaming_split(tiles: int, contraction: int, block_n: int, depth: int) -> int:
+  """Workgroups per (group, column tile) of the streaming small-m kernel. Unsplit, a launch has `tiles` workgroups;
+  with fewer than one per CU, splitting the contraction until there are 256 measured 1.3x (128 tiles) to 3.5x
+  (16 tiles) faster, 8 splits at most (beyond that the reduction costs more than the parallelism gains); from
+  about 190 tiles on it measured slower at every split (each workgroup's fixed costs outweigh the finer balance)."""
+  if block_n != 128 or depth > 4 or tiles < 1:
+    return 1
+  split = 1
+  while split < 8 and tiles * split * 2 <= 256 and contraction % (128 * split * 2 * min(depth, 4)) == 0:
+    split *= 2
+  return split
 
 
 _ACTIVATION_NAMES = {
@@ -311,6 +327,13 @@ def _route(lhs, rhs, *, dims, precision, rhs_scale, fuse_gateup_activation, pref
   gateup = fuse_gateup_activation is not None
   if (gateup or rhs_scale is not None) and mode != 0:
     raise NotImplementedError("rhs_scale and fuse_gateup_activation need the default dimension numbers.")
+  if isinstance(rhs, QArray) and rhs.packed:
+    # Packed int4 that `_settle_packed_int4` left packed: bf16 lhs x the streaming small-m kernel, scales as they are.
+    if not precision_lib.is_default(lhs.dtype, rhs.dtype, precision):
+      raise NotImplementedError(f"{precision=} not supported.")
+    if preferred_element_type is None:
+      preferred_element_type = torch.promote_types(lhs.dtype, rhs.dtype)
+    return _Route(0, lhs, rhs, torch.bfloat16, torch.uint8, False, False, False, False, preferred_element_type)
   lhs_dt, rhs_dt = _dtype_of(lhs), _dtype_of(rhs)
   widen_lhs = widen_rhs = native = False
   if mode == 0:
@@ -342,12 +365,31 @@ def _route(lhs, rhs, *, dims, precision, rhs_scale, fuse_gateup_activation, pref
   return _Route(mode, lhs, rhs, lhs_dt, rhs_dt, widen_lhs, widen_rhs, native, cast_bf16, preferred_element_type)
 
 
+def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True):
+  """An rhs of packed int4 (two values per byte along k) stays packed when the streaming small-m kernel takes the call:
+  default dimension numbers, a plain bf16 lhs, no bias and no gate-up fusion (`plain`), at most 8 rows per group on
+  average, k % 1024 == 0, n % 16 == 0, one scale per (group, column) or per (group, k-block, column) with blocks of a
+  power of two >= 32 rows. Every other call gets the values unpacked to int8 storage first (then the int8 paths).
+  Works on arrays and on shapes, so the forward pass and the choice of a config settle it alike."""
+  if not (isinstance(rhs, QArray) and rhs.packed):
+    return rhs
+  g, k, n = rhs.shape
+  scale = tuple(rhs.scale.shape)
+  blocks = scale[1] if len(scale) == 3 and scale[0] == g and scale[2] == n and scale[1] >= 1 and k % scale[1] == 0 else None
+  rows = k // blocks if blocks else 0
+  scale_ok = blocks == 1 or (blocks is not None and rows % 32 == 0 and rows & (rows - 1) == 0)
+  streams = (plain and dims == base.DEFAULT_RAGGED_DOT_DIM_NUMS and not isinstance(lhs, (QArray, AsQArray))
+             and lhs.dtype == torch.bfloat16 and rhs.zero_point is None and scale_ok and lhs.shape[0] <= 8 * g
+             and k % 1024 == 0 and n % 16 == 0 and (k // 8) * n < 2**31 and lhs.shape[0] * k * 2 < 2**32)
+  return rhs if streams else rhs.unpacked()
+
+
 def _abstract_operand(x):
   """The abstract form of what `_concrete_operand` returns."""
   if isinstance(x, AsQArray):
     return x.abstract_qarray()
   if isinstance(x, QArray) and x.zero_point is not None:
-    return ShapeDtype(tuple(x.qvalue.shape), torch.bfloat16)
+    return ShapeDtype(tuple(x.shape), torch.bfloat16)
   return x
 
 
@@ -418,7 +460,10 @@ class HipRaggedDot(base.RaggedDot):
       raise NotImplementedError("group_offset needs the default dimension numbers.")
 
     # Quantise / dequantise what the kernels cannot take as it is, then plan the call on shapes and types.
-    route = _route(_concrete_operand(lhs), _concrete_operand(rhs), dims=ragged_dot_dimension_numbers, precision=precision,
+    lhs, rhs = _concrete_operand(lhs), _concrete_operand(rhs)
+    rhs = _settle_packed_int4(lhs, rhs, dims=ragged_dot_dimension_numbers,
+                              plain=rhs_bias is None and fuse_gateup_activation is None and rhs_scale is None)
+    route = _route(lhs, rhs, dims=ragged_dot_dimension_numbers, precision=precision,
                    rhs_scale=rhs_scale, fuse_gateup_activation=fuse_gateup_activation,
                    preferred_element_type=preferred_element_type)
     lhs, rhs, preferred_element_type = route.lhs, route.rhs, route.preferred_element_type
@@ -433,7 +478,7 @@ class HipRaggedDot(base.RaggedDot):
     else:
       lhs_v = lhs
     if isinstance(rhs, QArray):
-      g, k, n = rhs.qvalue.shape
+      g, k, n = rhs.shape
       if not route.widen_rhs:
         # One scale per (group, column): applied in the epilogue. Native k-blocks: [g, k/t_k, n] goes as it is.
         rhs_scale_, rhs_v = rhs.scale, rhs.qvalue
@@ -527,8 +572,11 @@ class HipRaggedDot(base.RaggedDot):
 
   # -- configs ---------------------------------------------------------------------------------
   def _problem(self, ba: op.BoundArguments):
-    lhs, rhs = ba.args[:2]
-    route = _route(_abstract_operand(lhs), _abstract_operand(rhs), dims=ba.kwargs["ragged_dot_dimension_numbers"],
+    lhs, rhs = _abstract_operand(ba.args[0]), _abstract_operand(ba.args[1])
+    rhs = _settle_packed_int4(lhs, rhs, dims=ba.kwargs["ragged_dot_dimension_numbers"],
+                              plain=(ba.kwargs.get("rhs_bias") is None and ba.kwargs.get("fuse_gateup_activation") is None
+                                     and ba.kwargs.get("rhs_scale") is None))
+    route = _route(lhs, rhs, dims=ba.kwargs["ragged_dot_dimension_numbers"],
                    precision=ba.kwargs.get("precision"), rhs_scale=ba.kwargs.get("rhs_scale"),
                    fuse_gateup_activation=ba.kwargs.get("fuse_gateup_activation"),
                    preferred_element_type=ba.kwargs.get("preferred_element_type"))
@@ -555,7 +603,7 @@ class HipRaggedDot(base.RaggedDot):
       variants = variants + [v for v in _variant_table().get((0, key[1], key[2]), []) if v[0] == 16 and v[1] == 128]
     # The streaming small-m kernel (listed with block_m == 16; forward only) needs k % 1024 == 0 and
     # n % 8 == 0, and a weight slice (k/4 rows of n) that a 32-bit buffer offset spans.
-    wbytes = 1 if key[2] == _lib.TKX_I8 else 2
+    wbytes = 1 if key[2] in (_lib.TKX_I8, _lib.TKX_I4X2) else 2
     streaming_ok = (mode in (0, 4) and ba.kwargs.get("rhs_bias") is None and contraction % 1024 == 0 and cols % 8 == 0
                     and (contraction // 4) * cols * wbytes < 2**31)
     usable = [v for v in variants if v[0] != 16 or streaming_ok]
@@ -606,10 +654,12 @@ class HipRaggedDot(base.RaggedDot):
     # time, 8 wide x 4 n-panels needs the fewest distinct operand panels in its L2; 16 wide measured
     # the same speed on the Mixtral shape with 50% more traffic past L2.
     width = 8
+    split_k = 1
     if bm == 16:
       width = 1  # the streaming small-m kernel has no tile order to tune
+      split_k = _streaming_split(num_groups * -(-cols // bn), contraction, bn, ns)
     return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns, grid_tile_width=width,
-                  align_tile=8)
+                  align_tile=8, split_k=split_k)
 
   def _get_autotuning_configs(self, ba: op.BoundArguments) -> set[Config]:
     mode, key = self._problem(ba)[:2]
@@ -619,6 +669,12 @@ class HipRaggedDot(base.RaggedDot):
       for w in widths:
         configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns,
                            grid_tile_width=w))
+      if bm == 16 and bn == 128 and ns <= 4:
+        contraction = self._problem(ba)[5]
+        for split_k in (2, 4, 8):
+          if contraction % (128 * split_k * ns) == 0:
+            configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns,
+                               grid_tile_width=1, split_k=split_k))
     return configs
 
   def supported_on(self, device: torch.device) -> bool:

@@ -20,6 +20,7 @@ _DTYPE_CODE = {
     torch.float16: _lib.TKX_F16,
     torch.float8_e4m3fn: _lib.TKX_F8E4M3FN,
     torch.int8: _lib.TKX_I8,
+    torch.uint8: _lib.TKX_I4X2,  # uint8 storage = int4 packed two to a byte along the second-to-last axis
 }
 
 SCHEDULE_FIELDS = ("group_id", "block_start", "actual_start", "actual_end", "start_within_block", "actual_size")
@@ -44,6 +45,7 @@ class KernelConfig:
   num_stages: int = 2
   grid_tile_width: int = 1
   align_tile: int = 8
+  split_k: int = 1
 
   def to_c(self) -> _lib.TkxConfig:
     return _config_struct(self)
@@ -53,7 +55,7 @@ class KernelConfig:
 def _config_struct(c: "KernelConfig") -> _lib.TkxConfig:
   """The C struct of a config (built once per distinct config; the library only reads it)."""
   return _lib.TkxConfig(c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.grid_tile_width, c.align_tile,
-                        c.num_stages)
+                        c.num_stages, c.split_k)
 
 
 @functools.lru_cache(maxsize=1024)
@@ -93,6 +95,24 @@ def _group_sizes_i32(group_sizes: torch.Tensor) -> torch.Tensor:
 
 def workspace(m: int, num_groups: int, block_m: int, device) -> torch.Tensor:
   return torch.empty(_workspace_words(m, num_groups, block_m), dtype=torch.int32, device=device)
+
+
+_SPLIT_WORKSPACES: dict = {}
+
+
+def split_workspace(m: int, n: int, split_k: int, device) -> torch.Tensor:
+  """The workspace of a streaming-kernel call that splits the contraction over workgroups: arrival counters, which
+  the kernel needs zero on entry and leaves zero, then room for the partial sums. One buffer per (device, stream),
+  zeroed when it is made and grown when a call needs more; calls on one stream are ordered, so they can share it."""
+  device = torch.device(device)
+  nbytes = _lib.load().tkx_ragged_dot_decode_workspace_bytes(m, n, split_k)
+  key = (device.index if device.index is not None else torch.cuda.current_device(),
+         torch.cuda.current_stream(device).cuda_stream)
+  ws = _SPLIT_WORKSPACES.get(key)
+  if ws is None or ws.numel() * 4 < nbytes:
+    ws = torch.zeros(max(nbytes // 4, 1 << 20), dtype=torch.int32, device=device)
+    _SPLIT_WORKSPACES[key] = ws
+  return ws
 
 
 def schedule(group_sizes: torch.Tensor, m: int, block_m: int, align_tile: int = 8):
@@ -138,6 +158,10 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
   lhs, rhs = lhs.contiguous(), rhs.contiguous()
   gs = _group_sizes_i32(group_sizes)
   G, k, n = rhs.shape
+  if rhs.dtype == torch.uint8:
+    k *= 2  # packed int4: a byte row holds two contraction rows
+    if trans_rhs or gateup or config.block_m != 16:
+      raise NotImplementedError("packed int4 weights go to the streaming small-m kernel only; unpack_int4 them first")
   m = lhs.shape[0]
   if group_offset is None:
     if gs.numel() != G:
@@ -181,7 +205,10 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
       raise NotImplementedError("rhs bias must be one value per (group, column)")
   out_cols = k if trans_rhs else n // 2 if gateup else n
   out = torch.empty((m, out_cols), dtype=out_dtype, device=lhs.device)
-  ws = workspace(m, G, config.block_m, lhs.device)
+  if config.block_m == 16 and config.split_k > 1:
+    ws = split_workspace(m, n, config.split_k, lhs.device)
+  else:
+    ws = workspace(m, G, config.block_m, lhs.device)
   cfg = config.to_c()
   with _on_device(lhs.device):
     if rhs_bias is None and not gateup and scale_blocks == 1 and group_offset is None:
@@ -259,6 +286,35 @@ def quantize(x: torch.Tensor, qtype: torch.dtype, tile_shape) -> tuple[torch.Ten
                           ctypes.c_float(_QMAX[qtype]), _stream(x.device))
   _lib.check(st)
   return qvalue, scale
+
+
+def unpack_int4(packed: torch.Tensor) -> torch.Tensor:
+  """int8 [.., 2 r, c] from uint8 [.., r, c] holding two int4 per byte along the second-to-last axis (entry 2 i in
+  bits 0-3, entry 2 i + 1 in bits 4-7, two's complement)."""
+  return _int4_repack(packed, True)
+
+
+def pack_int4(values: torch.Tensor) -> torch.Tensor:
+  """The inverse of `unpack_int4` for int8 values in [-8, 7] (the low four bits of anything else are kept)."""
+  return _int4_repack(values, False)
+
+
+def _int4_repack(x: torch.Tensor, unpack: bool) -> torch.Tensor:
+  _require_cuda(x)
+  want = torch.uint8 if unpack else torch.int8
+  if x.dtype != want or x.dim() < 2 or x.shape[-1] % 16 or (not unpack and x.shape[-2] % 2):
+    raise NotImplementedError(f"expected {want} [.., rows, cols] with cols % 16 == 0 (and an even number of rows to pack),"
+                              f" got {x.dtype} {tuple(x.shape)}")
+  x = x.contiguous()
+  rows = x.shape[-2] * 2 if unpack else x.shape[-2] // 2
+  out = torch.empty((*x.shape[:-2], rows, x.shape[-1]), dtype=torch.int8 if unpack else torch.uint8, device=x.device)
+  packed_rows = (x.numel() if unpack else out.numel()) // x.shape[-1]
+  if packed_rows:
+    lib = _lib.load()
+    with _on_device(x.device):
+      fn = lib.tkx_unpack_int4 if unpack else lib.tkx_pack_int4
+      _lib.check(fn(_ptr(x), _ptr(out), packed_rows, x.shape[-1], _stream(x.device)))
+  return out
 
 
 def dequantize(qvalue: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tensor | None = None) -> torch.Tensor:
