@@ -20,6 +20,7 @@ box's host cores; it is a reported baseline, not the thing measured.
 from __future__ import annotations
 
 import argparse
+import dataclasses
 import json
 import os
 import statistics
@@ -382,7 +383,41 @@ def main():
         ms_per_step=round(m16, 5), gbs=round(nb16 / m16 / 1e6, 2), timing="HIP graph of 24 back-to-back launches",
         roofline=_roofline("hbm", w.flops, nb16, m16, "bf16"),
         kernel_config=[cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages])
-    del w, copies
+    del copies
+
+    # the decode shape with int4 weights packed two to a byte along k (half the weight bytes of int8)
+    packed = []
+    for _ in range(6):
+      q4 = torch.randint(-8, 8, (w.num_groups, w.k, w.n), device=device, dtype=torch.int8, generator=gen)
+      packed.append(tokamax_amd.pack_int4(tokamax_amd.QArray(q4, w.rhs_scale.clone(), None, torch.int4)))
+    del q4
+    cfg = op.bind(w.lhs, packed[0], group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    nb4 = w.nonempty_groups * (w.k * w.n // 2 + w.n * 4) + (w.m * w.k + w.m * w.n) * 2
+    m4 = _time_graph([(lambda r=r: op(w.lhs, r, group_sizes=gs, preferred_element_type=torch.bfloat16)) for r in packed], 24)
+    extras["decode_int4_packed_cold"] = dict(
+        ms_per_step=round(m4, 5), gbs=round(nb4 / m4 / 1e6, 2), timing="HIP graph of 24 back-to-back launches",
+        roofline=_roofline("hbm", w.flops, nb4, m4, "bf16"),
+        kernel_config=[cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages, cfg.split_k])
+    del w, packed
+
+    # few (group, column tile) pairs: 8 experts x 1024 columns, int8 weights, 2 rows per expert. Unsplit that is 64
+    # workgroups on 256 CUs; the heuristics split the contraction 4 ways.
+    G_, k_, n_ = 8, 8192, 1024
+    lhs_ = torch.randn(2 * G_, k_, device=device, generator=gen).to(torch.bfloat16)
+    gs_ = torch.full((G_,), 2, dtype=torch.int32, device=device)
+    few = [tokamax_amd.QArray(torch.randint(-127, 128, (G_, k_, n_), device=device, dtype=torch.int8, generator=gen),
+                              torch.rand(G_, 1, n_, device=device, generator=gen) / 127) for _ in range(6)]
+    nbf = G_ * (k_ * n_ + n_ * 4) + 2 * G_ * (k_ + n_) * 2
+    cfg = op.bind(lhs_, few[0], group_sizes=gs_, preferred_element_type=torch.bfloat16).default_config
+    unsplit = tokamax_amd.HipRaggedDot(config=dataclasses.replace(cfg, split_k=1))
+    t_split = _time_graph([(lambda r=r: op(lhs_, r, group_sizes=gs_, preferred_element_type=torch.bfloat16)) for r in few], 24)
+    t_unsplit = _time_graph([(lambda r=r: unsplit(lhs_, r, group_sizes=gs_, preferred_element_type=torch.bfloat16)) for r in few], 24)
+    extras["decode_few_tiles_split_k"] = dict(
+        shape=dict(m=2 * G_, k=k_, n=n_, num_groups=G_), ms_per_step=round(t_split, 5), ms_per_step_unsplit=round(t_unsplit, 5),
+        gbs=round(nbf / t_split / 1e6, 2), timing="HIP graph of 24 back-to-back launches",
+        roofline=_roofline("hbm", 2 * 2 * G_ * k_ * n_, nbf, t_split, "bf16"),
+        kernel_config=[cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages, cfg.split_k])
+    del lhs_, gs_, few
     result["extras"] = extras
 
   print(json.dumps(result), flush=True)

@@ -325,7 +325,7 @@ def _variant_cases():
 
 
 _TORCH_DTYPE = {_lib.TKX_F32: torch.float32, _lib.TKX_BF16: torch.bfloat16, _lib.TKX_F16: torch.float16,
-                _lib.TKX_F8E4M3FN: torch.float8_e4m3fn, _lib.TKX_I8: torch.int8}
+                _lib.TKX_F8E4M3FN: torch.float8_e4m3fn, _lib.TKX_I8: torch.int8, _lib.TKX_I4X2: torch.uint8}
 
 
 @pytest.mark.parametrize("v", _variant_cases())
@@ -414,6 +414,14 @@ def test_every_kernel_variant_through_c_abi(v, device):
     rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
     rhs_scale = mk((G, 1, n), 0.01).abs() + 1e-3
     rhs_f = O.dequantize(rhs.cpu().numpy(), _np(rhs_scale))
+    lhs = mk((m, k), 1.0).to(lt)
+    lhs_f = _np(lhs)
+    tol = 1e-5
+  elif rt == torch.uint8:  # int4 weights, two to a byte along k
+    values = rng.integers(-8, 8, (G, k, n)).astype(np.int8)
+    rhs = torch.tensor(O.pack_int4(values), device=device)
+    rhs_scale = mk((G, 1, n), 0.1).abs() + 1e-2
+    rhs_f = O.dequantize(values, _np(rhs_scale))
     lhs = mk((m, k), 1.0).to(lt)
     lhs_f = _np(lhs)
     tol = 1e-5
@@ -654,6 +662,49 @@ def test_public_op_on_packed_int4_weights(device):
   gs = torch.full((G,), 2, dtype=torch.int32, device=device)
   lhs = torch.tensor(rng.normal(0, 1, (G * 2, k)).astype(np.float32), device=device).to(torch.bfloat16)
   assert torch.equal(op(lhs, packed, group_sizes=gs, rhs_bias=bias), op(lhs, plain, group_sizes=gs, rhs_bias=bias))
+
+
+@pytest.mark.parametrize("groups,n", [(128, 768), (8, 512)])
+def test_small_m_call_replayed_from_a_captured_graph(groups, n, device):
+  """The call path for serving loops: the public op captured into a HIP graph once (after one eager call on the
+  capture stream, which creates whatever the op keeps per stream) and replayed with new activations and new group
+  sizes written into the captured tensors. Every replay is checked against an eager call, with eager work and
+  synchronisations in between. (8 groups x 512 columns takes the split contraction: its arrival counters must be
+  back at zero after every replay.)"""
+  rng = np.random.default_rng(groups)
+  k = 2048
+  m = 2 * groups
+  q = torch.tensor(rng.integers(-127, 128, (groups, k, n)).astype(np.int8), device=device)
+  scale = torch.tensor((rng.uniform(0.5, 1.5, (groups, 1, n)) / 127).astype(np.float32), device=device)
+  rhs = tokamax_amd.QArray(q, scale)
+  lhs = torch.zeros((m, k), dtype=torch.bfloat16, device=device)
+  gs = torch.zeros((groups,), dtype=torch.int32, device=device)
+  op = tokamax_amd.HipRaggedDot()
+
+  def fill(seed):
+    r = np.random.default_rng(seed)
+    sizes = r.multinomial(m - 3, np.ones(groups) / groups).astype(np.int32)
+    lhs.copy_(torch.tensor(r.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16))
+    gs.copy_(torch.tensor(sizes, device=device))
+
+  fill(0)
+  side = torch.cuda.Stream(device=device)
+  side.wait_stream(torch.cuda.current_stream(device))
+  with torch.cuda.stream(side):
+    op(lhs, rhs, group_sizes=gs, preferred_element_type=torch.bfloat16)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+      out = op(lhs, rhs, group_sizes=gs, preferred_element_type=torch.bfloat16)
+  torch.cuda.current_stream(device).wait_stream(side)
+  for seed in (1, 2, 3):
+    fill(seed)
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    eager = op(lhs, rhs, group_sizes=gs, preferred_element_type=torch.bfloat16)
+    assert torch.equal(out, eager), f"replay {seed}"
+    assert float(eager.float().abs().sum()) > 0
 
 
 def test_public_op_picks_the_wide_small_m_kernel_when_it_fills_the_chip(device):

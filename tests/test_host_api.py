@@ -358,7 +358,8 @@ def test_shipped_mi355x_cache_parses_and_names_compiled_variants():
     assert len(data) >= 4, key
     for cfg in data:
       assert (cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages) in compiled
-    assert data.fastest_config.block_m >= 128  # the tuned workloads are the large prefill / VJP shapes
+    small_m = "[256,2048]" in key.to_json()  # the decode shape: the streaming kernel; the others are large shapes
+    assert (data.fastest_config.block_m == 16) if small_m else (data.fastest_config.block_m >= 128)
 
 
 def test_cache_file_name_and_json_round_trip(tmp_path):

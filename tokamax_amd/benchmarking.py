@@ -69,11 +69,53 @@ def time_on_stream(fn: Callable[[], Any], *, iterations: int = 5, warmup: int = 
   return tuple(times)
 
 
+# Calls shorter than this are timed inside a captured graph: the host needs tens of microseconds to issue one
+# call, so events around eager calls of a shorter kernel measure the host, not the kernel.
+GRAPH_TIMING_BELOW_MS = 0.25
+
+
+def time_in_graph(fn: Callable[[], Any], *, iterations: int = 5, launches: int = 16, device=None) -> tuple[float, ...]:
+  """Device time per call of `fn`, in ms, from `iterations` replays of a HIP graph that holds `launches` back-to-back
+  calls (events around each replay; the reference's timer, CUPTI kernel times, likewise leaves the host out,
+  benchmarking.py:432-471). `fn` must be capturable: device work on the current stream only, no synchronisation."""
+  side = torch.cuda.Stream(device=device)
+  side.wait_stream(torch.cuda.current_stream(device))
+  with torch.cuda.stream(side):
+    fn()  # once outside capture on this stream: whatever the call sets up per stream exists before capture
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+      for _ in range(launches):
+        fn()
+    graph.replay()
+    side.synchronize()
+    times = []
+    for _ in range(iterations):
+      start = torch.cuda.Event(enable_timing=True)
+      end = torch.cuda.Event(enable_timing=True)
+      start.record(side)
+      graph.replay()
+      end.record(side)
+      end.synchronize()
+      times.append(start.elapsed_time(end) / launches)
+  torch.cuda.current_stream(device).wait_stream(side)
+  del graph
+  return tuple(times)
+
+
 def benchmark(fn: Callable[[], Any], *, iterations: int = 5, warmup: int = 1, device=None) -> BenchmarkData:
-  """Runs `fn` once untimed (the "compile"/first-launch cost), then times it."""
+  """Runs `fn` once untimed (the "compile"/first-launch cost), then times it: eagerly, and calls that turn out
+  shorter than GRAPH_TIMING_BELOW_MS again inside a captured graph (`metadata["timing"]` says which)."""
   t0 = time.perf_counter()
   fn()
   torch.cuda.current_stream(device).synchronize()
   first_ms = (time.perf_counter() - t0) * 1e3
   times = time_on_stream(fn, iterations=iterations, warmup=warmup, device=device)
-  return BenchmarkData(compile_time_ms=first_ms, lower_time_ms=0.0, evaluation_times_ms=times)
+  metadata = {"timing": "eager"}
+  if statistics.median(times) < GRAPH_TIMING_BELOW_MS:
+    try:
+      times = time_in_graph(fn, iterations=iterations, device=device)
+      metadata = {"timing": "graph"}
+    except RuntimeError:  # not capturable: the eager times stand
+      torch.cuda.synchronize(device)
+  return BenchmarkData(compile_time_ms=first_ms, lower_time_ms=0.0, evaluation_times_ms=times, metadata=metadata)

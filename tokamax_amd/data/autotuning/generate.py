@@ -1,8 +1,8 @@
 """Regenerates the shipped autotuning cache for the device this runs on.
 
-Times every compiled kernel variant on the benchmark workloads whose
-kernels run long enough for eager timing to separate them (the prefill shapes, the fp8 shape, both
-VJP products and the gate-up fused FFN shape) and writes
+Times every compiled kernel variant on the benchmark workloads (the prefill shapes, the fp8 shape, both
+VJP products, the gate-up fused FFN shape, and the small-m decode shape with int8 and with bf16 weights, whose
+calls are short enough to be timed inside a captured graph) and writes
 `tokamax_amd/data/autotuning/<device kind>/hip_ragged_dot.json`, the file `Op.get_autotuning_cache`
 reads (layout of the reference's tokamax/data/autotuning/<device>/<op>.json).
 
@@ -47,6 +47,13 @@ def bound_arguments(op, device):
   yield "dlhs", op.bind(w.dout, w.rhs, group_sizes=gs, ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS)
   yield "drhs", op.bind(w.lhs, w.dout, group_sizes=gs,
                         ragged_dot_dimension_numbers=base.RAGGED_CONTRACTING_DOT_DIM_NUMS)
+  del w
+  w = workloads.make("decode", device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  yield "decode int8", op.bind(w.lhs, tokamax_amd.QArray(w.rhs, w.rhs_scale), group_sizes=gs,
+                               preferred_element_type=torch.bfloat16)
+  dense = (w.rhs.to(torch.float32) * w.rhs_scale).to(torch.bfloat16)
+  yield "decode bf16", op.bind(w.lhs, dense, group_sizes=gs)
 
 
 def main():
