@@ -42,8 +42,9 @@ PEAK_HBM_GBS = 8000.0
 # this script, each scaled by what the same counter reads for a copy kernel of known size; None
 # where no counter run has been made for the current kernel.
 MEASURED_TRAFFIC_BYTES = {
-    "mixtral": 4.19e9,  # 256x256x32 kernel: 3.60e9 read + 0.60e9 written past L2 (algorithmic: 1.543e9)
-    "decode": 1.838e8,  # streaming int8 kernel: 1.834e8 read + 3.9e5 written (algorithmic: 1.748e8)
+    "mixtral": 4.213e9,  # 256x256x64 split-pipeline kernel: 3.617e9 read + 0.596e9 written past L2 (algorithmic: 1.543e9)
+    "deepseek": 1.2251e10,  # the same kernel on the DeepSeek-V3 shape: 1.1872e10 read + 3.80e8 written
+    "decode": 1.839e8,  # streaming int8 kernel: 1.835e8 read + 3.9e5 written (algorithmic: 1.748e8)
 }
 
 
@@ -231,6 +232,7 @@ def main():
     cfg = op.bind(w.lhs, w.rhs, group_sizes=gs).default_config
     measure("deepseek_v3_prefill_bf16", lambda: op(w.lhs, w.rhs, group_sizes=gs), w.flops, w.algorithmic_bytes(),
             "hbm", "bf16", cfg)
+    extras["deepseek_v3_prefill_bf16"]["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES.get("deepseek")
     extras["deepseek_v3_prefill_bf16"]["pct_mfma_peak"] = round(
         100 * extras["deepseek_v3_prefill_bf16"]["tflops"] / PEAK_TFLOPS["bf16"], 2)
     del w
