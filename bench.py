@@ -275,6 +275,18 @@ def main():
     cfg = op.bind(qlk, qrk, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
     measure("mixtral_prefill_fp8_k_block_scales", lambda: op(qlk, qrk, group_sizes=gs, preferred_element_type=torch.bfloat16),
             w.flops, w.algorithmic_bytes() + (w.m * kb + w.nonempty_groups * kb * w.n) * 4, "mfma", "fp8", cfg)
+    # fp8 x fp8 with the result quantised to fp8 per (row, 128 columns) in the kernel's epilogue, against the same
+    # GEMM with an f32 result followed by the standalone quantisation pass
+    from tokamax_amd.ragged_dot import hip as hip_backend, hip_ops  # pylint: disable=g-import-not-at-top
+    op_q = hip_backend.HipRaggedDot(enable_fused_epilogue_quant=True)
+    cfg = op.bind(ql, qr, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_prefill_fp8_quantised_output", lambda: op_q(ql, qr, group_sizes=gs, preferred_element_type=torch.float8_e4m3fn),
+            w.flops, w.m * w.k + w.nonempty_groups * w.k * w.n + w.m * w.n + w.m * (w.n // 128) * 4, "mfma", "fp8", cfg)
+    def two_passes():
+      dense = op(ql, qr, group_sizes=gs, preferred_element_type=torch.float32)
+      return hip_ops.quantize(dense, torch.float8_e4m3fn, (1, 128))
+    t2, _, _ = _time_steps(two_passes, steps, warm, stream)
+    extras["mixtral_prefill_fp8_quantised_output"]["ms_per_step_gemm_then_quantise_pass"] = round(t2 / steps, 5)
     del w, ql, qr, qlk, qrk
 
     # the Mixtral shape with int8 weights (one f32 scale per (group, column)): the weight stream into LDS is half of bf16's

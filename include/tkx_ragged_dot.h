@@ -141,12 +141,25 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
                            int32_t rhs_dtype, int32_t out_dtype, int32_t mode, int32_t activation,
                            const TkxConfig* config, tkx_stream_t stream);
 
+/* tkx_ragged_dot_fwd (default mode) with the result quantised in the kernel's epilogue: out is fp8 (e4m3fn) [m, n] and
+ * out_scale f32 [m, n / 128], one scale per (row, 128 columns) = absmax / 448 (1 for a run of zeros); values are divided
+ * by their scale and converted with saturation, after the operand scales and the activation. The fused output
+ * quantisation of pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:797-824 with the (1, 128) tile of
+ * pallas_mosaic_gpu_common.py:63-68; bit-identical to tkx_ragged_dot_fwd with an f32 result followed by tkx_quantize.
+ * n % 128 == 0; bf16 x bf16 and fp8 x fp8 tile variants whose wave columns tile 128 output columns (all the 256-column
+ * ones); rows of no group come out as zeros with scale 1. TKX_ERR_UNSUPPORTED otherwise. */
+int32_t tkx_ragged_dot_fwd_fp8_out(const void* lhs, const void* rhs, const int32_t* group_sizes, const float* lhs_scale,
+                                   const float* rhs_scale, void* out, float* out_scale, void* workspace, int64_t m,
+                                   int64_t k, int64_t n, int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype,
+                                   int32_t activation, const TkxConfig* config, tkx_stream_t stream);
+
 /* tkx_ragged_dot_fwd for callers that cannot hand over a workspace they allocated: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference (XLA owns every buffer
  * there). Same arguments and results as tkx_ragged_dot_fwd, without `workspace`: the schedule arrays live in a
  * 256 KiB device array inside the library (one copy per GPU, held until the process ends), which limits
  * tkx_ragged_dot_workspace_bytes(m, num_groups, block_m) to 262144, i.e. about cdiv(m, block_m) + num_groups <= 8100;
- * larger problems return TKX_ERR_UNSUPPORTED. The call allocates and frees nothing. All calls on one GPU share that
+ * larger problems return TKX_ERR_UNSUPPORTED, and so does config->split_k > 1 (its arrival counters need a workspace
+ * that was cleared). The call allocates and frees nothing. All calls on one GPU share that
  * array: two of them that overlap in time (different streams or threads) race; calls on one stream are ordered.
  * The first call on a device looks the array's address up (hipGetSymbolAddress) and should be made outside capture. */
 int32_t tkx_ragged_dot_fwd_static_workspace(const void* lhs, const void* rhs, const int32_t* group_sizes,

@@ -707,6 +707,49 @@ def test_small_m_call_replayed_from_a_captured_graph(groups, n, device):
     assert float(eager.float().abs().sum()) > 0
 
 
+@pytest.mark.parametrize("dtype,cfg", [
+    (torch.bfloat16, (256, 256, 64, 2, 4, 3)), (torch.bfloat16, (256, 256, 32, 2, 4, 4)), (torch.bfloat16, (128, 128, 64, 2, 2, 4)),
+    (torch.bfloat16, (64, 128, 64, 2, 2, 4)), (torch.float8_e4m3fn, (128, 256, 128, 2, 4, 3)), (torch.float8_e4m3fn, (256, 256, 128, 2, 4, 2))])
+def test_fp8_output_quantised_in_the_epilogue(dtype, cfg, device):
+  """tkx_ragged_dot_fwd_fp8_out: values and scales are those of the absmax quantisation (oracle) of the f32 result of
+  the same kernel, bit for bit; rows of no group are zeros with scale 1; ragged groups with an empty one, partial
+  tiles at group boundaries and a column count that is not a multiple of the tile."""
+  variants = {(v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"], v["num_stages"])
+              for v in _lib.variants(0) if v["lhs_dtype"] == hip_ops.dtype_code(dtype)}
+  if cfg not in variants:
+    pytest.skip("variant not compiled")
+  rng = np.random.default_rng(sum(cfg))
+  G, m, k, n = 5, 700, 256, 384
+  gs = np.array([130, 0, 257, 9, 280], np.int32)  # 676 rows, 24 of no group
+  gst = torch.tensor(gs, device=device)
+  kc = hip_ops.KernelConfig(*cfg, grid_tile_width=2)
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(dtype)
+  rhs = torch.tensor(rng.normal(0, 1, (G, k, n)).astype(np.float32), device=device).to(dtype)
+  ls = rs = None
+  if dtype == torch.float8_e4m3fn:
+    ls = torch.tensor(rng.uniform(0.5, 1.5, (m, 1)).astype(np.float32), device=device)
+    rs = torch.tensor(rng.uniform(0.5, 1.5, (G, 1, n)).astype(np.float32), device=device)
+  for act in (None, "silu"):
+    q, s = hip_ops.ragged_dot_fwd_fp8_out(lhs, rhs, gst, config=kc, lhs_scale=ls, rhs_scale=rs, activation=act)
+    dense = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=kc, out_dtype=torch.float32, lhs_scale=ls, rhs_scale=rs, activation=act)
+    wq, wsc = O.quantize_absmax(_np(dense), "fp8", (1, 128))
+    assert np.array_equal(_np(s), wsc), act
+    assert np.array_equal(q.view(torch.uint8).cpu().numpy(), wq), act
+    assert torch.count_nonzero(q[676:].view(torch.uint8)) == 0 and torch.all(s[676:] == 1)
+    q2, s2 = hip_ops.quantize(dense, torch.float8_e4m3fn, (1, 128))  # the standalone pass agrees as well
+    assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s2, s)
+
+
+def test_fp8_output_needs_a_kernel_that_has_it(device):
+  lhs = torch.zeros((32, 1024), dtype=torch.bfloat16, device=device)
+  rhs = torch.zeros((4, 1024, 128), dtype=torch.bfloat16, device=device)
+  gs = torch.full((4,), 8, dtype=torch.int32, device=device)
+  with pytest.raises(NotImplementedError, match="cannot quantise"):
+    hip_ops.ragged_dot_fwd_fp8_out(lhs, rhs, gs, config=hip_ops.KernelConfig(16, 128, 32, 1, 4, 2))
+  with pytest.raises(NotImplementedError, match="128"):
+    hip_ops.ragged_dot_fwd_fp8_out(lhs, rhs[:, :, :64].contiguous(), gs, config=hip_ops.KernelConfig(128, 128, 64, 2, 2, 4))
+
+
 def test_public_op_picks_the_wide_small_m_kernel_when_it_fills_the_chip(device):
   """64 groups x 2048 columns = 512 workgroups of 256 columns (two per CU): the heuristics name the wide
   streaming kernel, and the public entry's result on it matches the oracle."""

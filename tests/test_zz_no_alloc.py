@@ -81,3 +81,16 @@ def test_static_workspace_entry_rejects_schedules_beyond_its_array(device):
                                                _lib.TKX_BF16, _lib.TKX_BF16, _lib.TKX_BF16, 0, 0, ctypes.byref(c),
                                                torch.cuda.current_stream().cuda_stream)
   assert st == _lib.TKX_ERR_UNSUPPORTED and "built-in workspace" in _lib.last_error()
+
+
+def test_static_workspace_entry_rejects_a_split_contraction(device):
+  """split_k > 1 keeps arrival counters in a workspace that must be zero on entry; the built-in array holds the last
+  call's schedule, so the entry point declines instead of reading it."""
+  lib = _lib.load()
+  c = hip_ops.KernelConfig(16, 128, 32, 1, 4, 2, split_k=2).to_c()
+  t = torch.zeros(16, dtype=torch.bfloat16, device=device)  # never touched: the check comes first
+  gs = torch.zeros(4, dtype=torch.int32, device=device)
+  st = lib.tkx_ragged_dot_fwd_static_workspace(t.data_ptr(), t.data_ptr(), gs.data_ptr(), None, None, t.data_ptr(), 8, 1024, 128, 4,
+                                               _lib.TKX_BF16, _lib.TKX_BF16, _lib.TKX_BF16, 0, 0, ctypes.byref(c),
+                                               torch.cuda.current_stream().cuda_stream)
+  assert st == _lib.TKX_ERR_UNSUPPORTED and "split contraction" in _lib.last_error()

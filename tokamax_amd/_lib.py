@@ -42,6 +42,7 @@ EXPORTED_SYMBOLS = (
     "tkx_ragged_dot_decode_counter_bytes",
     "tkx_unpack_int4",
     "tkx_pack_int4",
+    "tkx_ragged_dot_fwd_fp8_out",
 )
 
 
@@ -76,6 +77,8 @@ def _declare(lib):
   lib.tkx_ragged_dot_decode_workspace_bytes.argtypes = [i64, i64, i32]
   lib.tkx_ragged_dot_decode_counter_bytes.restype = i64
   lib.tkx_ragged_dot_decode_counter_bytes.argtypes = [i32]
+  lib.tkx_ragged_dot_fwd_fp8_out.restype = i32
+  lib.tkx_ragged_dot_fwd_fp8_out.argtypes = [vp] * 8 + [i64] * 4 + [i32] * 3 + [cfgp, vp]
   for fn in (lib.tkx_unpack_int4, lib.tkx_pack_int4):
     fn.restype = i32
     fn.argtypes = [vp, vp, i64, i64, vp]

@@ -176,7 +176,7 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
                  const float* lhs_scale, const float* rhs_scale, const float* rhs_bias, void* out, void* workspace,
                  int64_t m, int64_t k, int64_t n, int64_t num_groups, int64_t num_group_sizes, int32_t lhs_dtype,
                  int32_t rhs_dtype, int32_t out_dtype, int32_t mode, int32_t activation, bool gateup,
-                 int64_t rhs_scale_blocks, const TkxConfig* config, tkx_stream_t stream_) {
+                 int64_t rhs_scale_blocks, const TkxConfig* config, tkx_stream_t stream_, float* out_scale = nullptr) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (!lhs || !rhs || !group_sizes || !out || !workspace || !config)
     return set_error(TKX_ERR_INVALID, "null pointer argument");
@@ -187,7 +187,13 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
     return set_error(TKX_ERR_INVALID, "bad sizes m=%lld k=%lld n=%lld G=%lld", (long long)m, (long long)k,
                      (long long)n, (long long)num_groups);
   if (mode != TKX_MODE_DEFAULT && mode != TKX_MODE_TRANS_RHS) return set_error(TKX_ERR_INVALID, "bad mode %d", mode);
-  if (!valid_out_dtype(out_dtype)) return set_error(TKX_ERR_UNSUPPORTED, "out dtype %d not supported", out_dtype);
+  if (out_scale != nullptr) {
+    // fp8 output with one scale per (row, 128 columns), written by the kernel's epilogue.
+    if (out_dtype != TKX_F8E4M3FN || mode != TKX_MODE_DEFAULT || gateup || n % 128 != 0 || (uintptr_t)out_scale % 4 != 0)
+      return set_error(TKX_ERR_UNSUPPORTED, "a quantised result is fp8 (e4m3fn), default mode, no gate-up fusion, n %% 128 == 0");
+  } else if (!valid_out_dtype(out_dtype)) {
+    return set_error(TKX_ERR_UNSUPPORTED, "out dtype %d not supported", out_dtype);
+  }
   if (activation < TKX_ACT_NONE || activation > TKX_ACT_SILU_CLAMP)
     return set_error(TKX_ERR_INVALID, "bad activation %d", activation);
   if (activation > TKX_ACT_SIGMOID && !gateup)
@@ -255,6 +261,9 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
       (rhs_scale && (uintptr_t)rhs_scale % 16 != 0))
     return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
 
+  if (out_scale != nullptr && (v->fn == nullptr || !v->quant_out))
+    return set_error(TKX_ERR_UNSUPPORTED, "this kernel variant cannot quantise its result (bf16 or fp8 forward tiles whose"
+                                          " wave columns tile 128 output columns can)");
   if (v->fn == nullptr) {
     // Streaming decode kernel: one launch, no schedule.
     if (lhs_scale != nullptr) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no lhs scale");
@@ -286,6 +295,7 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
   p.a_scale = lhs_scale;
   p.b_scale = rhs_scale;
   p.b_bias = rhs_bias;
+  p.c_scale = out_scale;
   p.ws = static_cast<const int32_t*>(workspace);
   p.lda = dlhs ? n : k;
   p.ldb = n;
@@ -336,6 +346,16 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
                   num_groups, lhs_dtype, rhs_dtype, out_dtype, mode, activation, false, 1, config, stream);
 }
 
+int32_t tkx_ragged_dot_fwd_fp8_out(const void* lhs, const void* rhs, const int32_t* group_sizes, const float* lhs_scale,
+                                   const float* rhs_scale, void* out, float* out_scale, void* workspace, int64_t m,
+                                   int64_t k, int64_t n, int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype,
+                                   int32_t activation, const TkxConfig* config, tkx_stream_t stream) {
+  if (out_scale == nullptr) return set_error(TKX_ERR_INVALID, "null pointer argument");
+  return fwd_impl(lhs, rhs, group_sizes, nullptr, lhs_scale, rhs_scale, nullptr, out, workspace, m, k, n, num_groups,
+                  num_groups, lhs_dtype, rhs_dtype, TKX_F8E4M3FN, TKX_MODE_DEFAULT, activation, false, 1, config, stream,
+                  out_scale);
+}
+
 int32_t tkx_ragged_dot_fwd_static_workspace(const void* lhs, const void* rhs, const int32_t* group_sizes,
                                             const float* lhs_scale, const float* rhs_scale, void* out, int64_t m, int64_t k,
                                             int64_t n, int64_t num_groups, int32_t lhs_dtype, int32_t rhs_dtype,
@@ -344,6 +364,10 @@ int32_t tkx_ragged_dot_fwd_static_workspace(const void* lhs, const void* rhs, co
   if (config == nullptr) return set_error(TKX_ERR_INVALID, "null pointer argument");
   if (m < 1 || num_groups < 1 || config->block_m < 1)
     return set_error(TKX_ERR_INVALID, "bad sizes m=%lld G=%lld block_m=%d", (long long)m, (long long)num_groups, config->block_m);
+  if (config->split_k > 1)
+    return set_error(TKX_ERR_UNSUPPORTED,
+                     "a split contraction keeps arrival counters in a workspace that the caller cleared; the built-in"
+                     " workspace holds whatever the last call left there (use tkx_ragged_dot_fwd, or split_k = 1)");
   const int64_t words = ws_layout(m, num_groups, config->block_m).words;
   if (words > kScratchWords)
     return set_error(TKX_ERR_UNSUPPORTED,

@@ -75,6 +75,7 @@ struct GemmParams {
   const float* a_scale;  // per A row, or null
   const float* b_scale;  // per (group, column of B), or null
   const float* b_bias;   // per (group, column of B), added after the scales, or null
+  float* c_scale;        // out_dtype fp8: f32 [m_ext, n_ext / 128], one scale per (row, 128 columns) of the result
   const int32_t* ws;
   int64_t lda, ldb, ldc;            // leading dimensions, elements
   int64_t b_group_stride;           // elements between consecutive groups of B (fwd/dlhs)
@@ -98,6 +99,7 @@ struct Variant {
   int32_t smem_bytes;
   const void* fn;  // __global__ void (*)(GemmParams)
   int32_t split_b; // > 0: the split pipeline (that many B stages of block_k / 2; num_stages A stages of block_k)
+  int32_t quant_out;  // 1: the kernel can store fp8 with one scale per (row, 128 columns) (GemmParams::c_scale)
 };
 
 // ---- decode (small-m streaming kernel; int8 or 16-bit weights) -----------------------------------

@@ -525,6 +525,10 @@ struct GemmKernel {
   static constexpr int KA = Mma<EC>::KA;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int TM = WTM / 32, TN = WTN / 32;
+  // Kernels that can quantise their result to fp8 with one scale per (row, 128 columns): the plain forward of bf16 and
+  // fp8 operands, with whole quantisation tiles inside a workgroup's tile and inside or across whole wave columns.
+  static constexpr bool QOUT = MODE == kFwd && (EA == kEBF16 || EA == kEF8) && EB == EA && BN % 128 == 0 &&
+                               (128 % WTN == 0 || WTN % 128 == 0);
   static_assert(MODE != kFwdGlu || TN % 2 == 0, "gate-up tiles pair the two halves of a wave's column blocks");
   static constexpr int TNO = MODE == kFwdGlu ? TN / 2 : TN, WTNO = MODE == kFwdGlu ? WTN / 2 : WTN;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % KA == 0, "tile does not split into 32x32 atoms");
@@ -567,8 +571,14 @@ struct GemmKernel {
         // Tail duty: rows [total_rows, m_ext), and with a group offset the rows before the first
         // group, belong to no group of this call and are defined to be zero.
         const int total_rows = min(ws[1], p.m_ext), lead_rows = min(ws[2], p.m_ext);
-        const int64_t esz = p.out_dtype == TKX_F32 ? 4 : 2;
+        const int64_t esz = p.out_dtype == TKX_F32 ? 4 : p.out_dtype == TKX_F8E4M3FN ? 1 : 2;
         const int64_t lo = (int64_t)total_rows * p.ldc * esz, hi = (int64_t)p.m_ext * p.ldc * esz;
+        if (p.c_scale != nullptr) {
+          // Quantised output: rows of no group are zeros with scale 1, what quantising a row of zeros gives.
+          const int64_t per_row = p.ldc / 128, id = (int64_t)(b - p.real_slots) * THREADS + tid, step = (gridDim.x - p.real_slots) * (int64_t)THREADS;
+          for (int64_t o = total_rows * per_row + id; o < (int64_t)p.m_ext * per_row; o += step) p.c_scale[o] = 1.f;
+          for (int64_t o = id; o < (int64_t)lead_rows * per_row; o += step) p.c_scale[o] = 1.f;
+        }
         unsigned char* c = reinterpret_cast<unsigned char*>(p.C);
         const int64_t nzb = gridDim.x - p.real_slots;
         const i32x4 z = {0, 0, 0, 0};
@@ -1179,9 +1189,52 @@ struct GemmKernel {
       // lays its part of the tile out row-major in its own slice of LDS and reads it back 16 bytes
       // per lane, so that a store instruction writes whole 128-byte (or longer) row segments.
       __syncthreads();  // every wave is done reading the last stage
+      // fp8 output: one scale per (row, 128 columns) = absmax / 448 (1 for a run of zeros), values divided by it and
+      // converted with saturation; the arithmetic of the standalone quantisation pass (launch_quantize), so the two
+      // agree bit for bit. A row's 128 columns lie in 128 / WTN wave columns: each wave reduces its part of every
+      // row (a lane's 16 TN values, then the lane 32 further on, which holds the row's other columns) and the waves
+      // exchange them through LDS.
+      float row_scale[TM][WTN > 128 ? WTN / 128 : 1];
+      if constexpr (QOUT) {
+        if (p.out_dtype == TKX_F8E4M3FN) {
+          constexpr int QW = WTN >= 128 ? 1 : 128 / WTN;   // wave columns per quantisation tile
+          constexpr int QT = WTN > 128 ? WTN / 128 : 1;    // quantisation tiles per wave column
+          constexpr int JT = TN / QT;                      // accumulator blocks per quantisation tile
+          float* xchg = reinterpret_cast<float*>(smem);    // [waves][TM * 32 rows][QT]
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int q = 0; q < QT; ++q) {
+              float mx = 0.f;
+#pragma unroll
+              for (int j = q * JT; j < (q + 1) * JT; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mx = fmaxf(mx, fabsf(acc[i][j][e]));
+              mx = fmaxf(mx, __shfl_xor(mx, 32));
+              if (lane < 32) xchg[(wave * TM * 32 + i * 32 + lane) * QT + q] = mx;
+            }
+          __syncthreads();
+          const int wn0 = wn / QW * QW;  // first wave column of this wave's quantisation tile
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int q = 0; q < QT; ++q) {
+              float mx = 0.f;
+#pragma unroll
+              for (int w = 0; w < QW; ++w) mx = fmaxf(mx, xchg[((wm * WN + wn0 + w) * TM * 32 + i * 32 + (lane & 31)) * QT + q]);
+              const float scale = mx == 0.f ? 1.f : mx / 448.f;
+              row_scale[i][q] = scale;
+              const int row = row0 + row_block(i) * 32 + (lane & 31);
+              const int qcol = (col0 + wn * WTN) / 128 + q;
+              if (lane < 32 && wn == wn0 && row >= act_start && row < act_end && qcol * 128 < p.n_ext)
+                p.c_scale[(int64_t)row * (p.ldc / 128) + qcol] = scale;
+            }
+          __syncthreads();  // the exchange area is part of the staging slices below
+        }
+      }
       auto emit = [&](auto out_tag) {
         constexpr int OUT = decltype(out_tag)::value;
-        constexpr int ESZ = OUT == TKX_F32 ? 4 : 2;
+        constexpr int ESZ = OUT == TKX_F32 ? 4 : OUT == TKX_F8E4M3FN ? 1 : 2;
         constexpr int ROW_BYTES = WTNO * ESZ;
         constexpr int PITCH = ROW_BYTES + 16;                     // keeps 16-byte alignment, staggers banks
         constexpr int WAVE_LDS = (SMEM_BYTES / (WM * WN)) / 16 * 16;
@@ -1211,7 +1264,17 @@ struct GemmKernel {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * t + e];
                 unsigned char* dst = slice + (ii * 32 + (lane & 31)) * PITCH + (j * 32 + 8 * t + 4 * (lane >> 5)) * ESZ;
-                if constexpr (OUT == TKX_F32) {
+                if constexpr (OUT == TKX_F8E4M3FN) {
+                  constexpr int JT = WTN > 128 ? TN / (WTN / 128) : TN;
+                  const float scale = row_scale[i][j / JT];
+                  float q4[4];
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) q4[e] = fminf(fmaxf(v[e] / scale, -448.f), 448.f);
+                  int w = 0;
+                  w = __builtin_amdgcn_cvt_pk_fp8_f32(q4[0], q4[1], w, false);
+                  w = __builtin_amdgcn_cvt_pk_fp8_f32(q4[2], q4[3], w, true);
+                  *reinterpret_cast<int*>(dst) = w;
+                } else if constexpr (OUT == TKX_F32) {
                   *reinterpret_cast<f32x4*>(dst) = v;
                 } else if constexpr (OUT == TKX_BF16) {
                   bf16x4 o;
@@ -1245,7 +1308,9 @@ struct GemmKernel {
       };
       if (p.out_dtype == TKX_BF16) emit(std::integral_constant<int, TKX_BF16>{});
       else if (p.out_dtype == TKX_F32) emit(std::integral_constant<int, TKX_F32>{});
-      else emit(std::integral_constant<int, TKX_F16>{});
+      else if (p.out_dtype == TKX_F8E4M3FN) {
+        if constexpr (QOUT) emit(std::integral_constant<int, TKX_F8E4M3FN>{});  // (the host takes no other kernel there)
+      } else emit(std::integral_constant<int, TKX_F16>{});
     }
   }
 };
@@ -1260,13 +1325,15 @@ __global__ __launch_bounds__(K::THREADS, K::THREADS <= 256 ? 2 : 1) void gemm_en
 #define TKX_VARIANT_SPLIT(MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB)                                           \
   {                                                                                                            \
     MODE, EA, EB, BM, BN, BK, WM, WN, NS, ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>::SMEM_BYTES, \
-        reinterpret_cast<const void*>(&::tkx::gemm_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>>), HB \
+        reinterpret_cast<const void*>(&::tkx::gemm_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>>), HB, \
+        ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>::QOUT ? 1 : 0                                  \
   }
 
 #define TKX_VARIANT(MODE, EA, EB, BM, BN, BK, WM, WN, NS)                                            \
   {                                                                                                  \
     MODE, EA, EB, BM, BN, BK, WM, WN, NS, ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>::SMEM_BYTES, \
-        reinterpret_cast<const void*>(&::tkx::gemm_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>>) \
+        reinterpret_cast<const void*>(&::tkx::gemm_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>>), 0, \
+        ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>::QOUT ? 1 : 0                                   \
   }
 
 }  // namespace tkx

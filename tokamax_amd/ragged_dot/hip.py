@@ -544,6 +544,18 @@ class HipRaggedDot(base.RaggedDot):
         dot_out = activation(dot_out).to(preferred_element_type)
       return dot_out, None
 
+    if (quantize_out and rhs_v.shape[2] % 128 == 0 and rhs_bias is None and group_offset is None
+        and (activation is None or fused is not None) and lhs_v.dtype == rhs_v.dtype
+        and lhs_v.dtype in (torch.bfloat16, torch.float8_e4m3fn)
+        and (rhs_scale_ is None or rhs_scale_.numel() == rhs_v.shape[0] * rhs_v.shape[2])
+        and (lhs_scale is None or lhs_scale.numel() == lhs_v.shape[0])):
+      # Quantised in the GEMM's epilogue, where the kernel has one (bf16 x bf16, fp8 x fp8; tiled variants).
+      try:
+        qvalue, scale = hip_ops.ragged_dot_fwd_fp8_out(lhs_v, rhs_v, gs, config=kcfg, lhs_scale=lhs_scale,
+                                                       rhs_scale=rhs_scale_, activation=fused)
+        return QArray(qvalue, scale, None, torch.float8_e4m3fn), None
+      except NotImplementedError:
+        pass  # (this variant cannot: the pass over an f32 result below)
     if mode == 2:
       dot_out = hip_ops.ragged_dot_drhs(lhs_v, rhs_v, gs, gs.numel(), config=kcfg, out_dtype=preferred_element_type)
     else:
@@ -557,7 +569,7 @@ class HipRaggedDot(base.RaggedDot):
       if unfused:
         dot_out = activation(dot_out).to(preferred_element_type)
     if quantize_out:
-      # (a pass of its own over the f32 result, not yet part of the GEMM's epilogue)
+      # (a pass of its own over the f32 result, where the epilogue above could not do it)
       n_out = dot_out.shape[1]
       sub = 128 if n_out % 128 == 0 else n_out
       qvalue, scale = hip_ops.quantize(dot_out, torch.float8_e4m3fn, (1, sub))

@@ -110,6 +110,10 @@ def split_workspace(m: int, n: int, split_k: int, device) -> torch.Tensor:
          torch.cuda.current_stream(device).cuda_stream)
   ws = _SPLIT_WORKSPACES.get(key)
   if ws is None or ws.numel() * 4 < nbytes:
+    if torch.cuda.is_current_stream_capturing():
+      # (Memory allocated under capture belongs to the graph, and the counters must be zero before its first replay.)
+      raise RuntimeError("the workspace of a split contraction has to exist before a HIP graph is captured: make one"
+                         " call with these shapes on the capture stream first")
     ws = torch.zeros(max(nbytes // 4, 1 << 20), dtype=torch.int32, device=device)
     _SPLIT_WORKSPACES[key] = ws
   return ws
@@ -286,6 +290,43 @@ def quantize(x: torch.Tensor, qtype: torch.dtype, tile_shape) -> tuple[torch.Ten
                           ctypes.c_float(_QMAX[qtype]), _stream(x.device))
   _lib.check(st)
   return qvalue, scale
+
+
+def ragged_dot_fwd_fp8_out(lhs, rhs, group_sizes, *, config: KernelConfig, lhs_scale=None, rhs_scale=None,
+                           activation: str | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+  """(qvalue fp8 [m,n], scale f32 [m, n/128]) of lhs[m,k] . rhs[g,k,n], quantised per (row, 128 columns) in the
+  kernel's epilogue (`tkx_ragged_dot_fwd_fp8_out`): bf16 x bf16 or fp8 x fp8 with one scale per row / per (group,
+  column), n % 128 == 0, a tiled variant. NotImplementedError where the library has no such kernel."""
+  _require_cuda(lhs, rhs, group_sizes, lhs_scale, rhs_scale)
+  lib = _lib.load()
+  if lhs.dim() != 2 or rhs.dim() != 3:
+    raise ValueError(f"expected lhs [m,k] and rhs [g,k,n], got {tuple(lhs.shape)} and {tuple(rhs.shape)}")
+  lhs, rhs = lhs.contiguous(), rhs.contiguous()
+  gs = _group_sizes_i32(group_sizes)
+  G, k, n = rhs.shape
+  m = lhs.shape[0]
+  if gs.numel() != G or lhs.shape[1] != k:
+    raise ValueError("group_sizes / contraction sizes do not fit rhs")
+  if n % 128:
+    raise NotImplementedError("a quantised result needs n % 128 == 0")
+  if lhs_scale is not None:
+    lhs_scale = lhs_scale.to(torch.float32).contiguous().view(-1)
+    if lhs_scale.numel() != m:
+      raise NotImplementedError("lhs scale must be one f32 per row")
+  if rhs_scale is not None:
+    rhs_scale = rhs_scale.to(torch.float32).contiguous().view(-1)
+    if rhs_scale.numel() != G * n:
+      raise NotImplementedError("rhs scale must be one f32 per (group, column)")
+  out = torch.empty((m, n), dtype=torch.float8_e4m3fn, device=lhs.device)
+  out_scale = torch.empty((m, n // 128), dtype=torch.float32, device=lhs.device)
+  ws = workspace(m, G, config.block_m, lhs.device)
+  cfg = config.to_c()
+  with _on_device(lhs.device):
+    st = lib.tkx_ragged_dot_fwd_fp8_out(_ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(out),
+                                        _ptr(out_scale), _ptr(ws), m, k, n, G, dtype_code(lhs.dtype), dtype_code(rhs.dtype),
+                                        _lib.ACTIVATIONS[activation], ctypes.byref(cfg), _stream(lhs.device))
+  _lib.check(st)
+  return out, out_scale
 
 
 def unpack_int4(packed: torch.Tensor) -> torch.Tensor:
