@@ -32,6 +32,9 @@ class QArray:
     if self.qtype is None:
       object.__setattr__(self, "qtype", self.qvalue.dtype)
 
+  def _leaves(self):
+    return (self.qvalue, self.scale, self.zero_point)
+
   def _fast_signature(self):
     """Structural stand-in used by the op's config memo (shapes, dtypes, devices)."""
     sig = lambda t: None if t is None else (tuple(t.shape), t.dtype, getattr(t, "device", None))

@@ -213,9 +213,9 @@ class RaggedDot(op.Op):
 
     if preferred_element_type is not None:
       preferred_element_type = serialization.as_dtype(preferred_element_type)
-    return super().bind(
-        lhs,
-        rhs,
+    return self._bind_all(
+        lhs=lhs,
+        rhs=rhs,
         group_sizes=group_sizes,
         ragged_dot_dimension_numbers=ragged_dot_dimension_numbers,
         precision=precision_lib.canonicalize_precision(precision),

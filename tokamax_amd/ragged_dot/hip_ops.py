@@ -98,6 +98,7 @@ def workspace(m: int, num_groups: int, block_m: int, device) -> torch.Tensor:
 
 
 _SPLIT_WORKSPACES: dict = {}
+_UNUSED_WORKSPACES: dict = {}
 
 
 def split_workspace(m: int, n: int, split_k: int, device) -> torch.Tensor:
@@ -211,6 +212,12 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
   out = torch.empty((m, out_cols), dtype=out_dtype, device=lhs.device)
   if config.block_m == 16 and config.split_k > 1:
     ws = split_workspace(m, n, config.split_k, lhs.device)
+  elif config.block_m == 16:
+    # The streaming kernel without a split touches no workspace (the entry point only wants a pointer): one
+    # allocation per device, not one per call.
+    ws = _UNUSED_WORKSPACES.get(lhs.device)
+    if ws is None:
+      ws = _UNUSED_WORKSPACES[lhs.device] = torch.empty(64, dtype=torch.int32, device=lhs.device)
   else:
     ws = workspace(m, G, config.block_m, lhs.device)
   cfg = config.to_c()
