@@ -69,27 +69,28 @@ const Variant* find_variant(int mode, int a_dtype, int b_dtype, const TkxConfig&
 int dtype_bytes(int d) { return d == TKX_F32 ? 4 : (d == TKX_BF16 || d == TKX_F16) ? 2 : 1; }
 
 // Raises the dynamic-LDS limit of a kernel once per (device, kernel).
-int32_t prepare(const Variant* v) {
+int32_t prepare(const void* fn, int32_t smem_bytes) {
   static std::mutex mu;
   static std::vector<std::pair<int, const void*>> done;
   int dev = 0;
   TKX_HIP_CHECK(hipGetDevice(&dev));
   std::lock_guard<std::mutex> lock(mu);
   for (auto& d : done)
-    if (d.first == dev && d.second == v->fn) return TKX_OK;
-  TKX_HIP_CHECK(hipFuncSetAttribute(v->fn, hipFuncAttributeMaxDynamicSharedMemorySize, v->smem_bytes));
-  done.emplace_back(dev, v->fn);  // (host memory, once per kernel and device)
+    if (d.first == dev && d.second == fn) return TKX_OK;
+  TKX_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes));
+  done.emplace_back(dev, fn);  // (host memory, once per kernel and device)
   return TKX_OK;
 }
 
 int32_t launch(const Variant* v, const GemmParams& p, int64_t grid, hipStream_t stream) {
-  int32_t st = prepare(v);
+  const void* fn = p.c_scale != nullptr ? v->fn_fp8_out : v->fn;
+  int32_t st = prepare(fn, v->smem_bytes);
   if (st != TKX_OK) return st;
   if (grid <= 0 || grid > 0x7fffffffLL) return set_error(TKX_ERR_INVALID, "grid size %lld out of range", (long long)grid);
   GemmParams params = p;
   void* args[] = {&params};
   const int threads = v->waves_m * v->waves_n * 64;
-  TKX_HIP_CHECK(hipLaunchKernel(v->fn, dim3((unsigned)grid), dim3(threads), args, (size_t)v->smem_bytes, stream));
+  TKX_HIP_CHECK(hipLaunchKernel(fn, dim3((unsigned)grid), dim3(threads), args, (size_t)v->smem_bytes, stream));
   return TKX_OK;
 }
 
@@ -261,7 +262,7 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
       (rhs_scale && (uintptr_t)rhs_scale % 16 != 0))
     return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
 
-  if (out_scale != nullptr && (v->fn == nullptr || !v->quant_out))
+  if (out_scale != nullptr && (v->fn == nullptr || v->fn_fp8_out == nullptr))
     return set_error(TKX_ERR_UNSUPPORTED, "this kernel variant cannot quantise its result (bf16 or fp8 forward tiles whose"
                                           " wave columns tile 128 output columns can)");
   if (v->fn == nullptr) {

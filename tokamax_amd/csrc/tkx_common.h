@@ -99,7 +99,7 @@ struct Variant {
   int32_t smem_bytes;
   const void* fn;  // __global__ void (*)(GemmParams)
   int32_t split_b; // > 0: the split pipeline (that many B stages of block_k / 2; num_stages A stages of block_k)
-  int32_t quant_out;  // 1: the kernel can store fp8 with one scale per (row, 128 columns) (GemmParams::c_scale)
+  const void* fn_fp8_out;  // the same kernel storing fp8 with one scale per (row, 128 columns) (GemmParams::c_scale), or null
 };
 
 // ---- decode (small-m streaming kernel; int8 or 16-bit weights) -----------------------------------

@@ -549,7 +549,11 @@ struct GemmKernel {
   static constexpr int SMEM_BYTES = SPLIT ? NS * StageA::BYTES + HB * StageB::BYTES : NS * STAGE_BYTES + (NS + 1) * RING_SLOT;
   static_assert(NS >= 2 && SMEM_BYTES <= 160 * 1024, "stages must fit the 160 KB LDS");
 
+  // QO: the instantiation that stores fp8 with one scale per (row, 128 columns) (QOUT kernels only). It is a kernel of
+  // its own so that the plain one carries none of its code or registers.
+  template <bool QO = false>
   static __device__ __forceinline__ void run(const GemmParams& p, unsigned char* smem) {
+    static_assert(!QO || QOUT, "this kernel has no quantising epilogue");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: all that derives from it is uniform
     const int wm = wave / WN, wn = wave % WN;
@@ -571,9 +575,9 @@ struct GemmKernel {
         // Tail duty: rows [total_rows, m_ext), and with a group offset the rows before the first
         // group, belong to no group of this call and are defined to be zero.
         const int total_rows = min(ws[1], p.m_ext), lead_rows = min(ws[2], p.m_ext);
-        const int64_t esz = p.out_dtype == TKX_F32 ? 4 : p.out_dtype == TKX_F8E4M3FN ? 1 : 2;
+        const int64_t esz = QO ? 1 : p.out_dtype == TKX_F32 ? 4 : 2;
         const int64_t lo = (int64_t)total_rows * p.ldc * esz, hi = (int64_t)p.m_ext * p.ldc * esz;
-        if (p.c_scale != nullptr) {
+        if constexpr (QO) {
           // Quantised output: rows of no group are zeros with scale 1, what quantising a row of zeros gives.
           const int64_t per_row = p.ldc / 128, id = (int64_t)(b - p.real_slots) * THREADS + tid, step = (gridDim.x - p.real_slots) * (int64_t)THREADS;
           for (int64_t o = total_rows * per_row + id; o < (int64_t)p.m_ext * per_row; o += step) p.c_scale[o] = 1.f;
@@ -1195,8 +1199,8 @@ struct GemmKernel {
       // row (a lane's 16 TN values, then the lane 32 further on, which holds the row's other columns) and the waves
       // exchange them through LDS.
       float row_scale[TM][WTN > 128 ? WTN / 128 : 1];
-      if constexpr (QOUT) {
-        if (p.out_dtype == TKX_F8E4M3FN) {
+      if constexpr (QO) {
+        {
           constexpr int QW = WTN >= 128 ? 1 : 128 / WTN;   // wave columns per quantisation tile
           constexpr int QT = WTN > 128 ? WTN / 128 : 1;    // quantisation tiles per wave column
           constexpr int JT = TN / QT;                      // accumulator blocks per quantisation tile
@@ -1306,11 +1310,10 @@ struct GemmKernel {
           }
         }
       };
-      if (p.out_dtype == TKX_BF16) emit(std::integral_constant<int, TKX_BF16>{});
+      if constexpr (QO) emit(std::integral_constant<int, TKX_F8E4M3FN>{});
+      else if (p.out_dtype == TKX_BF16) emit(std::integral_constant<int, TKX_BF16>{});
       else if (p.out_dtype == TKX_F32) emit(std::integral_constant<int, TKX_F32>{});
-      else if (p.out_dtype == TKX_F8E4M3FN) {
-        if constexpr (QOUT) emit(std::integral_constant<int, TKX_F8E4M3FN>{});  // (the host takes no other kernel there)
-      } else emit(std::integral_constant<int, TKX_F16>{});
+      else emit(std::integral_constant<int, TKX_F16>{});
     }
   }
 };
@@ -1321,19 +1324,30 @@ __global__ __launch_bounds__(K::THREADS, K::THREADS <= 256 ? 2 : 1) void gemm_en
   extern __shared__ __attribute__((aligned(1024))) unsigned char tkx_smem[];
   K::run(p, tkx_smem);
 }
+template <class K>
+__global__ __launch_bounds__(K::THREADS, K::THREADS <= 256 ? 2 : 1) void gemm_entry_fp8_out(const GemmParams p) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char tkx_smem[];
+  K::template run<true>(p, tkx_smem);
+}
+// The quantising entry of a kernel that has one, else null.
+template <class K>
+const void* fp8_out_entry() {
+  if constexpr (K::QOUT) return reinterpret_cast<const void*>(&gemm_entry_fp8_out<K>);
+  else return nullptr;
+}
 
 #define TKX_VARIANT_SPLIT(MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB)                                           \
   {                                                                                                            \
     MODE, EA, EB, BM, BN, BK, WM, WN, NS, ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>::SMEM_BYTES, \
         reinterpret_cast<const void*>(&::tkx::gemm_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>>), HB, \
-        ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>::QOUT ? 1 : 0                                  \
+        ::tkx::fp8_out_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>>()                       \
   }
 
 #define TKX_VARIANT(MODE, EA, EB, BM, BN, BK, WM, WN, NS)                                            \
   {                                                                                                  \
     MODE, EA, EB, BM, BN, BK, WM, WN, NS, ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>::SMEM_BYTES, \
         reinterpret_cast<const void*>(&::tkx::gemm_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>>), 0, \
-        ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>::QOUT ? 1 : 0                                   \
+        ::tkx::fp8_out_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>>()                        \
   }
 
 }  // namespace tkx
