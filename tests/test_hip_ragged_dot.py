@@ -750,6 +750,85 @@ def test_fp8_output_needs_a_kernel_that_has_it(device):
     hip_ops.ragged_dot_fwd_fp8_out(lhs, rhs[:, :, :64].contiguous(), gs, config=hip_ops.KernelConfig(128, 128, 64, 2, 2, 4))
 
 
+@pytest.mark.parametrize("seed", range(48))
+def test_random_shapes_through_the_public_op(seed, device):
+  """Seeded random problems (any k and n that are multiples of 8, 1 to 9 groups, empty groups, a tail of rows of no
+  group, 0 to ~300 rows per group) through the public entry points with the heuristics' configs: forward and both
+  cotangent products against the oracle, rows of no group zero."""
+  rng = np.random.default_rng(1000 + seed)
+  dtype = (torch.bfloat16, torch.float16, torch.float32)[seed % 3]
+  G = int(rng.integers(1, 10))
+  k, n = 8 * int(rng.integers(1, 66)), 8 * int(rng.integers(1, 66))
+  scale = (1, 8, 60, 300)[int(rng.integers(0, 4))]
+  gs = rng.integers(0, scale + 1, G).astype(np.int32)
+  gs[rng.random(G) < 0.2] = 0
+  m = int(gs.sum()) + int(rng.integers(0, 20))
+  if m == 0:
+    m, gs[0] = 8, 5
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(dtype)
+  rhs = torch.tensor(rng.normal(0, k ** -0.5, (G, k, n)).astype(np.float32), device=device).to(dtype)
+  dout = torch.tensor(rng.normal(0, 1, (m, n)).astype(np.float32), device=device).to(dtype)
+  gst = torch.tensor(gs, device=device)
+  count, tol, f32 = int(gs.sum()), TOL[dtype], torch.float32
+  out = tokamax_amd.ragged_dot(lhs, rhs, gst, preferred_element_type=f32)
+  _check(out, _ref(lhs, rhs, gs), tol)
+  assert torch.count_nonzero(out[count:]) == 0
+  dlhs = tokamax_amd.ragged_dot_general(dout, rhs, gst, base.TRANS_RHS_RAGGED_DOT_DIM_NUMS, preferred_element_type=f32)
+  _check(dlhs, _ref(dout, rhs, gs, O.TRANS_RHS), tol)
+  assert torch.count_nonzero(dlhs[count:]) == 0
+  drhs = tokamax_amd.ragged_dot_general(lhs, dout, gst, base.RAGGED_CONTRACTING_DOT_DIM_NUMS, preferred_element_type=f32)
+  want = _ref(lhs, dout, gs, O.RAGGED_CONTRACTING)
+  if np.abs(want).max() > 0:
+    _check(drhs, want, tol)
+  assert torch.count_nonzero(drhs[torch.tensor(gs == 0, device=device)]) == 0
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_random_quantised_problems_through_the_public_op(seed, device):
+  """Seeded random problems with quantised operands: int8 weights with one scale per (group, column), per k-block or
+  per (k-block, 16-column block); int8 x int8 and fp8 x fp8 with per-row / per-column scales. Whatever route the
+  call takes (epilogue scales, scaled while widened, folded per k-block, widening pass, streaming kernel), the result
+  is the oracle's contraction of the dequantised operands."""
+  rng = np.random.default_rng(5000 + seed)
+  kind = ("int8_column", "int8_k_blocks", "int8_tiles", "int8_int8", "fp8_fp8")[seed % 5]
+  G = int(rng.integers(1, 8))
+  k, n = 64 * int(rng.integers(1, 9)), 16 * int(rng.integers(1, 30))
+  per_group = (2, 40, 200)[int(rng.integers(0, 3))]
+  gs = rng.integers(0, per_group + 1, G).astype(np.int32)
+  m = int(gs.sum()) + int(rng.integers(0, 9))
+  if m == 0:
+    m, gs[0] = 4, 3
+  gst = torch.tensor(gs, device=device)
+  f32 = torch.float32
+  tensor = lambda x, dt=f32: torch.tensor(np.asarray(x), device=device).to(dt)
+  w8 = rng.integers(-127, 128, (G, k, n)).astype(np.int8)
+  if kind in ("int8_column", "int8_k_blocks", "int8_tiles"):
+    lhs = tensor(rng.normal(0, 1, (m, k)).astype(np.float32), torch.bfloat16)
+    blocks = 1 if kind == "int8_column" else k // 64
+    cols = n // 16 if kind == "int8_tiles" else n
+    scale = (rng.uniform(0.5, 1.5, (G, blocks, cols)) / 127 * k ** -0.5).astype(np.float32)
+    rhs = tokamax_amd.QArray(tensor(w8, torch.int8), tensor(scale))
+    lhs_f, rhs_f, tol = _np(lhs), O.dequantize(w8, scale), 2e-3
+  elif kind == "int8_int8":
+    a8 = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    sa = (rng.uniform(0.5, 1.5, (m, 1)) / 127).astype(np.float32)
+    sb = (rng.uniform(0.5, 1.5, (G, 1, n)) / 127 * k ** -0.5).astype(np.float32)
+    lhs = tokamax_amd.QArray(tensor(a8, torch.int8), tensor(sa))
+    rhs = tokamax_amd.QArray(tensor(w8, torch.int8), tensor(sb))
+    lhs_f, rhs_f, tol = O.dequantize(a8, sa), O.dequantize(w8, sb), 2e-3
+  else:
+    a = tensor(rng.normal(0, 1, (m, k)).astype(np.float32), torch.float8_e4m3fn)
+    b = tensor(rng.normal(0, 1, (G, k, n)).astype(np.float32), torch.float8_e4m3fn)
+    sa = rng.uniform(0.5, 1.5, (m, 1)).astype(np.float32)
+    sb = (rng.uniform(0.5, 1.5, (G, 1, n)) * k ** -0.5).astype(np.float32)
+    lhs, rhs = tokamax_amd.QArray(a, tensor(sa)), tokamax_amd.QArray(b, tensor(sb))
+    lhs_f, rhs_f, tol = _np(a) * sa, _np(b) * sb, 2e-3
+  out = tokamax_amd.ragged_dot(lhs, rhs, gst, preferred_element_type=f32)
+  want = O.ragged_dot(lhs_f, rhs_f, gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, tol)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+
+
 def test_public_op_picks_the_wide_small_m_kernel_when_it_fills_the_chip(device):
   """64 groups x 2048 columns = 512 workgroups of 256 columns (two per CU): the heuristics name the wide
   streaming kernel, and the public entry's result on it matches the oracle."""
