@@ -1042,11 +1042,11 @@ def test_group_offset_shards_add_up_and_follow_the_device_value(device):
   assert torch.equal(total, full)
 
 
-@pytest.mark.parametrize("block_n", [128, 256])
+@pytest.mark.parametrize("block_n,split_k", [(128, 1), (256, 1), (128, 2), (128, 4)])
 @pytest.mark.parametrize("offset,local", [(0, 9), (3, 4), (7, 4), (-2, 5)])
-def test_group_offset_small_m_kernel(offset, local, block_n, device):
-  """`group_offset` in the streaming small-m kernel (int8 weights): the kernel derives its row ranges
-  from the job's sizes and the device-side offset; rows of other groups are zero."""
+def test_group_offset_small_m_kernel(offset, local, block_n, split_k, device):
+  """`group_offset` in the streaming small-m kernel (int8 weights), also with the contraction split over workgroups:
+  the kernel derives its row ranges from the job's sizes and the device-side offset; rows of other groups are zero."""
   rng = np.random.default_rng(60 + offset)
   gs = np.array([3, 0, 5, 17, 1, 0, 16, 2, 4], np.int32)
   k, n = 1024, 464
@@ -1054,7 +1054,7 @@ def test_group_offset_small_m_kernel(offset, local, block_n, device):
   lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
   rhs = torch.tensor(rng.integers(-128, 128, (local, k, n)).astype(np.int8), device=device)
   scale = torch.tensor((np.abs(rng.normal(0, 0.01, (local, 1, n))) + 1e-3).astype(np.float32), device=device)
-  cfg = hip_ops.KernelConfig(16, block_n, 32, 1, 4, 2)
+  cfg = hip_ops.KernelConfig(16, block_n, 32, 1, 4, 2, split_k=split_k)
   goff = torch.tensor([offset], dtype=torch.int32, device=device)
   out = hip_ops.ragged_dot_fwd(lhs, rhs, torch.tensor(gs, device=device), config=cfg, out_dtype=torch.float32,
                                rhs_scale=scale, group_offset=goff)
