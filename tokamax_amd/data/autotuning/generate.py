@@ -1,8 +1,9 @@
 """Regenerates the shipped autotuning cache for the device this runs on.
 
 Times every compiled kernel variant on the benchmark workloads (the prefill shapes, the fp8 shape, both
-VJP products, the gate-up fused FFN shape, and the small-m decode shape with int8 and with bf16 weights, whose
-calls are short enough to be timed inside a captured graph) and writes
+VJP products, the gate-up fused FFN shape, the small-m decode shape with int8 and with bf16 weights, whose
+calls are short enough to be timed inside a captured graph, and the "primary" shapes of the reference's own
+benchmark list) and writes
 `tokamax_amd/data/autotuning/<device kind>/hip_ragged_dot.json`, the file `Op.get_autotuning_cache`
 reads (layout of the reference's tokamax/data/autotuning/<device>/<op>.json).
 
@@ -20,6 +21,7 @@ import tokamax_amd
 from tokamax_amd import op as op_lib
 from tokamax_amd.autotuning import autotuner as autotuner_lib
 from tokamax_amd.autotuning import cache as cache_lib
+from tokamax_amd.ragged_dot import arg_specs
 from tokamax_amd.ragged_dot import base
 from tokamax_amd.ragged_dot import workloads
 
@@ -54,6 +56,14 @@ def bound_arguments(op, device):
                                preferred_element_type=torch.bfloat16)
   dense = (w.rhs.to(torch.float32) * w.rhs_scale).to(torch.bfloat16)
   yield "decode bf16", op.bind(w.lhs, dense, group_sizes=gs)
+  del w, dense
+  # The reference's own benchmark list (tokamax/_src/ops/ragged_dot/arg_specs.py): its "primary" shapes.
+  for spec in arg_specs.ARG_SPECS:
+    if "primary" not in spec.tags:
+      continue
+    args = arg_specs.random_initialize(spec.args, device)
+    yield spec.full_name, op.bind(args["lhs"], args["rhs"], group_sizes=args["group_sizes"])
+    del args
 
 
 def main():
