@@ -7,7 +7,7 @@ benchmark list) and writes
 `tokamax_amd/data/autotuning/<device kind>/hip_ragged_dot.json`, the file `Op.get_autotuning_cache`
 reads (layout of the reference's tokamax/data/autotuning/<device>/<op>.json).
 
-  python -m tokamax_amd.data.autotuning.generate [--iterations N]
+  python -m tokamax_amd.data.autotuning.generate [--iterations N] [--only NAME]
 """
 
 from __future__ import annotations
@@ -57,6 +57,17 @@ def bound_arguments(op, device):
   dense = (w.rhs.to(torch.float32) * w.rhs_scale).to(torch.bfloat16)
   yield "decode bf16", op.bind(w.lhs, dense, group_sizes=gs)
   del w, dense
+  # The Mixtral shape with int8 weights (one scale per (group, column)) under a bf16 lhs, and int8 x int8.
+  w = workloads.make("mixtral", device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  gen = torch.Generator(device=device).manual_seed(1)
+  q8 = tokamax_amd.QArray(torch.randint(-127, 128, tuple(w.rhs.shape), device=device, dtype=torch.int8, generator=gen),
+                          (torch.rand(w.num_groups, 1, w.n, device=device, generator=gen) + 0.5) / (127 * w.k ** 0.5))
+  yield "mixtral int8 weights", op.bind(w.lhs, q8, group_sizes=gs, preferred_element_type=torch.bfloat16)
+  a8 = tokamax_amd.QArray(torch.randint(-127, 128, (w.m, w.k), device=device, dtype=torch.int8, generator=gen),
+                          (torch.rand(w.m, 1, device=device, generator=gen) + 0.5) / 127)
+  yield "mixtral int8 x int8", op.bind(a8, q8, group_sizes=gs, preferred_element_type=torch.bfloat16)
+  del w, q8, a8
   # The reference's own benchmark list (tokamax/_src/ops/ragged_dot/arg_specs.py): its "primary" shapes.
   for spec in arg_specs.ARG_SPECS:
     if "primary" not in spec.tags:
@@ -69,11 +80,15 @@ def bound_arguments(op, device):
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--iterations", type=int, default=10)
+  ap.add_argument("--only", default="", help="tune only the workloads whose name contains this; the other keys of the"
+                  " shipped file are kept as they are")
   args = ap.parse_args()
   device = torch.device("cuda:0")
   op = tokamax_amd.HipRaggedDot()
   tuner = autotuner_lib.Autotuner(iterations=args.iterations, warmup=2)
   for name, ba in bound_arguments(op, device):
+    if args.only not in name:
+      continue
     # The span width stays at the heuristics' value: widths 4..16 time within 1% of each other and the
     # heuristics' width moves the fewest bytes past L2.
     width = ba.heuristics_config.grid_tile_width
