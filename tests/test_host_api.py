@@ -559,3 +559,67 @@ def test_ffi_shim_compiles_to_its_stub_without_the_xla_header(tmp_path):
   text = open(src).read()
   for symbol in ("TkxRaggedDotFwd", "TkxRaggedDotFwdFused", "TkxRaggedDotDrhs"):
     assert f"XLA_FFI_DEFINE_HANDLER_SYMBOL({symbol}," in text
+
+
+def test_heuristics_on_abstract_arguments_split_and_packed_int4():
+  """Config choice needs no GPU: shapes and types only. A launch of the streaming kernel with fewer (group, column
+  tile) pairs than CUs gets its contraction split (8 ways at most, and only as far as k divides); packed int4 weights
+  stay packed (their own variant key) in the small-m regime and count as int8 storage otherwise; a QArray of packed
+  int4 reports the shape of its values."""
+  op = hip.HipRaggedDot()
+  bf16, f32, i8, u8 = torch.bfloat16, torch.float32, torch.int8, torch.uint8
+
+  def config(m, k, n, groups, rhs_dtype=bf16, packed=False):
+    lhs = ShapeDtype((m, k), bf16)
+    gs = ShapeDtype((groups,), torch.int32)
+    if rhs_dtype == bf16:
+      rhs = ShapeDtype((groups, k, n), bf16)
+    else:
+      rhs = tokamax_amd.QArray(ShapeDtype((groups, k // 2 if packed else k, n), rhs_dtype), ShapeDtype((groups, 1, n), f32),
+                               None, getattr(torch, "int4", i8) if packed else None)
+    return op._get_heuristics_config(op.bind(lhs, rhs, group_sizes=gs))
+
+  assert hip._streaming_split(768, 2048, 128, 2) == 1     # a tile or more per CU: never split
+  assert hip._streaming_split(64, 8192, 128, 2) == 4      # up to 256 workgroups
+  assert hip._streaming_split(16, 16384, 128, 4) == 8     # 8 ways at most
+  assert hip._streaming_split(16, 1024, 128, 2) == 4      # as far as k divides: 1024 % (128 * 8 * 2) != 0
+  assert hip._streaming_split(16, 16384, 256, 2) == 1     # the wide form has no split
+  c = config(16, 8192, 1024, 8, i8)
+  assert (c.block_m, c.block_n, c.split_k) == (16, 128, 4)
+  c = config(256, 2048, 768, 128, i8)
+  assert (c.block_m, c.split_k) == (16, 1)
+  packed = tokamax_amd.QArray(ShapeDtype((8, 512, 256), u8), ShapeDtype((8, 1, 256), f32), None, getattr(torch, "int4", i8))
+  assert packed.packed and packed.shape == (8, 1024, 256) and packed.scale_tile_shape == (1, 1024, 1)
+  assert packed.unpacked().qvalue.shape == (8, 1024, 256) and packed.unpacked().qvalue.dtype == i8
+  c = config(16, 1024, 256, 8, u8, packed=True)          # 2 rows per group: the streaming kernel reads the bytes
+  assert c.block_m == 16
+  c = config(4096, 1024, 256, 8, u8, packed=True)        # 512 rows per group: unpacked first, then an int8 tile variant
+  assert c.block_m >= 128
+
+
+def test_bind_without_inspect_matches_the_signature_path():
+  """`RaggedDot.bind` names every parameter of `_fwd` itself and skips `inspect`; the result is the one
+  `Signature.bind` + `apply_defaults` gives, in signature order, and unknown or missing names still fail."""
+  op = hip.HipRaggedDot()
+  lhs, rhs = ShapeDtype((64, 128), torch.bfloat16), ShapeDtype((4, 128, 256), torch.bfloat16)
+  gs = ShapeDtype((4,), torch.int32)
+  ba = op.bind(lhs, rhs, group_sizes=gs, preferred_element_type=torch.float32)
+  names = list(op._fwd_signature.parameters)
+  assert list(ba.arguments) == names
+  slow = op_lib.Op.bind(op, **dict(ba.arguments))
+  assert list(slow.arguments) == names and all(slow.arguments[n] is ba.arguments[n] or slow.arguments[n] == ba.arguments[n]
+                                                for n in names)
+  with pytest.raises(TypeError):
+    op._bind_all(lhs=lhs, rhs=rhs, group_sizes=gs, no_such_parameter=1)
+  with pytest.raises(TypeError):
+    op._bind_all(lhs=lhs, rhs=rhs)
+
+
+def test_config_json_without_split_k_loads_with_the_default():
+  """Cache files written before `split_k` existed name configs without it; they load as split_k = 1."""
+  cfg = hip.Config(**json.loads('{"block_m":16,"block_n":128,"block_k":32,"waves_m":1,"waves_n":4,"num_stages":2,'
+                                '"grid_tile_width":1,"align_tile":8}'))
+  assert cfg.split_k == 1 and cfg.to_kernel_config().split_k == 1
+  assert json.loads(cache_lib.config_to_json(hip.Config(16, 128, 32, 1, 4, 2, 1, 8, 4)))["split_k"] == 4
+  c = cfg.to_kernel_config().to_c()
+  assert ctypes.sizeof(c) == 9 * 4 and c.split_k == 1
