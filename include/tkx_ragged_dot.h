@@ -88,9 +88,22 @@ typedef struct TkxConfig {
                               tkx_ragged_dot_decode_workspace_bytes long with its first
                               tkx_ragged_dot_decode_counter_bytes ZERO on entry; the call leaves them zero, so a caller
                               that keeps one workspace per stream clears it once. */
+  int32_t persistent;      /* the reference's `persistent` (pallas_mosaic_gpu_common.py:55): resident workgroups that share
+                              the work out evenly instead of one workgroup per tile and nothing else. 0: off. 1 (the
+                              streaming small-m kernel: block_m == 16, block_n == 128, num_stages <= 4, one scale per
+                              (group, column), num_groups <= 256, at most 1024 (group, column tile) pairs, k % 32 == 0,
+                              split_k <= 1): the workgroups of EMPTY groups stay and contract a share of the non-empty
+                              tiles' weights, so that every workgroup streams about the same number of bytes; a tile's
+                              parts meet through the workspace, which then is
+                              tkx_ragged_dot_decode_persistent_workspace_bytes long with its first
+                              tkx_ragged_dot_decode_counter_bytes(2) ZERO on entry (left zero on exit, like split_k).
+                              Takes effect when the device holds the whole grid at once and no group has more than 16
+                              rows (decided per launch; otherwise the launch runs as with 0). */
 } TkxConfig;
 
-/* Library / ABI version (major*1000 + minor). 1001: TkxConfig gained split_k (a trailing field). */
+/* Library / ABI version (major*1000 + minor). A change of the major number means that structs passed by pointer
+ * changed size: 2000: TkxConfig gained `persistent` (after `split_k`, which 1001 added); a caller built against an
+ * older header must be rebuilt (the library reads sizeof(TkxConfig) bytes of the config it is handed). */
 int32_t tkx_version(void);
 
 /* Thread-local message for the last non-zero status returned on this thread. */
@@ -104,6 +117,13 @@ const char* tkx_last_error(void);
  * workgroup arrives last, so results are reproducible run to run. */
 int64_t tkx_ragged_dot_decode_workspace_bytes(int64_t m, int64_t n, int32_t split_k);
 int64_t tkx_ragged_dot_decode_counter_bytes(int32_t split_k);
+
+/* Workspace of the streaming small-m kernel in its persistent form (TkxConfig.persistent = 1), whatever the shapes:
+ * the same 256 KiB counter block (zero on entry, zero on exit), then four partial tiles (16 x 128 f32) for each of at
+ * most 1024 workgroups (32.25 MiB in all). A workspace serves split_k and persistent calls alike, one call at a time.
+ * The parts of a tile are added in a fixed order whenever they arrive: results are reproducible run to run (they
+ * differ in the last bits from the plain kernel's, which cuts the contraction elsewhere). */
+int64_t tkx_ragged_dot_decode_persistent_workspace_bytes(void);
 
 /* Number of task slots the schedule uses for (m, G, block_m): cdiv(m, block_m) + G - 1
  * (pallas_mosaic_gpu_kernel_sm90.py:54). */

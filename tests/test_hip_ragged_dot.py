@@ -568,6 +568,108 @@ def test_small_m_kernel_with_the_contraction_split_over_workgroups(case, split_k
   assert torch.equal(out16, out.to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("depth", [2, 4])
+@pytest.mark.parametrize("case", ["sparse", "sparse_many_tiles", "mostly_empty", "ragged_tall", "two_chunks", "all_empty",
+                                  "none_empty", "beyond_m", "one_row"])
+@pytest.mark.parametrize("weights", ["int8", "fp8", "int4"])
+def test_small_m_kernel_persistent_form(case, depth, weights, device):
+  """`persistent = 1`: the workgroups of empty groups contract the tails of the other groups' tiles, whose parts meet
+  through the workspace. Cases in which they help (no group above 16 rows, some groups empty: few or many helpers per
+  tile, one or several column tiles, a partial last tile) and cases that run as the plain kernel does (a tall group, no
+  empty group, nothing but empty groups); sizes that add up to more than m; lhs rows of no group that hold NaN (nothing
+  of them may reach a result); the same bits on a second run; the arrival counters back at zero afterwards."""
+  rng = np.random.default_rng(len(case) + depth)
+  k, n = 1024, 208
+  if case == "sparse":
+    gs = np.array([3, 0, 0, 16, 1, 0, 7, 2, 0, 0, 4], np.int32)
+  elif case == "sparse_many_tiles":
+    gs, k, n = np.array([2, 0, 1, 0, 0, 5, 1, 0], np.int32), 512, 848
+  elif case == "mostly_empty":  # several helper workgroups per tile: tails cut into pieces
+    gs, k = np.zeros(40, np.int32), 2048
+    gs[[3, 17, 38]] = [2, 16, 1]
+  elif case == "ragged_tall":
+    gs = np.array([3, 0, 0, 17, 1, 0, 45, 2], np.int32)
+  elif case == "two_chunks":
+    gs = rng.integers(0, 4, 70).astype(np.int32)
+    gs[[0, 63, 64, 69]] = [0, 2, 0, 5]
+  elif case == "all_empty":
+    gs = np.zeros(5, np.int32)
+  elif case == "none_empty":
+    gs = np.array([1, 4, 16, 2], np.int32)
+  elif case == "beyond_m":
+    gs = np.array([5, 0, 9, 7, 0, 4], np.int32)
+  else:
+    gs, k = np.array([0, 0, 1, 0], np.int32), 128
+  G = len(gs)
+  m = 17 if case == "beyond_m" else int(gs.sum()) + 11
+  clipped = np.diff(np.minimum(np.concatenate([[0], np.cumsum(gs)]), m)).astype(np.int32)
+  lhs_np = rng.normal(0, 1, (m, k)).astype(np.float32)
+  lhs = torch.tensor(lhs_np, device=device).to(torch.bfloat16)
+  lhs[int(clipped.sum()):] = float("nan")
+  scale = torch.tensor((np.abs(rng.normal(0, 0.01, (G, 1, n))) + 1e-3).astype(np.float32), device=device)
+  if weights == "fp8":
+    rhs = torch.tensor(rng.normal(0, 1, (G, k, n)).astype(np.float32), device=device).to(torch.float8_e4m3fn)
+    dense = rhs.float().cpu().numpy() * _np(scale)
+    call_rhs = rhs
+  elif weights == "int4":
+    q4 = torch.tensor(rng.integers(-8, 8, (G, k, n)).astype(np.int8), device=device)
+    dense = O.dequantize(q4.cpu().numpy(), _np(scale))
+    call_rhs = hip_ops.pack_int4(q4)
+  else:
+    rhs = torch.tensor(rng.integers(-128, 128, (G, k, n)).astype(np.int8), device=device)
+    dense = O.dequantize(rhs.cpu().numpy(), _np(scale))
+    call_rhs = rhs
+  cfg = hip_ops.KernelConfig(16, 128, 32, 1, 4, depth, persistent=1)
+  gst = torch.tensor(gs, device=device)
+  out = hip_ops.ragged_dot_fwd(lhs, call_rhs, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale)
+  lhs_f = _np(lhs)
+  lhs_f[int(clipped.sum()):] = 0
+  want = O.ragged_dot(lhs_f, dense, clipped, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, 1e-5)
+  assert torch.count_nonzero(out[int(clipped.sum()):]) == 0
+  ws = hip_ops.split_workspace(m, n, 1, device, persistent=1)
+  counter_words = _lib.load().tkx_ragged_dot_decode_counter_bytes(2) // 4
+  assert ws.numel() * 4 >= _lib.load().tkx_ragged_dot_decode_persistent_workspace_bytes()
+  assert torch.count_nonzero(ws[:counter_words]) == 0
+  again = hip_ops.ragged_dot_fwd(lhs, call_rhs, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale)
+  assert torch.equal(out, again)
+  out16 = hip_ops.ragged_dot_fwd(lhs, call_rhs, gst, config=cfg, out_dtype=torch.bfloat16, rhs_scale=scale)
+  assert torch.equal(out16, out.to(torch.bfloat16))
+
+
+def test_persistent_form_declines_what_it_does_not_take(device):
+  """bf16 weights, scales per k-block, the wide tile, a split contraction on top and more than 256 groups are
+  `NotImplementedError` with `persistent = 1`; the entry point without a workspace declines it too."""
+  rng = np.random.default_rng(2)
+  k, n = 1024, 256
+  mk_lhs = lambda m: torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  gs = torch.tensor([1, 0, 2, 1], dtype=torch.int32, device=device)
+  i8 = torch.tensor(rng.integers(-128, 128, (4, k, n)).astype(np.int8), device=device)
+  one = torch.ones(4, 1, n, device=device)
+  with pytest.raises(NotImplementedError):
+    hip_ops.ragged_dot_fwd(mk_lhs(4), i8.to(torch.bfloat16), gs, config=hip_ops.KernelConfig(16, 128, 32, 1, 4, 2, persistent=1),
+                           out_dtype=torch.float32)
+  with pytest.raises(NotImplementedError):
+    hip_ops.ragged_dot_fwd(mk_lhs(4), i8, gs, config=hip_ops.KernelConfig(16, 128, 32, 1, 4, 2, persistent=1),
+                           out_dtype=torch.float32, rhs_scale=torch.ones(4, 4, n, device=device))
+  with pytest.raises(NotImplementedError):
+    hip_ops.ragged_dot_fwd(mk_lhs(4), i8, gs, config=hip_ops.KernelConfig(16, 256, 32, 1, 4, 2, persistent=1),
+                           out_dtype=torch.float32, rhs_scale=one)
+  with pytest.raises(NotImplementedError):
+    hip_ops.ragged_dot_fwd(mk_lhs(4), i8, gs, config=hip_ops.KernelConfig(16, 128, 32, 1, 4, 2, split_k=2, persistent=1),
+                           out_dtype=torch.float32, rhs_scale=one)
+  with pytest.raises(ValueError):
+    hip_ops.ragged_dot_fwd(mk_lhs(4), i8, gs, config=hip_ops.KernelConfig(16, 128, 32, 1, 4, 2, persistent=3),
+                           out_dtype=torch.float32, rhs_scale=one)
+  G = 300
+  big = torch.zeros(G, 128, 128, dtype=torch.int8, device=device)
+  with pytest.raises(NotImplementedError):
+    hip_ops.ragged_dot_fwd(torch.zeros(8, 128, dtype=torch.bfloat16, device=device), big,
+                           torch.zeros(G, dtype=torch.int32, device=device),
+                           config=hip_ops.KernelConfig(16, 128, 32, 1, 4, 2, persistent=1), out_dtype=torch.float32,
+                           rhs_scale=torch.ones(G, 1, 128, device=device))
+
+
 def test_public_op_splits_the_contraction_when_a_launch_has_few_tiles(device):
   """8 groups x 512 columns = 32 (group, column tile) pairs: the heuristics split the contraction 8 ways (256
   workgroups), the autotuning search space offers the splits that divide k, and the result matches the oracle."""
@@ -1042,19 +1144,22 @@ def test_group_offset_shards_add_up_and_follow_the_device_value(device):
   assert torch.equal(total, full)
 
 
-@pytest.mark.parametrize("block_n,split_k", [(128, 1), (256, 1), (128, 2), (128, 4)])
+@pytest.mark.parametrize("block_n,split_k", [(128, 1), (256, 1), (128, 2), (128, 4), (128, -1), (128, -2)])
 @pytest.mark.parametrize("offset,local", [(0, 9), (3, 4), (7, 4), (-2, 5)])
 def test_group_offset_small_m_kernel(offset, local, block_n, split_k, device):
-  """`group_offset` in the streaming small-m kernel (int8 weights), also with the contraction split over workgroups:
+  """`group_offset` in the streaming small-m kernel (int8 weights), also with the contraction split over workgroups
+  and in the persistent form (split_k -1 here; -2: with no group above 16 rows, so that empty groups' workgroups help):
   the kernel derives its row ranges from the job's sizes and the device-side offset; rows of other groups are zero."""
   rng = np.random.default_rng(60 + offset)
   gs = np.array([3, 0, 5, 17, 1, 0, 16, 2, 4], np.int32)
+  if split_k == -2:
+    gs[3] = 12
   k, n = 1024, 464
   m = int(gs.sum()) + 5
   lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
   rhs = torch.tensor(rng.integers(-128, 128, (local, k, n)).astype(np.int8), device=device)
   scale = torch.tensor((np.abs(rng.normal(0, 0.01, (local, 1, n))) + 1e-3).astype(np.float32), device=device)
-  cfg = hip_ops.KernelConfig(16, block_n, 32, 1, 4, 2, split_k=split_k)
+  cfg = hip_ops.KernelConfig(16, block_n, 32, 1, 4, 2, split_k=max(split_k, 1), persistent=int(split_k < 0))
   goff = torch.tensor([offset], dtype=torch.int32, device=device)
   out = hip_ops.ragged_dot_fwd(lhs, rhs, torch.tensor(gs, device=device), config=cfg, out_dtype=torch.float32,
                                rhs_scale=scale, group_offset=goff)

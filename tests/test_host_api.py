@@ -38,7 +38,7 @@ def test_library_loads_and_exports_every_declared_symbol():
   lib = ctypes.CDLL(_lib.LIB_PATH)
   for name in declared:
     assert hasattr(lib, name), name
-  assert _lib.load().tkx_version() == 1001  # 1001: TkxConfig.split_k
+  assert _lib.load().tkx_version() == 2000  # 2000: TkxConfig.persistent (1001: split_k)
 
 
 def test_workspace_layout_queries():
@@ -622,4 +622,7 @@ def test_config_json_without_split_k_loads_with_the_default():
   assert cfg.split_k == 1 and cfg.to_kernel_config().split_k == 1
   assert json.loads(cache_lib.config_to_json(hip.Config(16, 128, 32, 1, 4, 2, 1, 8, 4)))["split_k"] == 4
   c = cfg.to_kernel_config().to_c()
-  assert ctypes.sizeof(c) == 9 * 4 and c.split_k == 1
+  assert cfg.persistent == 0 and json.loads(cache_lib.config_to_json(hip.Config(16, 128, 32, 1, 4, 2, 1, 8, 1, 3)))["persistent"] == 3
+  assert ctypes.sizeof(c) == 10 * 4 and c.split_k == 1 and c.persistent == 0
+  with pytest.raises(ValueError):
+    hip.Config(16, 128, 32, 1, 4, 2, 1, 8, 1, -1)

@@ -40,6 +40,7 @@ EXPORTED_SYMBOLS = (
     "tkx_ragged_dot_variant",
     "tkx_ragged_dot_decode_workspace_bytes",
     "tkx_ragged_dot_decode_counter_bytes",
+    "tkx_ragged_dot_decode_persistent_workspace_bytes",
     "tkx_unpack_int4",
     "tkx_pack_int4",
     "tkx_ragged_dot_fwd_fp8_out",
@@ -61,6 +62,7 @@ class TkxConfig(ctypes.Structure):
       ("align_tile", ctypes.c_int32),
       ("num_stages", ctypes.c_int32),
       ("split_k", ctypes.c_int32),
+      ("persistent", ctypes.c_int32),
   ]
 
 
@@ -75,6 +77,8 @@ def _declare(lib):
   lib.tkx_version.argtypes = []
   lib.tkx_ragged_dot_decode_workspace_bytes.restype = i64
   lib.tkx_ragged_dot_decode_workspace_bytes.argtypes = [i64, i64, i32]
+  lib.tkx_ragged_dot_decode_persistent_workspace_bytes.restype = i64
+  lib.tkx_ragged_dot_decode_persistent_workspace_bytes.argtypes = []
   lib.tkx_ragged_dot_decode_counter_bytes.restype = i64
   lib.tkx_ragged_dot_decode_counter_bytes.argtypes = [i32]
   lib.tkx_ragged_dot_fwd_fp8_out.restype = i32

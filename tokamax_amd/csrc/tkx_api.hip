@@ -123,7 +123,7 @@ using namespace tkx;
 
 extern "C" {
 
-int32_t tkx_version(void) { return 1001; }
+int32_t tkx_version(void) { return 2000; }
 
 const char* tkx_last_error(void) { return g_err; }
 
@@ -131,6 +131,8 @@ int64_t tkx_ragged_dot_decode_workspace_bytes(int64_t m, int64_t n, int32_t spli
   if (m < 0 || n < 1) return -1;
   return decode_split_workspace_words(m, n, split_k) * 4;
 }
+
+int64_t tkx_ragged_dot_decode_persistent_workspace_bytes(void) { return decode_persistent_workspace_words() * 4; }
 
 int64_t tkx_ragged_dot_decode_counter_bytes(int32_t split_k) {
   return split_k > 1 ? decode_split_counter_words() * 4 : 0;
@@ -271,7 +273,20 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
     if (rhs_bias != nullptr || gateup) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no bias or gate-up fusion");
     if (rhs_scale != nullptr && rhs_dtype != TKX_I8 && rhs_dtype != TKX_F8E4M3FN && rhs_dtype != TKX_I4X2)
       return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes an rhs scale with int8, packed int4 or fp8 weights only");
-    const int32_t split_k = c.split_k > 1 ? c.split_k : 1;  // (0, from a caller that never heard of the field, is 1)
+    const int32_t split_k = c.split_k > 1 ? c.split_k : 1;  // (0 is 1)
+    if (c.persistent != 0) {
+      if (c.persistent != 1) return set_error(TKX_ERR_INVALID, "persistent must be 0 or 1, got %d", c.persistent);
+      if (split_k > 1) return set_error(TKX_ERR_UNSUPPORTED, "persistent and split_k > 1 exclude each other");
+      if (!decode_persistent_supported(lhs_dtype, rhs_dtype, m, k, n, num_groups, rhs_scale ? rhs_scale_blocks : 1, c.block_n,
+                                       c.num_stages))
+        return set_error(TKX_ERR_UNSUPPORTED,
+                         "the persistent decode kernel needs block_n 128, num_stages <= 4, one scale per (group, column),"
+                         " num_groups <= 256, at most 1024 tiles, k %% 32 == 0 and n %% 8 == 0 (k=%lld n=%lld G=%lld scale blocks=%lld)",
+                         (long long)k, (long long)n, (long long)num_groups, (long long)rhs_scale_blocks);
+      return launch_decode(lhs, rhs, rhs_scale, group_sizes, out, m, k, n, num_groups, rhs_dtype, out_dtype, activation,
+                           c.num_stages, 1, c.block_n, group_offset, num_group_sizes, 1, c.persistent,
+                           static_cast<int32_t*>(workspace), stream);
+    }
     if (!decode_supported(lhs_dtype, rhs_dtype, m, k, n, num_groups, rhs_scale ? rhs_scale_blocks : 1, c.block_n,
                           c.num_stages, split_k))
       return set_error(TKX_ERR_UNSUPPORTED,
@@ -281,9 +296,10 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
                        (long long)k, (long long)n, (long long)num_groups, (long long)rhs_scale_blocks, split_k);
     return launch_decode(lhs, rhs, rhs_scale, group_sizes, out, m, k, n, num_groups, rhs_dtype, out_dtype, activation,
                          c.num_stages, rhs_scale ? rhs_scale_blocks : 1, c.block_n, group_offset, num_group_sizes,
-                         split_k, static_cast<int32_t*>(workspace), stream);
+                         split_k, 0, static_cast<int32_t*>(workspace), stream);
   }
 
+  if (c.persistent != 0) return set_error(TKX_ERR_UNSUPPORTED, "persistent belongs to the streaming small-m kernel (block_m == 16)");
   const WsLayout L = ws_layout(m, num_groups, c.block_m);
   int32_t st = launch_schedule(group_sizes, num_groups, group_offset, num_group_sizes, m, c.block_m, c.align_tile,
                                c.grid_tile_width, static_cast<int32_t*>(workspace), L, stream);
@@ -365,10 +381,11 @@ int32_t tkx_ragged_dot_fwd_static_workspace(const void* lhs, const void* rhs, co
   if (config == nullptr) return set_error(TKX_ERR_INVALID, "null pointer argument");
   if (m < 1 || num_groups < 1 || config->block_m < 1)
     return set_error(TKX_ERR_INVALID, "bad sizes m=%lld G=%lld block_m=%d", (long long)m, (long long)num_groups, config->block_m);
-  if (config->split_k > 1)
+  if (config->split_k > 1 || config->persistent != 0)
     return set_error(TKX_ERR_UNSUPPORTED,
-                     "a split contraction keeps arrival counters in a workspace that the caller cleared; the built-in"
-                     " workspace holds whatever the last call left there (use tkx_ragged_dot_fwd, or split_k = 1)");
+                     "a split contraction (split_k > 1, persistent) keeps arrival counters in a workspace that the caller"
+                     " cleared; the built-in workspace holds whatever the last call left there (use tkx_ragged_dot_fwd, or"
+                     " split_k = 1 and persistent = 0)");
   const int64_t words = ws_layout(m, num_groups, config->block_m).words;
   if (words > kScratchWords)
     return set_error(TKX_ERR_UNSUPPORTED,
@@ -604,6 +621,7 @@ int32_t tkx_ragged_dot_variant(int32_t kind, int32_t index, TkxConfig* config, i
     config->align_tile = 8;
     config->num_stages = v.num_stages;
     config->split_k = 1;
+    config->persistent = 0;
     *lhs_dtype = v.a_dtype;
     *rhs_dtype = v.b_dtype;
     *mode = v.mode;

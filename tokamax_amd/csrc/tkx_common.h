@@ -109,16 +109,21 @@ constexpr int32_t kDecodeWideBlockN = 256;  // int8 weights with per-column scal
 // `block_n`: output columns per workgroup, kDecodeBlockN or kDecodeWideBlockN.
 // `depth`: steps of loads in flight per wave. `split_k`: workgroups that share the contraction of one
 // (group, column tile); above 1, `split_workspace` holds decode_split_workspace_words words whose first
-// decode_split_counter_words are zero on entry (and again on exit).
+// decode_split_counter_words are zero on entry (and again on exit). `persistent` > 0: the form in which the
+// workgroups of empty groups take a share of the non-empty tiles' weight bytes; `split_workspace` then holds
+// decode_persistent_workspace_words words with the same zeroed counter block in front.
 bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k, int64_t n, int64_t G,
                       int64_t scale_blocks, int32_t block_n, int32_t depth, int32_t split_k);
+bool decode_persistent_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k, int64_t n, int64_t G,
+                                 int64_t scale_blocks, int32_t block_n, int32_t depth);
+int64_t decode_persistent_workspace_words();
 int64_t decode_split_counter_words();
 int64_t decode_split_workspace_words(int64_t m, int64_t n, int32_t split_k);
 int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
                       int64_t m, int64_t k, int64_t n, int64_t G, int32_t rhs_dtype, int32_t out_dtype,
                       int32_t activation, int32_t depth, int64_t scale_blocks, int32_t block_n,
-                      const int32_t* group_offset, int64_t num_global, int32_t split_k, int32_t* split_workspace,
-                      hipStream_t stream);
+                      const int32_t* group_offset, int64_t num_global, int32_t split_k, int32_t persistent,
+                      int32_t* split_workspace, hipStream_t stream);
 
 // ---- packed int4 (TKX_I4X2) <-> int8: `packed_rows` rows of n bytes against 2 * packed_rows rows of n values ----
 int32_t launch_int4_repack(const void* in, void* out, int64_t packed_rows, int64_t n, bool unpack, hipStream_t stream);

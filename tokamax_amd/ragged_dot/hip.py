@@ -39,7 +39,10 @@ class Config:
   `grid_tile_width` m-tasks share one n-panel of rhs in launch order (L2 reuse);
   `align_tile` is the row alignment of task starts (the reference's `align_tile`, default 8);
   `split_k` workgroups share the contraction of one output tile (the reference's field of that name; here the
-  streaming small-m kernel, block_m == 16, is the one that takes values above 1).
+  streaming small-m kernel, block_m == 16, is the one that takes values above 1);
+  `persistent` (the reference's flag of that name, pallas_mosaic_gpu_common.py:55; here a count): above 0 the streaming
+  small-m kernel runs as that many resident workgroups per compute unit, each with an equal share of the weight bytes
+  of the non-empty tiles, instead of one workgroup per (group, column tile).
   """
 
   block_m: int
@@ -51,18 +54,19 @@ class Config:
   grid_tile_width: int = 8
   align_tile: int = 8
   split_k: int = 1
+  persistent: int = 0
 
   def __post_init__(self):
     for f in dataclasses.fields(self):
       v = getattr(self, f.name)
-      if not isinstance(v, int) or isinstance(v, bool) or v <= 0:
+      if not isinstance(v, int) or isinstance(v, bool) or v < (0 if f.name == "persistent" else 1):
         raise ValueError(f"Config.{f.name} must be a positive int, got {v!r}")
     if self.block_m % 8 != 0:
       raise ValueError(f"Config.block_m must be a multiple of 8, got {self.block_m}")
 
   def to_kernel_config(self) -> hip_ops.KernelConfig:
     return hip_ops.KernelConfig(self.block_m, self.block_n, self.block_k, self.waves_m, self.waves_n,
-                                self.num_stages, self.grid_tile_width, self.align_tile, self.split_k)
+                                self.num_stages, self.grid_tile_width, self.align_tile, self.split_k, self.persistent)
 
 
 def _streaming_split(tiles: int, contraction: int, block_n: int, depth: int) -> int:
@@ -682,11 +686,16 @@ class HipRaggedDot(base.RaggedDot):
         configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns,
                            grid_tile_width=w))
       if bm == 16 and bn == 128 and ns <= 4:
-        contraction = self._problem(ba)[5]
+        _, _, num_groups, _, cols, contraction, _ = self._problem(ba)
         for split_k in (2, 4, 8):
           if contraction % (128 * split_k * ns) == 0:
             configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns,
                                grid_tile_width=1, split_k=split_k))
+        # The persistent form (empty groups' workgroups help): one-byte weights with one scale per (group, column).
+        if (mode == 0 and key[2] in (_lib.TKX_I8, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2) and num_groups <= 256
+            and num_groups * -(-cols // 128) <= 1024):
+          configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns,
+                             grid_tile_width=1, persistent=1))
     return configs
 
   def supported_on(self, device: torch.device) -> bool:

@@ -46,6 +46,7 @@ class KernelConfig:
   grid_tile_width: int = 1
   align_tile: int = 8
   split_k: int = 1
+  persistent: int = 0
 
   def to_c(self) -> _lib.TkxConfig:
     return _config_struct(self)
@@ -55,7 +56,7 @@ class KernelConfig:
 def _config_struct(c: "KernelConfig") -> _lib.TkxConfig:
   """The C struct of a config (built once per distinct config; the library only reads it)."""
   return _lib.TkxConfig(c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.grid_tile_width, c.align_tile,
-                        c.num_stages, c.split_k)
+                        c.num_stages, c.split_k, c.persistent)
 
 
 @functools.lru_cache(maxsize=1024)
@@ -98,15 +99,24 @@ def workspace(m: int, num_groups: int, block_m: int, device) -> torch.Tensor:
 
 
 _SPLIT_WORKSPACES: dict = {}
+_SUPERSEDED_WORKSPACES: list = []
 _UNUSED_WORKSPACES: dict = {}
 
 
-def split_workspace(m: int, n: int, split_k: int, device) -> torch.Tensor:
-  """The workspace of a streaming-kernel call that splits the contraction over workgroups: arrival counters, which
-  the kernel needs zero on entry and leaves zero, then room for the partial sums. One buffer per (device, stream),
-  zeroed when it is made and grown when a call needs more; calls on one stream are ordered, so they can share it."""
+def split_workspace(m: int, n: int, split_k: int, device, persistent: int = 0) -> torch.Tensor:
+  """The workspace of a streaming-kernel call that completes tiles across workgroups (a split contraction, or the
+  persistent form): arrival counters, which the kernel needs zero on entry and leaves zero, then room for the partial
+  sums. One buffer per (device, stream), zeroed when it is made and replaced by a larger one when a call needs more;
+  calls on one stream are ordered, so they can share it.
+
+  A buffer that was handed out is never released: a HIP graph captured earlier holds its address, and replays must
+  keep finding counters that nobody else writes (superseded buffers stay referenced until the process ends). The
+  buffer belongs to the stream the call was made (or captured) on: a captured graph must be replayed on a stream that
+  no other split or persistent call uses at the same time, since they would share one set of counters."""
   device = torch.device(device)
-  nbytes = _lib.load().tkx_ragged_dot_decode_workspace_bytes(m, n, split_k)
+  lib = _lib.load()
+  nbytes = (lib.tkx_ragged_dot_decode_persistent_workspace_bytes() if persistent
+            else lib.tkx_ragged_dot_decode_workspace_bytes(m, n, split_k))
   key = (device.index if device.index is not None else torch.cuda.current_device(),
          torch.cuda.current_stream(device).cuda_stream)
   ws = _SPLIT_WORKSPACES.get(key)
@@ -115,6 +125,8 @@ def split_workspace(m: int, n: int, split_k: int, device) -> torch.Tensor:
       # (Memory allocated under capture belongs to the graph, and the counters must be zero before its first replay.)
       raise RuntimeError("the workspace of a split contraction has to exist before a HIP graph is captured: make one"
                          " call with these shapes on the capture stream first")
+    if ws is not None:
+      _SUPERSEDED_WORKSPACES.append(ws)
     ws = torch.zeros(max(nbytes // 4, 1 << 20), dtype=torch.int32, device=device)
     _SPLIT_WORKSPACES[key] = ws
   return ws
@@ -210,8 +222,8 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
       raise NotImplementedError("rhs bias must be one value per (group, column)")
   out_cols = k if trans_rhs else n // 2 if gateup else n
   out = torch.empty((m, out_cols), dtype=out_dtype, device=lhs.device)
-  if config.block_m == 16 and config.split_k > 1:
-    ws = split_workspace(m, n, config.split_k, lhs.device)
+  if config.block_m == 16 and (config.split_k > 1 or config.persistent > 0):
+    ws = split_workspace(m, n, config.split_k, lhs.device, config.persistent)
   elif config.block_m == 16:
     # The streaming kernel without a split touches no workspace (the entry point only wants a pointer): one
     # allocation per device, not one per call.
