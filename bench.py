@@ -38,14 +38,34 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "f32": 157.3}  # (int8: TOP/s)
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this script, each scaled by what the same counter reads for a copy kernel of known size; None
-# where no counter run has been made for the current kernel.
-MEASURED_TRAFFIC_BYTES = {
-    "mixtral": 4.213e9,  # 256x256x64 split-pipeline kernel: 3.617e9 read + 0.596e9 written past L2 (algorithmic: 1.543e9)
-    "deepseek": 1.2251e10,  # the same kernel on the DeepSeek-V3 shape: 1.1872e10 read + 3.80e8 written
-    "decode": 1.839e8,  # streaming int8 kernel: 1.835e8 read + 3.9e5 written (algorithmic: 1.748e8)
-}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_all_workloads.hbm_traffic_pmc.txt")
+
+
+def _measured_traffic(kernel_prefix, workload_prefix):
+  """HBM-side bytes per launch (read + written) of a kernel on a workload, from the committed summary of the
+  rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (each counter scaled by what it reads for a copy kernel
+  of known size). The row is found by the kernel's template arguments and the workload's name: None when the summary
+  has no row for the kernel the current config selects (a changed kernel must not inherit an old figure)."""
+  try:
+    with open(TRAFFIC_PROFILE) as f:
+      lines = f.read().splitlines()
+  except OSError:
+    return None
+  for line in lines:
+    cols = [c for c in line.split("  ") if c.strip()]
+    if len(cols) < 9 or not cols[0].strip().startswith(kernel_prefix) or not cols[1].strip().startswith(workload_prefix):
+      continue
+    try:
+      read_mb, write_mb = float(cols[4]), float(cols[7])
+    except ValueError:
+      continue
+    return (read_mb + write_mb) * 1e6
+  return None
+
+
+def _gemm_kernel_prefix(mode, lhs_code, rhs_code, cfg):
+  return (f"GemmKernel<{mode}, {lhs_code}, {rhs_code}, {cfg.block_m}, {cfg.block_n}, {cfg.block_k}, {cfg.waves_m}, "
+          f"{cfg.waves_n}, {cfg.num_stages},")
 
 
 def _time_steps(fn, steps, warmup, stream):
@@ -201,7 +221,7 @@ def main():
                                                             "grid_tile_width")},
       },
       "roofline": _roofline("mfma", w.flops, w.algorithmic_bytes(), gemm_ms, "bf16",
-                            traffic=MEASURED_TRAFFIC_BYTES.get("mixtral")),
+                            traffic=_measured_traffic(_gemm_kernel_prefix(0, 1, 1, config), "Mixtral prefill bf16 fwd")),
       "schedule_kernel_ms": round(sched_ms, 5),
       "ms_median_step": round(statistics.median(per), 5),
       "ms_min_step": round(min(per), 5),
@@ -232,7 +252,8 @@ def main():
     cfg = op.bind(w.lhs, w.rhs, group_sizes=gs).default_config
     measure("deepseek_v3_prefill_bf16", lambda: op(w.lhs, w.rhs, group_sizes=gs), w.flops, w.algorithmic_bytes(),
             "hbm", "bf16", cfg)
-    extras["deepseek_v3_prefill_bf16"]["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES.get("deepseek")
+    extras["deepseek_v3_prefill_bf16"]["roofline"]["traffic"] = _measured_traffic(
+        _gemm_kernel_prefix(0, 1, 1, cfg), "DeepSeek-V3 prefill bf16 fwd")
     extras["deepseek_v3_prefill_bf16"]["pct_mfma_peak"] = round(
         100 * extras["deepseek_v3_prefill_bf16"]["tflops"] / PEAK_TFLOPS["bf16"], 2)
     del w
@@ -253,7 +274,8 @@ def main():
                           roofline=_roofline("hbm", w.flops, w.algorithmic_bytes(), m_, "bf16", traffic=traffic),
                           kernel_config=[cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages])
 
-    measure_graph("decode_int8_cold", [decode_call(q) for q in copies], MEASURED_TRAFFIC_BYTES.get("decode"))
+    measure_graph("decode_int8_cold", [decode_call(q) for q in copies],
+                  _measured_traffic(f"decode_kernel<4, {cfg.num_stages},", "int8-weight decode") if not cfg.persistent else None)
     measure_graph("decode_int8_warm", [decode_call(copies[0])])
     t, p, wall = _time_steps(decode_call(copies[0]), steps, warm, stream)
     extras["decode_int8_cold"]["eager_wall_ms_per_call"] = round(wall / steps, 5)  # host dispatch included

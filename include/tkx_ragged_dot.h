@@ -125,6 +125,11 @@ int64_t tkx_ragged_dot_decode_counter_bytes(int32_t split_k);
  * differ in the last bits from the plain kernel's, which cuts the contraction elsewhere). */
 int64_t tkx_ragged_dot_decode_persistent_workspace_bytes(void);
 
+/* Clears the counter block (the first tkx_ragged_dot_decode_counter_bytes(2) bytes) of such a workspace with a small
+ * fill kernel on `stream`: for callers whose workspace is not theirs to keep between calls (an XLA FFI handler gets a
+ * fresh, uninitialised result buffer per call) and for code under graph capture. No counterpart in the reference. */
+int32_t tkx_ragged_dot_decode_clear_counters(void* workspace, tkx_stream_t stream);
+
 /* Number of task slots the schedule uses for (m, G, block_m): cdiv(m, block_m) + G - 1
  * (pallas_mosaic_gpu_kernel_sm90.py:54). */
 int64_t tkx_ragged_dot_tid_size(int64_t m, int64_t num_groups, int32_t block_m);
@@ -162,10 +167,12 @@ int32_t tkx_ragged_dot_fwd(const void* lhs, const void* rhs, const int32_t* grou
                            const TkxConfig* config, tkx_stream_t stream);
 
 /* tkx_ragged_dot_fwd (default mode) with the result quantised in the kernel's epilogue: out is fp8 (e4m3fn) [m, n] and
- * out_scale f32 [m, n / 128], one scale per (row, 128 columns) = absmax / 448 (1 for a run of zeros); values are divided
- * by their scale and converted with saturation, after the operand scales and the activation. The fused output
- * quantisation of pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:797-824 with the (1, 128) tile of
- * pallas_mosaic_gpu_common.py:63-68; bit-identical to tkx_ragged_dot_fwd with an f32 result followed by tkx_quantize.
+ * out_scale f32 [m, n / 128], one scale per (row, 128 columns) = absmax / 448 (1 for a run of zeros); values are
+ * multiplied by the reciprocal of their scale and converted with saturation, after the operand scales and the
+ * activation: the arithmetic of the fused output quantisation of pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:797-824
+ * (`q = acc * (1.0 / out_scale)`), with the (1, 128) tile of pallas_mosaic_gpu_common.py:63-68. The scales are those of
+ * tkx_ragged_dot_fwd with an f32 result followed by tkx_quantize; the values can differ from that pass, which divides,
+ * by one fp8 step where a quotient lies on a rounding boundary.
  * n % 128 == 0; bf16 x bf16 and fp8 x fp8 tile variants whose wave columns tile 128 output columns (all the 256-column
  * ones); rows of no group come out as zeros with scale 1. TKX_ERR_UNSUPPORTED otherwise. */
 int32_t tkx_ragged_dot_fwd_fp8_out(const void* lhs, const void* rhs, const int32_t* group_sizes, const float* lhs_scale,
@@ -181,7 +188,9 @@ int32_t tkx_ragged_dot_fwd_fp8_out(const void* lhs, const void* rhs, const int32
  * larger problems return TKX_ERR_UNSUPPORTED, and so does config->split_k > 1 (its arrival counters need a workspace
  * that was cleared). The call allocates and frees nothing. All calls on one GPU share that
  * array: two of them that overlap in time (different streams or threads) race; calls on one stream are ordered.
- * The first call on a device looks the array's address up (hipGetSymbolAddress) and should be made outside capture. */
+ * The first call on a device looks the array's address up (hipGetSymbolAddress), and the first call of a kernel on a
+ * device raises that kernel's limit of dynamic LDS (hipFuncSetAttribute): both are remembered in fixed tables (no host
+ * allocation either) and should happen outside capture, i.e. make one eager call per (device, config) first. */
 int32_t tkx_ragged_dot_fwd_static_workspace(const void* lhs, const void* rhs, const int32_t* group_sizes,
                                             const float* lhs_scale, const float* rhs_scale, void* out, int64_t m,
                                             int64_t k, int64_t n, int64_t num_groups, int32_t lhs_dtype,
@@ -263,18 +272,24 @@ int32_t tkx_pack_int4(const void* values, void* packed, int64_t packed_rows, int
 
 /* Quantisation on the fly (AsQArray.as_qarray, quantization.py:65-78: qwix.quantize with the "absmax" calibration), the
  * inverse of tkx_dequantize:
- *   scale[R, C] = max |x[r, c]| over the tile (R, C) / qmax   (1 where the tile is all zero)
+ *   scale[R, C] = max |x[r, c]| over the tile (R, C) / bound   (1 where the tile is all zero)
  *   qvalue[r, c] = convert(x[r, c] / scale[r / scale_block_rows, c / scale_block_cols])
  * `qmax`: the largest quantised magnitude, at most 127 (int8) or 448 (fp8 e4m3fn); 0 means that maximum (7 gives int4
- * values in int8 storage). convert rounds to nearest even and saturates at +-qmax (the form the reference gives the
- * same calibration in pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:802-822).
+ * values in int8 storage). `bound`: what the tile's absmax is divided by, in [qmax, qmax + 1]; 0 means qmax, the form the
+ * reference writes out for fp8 (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:802-822) and for integers in its TPU kernels
+ * (pallas_mosaic_tpu_kernel.py:267-277, experimental/gmm_v2/util.py:28-50: iinfo.max). qwix, the library behind
+ * `AsQArray`, is not part of the reference tree; should its integer bound be 2^(bits-1) - 0.5 (127.5, 7.5), that is
+ * `bound = qmax + 0.5` here (integer types only). convert rounds to nearest even and saturates at [-qmax, qmax], or at
+ * [-qmax - 1, qmax] with a bound above qmax.
  * x f32, bf16 or f16 [rows, cols] row-major; qvalue int8 or fp8 [rows, cols]; scale f32
  * [rows / scale_block_rows, cols / scale_block_cols]. Tiles: one row tall and a multiple of 8 columns wide (an lhs with
  * one scale per row, scale_block_cols = cols, or per (row, k-block)); or several rows tall and 1, 8, 16, ... or 256
  * columns wide (weights [g, k, n] as g * k rows: (k, 1) is one scale per (group, column), (t_k, 1) the scale tile
- * (1, t_k, 1), (128, 128) square blocks). cols % 8 == 0. */
+ * (1, t_k, 1), (128, 128) square blocks; a tile wider than 256 columns, e.g. one scale per tensor, is not taken).
+ * cols % 8 == 0. */
 int32_t tkx_quantize(const void* x, void* qvalue, float* scale, int64_t rows, int64_t cols, int64_t scale_block_rows,
-                     int64_t scale_block_cols, int32_t x_dtype, int32_t q_dtype, float qmax, tkx_stream_t stream);
+                     int64_t scale_block_cols, int32_t x_dtype, int32_t q_dtype, float qmax, float bound,
+                     tkx_stream_t stream);
 
 /* The token permute / un-permute steps either side of the ragged dot in an MoE layer, one kernel:
  *   out[j, :] = sum over r < reduce_group_size of keep(g) * weights[g] * x[indices[g], :],  g = j * reduce_group_size + r

@@ -59,6 +59,8 @@ below therefore cites the reference call site it follows, and says what pins it:
 Status of "parity unpinned": `qwix.quantize` itself (qwix>=0.1.2, pyproject.toml:27) is not in the tree.
 `quantize_absmax` follows the form of its absmax calibration that the reference writes out for fp8; for the integer
 types the bound qwix divides by (127 against 127.5 for int8) is NOT fixed by anything in the tree: parity unpinned.
+The integer quantisers that ARE in the tree divide by iinfo.max, i.e. 127 (pallas_mosaic_tpu_kernel.py:267-277,
+experimental/gmm_v2/util.py:28-50, gmm_v2.py:563): the default here; `bound` selects the other convention.
 Quantising and dequantising with one and the same rule, as every test of the reference does
 (test_base.py:36-62, :187-242), keeps that choice out of the results compared.
 "gelu" in the gate-up forms is `jax.nn.gelu(gate)` (gmm_v2.py:99-100); JAX is not
@@ -248,15 +250,21 @@ def unpack_int4(packed) -> np.ndarray:
 QMAX = {"int8": 127.0, "int4": 7.0, "fp8": 448.0}
 
 
-def quantize_absmax(x, qtype: str, tile_shape):
+def quantize_absmax(x, qtype: str, tile_shape, bound=None, reciprocal=False):
   """Symmetric absmax quantisation with one f32 scale per tile: what `AsQArray.as_qarray` asks of
   `qwix.quantize(x, qtype, tiled_axes=dict(enumerate(tile_shape)))` (quantization.py:65-78), stated the way the
   reference states the same calibration itself (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:802-822):
     scale = absmax(tile) / qmax, 1 where the tile is all zero;  q = x / scale, rounded to nearest even, clipped to +-qmax
-  with qmax the largest finite value of the type (127, 7, 448). Returns (q, scale): q int8 for the integer types, the
-  uint8 e4m3fn codes for "fp8"; scale float32 of shape x.shape / tile_shape. All arithmetic in float32."""
+  with qmax the largest finite value of the type (127, 7, 448). `bound` (default qmax) replaces qmax in the scale;
+  with a bound above qmax (integers: qmax + 0.5) values are clipped to [-qmax - 1, qmax]. The reference's own integer
+  quantisers divide by iinfo.max = qmax (pallas_mosaic_tpu_kernel.py:267-277, experimental/gmm_v2/util.py:28-50); what
+  qwix divides by is PARITY UNPINNED (qwix is not in the reference tree). `reciprocal`: x * (1 / scale) instead of
+  x / scale, the form of the reference's quantisation fused into a kernel's epilogue. Returns (q, scale): q int8 for the integer
+  types, the uint8 e4m3fn codes for "fp8"; scale float32 of shape x.shape / tile_shape. All arithmetic in float32."""
   x = np.asarray(x, np.float32)
   qmax = np.float32(QMAX[qtype])
+  bound = qmax if bound is None else np.float32(bound)
+  lo = -qmax - np.float32(1) if bound > qmax else -qmax
   tile_shape = tuple(int(t) for t in tile_shape)
   assert x.ndim == len(tile_shape) and all(d % t == 0 for d, t in zip(x.shape, tile_shape)), (x.shape, tile_shape)
   split = []
@@ -265,11 +273,16 @@ def quantize_absmax(x, qtype: str, tile_shape):
   tiles = x.reshape(split)
   inner = tuple(range(1, 2 * x.ndim, 2))
   absmax = np.abs(tiles).max(axis=inner)
-  scale = np.where(absmax == 0, np.float32(1), absmax / qmax).astype(np.float32)
+  scale = np.where(absmax == 0, np.float32(1), absmax / bound).astype(np.float32)
   full = scale
   for ax, t in enumerate(tile_shape):
     full = np.repeat(full, t, axis=ax)
-  q = np.clip((x / full).astype(np.float32), -qmax, qmax)
+  if reciprocal:
+    # the reference's fused output quantisation multiplies by the reciprocal of the (rounded) scale
+    # (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:813-822)
+    q = np.clip((x * (np.float32(1) / full)).astype(np.float32), lo, qmax)
+  else:
+    q = np.clip((x / full).astype(np.float32), lo, qmax)
   if qtype == "fp8":
     return e4m3fn_encode(q), scale
   return np.rint(q).astype(np.int8), scale

@@ -542,6 +542,21 @@ def test_arg_specs_and_flops():
   assert arg_specs.flops(**s.args) == 2 * 8192 * 4096 * 14336  # bench.py:52-56
 
 
+def test_uint8_storage_is_packed_int4_and_nothing_else():
+  """A uint8 `qvalue` is two int4 per byte only under a 4-bit `qtype`; any other uint8 quantised array is declined when
+  it is made, instead of being read as nibbles."""
+  from tokamax_amd import quantization
+  q = ShapeDtype((4, 64, 32), torch.uint8)
+  scale = ShapeDtype((4, 1, 32), torch.float32)
+  packed = quantization.QArray(q, scale, None, torch.int4)
+  assert packed.packed and packed.shape == (4, 128, 32)
+  for qtype in (None, torch.uint8, torch.int8):
+    with pytest.raises(NotImplementedError):
+      quantization.QArray(q, scale, None, qtype)
+  plain = quantization.QArray(ShapeDtype((4, 64, 32), torch.int8), scale, None, torch.int4)
+  assert not plain.packed and plain.shape == (4, 64, 32)
+
+
 def test_ffi_shim_compiles_to_its_stub_without_the_xla_header(tmp_path):
   """tokamax_amd/csrc/ffi_shim.cc holds the XLA FFI handlers behind `__has_include("xla/ffi/api/ffi.h")`; without the
   header (this image has no jaxlib) it must still compile, to a stub that says so."""
@@ -557,8 +572,19 @@ def test_ffi_shim_compiles_to_its_stub_without_the_xla_header(tmp_path):
   lib.tkx_ffi_shim_available.restype = ctypes.c_int32
   assert lib.tkx_ffi_shim_available() == 0
   text = open(src).read()
-  for symbol in ("TkxRaggedDotFwd", "TkxRaggedDotFwdFused", "TkxRaggedDotDrhs"):
+  for symbol in ("TkxRaggedDotFwd", "TkxRaggedDotFwdFused", "TkxRaggedDotFwdFp8Out", "TkxRaggedDotDrhs"):
     assert f"XLA_FFI_DEFINE_HANDLER_SYMBOL({symbol}," in text
+    assert text.count("TKX_CONFIG_ATTRS") >= 5  # the definition and one use per handler
+  # Every field of TkxConfig travels as an attribute of its name and is assigned by name (no positional initialiser
+  # that a new trailing field would silently leave out).
+  for name, _ in _lib.TkxConfig._fields_:
+    assert f'.Attr<int32_t>("{name}")' in text, name
+    assert f"cfg.{name} = {name};" in text, name
+  assert "const TkxConfig cfg{" not in text
+  header = open(os.path.join(ROOT, "include", "tkx_ragged_dot.h")).read()
+  struct = header[header.index("typedef struct TkxConfig {"):header.index("} TkxConfig;")]
+  declared = [line.split()[1].rstrip(";") for line in struct.splitlines() if line.strip().startswith("int32_t ")]
+  assert declared == [name for name, _ in _lib.TkxConfig._fields_]
 
 
 def test_heuristics_on_abstract_arguments_split_and_packed_int4():

@@ -458,6 +458,37 @@ def test_quantize_absmax_exact_cases():
     assert np.array_equal(q[:, c], np.rint(w[:, c] / s[0, c]).astype(np.int8))
 
 
+def test_quantize_absmax_with_the_half_step_bound_by_hand():
+  """bound = qmax + 0.5 (the convention of symmetric integer quantisers that use the type's whole range): the scale is
+  absmax / 127.5, the extreme value rounds to an end of [-128, 127], everything else follows from the scale."""
+  x = np.array([[-127.5, 127.5, 63.75, 0.4, -0.6, 1.5, 2.5, 0.0]], np.float32)
+  q, s = O.quantize_absmax(x, "int8", (1, 8), bound=127.5)
+  assert s[0, 0] == 1.0 and q.tolist() == [[-128, 127, 64, 0, -1, 2, 2, 0]]  # -127.5 -> -128 (even), +127.5 -> 128 -> clipped
+  q, s = O.quantize_absmax(np.array([[3.75, -3.75, 0.25, -1.0]], np.float32), "int4", (1, 4), bound=7.5)
+  assert s[0, 0] == 0.5 and q.tolist() == [[7, -8, 0, -2]]
+  # the default bound is qmax: nothing below -qmax
+  q, s = O.quantize_absmax(x, "int8", (1, 8))
+  assert s[0, 0] == np.float32(127.5) / np.float32(127) and q.min() == -127
+
+
+def test_quantize_absmax_reciprocal_form():
+  """`reciprocal=True` (the reference's fused output quantisation, acc * (1.0 / out_scale)): the same scales, values
+  equal to torch's own float8 cast of x * (1 / scale) in f32, and within one code of the dividing form."""
+  rng = np.random.default_rng(5)
+  x = rng.normal(0, 3, (32, 256)).astype(np.float32)
+  q_div, s_div = O.quantize_absmax(x, "fp8", (1, 128))
+  q_rcp, s_rcp = O.quantize_absmax(x, "fp8", (1, 128), reciprocal=True)
+  assert np.array_equal(s_div, s_rcp)
+  inv = (torch.tensor(1.0) / torch.tensor(np.repeat(s_rcp, 128, axis=1)))
+  want = (torch.tensor(x) * inv).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+  assert np.array_equal(q_rcp, want)
+  diff = np.abs(q_div.astype(np.int16) - q_rcp.astype(np.int16))
+  assert diff.max() <= 1 and (diff != 0).mean() < 0.01
+  # 1 / 3 is not a float: 3 * fl(1 / 3) rounds to 1 here, but a quotient on a boundary can land on its other side
+  one = O.quantize_absmax(np.array([[1344.0, 3.0] + [0.0] * 6], np.float32), "fp8", (1, 8), reciprocal=True)
+  assert one[1][0, 0] == 3.0 and O.e4m3fn_decode(one[0])[0, :2].tolist() == [448.0, 1.0]
+
+
 def test_dequantize_zero_point_by_hand():
   q = np.array([[10, -3, 0, 7]], np.int8)
   got = O.dequantize_zero_point(q, np.array([[0.5, 2.0]], np.float32), np.array([[2.0, -1.0]], np.float32))

@@ -94,3 +94,41 @@ def test_static_workspace_entry_rejects_a_split_contraction(device):
                                                _lib.TKX_BF16, _lib.TKX_BF16, _lib.TKX_BF16, 0, 0, ctypes.byref(c),
                                                torch.cuda.current_stream().cuda_stream)
   assert st == _lib.TKX_ERR_UNSUPPORTED and "split contraction" in _lib.last_error()
+
+
+def test_static_workspace_entry_under_graph_capture_allocates_nothing(device):
+  """The use the entry point is for: one eager call (the first on a device looks the array's address up and raises the
+  kernel's LDS limit), then the same call recorded into a HIP graph and replayed with new operands written into the
+  captured tensors. Every replay equals the eager result of the workspace entry point bit for bit, and the device's free
+  memory is the same before and after the calls: nothing was allocated."""
+  cfg = hip_ops.KernelConfig(128, 128, 64, 2, 2, 4, grid_tile_width=4)
+  rng = np.random.default_rng(23)
+  G, m, k, n = 5, 900, 256, 384
+  mk = lambda shape, std: torch.tensor(rng.normal(0, std, shape).astype(np.float32), device=device).to(torch.bfloat16)
+  lhs, rhs = mk((m, k), 1.0), mk((G, k, n), k ** -0.5)
+  gs = torch.tensor(np.array([200, 0, 310, 150, 180], np.int32), device=device)
+  got = torch.zeros((m, n), dtype=torch.bfloat16, device=device)
+  want = torch.zeros_like(got)
+  ws = hip_ops.workspace(m, G, cfg.block_m, device)
+  side = torch.cuda.Stream()
+  with torch.cuda.stream(side):
+    _call("static", lhs, rhs, gs, got, cfg, 0)  # eager, outside capture
+    side.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    _call("static", lhs, rhs, gs, got, cfg, 0)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+      _call("static", lhs, rhs, gs, got, cfg, 0)
+  torch.cuda.synchronize()
+  for sizes in ([200, 0, 310, 150, 180], [90, 400, 0, 0, 300], [0, 0, 0, 0, 7]):
+    lhs.copy_(mk((m, k), 1.0))
+    gs.copy_(torch.tensor(np.array(sizes, np.int32), device=device))
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    _call("workspace", lhs, rhs, gs, want, cfg, 0, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16)), sizes
+  free_after, _ = torch.cuda.mem_get_info()
+  assert free_after == free_before

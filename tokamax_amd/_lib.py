@@ -41,6 +41,7 @@ EXPORTED_SYMBOLS = (
     "tkx_ragged_dot_decode_workspace_bytes",
     "tkx_ragged_dot_decode_counter_bytes",
     "tkx_ragged_dot_decode_persistent_workspace_bytes",
+    "tkx_ragged_dot_decode_clear_counters",
     "tkx_unpack_int4",
     "tkx_pack_int4",
     "tkx_ragged_dot_fwd_fp8_out",
@@ -79,6 +80,8 @@ def _declare(lib):
   lib.tkx_ragged_dot_decode_workspace_bytes.argtypes = [i64, i64, i32]
   lib.tkx_ragged_dot_decode_persistent_workspace_bytes.restype = i64
   lib.tkx_ragged_dot_decode_persistent_workspace_bytes.argtypes = []
+  lib.tkx_ragged_dot_decode_clear_counters.restype = i32
+  lib.tkx_ragged_dot_decode_clear_counters.argtypes = [vp, vp]
   lib.tkx_ragged_dot_decode_counter_bytes.restype = i64
   lib.tkx_ragged_dot_decode_counter_bytes.argtypes = [i32]
   lib.tkx_ragged_dot_fwd_fp8_out.restype = i32
@@ -112,7 +115,7 @@ def _declare(lib):
   lib.tkx_dequantize_zero_point.restype = i32
   lib.tkx_dequantize_zero_point.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
   lib.tkx_quantize.restype = i32
-  lib.tkx_quantize.argtypes = [vp, vp, vp, i64, i64, i64, i64, i32, i32, ctypes.c_float, vp]
+  lib.tkx_quantize.argtypes = [vp, vp, vp, i64, i64, i64, i64, i32, i32, ctypes.c_float, ctypes.c_float, vp]
   lib.tkx_ragged_gather_rows.restype = i32
   lib.tkx_ragged_gather_rows.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]
   lib.tkx_ragged_dot_num_variants.restype = i32

@@ -2,7 +2,6 @@
 #include <cstdarg>
 #include <cstdio>
 #include <mutex>
-#include <vector>
 
 #include "tkx_common.h"
 
@@ -26,29 +25,40 @@ int32_t set_error(int32_t code, const char* fmt, ...) {
 
 namespace {
 
+// Every compiled variant, in one fixed table (filled once; nothing here allocates).
 struct Registry {
-  std::vector<Variant> all;
+  static constexpr int kCapacity = 256;
+  Variant all_[kCapacity];
+  int count_ = 0;
+  void add(const Variant& v) {
+    if (count_ < kCapacity) all_[count_++] = v;
+  }
+  void add(const Variant* v, int n) {
+    for (int i = 0; i < n; ++i) add(v[i]);
+  }
+  const Variant* begin() const { return all_; }
+  const Variant* end() const { return all_ + count_; }
   Registry() {
     int n = 0;
     const Variant* v;
-    v = variants_bf16(&n); all.insert(all.end(), v, v + n);
-    v = variants_f16(&n);  all.insert(all.end(), v, v + n);
-    v = variants_f32(&n);  all.insert(all.end(), v, v + n);
-    v = variants_f8(&n);   all.insert(all.end(), v, v + n);
-    v = variants_i8w(&n);  all.insert(all.end(), v, v + n);
+    v = variants_bf16(&n); add(v, n);
+    v = variants_f16(&n);  add(v, n);
+    v = variants_f32(&n);  add(v, n);
+    v = variants_f8(&n);   add(v, n);
+    v = variants_i8w(&n);  add(v, n);
     // The streaming small-m kernel is not a tile variant of the GEMM template; it is listed here
     // (fn == nullptr, num_stages = steps of loads in flight) so that configs can name it.
     for (int depth : {2, 4, 8})
-      all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
+      add({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
     for (int depth : {2, 4})
-      all.push_back({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeWideBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
+      add({kFwd, TKX_BF16, TKX_I8, kDecodeBlockM, kDecodeWideBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
     for (int depth : {2, 4})
-      all.push_back({kFwd, TKX_BF16, TKX_F8E4M3FN, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
+      add({kFwd, TKX_BF16, TKX_F8E4M3FN, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
     for (int dtype : {TKX_BF16, TKX_F16})
       for (int depth : {2, 4})
-        all.push_back({kFwd, dtype, dtype, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
+        add({kFwd, dtype, dtype, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
     for (int depth : {2, 4, 8})  // packed int4 weights: the streaming kernel is their only kernel
-      all.push_back({kFwd, TKX_BF16, TKX_I4X2, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
+      add({kFwd, TKX_BF16, TKX_I4X2, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
   }
 };
 
@@ -58,7 +68,7 @@ const Registry& registry() {
 }
 
 const Variant* find_variant(int mode, int a_dtype, int b_dtype, const TkxConfig& c) {
-  for (const Variant& v : registry().all)
+  for (const Variant& v : registry())
     if (v.mode == mode && v.a_dtype == a_dtype && v.b_dtype == b_dtype && v.block_m == c.block_m &&
         v.block_n == c.block_n && v.block_k == c.block_k && v.waves_m == c.waves_m && v.waves_n == c.waves_n &&
         v.num_stages == c.num_stages)
@@ -68,17 +78,21 @@ const Variant* find_variant(int mode, int a_dtype, int b_dtype, const TkxConfig&
 
 int dtype_bytes(int d) { return d == TKX_F32 ? 4 : (d == TKX_BF16 || d == TKX_F16) ? 2 : 1; }
 
-// Raises the dynamic-LDS limit of a kernel once per (device, kernel).
+// Raises the dynamic-LDS limit of a kernel once per (device, kernel); remembered in a fixed table, so that no entry
+// point touches the host heap.
 int32_t prepare(const void* fn, int32_t smem_bytes) {
+  struct Entry { int dev; const void* fn; };
+  constexpr int kSlots = 2048;
   static std::mutex mu;
-  static std::vector<std::pair<int, const void*>> done;
+  static Entry done[kSlots];
+  static int used = 0;
   int dev = 0;
   TKX_HIP_CHECK(hipGetDevice(&dev));
   std::lock_guard<std::mutex> lock(mu);
-  for (auto& d : done)
-    if (d.first == dev && d.second == fn) return TKX_OK;
+  for (int i = 0; i < used; ++i)
+    if (done[i].dev == dev && done[i].fn == fn) return TKX_OK;
   TKX_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes));
-  done.emplace_back(dev, fn);  // (host memory, once per kernel and device)
+  if (used < kSlots) done[used++] = {dev, fn};  // (a full table only means the attribute is set again)
   return TKX_OK;
 }
 
@@ -136,6 +150,11 @@ int64_t tkx_ragged_dot_decode_persistent_workspace_bytes(void) { return decode_p
 
 int64_t tkx_ragged_dot_decode_counter_bytes(int32_t split_k) {
   return split_k > 1 ? decode_split_counter_words() * 4 : 0;
+}
+
+int32_t tkx_ragged_dot_decode_clear_counters(void* workspace, tkx_stream_t stream) {
+  if (workspace == nullptr || (uintptr_t)workspace % 4 != 0) return set_error(TKX_ERR_INVALID, "null or misaligned workspace");
+  return launch_clear_decode_counters(static_cast<int32_t*>(workspace), static_cast<hipStream_t>(stream));
 }
 
 int64_t tkx_ragged_dot_tid_size(int64_t m, int64_t num_groups, int32_t block_m) {
@@ -549,7 +568,8 @@ int32_t tkx_pack_int4(const void* values, void* packed, int64_t packed_rows, int
 }
 
 int32_t tkx_quantize(const void* x, void* qvalue, float* scale, int64_t rows, int64_t cols, int64_t scale_block_rows,
-                     int64_t scale_block_cols, int32_t x_dtype, int32_t q_dtype, float qmax, tkx_stream_t stream) {
+                     int64_t scale_block_cols, int32_t x_dtype, int32_t q_dtype, float qmax, float bound,
+                     tkx_stream_t stream) {
   if (!x || !qvalue || !scale) return set_error(TKX_ERR_INVALID, "null pointer argument");
   if (rows < 1 || cols < 1 || scale_block_rows < 1 || scale_block_cols < 1)
     return set_error(TKX_ERR_INVALID, "bad sizes rows=%lld cols=%lld block=%lldx%lld", (long long)rows, (long long)cols,
@@ -577,7 +597,16 @@ int32_t tkx_quantize(const void* x, void* qvalue, float* scale, int64_t rows, in
   const float type_max = q_dtype == TKX_I8 ? 127.f : 448.f;
   if (qmax == 0.f) qmax = type_max;
   if (!(qmax > 0.f) || qmax > type_max) return set_error(TKX_ERR_INVALID, "qmax must lie in (0, %g]", (double)type_max);
-  return launch_quantize(x, qvalue, scale, rows, cols, scale_block_rows, scale_block_cols, x_dtype, q_dtype, qmax,
+  if (bound == 0.f) bound = qmax;
+  if (!(bound >= qmax) || bound > qmax + 1.f)
+    return set_error(TKX_ERR_INVALID, "bound must lie in [qmax, qmax + 1] (got %g for qmax %g)", (double)bound, (double)qmax);
+  // A bound above qmax (integers: 2^(b-1) - 0.5) lets -qmax - 1, the type's most negative value, appear.
+  QuantRange range = {bound, -qmax, qmax};
+  if (bound > qmax) {
+    if (q_dtype != TKX_I8) return set_error(TKX_ERR_INVALID, "a bound above qmax belongs to the integer types");
+    range.lo = -qmax - 1.f;
+  }
+  return launch_quantize(x, qvalue, scale, rows, cols, scale_block_rows, scale_block_cols, x_dtype, q_dtype, range,
                          static_cast<hipStream_t>(stream));
 }
 
@@ -601,7 +630,7 @@ int32_t tkx_ragged_gather_rows(const void* x, const int32_t* indices, const floa
 
 int32_t tkx_ragged_dot_num_variants(int32_t kind) {
   int32_t n = 0;
-  for (const Variant& v : registry().all) n += ((v.mode == kDrhs) == (kind == 1));
+  for (const Variant& v : registry()) n += ((v.mode == kDrhs) == (kind == 1));
   return n;
 }
 
@@ -609,7 +638,7 @@ int32_t tkx_ragged_dot_variant(int32_t kind, int32_t index, TkxConfig* config, i
                                int32_t* mode) {
   if (!config || !lhs_dtype || !rhs_dtype || !mode) return set_error(TKX_ERR_INVALID, "null pointer argument");
   int32_t i = 0;
-  for (const Variant& v : registry().all) {
+  for (const Variant& v : registry()) {
     if ((v.mode == kDrhs) != (kind == 1)) continue;
     if (i++ != index) continue;
     config->block_m = v.block_m;

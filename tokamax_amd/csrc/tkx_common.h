@@ -118,6 +118,7 @@ bool decode_persistent_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m
                                  int64_t scale_blocks, int32_t block_n, int32_t depth);
 int64_t decode_persistent_workspace_words();
 int64_t decode_split_counter_words();
+int32_t launch_clear_decode_counters(int32_t* workspace, hipStream_t stream);
 int64_t decode_split_workspace_words(int64_t m, int64_t n, int32_t split_k);
 int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, const int32_t* group_sizes, void* out,
                       int64_t m, int64_t k, int64_t n, int64_t G, int32_t rhs_dtype, int32_t out_dtype,
@@ -135,9 +136,11 @@ int32_t launch_dequant(const void* q, const float* scale, const float* zero_poin
                        int64_t t_r, int64_t t_c, int32_t q_dtype, hipStream_t stream);
 
 // ---- absmax quantisation to int8 / fp8 with block scales (the inverse pass) -------------------------
-// scale[R, C] = absmax of tile (R, C) / qmax (1 for an all-zero tile); q = convert(x / scale). x f32, bf16 or f16.
+// scale[R, C] = absmax of tile (R, C) / bound (1 for an all-zero tile); q = convert(clip(x / scale)). x f32, bf16 or f16.
+// `bound`: what the tile's absmax is divided by; values are clipped to [lo, hi] after the division.
+struct QuantRange { float bound, lo, hi; };
 int32_t launch_quantize(const void* x, void* q, float* scale, int64_t rows, int64_t cols, int64_t t_r, int64_t t_c,
-                        int32_t x_dtype, int32_t q_dtype, float qmax, hipStream_t stream);
+                        int32_t x_dtype, int32_t q_dtype, QuantRange range, hipStream_t stream);
 
 // ---- row gather with optional mask, weight and reduction (token permute / un-permute) -------------
 int32_t launch_gather_rows(const void* x, const int32_t* indices, const float* weights, const unsigned char* valid,

@@ -1060,6 +1060,20 @@ bool decode_supported(int32_t lhs_dtype, int32_t rhs_dtype, int64_t m, int64_t k
 // the same number of words whatever the shapes, so that calls of different shapes can share one workspace without
 // one call's partial sums landing where another expects zeroed counters.
 int64_t decode_split_counter_words() { return kDecCounterWords; }
+
+namespace {
+__global__ void clear_words_kernel(int32_t* words, int64_t count) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) words[i] = 0;
+}
+}  // namespace
+// Clears the counter block of a split / persistent workspace with a fill kernel (a memset node recorded into a captured
+// graph is what callers under capture should not have to rely on).
+int32_t launch_clear_decode_counters(int32_t* workspace, hipStream_t stream) {
+  clear_words_kernel<<<dim3((unsigned)(kDecCounterWords / 256)), dim3(256), 0, stream>>>(workspace, kDecCounterWords);
+  TKX_HIP_CHECK(hipGetLastError());
+  return TKX_OK;
+}
 int64_t decode_split_workspace_words(int64_t m, int64_t n, int32_t split_k) {
   if (split_k <= 1) return 0;
   return kDecCounterWords + (int64_t)split_k * m * n;

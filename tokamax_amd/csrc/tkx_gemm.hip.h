@@ -1193,9 +1193,11 @@ struct GemmKernel {
       // lays its part of the tile out row-major in its own slice of LDS and reads it back 16 bytes
       // per lane, so that a store instruction writes whole 128-byte (or longer) row segments.
       __syncthreads();  // every wave is done reading the last stage
-      // fp8 output: one scale per (row, 128 columns) = absmax / 448 (1 for a run of zeros), values divided by it and
-      // converted with saturation; the arithmetic of the standalone quantisation pass (launch_quantize), so the two
-      // agree bit for bit. A row's 128 columns lie in 128 / WTN wave columns: each wave reduces its part of every
+      // fp8 output: one scale per (row, 128 columns) = absmax / 448 (1 for a run of zeros), values multiplied by the
+      // reciprocal of the scale and converted with saturation: the arithmetic of the reference's fused quantisation
+      // (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:802-822). (The standalone pass, launch_quantize, divides, as a
+      // quantiser that never sees the accumulator would: the two can differ by one fp8 step where a quotient lies on
+      // a rounding boundary.) A row's 128 columns lie in 128 / WTN wave columns: each wave reduces its part of every
       // row (a lane's 16 TN values, then the lane 32 further on, which holds the row's other columns) and the waves
       // exchange them through LDS.
       float row_scale[TM][WTN > 128 ? WTN / 128 : 1];
@@ -1227,7 +1229,7 @@ struct GemmKernel {
 #pragma unroll
               for (int w = 0; w < QW; ++w) mx = fmaxf(mx, xchg[((wm * WN + wn0 + w) * TM * 32 + i * 32 + (lane & 31)) * QT + q]);
               const float scale = mx == 0.f ? 1.f : mx / 448.f;
-              row_scale[i][q] = scale;
+              row_scale[i][q] = 1.f / scale;  // (the values are multiplied by the reciprocal, as the reference's epilogue does)
               const int row = row0 + row_block(i) * 32 + (lane & 31);
               const int qcol = (col0 + wn * WTN) / 128 + q;
               if (lane < 32 && wn == wn0 && row >= act_start && row < act_end && qcol * 128 < p.n_ext)
@@ -1270,10 +1272,10 @@ struct GemmKernel {
                 unsigned char* dst = slice + (ii * 32 + (lane & 31)) * PITCH + (j * 32 + 8 * t + 4 * (lane >> 5)) * ESZ;
                 if constexpr (OUT == TKX_F8E4M3FN) {
                   constexpr int JT = WTN > 128 ? TN / (WTN / 128) : TN;
-                  const float scale = row_scale[i][j / JT];
+                  const float inv = row_scale[i][j / JT];
                   float q4[4];
 #pragma unroll
-                  for (int e = 0; e < 4; ++e) q4[e] = fminf(fmaxf(v[e] / scale, -448.f), 448.f);
+                  for (int e = 0; e < 4; ++e) q4[e] = fminf(fmaxf(v[e] * inv, -448.f), 448.f);
                   int w = 0;
                   w = __builtin_amdgcn_cvt_pk_fp8_f32(q4[0], q4[1], w, false);
                   w = __builtin_amdgcn_cvt_pk_fp8_f32(q4[2], q4[3], w, true);

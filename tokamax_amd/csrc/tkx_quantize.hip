@@ -52,17 +52,17 @@ __device__ __forceinline__ float absmax8(const float (&v)[8]) {
   return m;
 }
 
-__device__ __forceinline__ float scale_of(float absmax, float qmax) { return absmax == 0.f ? 1.f : absmax / qmax; }
+__device__ __forceinline__ float scale_of(float absmax, QuantRange qr) { return absmax == 0.f ? 1.f : absmax / qr.bound; }
 
 // 8 values / scale -> 8 quantised bytes (two dwords).
 template <int EQ>
-__device__ __forceinline__ i32x2 quantize8(const float (&v)[8], const float (&scale)[8], float qmax) {
+__device__ __forceinline__ i32x2 quantize8(const float (&v)[8], const float (&scale)[8], QuantRange qr) {
   i32x2 out;
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     float q[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) q[e] = fminf(fmaxf(v[4 * h + e] / scale[4 * h + e], -qmax), qmax);
+    for (int e = 0; e < 4; ++e) q[e] = fminf(fmaxf(v[4 * h + e] / scale[4 * h + e], qr.lo), qr.hi);
     if constexpr (EQ == kEI8) {
       unsigned w = 0;
 #pragma unroll
@@ -84,7 +84,7 @@ template <int EX, int EQ>
 __global__ __launch_bounds__(kQThreads) void quantize_rows_kernel(const unsigned char* __restrict__ x,
                                                                   unsigned char* __restrict__ q, float* __restrict__ scale,
                                                                   int64_t rows, int32_t cols, int32_t t_c, int32_t L,
-                                                                  float qmax) {
+                                                                  QuantRange qmax) {
   constexpr int XB = XVec<EX>::BYTES;  // bytes of 8 elements of x
   const int lane = threadIdx.x & 63;
   const int tiles_per_row = cols / t_c;
@@ -132,7 +132,7 @@ template <int EX, int EQ>
 __global__ __launch_bounds__(kQThreads) void quantize_blocks_kernel(const unsigned char* __restrict__ x,
                                                                     unsigned char* __restrict__ q, float* __restrict__ scale,
                                                                     int64_t rows, int32_t cols, int32_t t_r, int32_t t_c,
-                                                                    float qmax) {
+                                                                    QuantRange qmax) {
   constexpr int XB = XVec<EX>::BYTES;
   __shared__ float red[8][256];
   const int tid = threadIdx.x, slice = tid >> 5, l32 = tid & 31;
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(kQThreads) void quantize_blocks_kernel(const unsign
 
 template <int EX>
 int32_t launch_for_x(const void* x, void* q, float* scale, int64_t rows, int64_t cols, int64_t t_r, int64_t t_c,
-                     int32_t q_dtype, float qmax, hipStream_t stream) {
+                     int32_t q_dtype, QuantRange qmax, hipStream_t stream) {
   const auto* xb = static_cast<const unsigned char*>(x);
   auto* qb = static_cast<unsigned char*>(q);
   if (t_r == 1) {
@@ -223,7 +223,7 @@ int32_t launch_for_x(const void* x, void* q, float* scale, int64_t rows, int64_t
 }  // namespace
 
 int32_t launch_quantize(const void* x, void* q, float* scale, int64_t rows, int64_t cols, int64_t t_r, int64_t t_c,
-                        int32_t x_dtype, int32_t q_dtype, float qmax, hipStream_t stream) {
+                        int32_t x_dtype, int32_t q_dtype, QuantRange qmax, hipStream_t stream) {
   if (x_dtype == TKX_F32) return launch_for_x<kEF32>(x, q, scale, rows, cols, t_r, t_c, q_dtype, qmax, stream);
   if (x_dtype == TKX_BF16) return launch_for_x<kEBF16>(x, q, scale, rows, cols, t_r, t_c, q_dtype, qmax, stream);
   return launch_for_x<kEF16>(x, q, scale, rows, cols, t_r, t_c, q_dtype, qmax, stream);

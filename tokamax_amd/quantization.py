@@ -21,6 +21,11 @@ from typing import Any, Collection, Mapping
 import torch
 
 
+# torch builds without an int4 dtype cannot name the type: there `PACKED_INT4` marks a packed array.
+PACKED_INT4 = getattr(torch, "int4", "int4x2")
+_FOUR_BIT_TYPES = tuple({PACKED_INT4, "int4x2"})
+
+
 @dataclasses.dataclass(frozen=True)
 class QArray:
   qvalue: Any  # torch.Tensor or ShapeDtype
@@ -31,6 +36,11 @@ class QArray:
   def __post_init__(self):
     if self.qtype is None:
       object.__setattr__(self, "qtype", self.qvalue.dtype)
+    if self.qvalue.dtype == torch.uint8 and self.qtype not in _FOUR_BIT_TYPES:
+      # uint8 storage means one thing here: int4 packed two to a byte. Anything else in bytes would be unpacked as
+      # nibbles and give wrong results without a word.
+      raise NotImplementedError(f"a uint8 qvalue is packed int4 and needs qtype int4 (got {self.qtype}); other uint8"
+                                " quantised types are not supported")
 
   def _leaves(self):
     return (self.qvalue, self.scale, self.zero_point)
@@ -42,8 +52,8 @@ class QArray:
 
   @property
   def packed(self) -> bool:
-    """Two int4 values per byte of `qvalue` along its second-to-last axis."""
-    return self.qvalue.dtype == torch.uint8
+    """Two int4 values per byte of `qvalue` along its second-to-last axis: uint8 storage under a 4-bit qtype."""
+    return self.qvalue.dtype == torch.uint8 and self.qtype in _FOUR_BIT_TYPES
 
   @property
   def shape(self) -> tuple[int, ...]:
@@ -143,8 +153,7 @@ def pack_int4(q: QArray) -> QArray:
   if q.qvalue.dtype != torch.int8 or q.zero_point is not None:
     raise NotImplementedError("pack_int4 takes int4 values in int8 storage without a zero point")
   from tokamax_amd.ragged_dot import hip_ops  # pylint: disable=g-import-not-at-top
-  int4 = getattr(torch, "int4", None)
-  return QArray(hip_ops.pack_int4(q.qvalue), q.scale, None, int4 if int4 is not None else q.qtype)
+  return QArray(hip_ops.pack_int4(q.qvalue), q.scale, None, PACKED_INT4)
 
 
 def as_array_or_qarray(x):

@@ -276,10 +276,11 @@ for _bits in range(2, 8):
     _QMAX[getattr(torch, f"int{_bits}")] = float(2 ** (_bits - 1) - 1)  # sub-byte integers live in int8 storage
 
 
-def quantize(x: torch.Tensor, qtype: torch.dtype, tile_shape) -> tuple[torch.Tensor, torch.Tensor]:
+def quantize(x: torch.Tensor, qtype: torch.dtype, tile_shape, bound: float | None = None) -> tuple[torch.Tensor, torch.Tensor]:
   """(qvalue, scale) of the absmax quantisation of `x` with one scale per tile of `tile_shape`
   (`qwix.quantize(x, qtype, tiled_axes=dict(enumerate(tile_shape)))`, quantization.py:65-78):
-  scale = absmax(tile) / qmax (1 for an all-zero tile), qvalue = round_to_nearest_even(x / scale), saturated at qmax.
+  scale = absmax(tile) / bound (1 for an all-zero tile), qvalue = round_to_nearest_even(x / scale), saturated at qmax.
+  `bound` defaults to qmax (127, 7, 448); qmax + 0.5 is the other convention in use for integers (then -qmax - 1 appears).
 
   x f32, bf16 or f16: [rows, cols] with tiles one row tall and a multiple of 8 columns wide, or several rows tall and
   1, 8, 16, ... or 256 columns wide; or weights [g, k, n] with a tile (1, t_k, t_n) (taken as g * k rows). qtype int8,
@@ -306,7 +307,7 @@ def quantize(x: torch.Tensor, qtype: torch.dtype, tile_shape) -> tuple[torch.Ten
   scale = torch.empty(tuple(d // t for d, t in zip(x.shape, tile_shape)), dtype=torch.float32, device=x.device)
   with _on_device(x.device):
     st = lib.tkx_quantize(_ptr(x), _ptr(qvalue), _ptr(scale), rows, cols, t_r, t_c, dtype_code(x.dtype), dtype_code(storage),
-                          ctypes.c_float(_QMAX[qtype]), _stream(x.device))
+                          ctypes.c_float(_QMAX[qtype]), ctypes.c_float(0.0 if bound is None else bound), _stream(x.device))
   _lib.check(st)
   return qvalue, scale
 
