@@ -100,7 +100,7 @@ def test_static_workspace_entry_under_graph_capture_allocates_nothing(device):
   """The use the entry point is for: one eager call (the first on a device looks the array's address up and raises the
   kernel's LDS limit), then the same call recorded into a HIP graph and replayed with new operands written into the
   captured tensors. Every replay equals the eager result of the workspace entry point bit for bit, and the device's free
-  memory is the same before and after the calls: nothing was allocated."""
+  memory is the same before and after eager calls: nothing was allocated. (The graph object itself is torch's.)"""
   cfg = hip_ops.KernelConfig(128, 128, 64, 2, 2, 4, grid_tile_width=4)
   rng = np.random.default_rng(23)
   G, m, k, n = 5, 900, 256, 384
@@ -110,25 +110,30 @@ def test_static_workspace_entry_under_graph_capture_allocates_nothing(device):
   got = torch.zeros((m, n), dtype=torch.bfloat16, device=device)
   want = torch.zeros_like(got)
   ws = hip_ops.workspace(m, G, cfg.block_m, device)
+  all_sizes = ([200, 0, 310, 150, 180], [90, 400, 0, 0, 300], [0, 0, 0, 0, 7])
+  # (every tensor the loop below needs exists before the memory reading is taken)
+  new_lhs = [mk((m, k), 1.0) for _ in all_sizes]
+  new_gs = [torch.tensor(np.array(sizes, np.int32), device=device) for sizes in all_sizes]
   side = torch.cuda.Stream()
   with torch.cuda.stream(side):
     _call("static", lhs, rhs, gs, got, cfg, 0)  # eager, outside capture
     side.synchronize()
+    torch.cuda.synchronize()
     free_before, _ = torch.cuda.mem_get_info()
-    _call("static", lhs, rhs, gs, got, cfg, 0)
+    for _ in range(3):
+      _call("static", lhs, rhs, gs, got, cfg, 0)
     side.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before  # three calls later: nothing was allocated
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
       _call("static", lhs, rhs, gs, got, cfg, 0)
   torch.cuda.synchronize()
-  for sizes in ([200, 0, 310, 150, 180], [90, 400, 0, 0, 300], [0, 0, 0, 0, 7]):
-    lhs.copy_(mk((m, k), 1.0))
-    gs.copy_(torch.tensor(np.array(sizes, np.int32), device=device))
+  for sizes, l, g in zip(all_sizes, new_lhs, new_gs):
+    lhs.copy_(l)
+    gs.copy_(g)
     torch.cuda.synchronize()
     graph.replay()
     torch.cuda.synchronize()
     _call("workspace", lhs, rhs, gs, want, cfg, 0, ws)
     torch.cuda.synchronize()
     assert torch.equal(got.view(torch.int16), want.view(torch.int16)), sizes
-  free_after, _ = torch.cuda.mem_get_info()
-  assert free_after == free_before
