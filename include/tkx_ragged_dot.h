@@ -82,12 +82,18 @@ typedef struct TkxConfig {
   int32_t align_tile;      /* task starts are aligned down to this many rows (reference default 8) */
   int32_t num_stages;      /* LDS stages of block_k contraction elements kept in flight */
   int32_t split_k;         /* workgroups that share the contraction of one output tile (the reference's split_k,
-                              pallas_mosaic_gpu_common.py:53). 0 and 1: no split. Above 1: the streaming small-m kernel
-                              only (block_m == 16, block_n == 128, num_stages <= 4, k a multiple of
-                              128 * split_k * num_stages), and `workspace` then is
+                              pallas_mosaic_gpu_common.py:53, pallas_triton.py:41-48). 0 and 1: no split. Above 1, on the
+                              streaming small-m kernel (block_m == 16, block_n == 128, num_stages <= 4, k a multiple of
+                              128 * split_k * num_stages): every tile is split, and `workspace` then is
                               tkx_ragged_dot_decode_workspace_bytes long with its first
                               tkx_ragged_dot_decode_counter_bytes ZERO on entry; the call leaves them zero, so a caller
-                              that keeps one workspace per stream clears it once. */
+                              that keeps one workspace per stream clears it once. Above 1 (at most 16), on a tiled
+                              kernel (plain forward and TRANS_RHS; no gate-up fusion, scales per k-block or quantised
+                              result): only the tiles of the launch's last, partial round of workgroups are split, into
+                              floor(CUs / their number) parts, at most split_k, so that a launch of 1.25 rounds costs
+                              1.25 rounds instead of 2; `workspace` then is tkx_ragged_dot_split_workspace_bytes long and
+                              needs no clearing (the schedule kernel clears the counters). Parts are added in the order
+                              of their index whoever arrives last: results are reproducible run to run. */
   int32_t persistent;      /* the reference's `persistent` (pallas_mosaic_gpu_common.py:55): resident workgroups that share
                               the work out evenly instead of one workgroup per tile and nothing else. 0: off. 1 (the
                               streaming small-m kernel: block_m == 16, block_n == 128, num_stages <= 4, one scale per
@@ -136,6 +142,10 @@ int64_t tkx_ragged_dot_tid_size(int64_t m, int64_t num_groups, int32_t block_m);
 
 /* Bytes of device workspace needed by schedule/fwd/drhs for these sizes (int32 arrays, 256-aligned). */
 int64_t tkx_ragged_dot_workspace_bytes(int64_t m, int64_t num_groups, int32_t block_m);
+
+/* Bytes of workspace of a tiled forward / TRANS_RHS call with config->split_k > 1: the schedule arrays, then one f32
+ * partial tile (block_m x block_n) for each of at most 256 parts. */
+int64_t tkx_ragged_dot_split_workspace_bytes(int64_t m, int64_t num_groups, int32_t block_m, int32_t block_n);
 
 /* Word offsets (int32 units) inside the workspace, for callers/tests that read the schedule back:
  * which = 0 num_tasks (1 word), 1 total_rows (1 word), 2 group_offsets (G+1 words),

@@ -6,6 +6,7 @@ Case list and tolerances follow the reference's shared suite
 error vs an f32/f64-accumulated reference <= 1e-5 (f32), <= 2e-3 (bf16/f16), <= 3e-2 (fp8, int8-dequant).
 """
 
+import dataclasses
 import itertools
 import json
 import os
@@ -449,6 +450,88 @@ def test_every_kernel_variant_through_c_abi(v, device):
   want = O.ragged_dot(lhs_f, rhs_f, gs, O.TRANS_RHS if v["mode"] == 1 else O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
   _check(out, want, tol)
   assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  if v["block_m"] >= 128:
+    # The same call with its tiles cut along the contraction (a launch this small is one partial round of workgroups,
+    # so every tile is split): 2 and 3 parts, and 12 = 256 CUs / 20 tiles, most of which get no k-step at all.
+    for split_k in (2, 3, 16):
+      split = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=dataclasses.replace(cfg, split_k=split_k), out_dtype=torch.float32,
+                                     trans_rhs=(v["mode"] == 1), lhs_scale=lhs_scale, rhs_scale=rhs_scale)
+      _check(split, want, tol)
+      assert torch.count_nonzero(split[int(gs.sum()):]) == 0
+      if lt == torch.int8:
+        assert torch.equal(split, out)  # int32 sums do not depend on how they are grouped
+      again = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=dataclasses.replace(cfg, split_k=split_k), out_dtype=torch.float32,
+                                     trans_rhs=(v["mode"] == 1), lhs_scale=lhs_scale, rhs_scale=rhs_scale)
+      assert torch.equal(again, split)  # parts are added in the order of their index, whoever arrives last
+
+
+@pytest.mark.parametrize("trans", [False, True])
+@pytest.mark.parametrize("m,split_k,parts", [(4096, 4, 4), (4096, 2, 2), (4608, 4, 2), (5632, 4, 1), (8192, 8, 1)])
+def test_last_round_of_a_tiled_launch_split_along_the_contraction(m, split_k, parts, trans, device):
+  """`split_k` on a tiled kernel: only the tiles beyond the last multiple of the CU count are cut, into
+  min(split_k, CUs / their number) parts. 128 x 256 tiles on n = 2304: m = 4096 gives 33 m-tasks x 9 = 297 tiles, 41
+  beyond 256 (6 parts would fit, split_k decides); 4608: 37 x 9 = 333, 77 beyond (3 fit: 2 when split_k is 2... here 4
+  asks, 3 fit); 5632: 45 x 9 = 405, 149 beyond (no split: the round is more than half full); 8192: 65 x 9 = 585, 73
+  beyond 512."""
+  del parts  # (documentation of the case; the result must be the same whatever the kernel decides)
+  rng = np.random.default_rng(m + split_k)
+  G, contraction, other = 2, 520, 2304
+  gs = np.array([m // 2 + 37, m // 2 - 37 - 5], np.int32)
+  k, n = (other, contraction) if trans else (contraction, other)
+  mk = lambda shape, std: torch.tensor(rng.normal(0, std, shape).astype(np.float32), device=device).to(torch.bfloat16)
+  lhs, rhs = mk((m, contraction), 1.0), mk((G, k, n), contraction ** -0.5)
+  gst = torch.tensor(gs, device=device)
+  cfg = hip_ops.KernelConfig(128, 256, 64, 2, 4, 3, grid_tile_width=4)
+  plain = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, trans_rhs=trans)
+  split_cfg = dataclasses.replace(cfg, split_k=split_k)
+  split = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=split_cfg, out_dtype=torch.float32, trans_rhs=trans)
+  # f32 sums of exact products in another grouping: equal to rounding, and equal bits where nothing was split
+  assert O.rel_l2(_np(split), _np(plain)) <= 1e-6
+  assert torch.equal(split[:1024], plain[:1024])  # (the launch's first 256 tiles cover these rows)
+  assert torch.count_nonzero(split[int(gs.sum()):]) == 0
+  # the launch's last tiles, which are the split ones, hold the last rows: those against the oracle's definition
+  first = int(gs.sum()) - 400
+  assert first > gs[0]
+  w1 = _np(rhs[1]).astype(np.float64)
+  want = _np(lhs[first:int(gs.sum())]).astype(np.float64) @ (w1.T if trans else w1)
+  _check(split[first:int(gs.sum())], want, 1e-5)
+  for _ in range(3):
+    assert torch.equal(hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=split_cfg, out_dtype=torch.float32, trans_rhs=trans), split)
+  if not trans:
+    # the fused entry point: bias, activation and a group offset ride on the split tiles' epilogue
+    bias = torch.tensor(rng.normal(0, 0.5, (G, 1, n)).astype(np.float32), device=device)
+    a = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.bfloat16, rhs_bias=bias, activation="silu")
+    b = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=split_cfg, out_dtype=torch.bfloat16, rhs_bias=bias, activation="silu")
+    assert O.rel_l2(_np(b), _np(a)) <= 3e-3 and (b != a).float().mean() < 0.01  # a bf16 rounding flips here and there
+    off = torch.tensor([1], dtype=torch.int32, device=device)
+    gs3 = torch.tensor(np.array([100, gs[0] - 100, gs[1]], np.int32), device=device)
+    a = hip_ops.ragged_dot_fwd(lhs, rhs, gs3, config=cfg, out_dtype=torch.float32, group_offset=off)
+    b = hip_ops.ragged_dot_fwd(lhs, rhs, gs3, config=split_cfg, out_dtype=torch.float32, group_offset=off)
+    assert O.rel_l2(_np(b), _np(a)) <= 1e-6 and torch.count_nonzero(b[:100]) == 0
+
+
+def test_tiled_split_is_declined_where_no_kernel_has_it(device):
+  G, m, k, n = 2, 512, 256, 512
+  a, b, gs = _inputs("split_declined", G, m, k, n, torch.bfloat16, device)
+  gst = torch.tensor(gs, device=device)
+  small = hip_ops.KernelConfig(64, 128, 64, 2, 2, 4, split_k=2)  # tiles of fewer than 128 rows
+  with pytest.raises(NotImplementedError, match="split"):
+    hip_ops.ragged_dot_fwd(a, b, gst, config=small, out_dtype=torch.float32)
+  glu = dataclasses.replace(next(hip_ops.KernelConfig(*v[:6]) for v in hip._variant_table()[(3, _lib.TKX_BF16, _lib.TKX_BF16)]
+                                 if v[0] >= 128), split_k=2)
+  with pytest.raises(NotImplementedError, match="split"):
+    hip_ops.ragged_dot_fwd(a, b, gst, config=glu, out_dtype=torch.float32, gateup=True, activation="silu")
+  with pytest.raises(ValueError, match="split_k"):
+    hip_ops.ragged_dot_fwd(a, b, gst, config=hip_ops.KernelConfig(128, 256, 64, 2, 4, 3, split_k=17), out_dtype=torch.float32)
+  drhs = dataclasses.replace(next(hip_ops.KernelConfig(*v[:6]) for v in hip._variant_table()[(2, _lib.TKX_BF16, _lib.TKX_BF16)]),
+                             split_k=2)
+  # (drhs has no last-round split either: its entry point ignores the field, as it always has)
+  out = hip_ops.ragged_dot_drhs(a, torch.randn(m, n, device=device).to(torch.bfloat16), gst, G, config=drhs, out_dtype=torch.float32)
+  assert out.shape == (G, k, n)
+  # the quantised-output entry point drops the split (its epilogue needs whole rows of 128 columns in one workgroup)
+  q, s = hip_ops.ragged_dot_fwd_fp8_out(a, b, gst, config=hip_ops.KernelConfig(128, 256, 64, 2, 4, 3, split_k=4))
+  q1, s1 = hip_ops.ragged_dot_fwd_fp8_out(a, b, gst, config=hip_ops.KernelConfig(128, 256, 64, 2, 4, 3))
+  assert torch.equal(q.view(torch.uint8), q1.view(torch.uint8)) and torch.equal(s, s1)
 
 
 def _plain_tiled_variants():
@@ -1128,9 +1211,11 @@ def test_group_offset_tiled_kernels(offset, local, device):
 
 
 def test_group_offset_shards_add_up_and_follow_the_device_value(device):
-  """Four expert-parallel shards of 8 experts (2 each) of one job add up to the unsharded result, bit for bit
-  in f32 (every row is computed by exactly one shard, by the same kernel); the offset is read on the device, so
-  one tensor updated in place serves all four calls."""
+  """Four expert-parallel shards of 8 experts (2 each) of one job add up to the unsharded result: bit for bit in f32
+  under one fixed tile configuration without a split last round (every row is computed by exactly one shard, by the
+  same kernel), and to f32 rounding under the configurations the heuristics choose per call (a launch of few tiles
+  has its last round split along the contraction, and the shards' launches are smaller than the whole job's); the
+  offset is read on the device, so one tensor updated in place serves all four calls."""
   rng = np.random.default_rng(8)
   G, k, n = 8, 512, 1024
   gs = rng.multinomial(1500, [1 / G] * G).astype(np.int32)
@@ -1138,17 +1223,20 @@ def test_group_offset_shards_add_up_and_follow_the_device_value(device):
   gst = torch.tensor(gs, device=device)
   lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
   rhs = torch.tensor(rng.normal(0, k ** -0.5, (G, k, n)).astype(np.float32), device=device).to(torch.bfloat16)
-  op = tokamax_amd.HipRaggedDot()
-  full = op(lhs, rhs, group_sizes=gst, preferred_element_type=torch.float32)
   goff = torch.zeros(1, dtype=torch.int32, device=device)
-  total = torch.zeros_like(full)
-  for shard in range(4):
-    goff.fill_(2 * shard)
-    part = op(lhs, rhs[2 * shard:2 * shard + 2], group_sizes=gst, group_offset=goff, preferred_element_type=torch.float32)
-    rows = slice(int(gs[:2 * shard].sum()), int(gs[:2 * shard + 2].sum()))
-    assert torch.count_nonzero(part[:rows.start]) == 0 and torch.count_nonzero(part[rows.stop:]) == 0
-    total += part
-  assert torch.equal(total, full)
+  for op in (tokamax_amd.HipRaggedDot(config=hip.Config(128, 256, 64, 2, 4, 3)), tokamax_amd.HipRaggedDot()):
+    full = op(lhs, rhs, group_sizes=gst, preferred_element_type=torch.float32)
+    total = torch.zeros_like(full)
+    for shard in range(4):
+      goff.fill_(2 * shard)
+      part = op(lhs, rhs[2 * shard:2 * shard + 2], group_sizes=gst, group_offset=goff, preferred_element_type=torch.float32)
+      rows = slice(int(gs[:2 * shard].sum()), int(gs[:2 * shard + 2].sum()))
+      assert torch.count_nonzero(part[:rows.start]) == 0 and torch.count_nonzero(part[rows.stop:]) == 0
+      total += part
+    if op.config is not None:
+      assert torch.equal(total, full)
+    else:
+      assert O.rel_l2(_np(total), _np(full)) <= 1e-6
 
 
 @pytest.mark.parametrize("block_n,split_k", [(128, 1), (256, 1), (128, 2), (128, 4), (128, -1), (128, -2)])

@@ -25,6 +25,7 @@ EXPORTED_SYMBOLS = (
     "tkx_last_error",
     "tkx_ragged_dot_tid_size",
     "tkx_ragged_dot_workspace_bytes",
+    "tkx_ragged_dot_split_workspace_bytes",
     "tkx_ragged_dot_workspace_offset",
     "tkx_ragged_dot_schedule",
     "tkx_ragged_dot_fwd",
@@ -95,6 +96,8 @@ def _declare(lib):
   lib.tkx_ragged_dot_tid_size.argtypes = [i64, i64, i32]
   lib.tkx_ragged_dot_workspace_bytes.restype = i64
   lib.tkx_ragged_dot_workspace_bytes.argtypes = [i64, i64, i32]
+  lib.tkx_ragged_dot_split_workspace_bytes.restype = i64
+  lib.tkx_ragged_dot_split_workspace_bytes.argtypes = [i64, i64, i32, i32]
   lib.tkx_ragged_dot_workspace_offset.restype = i64
   lib.tkx_ragged_dot_workspace_offset.argtypes = [i64, i64, i32, i32]
   lib.tkx_ragged_dot_schedule.restype = i32

@@ -15,6 +15,25 @@ namespace tkx {
 
 static thread_local char g_err[512] = "";
 
+// Compute units of the current device (fixed table: no allocation after the library is loaded).
+int32_t device_compute_units(int* out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static int count[kMaxDevices] = {};
+  int dev = 0;
+  TKX_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return set_error(TKX_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (count[dev] == 0) {
+    int cus = 0;
+    TKX_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (cus < 1) return set_error(TKX_ERR_RUNTIME, "device reports %d compute units", cus);
+    count[dev] = cus;
+  }
+  *out = count[dev];
+  return TKX_OK;
+}
+
 int32_t set_error(int32_t code, const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
@@ -97,7 +116,7 @@ int32_t prepare(const void* fn, int32_t smem_bytes) {
 }
 
 int32_t launch(const Variant* v, const GemmParams& p, int64_t grid, hipStream_t stream) {
-  const void* fn = p.c_scale != nullptr ? v->fn_fp8_out : v->fn;
+  const void* fn = p.c_scale != nullptr ? v->fn_fp8_out : p.split_k > 1 ? v->fn_split : v->fn;
   int32_t st = prepare(fn, v->smem_bytes);
   if (st != TKX_OK) return st;
   if (grid <= 0 || grid > 0x7fffffffLL) return set_error(TKX_ERR_INVALID, "grid size %lld out of range", (long long)grid);
@@ -165,6 +184,11 @@ int64_t tkx_ragged_dot_tid_size(int64_t m, int64_t num_groups, int32_t block_m) 
 int64_t tkx_ragged_dot_workspace_bytes(int64_t m, int64_t num_groups, int32_t block_m) {
   if (m < 0 || num_groups < 1 || block_m < 1) return -1;
   return ws_layout(m, num_groups, block_m).words * 4;
+}
+
+int64_t tkx_ragged_dot_split_workspace_bytes(int64_t m, int64_t num_groups, int32_t block_m, int32_t block_n) {
+  if (m < 0 || num_groups < 1 || block_m < 1 || block_n < 1) return -1;
+  return ws_layout(m, num_groups, block_m).words * 4 + (int64_t)kSplitUnits * block_m * block_n * 4;
 }
 
 int64_t tkx_ragged_dot_workspace_offset(int64_t m, int64_t num_groups, int32_t block_m, int32_t which) {
@@ -286,6 +310,8 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
   if (out_scale != nullptr && (v->fn == nullptr || v->fn_fp8_out == nullptr))
     return set_error(TKX_ERR_UNSUPPORTED, "this kernel variant cannot quantise its result (bf16 or fp8 forward tiles whose"
                                           " wave columns tile 128 output columns can)");
+  if (v->fn != nullptr && c.split_k > 1 && v->fn_split == nullptr)
+    return set_error(TKX_ERR_UNSUPPORTED, "this kernel variant cannot split its last round (plain forward and TRANS_RHS tiles of at least 128 rows can)");
   if (v->fn == nullptr) {
     // Streaming decode kernel: one launch, no schedule.
     if (lhs_scale != nullptr) return set_error(TKX_ERR_UNSUPPORTED, "the decode kernel takes no lhs scale");
@@ -319,6 +345,12 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
   }
 
   if (c.persistent != 0) return set_error(TKX_ERR_UNSUPPORTED, "persistent belongs to the streaming small-m kernel (block_m == 16)");
+  // split_k > 1 on a tiled kernel: the tiles of the last, partial round of workgroups are cut along the contraction
+  // (plain forward and dlhs variants; the workspace then is tkx_ragged_dot_split_workspace_bytes long).
+  const int32_t split_k = c.split_k > 1 ? c.split_k : 1;
+  if (split_k > 1 && (gateup || subk || out_scale != nullptr))
+    return set_error(TKX_ERR_UNSUPPORTED, "split_k > 1 on a tiled kernel: plain forward and TRANS_RHS only (no gate-up fusion, scales per k-block or quantised result)");
+  if (split_k > 16) return set_error(TKX_ERR_INVALID, "split_k must lie in [1, 16], got %d", split_k);
   const WsLayout L = ws_layout(m, num_groups, c.block_m);
   int32_t st = launch_schedule(group_sizes, num_groups, group_offset, num_group_sizes, m, c.block_m, c.align_tile,
                                c.grid_tile_width, static_cast<int32_t*>(workspace), L, stream);
@@ -368,7 +400,20 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
   int64_t zero_wgs = (m * cols * ob + (64 << 10) - 1) / (64 << 10);
   if (zero_wgs > 256) zero_wgs = 256;
   if (zero_wgs < 1) zero_wgs = 1;
-  return launch(v, p, slots + zero_wgs, stream);
+  p.zero_wgs = (int32_t)zero_wgs;
+  p.split_k = split_k;
+  p.split_cus = 1;
+  int64_t split_wgs = 0;
+  if (split_k > 1) {
+    int cus = 0;
+    st = device_compute_units(&cus);
+    if (st != TKX_OK) return st;
+    p.split_cus = cus < kSplitUnits ? cus : kSplitUnits;
+    p.ws_split_counters = (int32_t)L.split_counters;
+    p.split_partials = reinterpret_cast<float*>(static_cast<int32_t*>(workspace) + L.words);
+    split_wgs = p.split_cus;  // at most that many parts beside the tiles' own workgroups
+  }
+  return launch(v, p, slots + zero_wgs + split_wgs, stream);
 }
 }  // namespace
 
@@ -486,6 +531,8 @@ int32_t tkx_ragged_dot_drhs(const void* lhs, const void* dout, const int32_t* gr
   p.out_dtype = out_dtype;
   p.activation = TKX_ACT_NONE;
   p.ws_offsets = (int32_t)L.offsets;
+  p.split_k = 1;
+  p.split_cus = 1;
   return launch(v, p, (int64_t)num_groups * p.m_tiles * p.n_tiles, stream);
 }
 

@@ -20,9 +20,15 @@ constexpr int64_t kWsHeader = 64;
 struct WsLayout {
   int64_t offsets;   // word offset of group_offsets
   int64_t task[8];   // word offsets of the task arrays
-  int64_t words;     // total words
+  int64_t split_counters;  // word offset of kSplitUnits arrival counters (tiled kernels with split_k > 1); the
+                           // scheduler kernel clears them in every call
+  int64_t words;     // total words (the partial tiles of a split launch lie behind them)
   int32_t tid_size;
 };
+
+// Tiled kernels with split_k > 1: the tiles of the last, partial round of workgroups are cut along the contraction
+// into parts, at most this many parts in all (one per CU of a 256-CU device).
+constexpr int32_t kSplitUnits = 256;
 
 inline int64_t round_up64(int64_t x) { return (x + 63) / 64 * 64; }
 
@@ -37,6 +43,8 @@ inline WsLayout ws_layout(int64_t m, int64_t G, int32_t block_m) {
     L.task[i] = w;
     w += round_up64(L.tid_size);
   }
+  L.split_counters = w;
+  w += kSplitUnits;
   L.words = w;
   return L;
 }
@@ -57,6 +65,7 @@ int32_t set_error(int32_t code, const char* fmt, ...);
 int32_t launch_schedule(const int32_t* group_sizes, int64_t G, const int32_t* group_offset, int64_t num_global, int64_t m,
                         int32_t block_m, int32_t align_tile, int32_t span_width, int32_t* ws, const WsLayout& L,
                         hipStream_t stream);
+int32_t device_compute_units(int* out);
 
 // ---- grouped GEMM -----------------------------------------------------------------------------
 // kFwdGlu = forward over weights [gate | up] ([g, k, 2 n_out]) with the epilogue act(gate) * up.
@@ -85,6 +94,13 @@ struct GemmParams {
   int32_t num_groups;
   int32_t n_tiles, m_tiles;         // tiles along C columns; along C rows (drhs only)
   int32_t real_slots;               // fwd/dlhs: workgroups that may own a task tile (multiple of 8 * kXcdChunk)
+  int32_t zero_wgs;                 // fwd/dlhs: workgroups after those that clear the rows of no group
+  // Split of the last round (fwd/dlhs, split_k > 1): the launch's tiles beyond the last multiple of `split_cus` are
+  // cut along the contraction into floor(split_cus / their number) parts, at most split_k; part 0 belongs to the
+  // tile's own workgroup, the others to workgroups behind the zeroing ones. f32 partial tiles in split_partials
+  // ([unit][BM * BN]), arrival counters at ws[ws_split_counters + tile].
+  int32_t split_k, split_cus, ws_split_counters;
+  float* split_partials;
   int32_t tid_size;                 // fwd/dlhs: slots of the schedule's task arrays
   int32_t grid_tile_width;
   int32_t out_dtype, activation;
@@ -100,6 +116,7 @@ struct Variant {
   const void* fn;  // __global__ void (*)(GemmParams)
   int32_t split_b; // > 0: the split pipeline (that many B stages of block_k / 2; num_stages A stages of block_k)
   const void* fn_fp8_out;  // the same kernel storing fp8 with one scale per (row, 128 columns) (GemmParams::c_scale), or null
+  const void* fn_split;    // the same kernel splitting the tiles of the last round along the contraction (GemmParams::split_k), or null
 };
 
 // ---- decode (small-m streaming kernel; int8 or 16-bit weights) -----------------------------------

@@ -1159,25 +1159,6 @@ int32_t resident_workgroups_per_cu(const void* fn, size_t lds, int* out) {
   return TKX_OK;
 }
 
-// Compute units of a device (fixed table: no allocation after the library is loaded).
-int32_t compute_units(int* out) {
-  constexpr int kMaxDevices = 64;
-  static std::mutex mu;
-  static int count[kMaxDevices] = {};
-  int dev = 0;
-  TKX_HIP_CHECK(hipGetDevice(&dev));
-  if (dev < 0 || dev >= kMaxDevices) return set_error(TKX_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
-  std::lock_guard<std::mutex> lock(mu);
-  if (count[dev] == 0) {
-    int cus = 0;
-    TKX_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    if (cus < 1) return set_error(TKX_ERR_RUNTIME, "device reports %d compute units", cus);
-    count[dev] = cus;
-  }
-  *out = count[dev];
-  return TKX_OK;
-}
-
 // The persistent kernel for (one-byte weights, depth) that keeps its registers with `wgs_per_cu` workgroups resident per
 // CU, or null: 3 per CU at depth 2 (packed int4: 4), 2 at depth 4. (The 16-bit instances spill and are not built.)
 template <int EW>
@@ -1244,7 +1225,7 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
     // placing more of them on one CU than on another. A grid the device cannot hold runs as the plain kernel.
     if (split_workspace == nullptr) return set_error(TKX_ERR_INVALID, "the persistent form needs its workspace");
     int cus = 0;
-    int32_t st = compute_units(&cus);
+    int32_t st = device_compute_units(&cus);
     if (st != TKX_OK) return st;
     const int64_t wgs = G * p.n_tiles;
     const int per_cu = (int)((wgs + cus - 1) / cus);

@@ -551,9 +551,13 @@ struct GemmKernel {
 
   // QO: the instantiation that stores fp8 with one scale per (row, 128 columns) (QOUT kernels only). It is a kernel of
   // its own so that the plain one carries none of its code or registers.
-  template <bool QO = false>
+  // Kernels that can split the tiles of a launch's last round along the contraction (GemmParams::split_k).
+  static constexpr bool SPLITK = (MODE == kFwd || MODE == kDlhs) && BM >= 128;
+  // SK: the instantiation that does (a kernel of its own, like the quantising one).
+  template <bool QO = false, bool SK = false>
   static __device__ __forceinline__ void run(const GemmParams& p, unsigned char* smem) {
     static_assert(!QO || QOUT, "this kernel has no quantising epilogue");
+    static_assert(!SK || (SPLITK && !QO), "this kernel has no split of the last round");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: all that derives from it is uniform
     const int wm = wave / WN, wn = wave % WN;
@@ -566,12 +570,33 @@ struct GemmKernel {
     const int b = blockIdx.x;
 
     int group, row0, act_start, act_end, col0, kc_begin, kc_end;
+    int part = 0, parts = 1, split_unit = 0;  // (fwd/dlhs) this workgroup contracts part `part` of `parts` of its tile
     if constexpr (MODE != kDrhs) {
       // (Group sizes are device data nobody has checked: when they add up to more than m_ext rows the schedule
       // holds more tasks than its arrays have slots for. Every task with a row below m_ext has a slot, so the rest
       // are dropped here, and the tasks kept store no row at or past m_ext.)
       const int num_tasks = min(ws[0], p.tid_size);
-      if (b >= p.real_slots) {
+      // Split of the last round: the launch's tiles beyond the last multiple of `split_cus` (a round of workgroups
+      // that would leave most CUs idle) are cut along the contraction into `parts` parts. Part 0 is the tile's own
+      // workgroup, the others are workgroups behind the zeroing ones.
+      const int total = num_tasks * p.n_tiles;
+      int first_split = total;  // list index of the first tile that is split
+      if (SK && p.split_k > 1) {
+        const int full = total / p.split_cus * p.split_cus, rem = total - full;
+        const int s = rem > 0 ? min(p.split_k, p.split_cus / rem) : 1;
+        if (s > 1) {
+          first_split = full;
+          parts = s;
+        }
+      }
+      int L = -1;
+      if (b >= p.real_slots + p.zero_wgs) {
+        if (parts < 2) return;
+        const int x = b - p.real_slots - p.zero_wgs, t = x / (parts - 1);
+        if (t >= total - first_split) return;
+        L = first_split + t;
+        part = 1 + x - t * (parts - 1);
+      } else if (b >= p.real_slots) {
         // Tail duty: rows [total_rows, m_ext), and with a group offset the rows before the first
         // group, belong to no group of this call and are defined to be zero.
         const int total_rows = min(ws[1], p.m_ext), lead_rows = min(ws[2], p.m_ext);
@@ -579,12 +604,12 @@ struct GemmKernel {
         const int64_t lo = (int64_t)total_rows * p.ldc * esz, hi = (int64_t)p.m_ext * p.ldc * esz;
         if constexpr (QO) {
           // Quantised output: rows of no group are zeros with scale 1, what quantising a row of zeros gives.
-          const int64_t per_row = p.ldc / 128, id = (int64_t)(b - p.real_slots) * THREADS + tid, step = (gridDim.x - p.real_slots) * (int64_t)THREADS;
+          const int64_t per_row = p.ldc / 128, id = (int64_t)(b - p.real_slots) * THREADS + tid, step = p.zero_wgs * (int64_t)THREADS;
           for (int64_t o = total_rows * per_row + id; o < (int64_t)p.m_ext * per_row; o += step) p.c_scale[o] = 1.f;
           for (int64_t o = id; o < (int64_t)lead_rows * per_row; o += step) p.c_scale[o] = 1.f;
         }
         unsigned char* c = reinterpret_cast<unsigned char*>(p.C);
-        const int64_t nzb = gridDim.x - p.real_slots;
+        const int64_t nzb = p.zero_wgs;
         const i32x4 z = {0, 0, 0, 0};
         const int64_t first = ((int64_t)(b - p.real_slots) * THREADS + tid) * 16;
         for (int64_t o = lo + first; o < hi; o += nzb * THREADS * 16) *reinterpret_cast<i32x4*>(c + o) = z;
@@ -600,10 +625,13 @@ struct GemmKernel {
       // an n-panel of the group's weights back to back, then the next n-panel: the tiles of a chunk
       // share panels in their XCD's L2, and neighbouring chunks share the span's lhs panels in the
       // memory-side cache.
-      const int total = num_tasks * p.n_tiles;
-      const int idx = b >> 3, xcd = b & 7;
-      const int L = ((idx / kXcdChunk) * 8 + xcd) * kXcdChunk + idx % kXcdChunk;
-      if (L >= total) return;
+      if (L < 0) {
+        const int idx = b >> 3, xcd = b & 7;
+        L = ((idx / kXcdChunk) * 8 + xcd) * kXcdChunk + idx % kXcdChunk;
+        if (L >= total) return;
+        if (L < first_split) parts = 1;
+      }
+      split_unit = (L - first_split) * parts + part;
       const int t0 = L / p.n_tiles;  // some task of the span that holds L (every task owns n_tiles list entries)
       const int first = ws[p.ws_span_first + t0], width = ws[p.ws_span_width + t0];
       const int rem = L - first * p.n_tiles;
@@ -618,6 +646,12 @@ struct GemmKernel {
       col0 = nt * BNO;
       kc_begin = 0;
       kc_end = p.k_ext;
+      if (parts > 1) {
+        // This part's share of the contraction, in whole A stages (the last part takes what is left over).
+        const int steps = (p.k_ext + BK - 1) / BK;
+        kc_begin = min((int)((int64_t)steps * part / parts) * BK, p.k_ext);
+        if (part + 1 < parts) kc_end = min((int)((int64_t)steps * (part + 1) / parts) * BK, p.k_ext);
+      }
     } else {
       const int per_group = p.m_tiles * p.n_tiles;
       group = b / per_group;
@@ -1076,6 +1110,73 @@ struct GemmKernel {
       }
     }
 
+    if constexpr (SK) if (parts > 1) {
+      // A tile in parts: every part writes its f32 sums to its slot of the workspace (stores of device scope: they go
+      // through to memory instead of staying in this XCD's L2), waits for them to complete and counts itself in at
+      // the tile's counter. Whoever arrives last adds all parts in the order of their index (its own from memory as
+      // well, so that the bits do not depend on who that is) and goes on to the epilogue; the others are done.
+      // Lane-major layout: quarter q of accumulator block (i, j) of thread t is 16 bytes at ((i TN + j) 4 + q) THREADS + t.
+      constexpr int TILE_FLOATS = BM * BN;
+      const uint32_t lane_off = (uint32_t)tid * 16u;
+      auto slot = [&](int unit) {
+        const unsigned char* ptr = uniform_pointer(reinterpret_cast<const unsigned char*>(p.split_partials + (int64_t)unit * TILE_FLOATS));
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(ptr), 0, TILE_FLOATS * 4, 0x00020000);
+      };
+      constexpr int kDeviceScope = 16;  // cache-policy operand of buffer accesses: sc1
+      {
+        const __amdgpu_buffer_rsrc_t mine = slot(split_unit);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+              __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), mine, (int)lane_off,
+                                                     ((i * TN + j) * 4 + q) * THREADS * 16, kDeviceScope);
+            }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();  // (also: every wave is done reading the last stage, whose first word carries the verdict below)
+      int* verdict = reinterpret_cast<int*>(smem);
+      if (tid == 0) {
+        int32_t* counter = const_cast<int32_t*>(ws) + p.ws_split_counters + (split_unit - part) / parts;
+        const int arrived = atomicAdd(counter, 1);
+        *verdict = arrived == parts - 1;
+        if (arrived == parts - 1) atomicExch(counter, 0);
+      }
+      __syncthreads();
+      const bool last = *verdict != 0;
+      __syncthreads();
+      if (!last) return;
+#pragma unroll 1
+      for (int pp = 0; pp < parts; ++pp) {
+        const __amdgpu_buffer_rsrc_t theirs = slot(split_unit - part + pp);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const f32x4 v = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                            theirs, (int)lane_off, ((i * TN + j) * 4 + q) * THREADS * 16, kDeviceScope));
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                if constexpr (EC == kEI8 && !SUBP) {
+                  // (int8 x int8: the registers hold the bits of exact int32 sums)
+                  // (scalar copies first: a bit cast applied to a vector's element read element 0)
+                  const float have = acc[i][j][4 * q + e], add = v[e];
+                  const int sum = __builtin_bit_cast(int, have) + __builtin_bit_cast(int, add);
+                  acc[i][j][4 * q + e] = pp == 0 ? add : __builtin_bit_cast(float, sum);
+                } else {
+                  acc[i][j][4 * q + e] = pp == 0 ? v[e] : acc[i][j][4 * q + e] + v[e];
+                }
+              }
+            }
+      }
+    }
+
     // Epilogue. After the swapped MFMA, lane l of atom (i, j) holds C row (l % 32) and, for
     // t = 0..3, columns 8t + 4*(l / 32) + {0,1,2,3} of that atom. Scales and the activation are
     // applied to the accumulators in registers first (each in one pass, with the run-time choices
@@ -1271,7 +1372,7 @@ struct GemmKernel {
                 for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * t + e];
                 unsigned char* dst = slice + (ii * 32 + (lane & 31)) * PITCH + (j * 32 + 8 * t + 4 * (lane >> 5)) * ESZ;
                 if constexpr (OUT == TKX_F8E4M3FN) {
-                  constexpr int JT = WTN > 128 ? TN / (WTN / 128) : TN;
+                  constexpr int JT = TN / (WTN > 128 ? WTN / 128 : 1);
                   const float inv = row_scale[i][j / JT];
                   float q4[4];
 #pragma unroll
@@ -1331,6 +1432,17 @@ __global__ __launch_bounds__(K::THREADS, K::THREADS <= 256 ? 2 : 1) void gemm_en
   extern __shared__ __attribute__((aligned(1024))) unsigned char tkx_smem[];
   K::template run<true>(p, tkx_smem);
 }
+template <class K>
+__global__ __launch_bounds__(K::THREADS, K::THREADS <= 256 ? 2 : 1) void gemm_entry_split(const GemmParams p) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char tkx_smem[];
+  K::template run<false, true>(p, tkx_smem);
+}
+// The entry that splits the last round of a kernel that has one, else null.
+template <class K>
+const void* split_entry() {
+  if constexpr (K::SPLITK) return reinterpret_cast<const void*>(&gemm_entry_split<K>);
+  else return nullptr;
+}
 // The quantising entry of a kernel that has one, else null.
 template <class K>
 const void* fp8_out_entry() {
@@ -1342,14 +1454,16 @@ const void* fp8_out_entry() {
   {                                                                                                            \
     MODE, EA, EB, BM, BN, BK, WM, WN, NS, ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>::SMEM_BYTES, \
         reinterpret_cast<const void*>(&::tkx::gemm_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>>), HB, \
-        ::tkx::fp8_out_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>>()                       \
+        ::tkx::fp8_out_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>>(),                      \
+        ::tkx::split_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS, HB>>()                         \
   }
 
 #define TKX_VARIANT(MODE, EA, EB, BM, BN, BK, WM, WN, NS)                                            \
   {                                                                                                  \
     MODE, EA, EB, BM, BN, BK, WM, WN, NS, ::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>::SMEM_BYTES, \
         reinterpret_cast<const void*>(&::tkx::gemm_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>>), 0, \
-        ::tkx::fp8_out_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>>()                        \
+        ::tkx::fp8_out_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>>(),                       \
+        ::tkx::split_entry<::tkx::GemmKernel<MODE, EA, EB, BM, BN, BK, WM, WN, NS>>()                          \
   }
 
 }  // namespace tkx

@@ -43,12 +43,14 @@ __global__ __launch_bounds__(kThreads) void schedule_kernel(const int32_t* __res
                                                              int32_t span_width, int32_t* __restrict__ ws,
                                                              int64_t off_offsets, int64_t off_gid, int64_t off_bstart,
                                                              int64_t off_astart, int64_t off_aend, int64_t off_swb,
-                                                             int64_t off_asize, int64_t off_sfirst, int64_t off_swidth) {
+                                                             int64_t off_asize, int64_t off_sfirst, int64_t off_swidth,
+                                                             int64_t off_split_counters) {
   extern __shared__ int32_t smem[];
   int32_t* scan_buf = smem;                         // 2*kThreads
   int32_t* starts = smem + 2 * kThreads;            // G+1 : exclusive cumsum of clamped sizes
   int32_t* start_tasks = starts + (G + 1);          // G+1 : exclusive cumsum of blocks per group
   const int t = threadIdx.x;
+  for (int i = t; i < kSplitUnits; i += kThreads) ws[off_split_counters + i] = 0;  // arrival counters of a split launch
   const int per = (G + kThreads - 1) / kThreads;
   const int lo = min(t * per, G), hi = min(lo + per, G);
 
@@ -156,7 +158,8 @@ int32_t launch_schedule(const int32_t* group_sizes, int64_t G, const int32_t* gr
   if (num_global < 0 || num_global > 0x7fffffffLL) return set_error(TKX_ERR_INVALID, "bad number of group sizes");
   schedule_kernel<<<1, kThreads, smem, stream>>>(group_sizes, (int32_t)G, group_offset, (int32_t)num_global, block_m, L.tid_size, align_tile,
                                                 span_width < 1 ? 1 : span_width, ws, L.offsets, L.task[0], L.task[1],
-                                                L.task[2], L.task[3], L.task[4], L.task[5], L.task[6], L.task[7]);
+                                                L.task[2], L.task[3], L.task[4], L.task[5], L.task[6], L.task[7],
+                                                L.split_counters);
   TKX_HIP_CHECK(hipGetLastError());
   return TKX_OK;
 }

@@ -38,8 +38,9 @@ class Config:
   (block_m, block_n, block_k, waves_m, waves_n, num_stages) selects a precompiled kernel variant;
   `grid_tile_width` m-tasks share one n-panel of rhs in launch order (L2 reuse);
   `align_tile` is the row alignment of task starts (the reference's `align_tile`, default 8);
-  `split_k` workgroups share the contraction of one output tile (the reference's field of that name; here the
-  streaming small-m kernel, block_m == 16, is the one that takes values above 1);
+  `split_k` workgroups share the contraction of one output tile (the reference's field of that name): on the streaming
+  small-m kernel (block_m == 16) every tile is split; on a tiled forward / dlhs kernel of at least 128 rows only the
+  tiles of the launch's last, partial round of workgroups are, into at most that many parts;
   `persistent` (the reference's flag of that name, pallas_mosaic_gpu_common.py:55; here a count): above 0 the streaming
   small-m kernel runs as that many resident workgroups per compute unit, each with an equal share of the weight bytes
   of the non-empty tiles, instead of one workgroup per (group, column tile).
@@ -67,6 +68,21 @@ class Config:
   def to_kernel_config(self) -> hip_ops.KernelConfig:
     return hip_ops.KernelConfig(self.block_m, self.block_n, self.block_k, self.waves_m, self.waves_n,
                                 self.num_stages, self.grid_tile_width, self.align_tile, self.split_k, self.persistent)
+
+
+_COMPUTE_UNITS = 256  # of an MI355X: a launch's tiles run in rounds of that many
+
+
+def _tiled_split_pays(mode: int, block_m: int, block_n: int, rows: int, cols: int, num_groups: int) -> bool:
+  """Whether a tiled forward / dlhs launch gets `split_k` (the tiles of its last, partial round of workgroups are cut
+  along the contraction; the kernel itself decides into how many parts, and leaves a round that is more than half full
+  alone). Measured on the backward product of the Mixtral shape (m = 4096: 2.4 rounds of 128 x 256 tiles): +23 %; on
+  the forward pass at m = 16384 (14.4 rounds) the exchange of partial tiles costs what the shorter round saves, so
+  launches of 8 rounds and more stay as they are. Tiles of at least 128 rows have the kernels for it."""
+  if mode not in (0, 1) or block_m < 128:
+    return False
+  tiles = (-(-rows // block_m) + (num_groups - 1) // 2) * -(-cols // block_n)
+  return tiles < 8 * _COMPUTE_UNITS
 
 
 def _streaming_split(tiles: int, contraction: int, block_n: int, depth: int) -> int:
@@ -674,17 +690,23 @@ class HipRaggedDot(base.RaggedDot):
     if bm == 16:
       width = 1  # the streaming small-m kernel has no tile order to tune
       split_k = _streaming_split(num_groups * -(-cols // bn), contraction, bn, ns)
+    elif _tiled_split_pays(mode, bm, bn, rows, cols, num_groups):
+      split_k = 4
     return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns, grid_tile_width=width,
                   align_tile=8, split_k=split_k)
 
   def _get_autotuning_configs(self, ba: op.BoundArguments) -> set[Config]:
     mode, key = self._problem(ba)[:2]
     configs = set()
+    problem = self._problem(ba)
     for bm, bn, bk, wm, wn, ns in _variant_table().get(key, []):
       widths = (1,) if (mode == 2 or bm == 16) else (1, 2, 4, 8, 16)
       for w in widths:
         configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns,
                            grid_tile_width=w))
+        if _tiled_split_pays(mode, bm, bn, problem[3], problem[4], problem[2]):
+          configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns,
+                             grid_tile_width=w, split_k=4))
       if bm == 16 and bn == 128 and ns <= 4:
         _, _, num_groups, _, cols, contraction, _ = self._problem(ba)
         for split_k in (2, 4, 8):

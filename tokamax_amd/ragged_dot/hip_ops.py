@@ -94,8 +94,19 @@ def _group_sizes_i32(group_sizes: torch.Tensor) -> torch.Tensor:
   return group_sizes.contiguous()
 
 
-def workspace(m: int, num_groups: int, block_m: int, device) -> torch.Tensor:
+def workspace(m: int, num_groups: int, block_m: int, device, block_n: int = 0, split_k: int = 1) -> torch.Tensor:
+  """The schedule workspace of a tiled call; with split_k > 1 the partial tiles of the split last round behind it."""
+  if split_k > 1:
+    return torch.empty(_split_workspace_words(m, num_groups, block_m, block_n), dtype=torch.int32, device=device)
   return torch.empty(_workspace_words(m, num_groups, block_m), dtype=torch.int32, device=device)
+
+
+@functools.lru_cache(maxsize=1024)
+def _split_workspace_words(m: int, num_groups: int, block_m: int, block_n: int) -> int:
+  nbytes = _lib.load().tkx_ragged_dot_split_workspace_bytes(m, num_groups, block_m, block_n)
+  if nbytes < 0:
+    raise ValueError(f"bad sizes m={m} G={num_groups} block_m={block_m} block_n={block_n}")
+  return nbytes // 4
 
 
 _SPLIT_WORKSPACES: dict = {}
@@ -231,7 +242,7 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
     if ws is None:
       ws = _UNUSED_WORKSPACES[lhs.device] = torch.empty(64, dtype=torch.int32, device=lhs.device)
   else:
-    ws = workspace(m, G, config.block_m, lhs.device)
+    ws = workspace(m, G, config.block_m, lhs.device, config.block_n, config.split_k)
   cfg = config.to_c()
   with _on_device(lhs.device):
     if rhs_bias is None and not gateup and scale_blocks == 1 and group_offset is None:
@@ -340,7 +351,8 @@ def ragged_dot_fwd_fp8_out(lhs, rhs, group_sizes, *, config: KernelConfig, lhs_s
   out = torch.empty((m, n), dtype=torch.float8_e4m3fn, device=lhs.device)
   out_scale = torch.empty((m, n // 128), dtype=torch.float32, device=lhs.device)
   ws = workspace(m, G, config.block_m, lhs.device)
-  cfg = config.to_c()
+  # (The quantising epilogue needs a row's 128 columns complete in one workgroup: no split last round here.)
+  cfg = dataclasses.replace(config, split_k=1).to_c()
   with _on_device(lhs.device):
     st = lib.tkx_ragged_dot_fwd_fp8_out(_ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(out),
                                         _ptr(out_scale), _ptr(ws), m, k, n, G, dtype_code(lhs.dtype), dtype_code(rhs.dtype),
