@@ -1276,7 +1276,7 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
     // Half the registers of int8 per step in flight: the same occupancy one depth further.
     fn = depth <= 2   ? decode_fn<kEI4, 2, 4>(sk)
          : depth <= 4 ? decode_fn<kEI4, 4, 4>(sk)
-                      : reinterpret_cast<const void*>(&decode_kernel<kEI4, 8, 3>);
+                      : reinterpret_cast<const void*>(&decode_kernel<kEI4, 8, 2>);  // (3 workgroups per CU would spill)
   } else if (sub && rhs_dtype == TKX_F8E4M3FN) {
     fn = depth <= 2 ? decode_fn<kEF8, 2, 3, true>(sk) : decode_fn<kEF8, 4, 2, true>(sk);
   } else if (rhs_dtype == TKX_F8E4M3FN) {

@@ -547,6 +547,10 @@ struct GemmKernel {
   // stage is already being refilled, so they live in a ring of NS + 1 slots behind the stages.
   static constexpr int RING_SLOT = SUBP ? (BN + BM) * 4 : 0;
   static constexpr int SMEM_BYTES = SPLIT ? NS * StageA::BYTES + HB * StageB::BYTES : NS * STAGE_BYTES + (NS + 1) * RING_SLOT;
+  // Workgroups the register budget is set for: two 4-wave workgroups share a CU when their LDS fits twice (256
+  // registers per lane each); every other shape has the CU, and a SIMD's 512 registers per lane, to itself or to the
+  // two waves of one 8-wave workgroup.
+  static constexpr int kWorkgroupsPerCu = THREADS <= 256 && 2 * SMEM_BYTES <= 160 * 1024 ? 2 : 1;
   static_assert(NS >= 2 && SMEM_BYTES <= 160 * 1024, "stages must fit the 160 KB LDS");
 
   // QO: the instantiation that stores fp8 with one scale per (row, 128 columns) (QOUT kernels only). It is a kernel of
@@ -1154,7 +1158,10 @@ struct GemmKernel {
       for (int pp = 0; pp < parts; ++pp) {
         const __amdgpu_buffer_rsrc_t theirs = slot(split_unit - part + pp);
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i) {
+          // (One row block's loads in flight at a time: all of a part's at once need as many registers again as the
+          // accumulators they are added to.)
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -1174,6 +1181,7 @@ struct GemmKernel {
                 }
               }
             }
+        }
       }
     }
 
@@ -1258,26 +1266,31 @@ struct GemmKernel {
         }
       }
       if (p.activation != TKX_ACT_NONE) {
-        auto for_all = [&](auto fn) {
-#pragma unroll
-          for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TNO; ++j)  // (gate-up: the gate blocks only)
-#pragma unroll
-              for (int e = 0; e < 16; ++e) acc[i][j][e] = fn(acc[i][j][e]);
-        };
         // tanh(x) = 1 - 2 / (exp(2x) + 1): a handful of instructions per element with the hardware
         // exponential and reciprocal.
         auto fast_tanh = [](float x) { return 1.f - 2.f * __builtin_amdgcn_rcpf(__expf(2.f * x) + 1.f); };
-        if (p.activation == TKX_ACT_RELU) for_all([](float x) { return x > 0.f ? x : 0.f; });
-        else if (p.activation == TKX_ACT_TANH) for_all(fast_tanh);
-        else if (p.activation == TKX_ACT_SILU || p.activation == TKX_ACT_SILU_CLAMP)
-          for_all([](float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-x)); });
-        else if (p.activation == TKX_ACT_SWIGLU_OAI)
-          for_all([](float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-1.702f * x)); });
-        else if (p.activation == TKX_ACT_SIGMOID) for_all([](float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); });
-        else if (p.activation == TKX_ACT_GELU_TANH)
-          for_all([&](float x) { return 0.5f * x * (1.f + fast_tanh(0.7978845608028654f * (x + 0.044715f * x * x * x))); });
+        // Block by block, with the choice of the function inside: one choice around all blocks made every
+        // accumulator meet again after six branches, and the register allocator spilled one of them on the way.
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TNO; ++j) {  // (gate-up: the gate blocks only)
+            f32x16 c = acc[i][j];
+            auto apply = [&](auto fn) {
+#pragma unroll
+              for (int e = 0; e < 16; ++e) c[e] = fn(c[e]);
+            };
+            if (p.activation == TKX_ACT_RELU) apply([](float x) { return x > 0.f ? x : 0.f; });
+            else if (p.activation == TKX_ACT_TANH) apply(fast_tanh);
+            else if (p.activation == TKX_ACT_SILU || p.activation == TKX_ACT_SILU_CLAMP)
+              apply([](float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-x)); });
+            else if (p.activation == TKX_ACT_SWIGLU_OAI)
+              apply([](float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-1.702f * x)); });
+            else if (p.activation == TKX_ACT_SIGMOID) apply([](float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); });
+            else if (p.activation == TKX_ACT_GELU_TANH)
+              apply([&](float x) { return 0.5f * x * (1.f + fast_tanh(0.7978845608028654f * (x + 0.044715f * x * x * x))); });
+            acc[i][j] = c;
+          }
       }
       if constexpr (GLU) {
         // act(gate) * up: block j and block j + TNO of a lane are gate and up of the same output columns.
@@ -1421,19 +1434,19 @@ struct GemmKernel {
   }
 };
 
-// (4-wave workgroups: at most 256 registers per lane, so that two of them fit a CU when their LDS does.)
+// (4-wave workgroups whose LDS lets two of them share a CU: at most 256 registers per lane, so that two do fit.)
 template <class K>
-__global__ __launch_bounds__(K::THREADS, K::THREADS <= 256 ? 2 : 1) void gemm_entry(const GemmParams p) {
+__global__ __launch_bounds__(K::THREADS, K::kWorkgroupsPerCu) void gemm_entry(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char tkx_smem[];
   K::run(p, tkx_smem);
 }
 template <class K>
-__global__ __launch_bounds__(K::THREADS, K::THREADS <= 256 ? 2 : 1) void gemm_entry_fp8_out(const GemmParams p) {
+__global__ __launch_bounds__(K::THREADS, K::kWorkgroupsPerCu) void gemm_entry_fp8_out(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char tkx_smem[];
   K::template run<true>(p, tkx_smem);
 }
 template <class K>
-__global__ __launch_bounds__(K::THREADS, K::THREADS <= 256 ? 2 : 1) void gemm_entry_split(const GemmParams p) {
+__global__ __launch_bounds__(K::THREADS, K::kWorkgroupsPerCu) void gemm_entry_split(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char tkx_smem[];
   K::template run<false, true>(p, tkx_smem);
 }
