@@ -401,12 +401,37 @@ def main():
     src_ = torch.zeros(1 << 28, dtype=torch.int32, device=device)
     dst_ = torch.empty_like(src_)
     t_cp, _, _ = _time_steps(lambda: dst_.copy_(src_), steps, warm, stream)
-    extras["ceilings_same_box"] = dict(
+    ceilings = dict(
         dense_bf16_matmul_nn_tflops=round(dense_flops / (t_nn / steps) / 1e9, 1),
         dense_bf16_matmul_nt_tflops=round(dense_flops / (t_nt / steps) / 1e9, 1),
         copy_1gib_read_plus_write_gbs=round(2 * (1 << 30) / (t_cp / steps) / 1e6, 1),
         note="torch.matmul [16384,4096] x [4096,14336] bf16 (random normal data) and torch copy_ of 1 GiB, HIP-event timed")
-    del a_, b_nn, b_nt, c_, src_, dst_
+    del b_nn, c_, src_, dst_
+    # The vendor's dense fp8 GEMM (e4m3fn x e4m3fn -> bf16, one scale per tensor) at the same shape, where this torch
+    # build has it for the device; it takes the weights k-contiguous (the NT layout).
+    try:
+      a8, b8 = a_.to(torch.float8_e4m3fn), b_nt.to(torch.float8_e4m3fn)
+      one = torch.ones((), device=device, dtype=torch.float32)
+      f8 = lambda: torch._scaled_mm(a8, b8.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+      t_f8, _, _ = _time_steps(f8, steps, warm, stream)
+      ceilings["dense_fp8_scaled_mm_nt_tflops"] = round(dense_flops / (t_f8 / steps) / 1e9, 1)
+      del a8, b8
+    except Exception as e:  # (not built for this device, or another signature: the ceiling is simply not reported)
+      ceilings["dense_fp8_scaled_mm_nt_tflops"] = None
+      ceilings["dense_fp8_note"] = f"torch._scaled_mm not usable here: {type(e).__name__}"
+    del a_, b_nt
+    # The chip's own ceilings by the probes of libtkx_microbench.so: the matrix cores on a register-resident MFMA
+    # loop (the clock they settle at depends on the operand bits), and the operand stream of a tiled GEMM without
+    # arithmetic, by how many workgroups of an XCD share a panel.
+    try:
+      from tokamax_amd import microbench
+      ceilings["mfma_only_bf16_zeros_tflops"] = round(microbench.mfma_bf16_tflops("zeros", device), 1)
+      ceilings["mfma_only_bf16_random_tflops"] = round(microbench.mfma_bf16_tflops("random", device), 1)
+      for share in (1, 8, 32):
+        ceilings[f"operand_stream_into_lds_share{share}_tbs"] = round(microbench.operand_stream_tbs(share, device), 2)
+    except (RuntimeError, OSError) as e:
+      ceilings["microbench_note"] = f"libtkx_microbench.so not usable: {e}"
+    extras["ceilings_same_box"] = ceilings
 
     w = workloads.make("decode", device, seed=0)
     gs = torch.tensor(w.group_sizes, device=device)

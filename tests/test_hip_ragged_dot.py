@@ -896,7 +896,7 @@ def test_small_m_call_replayed_from_a_captured_graph(groups, n, device):
 
 @pytest.mark.parametrize("dtype,cfg", [
     (torch.bfloat16, (256, 256, 64, 2, 4, 3)), (torch.bfloat16, (256, 256, 32, 2, 4, 4)), (torch.bfloat16, (128, 128, 64, 2, 2, 4)),
-    (torch.bfloat16, (64, 128, 64, 2, 2, 4)), (torch.float8_e4m3fn, (128, 256, 128, 2, 4, 3))])
+    (torch.bfloat16, (64, 128, 64, 2, 2, 4)), (torch.float8_e4m3fn, (128, 256, 128, 2, 4, 3)), (torch.float8_e4m3fn, (256, 256, 128, 2, 4, 2))])
 def test_fp8_output_quantised_in_the_epilogue(dtype, cfg, device):
   """tkx_ragged_dot_fwd_fp8_out: values and scales are those of the absmax quantisation (oracle, in the reciprocal
   form of the reference's fused epilogue) of the f32 result of the same kernel, bit for bit; rows of no group are

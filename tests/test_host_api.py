@@ -41,6 +41,20 @@ def test_library_loads_and_exports_every_declared_symbol():
   assert _lib.load().tkx_version() == 2000  # 2000: TkxConfig.persistent (1001: split_k)
 
 
+def test_probe_library_loads_and_exports_every_declared_symbol():
+  """The ceiling probes bench.py times (a library of their own: nothing of the operator depends on it)."""
+  from tokamax_amd import microbench
+  header = open(os.path.join(ROOT, "include", "tkx_microbench.h")).read()
+  declared = set(re.findall(r"\b(tkxmb_[a-z_0-9]+)\s*\(", header))
+  assert declared == set(microbench.EXPORTED_SYMBOLS)
+  lib = ctypes.CDLL(microbench.LIB_PATH)
+  for name in declared:
+    assert hasattr(lib, name), name
+  assert microbench.load().tkxmb_operand_stream_bytes(2 << 20) == 2048 * (2 << 20)
+  for module in ("hip", "hip_ops", "api", "base"):
+    assert "microbench" not in open(os.path.join(ROOT, "tokamax_amd", "ragged_dot", module + ".py")).read()
+
+
 def test_workspace_layout_queries():
   lib = _lib.load()
   assert lib.tkx_ragged_dot_tid_size(1024, 8, 128) == 1024 // 128 + 8 - 1

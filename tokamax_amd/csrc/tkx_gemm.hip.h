@@ -144,15 +144,20 @@ __device__ __forceinline__ i32x4 i8x8_to_bf16x8(i32x2 v) {
   return out;
 }
 
-// Fragment of one 32-wide atom at row/column base `rc0`, contraction atom `kk`.
+// Fragment of one 32-wide atom at row/column base `rc0` + `rc_step`, contraction atom `kk`.
 //   ES = storage element kind in LDS, EC = compute (MFMA) kind.
+// `rc_step` (a multiple of 16) is the part of the base that is a compile-time constant at the call (the wave's
+// row block i sits i * WM * 32 rows below its first). A contraction-contiguous tile's swizzle looks at row bits
+// 0..3 only, so those rows add a constant number of bytes to the address: kept apart from the lane's part, the
+// constant goes into the read instruction's offset field and the blocks of a wave share their address registers.
 template <int LAYOUT, int ES, int EC, int ROW_BYTES>
-__device__ __forceinline__ typename Mma<EC>::Frag load_frag(const unsigned char* tile, int rc0, int kk, int lane) {
+__device__ __forceinline__ typename Mma<EC>::Frag load_frag(const unsigned char* tile, int rc0, int kk, int lane, int rc_step = 0) {
   typedef typename Mma<EC>::Frag Frag;
   constexpr int KA = Mma<EC>::KA;
   if constexpr (LAYOUT == kKC) {
     static_assert(ES == EC, "contraction-contiguous operands are stored in the compute type");
     const int row = rc0 + (lane & 31), q = lane >> 5;
+    tile += rc_step * ROW_BYTES;
     if constexpr (EC == kEF8) {
       const int c0 = kk * 4 + q * 2;
       i32x4 lo = lds_read_b128(tile, kc_offset<ROW_BYTES>(row, c0));
@@ -165,6 +170,7 @@ __device__ __forceinline__ typename Mma<EC>::Frag load_frag(const unsigned char*
       return lds_read_b128(tile, kc_offset<ROW_BYTES>(row, kk * 2 + q));
     }
   } else {
+    rc0 += rc_step;
     const int kb = kk * KA;
     if constexpr (ES == kEF32) {
       const int col = rc0 + (lane & 31), q = lane >> 5;
@@ -533,6 +539,11 @@ struct GemmKernel {
   static constexpr int TNO = MODE == kFwdGlu ? TN / 2 : TN, WTNO = MODE == kFwdGlu ? WTN / 2 : WTN;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % KA == 0, "tile does not split into 32x32 atoms");
   static constexpr int KSTEPS = BKC / KA;
+  // Lean fragments: the 32-byte fragments of the fp8 MFMA, double-buffered for a 4 x 2 wave tile, take 96 registers
+  // next to 128 accumulators. The lhs fragments are then kept once: row block i's is re-read for the next atom right
+  // after the atom's last MFMA on it (TM * TN - TN MFMAs of 64 cycles before its next use); the two rhs fragments stay
+  // double-buffered.
+  static constexpr bool LEAN = EA == kEF8 && EB == kEF8 && !SUBK && !SPLIT && TM * TN >= 8;
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
   static_assert(!SPLIT || (MODE == kFwd && EA == EB && BK % 2 == 0), "split pipeline: plain forward, operands of one type");
   typedef TileStage<LA, EA, BM, BK, THREADS> StageA;
@@ -779,7 +790,7 @@ struct GemmKernel {
           if (r >= TM + TN) return;
           const int f = r == 0 ? 0 : r <= TN ? TM + r - 1 : r - TN;
           if (f < TM) {
-            if (f < NV) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(atile, row_block(f) * 32, akk, lane);
+            if (f < NV) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(atile, wm * 32, akk, lane, f * WM * 32);
           } else {
             if (NV > 0) b[f - TM] = load_frag<LB, EB, EC, StageB::ROW_BYTES>(btile, wn * WTN + (f - TM) * 32, bkk, lane);
           }
@@ -947,9 +958,9 @@ struct GemmKernel {
       // never left waiting behind a block of memory instructions.
       auto k_loop = [&](auto nv_tag) {
         constexpr int NV = decltype(nv_tag)::value;  // row blocks of this wave that hold rows of the task
-        Frag fa[2][TM], fb[2][TN];
+        Frag fa[LEAN ? 1 : 2][TM], fb[2][TN];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[0][i] = fa[1][i] = Frag{};
+        for (int i = 0; i < TM; ++i) fa[0][i] = fa[LEAN ? 0 : 1][i] = Frag{};
 #pragma unroll
         for (int j = 0; j < TN; ++j) fb[0][j] = fb[1][j] = Frag{};
         // Read number r of an atom, in the order the atom's MFMAs (row block major) first use the
@@ -960,7 +971,7 @@ struct GemmKernel {
           if (r >= TM + TN) return;
           const int f = r == 0 ? 0 : r <= TN ? TM + r - 1 : r - TN;
           if (f < TM) {
-            if (f < NV) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, row_block(f) * 32, kk, lane);
+            if (f < NV) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, wm * 32, kk, lane, f * WM * 32);
           } else if (f < TM + TN) {
             if (NV > 0) b[f - TM] = load_b_frag(stage, f - TM, kk);
           }
@@ -990,8 +1001,14 @@ struct GemmKernel {
               if (i < NV) acc[i][j] = mma_atom<EC>(b[j], a[i], acc[i][j]);
             }
             if (reads) {
+              if constexpr (LEAN) {
+                // rhs fragment t after MFMA t; the lhs fragment of a row block after the block's last MFMA
+                if (t < TN) read_frag(na, nb, t + 1, rd_stage, rd_kk);
+                if (j == TN - 1) read_frag(na, nb, i == 0 ? 0 : TN + i, rd_stage, rd_kk);
+              } else {
 #pragma unroll
-              for (int r = 0; r < RPM; ++r) read_frag(na, nb, t * RPM + r, rd_stage, rd_kk);
+                for (int r = 0; r < RPM; ++r) read_frag(na, nb, t * RPM + r, rd_stage, rd_kk);
+              }
             }
             if (loads) {
 #pragma unroll
@@ -1039,14 +1056,14 @@ struct GemmKernel {
           } else {
 #pragma unroll
             for (int kk = 0; kk + 1 < KSTEPS; ++kk)
-              atom(std::true_type{}, std::false_type{}, fa[kk & 1], fb[kk & 1], fa[(kk + 1) & 1], fb[(kk + 1) & 1], cur,
-                   kk + 1, none, std::false_type{});
+              atom(std::true_type{}, std::false_type{}, fa[LEAN ? 0 : kk & 1], fb[kk & 1], fa[LEAN ? 0 : (kk + 1) & 1],
+                   fb[(kk + 1) & 1], cur, kk + 1, none, std::false_type{});
           }
           // All LDS reads of `cur` are issued. After the barrier the next stage is complete and `cur`
           // is free: the last atom's MFMAs cover the first fragment reads of the next stage and the
           // issue of the loads that refill `cur` with k-step kt + NS.
           step_barrier(decltype(refill_tag)::value || kt + NS - 1 < nfull);
-          atom(more_tag, refill_tag, fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1], fa[0], fb[0], nxt, 0, sp, std::false_type{});
+          atom(more_tag, refill_tag, fa[LEAN ? 0 : (KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1], fa[0], fb[0], nxt, 0, sp, std::false_type{});
           if constexpr (SUBP) if (block_end) {
             // Fold the products into the result with the scales of their k-block: lane l holds row l % 32
             // and, for t = 0..3, columns 8 t + 4 (l / 32) + {0..3} of every 32 x 32 block.

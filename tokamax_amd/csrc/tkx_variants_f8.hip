@@ -5,9 +5,8 @@
 namespace tkx {
 #define FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEF8, kEF8, BM, BN, BK, WM, WN, NS)
 
-// (No 256 x 256 tile: the 32-byte fragments of the fp8 MFMA on top of 128 accumulator registers leave the k loop
-// short of registers at two waves per SIMD, and it reloads spilled values in every k-step.)
 static const Variant kVariants[] = {
+    FWD(256, 256, 128, 2, 4, 2),  // (lhs fragments kept once, GemmKernel::LEAN: 32-byte fragments next to 128 accumulators)
     FWD(128, 256, 128, 2, 4, 3),
     FWD(128, 128, 128, 2, 2, 4),
     FWD(64, 128, 128, 2, 2, 4),
