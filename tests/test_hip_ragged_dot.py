@@ -1907,3 +1907,16 @@ def test_fp8_output_quantisation(activation, device):
   again = op_q(a, b, group_sizes=gst, preferred_element_type=torch.float8_e4m3fn, activation=activation)
   assert torch.equal(again.qvalue.view(torch.uint8), out.qvalue.view(torch.uint8)) and torch.equal(again.scale, out.scale)
   assert OP(a, b, group_sizes=gst, preferred_element_type=torch.float8_e4m3fn).dtype == torch.bfloat16
+
+
+def test_ceiling_probes_run_and_give_plausible_figures(device):
+  """The probes bench.py times beside the operator (libtkx_microbench.so): the matrix cores alone are faster on
+  constant operands than on random ones and stay below the published peak; a panel shared by 32 workgroups of an XCD
+  streams into LDS several times faster than one nobody shares."""
+  from tokamax_amd import microbench
+  zeros = microbench.mfma_bf16_tflops("zeros", device, iters=4000)
+  random = microbench.mfma_bf16_tflops("random", device, iters=4000)
+  assert 800 < random < zeros < 2600, (random, zeros)
+  alone = microbench.operand_stream_tbs(1, device)    # 1 GB of panels: past the 256 MB memory-side cache
+  shared = microbench.operand_stream_tbs(32, device)
+  assert 1.0 < alone < 9.0 and shared > 2 * alone, (alone, shared)

@@ -637,6 +637,33 @@ def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   assert c.block_m >= 128
 
 
+def test_heuristics_split_the_last_round_of_tiled_launches_with_few_rounds():
+  """A tiled forward / dlhs launch of fewer than 8 rounds of 256 workgroups gets `split_k` = 4 (the kernel cuts only
+  the tiles of a partial last round, and decides into how many parts); longer launches, drhs, gate-up fusion and tiles
+  of fewer than 128 rows do not; the search space offers both forms where the heuristics split."""
+  op = hip.HipRaggedDot()
+  bf16 = torch.bfloat16
+  gs = lambda groups: ShapeDtype((groups,), torch.int32)
+  assert hip._tiled_split_pays(1, 128, 256, 4096, 4096, 8) and not hip._tiled_split_pays(0, 256, 256, 16384, 14336, 8)
+  assert not hip._tiled_split_pays(2, 256, 256, 4096, 4096, 8) and not hip._tiled_split_pays(0, 64, 128, 512, 512, 8)
+  vjp_dlhs = op.bind(ShapeDtype((4096, 14336), bf16), ShapeDtype((8, 4096, 14336), bf16), group_sizes=gs(8),
+                     ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS)
+  c = op._get_heuristics_config(vjp_dlhs)
+  assert c.block_m >= 128 and c.split_k == 4
+  space = op._get_autotuning_configs(vjp_dlhs)
+  assert any(x.split_k == 4 for x in space) and any(x.split_k == 1 and x.block_m == c.block_m for x in space)
+  assert all(x.split_k == 1 for x in space if x.block_m < 128)
+  mixtral = op.bind(ShapeDtype((16384, 4096), bf16), ShapeDtype((8, 4096, 14336), bf16), group_sizes=gs(8))
+  assert op._get_heuristics_config(mixtral).split_k == 1
+  assert all(x.split_k == 1 for x in op._get_autotuning_configs(mixtral) if x.block_m != 16)
+  drhs = op.bind(ShapeDtype((4096, 4096), bf16), ShapeDtype((4096, 14336), bf16), group_sizes=gs(8),
+                 ragged_dot_dimension_numbers=base.RAGGED_CONTRACTING_DOT_DIM_NUMS)
+  assert op._get_heuristics_config(drhs).split_k == 1
+  glu = op.bind(ShapeDtype((2048, 1024), bf16), ShapeDtype((8, 1024, 2048), bf16), group_sizes=gs(8),
+                fuse_gateup_activation="silu")
+  assert op._get_heuristics_config(glu).split_k == 1
+
+
 def test_bind_without_inspect_matches_the_signature_path():
   """`RaggedDot.bind` names every parameter of `_fwd` itself and skips `inspect`; the result is the one
   `Signature.bind` + `apply_defaults` gives, in signature order, and unknown or missing names still fail."""
