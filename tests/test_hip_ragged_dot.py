@@ -1920,3 +1920,73 @@ def test_ceiling_probes_run_and_give_plausible_figures(device):
   alone = microbench.operand_stream_tbs(1, device)    # 1 GB of panels: past the 256 MB memory-side cache
   shared = microbench.operand_stream_tbs(32, device)
   assert 1.0 < alone < 9.0 and shared > 2 * alone, (alone, shared)
+
+
+def test_repeated_eager_calls_take_the_remembered_launch(device):
+  """The operator's shortcut for repeated eager calls: same bits as the full path, taken only for calls that are one
+  forward launch on the caller's own tensors, and never when a gradient is wanted."""
+  rng = np.random.default_rng(11)
+  G, m, k, n = 8, 64, 1024, 256
+  gs = np.array([3, 0, 9, 1, 0, 20, 7, 5], np.int32)
+  gst = torch.tensor(gs, device=device)
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  q = tokamax_amd.QArray(torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device),
+                         torch.tensor((rng.random((G, 1, n)) * 0.01 + 0.001).astype(np.float32), device=device))
+  op = tokamax_amd.HipRaggedDot()
+  first = op(lhs, q, group_sizes=gst, preferred_element_type=torch.bfloat16)
+  plans = op.__dict__["_plans"]
+  assert len(plans) == 1
+  again = op(lhs, q, group_sizes=gst, preferred_element_type=torch.bfloat16)
+  assert torch.equal(again, first) and again.data_ptr() != first.data_ptr() and len(plans) == 1
+  want = O.ragged_dot(_np(lhs), O.dequantize(q.qvalue.cpu().numpy(), _np(q.scale)), gs, acc_dtype=np.float64, out_dtype="f64")
+  _check(again, want, 3e-3)
+  # other buffers of the same shapes, and group sizes updated in place: the launch reads what it is given
+  lhs2 = (lhs.float() * 0.5).to(torch.bfloat16)
+  gst.copy_(torch.tensor(gs[::-1].copy(), device=device))
+  out2 = op(lhs2, q, group_sizes=gst, preferred_element_type=torch.bfloat16)
+  fresh = tokamax_amd.HipRaggedDot()(lhs2, q, group_sizes=gst, preferred_element_type=torch.bfloat16)
+  assert torch.equal(out2, fresh) and len(plans) == 1
+  # another shape, another output type: plans of their own
+  op(lhs[:32], q, group_sizes=torch.tensor(gs // 2, device=device), preferred_element_type=torch.bfloat16)
+  op(lhs, q, group_sizes=gst, preferred_element_type=torch.float32)
+  assert len(plans) == 3
+  # calls that are more than one launch on the caller's tensors are not remembered: int64 group sizes (converted),
+  # scales per k-block that need widening first, an activation given as a callable
+  n_before = len(plans)
+  a = op(lhs2, q, group_sizes=gst.to(torch.int64), preferred_element_type=torch.bfloat16)
+  assert torch.equal(a, out2)
+  blocks = tokamax_amd.QArray(q.qvalue, q.scale.expand(G, 4, n).contiguous() * torch.arange(1, 5, device=device).view(1, 4, 1))
+  big = torch.tensor(rng.normal(0, 1, (2048, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  gs_big = torch.full((G,), 256, dtype=torch.int32, device=device)
+  b1 = op(big, blocks, group_sizes=gs_big, preferred_element_type=torch.bfloat16)
+  b2 = op(big, blocks, group_sizes=gs_big, preferred_element_type=torch.bfloat16)
+  assert torch.equal(b1, b2)
+  c = op(lhs2, q, group_sizes=gst, preferred_element_type=torch.bfloat16, activation=torch.relu)
+  assert torch.equal(c, torch.relu(out2))
+  assert len(plans) <= n_before + 1  # (the k-block call may be one launch of a variant of its own; the others are not)
+  # a gradient: the full path with its custom VJP
+  lhs_g = lhs.float().clone().to(torch.bfloat16).requires_grad_(True)
+  w = torch.tensor(rng.normal(0, k ** -0.5, (G, k, n)).astype(np.float32), device=device).to(torch.bfloat16)
+  op(lhs_g.detach(), w, group_sizes=gst)
+  op(lhs_g.detach(), w, group_sizes=gst)  # remembered
+  out = op(lhs_g, w, group_sizes=gst)
+  out.backward(torch.ones_like(out))
+  assert lhs_g.grad is not None and torch.count_nonzero(lhs_g.grad) > 0
+  with torch.no_grad():
+    assert torch.equal(op(lhs_g, w, group_sizes=gst), out)
+  # a change of the cached autotuning data forgets nothing but asks again
+  from tokamax_amd import op as op_lib
+  key_before = op._plan_key(lhs, q, dict(group_sizes=gst, preferred_element_type=torch.bfloat16))
+  op_lib.bump_config_epoch()
+  assert op._plan_key(lhs, q, dict(group_sizes=gst, preferred_element_type=torch.bfloat16)) != key_before
+  assert torch.equal(op(lhs2, q, group_sizes=gst, preferred_element_type=torch.bfloat16), out2)
+  # while an autotuning run records the ops a function calls, every call is a full one
+  token = op_lib.OP_CALL_RECORDER.set([])
+  try:
+    assert op._plan_key(lhs, q, dict(group_sizes=gst)) is None
+  finally:
+    op_lib.OP_CALL_RECORDER.reset(token)
+  # the public entry point goes through the same op objects
+  r1 = tokamax_amd.ragged_dot(lhs, w, gst)
+  r2 = tokamax_amd.ragged_dot(lhs, w, gst)
+  assert torch.equal(r1, r2)

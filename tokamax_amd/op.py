@@ -214,6 +214,11 @@ _CONFIG_EPOCH = [0]
 _FWD_PARAMETER_NAMES: dict = {}
 
 
+def config_epoch() -> int:
+  """The counter that `bump_config_epoch` advances (for callers that memoise on top of the resolved config)."""
+  return _CONFIG_EPOCH[0]
+
+
 def bump_config_epoch() -> None:
   _CONFIG_EPOCH[0] += 1
 

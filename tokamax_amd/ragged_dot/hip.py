@@ -419,6 +419,48 @@ def _concrete_operand(x):
   return quantization.as_array_or_qarray_without_zero_point(x)
 
 
+_PLAIN_ARGUMENT_TYPES = (bool, int, float, str, torch.dtype, base.RaggedDotDimensionNumbers)
+
+
+def _make_plan(records, out, lhs, rhs, group_sizes):
+  """The shortcut for calls like the one that left `records` and returned `out`, or None if that call was more than
+  one forward launch on the caller's own buffers."""
+  if len(records) != 1 or not isinstance(records[0], hip_ops.ForwardLaunch) or records[0].out is not out:
+    return None
+  record = records[0]
+
+  def leaves(lhs, rhs, group_sizes):
+    return ((lhs,) if type(lhs) is torch.Tensor else (lhs.qvalue, lhs.scale)) + \
+           ((rhs,) if type(rhs) is torch.Tensor else (rhs.qvalue, rhs.scale)) + (group_sizes,)
+
+  given = [t.data_ptr() for t in leaves(lhs, rhs, group_sizes)]
+  if 0 in given or len(set(given)) != len(given):
+    return None
+  source = []  # for every pointer of the launch: which of the caller's tensors it was, -1 for an absent operand
+  for p in record.pointers:
+    if p == 0:
+      source.append(-1)
+    elif p in given:
+      source.append(given.index(p))
+    else:
+      return None  # (a buffer this call made itself: a widened or repeated operand, converted group sizes)
+  source = tuple(source)
+  launch, new_workspace = record.launch, record.new_workspace
+  shape, dtype, device = tuple(out.shape), out.dtype, out.device
+
+  def plan(lhs, rhs, group_sizes):
+    tensors = leaves(lhs, rhs, group_sizes)
+    result = torch.empty(shape, dtype=dtype, device=device)
+    ws = new_workspace()
+    status = launch([0 if i < 0 else tensors[i].data_ptr() for i in source], result.data_ptr(), ws.data_ptr(),
+                    torch.cuda.current_stream(device).cuda_stream)
+    if status != 0:
+      _lib.check(status)
+    return result
+
+  return plan
+
+
 @dataclasses.dataclass(frozen=True)
 class HipRaggedDot(base.RaggedDot):
   """Hand-written HIP ragged dot for gfx950. Physical layout `mk,gkn->mn`, rhs never transposed."""
@@ -434,6 +476,72 @@ class HipRaggedDot(base.RaggedDot):
       # A fresh op per call avoids infinite recursion (pallas_mosaic_gpu.py:95-100).
       fn = lambda *a, **kw: HipRaggedDot()(*a, **kw)  # pylint: disable=unnecessary-lambda
       object.__setattr__(self, "vjp", partial(base.vjp, dlhs_ragged_dot=fn, drhs_ragged_dot=fn))
+
+  # -- eager fast path -------------------------------------------------------------------------
+  def __call__(self, lhs, rhs, *, return_residuals: bool = False, **kwargs):
+    """The operator call (`Op.__call__`) with a shortcut for repeated eager calls: a call that came down to one
+    forward launch on the caller's own tensors (no pass over an operand in front of it, nothing applied to the result
+    behind it, no gradient wanted) is remembered under the shapes, types and arguments it was made with, and the next
+    call of that kind goes straight to the C ABI: allocate the result, pass the addresses. Binding, the choice of a
+    config and the routing cost about 45 us of Python per call, more than the small-m kernels take."""
+    key = None if return_residuals else self._plan_key(lhs, rhs, kwargs)
+    plans = self.__dict__.get("_plans")
+    if key is not None and plans is not None:
+      plan = plans.get(key)
+      if plan is not None:
+        return plan(lhs, rhs, kwargs["group_sizes"])
+    if key is None:
+      return super().__call__(lhs, rhs, return_residuals=return_residuals, **kwargs)
+    log = hip_ops.LAUNCH_LOG
+    outer, log.records = log.records, []
+    try:
+      out = super().__call__(lhs, rhs, **kwargs)
+      records = log.records
+    finally:
+      log.records = outer
+    if outer is not None:
+      outer.extend(records)
+    plan = _make_plan(records, out, lhs, rhs, kwargs["group_sizes"])
+    if plan is not None:
+      if plans is None or len(plans) > 64:
+        plans = {}
+        object.__setattr__(self, "_plans", plans)
+      plans[key] = plan
+    return out
+
+  def _plan_key(self, lhs, rhs, kwargs):
+    """What a remembered launch depends on, or None for a call that always takes the full path."""
+    if self.checkify_group_sizes or op.OP_CALL_RECORDER.get() is not None:
+      return None
+    group_sizes = kwargs.get("group_sizes")
+    if type(group_sizes) is not torch.Tensor or not group_sizes.is_cuda:
+      return None
+    grad = torch.is_grad_enabled()
+    parts = []
+    for x in (lhs, rhs):
+      if type(x) is torch.Tensor:
+        leaves = (x,)
+      elif type(x) is QArray and x.zero_point is None:
+        leaves = (x.qvalue, x.scale)
+        parts.append(x.qtype)
+      else:
+        return None
+      for t in leaves:
+        if type(t) is not torch.Tensor or not t.is_cuda or (grad and t.requires_grad):
+          return None
+        parts.append((t.shape, t.dtype, t.is_contiguous()))
+    parts.append((group_sizes.shape, group_sizes.dtype, group_sizes.is_contiguous(), lhs.device if type(lhs) is torch.Tensor
+                  else lhs.qvalue.device))
+    for name, v in kwargs.items():
+      if name == "group_sizes":
+        continue
+      if not (v is None or type(v) in _PLAIN_ARGUMENT_TYPES):
+        return None  # (tensors, callables: the full path)
+      parts.append((name, v))
+    parts.append((op.config_epoch(), config_lib.autotuning_cache_miss_fallback.value,
+                  config_lib.ignore_autotuning_cache.value, id(op.AUTOTUNING_CACHE_OVERLAY_STACK.get()),
+                  torch.cuda.current_device()))
+    return tuple(parts)
 
   # -- forward ---------------------------------------------------------------------------------
   def _fwd(

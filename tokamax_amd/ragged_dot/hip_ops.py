@@ -9,6 +9,7 @@ import contextlib
 import ctypes
 import dataclasses
 import functools
+import threading
 
 import torch
 
@@ -24,6 +25,34 @@ _DTYPE_CODE = {
 }
 
 SCHEDULE_FIELDS = ("group_id", "block_start", "actual_start", "actual_end", "start_within_block", "actual_size")
+
+
+class _LaunchLog(threading.local):
+  """What the functions of this module launched while a caller was listening (`records` is a list then): a
+  `ForwardLaunch` for a forward call, None for anything else (a pass over an operand, a quantisation, drhs). The
+  operator's eager fast path reads it to learn whether a call came down to one forward launch on the caller's own
+  tensors, which it can then repeat without the planning in front of it."""
+  records = None
+
+
+LAUNCH_LOG = _LaunchLog()
+
+
+def _log_launch(entry) -> None:
+  if LAUNCH_LOG.records is not None:
+    LAUNCH_LOG.records.append(entry)
+
+
+@dataclasses.dataclass
+class ForwardLaunch:
+  """One forward launch, repeatable on other buffers of the same shapes: `launch(pointers, out_ptr, ws_ptr, stream)`
+  with `pointers` in the order of `POINTER_NAMES` (0 for an absent operand) returns the C status."""
+
+  POINTER_NAMES = ("lhs", "rhs", "group_sizes", "group_offset", "lhs_scale", "rhs_scale", "rhs_bias")
+  pointers: tuple          # the addresses this launch was made with, in that order
+  launch: object
+  out: torch.Tensor        # the result it returned (for the caller to recognise it)
+  new_workspace: object    # () -> the int32 workspace tensor of a repeat
 
 
 def dtype_code(dtype: torch.dtype) -> int:
@@ -232,38 +261,50 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
     if rhs_bias.numel() != G * n:
       raise NotImplementedError("rhs bias must be one value per (group, column)")
   out_cols = k if trans_rhs else n // 2 if gateup else n
-  out = torch.empty((m, out_cols), dtype=out_dtype, device=lhs.device)
+  device = lhs.device
+  out = torch.empty((m, out_cols), dtype=out_dtype, device=device)
   if config.block_m == 16 and (config.split_k > 1 or config.persistent > 0):
-    ws = split_workspace(m, n, config.split_k, lhs.device, config.persistent)
+    new_workspace = lambda: split_workspace(m, n, config.split_k, device, config.persistent)
   elif config.block_m == 16:
     # The streaming kernel without a split touches no workspace (the entry point only wants a pointer): one
     # allocation per device, not one per call.
-    ws = _UNUSED_WORKSPACES.get(lhs.device)
-    if ws is None:
-      ws = _UNUSED_WORKSPACES[lhs.device] = torch.empty(64, dtype=torch.int32, device=lhs.device)
+    unused = _UNUSED_WORKSPACES.get(device)
+    if unused is None:
+      unused = _UNUSED_WORKSPACES[device] = torch.empty(64, dtype=torch.int32, device=device)
+    new_workspace = lambda: unused
   else:
-    ws = workspace(m, G, config.block_m, lhs.device, config.block_n, config.split_k)
-  cfg = config.to_c()
-  with _on_device(lhs.device):
-    if rhs_bias is None and not gateup and scale_blocks == 1 and group_offset is None:
-      st = lib.tkx_ragged_dot_fwd(
-          _ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(out), _ptr(ws), m, k, n, G,
-          dtype_code(lhs.dtype), dtype_code(rhs.dtype), dtype_code(out_dtype),
-          _lib.TKX_MODE_TRANS_RHS if trans_rhs else _lib.TKX_MODE_DEFAULT, _lib.ACTIVATIONS[activation],
-          ctypes.byref(cfg), _stream(lhs.device))
-    else:
-      st = lib.tkx_ragged_dot_fwd_fused(
-          _ptr(lhs), _ptr(rhs), _ptr(gs), _ptr(group_offset), _ptr(lhs_scale), _ptr(rhs_scale), _ptr(rhs_bias), _ptr(out),
-          _ptr(ws), m, k, n, G, gs.numel(), scale_blocks, dtype_code(lhs.dtype), dtype_code(rhs.dtype),
-          dtype_code(out_dtype), _lib.ACTIVATIONS[activation], 1 if gateup else 0, ctypes.byref(cfg), _stream(lhs.device))
+    new_workspace = lambda: workspace(m, G, config.block_m, device, config.block_n, config.split_k)
+  ws = new_workspace()
+  cfg = ctypes.byref(config.to_c())
+  a_code, b_code, o_code = dtype_code(lhs.dtype), dtype_code(rhs.dtype), dtype_code(out_dtype)
+  act_code = _lib.ACTIVATIONS[activation]
+  # (Addresses go to the C ABI as plain integers: the declared argument types convert them.)
+  if rhs_bias is None and not gateup and scale_blocks == 1 and group_offset is None:
+    mode = _lib.TKX_MODE_TRANS_RHS if trans_rhs else _lib.TKX_MODE_DEFAULT
+    fwd = lib.tkx_ragged_dot_fwd
+
+    def launch(p, out_ptr, ws_ptr, stream):
+      return fwd(p[0], p[1], p[2], p[4], p[5], out_ptr, ws_ptr, m, k, n, G, a_code, b_code, o_code, mode, act_code, cfg, stream)
+  else:
+    num_sizes, glu = gs.numel(), 1 if gateup else 0
+    fused = lib.tkx_ragged_dot_fwd_fused
+
+    def launch(p, out_ptr, ws_ptr, stream):
+      return fused(p[0], p[1], p[2], p[3], p[4], p[5], p[6], out_ptr, ws_ptr, m, k, n, G, num_sizes, scale_blocks, a_code,
+                   b_code, o_code, act_code, glu, cfg, stream)
+  pointers = tuple(0 if t is None else t.data_ptr() for t in (lhs, rhs, gs, group_offset, lhs_scale, rhs_scale, rhs_bias))
+  with _on_device(device):
+    st = launch(pointers, out.data_ptr(), ws.data_ptr(), torch.cuda.current_stream(device).cuda_stream)
   _lib.check(st)
   if workspace_out is not None:
     workspace_out.append(ws)
+  _log_launch(ForwardLaunch(pointers, launch, out, new_workspace))
   return out
 
 
 def dequantize_weights(qvalue: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
   """bf16 [g,k,n] = int8 qvalue [g,k,n] * scale [g, k/t_k, n] repeated t_k times along k (quantization.py:80-83)."""
+  _log_launch(None)
   _require_cuda(qvalue, scale)
   lib = _lib.load()
   if qvalue.dim() != 3 or scale.dim() != 3 or qvalue.dtype != torch.int8:
@@ -296,6 +337,7 @@ def quantize(x: torch.Tensor, qtype: torch.dtype, tile_shape, bound: float | Non
   x f32, bf16 or f16: [rows, cols] with tiles one row tall and a multiple of 8 columns wide, or several rows tall and
   1, 8, 16, ... or 256 columns wide; or weights [g, k, n] with a tile (1, t_k, t_n) (taken as g * k rows). qtype int8,
   fp8 (e4m3fn) or a sub-byte integer (int4: values in [-7, 7], kept in int8 storage)."""
+  _log_launch(None)
   _require_cuda(x)
   lib = _lib.load()
   if qtype not in _QMAX:
@@ -328,6 +370,7 @@ def ragged_dot_fwd_fp8_out(lhs, rhs, group_sizes, *, config: KernelConfig, lhs_s
   """(qvalue fp8 [m,n], scale f32 [m, n/128]) of lhs[m,k] . rhs[g,k,n], quantised per (row, 128 columns) in the
   kernel's epilogue (`tkx_ragged_dot_fwd_fp8_out`): bf16 x bf16 or fp8 x fp8 with one scale per row / per (group,
   column), n % 128 == 0, a tiled variant. NotImplementedError where the library has no such kernel."""
+  _log_launch(None)
   _require_cuda(lhs, rhs, group_sizes, lhs_scale, rhs_scale)
   lib = _lib.load()
   if lhs.dim() != 2 or rhs.dim() != 3:
@@ -373,6 +416,7 @@ def pack_int4(values: torch.Tensor) -> torch.Tensor:
 
 
 def _int4_repack(x: torch.Tensor, unpack: bool) -> torch.Tensor:
+  _log_launch(None)
   _require_cuda(x)
   want = torch.uint8 if unpack else torch.int8
   if x.dtype != want or x.dim() < 2 or x.shape[-1] % 16 or (not unpack and x.shape[-2] % 2):
@@ -396,6 +440,7 @@ def dequantize(qvalue: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tens
 
   qvalue int8 or fp8 (e4m3fn): [rows, cols] with scale [rows/t_r, cols/t_c], or weights [g,k,n] with scale
   [g, k/t_k, n/t_n]; t_c / t_n is 1 or a multiple of 16. `zero_point`, if given, has the scale's shape."""
+  _log_launch(None)
   _require_cuda(qvalue, scale, zero_point)
   lib = _lib.load()
   if qvalue.dtype not in (torch.int8, torch.float8_e4m3fn) or qvalue.dim() not in (2, 3) or scale.dim() != qvalue.dim():
@@ -429,6 +474,7 @@ def dequantize(qvalue: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tens
 def ragged_dot_drhs(lhs, dout, group_sizes, num_groups: int, *, config: KernelConfig,
                     out_dtype: torch.dtype) -> torch.Tensor:
   """out[g,k,n] = lhs[rows_g,k]^T . dout[rows_g,n]."""
+  _log_launch(None)
   _require_cuda(lhs, dout, group_sizes)
   lib = _lib.load()
   if lhs.dim() != 2 or dout.dim() != 2 or lhs.shape[0] != dout.shape[0]:
