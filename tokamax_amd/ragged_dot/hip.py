@@ -428,6 +428,8 @@ def _make_plan(records, out, lhs, rhs, group_sizes):
   if len(records) != 1 or not isinstance(records[0], hip_ops.ForwardLaunch) or records[0].out is not out:
     return None
   record = records[0]
+  if out.device.index != torch.cuda.current_device():
+    return None  # (the launch ran under a device guard; the shortcut has none)
 
   def leaves(lhs, rhs, group_sizes):
     return ((lhs,) if type(lhs) is torch.Tensor else (lhs.qvalue, lhs.scale)) + \
