@@ -1990,3 +1990,20 @@ def test_repeated_eager_calls_take_the_remembered_launch(device):
   r1 = tokamax_amd.ragged_dot(lhs, w, gst)
   r2 = tokamax_amd.ragged_dot(lhs, w, gst)
   assert torch.equal(r1, r2)
+
+
+def test_split_workspace_is_never_released_when_a_call_needs_a_larger_one(device):
+  """A HIP graph captured earlier holds the address of the workspace its split call used: when a later call on the
+  same stream needs more room, the old buffer stays referenced (and keeps its address) next to the new one."""
+  stream = torch.cuda.Stream(device)  # a stream of its own, so that no other test's workspace is in the way
+  with torch.cuda.stream(stream):
+    small = hip_ops.split_workspace(16, 1024, 4, device)
+    assert hip_ops.split_workspace(16, 1024, 2, device) is small  # room enough: the same buffer
+    address, words = small.data_ptr(), small.numel()
+    assert torch.count_nonzero(small) == 0  # the arrival counters start at zero
+    big = hip_ops.split_workspace(16, 1024, 1, device, persistent=1)
+    assert big is not small and big.numel() * 4 >= _lib.load().tkx_ragged_dot_decode_persistent_workspace_bytes()
+    assert any(t is small for t in hip_ops._SUPERSEDED_WORKSPACES)
+    assert small.data_ptr() == address and small.numel() == words
+    assert hip_ops.split_workspace(16, 1024, 4, device) is big  # later calls share the larger one
+  stream.synchronize()
