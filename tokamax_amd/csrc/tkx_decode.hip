@@ -1121,15 +1121,8 @@ int32_t raise_dynamic_lds(const void* fn, size_t bytes) {
 
 // Steps by which a helper wave's share is smaller than a home wave's, so that its partial tiles are in memory before
 // the home workgroup looks for them (a wave of a workgroup that shares a CU with two others takes about 2 us for a
-// step of 4 KB), at most a fifth of a wave's share of a tile.
-int32_t g_persistent_margin = -1;  // (>= 0: set through TKX_DECODE_MARGIN, for tuning runs)
+// step of 4 KB), 4 steps (the best of 0..8 measured on the 2048-deep decode shape), at most a quarter of a wave's share of a tile.
 int32_t persistent_margin_steps(int64_t k) {
-  if (g_persistent_margin < 0) {
-    const char* e = getenv("TKX_DECODE_MARGIN");
-    g_persistent_margin = e != nullptr ? atoi(e) : 1 << 20;
-    if (g_persistent_margin < 0) g_persistent_margin = 0;
-  }
-  if (g_persistent_margin < (1 << 20)) return g_persistent_margin;
   const int64_t steps = k / kDecKS / kDecWaves;
   int64_t margin = 4;
   if (margin > steps / 4) margin = steps / 4;
@@ -1244,9 +1237,6 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
       int resident = 0;
       st = resident_workgroups_per_cu(fn, lds, &resident);
       if (st != TKX_OK) return st;
-      if (getenv("TKX_DEBUG") != nullptr)
-        fprintf(stderr, "tkx: persistent decode: %lld workgroups, %d CUs, %d per CU wanted, %d resident with %zu bytes of LDS\n",
-                (long long)wgs, cus, per_cu, resident, lds);
       if (resident < per_cu) fn = nullptr;
     }
     if (fn != nullptr) {
