@@ -427,6 +427,7 @@ def main():
       from tokamax_amd import microbench
       ceilings["mfma_only_bf16_zeros_tflops"] = round(microbench.mfma_bf16_tflops("zeros", device), 1)
       ceilings["mfma_only_bf16_random_tflops"] = round(microbench.mfma_bf16_tflops("random", device), 1)
+      ceilings["mfma_only_fp8_random_tflops"] = round(microbench.mfma_fp8_tflops("random", device), 1)
       for share in (1, 8, 32):
         ceilings[f"operand_stream_into_lds_share{share}_tbs"] = round(microbench.operand_stream_tbs(share, device), 2)
     except (RuntimeError, OSError) as e:

@@ -19,6 +19,11 @@ int32_t tkxmb_mfma_bf16(const void* operands, int32_t iters, void* sink, void* s
 /* FLOP of one such launch on the current device. */
 int64_t tkxmb_mfma_bf16_flops(int32_t iters);
 
+/* The same loop on v_mfma_scale_f32_32x32x64_f8f6f4 with e4m3fn operands and no block scales (`operands`: 64 KB
+ * of fp8 bytes), and its FLOP per launch. */
+int32_t tkxmb_mfma_fp8(const void* operands, int32_t iters, void* sink, void* stream);
+int64_t tkxmb_mfma_fp8_flops(int32_t iters);
+
 /* 2048 workgroups of 8 waves; each streams one region of `region_bytes` (a multiple of 8192) out of `regions`
  * (a multiple of 8) consecutive ones at `src` into LDS with direct-to-LDS loads, 8 KB outstanding per wave; `share`
  * (1..32) workgroups that run on one XCD at the same time read the same region. */

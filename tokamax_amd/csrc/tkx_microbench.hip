@@ -57,6 +57,41 @@ __global__ __launch_bounds__(kThreads) void mfma_loop(const i32x4* src, float* o
   if (s == 12345.f) out[0] = s;  // keeps the loop alive
 }
 
+// The same loop on the fp8 (e4m3fn) form of the MFMA, 32x32x64 with 32-byte fragments and no block scales.
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+__global__ __launch_bounds__(kThreads) void mfma_fp8_loop(const i32x4* src, float* out, int iters) {
+  constexpr int NA = 4, NB = 2;
+  i32x8 a[NA], b[NB];
+  for (int i = 0; i < NA; ++i) {
+    const i32x4 lo = src[(threadIdx.x + kThreads * i) % kOperandWords], hi = src[(threadIdx.x * 3 + kThreads * i + 77) % kOperandWords];
+    a[i] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  }
+  for (int i = 0; i < NB; ++i) {
+    const i32x4 lo = src[(threadIdx.x * 7 + kThreads * i + 1234) % kOperandWords], hi = src[(threadIdx.x * 5 + kThreads * i + 4321) % kOperandWords];
+    b[i] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  }
+  f32x16 acc[NA][NB];
+  for (int i = 0; i < NA; ++i)
+    for (int j = 0; j < NB; ++j)
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i], b[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+    if ((it & 7) == 7) {
+      const i32x8 t = a[0];
+      for (int i = 0; i + 1 < NA; ++i) a[i] = a[i + 1];
+      a[NA - 1] = t;
+    }
+  }
+  float s = 0;
+  for (int i = 0; i < NA; ++i)
+    for (int j = 0; j < NB; ++j)
+      for (int e = 0; e < 16; ++e) s += acc[i][j][e];
+  if (s == 12345.f) out[0] = s;
+}
+
 // Workgroup b runs on XCD b % 8; `share` consecutive workgroups of one XCD take the same region. A wave keeps
 // INFLIGHT 1 KB loads outstanding.
 template <int INFLIGHT>
@@ -91,6 +126,16 @@ int32_t tkxmb_mfma_bf16(const void* operands, int32_t iters, void* sink, void* s
   int cus = 0;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, 0) != hipSuccess) return 3;
   mfma_loop<<<cus, kThreads, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const i32x4*>(operands), static_cast<float*>(sink), iters);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+int64_t tkxmb_mfma_fp8_flops(int32_t iters) { return 4 * tkxmb_mfma_bf16_flops(iters); }  // 32 x 32 x 64 against 32 x 32 x 16
+
+int32_t tkxmb_mfma_fp8(const void* operands, int32_t iters, void* sink, void* stream) {
+  if (operands == nullptr || sink == nullptr || iters < 1) return 1;
+  int cus = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, 0) != hipSuccess) return 3;
+  mfma_fp8_loop<<<cus, kThreads, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const i32x4*>(operands), static_cast<float*>(sink), iters);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 

@@ -11,7 +11,7 @@ import os
 import torch
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libtkx_microbench.so")
-EXPORTED_SYMBOLS = ("tkxmb_mfma_bf16", "tkxmb_mfma_bf16_flops", "tkxmb_operand_stream", "tkxmb_operand_stream_bytes")
+EXPORTED_SYMBOLS = ("tkxmb_mfma_bf16", "tkxmb_mfma_bf16_flops", "tkxmb_mfma_fp8", "tkxmb_mfma_fp8_flops", "tkxmb_operand_stream", "tkxmb_operand_stream_bytes")
 
 _lib = None
 
@@ -25,6 +25,8 @@ def load():
     i32, i64, vp = ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p
     lib.tkxmb_mfma_bf16.restype, lib.tkxmb_mfma_bf16.argtypes = i32, [vp, i32, vp, vp]
     lib.tkxmb_mfma_bf16_flops.restype, lib.tkxmb_mfma_bf16_flops.argtypes = i64, [i32]
+    lib.tkxmb_mfma_fp8.restype, lib.tkxmb_mfma_fp8.argtypes = i32, [vp, i32, vp, vp]
+    lib.tkxmb_mfma_fp8_flops.restype, lib.tkxmb_mfma_fp8_flops.argtypes = i64, [i32]
     lib.tkxmb_operand_stream.restype, lib.tkxmb_operand_stream.argtypes = i32, [vp, i64, i32, i32, vp]
     lib.tkxmb_operand_stream_bytes.restype, lib.tkxmb_operand_stream_bytes.argtypes = i64, [i64]
     _lib = lib
@@ -60,6 +62,22 @@ def mfma_bf16_tflops(data: str, device, iters: int = 20000, repeats: int = 3) ->
       raise RuntimeError("tkxmb_mfma_bf16 failed")
 
   return lib.tkxmb_mfma_bf16_flops(iters) / _timed(launch, repeats) / 1e9
+
+
+def mfma_fp8_tflops(data: str, device, iters: int = 10000, repeats: int = 3) -> float:
+  """TFLOP/s of the register-resident fp8 (e4m3fn) MFMA loop on operands that are all `"zeros"` or `"random"`."""
+  lib = load()
+  gen = torch.Generator(device=device).manual_seed(0)
+  operands = (torch.zeros(65536, device=device, dtype=torch.uint8) if data == "zeros"
+              else torch.randn(65536, device=device, generator=gen).to(torch.float8_e4m3fn).view(torch.uint8))
+  sink = torch.zeros(16, device=device, dtype=torch.float32)
+  stream = torch.cuda.current_stream(device).cuda_stream
+
+  def launch():
+    if lib.tkxmb_mfma_fp8(operands.data_ptr(), iters, sink.data_ptr(), stream) != 0:
+      raise RuntimeError("tkxmb_mfma_fp8 failed")
+
+  return lib.tkxmb_mfma_fp8_flops(iters) / _timed(launch, repeats) / 1e9
 
 
 def operand_stream_tbs(share: int, device, region_bytes: int = 2 << 20, regions: int = 512, repeats: int = 3) -> float:
