@@ -293,9 +293,11 @@ int32_t tkx_pack_int4(const void* values, void* packed, int64_t packed_rows, int
  * [-qmax - 1, qmax] with a bound above qmax.
  * x f32, bf16 or f16 [rows, cols] row-major; qvalue int8 or fp8 [rows, cols]; scale f32
  * [rows / scale_block_rows, cols / scale_block_cols]. Tiles: one row tall and a multiple of 8 columns wide (an lhs with
- * one scale per row, scale_block_cols = cols, or per (row, k-block)); or several rows tall and 1, 8, 16, ... or 256
- * columns wide (weights [g, k, n] as g * k rows: (k, 1) is one scale per (group, column), (t_k, 1) the scale tile
- * (1, t_k, 1), (128, 128) square blocks; a tile wider than 256 columns, e.g. one scale per tensor, is not taken).
+ * one scale per row, scale_block_cols = cols, or per (row, k-block)); or several rows tall and 1 column or a multiple
+ * of 8 columns wide (weights [g, k, n] as g * k rows: (k, 1) is one scale per (group, column), (t_k, 1) the scale tile
+ * (1, t_k, 1), (128, 128) square blocks, (rows, cols) one scale for the whole array). Tiles of 8, 16, ... 256 columns
+ * are reduced inside one workgroup; wider ones, and widths that are not a power of two, take three passes that collect
+ * each tile's maximum in its `scale` slot with an atomic maximum (the result does not depend on the order).
  * cols % 8 == 0. */
 int32_t tkx_quantize(const void* x, void* qvalue, float* scale, int64_t rows, int64_t cols, int64_t scale_block_rows,
                      int64_t scale_block_cols, int32_t x_dtype, int32_t q_dtype, float qmax, float bound,

@@ -258,10 +258,15 @@ def test_quantized_int8_weights(b_tile_shape, supported, device):
     count = int(gs.sum())
     _check(out, want.numpy(), TOL["int8"], rows=count)
     np.testing.assert_allclose(_np(out)[:count], want.numpy()[:count], atol=0.01, rtol=0.005)  # test_base.py:240-242
-  # One scale for a whole tensor is a tile wider than the quantisation kernel takes (tiles several rows tall are at most
-  # 256 columns wide, include/tkx_ragged_dot.h on tkx_quantize): declined, so that another implementation may take it.
-  with pytest.raises(NotImplementedError):
-    tokamax_amd.ragged_dot(a, tokamax_amd.AsQArray(q.to(torch.bfloat16), torch.int8), gst)
+  # An `AsQArray` without tiling: one scale for the whole tensor (quantised on the device, then repeated per column).
+  w = torch.tensor(rng.normal(0, k ** -0.5, (G, k, n)).astype(np.float32), device=device).to(torch.bfloat16)
+  out = tokamax_amd.ragged_dot(a, tokamax_amd.AsQArray(w, torch.int8), gst, preferred_element_type=torch.float32)
+  wq, ws = O.quantize_absmax(_np(w), "int8", (G, k, n))
+  assert ws.shape == (1, 1, 1)
+  want = O.ragged_dot(_np(a), O.dequantize(wq, ws), gs, acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, TOL["int8"], rows=int(gs.sum()))
+  with pytest.raises(NotImplementedError):  # a tile over several groups that does not span their contraction
+    hip_ops.quantize(w, torch.int8, (2, 16, 1))
 
 
 def test_fp8_with_row_and_column_scales(device):
@@ -1785,7 +1790,11 @@ def _dequantized(q):
 @pytest.mark.parametrize("shape,tile", [((96, 256), (1, 128)), ((96, 256), (1, 16)), ((96, 256), (1, 256)), ((300, 4096), (1, 4096)),
                                         ((512, 256), (256, 1)), ((512, 256), (16, 1)), ((256, 384), (128, 128)),
                                         ((8, 256, 512), (1, 256, 1)), ((8, 256, 512), (1, 16, 1)), ((8, 256, 512), (1, 1, 16)),
-                                        ((3, 128, 264), (1, 128, 8)), ((40, 2880), (1, 2880)), ((64, 8), (1, 8))])
+                                        ((3, 128, 264), (1, 128, 8)), ((40, 2880), (1, 2880)), ((64, 8), (1, 8)),
+                                        # tiles several rows tall that one workgroup does not reduce: one scale per tensor,
+                                        # 512-column and 96-column blocks, whole groups of a weight array, all of it
+                                        ((96, 512), (96, 512)), ((64, 1024), (32, 512)), ((96, 384), (48, 96)),
+                                        ((4, 64, 768), (2, 64, 384)), ((4, 64, 384), (4, 64, 384))])
 def test_quantize_kernel_bit_exact(shape, tile, qtype, xdtype, device):
   """`tkx_quantize` against the oracle's absmax quantisation: the same values and the same scales, bit for bit, for the
   tile shapes of the reference's quantised tests (test_base.py:187-192) and a few more; an all-zero tile included."""

@@ -629,13 +629,12 @@ int32_t tkx_quantize(const void* x, void* qvalue, float* scale, int64_t rows, in
     return set_error(TKX_ERR_INVALID, "scale blocks %lldx%lld do not tile %lldx%lld", (long long)scale_block_rows,
                      (long long)scale_block_cols, (long long)rows, (long long)cols);
   if (cols % 8 != 0 || cols > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "cols must be a multiple of 8");
-  const bool pow2 = (scale_block_cols & (scale_block_cols - 1)) == 0;
   if (scale_block_rows == 1) {
     if (scale_block_cols % 8 != 0) return set_error(TKX_ERR_UNSUPPORTED, "tiles one row tall must be a multiple of 8 columns wide");
   } else {
     if (scale_block_rows > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "scale block too tall");
-    if (scale_block_cols != 1 && !(pow2 && scale_block_cols >= 8 && scale_block_cols <= 256))
-      return set_error(TKX_ERR_UNSUPPORTED, "tiles several rows tall must be 1, 8, 16, ... or 256 columns wide (got %lld)",
+    if (scale_block_cols != 1 && scale_block_cols % 8 != 0)
+      return set_error(TKX_ERR_UNSUPPORTED, "tiles several rows tall must be 1 column or a multiple of 8 columns wide (got %lld)",
                        (long long)scale_block_cols);
     if (scale_block_cols == 1 && cols % 4 != 0) return set_error(TKX_ERR_UNSUPPORTED, "cols must be a multiple of 4");
   }

@@ -8,12 +8,14 @@
 // tokamax/_src/quantization.py:65-78 asks of qwix.quantize, in the form the reference states it itself for its fused
 // output quantisation (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:802-822). x is f32, bf16 or f16, row-major.
 //
-// Two kernels, both bound by HBM (the second read of a tile comes from cache):
+// Three forms, all bound by HBM (the second read of a tile comes from cache where the tile is small):
 //   * tiles one row tall (an lhs [m, k] with one scale per row or per (row, t_c columns)): a group of lanes owns a
 //     tile, 8 elements per lane and step, and reduces with lane shuffles;
 //   * tiles several rows tall (weights [g, k, n] as g * k rows with one scale per (group, column) or per
 //     (t_r rows, column) or per (t_r x t_c) block): a workgroup owns t_r rows x 256 columns, 8 row slices of 32 lanes x
-//     8 columns each, and reduces through LDS.
+//     8 columns each, and reduces through LDS;
+//   * any other tile several rows tall (one scale for a whole tensor, 512-column blocks, ...): the tile's maximum is
+//     collected with an atomic maximum on its bit pattern, then a second pass converts.
 #include "tkx_common.h"
 #include "tkx_gemm.hip.h"
 
@@ -191,6 +193,75 @@ __global__ __launch_bounds__(kQThreads) void quantize_blocks_kernel(const unsign
   }
 }
 
+// Any other tile several rows tall (wider than 256 columns, or not a power of two wide; t_c a multiple of 8): three
+// passes over chunks of 8 consecutive elements, which never straddle a tile. (1) The tile's scale slot collects the bit
+// pattern of max |x| with an integer atomic maximum (non-negative floats order like their bits; the result does not
+// depend on the order of arrival); a wave whose chunks all lie in one tile reduces with shuffles first. (2) The slot
+// becomes the scale. (3) The values are divided and converted. The slots are zeroed by the first kernel of the three.
+__global__ void tile_slots_clear_kernel(float* __restrict__ scale, int64_t num_tiles) {
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < num_tiles; t += (int64_t)gridDim.x * blockDim.x) scale[t] = 0.f;
+}
+
+__device__ __forceinline__ int64_t tile_of_chunk(int64_t chunk, int32_t chunks_per_row, int32_t t_r, int32_t t_c, int32_t tiles_per_row,
+                                                 int64_t* row, int32_t* col) {
+  *row = chunk / chunks_per_row;
+  *col = (int32_t)(chunk - *row * chunks_per_row) * 8;
+  return (*row / t_r) * tiles_per_row + *col / t_c;
+}
+
+template <int EX>
+__global__ __launch_bounds__(kQThreads) void tile_absmax_kernel(const unsigned char* __restrict__ x, float* __restrict__ scale,
+                                                                int64_t rows, int32_t cols, int32_t t_r, int32_t t_c) {
+  constexpr int XB = XVec<EX>::BYTES;
+  const int32_t chunks_per_row = cols / 8, tiles_per_row = cols / t_c;
+  const int64_t chunks = rows * chunks_per_row, stride = (int64_t)gridDim.x * kQThreads;
+  // (Every lane of a wave runs the same number of rounds, so that the shuffles below see all 64 lanes.)
+  for (int64_t base = (int64_t)blockIdx.x * kQThreads; base < chunks; base += stride) {
+    const int64_t chunk = base + threadIdx.x;
+    const bool live = chunk < chunks;
+    int64_t row;
+    int32_t col;
+    const int64_t tile = tile_of_chunk(live ? chunk : chunks - 1, chunks_per_row, t_r, t_c, tiles_per_row, &row, &col);
+    float m = 0.f;
+    if (live) {
+      float v[8];
+      load8<EX>(x + (row * cols + col) * (XB / 8), v);
+      m = absmax8(v);
+    }
+    const int64_t first = __shfl(tile, 0);
+    if (__all(tile == first)) {
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+      if ((threadIdx.x & 63) == 0) atomicMax(reinterpret_cast<unsigned*>(scale) + tile, __builtin_bit_cast(unsigned, m));
+    } else if (live) {
+      atomicMax(reinterpret_cast<unsigned*>(scale) + tile, __builtin_bit_cast(unsigned, m));
+    }
+  }
+}
+
+__global__ void tile_scale_kernel(float* __restrict__ scale, int64_t num_tiles, QuantRange qmax) {
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < num_tiles; t += (int64_t)gridDim.x * blockDim.x)
+    scale[t] = scale_of(scale[t], qmax);
+}
+
+template <int EX, int EQ>
+__global__ __launch_bounds__(kQThreads) void quantize_tiles_kernel(const unsigned char* __restrict__ x, unsigned char* __restrict__ q,
+                                                                   const float* __restrict__ scale, int64_t rows, int32_t cols,
+                                                                   int32_t t_r, int32_t t_c, QuantRange qmax) {
+  constexpr int XB = XVec<EX>::BYTES;
+  const int32_t chunks_per_row = cols / 8, tiles_per_row = cols / t_c;
+  const int64_t chunks = rows * chunks_per_row, stride = (int64_t)gridDim.x * kQThreads;
+  for (int64_t chunk = (int64_t)blockIdx.x * kQThreads + threadIdx.x; chunk < chunks; chunk += stride) {
+    int64_t row;
+    int32_t col;
+    const float s = scale[tile_of_chunk(chunk, chunks_per_row, t_r, t_c, tiles_per_row, &row, &col)];
+    const float sv[8] = {s, s, s, s, s, s, s, s};
+    float v[8];
+    load8<EX>(x + (row * cols + col) * (XB / 8), v);
+    *reinterpret_cast<i32x2*>(q + row * cols + col) = quantize8<EQ>(v, sv, qmax);
+  }
+}
+
 template <int EX>
 int32_t launch_for_x(const void* x, void* q, float* scale, int64_t rows, int64_t cols, int64_t t_r, int64_t t_c,
                      int32_t q_dtype, QuantRange qmax, hipStream_t stream) {
@@ -208,6 +279,19 @@ int32_t launch_for_x(const void* x, void* q, float* scale, int64_t rows, int64_t
       quantize_rows_kernel<EX, kEI8><<<dim3((unsigned)grid), dim3(kQThreads), 0, stream>>>(xb, qb, scale, rows, (int32_t)cols, (int32_t)t_c, L, qmax);
     else
       quantize_rows_kernel<EX, kEF8><<<dim3((unsigned)grid), dim3(kQThreads), 0, stream>>>(xb, qb, scale, rows, (int32_t)cols, (int32_t)t_c, L, qmax);
+  } else if (t_c != 1 && !((t_c & (t_c - 1)) == 0 && t_c >= 8 && t_c <= 256)) {
+    const int64_t num_tiles = (rows / t_r) * (cols / t_c), chunks = rows * (cols / 8);
+    int64_t grid = (chunks + kQThreads - 1) / kQThreads;
+    if (grid > 256 * 32) grid = 256 * 32;
+    int64_t small = (num_tiles + 255) / 256;
+    if (small > 1024) small = 1024;
+    tile_slots_clear_kernel<<<dim3((unsigned)small), dim3(256), 0, stream>>>(scale, num_tiles);
+    tile_absmax_kernel<EX><<<dim3((unsigned)grid), dim3(kQThreads), 0, stream>>>(xb, scale, rows, (int32_t)cols, (int32_t)t_r, (int32_t)t_c);
+    tile_scale_kernel<<<dim3((unsigned)small), dim3(256), 0, stream>>>(scale, num_tiles, qmax);
+    if (q_dtype == TKX_I8)
+      quantize_tiles_kernel<EX, kEI8><<<dim3((unsigned)grid), dim3(kQThreads), 0, stream>>>(xb, qb, scale, rows, (int32_t)cols, (int32_t)t_r, (int32_t)t_c, qmax);
+    else
+      quantize_tiles_kernel<EX, kEF8><<<dim3((unsigned)grid), dim3(kQThreads), 0, stream>>>(xb, qb, scale, rows, (int32_t)cols, (int32_t)t_r, (int32_t)t_c, qmax);
   } else {
     const int64_t grid = (rows / t_r) * ((cols + 255) / 256);
     if (grid > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "too many tiles");

@@ -335,8 +335,9 @@ def quantize(x: torch.Tensor, qtype: torch.dtype, tile_shape, bound: float | Non
   `bound` defaults to qmax (127, 7, 448); qmax + 0.5 is the other convention in use for integers (then -qmax - 1 appears).
 
   x f32, bf16 or f16: [rows, cols] with tiles one row tall and a multiple of 8 columns wide, or several rows tall and
-  1, 8, 16, ... or 256 columns wide; or weights [g, k, n] with a tile (1, t_k, t_n) (taken as g * k rows). qtype int8,
-  fp8 (e4m3fn) or a sub-byte integer (int4: values in [-7, 7], kept in int8 storage)."""
+  1 column or a multiple of 8 columns wide; or weights [g, k, n] with a tile (1, t_k, t_n) (taken as g * k rows) or a
+  tile (t_g, k, t_n) of whole groups (one scale per tensor: (g, k, n)). qtype int8, fp8 (e4m3fn) or a sub-byte integer
+  (int4: values in [-7, 7], kept in int8 storage)."""
   _log_launch(None)
   _require_cuda(x)
   lib = _lib.load()
@@ -347,13 +348,16 @@ def quantize(x: torch.Tensor, qtype: torch.dtype, tile_shape, bound: float | Non
   tile_shape = tuple(int(t) for t in tile_shape)
   if any(t < 1 or d % t for d, t in zip(x.shape, tile_shape)):
     raise NotImplementedError(f"tile shape {tile_shape} does not tile {tuple(x.shape)}")
+  t_r, t_c = tile_shape[-2], tile_shape[-1]
   if x.dim() == 3:
     if tile_shape[0] != 1:
-      raise NotImplementedError("weights are quantised per group: the tile must be (1, t_k, t_n)")
+      # A tile over several groups is a run of consecutive rows of [g * k, n] only when it takes whole groups.
+      if tile_shape[1] != x.shape[1]:
+        raise NotImplementedError("a tile over several groups must span their whole contraction: (t_g, k, t_n)")
+      t_r = tile_shape[0] * x.shape[1]
     rows, cols = x.shape[0] * x.shape[1], x.shape[2]
   else:
     rows, cols = x.shape
-  t_r, t_c = tile_shape[-2], tile_shape[-1]
   x = x.contiguous()
   storage = torch.float8_e4m3fn if qtype == torch.float8_e4m3fn else torch.int8
   qvalue = torch.empty(x.shape, dtype=storage, device=x.device)
