@@ -235,15 +235,17 @@ def test_vjp(m, k, n, activation, device):
 
 
 @pytest.mark.parametrize("b_tile_shape,supported", [((1, 256, 1), True), ((1, 16, 1), True), ((1, 1, 16), True),
-                                                    ((1, 64, 32), True), ((1, 1, 8), True), ((2, 1, 1), False)])
+                                                    ((1, 64, 32), True), ((1, 1, 8), True), ((2, 256, 1), True),
+                                                    ((4, 64, 128), True), ((3, 1, 1), False)])
 def test_quantized_int8_weights(b_tile_shape, supported, device):
   """bf16 x int8: per-(group, column) scales run in the kernels' epilogue, sub-channel scales along k and
-  scale tiles along n are repeated over their columns first; scales shared between groups are declined."""
+  scale tiles along n are repeated over their columns first, scales shared by runs of groups over those groups; a
+  tile that does not divide the array is declined."""
   G, m, k, n = 8, 512, 256, 512
   a, _, gs = _inputs("test_quantized", G, m, k, n, torch.bfloat16, device, random_groups=True)
   rng = np.random.default_rng(11)
   q = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
-  sshape = tuple(d // t for d, t in zip((G, k, n), b_tile_shape))
+  sshape = tuple(-(-d // t) for d, t in zip((G, k, n), b_tile_shape))
   scale = torch.tensor((rng.uniform(0.5, 1.5, sshape) / 127 * 0.1).astype(np.float32), device=device)
   rhs = tokamax_amd.QArray(q, scale)
   gst = torch.tensor(gs, device=device)

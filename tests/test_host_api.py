@@ -542,8 +542,9 @@ def test_quantised_operand_routes():
   assert key(q((m, k), f8, (m, 1)), q((G, k, n), f8, (G, k // 128, n))) == (4, BF, F8)       # lhs widened for it
   assert key(lhs16, q((G, k, n), i8, (G, k // 32, n))) == (0, BF, BF)                        # t_k = 32: the widening pass
   assert key(q((m, k), f8, (m, k // 32)), q((G, k, n), f8, (G, k // 32, n))) == (0, BF, BF)
+  assert key(lhs16, q((G, k, n), i8, (G // 2, 1, n))) == (0, BF, I8)                        # shared by pairs of groups: repeated
   with pytest.raises(NotImplementedError):
-    key(lhs16, q((G, k, n), i8, (G // 2, 1, n)))                                              # scales shared by pairs of groups
+    key(lhs16, q((G, k, n), i8, (3, 1, n)))                                                   # a scale array that tiles nothing
   # the k-step of the chosen variant divides the rows of a scale block
   ba = op.bind(q((m, k), i8, (m, k // 64)), q((G, k, n), i8, (G, k // 64, n)), group_sizes=gsz)
   assert 64 % ba.heuristics_config.block_k == 0

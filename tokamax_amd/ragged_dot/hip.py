@@ -148,10 +148,11 @@ def _per_column_rhs_scale(rhs):
     return rhs
   g, n = rhs.qvalue.shape[0], rhs.qvalue.shape[2]
   gs, nt = rhs.scale.shape[0], rhs.scale.shape[2]
-  if (nt == n and gs == g) or nt < 1 or n % nt != 0 or gs not in (1, g):
+  if (nt == n and gs == g) or nt < 1 or n % nt != 0 or gs < 1 or g % gs != 0:
     return rhs
   if isinstance(rhs.scale, torch.Tensor):
-    scale = rhs.scale.expand(g, -1, -1) if gs != g else rhs.scale  # (one scale set shared by all groups)
+    # (a scale set shared by runs of g / gs consecutive groups, e.g. by all of them, is repeated for each)
+    scale = rhs.scale.repeat_interleave(g // gs, dim=0) if gs != g else rhs.scale
     scale = scale.repeat_interleave(n // nt, dim=2) if nt != n else scale.contiguous()
   else:
     scale = ShapeDtype((g, rhs.scale.shape[1], n), rhs.scale.dtype)
@@ -159,15 +160,17 @@ def _per_column_rhs_scale(rhs):
 
 
 def _per_row_lhs_scale(lhs):
-  """A quantised lhs [m, k] whose scale has one row ([1, blocks]: shared by all rows, e.g. one scale per tensor)
-  with that row repeated for every lhs row. Works on tensors and on shapes."""
+  """A quantised lhs [m, k] whose scale rows are shared by runs of consecutive lhs rows ([m / t_m, blocks]: tiles
+  several rows tall, one scale per tensor) with each scale row repeated for its lhs rows. Works on tensors and on shapes."""
   if not isinstance(lhs, QArray) or len(lhs.scale.shape) != 2 or len(lhs.qvalue.shape) != 2:
     return lhs
   m = lhs.qvalue.shape[0]
-  if lhs.scale.shape[0] != 1 or m == 1:
-    return lhs
+  rows, blocks = lhs.scale.shape
+  k = lhs.qvalue.shape[1]
+  if rows == m or rows < 1 or m % rows != 0 or blocks < 1 or k % blocks != 0 or (blocks != 1 and (k // blocks) % 16 != 0):
+    return lhs  # (as it should be, or a form that is widened with its own tile shape)
   if isinstance(lhs.scale, torch.Tensor):
-    scale = lhs.scale.expand(m, -1)
+    scale = lhs.scale.repeat_interleave(m // rows, dim=0)  # (scale tiles several rows tall: (256, 1), one per tensor)
   else:
     scale = ShapeDtype((m, lhs.scale.shape[1]), lhs.scale.dtype)
   return QArray(lhs.qvalue, scale, lhs.zero_point, lhs.qtype)
