@@ -665,6 +665,35 @@ def test_heuristics_split_the_last_round_of_tiled_launches_with_few_rounds():
   assert op._get_heuristics_config(glu).split_k == 1
 
 
+def test_tile_cost_model_picks_near_the_fastest_measured_variant():
+  """The heuristics rank tiled variants of 16-bit forward / dlhs launches by `_tile_cost`. On the shipped timings (every
+  variant on 110 shapes) its pick stays within 6 % of the fastest variant on average and 35 % at worst, and its time
+  estimates follow the form of the data: more rows or a longer contraction never cost less, and a launch with a sliver
+  of a last round gains from the split while one without a partial round does not."""
+  from tokamax_amd.data.autotuning import tile_cost
+  entries = tile_cost.load()
+  assert len(entries) >= 100 and all(len(e["timings"]) >= 10 for e in entries)
+  mean, worst = tile_cost.summary(tile_cost.gaps(entries, hip._TILE_COST_FIT))
+  assert mean < 0.06 and worst < 0.35, (mean, worst)
+  v = (256, 256, 64, 2, 2, 2)
+  costs = [hip._tile_cost(v, 1, rows, 4096, 4096, 8) for rows in (1024, 4096, 16384, 65536, 262144)]
+  assert costs == sorted(costs) and costs[-1] > 30 * costs[1]
+  assert hip._tile_cost(v, 1, 16384, 4096, 8192, 8) > 1.8 * hip._tile_cost(v, 1, 16384, 4096, 4096, 8)
+  # 4096 x 14336 x 4096 in 8 groups of 512 rows: 16 * 56 = 896 tiles = 3.5 rounds of 256
+  assert hip._tile_cost((256, 256, 64, 2, 4, 3), 4, 4096, 14336, 4096, 8) < hip._tile_cost((256, 256, 64, 2, 4, 3), 1, 4096, 14336, 4096, 8)
+  # ... and 16 * 64 = 1024 tiles = 4 full rounds: nothing to split
+  assert hip._tile_cost((256, 256, 64, 2, 4, 3), 4, 4096, 16384, 4096, 8) == hip._tile_cost((256, 256, 64, 2, 4, 3), 1, 4096, 16384, 4096, 8)
+  # the bound launch asks the same model: the headline prefill shape gets the 256 x 256 tile, 64 rows per group a 128-row one
+  # (both the fastest measured)
+  op = hip.HipRaggedDot()
+  bf16 = torch.bfloat16
+  big = op.bind(ShapeDtype((16384, 4096), bf16), ShapeDtype((8, 4096, 14336), bf16), group_sizes=ShapeDtype((8,), torch.int32))
+  c = op._get_heuristics_config(big)
+  assert (c.block_m, c.block_n) == (256, 256)
+  small = op.bind(ShapeDtype((3584, 1536), bf16), ShapeDtype((56, 1536, 9216), bf16), group_sizes=ShapeDtype((56,), torch.int32))
+  assert op._get_heuristics_config(small).block_m == 128
+
+
 def test_bind_without_inspect_matches_the_signature_path():
   """`RaggedDot.bind` names every parameter of `_fwd` itself and skips `inspect`; the result is the one
   `Signature.bind` + `apply_defaults` gives, in signature order, and unknown or missing names still fail."""

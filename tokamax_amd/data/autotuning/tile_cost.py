@@ -1,0 +1,169 @@
+"""The timings behind the tile cost model of `HipRaggedDot`'s heuristics, and the fit of its constants.
+
+`<device kind>/tile_cost_timings.json` holds, per shape, the measured time of every compiled tiled variant (with and
+without the split of the last round): entries `{"shape": [rows, contraction, cols, groups], "mode": 0 forward | 1 dlhs,
+"streaming_best_us": fastest small-m streaming variant or null, "timings": [[block_m, block_n, block_k, waves_m,
+waves_n, num_stages, split_k, microseconds], ...]}`.
+
+  python -m tokamax_amd.data.autotuning.tile_cost check              # how far the model's pick is from the fastest
+  python -m tokamax_amd.data.autotuning.tile_cost fit [--iterations N]  # refit; prints the constants to paste
+  python -m tokamax_amd.data.autotuning.tile_cost collect M,K,N,G[,dlhs] ...   # time shapes on this GPU and add them
+
+`check` and `fit` need no GPU.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import random
+
+from tokamax_amd.ragged_dot import hip
+
+
+def timings_path(device_kind: str = "amd_instinct_mi355x") -> str:
+  return os.path.join(os.path.dirname(__file__), device_kind, "tile_cost_timings.json")
+
+
+def load(path: str | None = None) -> list[dict]:
+  with open(path or timings_path()) as f:
+    return json.load(f)
+
+
+def save(entries: list[dict], path: str | None = None) -> None:
+  with open(path or timings_path(), "w") as f:
+    f.write("[\n" + ",\n".join(json.dumps(e, separators=(",", ":")) for e in entries) + "\n]\n")
+
+
+def estimate(entry: dict, timing: list, fit: dict) -> float:
+  rows, contraction, cols, groups = entry["shape"]
+  return hip._tile_cost(tuple(timing[:6]), timing[6], rows, cols, contraction, groups, fit)  # pylint: disable=protected-access
+
+
+def pick(entry: dict, fit: dict) -> list:
+  """The timing row the heuristics' ranking would choose (ties: longer k-step, deeper pipeline, no split)."""
+  return min(entry["timings"], key=lambda t: (round(estimate(entry, t, fit), 3), -t[2], -t[5], t[6]))
+
+
+def gaps(entries: list[dict], fit: dict) -> list[float]:
+  """Per shape: time of the picked variant / time of the fastest tiled variant."""
+  return [pick(e, fit)[7] / min(t[7] for t in e["timings"]) for e in entries]
+
+
+def summary(ratios: list[float]) -> tuple[float, float]:
+  return math.exp(sum(math.log(r) for r in ratios) / len(ratios)) - 1, max(ratios) - 1
+
+
+def log_error(entries: list[dict], fit: dict, launch_us: float) -> float:
+  """Mean squared log ratio of estimate (+ a launch's fixed time, which does not rank variants) to measurement."""
+  total, count = 0.0, 0
+  for e in entries:
+    for t in e["timings"]:
+      total += math.log((estimate(e, t, fit) + launch_us) / t[7]) ** 2
+      count += 1
+  return total / count
+
+
+def refit(entries: list[dict], start: dict, iterations: int, seed: int = 0) -> dict:
+  """Random search from `start`: two constants at a time, scaled by exp(N(0, 0.12)), kept when the score (log error
+  of the estimates plus twice the mean gap of the picks plus a tenth of the worst gap) falls."""
+  rng = random.Random(seed)
+
+  def score(p):
+    mean, worst = summary(gaps(entries, p))
+    return log_error(entries, p, p["launch_us"]) + 2.0 * mean + 0.1 * worst
+
+  best = dict(start)
+  best_score = score(best)
+  for _ in range(iterations):
+    trial = dict(best)
+    for name in rng.sample(list(trial), 2):
+      trial[name] *= math.exp(rng.gauss(0, 0.12))
+    s = score(trial)
+    if s < best_score:
+      best, best_score = trial, s
+  return best
+
+
+def collect(specs: list[str], iterations: int) -> None:
+  import numpy as np  # pylint: disable=g-import-not-at-top
+  import torch  # pylint: disable=g-import-not-at-top
+  import tokamax_amd  # pylint: disable=g-import-not-at-top
+  from tokamax_amd import op as op_lib  # pylint: disable=g-import-not-at-top
+  from tokamax_amd.autotuning import autotuner as autotuner_lib  # pylint: disable=g-import-not-at-top
+  from tokamax_amd.autotuning import cache as cache_lib  # pylint: disable=g-import-not-at-top
+  from tokamax_amd.ragged_dot import base  # pylint: disable=g-import-not-at-top
+
+  device = torch.device("cuda:0")
+  path = timings_path(cache_lib.device_dir_name(op_lib.device_kind(device)))
+  os.makedirs(os.path.dirname(path), exist_ok=True)
+  entries = load(path) if os.path.exists(path) else []
+  tuner = autotuner_lib.Autotuner(iterations=iterations, warmup=2)
+  op = tokamax_amd.HipRaggedDot()
+  gen = torch.Generator(device=device).manual_seed(1)
+  for spec in specs:
+    parts = spec.split(",")
+    mode = 1 if parts[4:] == ["dlhs"] else 0
+    rows, contraction, cols, groups = (int(x) for x in parts[:4])
+    rng = np.random.default_rng(rows + contraction + cols + groups)
+    sizes = rng.multinomial(rows, rng.dirichlet(np.ones(groups) * 4)).astype(np.int32)
+    group_sizes = torch.tensor(sizes, device=device)
+    lhs = torch.randn(rows, contraction, device=device, generator=gen).to(torch.bfloat16)
+    shape = (groups, contraction, cols) if mode == 0 else (groups, cols, contraction)
+    rhs = (torch.randn(*shape, device=device, generator=gen) * contraction**-0.5).to(torch.bfloat16)
+    kwargs = {} if mode == 0 else dict(ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS)
+    bound = op.bind(lhs, rhs, group_sizes=group_sizes, **kwargs)
+    configs = {c for c in bound.autotuning_configs if c.block_m == 16 or c.grid_tile_width == 8}
+    data = tuner.autotune(
+        lambda c: (lambda: tokamax_amd.HipRaggedDot(config=c)(lhs, rhs, group_sizes=group_sizes, **kwargs)), configs
+    )
+    us = {c: d.median_evaluation_time_ms * 1e3 for c, d in data.items() if hasattr(d, "median_evaluation_time_ms")}
+    streaming = [t for c, t in us.items() if c.block_m == 16]
+    entry = dict(
+        shape=[rows, contraction, cols, groups],
+        mode=mode,
+        streaming_best_us=round(min(streaming), 2) if streaming else None,
+        timings=sorted(
+            (
+                [c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages, c.split_k, round(t, 2)]
+                for c, t in us.items()
+                if c.block_m != 16
+            ),
+            key=lambda t: t[7],
+        ),
+    )
+    entries = [e for e in entries if (e["shape"], e["mode"]) != (entry["shape"], mode)] + [entry]
+    save(entries, path)
+    chosen = pick(entry, hip._TILE_COST_FIT)  # pylint: disable=protected-access
+    print(spec, "fastest", entry["timings"][0], "model's pick", chosen, flush=True)
+    del lhs, rhs, bound
+
+
+def main() -> None:
+  parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+  parser.add_argument("command", choices=("check", "fit", "collect"))
+  parser.add_argument("shapes", nargs="*")
+  parser.add_argument("--iterations", type=int, default=None)
+  args = parser.parse_args()
+  current = dict(hip._TILE_COST_FIT)  # pylint: disable=protected-access
+  if args.command == "collect":
+    collect(args.shapes, args.iterations or 6)
+    return
+  entries = load()
+  if args.command == "fit":
+    fitted = refit(entries, dict(current, launch_us=7.0), args.iterations or 3000)
+    fitted.pop("launch_us")
+    print("_TILE_COST_FIT = dict(")
+    for name, value in fitted.items():
+      print(f"    {name}={float('%.4g' % value)!r},")
+    print(")")
+    current = {name: float("%.4g" % value) for name, value in fitted.items()}
+  mean, worst = summary(gaps(entries, current))
+  print(f"{len(entries)} shapes, {sum(len(e['timings']) for e in entries)} timings: the model's pick is "
+        f"{100 * mean:.1f} % above the fastest variant on average, {100 * worst:.0f} % at worst")
+
+
+if __name__ == "__main__":
+  main()

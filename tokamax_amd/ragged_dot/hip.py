@@ -85,6 +85,72 @@ def _tiled_split_pays(mode: int, block_m: int, block_n: int, rows: int, cols: in
   return tiles < 8 * _COMPUTE_UNITS
 
 
+# Constants of `_tile_cost`, fitted by tokamax_amd/data/autotuning/tile_cost.py to the timings beside it.
+_TILE_COST_FIT = dict(
+    mfma_flop_per_us=3.969e6,    # a CU's MFMA rate on a full tile
+    load_byte_per_us=60.38e3,    # a CU's rate of bringing operand slices into LDS
+    partial_block=0.4989,        # share of a 32-row block's time that a block without rows of the task still costs
+    four_wave_factor=1.045,      # MFMA time of a 4-wave tile against an 8-wave one
+    in_flight_full=69.55,        # contraction elements in flight from which loads run at their full rate
+    in_flight_exponent=1.585,
+    fixed_us=3.122,              # per tile: start-up and epilogue
+    fixed_area_us=3.368,         # ... more per 256x256 of output
+    shared_cu_mfma=1.035,        # two workgroups on a CU: each k-step takes 2x this (MFMA bound)
+    shared_cu_load=1.021,        # ... or 2x this (load bound)
+    tail_floor=0.3496,           # a partial round behind full ones costs at least this share of a round
+    exchange_us=25.46,           # price of splitting the last round along the contraction
+    group_straddle=0.8607,       # extra tiles per group at an arbitrary row offset
+)
+
+
+def _tile_cost(variant, split_k: int, rows: int, cols: int, contraction: int, num_groups: int,
+               fit=_TILE_COST_FIT) -> float:
+  """Estimated time (us) of a tiled forward / dlhs launch of 16-bit operands: rounds of workgroups times the time of a
+  tile. A tile's k-step costs the larger of its MFMA time (only the 32-row blocks that hold rows of the task run at
+  full price) and the time to bring its operand slices into LDS, which a pipeline with less than about 70 contraction
+  elements in flight stretches; a tile also pays a fixed time (start-up and epilogue, growing with its area). Shapes
+  whose LDS lets two 4-wave workgroups share a CU run two tiles at a time at half the pace each, so that their fixed
+  times overlap. A group of r rows at an arbitrary offset touches about r / block_m + 0.86 tiles. A partial round
+  behind full ones overlaps with them in part; with `split_k` its tiles are cut into parts at the price of the
+  exchange.
+  The constants were fitted to the measured times of every compiled variant on 110 shapes (m = 256 .. 262144, k and
+  n = 256 .. 14336, 2 .. 256 groups, forward and dlhs; 2570 timings): the variant this picks is within 4 % of the
+  fastest one on average and 32 % at worst on those shapes. On 16 shapes measured before they joined the fit it was
+  within 11 % on average and 31 % at worst, against 13 % and 55 % for rules on rows per group alone (17-20 % and
+  75-77 % on the two earlier sets)."""
+  bm, bn, bk, wm, wn, ns = variant
+  tasks = min(rows / bm + fit["group_straddle"] * num_groups, -(-rows // bm) + num_groups - 1)
+  tiles = tasks * -(-cols // bn)
+  four_waves = wm * wn == 4
+  two_per_cu = four_waves and 2 * ns * (bm + bn) * bk * 2 <= 160 * 1024
+  active = min(1.0, rows / (tasks * bm) + fit["partial_block"] * 32 / bm)
+  mma_us = bm * bn * bk * 2 / fit["mfma_flop_per_us"] * active * (fit["four_wave_factor"] if four_waves else 1.0)
+  in_flight = min(1.0, ((ns - 1) * bk / fit["in_flight_full"]) ** fit["in_flight_exponent"])
+  load_us = (bm + bn) * bk * 2 / fit["load_byte_per_us"] / in_flight
+  steps = -(-contraction // bk)
+  fixed_us = fit["fixed_us"] + fit["fixed_area_us"] * bm * bn / 65536
+  alone_us = steps * max(mma_us, load_us) + fixed_us
+  if two_per_cu:
+    tile_us = steps * 2 * max(fit["shared_cu_mfma"] * mma_us, fit["shared_cu_load"] * load_us) + fixed_us
+  else:
+    tile_us = alone_us
+  slots = _COMPUTE_UNITS * (2 if two_per_cu else 1)
+  full_rounds = int(tiles // slots)
+  rest = tiles - full_rounds * slots
+  total = full_rounds * tile_us
+  if rest > 0:
+    last = alone_us if two_per_cu and rest <= _COMPUTE_UNITS else tile_us
+    if full_rounds > 0:
+      last *= fit["tail_floor"] + (1 - fit["tail_floor"]) * rest / slots
+    if split_k > 1:
+      beyond = int(tiles) % _COMPUTE_UNITS
+      parts = min(split_k, _COMPUTE_UNITS // beyond) if beyond > 0 else 1
+      if parts > 1:
+        last = last / parts + fit["exchange_us"]
+    total += last
+  return total
+
+
 def _streaming_split(tiles: int, contraction: int, block_n: int, depth: int) -> int:
   """Workgroups per (group, column tile) of the streaming small-m kernel. Unsplit, a launch has `tiles` workgroups;
   with fewer than one per CU, splitting the contraction until there are 256 measured 1.3x (128 tiles) to 3.5x
@@ -794,6 +860,21 @@ class HipRaggedDot(base.RaggedDot):
       return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -in_flight, bk if short_k else -bk, ns)
 
     bm, bn, bk, wm, wn, ns = min(usable, key=score)
+    modelled_split = None
+    if bm != 16 and mode in (0, 1) and key[1] == key[2] and key[1] in (_lib.TKX_BF16, _lib.TKX_F16):
+      # 16-bit operands without scales: the tile that the cost model expects to finish first, with or without the
+      # split of the last round (the rules above stay in charge of the choice for the streaming small-m kernel).
+      best = None
+      for v in usable:
+        if v[0] == 16:
+          continue
+        for sk in (1, 4) if _tiled_split_pays(mode, v[0], v[1], rows, cols, num_groups) else (1,):
+          # (ties: the longer k-step has fewer barriers per flop, then the deeper pipeline)
+          cost = (round(_tile_cost(v, sk, rows, cols, contraction, num_groups), 3), -v[2], -v[5], sk)
+          if best is None or cost < best[0]:
+            best = (cost, v, sk)
+      if best is not None:
+        (bm, bn, bk, wm, wn, ns), modelled_split = best[1], best[2]
     # grid_tile_width m-tasks of one group run side by side on an n-panel of its weights (a span never
     # crosses a group, so small groups simply get short spans). With the 32 tiles an XCD runs at a
     # time, 8 wide x 4 n-panels needs the fewest distinct operand panels in its L2; 16 wide measured
@@ -803,6 +884,8 @@ class HipRaggedDot(base.RaggedDot):
     if bm == 16:
       width = 1  # the streaming small-m kernel has no tile order to tune
       split_k = _streaming_split(num_groups * -(-cols // bn), contraction, bn, ns)
+    elif modelled_split is not None:
+      split_k = modelled_split
     elif _tiled_split_pays(mode, bm, bn, rows, cols, num_groups):
       split_k = 4
     return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns, grid_tile_width=width,
