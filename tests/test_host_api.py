@@ -667,7 +667,7 @@ def test_heuristics_split_the_last_round_of_tiled_launches_with_few_rounds():
 
 def test_tile_cost_model_picks_near_the_fastest_measured_variant():
   """The heuristics rank tiled variants of 16-bit forward / dlhs launches by `_tile_cost`. On the shipped timings (every
-  variant on 110 shapes) its pick stays within 6 % of the fastest variant on average and 35 % at worst, and its time
+  variant on 122 shapes) its pick stays within 6 % of the fastest variant on average and 35 % at worst, and its time
   estimates follow the form of the data: more rows or a longer contraction never cost less, and a launch with a sliver
   of a last round gains from the split while one without a partial round does not."""
   from tokamax_amd.data.autotuning import tile_cost

@@ -39,7 +39,7 @@ def save(entries: list[dict], path: str | None = None) -> None:
 
 def estimate(entry: dict, timing: list, fit: dict) -> float:
   rows, contraction, cols, groups = entry["shape"]
-  return hip._tile_cost(tuple(timing[:6]), timing[6], rows, cols, contraction, groups, fit)  # pylint: disable=protected-access
+  return hip._tile_cost(tuple(timing[:6]), timing[6], rows, cols, contraction, groups, entry["mode"], fit)  # pylint: disable=protected-access
 
 
 def pick(entry: dict, fit: dict) -> list:

@@ -87,46 +87,52 @@ def _tiled_split_pays(mode: int, block_m: int, block_n: int, rows: int, cols: in
 
 # Constants of `_tile_cost`, fitted by tokamax_amd/data/autotuning/tile_cost.py to the timings beside it.
 _TILE_COST_FIT = dict(
-    mfma_flop_per_us=3.969e6,    # a CU's MFMA rate on a full tile
-    load_byte_per_us=60.38e3,    # a CU's rate of bringing operand slices into LDS
-    partial_block=0.4989,        # share of a 32-row block's time that a block without rows of the task still costs
-    four_wave_factor=1.045,      # MFMA time of a 4-wave tile against an 8-wave one
-    in_flight_full=69.55,        # contraction elements in flight from which loads run at their full rate
-    in_flight_exponent=1.585,
-    fixed_us=3.122,              # per tile: start-up and epilogue
-    fixed_area_us=3.368,         # ... more per 256x256 of output
-    shared_cu_mfma=1.035,        # two workgroups on a CU: each k-step takes 2x this (MFMA bound)
-    shared_cu_load=1.021,        # ... or 2x this (load bound)
-    tail_floor=0.3496,           # a partial round behind full ones costs at least this share of a round
-    exchange_us=25.46,           # price of splitting the last round along the contraction
-    group_straddle=0.8607,       # extra tiles per group at an arbitrary row offset
+    mfma_flop_per_us=6.142e6,    # a CU's MFMA rate on a full tile
+    load_byte_per_us=59.31e3,    # a CU's rate of bringing operand slices into LDS
+    partial_block=1.475,         # 32-row blocks' worth of rows that a task costs beyond the rows it has
+    four_wave_factor=1.033,      # MFMA time of a 4-wave tile against an 8-wave one
+    in_flight_full=64.97,        # contraction elements in flight from which loads run at their full rate
+    in_flight_exponent=1.802,
+    fixed_us=3.348,              # per tile: start-up and epilogue
+    fixed_area_us=3.636,         # ... more per 256x256 of output
+    shared_cu_mfma=1.396,        # two workgroups on a CU: each k-step takes 2x this (MFMA bound)
+    shared_cu_load=0.9206,       # ... or 2x this (load bound)
+    tail_floor=0.4117,           # a partial round behind full ones costs at least this share of a round
+    exchange_us=26.43,           # price of splitting the last round along the contraction
+    group_straddle=0.8914,       # extra tiles per group at an arbitrary row offset
+    short_piece=1.526,           # time of loading 64-byte pieces of rows against 128-byte ones
 )
 
 
-def _tile_cost(variant, split_k: int, rows: int, cols: int, contraction: int, num_groups: int,
+def _tile_cost(variant, split_k: int, rows: int, cols: int, contraction: int, num_groups: int, mode: int = 0,
                fit=_TILE_COST_FIT) -> float:
   """Estimated time (us) of a tiled forward / dlhs launch of 16-bit operands: rounds of workgroups times the time of a
-  tile. A tile's k-step costs the larger of its MFMA time (only the 32-row blocks that hold rows of the task run at
-  full price) and the time to bring its operand slices into LDS, which a pipeline with less than about 70 contraction
-  elements in flight stretches; a tile also pays a fixed time (start-up and epilogue, growing with its area). Shapes
-  whose LDS lets two 4-wave workgroups share a CU run two tiles at a time at half the pace each, so that their fixed
-  times overlap. A group of r rows at an arbitrary offset touches about r / block_m + 0.86 tiles. A partial round
-  behind full ones overlaps with them in part; with `split_k` its tiles are cut into parts at the price of the
-  exchange.
-  The constants were fitted to the measured times of every compiled variant on 110 shapes (m = 256 .. 262144, k and
-  n = 256 .. 14336, 2 .. 256 groups, forward and dlhs; 2570 timings): the variant this picks is within 4 % of the
-  fastest one on average and 32 % at worst on those shapes. On 16 shapes measured before they joined the fit it was
-  within 11 % on average and 31 % at worst, against 13 % and 55 % for rules on rows per group alone (17-20 % and
-  75-77 % on the two earlier sets)."""
+  tile. A tile's k-step costs the larger of its MFMA time (less where the task's rows do not fill the share of the
+  wave that holds them) and the time to bring its operand slices into LDS, which a pipeline with less than about 65
+  contraction elements in flight stretches; a tile also pays a fixed time (start-up and epilogue, growing with its
+  area). Shapes whose LDS lets two 4-wave workgroups share a CU run two tiles at a time at less than half the pace
+  each, so that their fixed times overlap. A group of r rows at an arbitrary offset touches about r / block_m + 0.89
+  tiles. A partial round behind full ones overlaps with them in part; with `split_k` its tiles are cut into parts at
+  the price of the exchange.
+  The constants were fitted to the measured times of every compiled variant on 122 shapes (m = 256 .. 262144, k and
+  n = 256 .. 14336, 2 .. 256 groups, forward and dlhs; 2852 timings): the variant this picks is within 4 % of the
+  fastest one on average and 31 % at worst on those shapes. On 12 further shapes that no fit has seen it is within
+  6 % on average and 24 % at worst (8 % and 48 % before the term for 64-byte pieces, which one of them prompted),
+  against 21 % and 52 % for rules on rows per group alone; an earlier fit to 110 of the shapes was within 10 % and 47 %
+  on the 12 others, against 30 % and 77 % for those rules."""
   bm, bn, bk, wm, wn, ns = variant
   tasks = min(rows / bm + fit["group_straddle"] * num_groups, -(-rows // bm) + num_groups - 1)
   tiles = tasks * -(-cols // bn)
   four_waves = wm * wn == 4
   two_per_cu = four_waves and 2 * ns * (bm + bn) * bk * 2 <= 160 * 1024
-  active = min(1.0, rows / (tasks * bm) + fit["partial_block"] * 32 / bm)
+  # (the waves of a tile split its rows `wm` ways and the slowest one sets the pace: the rows count against a wave's share)
+  active = min(1.0, (rows / tasks + fit["partial_block"] * 32) * wm / bm)
   mma_us = bm * bn * bk * 2 / fit["mfma_flop_per_us"] * active * (fit["four_wave_factor"] if four_waves else 1.0)
   in_flight = min(1.0, ((ns - 1) * bk / fit["in_flight_full"]) ** fit["in_flight_exponent"])
-  load_us = (bm + bn) * bk * 2 / fit["load_byte_per_us"] / in_flight
+  # (a 32-element slice of an operand that is contiguous along the contraction, as the lhs is and in dlhs the weights
+  # are too, is read in 64-byte pieces)
+  short = fit["short_piece"] if bk < 64 else 1.0
+  load_us = (bm * short + bn * (short if mode == 1 else 1.0)) * bk * 2 / fit["load_byte_per_us"] / in_flight
   steps = -(-contraction // bk)
   fixed_us = fit["fixed_us"] + fit["fixed_area_us"] * bm * bn / 65536
   alone_us = steps * max(mma_us, load_us) + fixed_us
@@ -870,7 +876,7 @@ class HipRaggedDot(base.RaggedDot):
           continue
         for sk in (1, 4) if _tiled_split_pays(mode, v[0], v[1], rows, cols, num_groups) else (1,):
           # (ties: the longer k-step has fewer barriers per flop, then the deeper pipeline)
-          cost = (round(_tile_cost(v, sk, rows, cols, contraction, num_groups), 3), -v[2], -v[5], sk)
+          cost = (round(_tile_cost(v, sk, rows, cols, contraction, num_groups, mode), 3), -v[2], -v[5], sk)
           if best is None or cost < best[0]:
             best = (cost, v, sk)
       if best is not None:
