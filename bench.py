@@ -333,7 +333,15 @@ def main():
     cfg = op.bind(a8, q8, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
     measure("mixtral_prefill_int8_int8", lambda: op(a8, q8, group_sizes=gs, preferred_element_type=torch.bfloat16),
             w.flops, w.m * w.k + w.nonempty_groups * w.k * w.n + w.m * w.n * 2, "mfma", "int8", cfg)
-    del w, q8, q8k, a8
+    # int4 weights packed two to a byte along k, read as they are by the tiled kernels (a quarter of bf16's weight stream)
+    int4 = getattr(torch, "int4", torch.int8)
+    q4 = tokamax_amd.pack_int4(tokamax_amd.QArray(
+        torch.randint(-8, 8, tuple(w.rhs.shape), device=device, dtype=torch.int8, generator=gen8),
+        (torch.rand(w.num_groups, 1, w.n, device=device, generator=gen8) + 0.5) / (7 * w.k ** 0.5), None, int4))
+    cfg = op.bind(w.lhs, q4, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_prefill_int4_packed_weights", lambda: op(w.lhs, q4, group_sizes=gs, preferred_element_type=torch.bfloat16),
+            w.flops, w.m * w.k * 2 + w.nonempty_groups * w.k * w.n // 2 + w.m * w.n * 2, "mfma", "bf16", cfg)
+    del w, q8, q8k, a8, q4
 
     w = workloads.make("vjp", device, seed=0)
     gs = torch.tensor(w.group_sizes, device=device)

@@ -828,10 +828,53 @@ def test_small_m_kernel_on_packed_int4_weights(case, scales, depth, split_k, dev
   assert torch.equal(out, same)
 
 
+def _packed_int4_tile_cases():
+  return [pytest.param(v, id="{block_m}x{block_n}x{block_k}-w{waves_m}x{waves_n}-s{num_stages}".format(**v))
+          for v in _lib.variants(0) if v["rhs_dtype"] == _lib.TKX_I4X2 and v["block_m"] != 16]
+
+
+@pytest.mark.parametrize("v", _packed_int4_tile_cases())
+def test_tiled_kernels_on_packed_int4_weights(v, device):
+  """The tiled kernels read int4 weights two to a byte along k: an odd number of k-steps, a ragged last column tile,
+  groups that start and end inside tiles, an empty group, rows after the last group. Against the oracle on the
+  unpacked values, against the int8 kernel of the same tile on them (the same products, summed in another order
+  inside a pair of MFMA atoms), and bit for bit against itself."""
+  rng = np.random.default_rng(v["block_m"] + v["num_stages"])
+  G, k, n = 5, 5 * v["block_k"], 272
+  gs = np.array([3, 300, 0, 70, 129], np.int32)
+  m = int(gs.sum()) + 9
+  gst = torch.tensor(gs, device=device)
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  values = rng.integers(-8, 8, (G, k, n)).astype(np.int8)
+  scale = torch.tensor((np.abs(rng.normal(0, 0.05, (G, 1, n))) + 1e-2).astype(np.float32), device=device)
+  packed = torch.tensor(O.pack_int4(values), device=device)
+  cfg = hip_ops.KernelConfig(v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"], v["num_stages"], grid_tile_width=2)
+  out = hip_ops.ragged_dot_fwd(lhs, packed, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale)
+  want = O.ragged_dot(_np(lhs), O.dequantize(values, _np(scale)), gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, 1e-5)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  assert torch.equal(out, hip_ops.ragged_dot_fwd(lhs, packed, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale))
+  int8_tiles = {(x["block_m"], x["block_n"], x["block_k"], x["waves_m"], x["waves_n"], x["num_stages"])
+                for x in _lib.variants(0) if x["rhs_dtype"] == _lib.TKX_I8 and x["lhs_dtype"] == _lib.TKX_BF16}
+  if (cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages) in int8_tiles:
+    same = hip_ops.ragged_dot_fwd(lhs, torch.tensor(values, device=device), gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale)
+    torch.testing.assert_close(out, same, rtol=2e-6, atol=2e-5)
+  # bf16 result and no scale at all; a contraction that is not whole k-steps is declined, not mis-read
+  plain = hip_ops.ragged_dot_fwd(lhs, packed, gst, config=cfg, out_dtype=torch.bfloat16)
+  _check(plain, O.ragged_dot(_np(lhs), values.astype(np.float64), gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 4e-3)
+  with pytest.raises(NotImplementedError, match="block_k"):
+    hip_ops.ragged_dot_fwd(lhs[:, :k - 32].contiguous(), packed[:, :k // 2 - 16].contiguous(), gst, config=cfg, out_dtype=torch.float32)
+
+
+def _lib_key(op, lhs, rhs, gs):
+  return op._problem(op.bind(lhs, rhs, group_sizes=gs))[1]
+
+
 def test_public_op_on_packed_int4_weights(device):
-  """`pack_int4` of a quantised rhs: with a few rows per group the op keeps it packed (streaming kernel, heuristics
-  name it); with many rows per group, a bias or another lhs type it unpacks to int8 first. Same results as the
-  unpacked QArray either way."""
+  """`pack_int4` of a quantised rhs: the op keeps it packed, for the streaming kernel with a few rows per group and
+  for the tiled kernels with many (the heuristics name them); with a bias or another lhs type it unpacks to int8
+  first. Same results as the unpacked QArray: bit for bit where the same kernel contracts in the same order, else to
+  the rounding of f32 sums in another order."""
   rng = np.random.default_rng(8)
   G, k, n = 16, 1024, 256
   q = torch.tensor(rng.integers(-7, 8, (G, k, n)).astype(np.int8), device=device)
@@ -851,7 +894,11 @@ def test_public_op_on_packed_int4_weights(device):
     want = O.ragged_dot(_np(lhs), O.dequantize(q.cpu().numpy(), _np(scale)), np.full(G, rows, np.int32), O.DEFAULT,
                         acc_dtype=np.float64, out_dtype="f64")
     _check(out, want, 1e-5)
-    assert torch.equal(out, ref)
+    if rows == 2:
+      assert torch.equal(out, ref)
+    else:
+      assert cfg.block_m >= 32 and _lib_key(op, lhs, packed, gs)[2] == _lib.TKX_I4X2
+      torch.testing.assert_close(out, ref, rtol=1e-5, atol=1e-5)
   bias = torch.tensor(rng.normal(0, 1, (G, 1, n)).astype(np.float32), device=device)
   gs = torch.full((G,), 2, dtype=torch.int32, device=device)
   lhs = torch.tensor(rng.normal(0, 1, (G * 2, k)).astype(np.float32), device=device).to(torch.bfloat16)

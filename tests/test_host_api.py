@@ -605,8 +605,8 @@ def test_ffi_shim_compiles_to_its_stub_without_the_xla_header(tmp_path):
 def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   """Config choice needs no GPU: shapes and types only. A launch of the streaming kernel with fewer (group, column
   tile) pairs than CUs gets its contraction split (8 ways at most, and only as far as k divides); packed int4 weights
-  stay packed (their own variant key) in the small-m regime and count as int8 storage otherwise; a QArray of packed
-  int4 reports the shape of its values."""
+  stay packed (their own variant key) where a kernel reads them as they are and count as int8 storage otherwise; a QArray
+  of packed int4 reports the shape of its values."""
   op = hip.HipRaggedDot()
   bf16, f32, i8, u8 = torch.bfloat16, torch.float32, torch.int8, torch.uint8
 
@@ -634,8 +634,25 @@ def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   assert packed.unpacked().qvalue.shape == (8, 1024, 256) and packed.unpacked().qvalue.dtype == i8
   c = config(16, 1024, 256, 8, u8, packed=True)          # 2 rows per group: the streaming kernel reads the bytes
   assert c.block_m == 16
-  c = config(4096, 1024, 256, 8, u8, packed=True)        # 512 rows per group: unpacked first, then an int8 tile variant
+  c = config(4096, 1024, 256, 8, u8, packed=True)        # 512 rows per group: a tiled kernel reads the bytes too
   assert c.block_m >= 128
+  lhs, gs = ShapeDtype((4096, 1024), bf16), ShapeDtype((8,), torch.int32)
+  route = lambda rhs, **kw: op._problem(op.bind(lhs, rhs, group_sizes=gs, **kw))[1]
+  assert route(packed)[2] == _lib.TKX_I4X2
+  # ... unless the call has a bias, scale blocks along k (tiled kernels: one scale per (group, column)), a contraction
+  # that is not a multiple of the k-step, or columns that are not whole 16-byte pieces: int8 storage first
+  assert route(packed, rhs_bias=ShapeDtype((8, 1, 256), f32))[2] == _lib.TKX_I8
+  blocks = tokamax_amd.QArray(ShapeDtype((8, 512, 256), u8), ShapeDtype((8, 4, 256), f32), None, getattr(torch, "int4", i8))
+  assert route(blocks)[2] == _lib.TKX_I8
+  odd = tokamax_amd.QArray(ShapeDtype((8, 48, 256), u8), ShapeDtype((8, 1, 256), f32), None, getattr(torch, "int4", i8))
+  assert op._problem(op.bind(ShapeDtype((4096, 96), bf16), odd, group_sizes=gs))[1][2] == _lib.TKX_I8
+  space = op._get_autotuning_configs(op.bind(lhs, packed, group_sizes=gs))
+  assert {x.block_m for x in space} >= {16, 32, 128, 256}
+  # the key of an autotuning cache entry names the 4-bit type and comes back as the same abstract QArray
+  from tokamax_amd import serialization
+  spec = serialization.to_jsonable(packed)
+  assert spec["qvalue"] == "u8[8,512,256]" and spec["qtype"].endswith("int4" if hasattr(torch, "int4") else "int8")
+  assert serialization.array_spec_from_json(json.loads(json.dumps(spec))) == packed
 
 
 def test_heuristics_split_the_last_round_of_tiled_launches_with_few_rounds():

@@ -65,6 +65,7 @@ struct Registry {
     v = variants_f32(&n);  add(v, n);
     v = variants_f8(&n);   add(v, n);
     v = variants_i8w(&n);  add(v, n);
+    v = variants_i4w(&n);  add(v, n);
     // The streaming small-m kernel is not a tile variant of the GEMM template; it is listed here
     // (fn == nullptr, num_stages = steps of loads in flight) so that configs can name it.
     for (int depth : {2, 4, 8})
@@ -289,6 +290,13 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
       return set_error(TKX_ERR_UNSUPPORTED,
                        "fp8 x fp8 with scale blocks along k needs lhs scales f32[blocks, m], m %% 4 == 0 and align_tile %% 4 == 0");
   }
+  // Packed int4 weights in the tiled kernels: plain forward, one scale per (group, column), whole k-steps.
+  const bool packed_tiled = rhs_dtype == TKX_I4X2 && c.block_m != kDecodeBlockM;
+  if (packed_tiled && (dlhs || gateup || subk || c.block_k < 1 || k % c.block_k != 0))
+    return set_error(TKX_ERR_UNSUPPORTED,
+                     "packed int4 weights in a tiled kernel: default mode, one rhs scale per (group, column) or none, no gate-up"
+                     " fusion, k %% block_k == 0 (k=%lld block_k=%d); tkx_unpack_int4 gives int8 storage for everything else",
+                     (long long)k, c.block_k);
   const Variant* v = find_variant(dlhs ? kDlhs : gateup ? kFwdGlu : subk ? kFwdSubK : kFwd, lhs_dtype, rhs_dtype, c);
   if (v == nullptr)
     return set_error(TKX_ERR_UNSUPPORTED, "no kernel variant for mode=%d dtypes=(%d,%d) tile=%dx%dx%d waves=%dx%d stages=%d",
@@ -368,7 +376,7 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
   p.lda = dlhs ? n : k;
   p.ldb = n;
   p.ldc = cols;
-  p.b_group_stride = k * n;
+  p.b_group_stride = rhs_dtype == TKX_I4X2 ? k / 2 * n : k * n;  // (in stored elements: packed bytes)
   p.c_group_stride = 0;
   p.m_ext = (int32_t)m;
   p.n_ext = (int32_t)cols;

@@ -170,5 +170,6 @@ const Variant* variants_f16(int* count);
 const Variant* variants_f32(int* count);
 const Variant* variants_f8(int* count);
 const Variant* variants_i8w(int* count);
+const Variant* variants_i4w(int* count);
 
 }  // namespace tkx

@@ -79,7 +79,7 @@ __device__ __forceinline__ i32x4 buffer_load_16_streaming(__amdgpu_buffer_rsrc_t
   return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_offset, (int)uniform_offset, kStreamingLoad));
 }
 
-constexpr int kEI4 = TKX_I4X2;  // packed int4 weights: a stored row holds two contraction rows
+// (kEI4, packed int4 weights: a stored row holds two contraction rows)
 
 // What a lane holds of one weight row of a step: its CPL columns (8, or 16 of int8).
 template <int EW, int CPL> struct WeightRow { typedef i32x4 T; static constexpr int ESZ = 2; };

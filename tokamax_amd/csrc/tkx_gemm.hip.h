@@ -49,7 +49,8 @@ __device__ __forceinline__ i32x2 lds_read_tr8(const unsigned char* p) {
   return __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*)(p));
 }
 
-enum ElemKind { kEF32 = TKX_F32, kEBF16 = TKX_BF16, kEF16 = TKX_F16, kEF8 = TKX_F8E4M3FN, kEI8 = TKX_I8 };
+// (kEI4: weights only, two 4-bit values to a byte along the contraction; a tile of them is a tile of bytes half as deep)
+enum ElemKind { kEF32 = TKX_F32, kEBF16 = TKX_BF16, kEF16 = TKX_F16, kEF8 = TKX_F8E4M3FN, kEI8 = TKX_I8, kEI4 = TKX_I4X2 };
 enum OperandLayout { kKC = 0 /* contraction-contiguous */, kMC = 1 /* contiguous along rows/cols */ };
 
 __host__ __device__ constexpr int elem_bytes(int e) { return e == kEF32 ? 4 : (e == kEBF16 || e == kEF16) ? 2 : 1; }
@@ -144,13 +145,34 @@ __device__ __forceinline__ i32x4 i8x8_to_bf16x8(i32x2 v) {
   return out;
 }
 
+// Four packed bytes (eight signed 4-bit values: byte u holds contraction entries 2 u in bits 0-3 and 2 u + 1 in bits
+// 4-7) -> bf16 x8 in contraction order, each value TIMES 16: a nibble moved to the top of its byte is the int8 value
+// 16 v, which converts like the int8 weights do (one SDWA instruction per value, one byte permute per pair, three
+// instructions to line the nibbles up for all eight). |16 v| <= 128 is exact in bf16; the kernel takes the factor
+// out of its sums again (kPackedInt4Unscale, exact).
+constexpr float kPackedInt4Unscale = 0.0625f;
+__device__ __forceinline__ i32x4 i4x8_to_bf16x8_times16(int w) {
+  const int lo = (w << 4) & (int)0xF0F0F0F0u, hi = w & (int)0xF0F0F0F0u;
+  i32x4 out;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const float f0 = (float)(signed char)((lo >> (8 * u)) & 0xff);
+    const float f1 = (float)(signed char)((hi >> (8 * u)) & 0xff);
+    out[u] = (int)__builtin_amdgcn_perm(__builtin_bit_cast(unsigned, f1), __builtin_bit_cast(unsigned, f0), 0x07060302u);
+  }
+  return out;
+}
+
 // Fragment of one 32-wide atom at row/column base `rc0` + `rc_step`, contraction atom `kk`.
 //   ES = storage element kind in LDS, EC = compute (MFMA) kind.
 // `rc_step` (a multiple of 16) is the part of the base that is a compile-time constant at the call (the wave's
 // row block i sits i * WM * 32 rows below its first). A contraction-contiguous tile's swizzle looks at row bits
 // 0..3 only, so those rows add a constant number of bytes to the address: kept apart from the lane's part, the
 // constant goes into the read instruction's offset field and the blocks of a wave share their address registers.
-template <int LAYOUT, int ES, int EC, int ROW_BYTES>
+// `PAIRED` (contraction-contiguous 16-bit tiles): atoms 2 d and 2 d + 1 share their 32 contraction entries the way a
+// lane's eight packed int4 bytes hold them: lanes 0-31 own entries 0-15 (first half in the even atom, second in the
+// odd one) and lanes 32-63 entries 16-31, instead of 8 entries per half-wave and atom in ascending order.
+template <int LAYOUT, int ES, int EC, int ROW_BYTES, bool PAIRED = false>
 __device__ __forceinline__ typename Mma<EC>::Frag load_frag(const unsigned char* tile, int rc0, int kk, int lane, int rc_step = 0) {
   typedef typename Mma<EC>::Frag Frag;
   constexpr int KA = Mma<EC>::KA;
@@ -167,7 +189,7 @@ __device__ __forceinline__ typename Mma<EC>::Frag load_frag(const unsigned char*
       f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
       return f;
     } else {
-      return lds_read_b128(tile, kc_offset<ROW_BYTES>(row, kk * 2 + q));
+      return lds_read_b128(tile, kc_offset<ROW_BYTES>(row, PAIRED ? (kk >> 1) * 4 + 2 * q + (kk & 1) : kk * 2 + q));
     }
   } else {
     rc0 += rc_step;
@@ -528,6 +550,11 @@ struct GemmKernel {
                 "per-k-block scales: bf16 lhs with int8 or fp8 weights, fp8 x fp8 or int8 x int8; one 1 KB scale row per k-step");
   static constexpr int BNO = GLU ? BN / 2 : BN;  // output columns of a tile
   static constexpr int EC = EA;  // MFMA type follows A; B may be stored narrower (int8 weights)
+  // Packed int4 weights: a B stage is a byte tile of half the depth; a lane's transposing read of 8 bytes of its
+  // column gives it 16 consecutive contraction entries, the B fragments of two atoms, and the lhs fragments are read
+  // in the matching order (load_frag's PAIRED), so nothing is permuted.
+  static constexpr bool I4 = EB == kEI4;
+  static constexpr int EBS = I4 ? (int)kEI8 : EB;  // element kind of a B stage in LDS
   static constexpr int KA = Mma<EC>::KA;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -546,12 +573,14 @@ struct GemmKernel {
   static constexpr bool LEAN = EA == kEF8 && EB == kEF8 && !SUBK && !SPLIT && TM * TN >= 8;
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
   static_assert(!SPLIT || (MODE == kFwd && EA == EB && BK % 2 == 0), "split pipeline: plain forward, operands of one type");
+  static_assert(!I4 || (MODE == kFwd && EA == kEBF16 && !SPLIT), "packed int4 weights: plain forward with bf16 activations");
+  static constexpr int BKB = I4 ? BKC / 2 : BKC;  // rows of a B stage
   typedef TileStage<LA, EA, BM, BK, THREADS> StageA;
-  typedef TileStage<LB, EB, BN, BKC, THREADS> StageB;
+  typedef TileStage<LB, EBS, BN, BKB, THREADS> StageB;
   // Every wave takes an equal share of a k-step's direct-to-LDS loads.
   static constexpr int NLOAD = WM * WN;
   typedef DirectLoader<LA, EA, BM, BK, NLOAD> DirA;
-  typedef DirectLoader<LB, EB, BN, BKC, NLOAD> DirB;
+  typedef DirectLoader<LB, EBS, BN, BKB, NLOAD> DirB;
   static constexpr int SCALE_BYTES = (SUBK && !SUBP) ? BN * 4 : 0;  // kFwdSubK: the k-step's scale row behind its two tiles
   static constexpr int STAGE_BYTES = StageA::BYTES + StageB::BYTES + SCALE_BYTES;
   // fp8 x fp8: the scales of a k-step (BN weight-column scales, then BM lhs-row scales) are still needed when its
@@ -723,7 +752,7 @@ struct GemmKernel {
         if constexpr (EB == kEI8) return i8x8_to_bf16x8_scaled(v, scale);
         else return f8x8_to_bf16x8_scaled(v, scale);
       } else {
-        return load_frag<LB, EB, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + j * 32, kk, lane);
+        return load_frag<LB, EBS, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + j * 32, kk, lane);
       }
     };
     const int span = kc_end - kc_begin;
@@ -884,7 +913,7 @@ struct GemmKernel {
       da.init(row0, p.m_ext, p.lda, wave, lane, a_lo, a_hi);
       db.init(col0, p.nb_ext, p.ldb, wave, lane, 0, p.nb_ext, GLU ? TN : 0, GLU ? p.n_ext : 0);
       const unsigned char* const gA0 = Ab + DirA::step_base(row0, p.lda, kc_begin);
-      const unsigned char* const gB0 = Bb + DirB::step_base(col0, p.ldb, kc_begin);
+      const unsigned char* const gB0 = Bb + DirB::step_base(col0, p.ldb, I4 ? kc_begin / 2 : kc_begin);
       const int64_t stepA = DirA::step_bytes(p.lda), stepB = DirB::step_bytes(p.ldb);
       const unsigned smem_lds = lds_address32(smem);
       // A load wave may leave the loads of the NS-2 k-steps after the needed one in flight; that
@@ -967,17 +996,39 @@ struct GemmKernel {
         // fragments: A0, B0, B1, ..., then A1, A2, ... Every fragment is then requested at least
         // TM*TN - 2 MFMAs before its first use. A fragment f < TM is the A fragment of row block f,
         // else the B fragment f - TM.
+        // Packed int4 weights: the 8 bytes a lane reads for an even atom hold the B fragments of that atom and of the
+        // next; they are kept as read (`raw`) and converted half by half. The list of an even atom is then A0, the
+        // byte reads, A1, ..., and last the conversions of the first halves; that of an odd atom A0, the conversions
+        // of the second halves, A1, ...
+        [[maybe_unused]] i32x2 raw[I4 ? TN : 1];
+        constexpr int NRD = I4 ? TM + 2 * TN : TM + TN;  // entries of an atom's list
         auto read_frag = [&](Frag* a, Frag* b, int r, const unsigned char* stage, int kk) {
-          if (r >= TM + TN) return;
-          const int f = r == 0 ? 0 : r <= TN ? TM + r - 1 : r - TN;
+          if (r >= NRD) return;
+          const int f = r == 0 ? 0 : r <= TN ? TM + r - 1 : r < TM + TN ? r - TN : r;
           if (f < TM) {
-            if (f < NV) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(stage, wm * 32, kk, lane, f * WM * 32);
+            if (f < NV) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES, I4>(stage, wm * 32, kk, lane, f * WM * 32);
           } else if (f < TM + TN) {
-            if (NV > 0) b[f - TM] = load_b_frag(stage, f - TM, kk);
+            if constexpr (I4) {
+              const int j = f - TM;
+              if (NV > 0) {
+                if (kk & 1) {
+                  b[j] = i4x8_to_bf16x8_times16(raw[j][1]);
+                } else {
+                  const int blk = lane >> 4, s_ = lane & 15;
+                  const int col = wn * WTN + j * 32 + 16 * (blk & 1) + 8 * (s_ & 1);
+                  const int krow = (kk >> 1) * 16 + 8 * (blk >> 1) + (s_ >> 1);
+                  raw[j] = lds_read_tr8(stage + StageA::BYTES + mc_offset<StageB::ROW_BYTES, EBS>(krow, col));
+                }
+              }
+            } else {
+              if (NV > 0) b[f - TM] = load_b_frag(stage, f - TM, kk);
+            }
+          } else if constexpr (I4) {
+            if (NV > 0 && !(kk & 1)) b[f - TM - TN] = i4x8_to_bf16x8_times16(raw[f - TM - TN][0]);
           }
         };
         constexpr int NM = TM * TN;                      // MFMAs per atom
-        constexpr int RPM = (TM + TN + NM - 1) / NM;     // fragment reads threaded after each MFMA
+        constexpr int RPM = (NRD + NM - 1) / NM;         // list entries threaded after each MFMA
         constexpr int LPM = (NLD + NM - 1) / NM;         // load slots threaded after each MFMA
         // (`reads` and `loads` are compile-time tags: a run-time test after every MFMA would put two
         // branches into each MFMA slot.)
@@ -1019,7 +1070,7 @@ struct GemmKernel {
         };
 
 #pragma unroll
-        for (int f = 0; f < TM + TN; ++f) read_frag(fa[0], fb[0], f, smem, 0);
+        for (int f = 0; f < NRD; ++f) read_frag(fa[0], fb[0], f, smem, 0);
         int cur_stage = 0;
         const StepPtrs none = {};
         // One k-step. `refill_tag`: the stage it releases is refilled with k-step kt + NS;
@@ -1098,8 +1149,16 @@ struct GemmKernel {
         for (; kt < nfull; ++kt) k_step(std::false_type{}, std::false_type{}, kt);
       };
       dispatch_upto<0, TM>(nv_sel, k_loop);
+      if constexpr (I4) {
+        // (the weights went into the MFMAs times 16)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) acc[i][j] *= kPackedInt4Unscale;
+      }
     }
-    if constexpr (!GLU && !SUBK) if (tail) {  // (gate-up and per-k-block-scale problems are taken only with whole k-steps)
+    // (gate-up, per-k-block-scale and packed-int4 problems are taken only with whole k-steps)
+    if constexpr (!GLU && !SUBK && !I4) if (tail) {
       typedef TileStage<LA, EA, BM, BKC, THREADS> TailA;  // (an A tile as deep as a compute step)
       for (int kc0 = kc_begin + nmain * BKC; kc0 < kc_end; kc0 += BKC) {
         if (kc0 > kc_begin) __syncthreads();  // the tile's last reads of the LDS written below are done

@@ -1,0 +1,23 @@
+// bf16 activations x packed int4 weights (TKX_I4X2: two values to a byte along the contraction) forward variants.
+// A weight stage is a byte tile half as deep as the k-step; the nibbles are taken apart and converted to bf16 on the
+// way from LDS to the MFMA; per-(group, column) scales in the epilogue. Whole k-steps only (k % block_k == 0).
+#include "tkx_gemm.hip.h"
+
+namespace tkx {
+#define FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEBF16, kEI4, BM, BN, BK, WM, WN, NS)
+
+static const Variant kVariants[] = {
+    FWD(256, 256, 64, 2, 4, 2),
+    FWD(256, 256, 64, 2, 4, 3),
+    FWD(256, 256, 64, 2, 4, 4),
+    FWD(128, 256, 64, 2, 4, 3),
+    FWD(128, 128, 64, 2, 2, 4),
+    FWD(64, 128, 64, 2, 2, 4),
+    FWD(32, 128, 64, 1, 4, 4),
+};
+
+const Variant* variants_i4w(int* count) {
+  *count = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
+  return kVariants;
+}
+}  // namespace tkx

@@ -1,7 +1,8 @@
 """Regenerates the shipped autotuning cache for the device this runs on.
 
 Times every compiled kernel variant on the benchmark workloads (the prefill shapes, the fp8 shape, both
-VJP products, the gate-up fused FFN shape, the small-m decode shape with int8 and with bf16 weights, whose
+VJP products, the gate-up fused FFN shape, int8 and packed int4 weights at the prefill shape, the small-m decode shape
+with int8 and with bf16 weights, whose
 calls are short enough to be timed inside a captured graph, and the "primary" shapes of the reference's own
 benchmark list) and writes
 `tokamax_amd/data/autotuning/<device kind>/hip_ragged_dot.json`, the file `Op.get_autotuning_cache`
@@ -67,7 +68,12 @@ def bound_arguments(op, device):
   a8 = tokamax_amd.QArray(torch.randint(-127, 128, (w.m, w.k), device=device, dtype=torch.int8, generator=gen),
                           (torch.rand(w.m, 1, device=device, generator=gen) + 0.5) / 127)
   yield "mixtral int8 x int8", op.bind(a8, q8, group_sizes=gs, preferred_element_type=torch.bfloat16)
-  del w, q8, a8
+  q4 = tokamax_amd.pack_int4(tokamax_amd.QArray(
+      torch.randint(-8, 8, tuple(w.rhs.shape), device=device, dtype=torch.int8, generator=gen),
+      (torch.rand(w.num_groups, 1, w.n, device=device, generator=gen) + 0.5) / (7 * w.k ** 0.5), None,
+      getattr(torch, "int4", torch.int8)))
+  yield "mixtral int4 packed weights", op.bind(w.lhs, q4, group_sizes=gs, preferred_element_type=torch.bfloat16)
+  del w, q8, a8, q4
   # The reference's own benchmark list (tokamax/_src/ops/ragged_dot/arg_specs.py): its "primary" shapes.
   for spec in arg_specs.ARG_SPECS:
     if "primary" not in spec.tags:

@@ -460,11 +460,16 @@ def _route(lhs, rhs, *, dims, precision, rhs_scale, fuse_gateup_activation, pref
   return _Route(mode, lhs, rhs, lhs_dt, rhs_dt, widen_lhs, widen_rhs, native, cast_bf16, preferred_element_type)
 
 
+_PACKED_INT4_TILE_STEP = 64  # k-step of the tiled kernels that read packed int4 weights
+
+
 def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True):
-  """An rhs of packed int4 (two values per byte along k) stays packed when the streaming small-m kernel takes the call:
-  default dimension numbers, a plain bf16 lhs, no bias and no gate-up fusion (`plain`), at most 8 rows per group on
-  average, k % 1024 == 0, n % 16 == 0, one scale per (group, column) or per (group, k-block, column) with blocks of a
-  power of two >= 32 rows. Every other call gets the values unpacked to int8 storage first (then the int8 paths).
+  """An rhs of packed int4 (two values per byte along k) stays packed when a kernel reads it as it is: default
+  dimension numbers, a plain bf16 lhs, no bias and no gate-up fusion (`plain`), n % 16 == 0, and either
+  * the tiled kernels: one scale per (group, column), k a multiple of their k-step (64), or
+  * the streaming small-m kernel: at most 8 rows per group on average, k % 1024 == 0, one scale per (group, column) or
+    per (group, k-block, column) with blocks of a power of two >= 32 rows.
+  Every other call gets the values unpacked to int8 storage first (then the int8 paths).
   Works on arrays and on shapes, so the forward pass and the choice of a config settle it alike."""
   if not (isinstance(rhs, QArray) and rhs.packed):
     return rhs
@@ -473,10 +478,12 @@ def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True):
   blocks = scale[1] if len(scale) == 3 and scale[0] == g and scale[2] == n and scale[1] >= 1 and k % scale[1] == 0 else None
   rows = k // blocks if blocks else 0
   scale_ok = blocks == 1 or (blocks is not None and rows % 32 == 0 and rows & (rows - 1) == 0)
-  streams = (plain and dims == base.DEFAULT_RAGGED_DOT_DIM_NUMS and not isinstance(lhs, (QArray, AsQArray))
-             and lhs.dtype == torch.bfloat16 and rhs.zero_point is None and scale_ok and lhs.shape[0] <= 8 * g
-             and k % 1024 == 0 and n % 16 == 0 and (k // 8) * n < 2**31 and lhs.shape[0] * k * 2 < 2**32)
-  return rhs if streams else rhs.unpacked()
+  reads_packed = (plain and dims == base.DEFAULT_RAGGED_DOT_DIM_NUMS and not isinstance(lhs, (QArray, AsQArray))
+                  and lhs.dtype == torch.bfloat16 and rhs.zero_point is None and n % 16 == 0)
+  streams = (reads_packed and scale_ok and lhs.shape[0] <= 8 * g and k % 1024 == 0 and (k // 8) * n < 2**31
+             and lhs.shape[0] * k * 2 < 2**32)
+  tiles = reads_packed and blocks == 1 and k % _PACKED_INT4_TILE_STEP == 0
+  return rhs if streams or tiles else rhs.unpacked()
 
 
 def _abstract_operand(x):
@@ -824,6 +831,13 @@ class HipRaggedDot(base.RaggedDot):
     streaming_ok = (mode in (0, 4) and ba.kwargs.get("rhs_bias") is None and contraction % 1024 == 0 and cols % 8 == 0
                     and (contraction // 4) * cols * wbytes < 2**31)
     usable = [v for v in variants if v[0] != 16 or streaming_ok]
+    if key[2] == _lib.TKX_I4X2:
+      # Packed int4 weights: the tiled kernels take whole k-steps and one scale per (group, column); the streaming
+      # kernel a weight slice of whole 16-byte pieces.
+      one_block = route.rhs.scale.shape[1] == 1
+      usable = [v for v in usable if (cols % 16 == 0 if v[0] == 16 else one_block and contraction % v[2] == 0)]
+      if not usable:
+        raise NotImplementedError("No hip kernel reads these packed int4 weights as they are.")
     if mode == 4:
       # The k-step of a tiled variant has to divide the rows of a scale block (and the contraction).
       blocks = route.rhs.scale.shape[1]
@@ -902,6 +916,8 @@ class HipRaggedDot(base.RaggedDot):
     configs = set()
     problem = self._problem(ba)
     for bm, bn, bk, wm, wn, ns in _variant_table().get(key, []):
+      if key[2] == _lib.TKX_I4X2 and bm != 16 and (problem[5] % bk or problem[6].rhs.scale.shape[1] != 1):
+        continue  # (packed int4 weights in a tiled kernel: whole k-steps, one scale per (group, column))
       widths = (1,) if (mode == 2 or bm == 16) else (1, 2, 4, 8, 16)
       for w in widths:
         configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns,

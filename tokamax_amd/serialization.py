@@ -46,6 +46,9 @@ LONG_DTYPE_NAMES = {
     "float8_e4m3fn": torch.float8_e4m3fn, "float8_e5m2": torch.float8_e5m2,
     "float8_e4m3fnuz": torch.float8_e4m3fnuz, "float8_e5m2fnuz": torch.float8_e5m2fnuz,
 }
+# (sub-byte integers, where this torch names them: the qtype of an int4 QArray, "int4" in the reference's keys too)
+LONG_DTYPE_NAMES.update({f"{u}int{b}": getattr(torch, f"{u}int{b}") for u in ("", "u") for b in range(1, 8)
+                         if hasattr(torch, f"{u}int{b}")})
 _LONG_OF = {v: k for k, v in LONG_DTYPE_NAMES.items()}
 
 
@@ -62,8 +65,8 @@ def as_dtype(x) -> torch.dtype:
   raise ValueError(f"unknown dtype: {x!r}")
 
 
-def dtype_name(dtype: torch.dtype) -> str:
-  return _LONG_OF[dtype]
+def dtype_name(dtype) -> str:
+  return dtype if isinstance(dtype, str) else _LONG_OF[dtype]
 
 
 @dataclasses.dataclass(frozen=True)
