@@ -341,7 +341,14 @@ def main():
     cfg = op.bind(w.lhs, q4, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
     measure("mixtral_prefill_int4_packed_weights", lambda: op(w.lhs, q4, group_sizes=gs, preferred_element_type=torch.bfloat16),
             w.flops, w.m * w.k * 2 + w.nonempty_groups * w.k * w.n // 2 + w.m * w.n * 2, "mfma", "bf16", cfg)
-    del w, q8, q8k, a8, q4
+    # the same weights with a scale per (group, block of 128 k rows, column), the usual form of int4 weights
+    q4k = tokamax_amd.QArray(q4.qvalue, (torch.rand(w.num_groups, w.k // 128, w.n, device=device, generator=gen8) + 0.5)
+                             / (7 * w.k ** 0.5), None, q4.qtype)
+    cfg = op.bind(w.lhs, q4k, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_prefill_int4_packed_weights_k_block_scales",
+            lambda: op(w.lhs, q4k, group_sizes=gs, preferred_element_type=torch.bfloat16), w.flops,
+            w.m * w.k * 2 + w.nonempty_groups * (w.k * w.n // 2 + (w.k // 128) * w.n * 4) + w.m * w.n * 2, "mfma", "bf16", cfg)
+    del w, q8, q8k, a8, q4, q4k
 
     w = workloads.make("vjp", device, seed=0)
     gs = torch.tensor(w.group_sizes, device=device)

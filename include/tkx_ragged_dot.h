@@ -53,9 +53,8 @@ enum TkxDtype {
   TKX_I4X2 = 5 /* signed 4-bit integers, two to a byte along the contraction axis: byte [g, kk, c] of an rhs
                   [G, k/2, n] holds k = 2 kk in bits 0-3 and k = 2 kk + 1 in bits 4-7 (two's complement). Taken as the
                   rhs of a bf16 lhs in the default mode by the streaming small-m kernel (block_m == 16, block_n == 128)
-                  and by tiled forward variants of their own (one scale per (group, column) or none, k % block_k == 0,
-                  no gate-up fusion; listed by tkx_ragged_dot_variant); tkx_unpack_int4 turns it into TKX_I8 for
-                  everything else. The reference defines no packed layout (its int4 is jnp.int4; its sm90 kernels
+                  and by tiled forward variants of their own (plain, gate-up fusion, scales per k-block; k % block_k
+                  == 0; listed by tkx_ragged_dot_variant); tkx_unpack_int4 turns it into TKX_I8 for everything else. The reference defines no packed layout (its int4 is jnp.int4; its sm90 kernels
                   read int4 weights in pallas_mosaic_gpu_kernel_sm90_quant.py:46-387). */
 };
 

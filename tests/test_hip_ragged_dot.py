@@ -359,6 +359,11 @@ def test_every_kernel_variant_through_c_abi(v, device):
       rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
       scale = mk((G, 1, n), 0.005).abs() + 1e-3
       rhs_f = O.dequantize(rhs.cpu().numpy(), _np(scale))
+    elif rt == torch.uint8:  # int4 weights, two to a byte along k
+      values = rng.integers(-8, 8, (G, k, n)).astype(np.int8)
+      rhs = torch.tensor(O.pack_int4(values), device=device)
+      scale = mk((G, 1, n), 0.05).abs() + 1e-2
+      rhs_f = O.dequantize(values, _np(scale))
     else:
       rhs = mk((G, k, n), k ** -0.5).to(rt)
       rhs_f = _np(rhs)
@@ -395,6 +400,9 @@ def test_every_kernel_variant_through_c_abi(v, device):
     if rt == torch.int8:
       rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
       rhs_values = rhs.cpu().numpy()
+    elif rt == torch.uint8:  # int4 weights, two to a byte along k
+      rhs_values = rng.integers(-8, 8, (G, k, n)).astype(np.int8)
+      rhs = torch.tensor(O.pack_int4(rhs_values), device=device)
     else:
       rhs = mk((G, k, n), 1.0).to(rt)
       rhs_values = O.e4m3fn_decode(rhs.view(torch.uint8).cpu().numpy())
@@ -830,7 +838,7 @@ def test_small_m_kernel_on_packed_int4_weights(case, scales, depth, split_k, dev
 
 def _packed_int4_tile_cases():
   return [pytest.param(v, id="{block_m}x{block_n}x{block_k}-w{waves_m}x{waves_n}-s{num_stages}".format(**v))
-          for v in _lib.variants(0) if v["rhs_dtype"] == _lib.TKX_I4X2 and v["block_m"] != 16]
+          for v in _lib.variants(0) if v["rhs_dtype"] == _lib.TKX_I4X2 and v["block_m"] != 16 and v["mode"] == 0]
 
 
 @pytest.mark.parametrize("v", _packed_int4_tile_cases())
@@ -855,7 +863,7 @@ def test_tiled_kernels_on_packed_int4_weights(v, device):
   assert torch.count_nonzero(out[int(gs.sum()):]) == 0
   assert torch.equal(out, hip_ops.ragged_dot_fwd(lhs, packed, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale))
   int8_tiles = {(x["block_m"], x["block_n"], x["block_k"], x["waves_m"], x["waves_n"], x["num_stages"])
-                for x in _lib.variants(0) if x["rhs_dtype"] == _lib.TKX_I8 and x["lhs_dtype"] == _lib.TKX_BF16}
+                for x in _lib.variants(0) if x["rhs_dtype"] == _lib.TKX_I8 and x["lhs_dtype"] == _lib.TKX_BF16 and x["mode"] == 0}
   if (cfg.block_m, cfg.block_n, cfg.block_k, cfg.waves_m, cfg.waves_n, cfg.num_stages) in int8_tiles:
     same = hip_ops.ragged_dot_fwd(lhs, torch.tensor(values, device=device), gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale)
     torch.testing.assert_close(out, same, rtol=2e-6, atol=2e-5)
@@ -902,7 +910,24 @@ def test_public_op_on_packed_int4_weights(device):
   bias = torch.tensor(rng.normal(0, 1, (G, 1, n)).astype(np.float32), device=device)
   gs = torch.full((G,), 2, dtype=torch.int32, device=device)
   lhs = torch.tensor(rng.normal(0, 1, (G * 2, k)).astype(np.float32), device=device).to(torch.bfloat16)
-  assert torch.equal(op(lhs, packed, group_sizes=gs, rhs_bias=bias), op(lhs, plain, group_sizes=gs, rhs_bias=bias))
+  # (a bias: the tiled kernels still read the bytes)
+  torch.testing.assert_close(op(lhs, packed, group_sizes=gs, rhs_bias=bias, preferred_element_type=torch.float32),
+                             op(lhs, plain, group_sizes=gs, rhs_bias=bias, preferred_element_type=torch.float32), rtol=1e-5, atol=1e-5)
+  # gate-up fusion and scales per block of 256 k rows, with many rows per group: the tiled kernels' forms for them
+  gs = torch.full((G,), 40, dtype=torch.int32, device=device)
+  lhs = torch.tensor(rng.normal(0, 1, (G * 40, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  torch.testing.assert_close(op(lhs, packed, group_sizes=gs, fuse_gateup_activation="silu", preferred_element_type=torch.float32),
+                             op(lhs, plain, group_sizes=gs, fuse_gateup_activation="silu", preferred_element_type=torch.float32),
+                             rtol=1e-5, atol=1e-5)
+  scale_k = torch.tensor((rng.uniform(0.5, 1.5, (G, k // 256, n)) / 7 * 0.1).astype(np.float32), device=device)
+  plain_k = tokamax_amd.QArray(q, scale_k, None, int4)
+  packed_k = tokamax_amd.pack_int4(plain_k)
+  assert _lib_key(op, lhs, packed_k, gs)[::2] == (4, _lib.TKX_I4X2)
+  out = op(lhs, packed_k, group_sizes=gs, preferred_element_type=torch.float32)
+  want = O.ragged_dot(_np(lhs), O.round_to_bf16(O.dequantize(q.cpu().numpy(), _np(scale_k))), np.full(G, 40, np.int32), O.DEFAULT,
+                      acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, 1e-5)
+  torch.testing.assert_close(out, op(lhs, plain_k, group_sizes=gs, preferred_element_type=torch.float32), rtol=1e-5, atol=1e-5)
 
 
 @pytest.mark.parametrize("groups,n", [(128, 768), (8, 512)])

@@ -639,12 +639,22 @@ def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   lhs, gs = ShapeDtype((4096, 1024), bf16), ShapeDtype((8,), torch.int32)
   route = lambda rhs, **kw: op._problem(op.bind(lhs, rhs, group_sizes=gs, **kw))[1]
   assert route(packed)[2] == _lib.TKX_I4X2
-  # ... unless the call has a bias, scale blocks along k (tiled kernels: one scale per (group, column)), a contraction
-  # that is not a multiple of the k-step, or columns that are not whole 16-byte pieces: int8 storage first
-  assert route(packed, rhs_bias=ShapeDtype((8, 1, 256), f32))[2] == _lib.TKX_I8
-  blocks = tokamax_amd.QArray(ShapeDtype((8, 512, 256), u8), ShapeDtype((8, 4, 256), f32), None, getattr(torch, "int4", i8))
-  assert route(blocks)[2] == _lib.TKX_I8
-  odd = tokamax_amd.QArray(ShapeDtype((8, 48, 256), u8), ShapeDtype((8, 1, 256), f32), None, getattr(torch, "int4", i8))
+  # ... also with a bias, with gate-up fusion, and with scale blocks of a power of two >= 64 rows along k (the forms
+  # the tiled kernels have for int8 weights); unpacked first for gate-up fusion over scale blocks, blocks of 32
+  # rows, a contraction that is not a multiple of the k-step
+  assert route(packed, rhs_bias=ShapeDtype((8, 1, 256), f32))[2] == _lib.TKX_I4X2
+  assert route(packed, fuse_gateup_activation="silu")[::2] == (3, _lib.TKX_I4X2)
+  int4 = getattr(torch, "int4", i8)
+  blocks = tokamax_amd.QArray(ShapeDtype((8, 512, 256), u8), ShapeDtype((8, 4, 256), f32), None, int4)
+  assert route(blocks)[::2] == (4, _lib.TKX_I4X2)
+  assert op._get_heuristics_config(op.bind(lhs, blocks, group_sizes=gs)).block_n == 256
+  assert route(blocks, fuse_gateup_activation="silu")[2] != _lib.TKX_I4X2
+  small_blocks = tokamax_amd.QArray(ShapeDtype((8, 512, 256), u8), ShapeDtype((8, 32, 256), f32), None, int4)
+  assert route(small_blocks)[2] != _lib.TKX_I4X2
+  few_rows = op.bind(ShapeDtype((16, 1024), bf16), small_blocks, group_sizes=gs)   # ... which the streaming kernel takes
+  assert op._problem(few_rows)[1][::2] == (4, _lib.TKX_I4X2) and op._get_heuristics_config(few_rows).block_m == 16
+  assert {x.block_m for x in op._get_autotuning_configs(few_rows)} == {16}
+  odd = tokamax_amd.QArray(ShapeDtype((8, 48, 256), u8), ShapeDtype((8, 1, 256), f32), None, int4)
   assert op._problem(op.bind(ShapeDtype((4096, 96), bf16), odd, group_sizes=gs))[1][2] == _lib.TKX_I8
   space = op._get_autotuning_configs(op.bind(lhs, packed, group_sizes=gs))
   assert {x.block_m for x in space} >= {16, 32, 128, 256}

@@ -290,12 +290,12 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
       return set_error(TKX_ERR_UNSUPPORTED,
                        "fp8 x fp8 with scale blocks along k needs lhs scales f32[blocks, m], m %% 4 == 0 and align_tile %% 4 == 0");
   }
-  // Packed int4 weights in the tiled kernels: plain forward, one scale per (group, column), whole k-steps.
+  // Packed int4 weights in the tiled kernels: the forward forms, whole k-steps.
   const bool packed_tiled = rhs_dtype == TKX_I4X2 && c.block_m != kDecodeBlockM;
-  if (packed_tiled && (dlhs || gateup || subk || c.block_k < 1 || k % c.block_k != 0))
+  if (packed_tiled && (dlhs || c.block_k < 1 || k % c.block_k != 0))
     return set_error(TKX_ERR_UNSUPPORTED,
-                     "packed int4 weights in a tiled kernel: default mode, one rhs scale per (group, column) or none, no gate-up"
-                     " fusion, k %% block_k == 0 (k=%lld block_k=%d); tkx_unpack_int4 gives int8 storage for everything else",
+                     "packed int4 weights in a tiled kernel: default mode and k %% block_k == 0 (k=%lld block_k=%d);"
+                     " tkx_unpack_int4 gives int8 storage for everything else",
                      (long long)k, c.block_k);
   const Variant* v = find_variant(dlhs ? kDlhs : gateup ? kFwdGlu : subk ? kFwdSubK : kFwd, lhs_dtype, rhs_dtype, c);
   if (v == nullptr)

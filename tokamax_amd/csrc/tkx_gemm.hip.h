@@ -245,6 +245,19 @@ __device__ __forceinline__ typename Mma<EC>::Frag load_frag(const unsigned char*
   }
 }
 
+// Eight packed int4 values (see i4x8_to_bf16x8_times16) times one scale, rounded to bf16; `scale16` is the column's
+// scale for the current k-block divided by 16.
+__device__ __forceinline__ i32x4 i4x8_to_bf16x8_scaled(int w, float scale16) {
+  const int lo = (w << 4) & (int)0xF0F0F0F0u, hi = w & (int)0xF0F0F0F0u;
+  bf16x8 out;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    out[2 * u] = (__bf16)((float)(signed char)((lo >> (8 * u)) & 0xff) * scale16);
+    out[2 * u + 1] = (__bf16)((float)(signed char)((hi >> (8 * u)) & 0xff) * scale16);
+  }
+  return __builtin_bit_cast(i32x4, out);
+}
+
 // The same 8 int8 values times one scale (the column's scale for the current k-block), rounded to bf16.
 __device__ __forceinline__ i32x4 i8x8_to_bf16x8_scaled(i32x2 v, float scale) {
   bf16x8 out;
@@ -546,8 +559,8 @@ struct GemmKernel {
   // accumulate into partial accumulators, which are folded into the result with the block's scales.
   // int8 x int8 runs the same way on the int8 MFMAs (int32 partial sums, exact), also with one block.
   static constexpr bool SUBP = SUBK && (EA == kEF8 || EA == kEI8);
-  static_assert(!SUBK || ((EB == kEI8 || EB == kEF8) && (EA == kEBF16 || (SUBP && EB == EA)) && BN == 256),
-                "per-k-block scales: bf16 lhs with int8 or fp8 weights, fp8 x fp8 or int8 x int8; one 1 KB scale row per k-step");
+  static_assert(!SUBK || ((EB == kEI8 || EB == kEF8 || EB == kEI4) && (EA == kEBF16 || (SUBP && EB == EA)) && BN == 256),
+                "per-k-block scales: bf16 lhs with int8, packed int4 or fp8 weights, fp8 x fp8 or int8 x int8; one 1 KB scale row per k-step");
   static constexpr int BNO = GLU ? BN / 2 : BN;  // output columns of a tile
   static constexpr int EC = EA;  // MFMA type follows A; B may be stored narrower (int8 weights)
   // Packed int4 weights: a B stage is a byte tile of half the depth; a lane's transposing read of 8 bytes of its
@@ -573,7 +586,8 @@ struct GemmKernel {
   static constexpr bool LEAN = EA == kEF8 && EB == kEF8 && !SUBK && !SPLIT && TM * TN >= 8;
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
   static_assert(!SPLIT || (MODE == kFwd && EA == EB && BK % 2 == 0), "split pipeline: plain forward, operands of one type");
-  static_assert(!I4 || (MODE == kFwd && EA == kEBF16 && !SPLIT), "packed int4 weights: plain forward with bf16 activations");
+  static_assert(!I4 || ((MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK) && EA == kEBF16 && !SPLIT),
+                "packed int4 weights: forward with bf16 activations");
   static constexpr int BKB = I4 ? BKC / 2 : BKC;  // rows of a B stage
   typedef TileStage<LA, EA, BM, BK, THREADS> StageA;
   typedef TileStage<LB, EBS, BN, BKB, THREADS> StageB;
@@ -1001,6 +1015,16 @@ struct GemmKernel {
         // byte reads, A1, ..., and last the conversions of the first halves; that of an odd atom A0, the conversions
         // of the second halves, A1, ...
         [[maybe_unused]] i32x2 raw[I4 ? TN : 1];
+        // (kFwdSubK: times the scale of the lane's column for the stage's k-block, like load_b_frag)
+        [[maybe_unused]] auto convert_i4 = [&](int w, const unsigned char* stage, int j) -> i32x4 {
+          if constexpr (SUBK) {
+            const float scale = *reinterpret_cast<const float*>(stage + StageA::BYTES + StageB::BYTES +
+                                                                4 * (wn * WTN + j * 32 + (lane & 31)));
+            return i4x8_to_bf16x8_scaled(w, scale * kPackedInt4Unscale);
+          } else {
+            return i4x8_to_bf16x8_times16(w);
+          }
+        };
         constexpr int NRD = I4 ? TM + 2 * TN : TM + TN;  // entries of an atom's list
         auto read_frag = [&](Frag* a, Frag* b, int r, const unsigned char* stage, int kk) {
           if (r >= NRD) return;
@@ -1012,7 +1036,7 @@ struct GemmKernel {
               const int j = f - TM;
               if (NV > 0) {
                 if (kk & 1) {
-                  b[j] = i4x8_to_bf16x8_times16(raw[j][1]);
+                  b[j] = convert_i4(raw[j][1], stage, j);
                 } else {
                   const int blk = lane >> 4, s_ = lane & 15;
                   const int col = wn * WTN + j * 32 + 16 * (blk & 1) + 8 * (s_ & 1);
@@ -1024,7 +1048,7 @@ struct GemmKernel {
               if (NV > 0) b[f - TM] = load_b_frag(stage, f - TM, kk);
             }
           } else if constexpr (I4) {
-            if (NV > 0 && !(kk & 1)) b[f - TM - TN] = i4x8_to_bf16x8_times16(raw[f - TM - TN][0]);
+            if (NV > 0 && !(kk & 1)) b[f - TM - TN] = convert_i4(raw[f - TM - TN][0], stage, f - TM - TN);
           }
         };
         constexpr int NM = TM * TN;                      // MFMAs per atom
@@ -1149,7 +1173,7 @@ struct GemmKernel {
         for (; kt < nfull; ++kt) k_step(std::false_type{}, std::false_type{}, kt);
       };
       dispatch_upto<0, TM>(nv_sel, k_loop);
-      if constexpr (I4) {
+      if constexpr (I4 && !SUBK) {
         // (the weights went into the MFMAs times 16)
 #pragma unroll
         for (int i = 0; i < TM; ++i)

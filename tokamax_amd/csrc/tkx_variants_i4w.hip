@@ -1,10 +1,14 @@
 // bf16 activations x packed int4 weights (TKX_I4X2: two values to a byte along the contraction) forward variants.
 // A weight stage is a byte tile half as deep as the k-step; the nibbles are taken apart and converted to bf16 on the
-// way from LDS to the MFMA; per-(group, column) scales in the epilogue. Whole k-steps only (k % block_k == 0).
+// way from LDS to the MFMA; per-(group, column) scales in the epilogue, or per-(group, k-block, column) scales
+// multiplied in during that conversion (kFwdSubK, 256-column tiles). Whole k-steps only (k % block_k == 0).
 #include "tkx_gemm.hip.h"
 
 namespace tkx {
 #define FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEBF16, kEI4, BM, BN, BK, WM, WN, NS)
+// Gate-up fusion over weights [gate | up] with one scale per (group, column).
+#define GLU(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdGlu, kEBF16, kEI4, BM, BN, BK, WM, WN, NS)
+#define SUBK(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdSubK, kEBF16, kEI4, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
     FWD(256, 256, 64, 2, 4, 2),
@@ -14,6 +18,12 @@ static const Variant kVariants[] = {
     FWD(128, 128, 64, 2, 2, 4),
     FWD(64, 128, 64, 2, 2, 4),
     FWD(32, 128, 64, 1, 4, 4),
+    GLU(256, 256, 64, 2, 4, 3),
+    GLU(128, 256, 64, 2, 4, 3),
+    GLU(32, 256, 64, 1, 4, 4),
+    SUBK(256, 256, 64, 2, 4, 3),
+    SUBK(128, 256, 64, 2, 4, 3),
+    SUBK(32, 256, 64, 1, 4, 4),
 };
 
 const Variant* variants_i4w(int* count) {

@@ -423,12 +423,15 @@ def _route(lhs, rhs, *, dims, precision, rhs_scale, fuse_gateup_activation, pref
   if (gateup or rhs_scale is not None) and mode != 0:
     raise NotImplementedError("rhs_scale and fuse_gateup_activation need the default dimension numbers.")
   if isinstance(rhs, QArray) and rhs.packed:
-    # Packed int4 that `_settle_packed_int4` left packed: bf16 lhs x the streaming small-m kernel, scales as they are.
+    # Packed int4 that `_settle_packed_int4` left packed: bf16 lhs x a kernel that reads the bytes, scales as they are
+    # (blocks along k: the kernels' own form, as for int8 weights).
     if not precision_lib.is_default(lhs.dtype, rhs.dtype, precision):
       raise NotImplementedError(f"{precision=} not supported.")
     if preferred_element_type is None:
       preferred_element_type = torch.promote_types(lhs.dtype, rhs.dtype)
-    return _Route(0, lhs, rhs, torch.bfloat16, torch.uint8, False, False, False, False, preferred_element_type)
+    k_blocks = rhs.scale.shape[1] > 1
+    return _Route(3 if gateup else 4 if k_blocks else 0, lhs, rhs, torch.bfloat16, torch.uint8, False, False, k_blocks,
+                  False, preferred_element_type)
   lhs_dt, rhs_dt = _dtype_of(lhs), _dtype_of(rhs)
   widen_lhs = widen_rhs = native = False
   if mode == 0:
@@ -463,12 +466,13 @@ def _route(lhs, rhs, *, dims, precision, rhs_scale, fuse_gateup_activation, pref
 _PACKED_INT4_TILE_STEP = 64  # k-step of the tiled kernels that read packed int4 weights
 
 
-def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True):
+def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True, gateup: bool = False):
   """An rhs of packed int4 (two values per byte along k) stays packed when a kernel reads it as it is: default
-  dimension numbers, a plain bf16 lhs, no bias and no gate-up fusion (`plain`), n % 16 == 0, and either
-  * the tiled kernels: one scale per (group, column), k a multiple of their k-step (64), or
-  * the streaming small-m kernel: at most 8 rows per group on average, k % 1024 == 0, one scale per (group, column) or
-    per (group, k-block, column) with blocks of a power of two >= 32 rows.
+  dimension numbers, a plain bf16 lhs, n % 16 == 0, and either
+  * the tiled kernels: k a multiple of their k-step (64); one scale per (group, column), or, without gate-up fusion, per
+    (group, k-block, column) with blocks of a power of two >= 64 rows, or
+  * the streaming small-m kernel: no bias and no gate-up fusion (`plain`), at most 8 rows per group on average,
+    k % 1024 == 0, one scale per (group, column) or per (group, k-block, column) with blocks of a power of two >= 32 rows.
   Every other call gets the values unpacked to int8 storage first (then the int8 paths).
   Works on arrays and on shapes, so the forward pass and the choice of a config settle it alike."""
   if not (isinstance(rhs, QArray) and rhs.packed):
@@ -478,11 +482,12 @@ def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True):
   blocks = scale[1] if len(scale) == 3 and scale[0] == g and scale[2] == n and scale[1] >= 1 and k % scale[1] == 0 else None
   rows = k // blocks if blocks else 0
   scale_ok = blocks == 1 or (blocks is not None and rows % 32 == 0 and rows & (rows - 1) == 0)
-  reads_packed = (plain and dims == base.DEFAULT_RAGGED_DOT_DIM_NUMS and not isinstance(lhs, (QArray, AsQArray))
+  reads_packed = (dims == base.DEFAULT_RAGGED_DOT_DIM_NUMS and not isinstance(lhs, (QArray, AsQArray))
                   and lhs.dtype == torch.bfloat16 and rhs.zero_point is None and n % 16 == 0)
-  streams = (reads_packed and scale_ok and lhs.shape[0] <= 8 * g and k % 1024 == 0 and (k // 8) * n < 2**31
+  streams = (reads_packed and plain and scale_ok and lhs.shape[0] <= 8 * g and k % 1024 == 0 and (k // 8) * n < 2**31
              and lhs.shape[0] * k * 2 < 2**32)
-  tiles = reads_packed and blocks == 1 and k % _PACKED_INT4_TILE_STEP == 0
+  tiles = (reads_packed and k % _PACKED_INT4_TILE_STEP == 0
+           and (blocks == 1 or (scale_ok and not gateup and rows % _PACKED_INT4_TILE_STEP == 0)))
   return rhs if streams or tiles else rhs.unpacked()
 
 
@@ -674,7 +679,8 @@ class HipRaggedDot(base.RaggedDot):
     # Quantise / dequantise what the kernels cannot take as it is, then plan the call on shapes and types.
     lhs, rhs = _concrete_operand(lhs), _concrete_operand(rhs)
     rhs = _settle_packed_int4(lhs, rhs, dims=ragged_dot_dimension_numbers,
-                              plain=rhs_bias is None and fuse_gateup_activation is None and rhs_scale is None)
+                              plain=rhs_bias is None and fuse_gateup_activation is None and rhs_scale is None,
+                              gateup=fuse_gateup_activation is not None)
     route = _route(lhs, rhs, dims=ragged_dot_dimension_numbers, precision=precision,
                    rhs_scale=rhs_scale, fuse_gateup_activation=fuse_gateup_activation,
                    preferred_element_type=preferred_element_type)
@@ -799,7 +805,8 @@ class HipRaggedDot(base.RaggedDot):
     lhs, rhs = _abstract_operand(ba.args[0]), _abstract_operand(ba.args[1])
     rhs = _settle_packed_int4(lhs, rhs, dims=ba.kwargs["ragged_dot_dimension_numbers"],
                               plain=(ba.kwargs.get("rhs_bias") is None and ba.kwargs.get("fuse_gateup_activation") is None
-                                     and ba.kwargs.get("rhs_scale") is None))
+                                     and ba.kwargs.get("rhs_scale") is None),
+                              gateup=ba.kwargs.get("fuse_gateup_activation") is not None)
     route = _route(lhs, rhs, dims=ba.kwargs["ragged_dot_dimension_numbers"],
                    precision=ba.kwargs.get("precision"), rhs_scale=ba.kwargs.get("rhs_scale"),
                    fuse_gateup_activation=ba.kwargs.get("fuse_gateup_activation"),
@@ -832,10 +839,9 @@ class HipRaggedDot(base.RaggedDot):
                     and (contraction // 4) * cols * wbytes < 2**31)
     usable = [v for v in variants if v[0] != 16 or streaming_ok]
     if key[2] == _lib.TKX_I4X2:
-      # Packed int4 weights: the tiled kernels take whole k-steps and one scale per (group, column); the streaming
-      # kernel a weight slice of whole 16-byte pieces.
-      one_block = route.rhs.scale.shape[1] == 1
-      usable = [v for v in usable if (cols % 16 == 0 if v[0] == 16 else one_block and contraction % v[2] == 0)]
+      # Packed int4 weights: the tiled kernels take whole k-steps, the streaming kernel a weight slice of whole
+      # 16-byte pieces.
+      usable = [v for v in usable if (cols % 16 == 0 if v[0] == 16 else contraction % v[2] == 0)]
       if not usable:
         raise NotImplementedError("No hip kernel reads these packed int4 weights as they are.")
     if mode == 4:
@@ -915,9 +921,18 @@ class HipRaggedDot(base.RaggedDot):
     mode, key = self._problem(ba)[:2]
     configs = set()
     problem = self._problem(ba)
-    for bm, bn, bk, wm, wn, ns in _variant_table().get(key, []):
-      if key[2] == _lib.TKX_I4X2 and bm != 16 and (problem[5] % bk or problem[6].rhs.scale.shape[1] != 1):
-        continue  # (packed int4 weights in a tiled kernel: whole k-steps, one scale per (group, column))
+    variants = list(_variant_table().get(key, []))
+    if mode == 4:
+      # (the streaming small-m kernel takes scales per k-block in its 128-column form, listed with the plain variants)
+      variants += [v for v in _variant_table().get((0, key[1], key[2]), []) if v[0] == 16 and v[1] == 128]
+    block_rows = 0
+    if mode == 4 and problem[6].rhs.scale.shape[1] > 1:
+      block_rows = problem[5] // problem[6].rhs.scale.shape[1]
+    for bm, bn, bk, wm, wn, ns in variants:
+      if key[2] == _lib.TKX_I4X2 and bm != 16 and problem[5] % bk:
+        continue  # (packed int4 weights in a tiled kernel: whole k-steps)
+      if bm != 16 and block_rows % bk:
+        continue  # (the k-step of a tiled kernel divides the rows of a scale block)
       widths = (1,) if (mode == 2 or bm == 16) else (1, 2, 4, 8, 16)
       for w in widths:
         configs.add(Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns,

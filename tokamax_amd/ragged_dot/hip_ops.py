@@ -217,9 +217,8 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
   G, k, n = rhs.shape
   if rhs.dtype == torch.uint8:
     k *= 2  # packed int4: a byte row holds two contraction rows
-    if trans_rhs or gateup:
-      raise NotImplementedError("packed int4 weights take the default dimension numbers without gate-up fusion;"
-                                " unpack_int4 them first")
+    if trans_rhs:
+      raise NotImplementedError("packed int4 weights take the default dimension numbers; unpack_int4 them first")
   m = lhs.shape[0]
   if group_offset is None:
     if gs.numel() != G:
