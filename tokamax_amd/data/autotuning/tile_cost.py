@@ -3,11 +3,14 @@
 `<device kind>/tile_cost_timings.json` holds, per shape, the measured time of every compiled tiled variant (with and
 without the split of the last round): entries `{"shape": [rows, contraction, cols, groups], "mode": 0 forward | 1 dlhs,
 "streaming_best_us": fastest small-m streaming variant or null, "timings": [[block_m, block_n, block_k, waves_m,
-waves_n, num_stages, split_k, microseconds], ...]}`.
+waves_n, num_stages, split_k, microseconds], ...]}`; entries of bf16 activations over quantised weights (one scale per
+(group, column)) carry `"rhs": "int8"` or `"int4"` (packed two to a byte). The constants are fitted to the bf16 entries;
+the others are what the rules for quantised weights in `HipRaggedDot._get_heuristics_config` were set by and are
+checked against.
 
   python -m tokamax_amd.data.autotuning.tile_cost check              # how far the model's pick is from the fastest
   python -m tokamax_amd.data.autotuning.tile_cost fit [--iterations N]  # refit; prints the constants to paste
-  python -m tokamax_amd.data.autotuning.tile_cost collect M,K,N,G[,dlhs] ...   # time shapes on this GPU and add them
+  python -m tokamax_amd.data.autotuning.tile_cost collect M,K,N,G[,dlhs|int8|int4] ...   # time shapes on this GPU and add them
 
 `check` and `fit` need no GPU.
 """
@@ -37,9 +40,13 @@ def save(entries: list[dict], path: str | None = None) -> None:
     f.write("[\n" + ",\n".join(json.dumps(e, separators=(",", ":")) for e in entries) + "\n]\n")
 
 
+_RHS_BYTES = {"bf16": 2.0, "int8": 1.0, "int4": 0.5}
+
+
 def estimate(entry: dict, timing: list, fit: dict) -> float:
   rows, contraction, cols, groups = entry["shape"]
-  return hip._tile_cost(tuple(timing[:6]), timing[6], rows, cols, contraction, groups, entry["mode"], fit)  # pylint: disable=protected-access
+  return hip._tile_cost(tuple(timing[:6]), timing[6], rows, cols, contraction, groups, entry["mode"], fit,  # pylint: disable=protected-access
+                        _RHS_BYTES[entry.get("rhs", "bf16")])
 
 
 def pick(entry: dict, fit: dict) -> list:
@@ -50,6 +57,35 @@ def pick(entry: dict, fit: dict) -> list:
 def gaps(entries: list[dict], fit: dict) -> list[float]:
   """Per shape: time of the picked variant / time of the fastest tiled variant."""
   return [pick(e, fit)[7] / min(t[7] for t in e["timings"]) for e in entries]
+
+
+def heuristics_gap(entry: dict) -> float:
+  """Time of the config `HipRaggedDot`'s heuristics choose for the entry's problem (on abstract arguments: no GPU) /
+  time of the fastest tiled variant."""
+  import torch  # pylint: disable=g-import-not-at-top
+  import tokamax_amd  # pylint: disable=g-import-not-at-top
+  from tokamax_amd.ragged_dot import base  # pylint: disable=g-import-not-at-top
+  from tokamax_amd.serialization import ShapeDtype  # pylint: disable=g-import-not-at-top
+
+  rows, contraction, cols, groups = entry["shape"]
+  kind, bf16 = entry.get("rhs", "bf16"), torch.bfloat16
+  shape = (groups, contraction, cols) if entry["mode"] == 0 else (groups, cols, contraction)
+  if kind == "bf16":
+    rhs = ShapeDtype(shape, bf16)
+  elif kind == "int8":
+    rhs = tokamax_amd.QArray(ShapeDtype(shape, torch.int8), ShapeDtype((groups, 1, cols), torch.float32))
+  else:
+    rhs = tokamax_amd.QArray(ShapeDtype((groups, contraction // 2, cols), torch.uint8),
+                             ShapeDtype((groups, 1, cols), torch.float32), None, getattr(torch, "int4", torch.int8))
+  kwargs = {} if entry["mode"] == 0 else dict(ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS)
+  op = hip.HipRaggedDot()
+  c = op._get_heuristics_config(  # pylint: disable=protected-access
+      op.bind(ShapeDtype((rows, contraction), bf16), rhs, group_sizes=ShapeDtype((groups,), torch.int32), **kwargs))
+  chosen = [c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages, c.split_k]
+  fastest = min(t[7] for t in entry["timings"])
+  if c.block_m == 16:
+    return entry["streaming_best_us"] / fastest
+  return next(t[7] for t in entry["timings"] if t[:7] == chosen) / fastest
 
 
 def summary(ratios: list[float]) -> tuple[float, float]:
@@ -106,13 +142,23 @@ def collect(specs: list[str], iterations: int) -> None:
   for spec in specs:
     parts = spec.split(",")
     mode = 1 if parts[4:] == ["dlhs"] else 0
+    kind = parts[4] if parts[4:] and parts[4] in ("int8", "int4") else "bf16"
     rows, contraction, cols, groups = (int(x) for x in parts[:4])
     rng = np.random.default_rng(rows + contraction + cols + groups)
     sizes = rng.multinomial(rows, rng.dirichlet(np.ones(groups) * 4)).astype(np.int32)
     group_sizes = torch.tensor(sizes, device=device)
     lhs = torch.randn(rows, contraction, device=device, generator=gen).to(torch.bfloat16)
     shape = (groups, contraction, cols) if mode == 0 else (groups, cols, contraction)
-    rhs = (torch.randn(*shape, device=device, generator=gen) * contraction**-0.5).to(torch.bfloat16)
+    if kind == "bf16":
+      rhs = (torch.randn(*shape, device=device, generator=gen) * contraction**-0.5).to(torch.bfloat16)
+    else:
+      top = 127 if kind == "int8" else 7
+      rhs = tokamax_amd.QArray(
+          torch.randint(-top, top + 1, shape, device=device, dtype=torch.int8, generator=gen),
+          (torch.rand(groups, 1, cols, device=device, generator=gen) + 0.5) / (top * contraction**0.5), None,
+          None if kind == "int8" else getattr(torch, "int4", torch.int8))
+      if kind == "int4":
+        rhs = tokamax_amd.pack_int4(rhs)
     kwargs = {} if mode == 0 else dict(ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS)
     bound = op.bind(lhs, rhs, group_sizes=group_sizes, **kwargs)
     configs = {c for c in bound.autotuning_configs if c.block_m == 16 or c.grid_tile_width == 8}
@@ -124,6 +170,7 @@ def collect(specs: list[str], iterations: int) -> None:
     entry = dict(
         shape=[rows, contraction, cols, groups],
         mode=mode,
+        **({} if kind == "bf16" else {"rhs": kind}),
         streaming_best_us=round(min(streaming), 2) if streaming else None,
         timings=sorted(
             (
@@ -134,7 +181,8 @@ def collect(specs: list[str], iterations: int) -> None:
             key=lambda t: t[7],
         ),
     )
-    entries = [e for e in entries if (e["shape"], e["mode"]) != (entry["shape"], mode)] + [entry]
+    same = lambda e: (e["shape"], e["mode"], e.get("rhs", "bf16")) == (entry["shape"], mode, kind)
+    entries = [e for e in entries if not same(e)] + [entry]
     save(entries, path)
     chosen = pick(entry, hip._TILE_COST_FIT)  # pylint: disable=protected-access
     print(spec, "fastest", entry["timings"][0], "model's pick", chosen, flush=True)
@@ -152,6 +200,8 @@ def main() -> None:
     collect(args.shapes, args.iterations or 6)
     return
   entries = load()
+  others = [e for e in entries if e.get("rhs", "bf16") != "bf16"]
+  entries = [e for e in entries if e.get("rhs", "bf16") == "bf16"]
   if args.command == "fit":
     fitted = refit(entries, dict(current, launch_us=7.0), args.iterations or 3000)
     fitted.pop("launch_us")
@@ -163,6 +213,11 @@ def main() -> None:
   mean, worst = summary(gaps(entries, current))
   print(f"{len(entries)} shapes, {sum(len(e['timings']) for e in entries)} timings: the model's pick is "
         f"{100 * mean:.1f} % above the fastest variant on average, {100 * worst:.0f} % at worst")
+  for kind in ["bf16"] + sorted({e["rhs"] for e in others}):
+    some = [e for e in others if e["rhs"] == kind] if kind != "bf16" else entries
+    mean, worst = summary([heuristics_gap(e) for e in some])
+    print(f"the heuristics' config on the {len(some)} shapes with {kind} weights: {100 * mean:.1f} % above the fastest "
+          f"tiled variant on average, {100 * worst:.0f} % at worst")
 
 
 if __name__ == "__main__":

@@ -105,7 +105,7 @@ _TILE_COST_FIT = dict(
 
 
 def _tile_cost(variant, split_k: int, rows: int, cols: int, contraction: int, num_groups: int, mode: int = 0,
-               fit=_TILE_COST_FIT) -> float:
+               fit=_TILE_COST_FIT, rhs_bytes: float = 2.0) -> float:
   """Estimated time (us) of a tiled forward / dlhs launch of 16-bit operands: rounds of workgroups times the time of a
   tile. A tile's k-step costs the larger of its MFMA time (less where the task's rows do not fill the share of the
   wave that holds them) and the time to bring its operand slices into LDS, which a pipeline with less than about 65
@@ -124,7 +124,7 @@ def _tile_cost(variant, split_k: int, rows: int, cols: int, contraction: int, nu
   tasks = min(rows / bm + fit["group_straddle"] * num_groups, -(-rows // bm) + num_groups - 1)
   tiles = tasks * -(-cols // bn)
   four_waves = wm * wn == 4
-  two_per_cu = four_waves and 2 * ns * (bm + bn) * bk * 2 <= 160 * 1024
+  two_per_cu = four_waves and 2 * ns * (bm * 2 + bn * rhs_bytes) * bk <= 160 * 1024
   # (the waves of a tile split its rows `wm` ways and the slowest one sets the pace: the rows count against a wave's share)
   active = min(1.0, (rows / tasks + fit["partial_block"] * 32) * wm / bm)
   mma_us = bm * bn * bk * 2 / fit["mfma_flop_per_us"] * active * (fit["four_wave_factor"] if four_waves else 1.0)
@@ -132,7 +132,7 @@ def _tile_cost(variant, split_k: int, rows: int, cols: int, contraction: int, nu
   # (a 32-element slice of an operand that is contiguous along the contraction, as the lhs is and in dlhs the weights
   # are too, is read in 64-byte pieces)
   short = fit["short_piece"] if bk < 64 else 1.0
-  load_us = (bm * short + bn * (short if mode == 1 else 1.0)) * bk * 2 / fit["load_byte_per_us"] / in_flight
+  load_us = (bm * 2 * short + bn * rhs_bytes * (short if mode == 1 else 1.0)) * bk / fit["load_byte_per_us"] / in_flight
   steps = -(-contraction // bk)
   fixed_us = fit["fixed_us"] + fit["fixed_area_us"] * bm * bn / 65536
   alone_us = steps * max(mma_us, load_us) + fixed_us
@@ -858,6 +858,16 @@ class HipRaggedDot(base.RaggedDot):
               else 32 if rows_per_group > 8 else 16)  # 16 = one pass of the streaming kernel; the mean must
     # leave room for the largest group, which re-reads its weights for every further 16 rows
     want_n = 256 if cols >= 2048 else 128
+    if mode == 0 and key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2) and rows_per_group >= 96:
+      # int8 / packed int4 weights with one scale per (group, column): a tile converts its weight fragments once per
+      # wave row, so the taller tile pays off earlier (measured on 14 shapes each: the 256-row tile wins from about
+      # 256 rows per group, the 128-row one from about 100).
+      want_m = 256 if rows_per_group >= 224 else 128
+      # ... unless so few tiles come of it that half the chip would idle: then the largest tile that gives every CU one.
+      tiles = lambda bm, bn: (rows / bm + 0.88 * num_groups) * -(-cols // bn)
+      if tiles(want_m, want_n) < _COMPUTE_UNITS // 2:
+        want_m, want_n = next((t for t in ((256, 256), (128, 256), (128, 128), (64, 128)) if t[0] <= want_m
+                               and tiles(*t) >= _COMPUTE_UNITS), (32, 128))
     # The streaming kernel on int8 weights has a wide form (256 columns per workgroup, two workgroups
     # per CU) that streams 7-9% faster when its workgroups fill the chip evenly, and slower than the
     # 128-column form when they do not (measured: 384 workgroups on 256 CUs lose 10%).
@@ -913,7 +923,12 @@ class HipRaggedDot(base.RaggedDot):
     elif modelled_split is not None:
       split_k = modelled_split
     elif _tiled_split_pays(mode, bm, bn, rows, cols, num_groups):
-      split_k = 4
+      # (16-bit activations: only where the estimate of the launch says that the shorter last round is worth the
+      # exchange, which a short contraction is not)
+      v, rb = (bm, bn, bk, wm, wn, ns), {_lib.TKX_I8: 1.0, _lib.TKX_I4X2: 0.5}.get(key[2], 2.0)
+      estimate = lambda sk: _tile_cost(v, sk, rows, cols, contraction, num_groups, mode, rhs_bytes=rb)
+      if key[1] not in (_lib.TKX_BF16, _lib.TKX_F16) or estimate(4) < estimate(1):
+        split_k = 4
     return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns, grid_tile_width=width,
                   align_tile=8, split_k=split_k)
 
