@@ -700,17 +700,18 @@ def test_tile_cost_model_picks_near_the_fastest_measured_variant():
   estimates follow the form of the data: more rows or a longer contraction never cost less, and a launch with a sliver
   of a last round gains from the split while one without a partial round does not."""
   from tokamax_amd.data.autotuning import tile_cost
-  entries = [e for e in tile_cost.load() if e.get("rhs", "bf16") == "bf16"]
+  entries = [e for e in tile_cost.load() if e.get("rhs", "bf16") == "bf16" and e["mode"] != 2]
   assert len(entries) >= 100 and all(len(e["timings"]) >= 10 for e in entries)
   mean, worst = tile_cost.summary(tile_cost.gaps(entries, hip._TILE_COST_FIT))
   assert mean < 0.06 and worst < 0.35, (mean, worst)
   # the config the heuristics hand out for those problems (model, rules for the streaming kernel, split decision), and
-  # for bf16 activations over int8 / packed int4 weights, where rules on rows per group and on the fill of the chip
-  # choose the tile (26 measured shapes each)
-  for kind, most in (("bf16", 0.06), ("int8", 0.08), ("int4", 0.06)):
-    some = [e for e in tile_cost.load() if e.get("rhs", "bf16") == kind]
+  # for quantised operands and drhs, where rules on rows per group and on the fill of the chip choose the tile
+  label = lambda e: "drhs" if e["mode"] == 2 else e.get("rhs", "bf16")
+  for kind, count, most in (("bf16", 122, 0.06), ("int8", 26, 0.08), ("int4", 26, 0.06), ("fp8", 26, 0.03),
+                            ("int8x8", 12, 0.03), ("drhs", 26, 0.03)):
+    some = [e for e in tile_cost.load() if label(e) == kind]
     mean, worst = tile_cost.summary([tile_cost.heuristics_gap(e) for e in some])
-    assert len(some) >= 24 and mean < most and worst < 0.4, (kind, mean, worst)
+    assert len(some) >= count and mean < most and worst < 0.4, (kind, mean, worst)
   v = (256, 256, 64, 2, 2, 2)
   costs = [hip._tile_cost(v, 1, rows, 4096, 4096, 8) for rows in (1024, 4096, 16384, 65536, 262144)]
   assert costs == sorted(costs) and costs[-1] > 30 * costs[1]

@@ -4,13 +4,15 @@
 without the split of the last round): entries `{"shape": [rows, contraction, cols, groups], "mode": 0 forward | 1 dlhs,
 "streaming_best_us": fastest small-m streaming variant or null, "timings": [[block_m, block_n, block_k, waves_m,
 waves_n, num_stages, split_k, microseconds], ...]}`; entries of bf16 activations over quantised weights (one scale per
-(group, column)) carry `"rhs": "int8"` or `"int4"` (packed two to a byte). The constants are fitted to the bf16 entries;
+(group, column)) carry `"rhs": "int8"` or `"int4"` (packed two to a byte), fp8 x fp8 entries `"rhs": "fp8"`, int8 x int8
+entries `"rhs": "int8x8"`; mode 2 is
+drhs with `"shape": [m, k, n, groups]`. The constants are fitted to the bf16 entries;
 the others are what the rules for quantised weights in `HipRaggedDot._get_heuristics_config` were set by and are
 checked against.
 
   python -m tokamax_amd.data.autotuning.tile_cost check              # how far the model's pick is from the fastest
   python -m tokamax_amd.data.autotuning.tile_cost fit [--iterations N]  # refit; prints the constants to paste
-  python -m tokamax_amd.data.autotuning.tile_cost collect M,K,N,G[,dlhs|int8|int4] ...   # time shapes on this GPU and add them
+  python -m tokamax_amd.data.autotuning.tile_cost collect M,K,N,G[,dlhs|drhs|int8|int4|fp8|int8x8] ...   # time shapes on this GPU and add them
 
 `check` and `fit` need no GPU.
 """
@@ -59,28 +61,55 @@ def gaps(entries: list[dict], fit: dict) -> list[float]:
   return [pick(e, fit)[7] / min(t[7] for t in e["timings"]) for e in entries]
 
 
+def arguments(entry: dict, array):
+  """(lhs, rhs, keyword arguments) of the entry's problem. `array(shape, dtype, top)` makes one array (abstract, or
+  on the GPU with values of magnitude `top`)."""
+  import torch  # pylint: disable=g-import-not-at-top
+  import tokamax_amd  # pylint: disable=g-import-not-at-top
+  from tokamax_amd.ragged_dot import base  # pylint: disable=g-import-not-at-top
+
+  kind, mode = entry.get("rhs", "bf16"), entry["mode"]
+  bf16, f32 = torch.bfloat16, torch.float32
+  if mode == 2:  # drhs: shape = [m, k, n, groups], out[g, k, n] = lhs[rows of g, k]^T . dout[rows of g, n]
+    m, k, n, groups = entry["shape"]
+    return array((m, k), bf16, 1.0), array((m, n), bf16, 1.0), dict(
+        ragged_dot_dimension_numbers=base.RAGGED_CONTRACTING_DOT_DIM_NUMS)
+  rows, contraction, cols, groups = entry["shape"]
+  kwargs = {} if mode == 0 else dict(ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS)
+  shape = (groups, contraction, cols) if mode == 0 else (groups, cols, contraction)
+  lhs = array((rows, contraction), bf16, 1.0)
+  if kind == "bf16":
+    return lhs, array(shape, bf16, contraction**-0.5), kwargs
+  if kind == "fp8":  # both operands e4m3fn, one scale per row and per (group, column)
+    f8 = torch.float8_e4m3fn
+    lhs = tokamax_amd.QArray(array((rows, contraction), f8, 1.0), array((rows, 1), f32, 1.0))
+    return lhs, tokamax_amd.QArray(array(shape, f8, 1.0), array((groups, 1, cols), f32, contraction**-0.5)), dict(
+        kwargs, preferred_element_type=bf16)
+  if kind == "int8x8":  # int8 activations (one scale per row) over int8 weights (one per (group, column)): the int8 MFMAs
+    lhs = tokamax_amd.QArray(array((rows, contraction), torch.int8, 127), array((rows, 1), f32, 1 / 127))
+    rhs = tokamax_amd.QArray(array(shape, torch.int8, 127), array((groups, 1, cols), f32, 1.0 / (127 * contraction**0.5)))
+    return lhs, rhs, dict(kwargs, preferred_element_type=bf16)
+  top = 127 if kind == "int8" else 7
+  rhs = tokamax_amd.QArray(array(shape, torch.int8, top), array((groups, 1, cols), f32, 1.0 / (top * contraction**0.5)),
+                           None, None if kind == "int8" else getattr(torch, "int4", torch.int8))
+  if kind == "int4":
+    if isinstance(rhs.qvalue, torch.Tensor):
+      rhs = tokamax_amd.pack_int4(rhs)
+    else:
+      rhs = tokamax_amd.QArray(array((groups, contraction // 2, cols), torch.uint8, 0), rhs.scale, None, rhs.qtype)
+  return lhs, rhs, dict(kwargs, preferred_element_type=bf16)
+
+
 def heuristics_gap(entry: dict) -> float:
   """Time of the config `HipRaggedDot`'s heuristics choose for the entry's problem (on abstract arguments: no GPU) /
   time of the fastest tiled variant."""
   import torch  # pylint: disable=g-import-not-at-top
-  import tokamax_amd  # pylint: disable=g-import-not-at-top
-  from tokamax_amd.ragged_dot import base  # pylint: disable=g-import-not-at-top
   from tokamax_amd.serialization import ShapeDtype  # pylint: disable=g-import-not-at-top
 
-  rows, contraction, cols, groups = entry["shape"]
-  kind, bf16 = entry.get("rhs", "bf16"), torch.bfloat16
-  shape = (groups, contraction, cols) if entry["mode"] == 0 else (groups, cols, contraction)
-  if kind == "bf16":
-    rhs = ShapeDtype(shape, bf16)
-  elif kind == "int8":
-    rhs = tokamax_amd.QArray(ShapeDtype(shape, torch.int8), ShapeDtype((groups, 1, cols), torch.float32))
-  else:
-    rhs = tokamax_amd.QArray(ShapeDtype((groups, contraction // 2, cols), torch.uint8),
-                             ShapeDtype((groups, 1, cols), torch.float32), None, getattr(torch, "int4", torch.int8))
-  kwargs = {} if entry["mode"] == 0 else dict(ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS)
+  lhs, rhs, kwargs = arguments(entry, lambda shape, dtype, top: ShapeDtype(shape, dtype))
   op = hip.HipRaggedDot()
   c = op._get_heuristics_config(  # pylint: disable=protected-access
-      op.bind(ShapeDtype((rows, contraction), bf16), rhs, group_sizes=ShapeDtype((groups,), torch.int32), **kwargs))
+      op.bind(lhs, rhs, group_sizes=ShapeDtype((entry["shape"][3],), torch.int32), **kwargs))
   chosen = [c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages, c.split_k]
   fastest = min(t[7] for t in entry["timings"])
   if c.block_m == 16:
@@ -139,27 +168,24 @@ def collect(specs: list[str], iterations: int) -> None:
   tuner = autotuner_lib.Autotuner(iterations=iterations, warmup=2)
   op = tokamax_amd.HipRaggedDot()
   gen = torch.Generator(device=device).manual_seed(1)
+  def array(shape, dtype, top):
+    if dtype in (torch.int8, torch.uint8):
+      return torch.randint(-top, top + 1, shape, device=device, dtype=torch.int8, generator=gen)
+    if dtype == torch.float32:
+      return (torch.rand(shape, device=device, generator=gen) + 0.5) * top
+    return (torch.randn(shape, device=device, generator=gen) * top).to(dtype)
+
   for spec in specs:
     parts = spec.split(",")
-    mode = 1 if parts[4:] == ["dlhs"] else 0
-    kind = parts[4] if parts[4:] and parts[4] in ("int8", "int4") else "bf16"
-    rows, contraction, cols, groups = (int(x) for x in parts[:4])
-    rng = np.random.default_rng(rows + contraction + cols + groups)
-    sizes = rng.multinomial(rows, rng.dirichlet(np.ones(groups) * 4)).astype(np.int32)
+    tag = parts[4] if parts[4:] else ""
+    mode = {"dlhs": 1, "drhs": 2}.get(tag, 0)
+    kind = tag if tag in ("int8", "int4", "fp8", "int8x8") else "bf16"
+    dims = [int(x) for x in parts[:4]]
+    rng = np.random.default_rng(sum(dims))
+    sizes = rng.multinomial(dims[0], rng.dirichlet(np.ones(dims[3]) * 4)).astype(np.int32)
     group_sizes = torch.tensor(sizes, device=device)
-    lhs = torch.randn(rows, contraction, device=device, generator=gen).to(torch.bfloat16)
-    shape = (groups, contraction, cols) if mode == 0 else (groups, cols, contraction)
-    if kind == "bf16":
-      rhs = (torch.randn(*shape, device=device, generator=gen) * contraction**-0.5).to(torch.bfloat16)
-    else:
-      top = 127 if kind == "int8" else 7
-      rhs = tokamax_amd.QArray(
-          torch.randint(-top, top + 1, shape, device=device, dtype=torch.int8, generator=gen),
-          (torch.rand(groups, 1, cols, device=device, generator=gen) + 0.5) / (top * contraction**0.5), None,
-          None if kind == "int8" else getattr(torch, "int4", torch.int8))
-      if kind == "int4":
-        rhs = tokamax_amd.pack_int4(rhs)
-    kwargs = {} if mode == 0 else dict(ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS)
+    entry = dict(shape=dims, mode=mode, **({} if kind == "bf16" else {"rhs": kind}))
+    lhs, rhs, kwargs = arguments(entry, array)
     bound = op.bind(lhs, rhs, group_sizes=group_sizes, **kwargs)
     configs = {c for c in bound.autotuning_configs if c.block_m == 16 or c.grid_tile_width == 8}
     data = tuner.autotune(
@@ -167,10 +193,7 @@ def collect(specs: list[str], iterations: int) -> None:
     )
     us = {c: d.median_evaluation_time_ms * 1e3 for c, d in data.items() if hasattr(d, "median_evaluation_time_ms")}
     streaming = [t for c, t in us.items() if c.block_m == 16]
-    entry = dict(
-        shape=[rows, contraction, cols, groups],
-        mode=mode,
-        **({} if kind == "bf16" else {"rhs": kind}),
+    entry.update(
         streaming_best_us=round(min(streaming), 2) if streaming else None,
         timings=sorted(
             (
@@ -181,11 +204,10 @@ def collect(specs: list[str], iterations: int) -> None:
             key=lambda t: t[7],
         ),
     )
-    same = lambda e: (e["shape"], e["mode"], e.get("rhs", "bf16")) == (entry["shape"], mode, kind)
+    same = lambda e: (e["shape"], e["mode"], e.get("rhs", "bf16")) == (dims, mode, kind)
     entries = [e for e in entries if not same(e)] + [entry]
     save(entries, path)
-    chosen = pick(entry, hip._TILE_COST_FIT)  # pylint: disable=protected-access
-    print(spec, "fastest", entry["timings"][0], "model's pick", chosen, flush=True)
+    print(spec, "fastest", entry["timings"][0], f"heuristics {100 * (heuristics_gap(entry) - 1):.0f} % behind", flush=True)
     del lhs, rhs, bound
 
 
@@ -200,8 +222,9 @@ def main() -> None:
     collect(args.shapes, args.iterations or 6)
     return
   entries = load()
-  others = [e for e in entries if e.get("rhs", "bf16") != "bf16"]
-  entries = [e for e in entries if e.get("rhs", "bf16") == "bf16"]
+  label = lambda e: "drhs" if e["mode"] == 2 else e.get("rhs", "bf16")
+  others = [e for e in entries if label(e) != "bf16"]
+  entries = [e for e in entries if label(e) == "bf16"]  # (what the model is fitted to: forward and dlhs of bf16 operands)
   if args.command == "fit":
     fitted = refit(entries, dict(current, launch_us=7.0), args.iterations or 3000)
     fitted.pop("launch_us")
@@ -213,10 +236,10 @@ def main() -> None:
   mean, worst = summary(gaps(entries, current))
   print(f"{len(entries)} shapes, {sum(len(e['timings']) for e in entries)} timings: the model's pick is "
         f"{100 * mean:.1f} % above the fastest variant on average, {100 * worst:.0f} % at worst")
-  for kind in ["bf16"] + sorted({e["rhs"] for e in others}):
-    some = [e for e in others if e["rhs"] == kind] if kind != "bf16" else entries
+  for kind in ["bf16"] + sorted({label(e) for e in others}):
+    some = [e for e in others if label(e) == kind] if kind != "bf16" else entries
     mean, worst = summary([heuristics_gap(e) for e in some])
-    print(f"the heuristics' config on the {len(some)} shapes with {kind} weights: {100 * mean:.1f} % above the fastest "
+    print(f"the heuristics' config on the {len(some)} {kind} shapes: {100 * mean:.1f} % above the fastest "
           f"tiled variant on average, {100 * worst:.0f} % at worst")
 
 

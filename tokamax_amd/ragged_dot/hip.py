@@ -858,11 +858,15 @@ class HipRaggedDot(base.RaggedDot):
               else 32 if rows_per_group > 8 else 16)  # 16 = one pass of the streaming kernel; the mean must
     # leave room for the largest group, which re-reads its weights for every further 16 rows
     want_n = 256 if cols >= 2048 else 128
-    if mode == 0 and key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2) and rows_per_group >= 96:
-      # int8 / packed int4 weights with one scale per (group, column): a tile converts its weight fragments once per
-      # wave row, so the taller tile pays off earlier (measured on 14 shapes each: the 256-row tile wins from about
-      # 256 rows per group, the 128-row one from about 100).
+    quantised = ((key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2))
+                 or (key[1] == key[2] and key[1] in (_lib.TKX_F8E4M3FN, _lib.TKX_I8)))
+    if mode == 0 and quantised and rows_per_group >= 96:
+      # bf16 activations over int8 / packed int4 weights with one scale per (group, column), fp8 x fp8, int8 x int8:
+      # the taller and wider tile pays off earlier than the thresholds above say (measured on 14 shapes per kind,
+      # int8 x int8 excepted: the 256-row tile wins from about 256 rows per group, the 128-row one from about 100, and
+      # 256 columns from a few tiles' worth of them).
       want_m = 256 if rows_per_group >= 224 else 128
+      want_n = 256 if cols >= 512 else 128
       # ... unless so few tiles come of it that half the chip would idle: then the largest tile that gives every CU one.
       tiles = lambda bm, bn: (rows / bm + 0.88 * num_groups) * -(-cols // bn)
       if tiles(want_m, want_n) < _COMPUTE_UNITS // 2:
@@ -923,11 +927,14 @@ class HipRaggedDot(base.RaggedDot):
     elif modelled_split is not None:
       split_k = modelled_split
     elif _tiled_split_pays(mode, bm, bn, rows, cols, num_groups):
-      # (16-bit activations: only where the estimate of the launch says that the shorter last round is worth the
-      # exchange, which a short contraction is not)
-      v, rb = (bm, bn, bk, wm, wn, ns), {_lib.TKX_I8: 1.0, _lib.TKX_I4X2: 0.5}.get(key[2], 2.0)
-      estimate = lambda sk: _tile_cost(v, sk, rows, cols, contraction, num_groups, mode, rhs_bytes=rb)
-      if key[1] not in (_lib.TKX_BF16, _lib.TKX_F16) or estimate(4) < estimate(1):
+      # ... only where the estimate of the launch says that the shorter last round is worth the exchange, which a
+      # short contraction is not. (One-byte activations: a k-step moves the bytes and takes the MFMA time of a
+      # 16-bit k-step half as long.)
+      narrow = 2 if key[1] in (_lib.TKX_F8E4M3FN, _lib.TKX_I8) else 1
+      v, rb = (bm, bn, bk // narrow, wm, wn, ns), {_lib.TKX_I8: 1.0, _lib.TKX_I4X2: 0.5}.get(key[2], 2.0)
+      estimate = lambda sk: _tile_cost(v, sk, rows, cols, contraction // narrow, num_groups, mode,
+                                       rhs_bytes=2.0 if narrow == 2 else rb)
+      if key[1] == _lib.TKX_F32 or estimate(4) < estimate(1):
         split_k = 4
     return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns, grid_tile_width=width,
                   align_tile=8, split_k=split_k)
