@@ -858,17 +858,15 @@ class HipRaggedDot(base.RaggedDot):
               else 32 if rows_per_group > 8 else 16)  # 16 = one pass of the streaming kernel; the mean must
     # leave room for the largest group, which re-reads its weights for every further 16 rows
     want_n = 256 if cols >= 2048 else 128
-    quantised = ((key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2))
-                 or (key[1] == key[2] and key[1] in (_lib.TKX_F8E4M3FN, _lib.TKX_I8)))
-    if mode == 0 and quantised and rows_per_group >= 96:
-      # bf16 activations over int8 / packed int4 weights with one scale per (group, column), fp8 x fp8, int8 x int8:
-      # the taller and wider tile pays off earlier than the thresholds above say (measured on 14 shapes per kind,
-      # int8 x int8 excepted: the 256-row tile wins from about 256 rows per group, the 128-row one from about 100, and
-      # 256 columns from a few tiles' worth of them).
+    if mode in (0, 3, 4) and key[1] != _lib.TKX_F32 and rows_per_group >= 96:
+      # The forward kernels other than f32 (16-bit operands without scales are re-ranked by the cost model below): the
+      # taller and wider tile pays off earlier than the thresholds above say. Measured on 14 shapes per kind (int8 and
+      # packed int4 weights, fp8 x fp8, gate-up fusion, scales per k-block): the 256-row tile wins from about 256
+      # rows per group, the 128-row one from about 100, and 256 columns from a few tiles' worth of them.
       want_m = 256 if rows_per_group >= 224 else 128
       want_n = 256 if cols >= 512 else 128
       # ... unless so few tiles come of it that half the chip would idle: then the largest tile that gives every CU one.
-      tiles = lambda bm, bn: (rows / bm + 0.88 * num_groups) * -(-cols // bn)
+      tiles = lambda bm, bn: (rows / bm + 0.88 * num_groups) * -(-cols // (bn // 2 if mode == 3 else bn))
       if tiles(want_m, want_n) < _COMPUTE_UNITS // 2:
         want_m, want_n = next((t for t in ((256, 256), (128, 256), (128, 128), (64, 128)) if t[0] <= want_m
                                and tiles(*t) >= _COMPUTE_UNITS), (32, 128))
