@@ -5,14 +5,14 @@ without the split of the last round): entries `{"shape": [rows, contraction, col
 "streaming_best_us": fastest small-m streaming variant or null, "timings": [[block_m, block_n, block_k, waves_m,
 waves_n, num_stages, split_k, microseconds], ...]}`; entries of bf16 activations over quantised weights (one scale per
 (group, column)) carry `"rhs": "int8"` or `"int4"` (packed two to a byte), fp8 x fp8 entries `"rhs": "fp8"`, int8 x int8
-entries `"rhs": "int8x8"`, bf16 gate-up fusion `"glu"`, int8 weights with scales per 128 k rows `"int8k"`; mode 2 is
+entries `"rhs": "int8x8"`, bf16 gate-up fusion `"glu"`, int8 weights with scales per 128 k rows `"int8k"`, f32 operands `"f32"`; mode 2 is
 drhs with `"shape": [m, k, n, groups]`. The constants are fitted to the bf16 entries;
 the others are what the rules for quantised weights in `HipRaggedDot._get_heuristics_config` were set by and are
 checked against.
 
   python -m tokamax_amd.data.autotuning.tile_cost check              # how far the model's pick is from the fastest
   python -m tokamax_amd.data.autotuning.tile_cost fit [--iterations N]  # refit; prints the constants to paste
-  python -m tokamax_amd.data.autotuning.tile_cost collect M,K,N,G[,dlhs|drhs|int8|int4|fp8|int8x8|glu|int8k] ...   # time shapes on this GPU and add them
+  python -m tokamax_amd.data.autotuning.tile_cost collect M,K,N,G[,dlhs|drhs|int8|int4|fp8|int8x8|glu|int8k|f32] ...   # time shapes on this GPU and add them
 
 `check` and `fit` need no GPU.
 """
@@ -80,6 +80,8 @@ def arguments(entry: dict, array):
   lhs = array((rows, contraction), bf16, 1.0)
   if kind == "bf16":
     return lhs, array(shape, bf16, contraction**-0.5), kwargs
+  if kind == "f32":
+    return array((rows, contraction), f32, 1.0), array(shape, f32, contraction**-0.5), kwargs
   if kind == "glu":  # bf16 gate-up fusion: `cols` output columns from weights [gate | up] of twice as many
     return lhs, array((groups, contraction, 2 * cols), bf16, contraction**-0.5), dict(kwargs, fuse_gateup_activation="silu")
   if kind == "int8k":  # bf16 activations over int8 weights with one scale per (group, 128 k rows, column)
@@ -185,7 +187,7 @@ def collect(specs: list[str], iterations: int) -> None:
     parts = spec.split(",")
     tag = parts[4] if parts[4:] else ""
     mode = {"dlhs": 1, "drhs": 2}.get(tag, 0)
-    kind = tag if tag in ("int8", "int4", "fp8", "int8x8", "glu", "int8k") else "bf16"
+    kind = tag if tag in ("int8", "int4", "fp8", "int8x8", "glu", "int8k", "f32") else "bf16"
     dims = [int(x) for x in parts[:4]]
     rng = np.random.default_rng(sum(dims))
     sizes = rng.multinomial(dims[0], rng.dirichlet(np.ones(dims[3]) * 4)).astype(np.int32)

@@ -870,6 +870,11 @@ class HipRaggedDot(base.RaggedDot):
       if tiles(want_m, want_n) < _COMPUTE_UNITS // 2:
         want_m, want_n = next((t for t in ((256, 256), (128, 256), (128, 128), (64, 128)) if t[0] <= want_m
                                and tiles(*t) >= _COMPUTE_UNITS), (32, 128))
+    if mode == 0 and key[1] == _lib.TKX_F32:
+      # f32 operands run on the f32 MFMAs at a sixteenth of the bf16 rate: loads never bound them, and the 32-row tile
+      # (four of its workgroups share a CU) was the fastest of the three on every measured shape, 128 to 1400 rows
+      # per group (9-47 % ahead of the taller ones).
+      want_m, want_n = 32, 128
     # The streaming kernel on int8 weights has a wide form (256 columns per workgroup, two workgroups
     # per CU) that streams 7-9% faster when its workgroups fill the chip evenly, and slower than the
     # 128-column form when they do not (measured: 384 workgroups on 256 CUs lose 10%).
