@@ -2090,3 +2090,19 @@ def test_split_workspace_is_never_released_when_a_call_needs_a_larger_one(device
     assert small.data_ptr() == address and small.numel() == words
     assert hip_ops.split_workspace(16, 1024, 4, device) is big  # later calls share the larger one
   stream.synchronize()
+
+
+def test_timing_tool_collects_every_kind_of_problem(tmp_path, device):
+  """The tool behind the heuristics' thresholds (`tokamax_amd/data/autotuning/tile_cost.py collect`) times every
+  variant of a small problem of each kind it knows, writes entries `check` can read back, and finds the heuristics'
+  config among the timed ones."""
+  from tokamax_amd.data.autotuning import tile_cost
+  path = str(tmp_path / "timings.json")
+  kinds = ["", ",dlhs", ",drhs", ",int8", ",int4", ",fp8", ",int8x8", ",glu", ",int8k", ",f32"]
+  tile_cost.collect(["768,256,512,4" + k for k in kinds], 2, path=path)
+  entries = tile_cost.load(path)
+  assert len(entries) == len(kinds) and all(e["timings"] and e["timings"][0][7] > 0 for e in entries)
+  assert {e.get("rhs", "bf16") for e in entries} == {"bf16", "int8", "int4", "fp8", "int8x8", "glu", "int8k", "f32"}
+  assert sorted(e["mode"] for e in entries) == [0] * 8 + [1, 2]
+  for e in entries:
+    assert 1.0 <= tile_cost.heuristics_gap(e) < 3.0, e["shape"]

@@ -160,7 +160,9 @@ def refit(entries: list[dict], start: dict, iterations: int, seed: int = 0) -> d
   return best
 
 
-def collect(specs: list[str], iterations: int) -> None:
+def collect(specs: list[str], iterations: int, path: str | None = None) -> None:
+  """Times every tiled and streaming variant on the problems `specs` name and adds the entries to the timings file of
+  this device (or to `path`)."""
   import numpy as np  # pylint: disable=g-import-not-at-top
   import torch  # pylint: disable=g-import-not-at-top
   import tokamax_amd  # pylint: disable=g-import-not-at-top
@@ -170,7 +172,7 @@ def collect(specs: list[str], iterations: int) -> None:
   from tokamax_amd.ragged_dot import base  # pylint: disable=g-import-not-at-top
 
   device = torch.device("cuda:0")
-  path = timings_path(cache_lib.device_dir_name(op_lib.device_kind(device)))
+  path = path or timings_path(cache_lib.device_dir_name(op_lib.device_kind(device)))
   os.makedirs(os.path.dirname(path), exist_ok=True)
   entries = load(path) if os.path.exists(path) else []
   tuner = autotuner_lib.Autotuner(iterations=iterations, warmup=2)
