@@ -11,6 +11,7 @@ import pytest
 import torch
 
 import tokamax_amd
+from tokamax_amd import _lib
 from oracle import ragged_dot_oracle as O
 from tokamax_amd.ragged_dot import arg_specs, base, workloads
 
@@ -130,6 +131,38 @@ def test_fp8_config(device):
   _check_rows(out, lhs_f, lambda g: _np(w.rhs[g]) * _np(w.rhs_scale[g]), rows, groups, 3e-3)
   assert torch.equal(tokamax_amd.ragged_dot(tokamax_amd.QArray(w.lhs, w.lhs_scale), tokamax_amd.QArray(w.rhs, w.rhs_scale),
                                             gs, preferred_element_type=torch.bfloat16), out)
+
+
+@pytest.mark.parametrize("scales", ["per_column", "per_128_k_rows"])
+def test_packed_int4_weights_at_the_prefill_size(scales, device):
+  """The Mixtral prefill shape over int4 weights packed two to a byte, read by the tiled kernels as they are: one row
+  out of every 32-row block of every group against the oracle's definition on the unpacked, dequantised values (with
+  scales per k-block the kernel rounds weight x scale to bf16, like the reference's in-kernel dequantisation), exact
+  linearity, determinism."""
+  w = workloads.make("mixtral", device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  gen = torch.Generator(device=device).manual_seed(3)
+  q = torch.randint(-8, 8, tuple(w.rhs.shape), device=device, dtype=torch.int8, generator=gen)
+  blocks = 1 if scales == "per_column" else w.k // 128
+  scale = (torch.rand(w.num_groups, blocks, w.n, device=device, generator=gen) + 0.5) / (7 * w.k ** 0.5)
+  packed = tokamax_amd.pack_int4(tokamax_amd.QArray(q, scale, None, getattr(torch, "int4", torch.int8)))
+  assert packed.packed and tuple(packed.qvalue.shape) == (w.num_groups, w.k // 2, w.n)
+  op = tokamax_amd.HipRaggedDot()
+  bound = op.bind(w.lhs, packed, group_sizes=gs, preferred_element_type=torch.bfloat16)
+  assert op._problem(bound)[1][2] == _lib.TKX_I4X2 and bound.default_config.block_m >= 128  # stays packed, tiled kernel
+  out = tokamax_amd.ragged_dot(w.lhs, packed, gs, preferred_element_type=torch.bfloat16)
+  assert out.dtype == torch.bfloat16 and tuple(out.shape) == (w.m, w.n)
+  rows, groups = _sample_every_block(w.group_sizes, 2)
+  assert len(rows) >= w.m // 32
+  lhs_f = _np(w.lhs[torch.as_tensor(rows, device=device)])
+
+  def weights(g):
+    values = O.dequantize(q[g].cpu().numpy()[None], _np(scale[g])[None])[0]
+    return O.round_to_bf16(values) if blocks > 1 else values
+
+  _check_rows(out, lhs_f, weights, rows, groups, 3e-3)
+  assert torch.equal(tokamax_amd.ragged_dot(w.lhs * 2, packed, gs, preferred_element_type=torch.bfloat16), out * 2)
+  assert torch.equal(tokamax_amd.ragged_dot(w.lhs, packed, gs, preferred_element_type=torch.bfloat16), out)
 
 
 def test_vjp_config(device):
