@@ -421,6 +421,14 @@ def main():
         dense_bf16_matmul_nt_tflops=round(dense_flops / (t_nt / steps) / 1e9, 1),
         copy_1gib_read_plus_write_gbs=round(2 * (1 << 30) / (t_cp / steps) / 1e6, 1),
         note="torch.matmul [16384,4096] x [4096,14336] bf16 (random normal data) and torch copy_ of 1 GiB, HIP-event timed")
+    # This library's kernels on the same dense problem (one group holding every row), in both layouts: the forward
+    # kernel on the [k, n] weights and the TRANS_RHS kernel on the k-contiguous ones.
+    one_group = torch.tensor([16384], dtype=torch.int32, device=device)
+    t_own_nn, _, _ = _time_steps(lambda: op(a_, b_nn[None], group_sizes=one_group), steps, warm, stream)
+    t_own_nt, _, _ = _time_steps(lambda: op(a_, b_nt[None], group_sizes=one_group,
+                                            ragged_dot_dimension_numbers=base.TRANS_RHS_RAGGED_DOT_DIM_NUMS), steps, warm, stream)
+    ceilings["this_library_same_problem_nn_tflops"] = round(dense_flops / (t_own_nn / steps) / 1e9, 1)
+    ceilings["this_library_same_problem_nt_tflops"] = round(dense_flops / (t_own_nt / steps) / 1e9, 1)
     del b_nn, c_, src_, dst_
     # The vendor's dense fp8 GEMM (e4m3fn x e4m3fn -> bf16, one scale per tensor) at the same shape, where this torch
     # build has it for the device; it takes the weights k-contiguous (the NT layout).
