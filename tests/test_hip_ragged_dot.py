@@ -1054,14 +1054,15 @@ def test_random_shapes_through_the_public_op(seed, device):
   assert torch.count_nonzero(drhs[torch.tensor(gs == 0, device=device)]) == 0
 
 
-@pytest.mark.parametrize("seed", range(32))
+@pytest.mark.parametrize("seed", range(42))
 def test_random_quantised_problems_through_the_public_op(seed, device):
   """Seeded random problems with quantised operands: int8 weights with one scale per (group, column), per k-block or
-  per (k-block, 16-column block); int8 x int8 and fp8 x fp8 with per-row / per-column scales. Whatever route the
-  call takes (epilogue scales, scaled while widened, folded per k-block, widening pass, streaming kernel), the result
-  is the oracle's contraction of the dequantised operands."""
+  per (k-block, 16-column block); int8 x int8 and fp8 x fp8 with per-row / per-column scales; int4 weights packed two
+  to a byte with one scale per (group, column) or per k-block. Whatever route the call takes (epilogue scales, scaled
+  while widened, folded per k-block, widening pass, streaming kernel, packed bytes read as they are or unpacked first),
+  the result is the oracle's contraction of the dequantised operands."""
   rng = np.random.default_rng(5000 + seed)
-  kind = ("int8_column", "int8_k_blocks", "int8_tiles", "int8_int8", "fp8_fp8")[seed % 5]
+  kind = ("int8_column", "int8_k_blocks", "int8_tiles", "int8_int8", "fp8_fp8", "int4_column", "int4_k_blocks")[seed % 7]
   G = int(rng.integers(1, 8))
   k, n = 64 * int(rng.integers(1, 9)), 16 * int(rng.integers(1, 30))
   per_group = (2, 40, 200)[int(rng.integers(0, 3))]
@@ -1080,6 +1081,14 @@ def test_random_quantised_problems_through_the_public_op(seed, device):
     scale = (rng.uniform(0.5, 1.5, (G, blocks, cols)) / 127 * k ** -0.5).astype(np.float32)
     rhs = tokamax_amd.QArray(tensor(w8, torch.int8), tensor(scale))
     lhs_f, rhs_f, tol = _np(lhs), O.dequantize(w8, scale), 2e-3
+  elif kind in ("int4_column", "int4_k_blocks"):
+    lhs = tensor(rng.normal(0, 1, (m, k)).astype(np.float32), torch.bfloat16)
+    w4 = rng.integers(-8, 8, (G, k, n)).astype(np.int8)
+    blocks = 1 if kind == "int4_column" else k // 64
+    scale = (rng.uniform(0.5, 1.5, (G, blocks, n)) / 7 * k ** -0.5).astype(np.float32)
+    rhs = tokamax_amd.pack_int4(tokamax_amd.QArray(tensor(w4, torch.int8), tensor(scale), None, getattr(torch, "int4", torch.int8)))
+    assert rhs.packed
+    lhs_f, rhs_f, tol = _np(lhs), O.dequantize(w4, scale), 2e-3
   elif kind == "int8_int8":
     a8 = rng.integers(-127, 128, (m, k)).astype(np.int8)
     sa = (rng.uniform(0.5, 1.5, (m, 1)) / 127).astype(np.float32)
