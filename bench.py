@@ -374,7 +374,30 @@ def main():
     nb = (m_ * k_ + 8 * k_ * 2 * n_ + m_ * n_) * 2
     measure("mixtral_gateup_silu_bf16", lambda: op(lhs, rhs, group_sizes=gs, fuse_gateup_activation="silu"),
             2 * m_ * k_ * 2 * n_, nb, "mfma", "bf16", cfg)
-    del lhs, rhs
+    # The whole expert FFN of a Mixtral layer around those two products, as a caller strings it together: tokens
+    # permuted into expert order (ragged_gather), gate-up product with silu(gate) * up in the epilogue, down
+    # projection, weighted top-2 combine back into token order (ragged_gather_reduce). 8192 tokens, top 2 of 8 experts.
+    tokens = m_ // 2
+    h = torch.randn(tokens, k_, device=device, dtype=torch.bfloat16, generator=gen)
+    down = (torch.randn(8, n_, k_, device=device, dtype=torch.float32, generator=gen) * n_ ** -0.5).to(torch.bfloat16)
+    expert_of_slot = torch.repeat_interleave(torch.arange(8, device=device), gs.long())[torch.randperm(m_, device=device, generator=gen)]
+    order = torch.argsort(expert_of_slot, stable=True)             # slot (token, choice) -> position in expert order
+    token_of_row = (order // 2).to(torch.int32)
+    inverse = torch.argsort(order).to(torch.int32)
+    gate_w = torch.rand(m_, device=device, generator=gen)
+    valid = torch.ones(m_, dtype=torch.bool, device=device)
+
+    def ffn_block():
+      x = tokamax_amd.ragged_gather(h, token_of_row, 0, tokens)
+      y = op(x, rhs, group_sizes=gs, fuse_gateup_activation="silu")
+      z = op(y, down, group_sizes=gs)
+      return tokamax_amd.ragged_gather_reduce(z, inverse, gate_w, valid, 2)
+
+    block_flops = 3 * 2 * m_ * k_ * n_
+    block_bytes = (tokens * k_ * 2 + 8 * k_ * 3 * n_) * 2  # tokens in and out, the three weight matrices of every expert
+    measure("moe_ffn_block_mixtral_bf16", ffn_block, block_flops, block_bytes, "mfma", "bf16", cfg)
+    extras["moe_ffn_block_mixtral_bf16"]["steps"] = "ragged_gather, gate-up ragged_dot (silu fused), down ragged_dot, ragged_gather_reduce (top-2 combine)"
+    del lhs, rhs, h, down
 
     # The reference's own benchmark shapes with published timings on other hardware (tokamax/_src/ops/ragged_dot/
     # arg_specs.py:23-60; standard-normal inputs and representative group sizes as its benchmarks make them):
