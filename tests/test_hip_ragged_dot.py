@@ -872,6 +872,16 @@ def test_tiled_kernels_on_packed_int4_weights(v, device):
   _check(plain, O.ragged_dot(_np(lhs), values.astype(np.float64), gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 4e-3)
   with pytest.raises(NotImplementedError, match="block_k"):
     hip_ops.ragged_dot_fwd(lhs[:, :k - 32].contiguous(), packed[:, :k // 2 - 16].contiguous(), gst, config=cfg, out_dtype=torch.float32)
+  # one expert-parallel shard: the sizes of every group of the job, the weights of groups 1..3 only, a bias
+  offset = torch.tensor([1], dtype=torch.int32, device=device)
+  bias = torch.tensor(rng.normal(0, 1, (3, 1, n)).astype(np.float32), device=device)
+  shard = hip_ops.ragged_dot_fwd(lhs, packed[1:4].contiguous(), gst, config=cfg, out_dtype=torch.float32,
+                                 rhs_scale=scale[1:4].contiguous(), rhs_bias=bias, group_offset=offset)
+  lo, hi = int(gs[:1].sum()), int(gs[:4].sum())
+  want_shard = np.zeros((m, n))
+  want_shard[lo:hi] = want[lo:hi] + np.repeat(_np(bias)[:, 0], gs[1:4], axis=0)
+  _check(shard, want_shard, 1e-5)
+  assert torch.count_nonzero(shard[:lo]) == 0 and torch.count_nonzero(shard[hi:]) == 0
 
 
 def _lib_key(op, lhs, rhs, gs):
