@@ -634,8 +634,10 @@ def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   assert packed.unpacked().qvalue.shape == (8, 1024, 256) and packed.unpacked().qvalue.dtype == i8
   c = config(16, 1024, 256, 8, u8, packed=True)          # 2 rows per group: the streaming kernel reads the bytes
   assert c.block_m == 16
-  c = config(4096, 1024, 4096, 8, u8, packed=True)       # 512 rows per group: a tiled kernel reads the bytes too
-  assert c.block_m == 256
+  c = config(4096, 1024, 4096, 8, u8, packed=True)       # 512 rows per group: a tiled kernel reads the bytes too,
+  assert (c.block_m, c.block_n, c.waves_m, c.waves_n) == (128, 256, 1, 8)  # the one whose workgroups share a CU in pairs
+  c = config(4096, 1024, 4096, 8, i8)                    # ... as for int8 weights (two stages: 64 KB of LDS)
+  assert (c.block_m, c.block_n, c.waves_m, c.waves_n, c.num_stages) == (128, 256, 1, 8, 2)
   c = config(4096, 1024, 256, 8, u8, packed=True)        # ... a smaller tile where 256 x 256 would leave most CUs idle
   assert c.block_m in (32, 64)
   lhs, gs = ShapeDtype((4096, 1024), bf16), ShapeDtype((8,), torch.int32)

@@ -604,7 +604,12 @@ struct GemmKernel {
   // Workgroups the register budget is set for: two 4-wave workgroups share a CU when their LDS fits twice (256
   // registers per lane each); every other shape has the CU, and a SIMD's 512 registers per lane, to itself or to the
   // two waves of one 8-wave workgroup.
-  static constexpr int kWorkgroupsPerCu = THREADS <= 256 && 2 * SMEM_BYTES <= 160 * 1024 ? 2 : 1;
+  // (An 8-wave workgroup on one row of waves with 64 accumulators per lane, the 128 x 256 tile, fits twice as well
+  // when its LDS does: 128 registers each.)
+  static constexpr int kWorkgroupsPerCu =
+      (THREADS <= 256 || (WM == 1 && TM * TN * 16 <= 64)) && 2 * SMEM_BYTES <= 160 * 1024 ? 2 : 1;
+  // What the launch bound asks for: waves per SIMD with that many workgroups on the CU.
+  static constexpr int kWavesPerSimd = (THREADS / 64 + 3) / 4 * kWorkgroupsPerCu;
   static_assert(NS >= 2 && SMEM_BYTES <= 160 * 1024, "stages must fit the 160 KB LDS");
 
   // QO: the instantiation that stores fp8 with one scale per (row, 128 columns) (QOUT kernels only). It is a kernel of
@@ -1536,17 +1541,17 @@ struct GemmKernel {
 
 // (4-wave workgroups whose LDS lets two of them share a CU: at most 256 registers per lane, so that two do fit.)
 template <class K>
-__global__ __launch_bounds__(K::THREADS, K::kWorkgroupsPerCu) void gemm_entry(const GemmParams p) {
+__global__ __launch_bounds__(K::THREADS, K::kWavesPerSimd) void gemm_entry(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char tkx_smem[];
   K::run(p, tkx_smem);
 }
 template <class K>
-__global__ __launch_bounds__(K::THREADS, K::kWorkgroupsPerCu) void gemm_entry_fp8_out(const GemmParams p) {
+__global__ __launch_bounds__(K::THREADS, K::kWavesPerSimd) void gemm_entry_fp8_out(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char tkx_smem[];
   K::template run<true>(p, tkx_smem);
 }
 template <class K>
-__global__ __launch_bounds__(K::THREADS, K::kWorkgroupsPerCu) void gemm_entry_split(const GemmParams p) {
+__global__ __launch_bounds__(K::THREADS, K::kWavesPerSimd) void gemm_entry_split(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char tkx_smem[];
   K::template run<false, true>(p, tkx_smem);
 }

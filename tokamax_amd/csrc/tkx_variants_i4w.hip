@@ -2,6 +2,8 @@
 // A weight stage is a byte tile half as deep as the k-step; the nibbles are taken apart and converted to bf16 on the
 // way from LDS to the MFMA; per-(group, column) scales in the epilogue, or per-(group, k-block, column) scales
 // multiplied in during that conversion (kFwdSubK, 256-column tiles). Whole k-steps only (k % block_k == 0).
+// Variants with waves (1, 8) or (1, 4): one row of waves, every weight fragment converted once per workgroup; the
+// 128 x 256 x 64 ones keep 72-75 KB of LDS and 128 registers, so two of their workgroups share a CU.
 #include "tkx_gemm.hip.h"
 
 namespace tkx {
@@ -14,15 +16,21 @@ static const Variant kVariants[] = {
     FWD(256, 256, 64, 2, 4, 2),
     FWD(256, 256, 64, 2, 4, 3),
     FWD(256, 256, 64, 2, 4, 4),
+    FWD(256, 256, 64, 1, 8, 3),
     FWD(128, 256, 64, 2, 4, 3),
+    FWD(128, 256, 64, 1, 8, 3),
     FWD(128, 128, 64, 2, 2, 4),
+    FWD(128, 128, 64, 1, 4, 4),
     FWD(64, 128, 64, 2, 2, 4),
+    FWD(64, 128, 64, 1, 4, 4),
     FWD(32, 128, 64, 1, 4, 4),
     GLU(256, 256, 64, 2, 4, 3),
     GLU(128, 256, 64, 2, 4, 3),
     GLU(32, 256, 64, 1, 4, 4),
     SUBK(256, 256, 64, 2, 4, 3),
+    SUBK(256, 256, 64, 1, 8, 3),
     SUBK(128, 256, 64, 2, 4, 3),
+    SUBK(128, 256, 64, 1, 8, 3),
     SUBK(32, 256, 64, 1, 4, 4),
 };
 

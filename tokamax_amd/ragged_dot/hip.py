@@ -105,7 +105,7 @@ _TILE_COST_FIT = dict(
 
 
 def _tile_cost(variant, split_k: int, rows: int, cols: int, contraction: int, num_groups: int, mode: int = 0,
-               fit=_TILE_COST_FIT, rhs_bytes: float = 2.0) -> float:
+               fit=_TILE_COST_FIT, rhs_bytes: float = 2.0, shares_cu: bool | None = None) -> float:
   """Estimated time (us) of a tiled forward / dlhs launch of 16-bit operands: rounds of workgroups times the time of a
   tile. A tile's k-step costs the larger of its MFMA time (less where the task's rows do not fill the share of the
   wave that holds them) and the time to bring its operand slices into LDS, which a pipeline with less than about 65
@@ -125,6 +125,8 @@ def _tile_cost(variant, split_k: int, rows: int, cols: int, contraction: int, nu
   tiles = tasks * -(-cols // bn)
   four_waves = wm * wn == 4
   two_per_cu = four_waves and 2 * ns * (bm * 2 + bn * rhs_bytes) * bk <= 160 * 1024
+  if shares_cu is not None:
+    two_per_cu = shares_cu  # (the caller knows: 8-wave tiles of converted weights on one row of waves can share too)
   # (the waves of a tile split its rows `wm` ways and the slowest one sets the pace: the rows count against a wave's share)
   active = min(1.0, (rows / tasks + fit["partial_block"] * 32) * wm / bm)
   mma_us = bm * bn * bk * 2 / fit["mfma_flop_per_us"] * active * (fit["four_wave_factor"] if four_waves else 1.0)
@@ -146,7 +148,8 @@ def _tile_cost(variant, split_k: int, rows: int, cols: int, contraction: int, nu
   total = full_rounds * tile_us
   if rest > 0:
     last = alone_us if two_per_cu and rest <= _COMPUTE_UNITS else tile_us
-    if full_rounds > 0:
+    if full_rounds > 0 and not shares_cu:
+      # (not behind a round of paired 8-wave workgroups: those start together and end together)
       last *= fit["tail_floor"] + (1 - fit["tail_floor"]) * rest / slots
     if split_k > 1:
       beyond = int(tiles) % _COMPUTE_UNITS
@@ -859,13 +862,20 @@ class HipRaggedDot(base.RaggedDot):
     # leave room for the largest group, which re-reads its weights for every further 16 rows (measured: at 5 and 6 rows
     # per group the streaming kernel is ahead or within 10 %, at 8 the 32-row tiles are up to 40 % ahead)
     want_n = 256 if cols >= 2048 else 128
-    if mode in (0, 3, 4) and key[1] != _lib.TKX_F32 and rows_per_group >= 96:
+    # bf16 activations over int8 / packed int4 weights with one scale per (group, column): the 128 x 256 tile on one
+    # row of waves is small enough for two workgroups to share a CU (64 KB of LDS with two stages of int8 weights, 72 KB
+    # with three of int4; 128 registers) and was the fastest or within a few percent of it from 12 rows per group up to
+    # 2048 (43 measured shapes per kind).
+    converted_plain = mode == 0 and key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2)
+    if mode in (0, 3, 4) and key[1] != _lib.TKX_F32 and rows_per_group >= (12 if converted_plain else 96):
       # The forward kernels other than f32 (16-bit operands without scales are re-ranked by the cost model below): the
       # taller and wider tile pays off earlier than the thresholds above say. Measured on 14 shapes per kind (int8 and
       # packed int4 weights, fp8 x fp8, gate-up fusion, scales per k-block): the 256-row tile wins from about 256
       # rows per group, the 128-row one from about 100, and 256 columns from a few tiles' worth of them.
       want_m = 256 if rows_per_group >= 224 else 128
       want_n = 256 if cols >= 512 else 128
+      if converted_plain:
+        want_m = 128
       # ... unless so few tiles come of it that half the chip would idle: then the largest tile that gives every CU one.
       tiles = lambda bm, bn: (rows / bm + 0.88 * num_groups) * -(-cols // (bn // 2 if mode == 3 else bn))
       if tiles(want_m, want_n) < _COMPUTE_UNITS // 2:
@@ -901,7 +911,19 @@ class HipRaggedDot(base.RaggedDot):
       # (With per-k-block scales the shorter k-step measured 3 % faster at equal depth: 991 against 961 TFLOP/s.)
       # Integer or fp8 MFMAs on both sides: the longer k-step again.
       short_k = mode == 4 and key[1] == _lib.TKX_BF16
-      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), -in_flight, bk if short_k else -bk, ns)
+      # Weights that are converted on the way from LDS to the MFMA (int8, packed int4, fp8 under a bf16 lhs): every
+      # wave converts the fragments of its own columns, so one row of waves converts each weight once where two rows
+      # convert it twice (measured 1.01-1.44 x, typically 1.1-1.2 x, over three shapes, both scale forms, both tile
+      # heights; 16-bit operands lose 5 % with it: their LDS reads grow by half and nothing is saved).
+      converted = key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2, _lib.TKX_F8E4M3FN)
+      two_wave_rows = wm - 1 if converted else 0
+      # ... and among those, the variant whose LDS lets two of its workgroups share a CU (the library gives such a
+      # kernel 128 registers: 8 waves on one row, at most 64 accumulators per lane)
+      stage_bytes = (bm * 2 + bn * (0.5 if key[2] == _lib.TKX_I4X2 else 1.0)) * bk + (bn * 4 if mode == 4 else 0)
+      alone_on_cu = 0 if (converted and wm == 1 and wn == 8 and bm * bn <= 128 * 256
+                          and 2 * ns * stage_bytes <= 160 * 1024) else 1
+      return (abs(bm - want_m), abs(bn - want_n), -(wm * wn), two_wave_rows, alone_on_cu if converted else 0, -in_flight,
+              bk if short_k else -bk, ns)
 
     bm, bn, bk, wm, wn, ns = min(usable, key=score)
     modelled_split = None
@@ -936,8 +958,12 @@ class HipRaggedDot(base.RaggedDot):
       # 16-bit k-step half as long.)
       narrow = 2 if key[1] in (_lib.TKX_F8E4M3FN, _lib.TKX_I8) else 1
       v, rb = (bm, bn, bk // narrow, wm, wn, ns), {_lib.TKX_I8: 1.0, _lib.TKX_I4X2: 0.5}.get(key[2], 2.0)
+      shares = None
+      if key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2, _lib.TKX_F8E4M3FN) and wm == 1 and wn == 8:
+        stage = (bm * 2 + bn * rb) * bk + (bn * 4 if mode == 4 else 0)
+        shares = bm * bn <= 128 * 256 and 2 * ns * stage <= 160 * 1024
       estimate = lambda sk: _tile_cost(v, sk, rows, cols, contraction // narrow, num_groups, mode,
-                                       rhs_bytes=2.0 if narrow == 2 else rb)
+                                       rhs_bytes=2.0 if narrow == 2 else rb, shares_cu=shares)
       if key[1] == _lib.TKX_F32 or estimate(4) < estimate(1):
         split_k = 4
     return Config(block_m=bm, block_n=bn, block_k=bk, waves_m=wm, waves_n=wn, num_stages=ns, grid_tile_width=width,
