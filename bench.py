@@ -374,6 +374,15 @@ def main():
     nb = (m_ * k_ + 8 * k_ * 2 * n_ + m_ * n_) * 2
     measure("mixtral_gateup_silu_bf16", lambda: op(lhs, rhs, group_sizes=gs, fuse_gateup_activation="silu"),
             2 * m_ * k_ * 2 * n_, nb, "mfma", "bf16", cfg)
+    # the same call over int4 weights packed two to a byte (one scale per (group, column))
+    q4g = tokamax_amd.pack_int4(tokamax_amd.QArray(
+        torch.randint(-8, 8, (8, k_, 2 * n_), device=device, dtype=torch.int8, generator=gen),
+        (torch.rand(8, 1, 2 * n_, device=device, generator=gen) + 0.5) / (7 * k_ ** 0.5), None, getattr(torch, "int4", torch.int8)))
+    cfg4 = op.bind(lhs, q4g, group_sizes=gs, fuse_gateup_activation="silu", preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_gateup_silu_int4_packed_weights",
+            lambda: op(lhs, q4g, group_sizes=gs, fuse_gateup_activation="silu", preferred_element_type=torch.bfloat16),
+            2 * m_ * k_ * 2 * n_, (m_ * k_ + m_ * n_) * 2 + 8 * k_ * n_, "mfma", "bf16", cfg4)
+    del q4g
     # The whole expert FFN of a Mixtral layer around those two products, as a caller strings it together: tokens
     # permuted into expert order (ragged_gather), gate-up product with silu(gate) * up in the epilogue, down
     # projection, weighted top-2 combine back into token order (ragged_gather_reduce). 8192 tokens, top 2 of 8 experts.

@@ -26,6 +26,7 @@ static const Variant kVariants[] = {
     FWD(32, 128, 64, 1, 4, 4),
     GLU(256, 256, 64, 2, 4, 3),
     GLU(128, 256, 64, 2, 4, 3),
+    GLU(128, 256, 64, 1, 4, 3),
     GLU(32, 256, 64, 1, 4, 4),
     SUBK(256, 256, 64, 2, 4, 3),
     SUBK(256, 256, 64, 1, 8, 3),
