@@ -39,6 +39,7 @@ static const Variant kVariants[] = {
     SUBK(256, 256, 32, 2, 4, 4),
     SUBK(128, 256, 64, 2, 4, 3),
     SUBK(128, 256, 64, 1, 8, 3),
+    SUBK(128, 256, 64, 1, 8, 2),
     SUBK(32, 256, 64, 1, 4, 4),
     // int8 activations x int8 weights on the int8 MFMAs: int32 sums of a k-step, folded into the f32 result with
     // the scales of its k-block (one block = one scale per row and per (group, column)).
@@ -56,6 +57,7 @@ static const Variant kVariants[] = {
     SUBK_F8(256, 256, 32, 2, 4, 4),
     SUBK_F8(128, 256, 64, 2, 4, 3),
     SUBK_F8(128, 256, 64, 1, 8, 3),
+    SUBK_F8(128, 256, 64, 1, 8, 2),
     SUBK_F8(32, 256, 64, 1, 4, 4),
 };
 

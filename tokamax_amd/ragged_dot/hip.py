@@ -874,9 +874,10 @@ class HipRaggedDot(base.RaggedDot):
       # rows per group, the 128-row one from about 100, and 256 columns from a few tiles' worth of them.
       want_m = 256 if rows_per_group >= 224 else 128
       want_n = 256 if cols >= 512 else 128
-      if converted_plain or (mode == 3 and key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2)):
-        # (gate-up fusion over such weights: the 128 x 256 tile on one row of four waves, likewise two per CU, measured
-        # 6 % ahead of the 256-row tile at the Mixtral shape and 16-31 % at 128 rows per group)
+      if key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2, _lib.TKX_F8E4M3FN):
+        # (also with gate-up fusion, where the tile sits on one row of four waves, likewise two per CU: 6 % ahead of the
+        # 256-row tile at the Mixtral shape and 16-31 % at 128 rows per group; and with scales per k-block: 8-13 %
+        # ahead at 128-256 rows per group, even at the Mixtral shape)
         want_m = 128
       # ... unless so few tiles come of it that half the chip would idle: then the largest tile that gives every CU one.
       tiles = lambda bm, bn: (rows / bm + 0.88 * num_groups) * -(-cols // (bn // 2 if mode == 3 else bn))
