@@ -25,6 +25,7 @@ static const Variant kVariants[] = {
     FWD_DLHS(32, 256, 64, 1, 4, 3),
     FWD_DLHS(32, 128, 64, 1, 4, 4),
     GLU(256, 256, 32, 2, 4, 4),
+    GLU(256, 256, 64, 2, 4, 2),
     GLU(128, 256, 64, 2, 4, 3),
     GLU(64, 256, 64, 2, 2, 3),
     GLU(32, 256, 64, 1, 4, 3),
