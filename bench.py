@@ -256,7 +256,22 @@ def main():
         _gemm_kernel_prefix(0, 1, 1, cfg), "DeepSeek-V3 prefill bf16 fwd")
     extras["deepseek_v3_prefill_bf16"]["pct_mfma_peak"] = round(
         100 * extras["deepseek_v3_prefill_bf16"]["tflops"] / PEAK_TFLOPS["bf16"], 2)
-    del w
+    # The same activations and group sizes over int4 weights packed two to a byte (one scale per (group, column)): this
+    # workload is bound by the weights' way from HBM, and theirs is a quarter as long.
+    from tokamax_amd.ragged_dot import hip_ops  # pylint: disable=g-import-not-at-top
+    gen4 = torch.Generator(device=device).manual_seed(2)
+    q4 = torch.empty((w.num_groups, w.k // 2, w.n), dtype=torch.uint8, device=device)
+    for g0 in range(0, w.num_groups, 32):  # (packed in slices: the int8 form of all 256 experts would be 3.8 GB)
+      q4[g0:g0 + 32] = hip_ops.pack_int4(torch.randint(-8, 8, (min(32, w.num_groups - g0), w.k, w.n), device=device,
+                                                       dtype=torch.int8, generator=gen4))
+    q4 = tokamax_amd.QArray(q4, (torch.rand(w.num_groups, 1, w.n, device=device, generator=gen4) + 0.5) / (7 * w.k ** 0.5),
+                            None, tokamax_amd.quantization.PACKED_INT4)
+    cfg4 = op.bind(w.lhs, q4, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    nonempty = int((w.group_sizes > 0).sum())
+    measure("deepseek_v3_prefill_int4_packed_weights",
+            lambda: op(w.lhs, q4, group_sizes=gs, preferred_element_type=torch.bfloat16), w.flops,
+            w.m * w.k * 2 + nonempty * w.k * w.n // 2 + w.m * w.n * 2, "hbm", "bf16", cfg4)
+    del w, q4
 
     # decode: 6 rotating copies of the weights defeat the 256 MB last-level cache ("cold"); the same
     # copy every launch is the "warm" figure.
