@@ -324,7 +324,18 @@ def main():
       return hip_ops.quantize(dense, torch.float8_e4m3fn, (1, 128))
     t2, _, _ = _time_steps(two_passes, steps, warm, stream)
     extras["mixtral_prefill_fp8_quantised_output"]["ms_per_step_gemm_then_quantise_pass"] = round(t2 / steps, 5)
-    del w, ql, qr, qlk, qrk
+    # the same fp8 activations over int4 weights packed two to a byte along k: the nibbles go to the fp8 MFMAs as fp8
+    # bytes; the call includes the pass that sums the activation rows for the kernel's epilogue
+    gen4f = torch.Generator(device=device).manual_seed(3)
+    q4f = tokamax_amd.pack_int4(tokamax_amd.QArray(
+        torch.randint(-8, 8, tuple(w.rhs.shape), device=device, dtype=torch.int8, generator=gen4f),
+        (torch.rand(w.num_groups, 1, w.n, device=device, generator=gen4f) + 0.5) / (7 * w.k ** 0.5), None,
+        getattr(torch, "int4", torch.int8)))
+    cfg = op.bind(ql, q4f, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_prefill_fp8_activations_int4_packed_weights",
+            lambda: op(ql, q4f, group_sizes=gs, preferred_element_type=torch.bfloat16), w.flops,
+            w.m * w.k + w.nonempty_groups * w.k * w.n // 2 + w.m * w.n * 2, "mfma", "fp8", cfg)
+    del w, ql, qr, qlk, qrk, q4f
 
     # the Mixtral shape with int8 weights (one f32 scale per (group, column)): the weight stream into LDS is half of bf16's
     w = workloads.make("mixtral", device, seed=0)

@@ -282,6 +282,13 @@ int32_t tkx_dequantize_zero_point(const void* qvalue, const float* scale, const 
 int32_t tkx_unpack_int4(const void* packed, void* out, int64_t packed_rows, int64_t cols, tkx_stream_t stream);
 int32_t tkx_pack_int4(const void* values, void* packed, int64_t packed_rows, int64_t cols, tkx_stream_t stream);
 
+/* Row sums of an fp8 (e4m3fn) matrix [rows, cols] in f32: sums[r] = sum_c x[r, c]. cols % 16 == 0, x 16-byte aligned.
+ * The fp8 x packed-int4 forward (lhs TKX_F8E4M3FN, rhs TKX_I4X2, plain forward variants with block_k = 128) takes them
+ * behind the row scales, lhs_scale = f32[2, m]: it feeds weight w to the fp8 MFMAs as the e4m3 denormal (w + 8) / 512
+ * and computes (512 acc - 8 sums[row]) * lhs_scale[row] * rhs_scale[group, col]. The reference's kernel packs the
+ * sums with the activation scales the same way (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:258-300, 436-470). */
+int32_t tkx_row_sums_fp8(const void* x, float* sums, int64_t rows, int64_t cols, tkx_stream_t stream);
+
 /* Quantisation on the fly (AsQArray.as_qarray, quantization.py:65-78: qwix.quantize with the "absmax" calibration), the
  * inverse of tkx_dequantize:
  *   scale[R, C] = max |x[r, c]| over the tile (R, C) / bound   (1 where the tile is all zero)

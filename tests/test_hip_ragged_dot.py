@@ -435,6 +435,13 @@ def test_every_kernel_variant_through_c_abi(v, device):
     lhs = mk((m, k), 1.0).to(lt)
     lhs_f = _np(lhs)
     tol = 1e-5
+  elif rt == torch.uint8 and lt == torch.float8_e4m3fn:  # fp8 activations x packed int4 weights on the fp8 MFMAs
+    values = rng.integers(-8, 8, (G, k, n)).astype(np.int8)
+    rhs = torch.tensor(O.pack_int4(values), device=device)
+    lhs = mk((m, k), 1.0).to(lt)
+    lhs_scale, rhs_scale = mk((m, 1), 0.1).abs() + 0.05, mk((G, 1, n), 0.1).abs() + 1e-2
+    lhs_f, rhs_f = _np(lhs) * _np(lhs_scale), O.dequantize(values, _np(rhs_scale))
+    tol = 1e-4
   elif rt == torch.uint8:  # int4 weights, two to a byte along k
     values = rng.integers(-8, 8, (G, k, n)).astype(np.int8)
     rhs = torch.tensor(O.pack_int4(values), device=device)
@@ -838,7 +845,8 @@ def test_small_m_kernel_on_packed_int4_weights(case, scales, depth, split_k, dev
 
 def _packed_int4_tile_cases():
   return [pytest.param(v, id="{block_m}x{block_n}x{block_k}-w{waves_m}x{waves_n}-s{num_stages}".format(**v))
-          for v in _lib.variants(0) if v["rhs_dtype"] == _lib.TKX_I4X2 and v["block_m"] != 16 and v["mode"] == 0]
+          for v in _lib.variants(0) if v["rhs_dtype"] == _lib.TKX_I4X2 and v["lhs_dtype"] == _lib.TKX_BF16
+          and v["block_m"] != 16 and v["mode"] == 0]
 
 
 @pytest.mark.parametrize("v", _packed_int4_tile_cases())
@@ -882,6 +890,143 @@ def test_tiled_kernels_on_packed_int4_weights(v, device):
   want_shard[lo:hi] = want[lo:hi] + np.repeat(_np(bias)[:, 0], gs[1:4], axis=0)
   _check(shard, want_shard, 1e-5)
   assert torch.count_nonzero(shard[:lo]) == 0 and torch.count_nonzero(shard[hi:]) == 0
+
+
+def _fp8_over_packed_int4_cases():
+  return [pytest.param(v, id="{block_m}x{block_n}x{block_k}-w{waves_m}x{waves_n}-s{num_stages}".format(**v))
+          for v in _lib.variants(0) if v["rhs_dtype"] == _lib.TKX_I4X2 and v["lhs_dtype"] == _lib.TKX_F8E4M3FN]
+
+
+def test_row_sums_of_fp8_rows(device):
+  """tkx_row_sums_fp8 against sums in float64 of the decoded bytes: every finite e4m3fn value occurs, rows shorter and
+  longer than a wave's 1024-byte step, a row count that is not whole workgroups."""
+  rng = np.random.default_rng(31)
+  for rows, cols in ((7, 16), (33, 1040), (4, 4096)):
+    codes = rng.integers(0, 256, (rows, cols)).astype(np.uint8)
+    codes[(codes & 0x7f) == 0x7f] = 0x08  # (no NaN)
+    x = torch.tensor(codes, device=device).view(torch.float8_e4m3fn)
+    sums = hip_ops.row_sums_fp8(x)
+    want = O.e4m3fn_decode(codes).astype(np.float64).sum(axis=1)
+    scale = np.abs(O.e4m3fn_decode(codes).astype(np.float64)).sum(axis=1)
+    assert sums.dtype == torch.float32 and tuple(sums.shape) == (rows,)
+    assert np.all(np.abs(_np(sums) - want) <= 1e-6 * scale)
+  with pytest.raises(ValueError):
+    hip_ops.row_sums_fp8(torch.zeros(4, 16, device=device))
+  with pytest.raises(NotImplementedError, match="multiple of 16"):
+    hip_ops.row_sums_fp8(torch.zeros(4, 24, device=device).to(torch.float8_e4m3fn))
+
+
+@pytest.mark.parametrize("v", _fp8_over_packed_int4_cases())
+def test_tiled_kernels_on_fp8_activations_and_packed_int4_weights(v, device):
+  """The fp8 MFMAs on int4 weights (weight w goes in as the e4m3 denormal (w + 8) / 512, the epilogue takes
+  8 rowsum(x) off: pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:258-300): an odd number of k-steps, a ragged last column
+  tile, groups that start and end inside tiles, an empty group, rows after the last group. Against the oracle on the
+  dequantised operands, against the fp8 x fp8 kernels on the same values (int4 values are exact in fp8; another
+  summation order), bit for bit against itself, with the row sums computed by the call and handed in, split along the
+  contraction, and as one expert-parallel shard with a bias."""
+  rng = np.random.default_rng(v["block_m"] + v["num_stages"] + v["waves_m"])
+  G, k, n = 5, 5 * v["block_k"], 272
+  gs = np.array([3, 300, 0, 70, 129], np.int32)
+  m = int(gs.sum()) + 9
+  gst = torch.tensor(gs, device=device)
+  x = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32) * rng.uniform(0.1, 10, (m, 1)).astype(np.float32), device=device)
+  xs = x.abs().amax(dim=1, keepdim=True) / 448
+  xq = (x / xs).to(torch.float8_e4m3fn)
+  values = rng.integers(-8, 8, (G, k, n)).astype(np.int8)
+  values[0, :, 0], values[0, :, 1] = -8, 7  # (the two ends of the range in whole columns)
+  scale = torch.tensor((np.abs(rng.normal(0, 0.05, (G, 1, n))) + 1e-2).astype(np.float32), device=device)
+  packed = torch.tensor(O.pack_int4(values), device=device)
+  cfg = hip_ops.KernelConfig(v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"], v["num_stages"], grid_tile_width=2)
+  call = lambda cfg=cfg, lhs_scale=xs, **kw: hip_ops.ragged_dot_fwd(xq, packed, gst, config=cfg, out_dtype=torch.float32,
+                                                                    lhs_scale=lhs_scale, rhs_scale=scale, **kw)
+  out = call()
+  lhs_f = O.e4m3fn_decode(xq.view(torch.uint8).cpu().numpy()).astype(np.float64) * _np(xs)
+  want = O.ragged_dot(lhs_f, O.dequantize(values, _np(scale)), gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+  # f32 sums of up to 640 products of size up to 448 * 15 / 512 each, 512 times that, less 8 times an f32 row sum
+  _check(out, want, 5e-5)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  assert torch.equal(out, call())
+  both = torch.cat([xs.view(1, m), hip_ops.row_sums_fp8(xq).view(1, m)])
+  assert torch.equal(out, call(lhs_scale=both))
+  f8_tiles = [x_ for x_ in _lib.variants(0) if x_["rhs_dtype"] == x_["lhs_dtype"] == _lib.TKX_F8E4M3FN and x_["mode"] == 0
+              and x_["block_m"] == 128]
+  as_fp8 = torch.tensor(values, device=device).to(torch.float32).to(torch.float8_e4m3fn)
+  t = f8_tiles[0]
+  f8_cfg = hip_ops.KernelConfig(t["block_m"], t["block_n"], t["block_k"], t["waves_m"], t["waves_n"], t["num_stages"])
+  same = hip_ops.ragged_dot_fwd(xq, as_fp8, gst, config=f8_cfg, out_dtype=torch.float32, lhs_scale=xs, rhs_scale=scale)
+  assert O.rel_l2(_np(out), _np(same)) <= 2e-5
+  if v["block_m"] >= 128:
+    for split_k in (2, 3):
+      split = call(dataclasses.replace(cfg, split_k=split_k))
+      _check(split, want, 5e-5)
+      assert torch.equal(split, call(dataclasses.replace(cfg, split_k=split_k)))
+  # bf16 result without a weight scale; no lhs scale, scales per k-block, gate-up fusion and a contraction that is
+  # not whole k-steps are declined
+  plain = hip_ops.ragged_dot_fwd(xq, packed, gst, config=cfg, out_dtype=torch.bfloat16, lhs_scale=xs)
+  _check(plain, O.ragged_dot(lhs_f, values.astype(np.float64), gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 4e-3)
+  with pytest.raises(NotImplementedError, match="lhs scale"):
+    hip_ops.ragged_dot_fwd(xq, packed, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale)
+  with pytest.raises(NotImplementedError):
+    hip_ops.ragged_dot_fwd(xq, packed, gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs,
+                           rhs_scale=scale.expand(G, 5, n).contiguous())
+  with pytest.raises(NotImplementedError):
+    hip_ops.ragged_dot_fwd(xq, packed[:, :, :256].contiguous(), gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs,
+                           gateup=True, activation="silu")
+  with pytest.raises(NotImplementedError, match="block_k"):
+    hip_ops.ragged_dot_fwd(xq[:, :k - 32].contiguous(), packed[:, :k // 2 - 16].contiguous(), gst, config=cfg,
+                           out_dtype=torch.float32, lhs_scale=xs)
+  offset = torch.tensor([1], dtype=torch.int32, device=device)
+  bias = torch.tensor(rng.normal(0, 1, (3, 1, n)).astype(np.float32), device=device)
+  shard = hip_ops.ragged_dot_fwd(xq, packed[1:4].contiguous(), gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs,
+                                 rhs_scale=scale[1:4].contiguous(), rhs_bias=bias, group_offset=offset)
+  lo, hi = int(gs[:1].sum()), int(gs[:4].sum())
+  want_shard = np.zeros((m, n))
+  want_shard[lo:hi] = want[lo:hi] + np.repeat(_np(bias)[:, 0], gs[1:4], axis=0)
+  _check(shard, want_shard, 5e-5)
+  assert torch.count_nonzero(shard[:lo]) == 0 and torch.count_nonzero(shard[hi:]) == 0
+
+
+def test_public_op_on_fp8_activations_and_packed_int4_weights(device):
+  """An lhs quantised to fp8 per row (a QArray, or an AsQArray the op quantises) over packed int4 weights: the op
+  keeps the weights packed and the heuristics name a kernel of the fp8 x int4 kind; same result as on the unpacked
+  weights (which are widened for bf16 kernels), to the rounding of those; the oracle on the dequantised operands.
+  Scales per k-block fall back to the unpacked path."""
+  rng = np.random.default_rng(12)
+  G, k, n, rows = 4, 512, 256, 160
+  m = G * rows
+  q = torch.tensor(rng.integers(-8, 8, (G, k, n)).astype(np.int8), device=device)
+  scale = torch.tensor((rng.uniform(0.5, 1.5, (G, 1, n)) / 7 * 0.1).astype(np.float32), device=device)
+  int4 = getattr(torch, "int4", torch.int8)
+  plain = tokamax_amd.QArray(q, scale, None, int4)
+  packed = tokamax_amd.pack_int4(plain)
+  x = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device)
+  xs = x.abs().amax(dim=1, keepdim=True) / 448
+  lhs = tokamax_amd.QArray((x / xs).to(torch.float8_e4m3fn), xs)
+  gs = torch.full((G,), rows, dtype=torch.int32, device=device)
+  op = tokamax_amd.HipRaggedDot()
+  key = _lib_key(op, lhs, packed, gs)
+  assert key == (0, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
+  cfg = op._get_heuristics_config(op.bind(lhs, packed, group_sizes=gs))
+  assert cfg.block_k == 128 and cfg.block_m >= 32
+  out = op(lhs, packed, group_sizes=gs, preferred_element_type=torch.float32)
+  lhs_f = O.e4m3fn_decode(lhs.qvalue.view(torch.uint8).cpu().numpy()).astype(np.float64) * _np(xs)
+  want = O.ragged_dot(lhs_f, O.dequantize(q.cpu().numpy(), _np(scale)), np.full(G, rows, np.int32), O.DEFAULT,
+                      acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, 5e-5)
+  ref = op(lhs, plain, group_sizes=gs, preferred_element_type=torch.float32)
+  assert O.rel_l2(_np(out), _np(ref)) <= 1e-2  # (the unpacked path rounds scaled operands to bf16)
+  # an AsQArray lhs is quantised by the op, then takes the same kernels
+  as_q = tokamax_amd.AsQArray(x.to(torch.bfloat16), torch.float8_e4m3fn, channelwise_axes=(0,))
+  assert _lib_key(op, as_q, packed, gs) == key
+  quantised = as_q.as_qarray()
+  out_q = op(as_q, packed, group_sizes=gs, preferred_element_type=torch.float32)
+  lhs_q = O.e4m3fn_decode(quantised.qvalue.view(torch.uint8).cpu().numpy()).astype(np.float64) * _np(quantised.scale)
+  _check(out_q, O.ragged_dot(lhs_q, O.dequantize(q.cpu().numpy(), _np(scale)), np.full(G, rows, np.int32), O.DEFAULT,
+                             acc_dtype=np.float64, out_dtype="f64"), 5e-5)
+  # scales per k-block: no kernel of this kind; the weights are unpacked and the widened path runs
+  blocks = tokamax_amd.pack_int4(tokamax_amd.QArray(q, scale.expand(G, 4, n).contiguous(), None, int4))
+  assert _lib_key(op, lhs, blocks, gs)[2] != _lib.TKX_I4X2
+  _check(op(lhs, blocks, group_sizes=gs, preferred_element_type=torch.float32), want, 1e-2)
 
 
 def _lib_key(op, lhs, rhs, gs):
@@ -2117,11 +2262,11 @@ def test_timing_tool_collects_every_kind_of_problem(tmp_path, device):
   config among the timed ones."""
   from tokamax_amd.data.autotuning import tile_cost
   path = str(tmp_path / "timings.json")
-  kinds = ["", ",dlhs", ",drhs", ",int8", ",int4", ",fp8", ",int8x8", ",glu", ",int8k", ",f32"]
+  kinds = ["", ",dlhs", ",drhs", ",int8", ",int4", ",fp8", ",fp8i4", ",int8x8", ",glu", ",int8k", ",f32"]
   tile_cost.collect(["768,256,512,4" + k for k in kinds], 2, path=path)
   entries = tile_cost.load(path)
   assert len(entries) == len(kinds) and all(e["timings"] and e["timings"][0][7] > 0 for e in entries)
-  assert {e.get("rhs", "bf16") for e in entries} == {"bf16", "int8", "int4", "fp8", "int8x8", "glu", "int8k", "f32"}
-  assert sorted(e["mode"] for e in entries) == [0] * 8 + [1, 2]
+  assert {e.get("rhs", "bf16") for e in entries} == {"bf16", "int8", "int4", "fp8", "fp8i4", "int8x8", "glu", "int8k", "f32"}
+  assert sorted(e["mode"] for e in entries) == [0] * 9 + [1, 2]
   for e in entries:
     assert 1.0 <= tile_cost.heuristics_gap(e) < 3.0, e["shape"]

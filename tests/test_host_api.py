@@ -662,6 +662,25 @@ def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   assert op._problem(op.bind(ShapeDtype((4096, 96), bf16), odd, group_sizes=gs))[1][2] == _lib.TKX_I8
   space = op._get_autotuning_configs(op.bind(lhs, packed, group_sizes=gs))
   assert {x.block_m for x in space} >= {16, 32, 128, 256}
+  # fp8 activations with one scale per row (or per run of rows): the packed weights stay packed for the kernels that
+  # feed the nibbles to the fp8 MFMAs (one row of waves: each nibble becomes an fp8 byte once per workgroup); with scale
+  # blocks along k or gate-up fusion they are unpacked, and fp8 activations over int8 storage are widened to bf16
+  f8 = torch.float8_e4m3fn
+  x8 = tokamax_amd.QArray(ShapeDtype((4096, 1024), f8), ShapeDtype((4096, 1), f32))
+  route8 = lambda x, rhs, **kw: op._problem(op.bind(x, rhs, group_sizes=gs, **kw))[1]
+  assert route8(x8, packed) == (0, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
+  assert route8(x8, packed, rhs_bias=ShapeDtype((8, 1, 256), f32)) == (0, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
+  shared = tokamax_amd.QArray(ShapeDtype((4096, 1024), f8), ShapeDtype((16, 1), f32))
+  assert route8(shared, packed) == (0, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
+  wide = tokamax_amd.QArray(ShapeDtype((8, 512, 4096), u8), ShapeDtype((8, 1, 4096), f32), None, int4)
+  c = op._get_heuristics_config(op.bind(x8, wide, group_sizes=gs))
+  assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n) == (128, 256, 128, 1, 8)
+  assert {x.block_k for x in op._get_autotuning_configs(op.bind(x8, wide, group_sizes=gs))} == {128}
+  assert route8(x8, blocks) == (4, _lib.TKX_BF16, _lib.TKX_I8)
+  assert route8(x8, packed, fuse_gateup_activation="silu") == (3, _lib.TKX_BF16, _lib.TKX_I8)
+  assert route8(x8, packed.unpacked()) == (0, _lib.TKX_BF16, _lib.TKX_I8)
+  x8_blocks = tokamax_amd.QArray(ShapeDtype((4096, 1024), f8), ShapeDtype((4096, 8), f32))
+  assert route8(x8_blocks, packed)[1:] == (_lib.TKX_BF16, _lib.TKX_I8)
   # the key of an autotuning cache entry names the 4-bit type and comes back as the same abstract QArray
   from tokamax_amd import serialization
   spec = serialization.to_jsonable(packed)
@@ -709,7 +728,7 @@ def test_tile_cost_model_picks_near_the_fastest_measured_variant():
   # the config the heuristics hand out for those problems (model, rules for the streaming kernel, split decision), and
   # for quantised operands and drhs, where rules on rows per group and on the fill of the chip choose the tile
   label = lambda e: "drhs" if e["mode"] == 2 else e.get("rhs", "bf16")
-  for kind, count, most in (("bf16", 122, 0.06), ("int8", 26, 0.08), ("int4", 26, 0.06), ("fp8", 26, 0.03),
+  for kind, count, most in (("bf16", 122, 0.06), ("int8", 26, 0.08), ("int4", 26, 0.06), ("fp8", 26, 0.03), ("fp8i4", 43, 0.04),
                             ("int8x8", 12, 0.03), ("drhs", 26, 0.03), ("glu", 26, 0.06), ("int8k", 26, 0.04), ("f32", 12, 0.01)):
     some = [e for e in tile_cost.load() if label(e) == kind]
     mean, worst = tile_cost.summary([tile_cost.heuristics_gap(e) for e in some])

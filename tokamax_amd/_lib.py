@@ -45,6 +45,7 @@ EXPORTED_SYMBOLS = (
     "tkx_ragged_dot_decode_clear_counters",
     "tkx_unpack_int4",
     "tkx_pack_int4",
+    "tkx_row_sums_fp8",
     "tkx_ragged_dot_fwd_fp8_out",
 )
 
@@ -90,6 +91,8 @@ def _declare(lib):
   for fn in (lib.tkx_unpack_int4, lib.tkx_pack_int4):
     fn.restype = i32
     fn.argtypes = [vp, vp, i64, i64, vp]
+  lib.tkx_row_sums_fp8.restype = i32
+  lib.tkx_row_sums_fp8.argtypes = [vp, vp, i64, i64, vp]
   lib.tkx_last_error.restype = ctypes.c_char_p
   lib.tkx_last_error.argtypes = []
   lib.tkx_ragged_dot_tid_size.restype = i64

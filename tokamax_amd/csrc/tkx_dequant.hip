@@ -124,7 +124,33 @@ __global__ __launch_bounds__(kDqThreads) void pack_int4_kernel(const signed char
   }
 }
 
+// Row sums of an fp8 (e4m3fn) matrix [rows, n], n % 16 == 0: one wave per row, 16 bytes per lane and step, summed in
+// f32. The sums of activation rows, which the fp8 x packed-int4 kernels take their +8 weight bias off with.
+__global__ __launch_bounds__(kDqThreads) void row_sums_fp8_kernel(const unsigned char* __restrict__ x, float* __restrict__ sums,
+                                                                 int64_t rows, int32_t n) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * (kDqThreads / 64) + (threadIdx.x >> 6);
+  if (row >= rows) return;  // (whole waves leave together)
+  float s = 0.f;
+  for (int c0 = lane * 16; c0 < n; c0 += 64 * 16) {
+    const i32x4 w = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(x + row * n + c0));
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+      s += (widen_byte<kEF8, 0>(w[d]) + widen_byte<kEF8, 1>(w[d])) + (widen_byte<kEF8, 2>(w[d]) + widen_byte<kEF8, 3>(w[d]));
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+  if (lane == 0) sums[row] = s;
+}
+
 }  // namespace
+
+int32_t launch_row_sums_fp8(const void* x, float* sums, int64_t rows, int64_t n, hipStream_t stream) {
+  const int64_t grid = (rows + kDqThreads / 64 - 1) / (kDqThreads / 64);
+  row_sums_fp8_kernel<<<dim3((unsigned)grid), dim3(kDqThreads), 0, stream>>>(static_cast<const unsigned char*>(x), sums, rows, (int32_t)n);
+  TKX_HIP_CHECK(hipGetLastError());
+  return TKX_OK;
+}
 
 int32_t launch_int4_repack(const void* in, void* out, int64_t packed_rows, int64_t n, bool unpack, hipStream_t stream) {
   const int64_t total = packed_rows * (n / 16);

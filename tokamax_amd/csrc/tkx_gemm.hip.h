@@ -245,6 +245,20 @@ __device__ __forceinline__ typename Mma<EC>::Frag load_frag(const unsigned char*
   }
 }
 
+// 32 packed int4 values of one column (16 bytes, byte r = contraction entries 2 r and 2 r + 1, low nibble first) as the
+// 32 fp8 bytes 0000uuuu, u = nibble ^ 8, in contraction order: the e4m3 denormal (w + 8) / 512 for the weight w.
+__device__ __forceinline__ i32x8 i4x32_to_biased_f8x32(i32x4 w) {
+  i32x8 out;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const unsigned x = (unsigned)w[d] ^ 0x88888888u;
+    const unsigned lo = x & 0x0F0F0F0Fu, hi = (x >> 4) & 0x0F0F0F0Fu;
+    out[2 * d] = (int)__builtin_amdgcn_perm(hi, lo, 0x05010400u);
+    out[2 * d + 1] = (int)__builtin_amdgcn_perm(hi, lo, 0x07030602u);
+  }
+  return out;
+}
+
 // Eight packed int4 values (see i4x8_to_bf16x8_times16) times one scale, rounded to bf16; `scale16` is the column's
 // scale for the current k-block divided by 16.
 __device__ __forceinline__ i32x4 i4x8_to_bf16x8_scaled(int w, float scale16) {
@@ -567,6 +581,13 @@ struct GemmKernel {
   // column gives it 16 consecutive contraction entries, the B fragments of two atoms, and the lhs fragments are read
   // in the matching order (load_frag's PAIRED), so nothing is permuted.
   static constexpr bool I4 = EB == kEI4;
+  // bf16 activations: the nibbles are converted to bf16 (times 16) on their way into the MFMAs.
+  static constexpr bool I4P = I4 && EA == kEBF16;
+  // fp8 activations (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:258-300): a nibble w becomes the fp8 byte
+  // 0000uuuu with u = w + 8 = nibble ^ 8, which e4m3 reads as the denormal u / 512, exactly; the fp8 MFMAs then
+  // give sum(x u) / 512 and the epilogue takes 8 sum(x) off again: sum(x w) = 512 acc - 8 rowsum(x). The row sums
+  // of x lie behind its m_ext row scales.
+  static constexpr bool I4F = I4 && EA == kEF8;
   static constexpr int EBS = I4 ? (int)kEI8 : EB;  // element kind of a B stage in LDS
   static constexpr int KA = Mma<EC>::KA;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
@@ -583,11 +604,11 @@ struct GemmKernel {
   // next to 128 accumulators. The lhs fragments are then kept once: row block i's is re-read for the next atom right
   // after the atom's last MFMA on it (TM * TN - TN MFMAs of 64 cycles before its next use); the two rhs fragments stay
   // double-buffered.
-  static constexpr bool LEAN = EA == kEF8 && EB == kEF8 && !SUBK && !SPLIT && TM * TN >= 8;
+  static constexpr bool LEAN = EA == kEF8 && (EB == kEF8 || EB == kEI4) && !SUBK && !SPLIT && TM * TN >= 8;
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
   static_assert(!SPLIT || (MODE == kFwd && EA == EB && BK % 2 == 0), "split pipeline: plain forward, operands of one type");
-  static_assert(!I4 || ((MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK) && EA == kEBF16 && !SPLIT),
-                "packed int4 weights: forward with bf16 activations");
+  static_assert(!I4 || (((I4P && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK)) || (I4F && MODE == kFwd)) && !SPLIT),
+                "packed int4 weights: forward with bf16 activations, plain forward with fp8 activations");
   static constexpr int BKB = I4 ? BKC / 2 : BKC;  // rows of a B stage
   typedef TileStage<LA, EA, BM, BK, THREADS> StageA;
   typedef TileStage<LB, EBS, BN, BKB, THREADS> StageB;
@@ -760,6 +781,16 @@ struct GemmKernel {
     const int nv_sel = rmask == (1u << nv_count) - 1u ? nv_count : TM;
     // B fragment j of k-atom kk of a stage. kFwdSubK: the int8 values of the lane's column (lane % 32 of the
     // block) are multiplied by that column's scale for the stage's k-block, which lies behind the tiles.
+    // (fp8 activations over packed int4 weights) the 16 bytes of the lane's column that hold the 32 contraction
+    // entries of its half of k-atom kk: packed rows 32 kk + 16 (lane / 32) .. + 15.
+    [[maybe_unused]] auto load_b_raw = [&](const unsigned char* stage, int j, int kk) -> i32x4 {
+      const int blk = lane >> 4, s_ = lane & 15;
+      const int col = wn * WTN + j * 32 + 16 * (blk & 1) + 8 * (s_ & 1);
+      const int krow = kk * (KA / 2) + 16 * (blk >> 1) + (s_ >> 1);
+      const i32x2 lo = lds_read_tr8(stage + StageA::BYTES + mc_offset<StageB::ROW_BYTES, EBS>(krow, col));
+      const i32x2 hi = lds_read_tr8(stage + StageA::BYTES + mc_offset<StageB::ROW_BYTES, EBS>(krow + 8, col));
+      return i32x4{lo[0], lo[1], hi[0], hi[1]};
+    };
     auto load_b_frag = [&](const unsigned char* stage, int j, int kk) -> Frag {
       if constexpr (SUBK && !SUBP) {
         const int blk = lane >> 4, s_ = lane & 15;
@@ -770,6 +801,8 @@ struct GemmKernel {
                                                             4 * (wn * WTN + j * 32 + (lane & 31)));
         if constexpr (EB == kEI8) return i8x8_to_bf16x8_scaled(v, scale);
         else return f8x8_to_bf16x8_scaled(v, scale);
+      } else if constexpr (I4F) {
+        return i4x32_to_biased_f8x32(load_b_raw(stage, j, kk));
       } else {
         return load_frag<LB, EBS, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + j * 32, kk, lane);
       }
@@ -1019,7 +1052,8 @@ struct GemmKernel {
         // next; they are kept as read (`raw`) and converted half by half. The list of an even atom is then A0, the
         // byte reads, A1, ..., and last the conversions of the first halves; that of an odd atom A0, the conversions
         // of the second halves, A1, ...
-        [[maybe_unused]] i32x2 raw[I4 ? TN : 1];
+        [[maybe_unused]] i32x2 raw[I4P ? TN : 1];
+        [[maybe_unused]] i32x4 rawf[I4F ? TN : 1];  // (fp8 activations) a fragment's bytes as read
         // (kFwdSubK: times the scale of the lane's column for the stage's k-block, like load_b_frag)
         [[maybe_unused]] auto convert_i4 = [&](int w, const unsigned char* stage, int j) -> i32x4 {
           if constexpr (SUBK) {
@@ -1030,14 +1064,16 @@ struct GemmKernel {
             return i4x8_to_bf16x8_times16(w);
           }
         };
-        constexpr int NRD = I4 ? TM + 2 * TN : TM + TN;  // entries of an atom's list
+        constexpr int NRD = I4 ? TM + 2 * TN : TM + TN;  // (fp8 activations: A0, the byte reads, A1, ..., the conversions)  // entries of an atom's list
         auto read_frag = [&](Frag* a, Frag* b, int r, const unsigned char* stage, int kk) {
           if (r >= NRD) return;
           const int f = r == 0 ? 0 : r <= TN ? TM + r - 1 : r < TM + TN ? r - TN : r;
           if (f < TM) {
-            if (f < NV) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES, I4>(stage, wm * 32, kk, lane, f * WM * 32);
+            if (f < NV) a[f] = load_frag<LA, EA, EC, StageA::ROW_BYTES, I4P>(stage, wm * 32, kk, lane, f * WM * 32);
           } else if (f < TM + TN) {
-            if constexpr (I4) {
+            if constexpr (I4F) {
+              if (NV > 0) rawf[f - TM] = load_b_raw(stage, f - TM, kk);
+            } else if constexpr (I4P) {
               const int j = f - TM;
               if (NV > 0) {
                 if (kk & 1) {
@@ -1052,7 +1088,9 @@ struct GemmKernel {
             } else {
               if (NV > 0) b[f - TM] = load_b_frag(stage, f - TM, kk);
             }
-          } else if constexpr (I4) {
+          } else if constexpr (I4F) {
+            if (NV > 0) b[f - TM - TN] = i4x32_to_biased_f8x32(rawf[f - TM - TN]);
+          } else if constexpr (I4P) {
             if (NV > 0 && !(kk & 1)) b[f - TM - TN] = convert_i4(raw[f - TM - TN][0], stage, f - TM - TN);
           }
         };
@@ -1085,6 +1123,11 @@ struct GemmKernel {
                 // rhs fragment t after MFMA t; the lhs fragment of a row block after the block's last MFMA
                 if (t < TN) read_frag(na, nb, t + 1, rd_stage, rd_kk);
                 if (j == TN - 1) read_frag(na, nb, i == 0 ? 0 : TN + i, rd_stage, rd_kk);
+                if constexpr (I4F) {
+                  // the bytes of rhs fragment c become fp8 two MFMAs or more after their read was issued
+                  constexpr int LAG = TN == 1 ? 2 : TN;
+                  if (t >= LAG && t < LAG + TN) read_frag(na, nb, TM + TN + t - LAG, rd_stage, rd_kk);
+                }
               } else {
 #pragma unroll
                 for (int r = 0; r < RPM; ++r) read_frag(na, nb, t * RPM + r, rd_stage, rd_kk);
@@ -1178,7 +1221,7 @@ struct GemmKernel {
         for (; kt < nfull; ++kt) k_step(std::false_type{}, std::false_type{}, kt);
       };
       dispatch_upto<0, TM>(nv_sel, k_loop);
-      if constexpr (I4 && !SUBK) {
+      if constexpr (I4P && !SUBK) {
         // (the weights went into the MFMAs times 16)
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -1321,6 +1364,13 @@ struct GemmKernel {
         for (int i = 0; i < TM; ++i) {
           const int row = min(row0 + row_block(i) * 32 + (lane & 31), p.m_ext - 1);
           const float rs = p.a_scale[row];
+          if constexpr (I4F) {
+            const float off = 8.f * p.a_scale[p.m_ext + row];
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) acc[i][j][e] = 512.f * acc[i][j][e] - off;
+          }
 #pragma unroll
           for (int j = 0; j < TN; ++j)
 #pragma unroll

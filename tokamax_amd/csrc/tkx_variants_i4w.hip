@@ -1,4 +1,4 @@
-// bf16 activations x packed int4 weights (TKX_I4X2: two values to a byte along the contraction) forward variants.
+// bf16 (and, last in the list, fp8) activations x packed int4 weights (TKX_I4X2: two values to a byte along the contraction) forward variants.
 // A weight stage is a byte tile half as deep as the k-step; the nibbles are taken apart and converted to bf16 on the
 // way from LDS to the MFMA; per-(group, column) scales in the epilogue, or per-(group, k-block, column) scales
 // multiplied in during that conversion (kFwdSubK, 256-column tiles). Whole k-steps only (k % block_k == 0).
@@ -11,6 +11,9 @@ namespace tkx {
 // Gate-up fusion over weights [gate | up] with one scale per (group, column).
 #define GLU(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdGlu, kEBF16, kEI4, BM, BN, BK, WM, WN, NS)
 #define SUBK(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdSubK, kEBF16, kEI4, BM, BN, BK, WM, WN, NS)
+// fp8 activations: the nibbles go to the fp8 MFMAs as the e4m3 denormals (w + 8) / 512 and the epilogue takes the bias
+// off with the activations' row sums (lhs_scale holds [row scales | row sums]).
+#define F8FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEF8, kEI4, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
     FWD(256, 256, 64, 2, 4, 2),
@@ -33,6 +36,12 @@ static const Variant kVariants[] = {
     SUBK(128, 256, 64, 2, 4, 3),
     SUBK(128, 256, 64, 1, 8, 3),
     SUBK(32, 256, 64, 1, 4, 4),
+    F8FWD(128, 256, 128, 2, 4, 3),
+    F8FWD(128, 256, 128, 1, 8, 3),
+    F8FWD(128, 256, 128, 1, 8, 4),
+    F8FWD(128, 128, 128, 2, 2, 4),
+    F8FWD(64, 128, 128, 2, 2, 4),
+    F8FWD(32, 128, 128, 1, 4, 4),
 };
 
 const Variant* variants_i4w(int* count) {

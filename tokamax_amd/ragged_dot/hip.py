@@ -342,6 +342,10 @@ def _widening_plan(lhs, rhs, allow_native: bool = True) -> tuple[bool, bool, boo
     widen_lhs = True
   if widen_lhs and rhs_q and eight_bit_float(rhs):
     widen_rhs = True
+  if lhs_q and eight_bit_float(lhs) and not widen_lhs and not eight_bit_float(rhs):
+    # fp8 activations meet fp8 weights on the fp8 MFMAs (and packed int4 ones in kernels of their own, settled before
+    # this plan); under any other partner (int8 or 16-bit weights) they are widened.
+    widen_lhs = True
   if (widen_lhs and not rhs_q and eight_bit_float(rhs)) or (widen_rhs and not lhs_q and eight_bit_float(lhs)):
     raise NotImplementedError("A raw fp8 operand cannot meet a widened (bf16) one.")
   return widen_lhs, widen_rhs, False
@@ -433,6 +437,10 @@ def _route(lhs, rhs, *, dims, precision, rhs_scale, fuse_gateup_activation, pref
     if preferred_element_type is None:
       preferred_element_type = torch.promote_types(lhs.dtype, rhs.dtype)
     k_blocks = rhs.scale.shape[1] > 1
+    if isinstance(lhs, QArray):
+      # fp8 activations with one scale per row: the kernels that feed the nibbles to the fp8 MFMAs.
+      return _Route(0, _per_row_lhs_scale(lhs), rhs, torch.float8_e4m3fn, torch.uint8, False, False, False, False,
+                    preferred_element_type)
     return _Route(3 if gateup else 4 if k_blocks else 0, lhs, rhs, torch.bfloat16, torch.uint8, False, False, k_blocks,
                   False, preferred_element_type)
   lhs_dt, rhs_dt = _dtype_of(lhs), _dtype_of(rhs)
@@ -467,6 +475,7 @@ def _route(lhs, rhs, *, dims, precision, rhs_scale, fuse_gateup_activation, pref
 
 
 _PACKED_INT4_TILE_STEP = 64  # k-step of the tiled kernels that read packed int4 weights
+_PACKED_INT4_FP8_TILE_STEP = 128  # ... under fp8 activations
 
 
 def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True, gateup: bool = False):
@@ -475,7 +484,10 @@ def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True, gateup: bool = Fa
   * the tiled kernels: k a multiple of their k-step (64); one scale per (group, column), or, without gate-up fusion, per
     (group, k-block, column) with blocks of a power of two >= 64 rows, or
   * the streaming small-m kernel: no bias and no gate-up fusion (`plain`), at most 8 rows per group on average,
-    k % 1024 == 0, one scale per (group, column) or per (group, k-block, column) with blocks of a power of two >= 32 rows.
+    k % 1024 == 0, one scale per (group, column) or per (group, k-block, column) with blocks of a power of two >= 32 rows;
+  or under an lhs quantised to fp8 (e4m3fn) with one scale per row (or shared by runs of rows), no gate-up fusion, one
+  scale per (group, column) and k % 128 == 0: the tiled kernels that feed the nibbles to the fp8 MFMAs
+  (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:258-300).
   Every other call gets the values unpacked to int8 storage first (then the int8 paths).
   Works on arrays and on shapes, so the forward pass and the choice of a config settle it alike."""
   if not (isinstance(rhs, QArray) and rhs.packed):
@@ -491,7 +503,12 @@ def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True, gateup: bool = Fa
              and lhs.shape[0] * k * 2 < 2**32)
   tiles = (reads_packed and k % _PACKED_INT4_TILE_STEP == 0
            and (blocks == 1 or (scale_ok and not gateup and rows % _PACKED_INT4_TILE_STEP == 0)))
-  return rhs if streams or tiles else rhs.unpacked()
+  lhs_rows = _per_row_lhs_scale(lhs)
+  fp8_tiles = (dims == base.DEFAULT_RAGGED_DOT_DIM_NUMS and isinstance(lhs_rows, QArray) and lhs_rows.zero_point is None
+               and lhs_rows.qtype == torch.float8_e4m3fn and len(lhs_rows.qvalue.shape) == 2
+               and tuple(lhs_rows.scale.shape) == (lhs_rows.qvalue.shape[0], 1) and rhs.zero_point is None and n % 16 == 0
+               and blocks == 1 and not gateup and k % _PACKED_INT4_FP8_TILE_STEP == 0)
+  return rhs if streams or tiles or fp8_tiles else rhs.unpacked()
 
 
 def _abstract_operand(x):
@@ -919,7 +936,9 @@ class HipRaggedDot(base.RaggedDot):
       # convert it twice (measured 1.01-1.44 x, typically 1.1-1.2 x, over three shapes, both scale forms, both tile
       # heights; 16-bit operands lose 5 % with it: their LDS reads grow by half and nothing is saved).
       converted = key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2, _lib.TKX_F8E4M3FN)
-      two_wave_rows = wm - 1 if converted else 0
+      # (fp8 activations over packed int4 weights turn nibbles into fp8 bytes the same way: 2070-2230 TFLOP/s on one
+      # row of waves against 1660-2050 on two at the Mixtral shape)
+      two_wave_rows = wm - 1 if converted or (key[1] == _lib.TKX_F8E4M3FN and key[2] == _lib.TKX_I4X2) else 0
       # ... and among those, the variant whose LDS lets two of its workgroups share a CU (the library gives such a
       # kernel 128 registers: 8 waves on one row, at most 64 accumulators per lane)
       stage_bytes = (bm * 2 + bn * (0.5 if key[2] == _lib.TKX_I4X2 else 1.0)) * bk + (bn * 4 if mode == 4 else 0)
