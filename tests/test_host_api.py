@@ -673,7 +673,10 @@ def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   shared = tokamax_amd.QArray(ShapeDtype((4096, 1024), f8), ShapeDtype((16, 1), f32))
   assert route8(shared, packed) == (0, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
   wide = tokamax_amd.QArray(ShapeDtype((8, 512, 4096), u8), ShapeDtype((8, 1, 4096), f32), None, int4)
-  c = op._get_heuristics_config(op.bind(x8, wide, group_sizes=gs))
+  c = op._get_heuristics_config(op.bind(x8, wide, group_sizes=gs))   # 512 rows per group: the 256-row tile (two rows of waves)
+  assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages) == (256, 256, 128, 2, 4, 3)
+  fewer = tokamax_amd.QArray(ShapeDtype((1024, 1024), f8), ShapeDtype((1024, 1), f32))
+  c = op._get_heuristics_config(op.bind(fewer, wide, group_sizes=gs))  # 128 rows per group: 128 rows on one row of waves
   assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n) == (128, 256, 128, 1, 8)
   assert {x.block_k for x in op._get_autotuning_configs(op.bind(x8, wide, group_sizes=gs))} == {128}
   assert route8(x8, blocks) == (4, _lib.TKX_BF16, _lib.TKX_I8)

@@ -605,6 +605,12 @@ struct GemmKernel {
   // after the atom's last MFMA on it (TM * TN - TN MFMAs of 64 cycles before its next use); the two rhs fragments stay
   // double-buffered.
   static constexpr bool LEAN = EA == kEF8 && (EB == kEF8 || EB == kEI4) && !SUBK && !SPLIT && TM * TN >= 8;
+  // fp8 activations over packed int4 weights on a lean tile with two or more column blocks per wave: the MFMAs of an
+  // atom run column block by column block, so that the bytes read ahead (`rawf`) are the only second copy of the
+  // rhs fragments: fragment 0 of the next atom is converted once the MFMAs on the current one are issued, fragment
+  // c >= 1 at the start of its own atom, while the MFMAs on fragment 0 run. 16 registers fewer than two sets of
+  // converted fragments, which is what lets the 256 x 256 x 128 tile live in 256.
+  static constexpr bool JOUT = LEAN && I4F && TN >= 2;
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
   static_assert(!SPLIT || (MODE == kFwd && EA == EB && BK % 2 == 0), "split pipeline: plain forward, operands of one type");
   static_assert(!I4 || (((I4P && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK)) || (I4F && MODE == kFwd)) && !SPLIT),
@@ -1103,6 +1109,27 @@ struct GemmKernel {
                         const unsigned char* rd_stage, int rd_kk, const StepPtrs& sp, auto first_tag) {
           constexpr bool reads = decltype(reads_tag)::value, loads = decltype(loads_tag)::value;
           constexpr bool first_of_step = decltype(first_tag)::value;  // (SUBP) the partial accumulators start at zero
+          if constexpr (JOUT) {
+#pragma unroll
+            for (int t = 0; t < NM; ++t) {
+              const int j = t / TM, i = t % TM;
+              if (i < NV) acc[i][j] = mma_atom<EC>(fb[0][j], fa[0][i], acc[i][j]);
+              if (t < TN - 1 && NV > 0) fb[0][t + 1] = i4x32_to_biased_f8x32(rawf[t + 1]);
+              if (reads) {
+                // (the buffer of fragment 0's bytes is free since the previous atom, that of fragment t since the line above)
+                if (t < TN && NV > 0) rawf[t] = load_b_raw(rd_stage, t, rd_kk);
+                if (t == TM && NV > 0) fb[0][0] = i4x32_to_biased_f8x32(rawf[0]);
+                if (j == TN - 1 && i < NV)
+                  fa[0][i] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(rd_stage, wm * 32, rd_kk, lane, i * WM * 32);
+              }
+              if (loads) {
+#pragma unroll
+                for (int q = 0; q < LPM; ++q) issue_slot(t * LPM + q, sp);
+              }
+              __builtin_amdgcn_sched_barrier(0);
+            }
+            return;
+          }
 #pragma unroll
           for (int t = 0; t < NM; ++t) {
             const int i = t / TN, j = t % TN;
@@ -1141,8 +1168,18 @@ struct GemmKernel {
           }
         };
 
+        if constexpr (JOUT) {
 #pragma unroll
-        for (int f = 0; f < NRD; ++f) read_frag(fa[0], fb[0], f, smem, 0);
+          for (int i = 0; i < TM; ++i)
+            if (i < NV) fa[0][i] = load_frag<LA, EA, EC, StageA::ROW_BYTES>(smem, wm * 32, 0, lane, i * WM * 32);
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            if (NV > 0) rawf[j] = load_b_raw(smem, j, 0);
+          if (NV > 0) fb[0][0] = i4x32_to_biased_f8x32(rawf[0]);
+        } else {
+#pragma unroll
+          for (int f = 0; f < NRD; ++f) read_frag(fa[0], fb[0], f, smem, 0);
+        }
         int cur_stage = 0;
         const StepPtrs none = {};
         // One k-step. `refill_tag`: the stage it releases is refilled with k-step kt + NS;

@@ -12,7 +12,8 @@ namespace tkx {
 #define GLU(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdGlu, kEBF16, kEI4, BM, BN, BK, WM, WN, NS)
 #define SUBK(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdSubK, kEBF16, kEI4, BM, BN, BK, WM, WN, NS)
 // fp8 activations: the nibbles go to the fp8 MFMAs as the e4m3 denormals (w + 8) / 512 and the epilogue takes the bias
-// off with the activations' row sums (lhs_scale holds [row scales | row sums]).
+// off with the activations' row sums (lhs_scale holds [row scales | row sums]). The 256 x 256 x 128 tile runs an atom's
+// MFMAs column block by column block and keeps one set of converted rhs fragments (GemmKernel::JOUT).
 #define F8FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEF8, kEI4, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
@@ -36,6 +37,7 @@ static const Variant kVariants[] = {
     SUBK(128, 256, 64, 2, 4, 3),
     SUBK(128, 256, 64, 1, 8, 3),
     SUBK(32, 256, 64, 1, 4, 4),
+    F8FWD(256, 256, 128, 2, 4, 3),
     F8FWD(128, 256, 128, 2, 4, 3),
     F8FWD(128, 256, 128, 1, 8, 3),
     F8FWD(128, 256, 128, 1, 8, 4),

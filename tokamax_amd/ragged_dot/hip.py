@@ -936,8 +936,9 @@ class HipRaggedDot(base.RaggedDot):
       # convert it twice (measured 1.01-1.44 x, typically 1.1-1.2 x, over three shapes, both scale forms, both tile
       # heights; 16-bit operands lose 5 % with it: their LDS reads grow by half and nothing is saved).
       converted = key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2, _lib.TKX_F8E4M3FN)
-      # (fp8 activations over packed int4 weights turn nibbles into fp8 bytes the same way: 2070-2230 TFLOP/s on one
-      # row of waves against 1660-2050 on two at the Mixtral shape)
+      # (fp8 activations over packed int4 weights turn nibbles into fp8 bytes the same way: the 128-row tile runs at
+      # 2070-2270 TFLOP/s on one row of waves against 1660-2050 on two at the Mixtral shape; their 256-row tile exists
+      # on two rows only)
       two_wave_rows = wm - 1 if converted or (key[1] == _lib.TKX_F8E4M3FN and key[2] == _lib.TKX_I4X2) else 0
       # ... and among those, the variant whose LDS lets two of its workgroups share a CU (the library gives such a
       # kernel 128 registers: 8 waves on one row, at most 64 accumulators per lane)
