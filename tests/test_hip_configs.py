@@ -165,6 +165,34 @@ def test_packed_int4_weights_at_the_prefill_size(scales, device):
   assert torch.equal(tokamax_amd.ragged_dot(w.lhs, packed, gs, preferred_element_type=torch.bfloat16), out)
 
 
+def test_fp8_activations_over_packed_int4_weights_at_the_prefill_size(device):
+  """The Mixtral prefill shape with activations quantised to fp8 per row over int4 weights packed two to a byte, on the
+  fp8 MFMAs (the 256-row tile): one row out of every 32-row block of every group against the oracle's definition on
+  the dequantised operands; scaling the activations' scales by two doubles the result exactly (the affine correction
+  with the row sums is applied before the scales); determinism."""
+  w = workloads.make("fp8", device)
+  gs = torch.tensor(w.group_sizes, device=device)
+  gen = torch.Generator(device=device).manual_seed(5)
+  q = torch.randint(-8, 8, tuple(w.rhs.shape), device=device, dtype=torch.int8, generator=gen)
+  scale = (torch.rand(w.num_groups, 1, w.n, device=device, generator=gen) + 0.5) / (7 * w.k ** 0.5)
+  packed = tokamax_amd.pack_int4(tokamax_amd.QArray(q, scale, None, getattr(torch, "int4", torch.int8)))
+  lhs = tokamax_amd.QArray(w.lhs, w.lhs_scale)
+  op = tokamax_amd.HipRaggedDot()
+  bound = op.bind(lhs, packed, group_sizes=gs, preferred_element_type=torch.bfloat16)
+  assert op._problem(bound)[1] == (0, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2) and bound.default_config.block_m == 256
+  out = tokamax_amd.ragged_dot(lhs, packed, gs, preferred_element_type=torch.bfloat16)
+  assert out.dtype == torch.bfloat16 and tuple(out.shape) == (w.m, w.n)
+  rows, groups = _sample_every_block(w.group_sizes, 2)
+  assert len(rows) >= w.m // 32
+  index = torch.as_tensor(rows, device=device)
+  lhs_f = (O.e4m3fn_decode(w.lhs[index].view(torch.uint8).cpu().numpy()).astype(np.float64)
+           * _np(w.lhs_scale.reshape(w.m, 1)[index]))
+  _check_rows(out, lhs_f, lambda g: O.dequantize(q[g].cpu().numpy()[None], _np(scale[g])[None])[0], rows, groups, 3e-3)
+  doubled = tokamax_amd.QArray(w.lhs, w.lhs_scale * 2)
+  assert torch.equal(tokamax_amd.ragged_dot(doubled, packed, gs, preferred_element_type=torch.bfloat16), out * 2)
+  assert torch.equal(tokamax_amd.ragged_dot(lhs, packed, gs, preferred_element_type=torch.bfloat16), out)
+
+
 def test_vjp_config(device):
   w = workloads.make("vjp", device)
   gs = torch.tensor(w.group_sizes, device=device)
