@@ -408,7 +408,15 @@ def main():
     measure("mixtral_gateup_silu_int4_packed_weights",
             lambda: op(lhs, q4g, group_sizes=gs, fuse_gateup_activation="silu", preferred_element_type=torch.bfloat16),
             2 * m_ * k_ * 2 * n_, (m_ * k_ + m_ * n_) * 2 + 8 * k_ * n_, "mfma", "bf16", cfg4)
-    del q4g
+    # ... and with the activations quantised to fp8 per row on top: the fp8 MFMAs on the nibbles (the row-sum pass is
+    # part of the call)
+    from tokamax_amd.ragged_dot import hip_ops as _ops  # pylint: disable=g-import-not-at-top
+    lhs8 = tokamax_amd.QArray(*_ops.quantize(lhs, torch.float8_e4m3fn, (1, k_)))
+    cfg48 = op.bind(lhs8, q4g, group_sizes=gs, fuse_gateup_activation="silu", preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_gateup_silu_fp8_activations_int4_packed_weights",
+            lambda: op(lhs8, q4g, group_sizes=gs, fuse_gateup_activation="silu", preferred_element_type=torch.bfloat16),
+            2 * m_ * k_ * 2 * n_, m_ * k_ + m_ * n_ * 2 + 8 * k_ * n_, "mfma", "fp8", cfg48)
+    del q4g, lhs8
     # The whole expert FFN of a Mixtral layer around those two products, as a caller strings it together: tokens
     # permuted into expert order (ragged_gather), gate-up product with silu(gate) * up in the epilogue, down
     # projection, weighted top-2 combine back into token order (ragged_gather_reduce). 8192 tokens, top 2 of 8 experts.

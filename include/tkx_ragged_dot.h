@@ -54,7 +54,8 @@ enum TkxDtype {
                   [G, k/2, n] holds k = 2 kk in bits 0-3 and k = 2 kk + 1 in bits 4-7 (two's complement). Taken as the
                   rhs of a bf16 lhs in the default mode by the streaming small-m kernel (block_m == 16, block_n == 128)
                   and by tiled forward variants of their own (plain, gate-up fusion, scales per k-block; k % block_k
-                  == 0; listed by tkx_ragged_dot_variant); tkx_unpack_int4 turns it into TKX_I8 for everything else. The reference defines no packed layout (its int4 is jnp.int4; its sm90 kernels
+                  == 0; listed by tkx_ragged_dot_variant), and as the rhs of an fp8 lhs by the plain and gate-up
+                  variants described at tkx_row_sums_fp8; tkx_unpack_int4 turns it into TKX_I8 for everything else. The reference defines no packed layout (its int4 is jnp.int4; its sm90 kernels
                   read int4 weights in pallas_mosaic_gpu_kernel_sm90_quant.py:46-387). */
 };
 
@@ -283,7 +284,7 @@ int32_t tkx_unpack_int4(const void* packed, void* out, int64_t packed_rows, int6
 int32_t tkx_pack_int4(const void* values, void* packed, int64_t packed_rows, int64_t cols, tkx_stream_t stream);
 
 /* Row sums of an fp8 (e4m3fn) matrix [rows, cols] in f32: sums[r] = sum_c x[r, c]. cols % 16 == 0, x 16-byte aligned.
- * The fp8 x packed-int4 forward (lhs TKX_F8E4M3FN, rhs TKX_I4X2, plain forward variants with block_k = 128) takes them
+ * The fp8 x packed-int4 forward (lhs TKX_F8E4M3FN, rhs TKX_I4X2, plain and gate-up forward variants with block_k = 128) takes them
  * behind the row scales, lhs_scale = f32[2, m]: it feeds weight w to the fp8 MFMAs as the e4m3 denormal (w + 8) / 512
  * and computes (512 acc - 8 sums[row]) * lhs_scale[row] * rhs_scale[group, col]. The reference's kernel packs the
  * sums with the activation scales the same way (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:258-300, 436-470). */

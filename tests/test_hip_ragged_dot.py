@@ -354,7 +354,11 @@ def test_every_kernel_variant_through_c_abi(v, device):
   if v["mode"] == 3:  # forward with gate-up fusion and a bias: rhs [g, k, 2 n'] -> out [m, n']
     lhs = mk((m, k), 1.0).to(lt)
     bias = mk((G, 1, n), 0.5)
-    scale = None
+    scale = lhs_scale = None
+    lhs_f = _np(lhs)
+    if lt == torch.float8_e4m3fn:  # (over packed int4 weights) one scale per row
+      lhs_scale = mk((m, 1), 0.1).abs() + 0.05
+      lhs_f = lhs_f * _np(lhs_scale)
     if rt == torch.int8:  # int8 weights with one scale per (group, column)
       rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
       scale = mk((G, 1, n), 0.005).abs() + 1e-3
@@ -368,9 +372,9 @@ def test_every_kernel_variant_through_c_abi(v, device):
       rhs = mk((G, k, n), k ** -0.5).to(rt)
       rhs_f = _np(rhs)
     out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, rhs_bias=bias, activation="silu",
-                                 gateup=True, rhs_scale=scale)
-    want = O.ragged_dot_fused(_np(lhs), rhs_f, gs, rhs_bias=_np(bias), gateup_activation="silu")
-    _check(out, want, 1e-5)
+                                 gateup=True, rhs_scale=scale, lhs_scale=lhs_scale)
+    want = O.ragged_dot_fused(lhs_f, rhs_f, gs, rhs_bias=_np(bias), gateup_activation="silu")
+    _check(out, want, 1e-5 if lhs_scale is None else 1e-4)
     assert out.shape == (m, n // 2) and torch.count_nonzero(out[int(gs.sum()):]) == 0
     return
   if v["mode"] == 4 and lt == torch.float8_e4m3fn:  # fp8 x fp8, scales per block of 128 k rows on both sides, a bias
@@ -894,7 +898,7 @@ def test_tiled_kernels_on_packed_int4_weights(v, device):
 
 def _fp8_over_packed_int4_cases():
   return [pytest.param(v, id="{block_m}x{block_n}x{block_k}-w{waves_m}x{waves_n}-s{num_stages}".format(**v))
-          for v in _lib.variants(0) if v["rhs_dtype"] == _lib.TKX_I4X2 and v["lhs_dtype"] == _lib.TKX_F8E4M3FN]
+          for v in _lib.variants(0) if v["rhs_dtype"] == _lib.TKX_I4X2 and v["lhs_dtype"] == _lib.TKX_F8E4M3FN and v["mode"] == 0]
 
 
 def test_row_sums_of_fp8_rows(device):
@@ -960,8 +964,8 @@ def test_tiled_kernels_on_fp8_activations_and_packed_int4_weights(v, device):
       split = call(dataclasses.replace(cfg, split_k=split_k))
       _check(split, want, 5e-5)
       assert torch.equal(split, call(dataclasses.replace(cfg, split_k=split_k)))
-  # bf16 result without a weight scale; no lhs scale, scales per k-block, gate-up fusion and a contraction that is
-  # not whole k-steps are declined
+  # bf16 result without a weight scale; no lhs scale, scales per k-block and a contraction that is not whole k-steps
+  # are declined
   plain = hip_ops.ragged_dot_fwd(xq, packed, gst, config=cfg, out_dtype=torch.bfloat16, lhs_scale=xs)
   _check(plain, O.ragged_dot(lhs_f, values.astype(np.float64), gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 4e-3)
   with pytest.raises(NotImplementedError, match="lhs scale"):
@@ -969,9 +973,6 @@ def test_tiled_kernels_on_fp8_activations_and_packed_int4_weights(v, device):
   with pytest.raises(NotImplementedError):
     hip_ops.ragged_dot_fwd(xq, packed, gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs,
                            rhs_scale=scale.expand(G, 5, n).contiguous())
-  with pytest.raises(NotImplementedError):
-    hip_ops.ragged_dot_fwd(xq, packed[:, :, :256].contiguous(), gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs,
-                           gateup=True, activation="silu")
   with pytest.raises(NotImplementedError, match="block_k"):
     hip_ops.ragged_dot_fwd(xq[:, :k - 32].contiguous(), packed[:, :k // 2 - 16].contiguous(), gst, config=cfg,
                            out_dtype=torch.float32, lhs_scale=xs)
@@ -1023,6 +1024,13 @@ def test_public_op_on_fp8_activations_and_packed_int4_weights(device):
   lhs_q = O.e4m3fn_decode(quantised.qvalue.view(torch.uint8).cpu().numpy()).astype(np.float64) * _np(quantised.scale)
   _check(out_q, O.ragged_dot(lhs_q, O.dequantize(q.cpu().numpy(), _np(scale)), np.full(G, rows, np.int32), O.DEFAULT,
                              acc_dtype=np.float64, out_dtype="f64"), 5e-5)
+  # gate-up fusion over the same weights read as [gate | up]: the kernels of the fp8 x int4 kind again
+  bound = op.bind(lhs, packed, group_sizes=gs, preferred_element_type=torch.float32, fuse_gateup_activation="silu")
+  assert op._problem(bound)[1] == (3, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2) and bound.default_config.block_k == 128
+  fused = op(lhs, packed, group_sizes=gs, preferred_element_type=torch.float32, fuse_gateup_activation="silu")
+  assert tuple(fused.shape) == (m, n // 2)
+  _check(fused, O.ragged_dot_fused(lhs_f, O.dequantize(q.cpu().numpy(), _np(scale)), np.full(G, rows, np.int32),
+                                   gateup_activation="silu"), 5e-5)
   # scales per k-block: no kernel of this kind; the weights are unpacked and the widened path runs
   blocks = tokamax_amd.pack_int4(tokamax_amd.QArray(q, scale.expand(G, 4, n).contiguous(), None, int4))
   assert _lib_key(op, lhs, blocks, gs)[2] != _lib.TKX_I4X2

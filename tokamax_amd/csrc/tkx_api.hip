@@ -299,9 +299,9 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
                      (long long)k, c.block_k);
   // fp8 activations over packed int4 weights: the kernel feeds the weights to the fp8 MFMAs with a bias of +8 and
   // takes 8 times the row sum of the fp8 activations off in its epilogue.
-  if (rhs_dtype == TKX_I4X2 && lhs_dtype == TKX_F8E4M3FN && (lhs_scale == nullptr || gateup || subk))
+  if (rhs_dtype == TKX_I4X2 && lhs_dtype == TKX_F8E4M3FN && (lhs_scale == nullptr || subk))
     return set_error(TKX_ERR_UNSUPPORTED,
-                     "fp8 x packed int4 weights: plain forward with lhs_scale f32[2, m] (the row scales, then the row sums"
+                     "fp8 x packed int4 weights: plain or gate-up forward with lhs_scale f32[2, m] (the row scales, then the row sums"
                      " of the fp8 values, tkx_row_sums_fp8) and at most one rhs scale per (group, column)");
   const Variant* v = find_variant(dlhs ? kDlhs : gateup ? kFwdGlu : subk ? kFwdSubK : kFwd, lhs_dtype, rhs_dtype, c);
   if (v == nullptr)

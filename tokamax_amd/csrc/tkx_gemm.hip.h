@@ -613,8 +613,8 @@ struct GemmKernel {
   static constexpr bool JOUT = LEAN && I4F && TN >= 2;
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
   static_assert(!SPLIT || (MODE == kFwd && EA == EB && BK % 2 == 0), "split pipeline: plain forward, operands of one type");
-  static_assert(!I4 || (((I4P && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK)) || (I4F && MODE == kFwd)) && !SPLIT),
-                "packed int4 weights: forward with bf16 activations, plain forward with fp8 activations");
+  static_assert(!I4 || (((I4P && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK)) || (I4F && (MODE == kFwd || MODE == kFwdGlu))) && !SPLIT),
+                "packed int4 weights: forward with bf16 activations; plain or gate-up forward with fp8 activations");
   static constexpr int BKB = I4 ? BKC / 2 : BKC;  // rows of a B stage
   typedef TileStage<LA, EA, BM, BK, THREADS> StageA;
   typedef TileStage<LB, EBS, BN, BKB, THREADS> StageB;

@@ -15,6 +15,7 @@ namespace tkx {
 // off with the activations' row sums (lhs_scale holds [row scales | row sums]). The 256 x 256 x 128 tile runs an atom's
 // MFMAs column block by column block and keeps one set of converted rhs fragments (GemmKernel::JOUT).
 #define F8FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEF8, kEI4, BM, BN, BK, WM, WN, NS)
+#define F8GLU(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdGlu, kEF8, kEI4, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
     FWD(256, 256, 64, 2, 4, 2),
@@ -38,6 +39,10 @@ static const Variant kVariants[] = {
     SUBK(128, 256, 64, 1, 8, 3),
     SUBK(32, 256, 64, 1, 4, 4),
     F8FWD(256, 256, 128, 2, 4, 3),
+    F8GLU(256, 256, 128, 2, 4, 3),
+    F8GLU(128, 256, 128, 2, 4, 3),
+    F8GLU(64, 256, 128, 2, 4, 3),
+    F8GLU(32, 256, 128, 1, 4, 4),
     F8FWD(128, 256, 128, 2, 4, 3),
     F8FWD(128, 256, 128, 1, 8, 3),
     F8FWD(128, 256, 128, 1, 8, 4),
