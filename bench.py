@@ -335,7 +335,15 @@ def main():
     measure("mixtral_prefill_fp8_activations_int4_packed_weights",
             lambda: op(ql, q4f, group_sizes=gs, preferred_element_type=torch.bfloat16), w.flops,
             w.m * w.k + w.nonempty_groups * w.k * w.n // 2 + w.m * w.n * 2, "mfma", "fp8", cfg)
-    del w, ql, qr, qlk, qrk, q4f
+    # ... and with the usual scales of int4 weights, one per (group, 128 k rows, column): every k-step's products are
+    # folded in with its scales and the row sums of its own 128 activation columns
+    q4fk = tokamax_amd.QArray(q4f.qvalue, (torch.rand(w.num_groups, kb, w.n, device=device, generator=gen4f) + 0.5)
+                              / (7 * w.k ** 0.5), None, q4f.qtype)
+    cfg = op.bind(ql, q4fk, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_prefill_fp8_activations_int4_packed_weights_k_block_scales",
+            lambda: op(ql, q4fk, group_sizes=gs, preferred_element_type=torch.bfloat16), w.flops,
+            w.m * w.k + w.nonempty_groups * (w.k * w.n // 2 + kb * w.n * 4) + w.m * kb * 8 + w.m * w.n * 2, "mfma", "fp8", cfg)
+    del w, ql, qr, qlk, qrk, q4f, q4fk
 
     # the Mixtral shape with int8 weights (one f32 scale per (group, column)): the weight stream into LDS is half of bf16's
     w = workloads.make("mixtral", device, seed=0)

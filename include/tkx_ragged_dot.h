@@ -283,12 +283,17 @@ int32_t tkx_dequantize_zero_point(const void* qvalue, const float* scale, const 
 int32_t tkx_unpack_int4(const void* packed, void* out, int64_t packed_rows, int64_t cols, tkx_stream_t stream);
 int32_t tkx_pack_int4(const void* values, void* packed, int64_t packed_rows, int64_t cols, tkx_stream_t stream);
 
-/* Row sums of an fp8 (e4m3fn) matrix [rows, cols] in f32: sums[r] = sum_c x[r, c]. cols % 16 == 0, x 16-byte aligned.
+/* Row sums of an fp8 (e4m3fn) matrix [rows, cols] in f32: chunk_cols == cols: sums[r] = sum_c x[r, c]; chunk_cols ==
+ * 128 (cols % 128 == 0): sums[c / 128][r], one per run of 128 columns. cols % 16 == 0, x 16-byte aligned.
  * The fp8 x packed-int4 forward (lhs TKX_F8E4M3FN, rhs TKX_I4X2, plain and gate-up forward variants with block_k = 128) takes them
  * behind the row scales, lhs_scale = f32[2, m]: it feeds weight w to the fp8 MFMAs as the e4m3 denormal (w + 8) / 512
  * and computes (512 acc - 8 sums[row]) * lhs_scale[row] * rhs_scale[group, col]. The reference's kernel packs the
- * sums with the activation scales the same way (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:258-300, 436-470). */
-int32_t tkx_row_sums_fp8(const void* x, float* sums, int64_t rows, int64_t cols, tkx_stream_t stream);
+ * sums with the activation scales the same way (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:258-300, 436-470).
+ * With rhs scales per k-block (tkx_ragged_dot_fwd_fused, rhs_scale_blocks > 1; blocks of a power of two >= 128 rows;
+ * m % 4 == 0): lhs_scale = f32[blocks + k / 128, m], the lhs scales per k-block followed by the row sums per 128
+ * columns, and every 128-deep k-step's products are folded in as (512 part - 8 sums[step][row]) * lhs_scale[block][row]
+ * * rhs_scale[group, block, col] (the per-subchannel form of the same reference kernel, :740-790). */
+int32_t tkx_row_sums_fp8(const void* x, float* sums, int64_t rows, int64_t cols, int64_t chunk_cols, tkx_stream_t stream);
 
 /* Quantisation on the fly (AsQArray.as_qarray, quantization.py:65-78: qwix.quantize with the "absmax" calibration), the
  * inverse of tkx_dequantize:

@@ -378,12 +378,18 @@ def test_every_kernel_variant_through_c_abi(v, device):
     assert out.shape == (m, n // 2) and torch.count_nonzero(out[int(gs.sum()):]) == 0
     return
   if v["mode"] == 4 and lt == torch.float8_e4m3fn:  # fp8 x fp8, scales per block of 128 k rows on both sides, a bias
-    lhs, rhs = mk((m, k), 1.0).to(lt), mk((G, k, n), 1.0).to(rt)
+    lhs = mk((m, k), 1.0).to(lt)
+    if rt == torch.uint8:  # ... or fp8 over int4 weights, two to a byte along k
+      rhs_values = rng.integers(-8, 8, (G, k, n)).astype(np.float64)
+      rhs = torch.tensor(O.pack_int4(rhs_values.astype(np.int8)), device=device)
+    else:
+      rhs = mk((G, k, n), 1.0).to(rt)
+      rhs_values = O.e4m3fn_decode(rhs.view(torch.uint8).cpu().numpy()).astype(np.float64)
     xs, ws_ = mk((m, 2), 0.1).abs() + 0.05, mk((G, 2, n), 0.1).abs() + 0.05
     bias = mk((G, 1, n), 0.5)
     out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs, rhs_scale=ws_, rhs_bias=bias)
     lhs_f = O.dequantize(O.e4m3fn_decode(lhs.view(torch.uint8).cpu().numpy()).astype(np.float64), _np(xs))
-    rhs_f = O.dequantize(O.e4m3fn_decode(rhs.view(torch.uint8).cpu().numpy()).astype(np.float64), _np(ws_))
+    rhs_f = O.dequantize(rhs_values, _np(ws_))
     _check(out, O.ragged_dot_fused(lhs_f, rhs_f, gs, rhs_bias=_np(bias)), 1e-4)
     assert torch.count_nonzero(out[int(gs.sum()):]) == 0
     return
@@ -905,7 +911,7 @@ def test_row_sums_of_fp8_rows(device):
   """tkx_row_sums_fp8 against sums in float64 of the decoded bytes: every finite e4m3fn value occurs, rows shorter and
   longer than a wave's 1024-byte step, a row count that is not whole workgroups."""
   rng = np.random.default_rng(31)
-  for rows, cols in ((7, 16), (33, 1040), (4, 4096)):
+  for rows, cols in ((7, 16), (33, 1040), (4, 4096), (9, 1408)):
     codes = rng.integers(0, 256, (rows, cols)).astype(np.uint8)
     codes[(codes & 0x7f) == 0x7f] = 0x08  # (no NaN)
     x = torch.tensor(codes, device=device).view(torch.float8_e4m3fn)
@@ -914,6 +920,11 @@ def test_row_sums_of_fp8_rows(device):
     scale = np.abs(O.e4m3fn_decode(codes).astype(np.float64)).sum(axis=1)
     assert sums.dtype == torch.float32 and tuple(sums.shape) == (rows,)
     assert np.all(np.abs(_np(sums) - want) <= 1e-6 * scale)
+    if cols % 128 == 0:
+      chunks = hip_ops.row_sums_fp8(x, per_128_columns=True)
+      values = O.e4m3fn_decode(codes).astype(np.float64).reshape(rows, cols // 128, 128)
+      assert tuple(chunks.shape) == (cols // 128, rows)
+      assert np.all(np.abs(_np(chunks).T - values.sum(axis=2)) <= 1e-6 * np.abs(values).sum(axis=2))
   with pytest.raises(ValueError):
     hip_ops.row_sums_fp8(torch.zeros(4, 16, device=device))
   with pytest.raises(NotImplementedError, match="multiple of 16"):
@@ -964,15 +975,15 @@ def test_tiled_kernels_on_fp8_activations_and_packed_int4_weights(v, device):
       split = call(dataclasses.replace(cfg, split_k=split_k))
       _check(split, want, 5e-5)
       assert torch.equal(split, call(dataclasses.replace(cfg, split_k=split_k)))
-  # bf16 result without a weight scale; no lhs scale, scales per k-block and a contraction that is not whole k-steps
-  # are declined
+  # bf16 result without a weight scale; no lhs scale, scale blocks of another size than a power of two and a
+  # contraction that is not whole k-steps are declined
   plain = hip_ops.ragged_dot_fwd(xq, packed, gst, config=cfg, out_dtype=torch.bfloat16, lhs_scale=xs)
   _check(plain, O.ragged_dot(lhs_f, values.astype(np.float64), gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 4e-3)
   with pytest.raises(NotImplementedError, match="lhs scale"):
     hip_ops.ragged_dot_fwd(xq, packed, gst, config=cfg, out_dtype=torch.float32, rhs_scale=scale)
   with pytest.raises(NotImplementedError):
     hip_ops.ragged_dot_fwd(xq, packed, gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs,
-                           rhs_scale=scale.expand(G, 5, n).contiguous())
+                           rhs_scale=scale.expand(G, 2, n).contiguous())  # (blocks of 320 rows: not a power of two)
   with pytest.raises(NotImplementedError, match="block_k"):
     hip_ops.ragged_dot_fwd(xq[:, :k - 32].contiguous(), packed[:, :k // 2 - 16].contiguous(), gst, config=cfg,
                            out_dtype=torch.float32, lhs_scale=xs)
@@ -1031,10 +1042,24 @@ def test_public_op_on_fp8_activations_and_packed_int4_weights(device):
   assert tuple(fused.shape) == (m, n // 2)
   _check(fused, O.ragged_dot_fused(lhs_f, O.dequantize(q.cpu().numpy(), _np(scale)), np.full(G, rows, np.int32),
                                    gateup_activation="silu"), 5e-5)
-  # scales per k-block: no kernel of this kind; the weights are unpacked and the widened path runs
-  blocks = tokamax_amd.pack_int4(tokamax_amd.QArray(q, scale.expand(G, 4, n).contiguous(), None, int4))
-  assert _lib_key(op, lhs, blocks, gs)[2] != _lib.TKX_I4X2
-  _check(op(lhs, blocks, group_sizes=gs, preferred_element_type=torch.float32), want, 1e-2)
+  # scales per block of 128 k rows on the weights, per row or per (row, same block) on the activations: kernels of
+  # the same kind that fold every k-step in with its scales and its own row sums
+  scale4 = torch.tensor((rng.uniform(0.5, 1.5, (G, 4, n)) / 7 * 0.1).astype(np.float32), device=device)
+  blocks = tokamax_amd.pack_int4(tokamax_amd.QArray(q, scale4, None, int4))
+  assert _lib_key(op, lhs, blocks, gs) == (4, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
+  rhs_f = O.dequantize(q.cpu().numpy(), _np(scale4))
+  _check(op(lhs, blocks, group_sizes=gs, preferred_element_type=torch.float32),
+         O.ragged_dot(lhs_f, rhs_f, np.full(G, rows, np.int32), O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 5e-5)
+  xs4 = torch.tensor(rng.uniform(0.5, 1.5, (m, 4)).astype(np.float32), device=device) * xs
+  lhs4 = tokamax_amd.QArray(lhs.qvalue, xs4)
+  assert _lib_key(op, lhs4, blocks, gs) == (4, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
+  lhs4_f = O.dequantize(O.e4m3fn_decode(lhs.qvalue.view(torch.uint8).cpu().numpy()).astype(np.float64), _np(xs4))
+  _check(op(lhs4, blocks, group_sizes=gs, preferred_element_type=torch.float32),
+         O.ragged_dot(lhs4_f, rhs_f, np.full(G, rows, np.int32), O.DEFAULT, acc_dtype=np.float64, out_dtype="f64"), 5e-5)
+  # blocks of 32 rows: no kernel of this kind; the weights are unpacked and the widened path runs
+  small = tokamax_amd.pack_int4(tokamax_amd.QArray(q, scale.expand(G, 16, n).contiguous(), None, int4))
+  assert _lib_key(op, lhs, small, gs)[2] != _lib.TKX_I4X2
+  _check(op(lhs, small, group_sizes=gs, preferred_element_type=torch.float32), want, 1e-2)
 
 
 def _lib_key(op, lhs, rhs, gs):

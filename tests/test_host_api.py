@@ -664,8 +664,7 @@ def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   assert {x.block_m for x in space} >= {16, 32, 128, 256}
   # fp8 activations with one scale per row (or per run of rows): the packed weights stay packed for the kernels that
   # feed the nibbles to the fp8 MFMAs (one row of waves: each nibble becomes an fp8 byte once per workgroup); with scale
-  # blocks along k they are unpacked, and fp8 activations over int8 storage are widened to bf16; gate-up fusion has
-  # kernels of the same kind
+  # fp8 activations over int8 storage are widened to bf16; gate-up fusion has kernels of the same kind
   f8 = torch.float8_e4m3fn
   x8 = tokamax_amd.QArray(ShapeDtype((4096, 1024), f8), ShapeDtype((4096, 1), f32))
   route8 = lambda x, rhs, **kw: op._problem(op.bind(x, rhs, group_sizes=gs, **kw))[1]
@@ -680,7 +679,14 @@ def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   c = op._get_heuristics_config(op.bind(fewer, wide, group_sizes=gs))  # 128 rows per group: 128 rows on one row of waves
   assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n) == (128, 256, 128, 1, 8)
   assert {x.block_k for x in op._get_autotuning_configs(op.bind(x8, wide, group_sizes=gs))} == {128}
-  assert route8(x8, blocks) == (4, _lib.TKX_BF16, _lib.TKX_I8)
+  # scale blocks of a power of two >= 128 rows along k (lhs scales per row or per (row, same block)): kernels of the
+  # same kind that fold every k-step's products in with its scales; smaller blocks are unpacked and widened
+  assert route8(x8, blocks) == (4, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
+  c = op._get_heuristics_config(op.bind(x8, blocks, group_sizes=gs))
+  assert (c.block_n, c.block_k) == (256, 128)
+  x8_same = tokamax_amd.QArray(ShapeDtype((4096, 1024), f8), ShapeDtype((4096, 4), f32))
+  assert route8(x8_same, blocks) == (4, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
+  assert route8(x8, small_blocks)[2] != _lib.TKX_I4X2
   assert route8(x8, packed, fuse_gateup_activation="silu") == (3, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
   assert route8(x8, blocks, fuse_gateup_activation="silu") == (3, _lib.TKX_BF16, _lib.TKX_BF16)
   assert route8(x8, packed.unpacked()) == (0, _lib.TKX_BF16, _lib.TKX_I8)

@@ -92,7 +92,7 @@ def _declare(lib):
     fn.restype = i32
     fn.argtypes = [vp, vp, i64, i64, vp]
   lib.tkx_row_sums_fp8.restype = i32
-  lib.tkx_row_sums_fp8.argtypes = [vp, vp, i64, i64, vp]
+  lib.tkx_row_sums_fp8.argtypes = [vp, vp, i64, i64, i64, vp]
   lib.tkx_last_error.restype = ctypes.c_char_p
   lib.tkx_last_error.argtypes = []
   lib.tkx_ragged_dot_tid_size.restype = i64

@@ -299,10 +299,11 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
                      (long long)k, c.block_k);
   // fp8 activations over packed int4 weights: the kernel feeds the weights to the fp8 MFMAs with a bias of +8 and
   // takes 8 times the row sum of the fp8 activations off in its epilogue.
-  if (rhs_dtype == TKX_I4X2 && lhs_dtype == TKX_F8E4M3FN && (lhs_scale == nullptr || subk))
+  if (rhs_dtype == TKX_I4X2 && lhs_dtype == TKX_F8E4M3FN && (lhs_scale == nullptr || (subk && c.block_k != 128)))
     return set_error(TKX_ERR_UNSUPPORTED,
-                     "fp8 x packed int4 weights: plain or gate-up forward with lhs_scale f32[2, m] (the row scales, then the row sums"
-                     " of the fp8 values, tkx_row_sums_fp8) and at most one rhs scale per (group, column)");
+                     "fp8 x packed int4 weights: lhs_scale f32[2, m] (the row scales, then the row sums of the fp8 values,"
+                     " tkx_row_sums_fp8), or with rhs scales per k-block f32[blocks + k / 128, m] (scales per k-block, then row"
+                     " sums per 128 columns) and block_k == 128");
   const Variant* v = find_variant(dlhs ? kDlhs : gateup ? kFwdGlu : subk ? kFwdSubK : kFwd, lhs_dtype, rhs_dtype, c);
   if (v == nullptr)
     return set_error(TKX_ERR_UNSUPPORTED, "no kernel variant for mode=%d dtypes=(%d,%d) tile=%dx%dx%d waves=%dx%d stages=%d",
@@ -628,12 +629,14 @@ int32_t tkx_pack_int4(const void* values, void* packed, int64_t packed_rows, int
   return int4_repack(values, packed, packed_rows, cols, false, stream);
 }
 
-int32_t tkx_row_sums_fp8(const void* x, float* sums, int64_t rows, int64_t cols, tkx_stream_t stream) {
+int32_t tkx_row_sums_fp8(const void* x, float* sums, int64_t rows, int64_t cols, int64_t chunk_cols, tkx_stream_t stream) {
   if (!x || !sums) return set_error(TKX_ERR_INVALID, "null pointer argument");
   if (rows < 1 || cols < 1 || rows > 0x7fffffffLL) return set_error(TKX_ERR_INVALID, "bad sizes rows=%lld cols=%lld", (long long)rows, (long long)cols);
   if (cols % 16 != 0 || cols > 0x7fffffffLL) return set_error(TKX_ERR_UNSUPPORTED, "cols must be a multiple of 16");
   if ((uintptr_t)x % 16 != 0 || (uintptr_t)sums % 4 != 0) return set_error(TKX_ERR_UNSUPPORTED, "x must be 16-byte aligned, sums 4-byte aligned");
-  return launch_row_sums_fp8(x, sums, rows, cols, static_cast<hipStream_t>(stream));
+  if (chunk_cols != cols && (chunk_cols != 128 || cols % 128 != 0))
+    return set_error(TKX_ERR_UNSUPPORTED, "chunk_cols is cols (one sum per row) or 128 with cols %% 128 == 0 (got %lld)", (long long)chunk_cols);
+  return launch_row_sums_fp8(x, sums, rows, cols, chunk_cols != cols, static_cast<hipStream_t>(stream));
 }
 
 int32_t tkx_quantize(const void* x, void* qvalue, float* scale, int64_t rows, int64_t cols, int64_t scale_block_rows,

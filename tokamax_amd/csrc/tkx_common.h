@@ -145,7 +145,7 @@ int32_t launch_decode(const void* lhs, const void* rhs, const float* scale, cons
 
 // ---- packed int4 (TKX_I4X2) <-> int8: `packed_rows` rows of n bytes against 2 * packed_rows rows of n values ----
 int32_t launch_int4_repack(const void* in, void* out, int64_t packed_rows, int64_t n, bool unpack, hipStream_t stream);
-int32_t launch_row_sums_fp8(const void* x, float* sums, int64_t rows, int64_t n, hipStream_t stream);
+int32_t launch_row_sums_fp8(const void* x, float* sums, int64_t rows, int64_t n, bool per_128, hipStream_t stream);
 
 // ---- dequantisation of int8 weights with sub-channel scales to bf16 ------------------------------
 // out[r, c] = q[r, c] * scale[r / t_r, c / t_c]; q int8 or fp8 (e4m3fn), out bf16; t_c is 1 or a multiple of 16.

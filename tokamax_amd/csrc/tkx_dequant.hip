@@ -126,6 +126,8 @@ __global__ __launch_bounds__(kDqThreads) void pack_int4_kernel(const signed char
 
 // Row sums of an fp8 (e4m3fn) matrix [rows, n], n % 16 == 0: one wave per row, 16 bytes per lane and step, summed in
 // f32. The sums of activation rows, which the fp8 x packed-int4 kernels take their +8 weight bias off with.
+// PER_128 (n % 128 == 0): one sum per run of 128 columns (8 lanes), sums[n / 128][rows].
+template <bool PER_128>
 __global__ __launch_bounds__(kDqThreads) void row_sums_fp8_kernel(const unsigned char* __restrict__ x, float* __restrict__ sums,
                                                                  int64_t rows, int32_t n) {
   const int lane = threadIdx.x & 63;
@@ -137,17 +139,28 @@ __global__ __launch_bounds__(kDqThreads) void row_sums_fp8_kernel(const unsigned
 #pragma unroll
     for (int d = 0; d < 4; ++d)
       s += (widen_byte<kEF8, 0>(w[d]) + widen_byte<kEF8, 1>(w[d])) + (widen_byte<kEF8, 2>(w[d]) + widen_byte<kEF8, 3>(w[d]));
-  }
+    if constexpr (PER_128) {
+      // (the lanes of a group of 8 are in the loop together: n is a multiple of 128)
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
-  if (lane == 0) sums[row] = s;
+      for (int o = 4; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+      if ((lane & 7) == 0) sums[(int64_t)(c0 >> 7) * rows + row] = s;
+      s = 0.f;
+    }
+  }
+  if constexpr (!PER_128) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    if (lane == 0) sums[row] = s;
+  }
 }
 
 }  // namespace
 
-int32_t launch_row_sums_fp8(const void* x, float* sums, int64_t rows, int64_t n, hipStream_t stream) {
+int32_t launch_row_sums_fp8(const void* x, float* sums, int64_t rows, int64_t n, bool per_128, hipStream_t stream) {
   const int64_t grid = (rows + kDqThreads / 64 - 1) / (kDqThreads / 64);
-  row_sums_fp8_kernel<<<dim3((unsigned)grid), dim3(kDqThreads), 0, stream>>>(static_cast<const unsigned char*>(x), sums, rows, (int32_t)n);
+  const auto* xb = static_cast<const unsigned char*>(x);
+  if (per_128) row_sums_fp8_kernel<true><<<dim3((unsigned)grid), dim3(kDqThreads), 0, stream>>>(xb, sums, rows, (int32_t)n);
+  else row_sums_fp8_kernel<false><<<dim3((unsigned)grid), dim3(kDqThreads), 0, stream>>>(xb, sums, rows, (int32_t)n);
   TKX_HIP_CHECK(hipGetLastError());
   return TKX_OK;
 }

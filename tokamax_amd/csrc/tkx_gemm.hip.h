@@ -573,8 +573,10 @@ struct GemmKernel {
   // accumulate into partial accumulators, which are folded into the result with the block's scales.
   // int8 x int8 runs the same way on the int8 MFMAs (int32 partial sums, exact), also with one block.
   static constexpr bool SUBP = SUBK && (EA == kEF8 || EA == kEI8);
-  static_assert(!SUBK || ((EB == kEI8 || EB == kEF8 || EB == kEI4) && (EA == kEBF16 || (SUBP && EB == EA)) && BN == 256),
-                "per-k-block scales: bf16 lhs with int8, packed int4 or fp8 weights, fp8 x fp8 or int8 x int8; one 1 KB scale row per k-step");
+  static_assert(!SUBK || ((EB == kEI8 || EB == kEF8 || EB == kEI4) &&
+                          (EA == kEBF16 || (SUBP && EB == EA) || (EA == kEF8 && EB == kEI4 && BK == 128)) && BN == 256),
+                "per-k-block scales: bf16 lhs with int8, packed int4 or fp8 weights, fp8 x fp8, int8 x int8 or fp8 x packed int4"
+                " (whose row sums come per 128-deep k-step); one 1 KB scale row per k-step");
   static constexpr int BNO = GLU ? BN / 2 : BN;  // output columns of a tile
   static constexpr int EC = EA;  // MFMA type follows A; B may be stored narrower (int8 weights)
   // Packed int4 weights: a B stage is a byte tile of half the depth; a lane's transposing read of 8 bytes of its
@@ -613,8 +615,8 @@ struct GemmKernel {
   static constexpr bool JOUT = LEAN && I4F && TN >= 2;
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
   static_assert(!SPLIT || (MODE == kFwd && EA == EB && BK % 2 == 0), "split pipeline: plain forward, operands of one type");
-  static_assert(!I4 || (((I4P && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK)) || (I4F && (MODE == kFwd || MODE == kFwdGlu))) && !SPLIT),
-                "packed int4 weights: forward with bf16 activations; plain or gate-up forward with fp8 activations");
+  static_assert(!I4 || (((I4P && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK)) || (I4F && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK))) && !SPLIT),
+                "packed int4 weights: forward with bf16 or fp8 activations");
   static constexpr int BKB = I4 ? BKC / 2 : BKC;  // rows of a B stage
   typedef TileStage<LA, EA, BM, BK, THREADS> StageA;
   typedef TileStage<LB, EBS, BN, BKB, THREADS> StageB;
@@ -626,7 +628,8 @@ struct GemmKernel {
   static constexpr int STAGE_BYTES = StageA::BYTES + StageB::BYTES + SCALE_BYTES;
   // fp8 x fp8: the scales of a k-step (BN weight-column scales, then BM lhs-row scales) are still needed when its
   // stage is already being refilled, so they live in a ring of NS + 1 slots behind the stages.
-  static constexpr int RING_SLOT = SUBP ? (BN + BM) * 4 : 0;
+  // (fp8 x packed int4: behind them the BM row sums of the k-step's activations)
+  static constexpr int RING_SLOT = SUBP ? (BN + BM + (I4 ? BM : 0)) * 4 : 0;
   static constexpr int SMEM_BYTES = SPLIT ? NS * StageA::BYTES + HB * StageB::BYTES : NS * STAGE_BYTES + (NS + 1) * RING_SLOT;
   // Workgroups the register budget is set for: two 4-wave workgroups share a CU when their LDS fits twice (256
   // registers per lane each); every other shape has the CU, and a SIMD's 512 registers per lane, to itself or to the
@@ -981,10 +984,10 @@ struct GemmKernel {
       // on its own, so that the list can be threaded between MFMAs. kFwdSubK adds one: the 1 KB scale
       // row of the step's k-block, of which every wave fetches its 1/NLOAD with that many of its lanes
       // (so that all waves count the same number of loads).
-      constexpr int NLD = DirA::PER + DirB::PER + (SUBP ? 2 : SUBK ? 1 : 0);
+      constexpr int NLD = DirA::PER + DirB::PER + (SUBP ? (I4F ? 3 : 2) : SUBK ? 1 : 0);
       constexpr int kInFlight = kExact ? (NS - 2) * NLD : 0;
       static_assert(kInFlight < 64 && (NS - 1) * NLD < 64, "too many direct loads in flight for vmcnt");
-      struct StepPtrs { const unsigned char *a, *b, *s, *x; unsigned lds, ring; };
+      struct StepPtrs { const unsigned char *a, *b, *s, *x, *xsum; unsigned lds, ring; };
       // (kFwdSubK) scales of this tile's columns: row `block` of the group's [scale_blocks, n] table; lanes past
       // the last column re-read the last four (their products are never stored).
       const unsigned char* const gS0 =
@@ -1006,6 +1009,10 @@ struct GemmKernel {
         if constexpr (SUBP) {
           const int64_t block = (kc_begin + step * BK) >> p.log2_block_rows;
           sp.x = uniform_pointer(reinterpret_cast<const unsigned char*>(p.a_scale) + block * p.m_ext * 4);
+          // (fp8 x packed int4) behind the scale_blocks rows of lhs scales: one row of row sums per 128-deep k-step
+          if constexpr (I4F)
+            sp.xsum = uniform_pointer(reinterpret_cast<const unsigned char*>(p.a_scale) +
+                                      (int64_t)(p.scale_blocks + (kc_begin + step * BK) / BK) * p.m_ext * 4);
           sp.ring = smem_lds + NS * STAGE_BYTES + (step % (NS + 1)) * RING_SLOT;
         }
         sp.lds = smem_lds + stage * STAGE_BYTES;
@@ -1019,6 +1026,8 @@ struct GemmKernel {
           if (lane < SCALE_LANES) direct_load_16(sp.s, scale_voff, dst + wave * (SCALE_LANES * 16));
         } else if (SUBP && q == DirA::PER + DirB::PER + 1) {
           if (lane < XS_LANES) direct_load_16(sp.x, xs_voff, sp.ring + BN * 4 + wave * (XS_LANES * 16));
+        } else if (SUBP && I4F && q == DirA::PER + DirB::PER + 2) {
+          if (lane < XS_LANES) direct_load_16(sp.xsum, xs_voff, sp.ring + (BN + BM) * 4 + wave * (XS_LANES * 16));
         }
       };
       // Every wave drains the loads the next k-step needs before it arrives at a barrier.
@@ -1229,9 +1238,17 @@ struct GemmKernel {
             // and, for t = 0..3, columns 8 t + 4 (l / 32) + {0..3} of every 32 x 32 block.
             const unsigned char* slot = smem + NS * STAGE_BYTES + (kt % (NS + 1)) * RING_SLOT;
             float xs[TM];
+            // (fp8 x packed int4: the weights went in as (w + 8) / 512, so a product sum is 512 part - 8 rowsum(x); with
+            // xs' = 512 xs and xoff = -8 rowsum xs a fold is two fused multiply-adds per element: ws (xs' part + xoff))
+            [[maybe_unused]] float xoff[TM];
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i) {
               xs[i] = *reinterpret_cast<const float*>(slot + BN * 4 + 4 * (row_block(i) * 32 + (lane & 31)));
+              if constexpr (I4F) {
+                xoff[i] = -8.f * xs[i] * *reinterpret_cast<const float*>(slot + (BN + BM) * 4 + 4 * (row_block(i) * 32 + (lane & 31)));
+                xs[i] *= 512.f;
+              }
+            }
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -1244,7 +1261,8 @@ struct GemmKernel {
                     for (int e = 0; e < 4; ++e) {
                       float part = pacc[i][j][4 * t + e];
                       if constexpr (EC == kEI8) part = (float)__builtin_bit_cast(int, part);  // int32 partial sums
-                      acc[i][j][4 * t + e] += part * (xs[i] * wsc[e]);
+                      if constexpr (I4F) acc[i][j][4 * t + e] = fmaf(wsc[e], fmaf(xs[i], part, xoff[i]), acc[i][j][4 * t + e]);
+                      else acc[i][j][4 * t + e] += part * (xs[i] * wsc[e]);
                     }
                   }
               }

@@ -16,6 +16,8 @@ namespace tkx {
 // MFMAs column block by column block and keeps one set of converted rhs fragments (GemmKernel::JOUT).
 #define F8FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEF8, kEI4, BM, BN, BK, WM, WN, NS)
 #define F8GLU(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdGlu, kEF8, kEI4, BM, BN, BK, WM, WN, NS)
+// Scales per k-block on both sides (and row sums per 128-deep k-step): every k-step's products are folded in with them.
+#define F8SUBK(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdSubK, kEF8, kEI4, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
     FWD(256, 256, 64, 2, 4, 2),
@@ -43,6 +45,10 @@ static const Variant kVariants[] = {
     F8GLU(128, 256, 128, 2, 4, 3),
     F8GLU(64, 256, 128, 2, 4, 3),
     F8GLU(32, 256, 128, 1, 4, 4),
+    F8SUBK(128, 256, 128, 2, 4, 3),
+    F8SUBK(128, 256, 128, 1, 8, 3),
+    F8SUBK(64, 256, 128, 2, 2, 3),
+    F8SUBK(32, 256, 128, 1, 4, 3),
     F8FWD(128, 256, 128, 2, 4, 3),
     F8FWD(128, 256, 128, 1, 8, 3),
     F8FWD(128, 256, 128, 1, 8, 4),

@@ -439,8 +439,8 @@ def _route(lhs, rhs, *, dims, precision, rhs_scale, fuse_gateup_activation, pref
     k_blocks = rhs.scale.shape[1] > 1
     if isinstance(lhs, QArray):
       # fp8 activations with one scale per row: the kernels that feed the nibbles to the fp8 MFMAs.
-      return _Route(3 if gateup else 0, _per_row_lhs_scale(lhs), rhs, torch.float8_e4m3fn, torch.uint8, False, False,
-                    False, False, preferred_element_type)
+      return _Route(3 if gateup else 4 if k_blocks else 0, _per_row_lhs_scale(lhs), rhs, torch.float8_e4m3fn, torch.uint8,
+                    False, False, k_blocks, False, preferred_element_type)
     return _Route(3 if gateup else 4 if k_blocks else 0, lhs, rhs, torch.bfloat16, torch.uint8, False, False, k_blocks,
                   False, preferred_element_type)
   lhs_dt, rhs_dt = _dtype_of(lhs), _dtype_of(rhs)
@@ -485,9 +485,10 @@ def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True, gateup: bool = Fa
     (group, k-block, column) with blocks of a power of two >= 64 rows, or
   * the streaming small-m kernel: no bias and no gate-up fusion (`plain`), at most 8 rows per group on average,
     k % 1024 == 0, one scale per (group, column) or per (group, k-block, column) with blocks of a power of two >= 32 rows;
-  or under an lhs quantised to fp8 (e4m3fn) with one scale per row (or shared by runs of rows), one
-  scale per (group, column) and k % 128 == 0: the tiled kernels that feed the nibbles to the fp8 MFMAs
-  (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:258-300).
+  or under an lhs quantised to fp8 (e4m3fn) with one scale per row (or shared by runs of rows) and k % 128 == 0: the
+  tiled kernels that feed the nibbles to the fp8 MFMAs (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:258-300), with one
+  scale per (group, column), or, without gate-up fusion and with m % 4 == 0, per (group, k-block, column) with blocks
+  of a power of two >= 128 rows (the lhs scales then per row or per (row, same k-block)).
   Every other call gets the values unpacked to int8 storage first (then the int8 paths).
   Works on arrays and on shapes, so the forward pass and the choice of a config settle it alike."""
   if not (isinstance(rhs, QArray) and rhs.packed):
@@ -506,8 +507,10 @@ def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True, gateup: bool = Fa
   lhs_rows = _per_row_lhs_scale(lhs)
   fp8_tiles = (dims == base.DEFAULT_RAGGED_DOT_DIM_NUMS and isinstance(lhs_rows, QArray) and lhs_rows.zero_point is None
                and lhs_rows.qtype == torch.float8_e4m3fn and len(lhs_rows.qvalue.shape) == 2
-               and tuple(lhs_rows.scale.shape) == (lhs_rows.qvalue.shape[0], 1) and rhs.zero_point is None and n % 16 == 0
-               and blocks == 1 and k % _PACKED_INT4_FP8_TILE_STEP == 0)
+               and rhs.zero_point is None and n % 16 == 0 and k % _PACKED_INT4_FP8_TILE_STEP == 0 and blocks is not None
+               and tuple(lhs_rows.scale.shape) in ((lhs_rows.qvalue.shape[0], 1), (lhs_rows.qvalue.shape[0], blocks))
+               and (blocks == 1 or (scale_ok and not gateup and rows % _PACKED_INT4_FP8_TILE_STEP == 0
+                                    and lhs_rows.qvalue.shape[0] % 4 == 0)))
   return rhs if streams or tiles or fp8_tiles else rhs.unpacked()
 
 

@@ -9,6 +9,7 @@ import contextlib
 import ctypes
 import dataclasses
 import functools
+import math
 import threading
 
 import torch
@@ -241,16 +242,27 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
   if lhs.dtype == torch.float8_e4m3fn and rhs.dtype == torch.uint8:
     # The kernel takes the weights' +8 bias off with the row sums of the fp8 activations, which lie behind the row
     # scales: f32 [2, m]. A caller that holds both already passes them in that form.
+    # With rhs scales per k-block: [blocks + k / 128, m], the lhs scales per k-block and the row sums per 128 columns.
     if lhs_scale is None:
       raise NotImplementedError("fp8 activations over packed int4 weights need one lhs scale per row")
-    if tuple(lhs_scale.shape) != (2, m):
-      if lhs_scale.numel() != m:
-        raise NotImplementedError("fp8 activations over packed int4 weights: lhs scale [m] / [m, 1], or [2, m] with the row sums")
-      both = torch.empty((2, m), dtype=torch.float32, device=lhs.device)
-      both[0].copy_(lhs_scale.reshape(-1))
-      row_sums_fp8(lhs, out=both[1])
+    blocks = int(rhs_scale.shape[1]) if rhs_scale is not None and rhs_scale.dim() == 3 else 1
+    sum_rows = 1 if blocks == 1 else k // 128
+    if tuple(lhs_scale.shape) != (blocks + sum_rows, m):
+      if lhs_scale.numel() == m:
+        per_block = lhs_scale.reshape(1, m).expand(blocks, m)
+      elif tuple(lhs_scale.shape) == (m, blocks):
+        per_block = lhs_scale.t()
+      else:
+        raise NotImplementedError("fp8 activations over packed int4 weights: lhs scale [m] / [m, 1] / [m, k-blocks], or"
+                                  " [k-blocks + sum rows, m] with the row sums")
+      if blocks > 1 and k % 128:
+        raise NotImplementedError("scale blocks along k need k % 128 == 0 here")
+      both = torch.empty((blocks + sum_rows, m), dtype=torch.float32, device=lhs.device)
+      both[:blocks].copy_(per_block)
+      row_sums_fp8(lhs, out=both[blocks:], per_128_columns=blocks > 1)
       lhs_scale = both
     lhs_scale = lhs_scale.to(torch.float32).contiguous().view(-1)
+    lhs_scale_blocks = blocks
   elif lhs_scale is not None:
     if lhs_scale.dim() == 2 and lhs_scale.shape[1] > 1:
       # One scale per (row, k-block): the kernels take them as [k-blocks, m].
@@ -421,23 +433,28 @@ def ragged_dot_fwd_fp8_out(lhs, rhs, group_sizes, *, config: KernelConfig, lhs_s
   return out, out_scale
 
 
-def row_sums_fp8(x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-  """f32 [rows]: the sums of the rows of an fp8 (e4m3fn) matrix [rows, cols], cols % 16 == 0. What the fp8 x
-  packed-int4 forward takes behind its row scales (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:436-470 packs the sum
-  of an activation row with its scale the same way)."""
+def row_sums_fp8(x: torch.Tensor, out: torch.Tensor | None = None, per_128_columns: bool = False) -> torch.Tensor:
+  """f32 [rows]: the sums of the rows of an fp8 (e4m3fn) matrix [rows, cols], cols % 16 == 0; `per_128_columns`
+  (cols % 128 == 0): f32 [cols / 128, rows], one sum per run of 128 columns. What the fp8 x packed-int4 forward takes
+  behind its row scales (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:436-470 packs the sum of an activation row, or of
+  each of its subchannels, with its scales the same way)."""
   _log_launch(None)
   _require_cuda(x)
   if x.dtype != torch.float8_e4m3fn or x.dim() != 2:
     raise ValueError(f"expected an fp8 (e4m3fn) matrix, got {x.dtype} {tuple(x.shape)}")
   x = x.contiguous()
+  if per_128_columns and x.shape[1] % 128:
+    raise NotImplementedError("sums per 128 columns need cols % 128 == 0")
+  shape = (x.shape[1] // 128, x.shape[0]) if per_128_columns else (x.shape[0],)
   if out is None:
-    out = torch.empty(x.shape[0], dtype=torch.float32, device=x.device)
-  if out.dtype != torch.float32 or out.numel() != x.shape[0] or not out.is_contiguous() or out.device != x.device:
-    raise ValueError("out must be a contiguous f32 tensor with one entry per row, on x's device")
-  if x.shape[0]:
+    out = torch.empty(shape, dtype=torch.float32, device=x.device)
+  if out.dtype != torch.float32 or out.numel() != math.prod(shape) or not out.is_contiguous() or out.device != x.device:
+    raise ValueError("out must be a contiguous f32 tensor with one entry per sum, on x's device")
+  if x.shape[0] and x.shape[1]:
     lib = _lib.load()
     with _on_device(x.device):
-      _lib.check(lib.tkx_row_sums_fp8(_ptr(x), _ptr(out), x.shape[0], x.shape[1], _stream(x.device)))
+      _lib.check(lib.tkx_row_sums_fp8(_ptr(x), _ptr(out), x.shape[0], x.shape[1], 128 if per_128_columns else x.shape[1],
+                                      _stream(x.device)))
   return out
 
 
