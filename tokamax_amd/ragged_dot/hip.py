@@ -902,8 +902,10 @@ class HipRaggedDot(base.RaggedDot):
       # ... unless so few tiles come of it that half the chip would idle: then the largest tile that gives every CU one.
       tiles = lambda bm, bn: (rows / bm + 0.88 * num_groups) * -(-cols // (bn // 2 if mode == 3 else bn))
       if tiles(want_m, want_n) < _COMPUTE_UNITS // 2:
-        want_m, want_n = next((t for t in ((256, 256), (128, 256), (128, 128), (64, 128)) if t[0] <= want_m
-                               and tiles(*t) >= _COMPUTE_UNITS), (32, 128))
+        # (gate-up fusion and scales per k-block have 256-column tiles only: of the shapes there are)
+        shapes = ((256, 256), (128, 256), (128, 128), (64, 128), (32, 128)) if mode == 0 else sorted(
+            {(v[0], v[1]) for v in usable if v[0] > 16}, key=lambda t: (-t[0] * t[1], -t[1]))
+        want_m, want_n = next((t for t in shapes[:-1] if t[0] <= want_m and tiles(*t) >= _COMPUTE_UNITS), shapes[-1])
     if mode == 0 and key[1] == _lib.TKX_F32:
       # f32 operands run on the f32 MFMAs at a sixteenth of the bf16 rate: loads never bound them, and the 32-row tile
       # (four of its workgroups share a CU) was the fastest of the three on every measured shape, 128 to 1400 rows
@@ -943,6 +945,10 @@ class HipRaggedDot(base.RaggedDot):
       # 2070-2270 TFLOP/s on one row of waves against 1660-2050 on two at the Mixtral shape; their 256-row tile exists
       # on two rows only)
       two_wave_rows = wm - 1 if converted or (key[1] == _lib.TKX_F8E4M3FN and key[2] == _lib.TKX_I4X2) else 0
+      if mode == 4 and key[1] == _lib.TKX_F8E4M3FN and contraction < 1280:
+        # (with scales per k-block and a contraction of a few k-steps the tile on two rows of waves was ahead on the
+        # three such shapes measured: by 1-2 % at k = 896 and 1152, by 63 % at k = 768 with 12288 columns)
+        two_wave_rows = 0
       # ... and among those, the variant whose LDS lets two of its workgroups share a CU (the library gives such a
       # kernel 128 registers: 8 waves on one row, at most 64 accumulators per lane)
       stage_bytes = (bm * 2 + bn * (0.5 if key[2] == _lib.TKX_I4X2 else 1.0)) * bk + (bn * 4 if mode == 4 else 0)
