@@ -271,7 +271,14 @@ def main():
     measure("deepseek_v3_prefill_int4_packed_weights",
             lambda: op(w.lhs, q4, group_sizes=gs, preferred_element_type=torch.bfloat16), w.flops,
             w.m * w.k * 2 + nonempty * w.k * w.n // 2 + w.m * w.n * 2, "hbm", "bf16", cfg4)
-    del w, q4
+    # ... and with the activations quantised to fp8 per row as well (the fp8 MFMAs on the nibbles; the call includes the
+    # pass that sums the activation rows)
+    lhs8 = tokamax_amd.QArray(*hip_ops.quantize(w.lhs, torch.float8_e4m3fn, (1, w.k)))
+    cfg48 = op.bind(lhs8, q4, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    measure("deepseek_v3_prefill_fp8_activations_int4_packed_weights",
+            lambda: op(lhs8, q4, group_sizes=gs, preferred_element_type=torch.bfloat16), w.flops,
+            w.m * w.k + nonempty * w.k * w.n // 2 + w.m * w.n * 2, "hbm", "fp8", cfg48)
+    del w, q4, lhs8
 
     # decode: 6 rotating copies of the weights defeat the 256 MB last-level cache ("cold"); the same
     # copy every launch is the "warm" figure.
