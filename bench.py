@@ -389,6 +389,16 @@ def main():
     measure("mixtral_prefill_int4_packed_weights_k_block_scales",
             lambda: op(w.lhs, q4k, group_sizes=gs, preferred_element_type=torch.bfloat16), w.flops,
             w.m * w.k * 2 + w.nonempty_groups * (w.k * w.n // 2 + (w.k // 128) * w.n * 4) + w.m * w.n * 2, "mfma", "bf16", cfg)
+    # int8 activations over the packed int4 weights: the int8 MFMAs on the nibbles, exact int32 sums
+    cfg = op.bind(a8, q4, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_prefill_int8_activations_int4_packed_weights",
+            lambda: op(a8, q4, group_sizes=gs, preferred_element_type=torch.bfloat16), w.flops,
+            w.m * w.k + w.nonempty_groups * w.k * w.n // 2 + w.m * w.n * 2, "mfma", "int8", cfg)
+    cfg = op.bind(a8, q4k, group_sizes=gs, preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_prefill_int8_activations_int4_packed_weights_k_block_scales",
+            lambda: op(a8, q4k, group_sizes=gs, preferred_element_type=torch.bfloat16), w.flops,
+            w.m * w.k + w.nonempty_groups * (w.k * w.n // 2 + (w.k // 128) * w.n * 4) + w.m * (w.k // 128) * 4 + w.m * w.n * 2,
+            "mfma", "int8", cfg)
     del w, q8, q8k, a8, q4, q4k
 
     w = workloads.make("vjp", device, seed=0)

@@ -54,8 +54,9 @@ enum TkxDtype {
                   [G, k/2, n] holds k = 2 kk in bits 0-3 and k = 2 kk + 1 in bits 4-7 (two's complement). Taken as the
                   rhs of a bf16 lhs in the default mode by the streaming small-m kernel (block_m == 16, block_n == 128)
                   and by tiled forward variants of their own (plain, gate-up fusion, scales per k-block; k % block_k
-                  == 0; listed by tkx_ragged_dot_variant), and as the rhs of an fp8 lhs by the plain and gate-up
-                  variants described at tkx_row_sums_fp8; tkx_unpack_int4 turns it into TKX_I8 for everything else. The reference defines no packed layout (its int4 is jnp.int4; its sm90 kernels
+                  == 0; listed by tkx_ragged_dot_variant), and as the rhs of an fp8 lhs by the variants described
+                  at tkx_row_sums_fp8 and of an int8 lhs by plain and per-k-block-scale variants (scales as for
+                  int8 x int8; pallas_mosaic_gpu_kernel_sm100_i8_quant.py:114-190); tkx_unpack_int4 turns it into TKX_I8 for everything else. The reference defines no packed layout (its int4 is jnp.int4; its sm90 kernels
                   read int4 weights in pallas_mosaic_gpu_kernel_sm90_quant.py:46-387). */
 };
 

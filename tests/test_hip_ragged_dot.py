@@ -396,10 +396,13 @@ def test_every_kernel_variant_through_c_abi(v, device):
   if v["mode"] == 4 and lt == torch.int8:  # int8 x int8 on the int8 MFMAs, scales per block of 64 k rows on both sides
     lhs = torch.tensor(rng.integers(-127, 128, (m, k)).astype(np.int8), device=device)
     rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+    if rt == torch.uint8:  # ... or int8 over int4 weights, two to a byte along k
+      rhs = torch.tensor(rng.integers(-8, 8, (G, k, n)).astype(np.int8), device=device)
     for blocks in (k // v["block_k"],):  # scale blocks of one k-step (128 or 64 rows); one block runs the mode-0 variants
       xs, ws_ = mk((m, blocks), 0.01).abs() + 0.005, mk((G, blocks, n), 0.01).abs() + 0.005
       bias = mk((G, 1, n), 0.5)
-      out = hip_ops.ragged_dot_fwd(lhs, rhs, gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs, rhs_scale=ws_, rhs_bias=bias)
+      stored = hip_ops.pack_int4(rhs) if rt == torch.uint8 else rhs
+      out = hip_ops.ragged_dot_fwd(lhs, stored, gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs, rhs_scale=ws_, rhs_bias=bias)
       lhs_f = O.dequantize(lhs.cpu().numpy().astype(np.float64), _np(xs))
       rhs_f = O.dequantize(rhs.cpu().numpy().astype(np.float64), _np(ws_))
       _check(out, O.ragged_dot_fused(lhs_f, rhs_f, gs, rhs_bias=_np(bias)), 1e-5)  # int32 sums are exact
@@ -431,12 +434,15 @@ def test_every_kernel_variant_through_c_abi(v, device):
     _check(out, _ref(lhs, dout, gs, O.RAGGED_CONTRACTING), TOL[lt])
     return
   lhs_scale = rhs_scale = None
-  if rt == torch.int8 and lt == torch.int8:  # int8 x int8, one scale per row and per (group, column)
+  if rt in (torch.int8, torch.uint8) and lt == torch.int8:  # int8 x int8 (or packed int4), one scale per row and per (group, column)
     lhs = torch.tensor(rng.integers(-127, 128, (m, k)).astype(np.int8), device=device)
-    rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
+    top = 127 if rt == torch.int8 else 7
+    rhs = torch.tensor(rng.integers(-top - 1, top + 1, (G, k, n)).astype(np.int8), device=device)
     lhs_scale, rhs_scale = mk((m, 1), 0.01).abs() + 0.005, mk((G, 1, n), 0.01).abs() + 0.005
     lhs_f = O.dequantize(lhs.cpu().numpy().astype(np.float64), _np(lhs_scale))
     rhs_f = O.dequantize(rhs.cpu().numpy().astype(np.float64), _np(rhs_scale))
+    if rt == torch.uint8:
+      rhs = hip_ops.pack_int4(rhs)
     tol = 1e-5  # the int32 sums are exact
   elif rt == torch.int8:
     rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
@@ -996,6 +1002,58 @@ def test_tiled_kernels_on_fp8_activations_and_packed_int4_weights(v, device):
   want_shard[lo:hi] = want[lo:hi] + np.repeat(_np(bias)[:, 0], gs[1:4], axis=0)
   _check(shard, want_shard, 5e-5)
   assert torch.count_nonzero(shard[:lo]) == 0 and torch.count_nonzero(shard[hi:]) == 0
+
+
+def _int8_over_packed_int4_cases():
+  return [pytest.param(v, id="mode{mode}-{block_m}x{block_n}x{block_k}-w{waves_m}x{waves_n}-s{num_stages}".format(**v))
+          for v in _lib.variants(0) if v["rhs_dtype"] == _lib.TKX_I4X2 and v["lhs_dtype"] == _lib.TKX_I8]
+
+
+@pytest.mark.parametrize("v", _int8_over_packed_int4_cases())
+def test_tiled_kernels_on_int8_activations_and_packed_int4_weights(v, device):
+  """The int8 MFMAs on int4 weights read two to a byte (a nibble at the top of its byte is 16 w; the factor goes out
+  where the exact int32 sums become floats; pallas_mosaic_gpu_kernel_sm100_i8_quant.py:114-190): against the oracle on
+  the dequantised operands and bit for bit against the int8 x int8 kernels on the unpacked values, with one scale per
+  row and per (group, column) or with scales per k-block on both sides; the two ends of the int4 range in whole
+  columns, ragged groups, an empty one, rows of no group, a ragged last column tile; the split last round; the public
+  op keeps the weights packed."""
+  rng = np.random.default_rng(v["block_m"] + v["num_stages"] + v["mode"])
+  G, k, n = 5, 5 * 128, 272
+  gs = np.array([3, 300, 0, 70, 131], np.int32)
+  m = int(gs.sum()) + 8
+  gst = torch.tensor(gs, device=device)
+  lhs = torch.tensor(rng.integers(-127, 128, (m, k)).astype(np.int8), device=device)
+  values = rng.integers(-8, 8, (G, k, n)).astype(np.int8)
+  values[0, :, 0], values[0, :, 1] = -8, 7
+  unpacked = torch.tensor(values, device=device)
+  packed = hip_ops.pack_int4(unpacked)
+  blocks = 1 if v["mode"] == 0 else 5
+  mk = lambda shape, std: torch.tensor(np.abs(rng.normal(0, std, shape)).astype(np.float32) + std / 4, device=device)
+  xs, ws_ = mk((m, blocks), 0.01), mk((G, blocks, n), 0.05)
+  cfg = hip_ops.KernelConfig(v["block_m"], v["block_n"], v["block_k"], v["waves_m"], v["waves_n"], v["num_stages"], grid_tile_width=2)
+  out = hip_ops.ragged_dot_fwd(lhs, packed, gst, config=cfg, out_dtype=torch.float32, lhs_scale=xs, rhs_scale=ws_)
+  lhs_f = O.dequantize(lhs.cpu().numpy().astype(np.float64), _np(xs))
+  want = O.ragged_dot(lhs_f, O.dequantize(values.astype(np.float64), _np(ws_)), gs, O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+  _check(out, want, 1e-5 if blocks > 1 else 1e-6)
+  assert torch.count_nonzero(out[int(gs.sum()):]) == 0
+  twin = next(x for x in _lib.variants(0) if x["lhs_dtype"] == x["rhs_dtype"] == _lib.TKX_I8 and x["mode"] == v["mode"]
+              and k // blocks % x["block_k"] == 0)
+  twin_cfg = hip_ops.KernelConfig(twin["block_m"], twin["block_n"], twin["block_k"], twin["waves_m"], twin["waves_n"], twin["num_stages"])
+  same = hip_ops.ragged_dot_fwd(lhs, unpacked, gst, config=twin_cfg, out_dtype=torch.float32, lhs_scale=xs, rhs_scale=ws_)
+  assert torch.equal(out, same)  # the same integers, and 16 s / 16 rounds like s
+  if v["mode"] == 0 and v["block_m"] >= 128:
+    split = hip_ops.ragged_dot_fwd(lhs, packed, gst, config=dataclasses.replace(cfg, split_k=3), out_dtype=torch.float32,
+                                   lhs_scale=xs, rhs_scale=ws_)
+    assert torch.equal(split, out)  # int32 sums do not depend on how they are grouped
+  with pytest.raises(NotImplementedError):
+    hip_ops.ragged_dot_fwd(lhs, packed, gst, config=cfg, out_dtype=torch.float32, rhs_scale=ws_)
+  # the public op: a QArray of int8 activations over the packed weights names this kind of kernel
+  int4 = getattr(torch, "int4", torch.int8)
+  q_lhs = tokamax_amd.QArray(lhs, xs)
+  q_rhs = tokamax_amd.pack_int4(tokamax_amd.QArray(unpacked, ws_, None, int4))
+  op = tokamax_amd.HipRaggedDot()
+  assert _lib_key(op, q_lhs, q_rhs, gst) == (v["mode"], _lib.TKX_I8, _lib.TKX_I4X2)
+  _check(op(q_lhs, q_rhs, group_sizes=gst, preferred_element_type=torch.float32), want, 1e-5)
 
 
 def test_public_op_on_fp8_activations_and_packed_int4_weights(device):
@@ -2295,11 +2353,13 @@ def test_timing_tool_collects_every_kind_of_problem(tmp_path, device):
   config among the timed ones."""
   from tokamax_amd.data.autotuning import tile_cost
   path = str(tmp_path / "timings.json")
-  kinds = ["", ",dlhs", ",drhs", ",int8", ",int4", ",fp8", ",fp8i4", ",fp8i4k", ",fp8i4glu", ",int8x8", ",glu", ",int8k", ",f32"]
+  kinds = ["", ",dlhs", ",drhs", ",int8", ",int4", ",fp8", ",fp8i4", ",fp8i4k", ",fp8i4glu", ",int8i4", ",int8i4k", ",int8x8", ",glu",
+           ",int8k", ",f32"]
   tile_cost.collect(["768,256,512,4" + k for k in kinds], 2, path=path)
   entries = tile_cost.load(path)
   assert len(entries) == len(kinds) and all(e["timings"] and e["timings"][0][7] > 0 for e in entries)
-  assert {e.get("rhs", "bf16") for e in entries} == {"bf16", "int8", "int4", "fp8", "fp8i4", "fp8i4k", "fp8i4glu", "int8x8", "glu", "int8k", "f32"}
-  assert sorted(e["mode"] for e in entries) == [0] * 11 + [1, 2]
+  assert {e.get("rhs", "bf16") for e in entries} == {"bf16", "int8", "int4", "fp8", "fp8i4", "fp8i4k", "fp8i4glu", "int8i4", "int8i4k",
+                                                     "int8x8", "glu", "int8k", "f32"}
+  assert sorted(e["mode"] for e in entries) == [0] * 13 + [1, 2]
   for e in entries:
     assert 1.0 <= tile_cost.heuristics_gap(e) < 3.0, e["shape"]

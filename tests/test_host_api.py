@@ -690,6 +690,12 @@ def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   assert route8(x8, packed, fuse_gateup_activation="silu") == (3, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
   assert route8(x8, blocks, fuse_gateup_activation="silu") == (3, _lib.TKX_BF16, _lib.TKX_BF16)
   assert route8(x8, packed.unpacked()) == (0, _lib.TKX_BF16, _lib.TKX_I8)
+  # int8 activations: the int8 MFMAs on the nibbles; the tile whose workgroups share a CU in pairs (two stages: 64 KB)
+  xi8 = tokamax_amd.QArray(ShapeDtype((4096, 1024), i8), ShapeDtype((4096, 1), f32))
+  assert route8(xi8, packed) == (0, _lib.TKX_I8, _lib.TKX_I4X2) and route8(xi8, blocks) == (4, _lib.TKX_I8, _lib.TKX_I4X2)
+  assert route8(xi8, packed, fuse_gateup_activation="silu")[2] != _lib.TKX_I4X2
+  c = op._get_heuristics_config(op.bind(xi8, wide, group_sizes=gs))
+  assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages) == (128, 256, 128, 1, 8, 2)
   x8_blocks = tokamax_amd.QArray(ShapeDtype((4096, 1024), f8), ShapeDtype((4096, 8), f32))
   assert route8(x8_blocks, packed)[1:] == (_lib.TKX_BF16, _lib.TKX_I8)
   # the key of an autotuning cache entry names the 4-bit type and comes back as the same abstract QArray
@@ -739,7 +745,7 @@ def test_tile_cost_model_picks_near_the_fastest_measured_variant():
   # the config the heuristics hand out for those problems (model, rules for the streaming kernel, split decision), and
   # for quantised operands and drhs, where rules on rows per group and on the fill of the chip choose the tile
   label = lambda e: "drhs" if e["mode"] == 2 else e.get("rhs", "bf16")
-  for kind, count, most in (("bf16", 122, 0.06), ("int8", 26, 0.08), ("int4", 26, 0.06), ("fp8", 26, 0.03), ("fp8i4", 43, 0.04), ("fp8i4k", 26, 0.02), ("fp8i4glu", 26, 0.05),
+  for kind, count, most in (("bf16", 122, 0.06), ("int8", 26, 0.08), ("int4", 26, 0.06), ("fp8", 26, 0.03), ("fp8i4", 43, 0.04), ("fp8i4k", 26, 0.02), ("fp8i4glu", 26, 0.05), ("int8i4", 26, 0.04), ("int8i4k", 26, 0.03),
                             ("int8x8", 12, 0.03), ("drhs", 26, 0.03), ("glu", 26, 0.06), ("int8k", 26, 0.04), ("f32", 12, 0.01)):
     some = [e for e in tile_cost.load() if label(e) == kind]
     mean, worst = tile_cost.summary([tile_cost.heuristics_gap(e) for e in some])

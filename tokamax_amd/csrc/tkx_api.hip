@@ -265,9 +265,10 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
   if (a16w8f && (rhs_scale == nullptr || dlhs))
     return set_error(TKX_ERR_UNSUPPORTED, "bf16 x fp8 weights: default mode with an rhs scale only");
   // int8 x int8 likewise (the int8 MFMA kernels fold both operands' scales in per k-block).
-  const bool a8w8 = lhs_dtype == TKX_I8 && rhs_dtype == TKX_I8;
-  if (a8w8 && (rhs_scale == nullptr || lhs_scale == nullptr || dlhs))
-    return set_error(TKX_ERR_UNSUPPORTED, "int8 x int8: default mode with lhs and rhs scales only");
+  const bool a8w8 = lhs_dtype == TKX_I8 && (rhs_dtype == TKX_I8 || rhs_dtype == TKX_I4X2);
+  if (a8w8 && (rhs_scale == nullptr || lhs_scale == nullptr || dlhs || (gateup && rhs_dtype == TKX_I4X2)))
+    return set_error(TKX_ERR_UNSUPPORTED, "int8 x int8 (or packed int4): default mode with lhs and rhs scales only; no"
+                                          " gate-up fusion over packed int4");
   const bool subk = rhs_scale != nullptr && (rhs_scale_blocks != 1 || a16w8f) && !dlhs && c.block_m != kDecodeBlockM;
   int32_t log2_block_rows = 0;
   if (subk && rhs_scale_blocks == 1) {

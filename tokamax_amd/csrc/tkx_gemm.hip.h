@@ -259,6 +259,19 @@ __device__ __forceinline__ i32x8 i4x32_to_biased_f8x32(i32x4 w) {
   return out;
 }
 
+// 16 packed int4 values of one column (8 bytes, byte r = contraction entries 2 r and 2 r + 1, low nibble first) as the
+// 16 int8 values 16 w in contraction order: each nibble at the top of a byte of its own.
+__device__ __forceinline__ i32x4 i4x16_to_i8x16_times16(i32x2 w) {
+  i32x4 out;
+#pragma unroll
+  for (int d = 0; d < 2; ++d) {
+    const unsigned lo = ((unsigned)w[d] << 4) & 0xF0F0F0F0u, hi = (unsigned)w[d] & 0xF0F0F0F0u;
+    out[2 * d] = (int)__builtin_amdgcn_perm(hi, lo, 0x05010400u);
+    out[2 * d + 1] = (int)__builtin_amdgcn_perm(hi, lo, 0x07030602u);
+  }
+  return out;
+}
+
 // Eight packed int4 values (see i4x8_to_bf16x8_times16) times one scale, rounded to bf16; `scale16` is the column's
 // scale for the current k-block divided by 16.
 __device__ __forceinline__ i32x4 i4x8_to_bf16x8_scaled(int w, float scale16) {
@@ -574,7 +587,8 @@ struct GemmKernel {
   // int8 x int8 runs the same way on the int8 MFMAs (int32 partial sums, exact), also with one block.
   static constexpr bool SUBP = SUBK && (EA == kEF8 || EA == kEI8);
   static_assert(!SUBK || ((EB == kEI8 || EB == kEF8 || EB == kEI4) &&
-                          (EA == kEBF16 || (SUBP && EB == EA) || (EA == kEF8 && EB == kEI4 && BK == 128)) && BN == 256),
+                          (EA == kEBF16 || (SUBP && EB == EA) || (EA == kEF8 && EB == kEI4 && BK == 128) ||
+                           (EA == kEI8 && EB == kEI4)) && BN == 256),
                 "per-k-block scales: bf16 lhs with int8, packed int4 or fp8 weights, fp8 x fp8, int8 x int8 or fp8 x packed int4"
                 " (whose row sums come per 128-deep k-step); one 1 KB scale row per k-step");
   static constexpr int BNO = GLU ? BN / 2 : BN;  // output columns of a tile
@@ -590,6 +604,10 @@ struct GemmKernel {
   // give sum(x u) / 512 and the epilogue takes 8 sum(x) off again: sum(x w) = 512 acc - 8 rowsum(x). The row sums
   // of x lie behind its m_ext row scales.
   static constexpr bool I4F = I4 && EA == kEF8;
+  // int8 activations (pallas_mosaic_gpu_kernel_sm100_i8_quant.py:114-190, int8 x int4 on the native int8 matrix
+  // instructions): a nibble moved to the top of its byte is the int8 value 16 w; the int32 sums are exact and the
+  // factor 16 is taken out where they become floats.
+  static constexpr bool I4I = I4 && EA == kEI8;
   static constexpr int EBS = I4 ? (int)kEI8 : EB;  // element kind of a B stage in LDS
   static constexpr int KA = Mma<EC>::KA;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
@@ -615,8 +633,9 @@ struct GemmKernel {
   static constexpr bool JOUT = LEAN && I4F && TN >= 2;
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
   static_assert(!SPLIT || (MODE == kFwd && EA == EB && BK % 2 == 0), "split pipeline: plain forward, operands of one type");
-  static_assert(!I4 || (((I4P && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK)) || (I4F && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK))) && !SPLIT),
-                "packed int4 weights: forward with bf16 or fp8 activations");
+  static_assert(!I4 || (((I4P && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK)) || (I4F && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK)) ||
+                        (I4I && (MODE == kFwd || MODE == kFwdSubK))) && !SPLIT),
+                "packed int4 weights: forward with bf16, fp8 or int8 activations");
   static constexpr int BKB = I4 ? BKC / 2 : BKC;  // rows of a B stage
   typedef TileStage<LA, EA, BM, BK, THREADS> StageA;
   typedef TileStage<LB, EBS, BN, BKB, THREADS> StageB;
@@ -629,7 +648,7 @@ struct GemmKernel {
   // fp8 x fp8: the scales of a k-step (BN weight-column scales, then BM lhs-row scales) are still needed when its
   // stage is already being refilled, so they live in a ring of NS + 1 slots behind the stages.
   // (fp8 x packed int4: behind them the BM row sums of the k-step's activations)
-  static constexpr int RING_SLOT = SUBP ? (BN + BM + (I4 ? BM : 0)) * 4 : 0;
+  static constexpr int RING_SLOT = SUBP ? (BN + BM + (I4F ? BM : 0)) * 4 : 0;
   static constexpr int SMEM_BYTES = SPLIT ? NS * StageA::BYTES + HB * StageB::BYTES : NS * STAGE_BYTES + (NS + 1) * RING_SLOT;
   // Workgroups the register budget is set for: two 4-wave workgroups share a CU when their LDS fits twice (256
   // registers per lane each); every other shape has the CU, and a SIMD's 512 registers per lane, to itself or to the
@@ -800,6 +819,14 @@ struct GemmKernel {
       const i32x2 hi = lds_read_tr8(stage + StageA::BYTES + mc_offset<StageB::ROW_BYTES, EBS>(krow + 8, col));
       return i32x4{lo[0], lo[1], hi[0], hi[1]};
     };
+    // (int8 activations over packed int4 weights) the 8 bytes that hold the 16 contraction entries of the lane's half
+    // of k-atom kk: packed rows 16 kk + 8 (lane / 32) .. + 7.
+    [[maybe_unused]] auto load_b_raw8 = [&](const unsigned char* stage, int j, int kk) -> i32x2 {
+      const int blk = lane >> 4, s_ = lane & 15;
+      const int col = wn * WTN + j * 32 + 16 * (blk & 1) + 8 * (s_ & 1);
+      const int krow = kk * (KA / 2) + 8 * (blk >> 1) + (s_ >> 1);
+      return lds_read_tr8(stage + StageA::BYTES + mc_offset<StageB::ROW_BYTES, EBS>(krow, col));
+    };
     auto load_b_frag = [&](const unsigned char* stage, int j, int kk) -> Frag {
       if constexpr (SUBK && !SUBP) {
         const int blk = lane >> 4, s_ = lane & 15;
@@ -812,6 +839,8 @@ struct GemmKernel {
         else return f8x8_to_bf16x8_scaled(v, scale);
       } else if constexpr (I4F) {
         return i4x32_to_biased_f8x32(load_b_raw(stage, j, kk));
+      } else if constexpr (I4I) {
+        return i4x16_to_i8x16_times16(load_b_raw8(stage, j, kk));
       } else {
         return load_frag<LB, EBS, EC, StageB::ROW_BYTES>(stage + StageA::BYTES, wn * WTN + j * 32, kk, lane);
       }
@@ -1069,6 +1098,7 @@ struct GemmKernel {
         // of the second halves, A1, ...
         [[maybe_unused]] i32x2 raw[I4P ? TN : 1];
         [[maybe_unused]] i32x4 rawf[I4F ? TN : 1];  // (fp8 activations) a fragment's bytes as read
+        [[maybe_unused]] i32x2 rawi[I4I ? TN : 1];  // (int8 activations) likewise
         // (kFwdSubK: times the scale of the lane's column for the stage's k-block, like load_b_frag)
         [[maybe_unused]] auto convert_i4 = [&](int w, const unsigned char* stage, int j) -> i32x4 {
           if constexpr (SUBK) {
@@ -1088,6 +1118,8 @@ struct GemmKernel {
           } else if (f < TM + TN) {
             if constexpr (I4F) {
               if (NV > 0) rawf[f - TM] = load_b_raw(stage, f - TM, kk);
+            } else if constexpr (I4I) {
+              if (NV > 0) rawi[f - TM] = load_b_raw8(stage, f - TM, kk);
             } else if constexpr (I4P) {
               const int j = f - TM;
               if (NV > 0) {
@@ -1105,6 +1137,8 @@ struct GemmKernel {
             }
           } else if constexpr (I4F) {
             if (NV > 0) b[f - TM - TN] = i4x32_to_biased_f8x32(rawf[f - TM - TN]);
+          } else if constexpr (I4I) {
+            if (NV > 0) b[f - TM - TN] = i4x16_to_i8x16_times16(rawi[f - TM - TN]);
           } else if constexpr (I4P) {
             if (NV > 0 && !(kk & 1)) b[f - TM - TN] = convert_i4(raw[f - TM - TN][0], stage, f - TM - TN);
           }
@@ -1244,6 +1278,7 @@ struct GemmKernel {
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
               xs[i] = *reinterpret_cast<const float*>(slot + BN * 4 + 4 * (row_block(i) * 32 + (lane & 31)));
+              if constexpr (I4I) xs[i] *= kPackedInt4Unscale;  // (the weights went into the MFMAs times 16)
               if constexpr (I4F) {
                 xoff[i] = -8.f * xs[i] * *reinterpret_cast<const float*>(slot + (BN + BM) * 4 + 4 * (row_block(i) * 32 + (lane & 31)));
                 xs[i] *= 512.f;
@@ -1405,7 +1440,7 @@ struct GemmKernel {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
               const float bits = acc[i][j][e];  // (a scalar copy first: a bit cast straight from a vector element misreads)
-              acc[i][j][e] = (float)__builtin_bit_cast(int, bits);
+              acc[i][j][e] = (float)__builtin_bit_cast(int, bits) * (I4I ? kPackedInt4Unscale : 1.f);
             }
       }
       const bool inside = col0 + BNO <= p.n_ext;

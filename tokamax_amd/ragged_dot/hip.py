@@ -438,8 +438,9 @@ def _route(lhs, rhs, *, dims, precision, rhs_scale, fuse_gateup_activation, pref
       preferred_element_type = torch.promote_types(lhs.dtype, rhs.dtype)
     k_blocks = rhs.scale.shape[1] > 1
     if isinstance(lhs, QArray):
-      # fp8 activations with one scale per row: the kernels that feed the nibbles to the fp8 MFMAs.
-      return _Route(3 if gateup else 4 if k_blocks else 0, _per_row_lhs_scale(lhs), rhs, torch.float8_e4m3fn, torch.uint8,
+      # fp8 or int8 activations with one scale per row: the kernels that feed the nibbles to the fp8 / int8 MFMAs.
+      lhs_dt = torch.int8 if _dtype_of(lhs) == torch.int8 else torch.float8_e4m3fn
+      return _Route(3 if gateup else 4 if k_blocks else 0, _per_row_lhs_scale(lhs), rhs, lhs_dt, torch.uint8,
                     False, False, k_blocks, False, preferred_element_type)
     return _Route(3 if gateup else 4 if k_blocks else 0, lhs, rhs, torch.bfloat16, torch.uint8, False, False, k_blocks,
                   False, preferred_element_type)
@@ -511,7 +512,15 @@ def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True, gateup: bool = Fa
                and tuple(lhs_rows.scale.shape) in ((lhs_rows.qvalue.shape[0], 1), (lhs_rows.qvalue.shape[0], blocks))
                and (blocks == 1 or (scale_ok and not gateup and rows % _PACKED_INT4_FP8_TILE_STEP == 0
                                     and lhs_rows.qvalue.shape[0] % 4 == 0)))
-  return rhs if streams or tiles or fp8_tiles else rhs.unpacked()
+  # ... or quantised to int8 likewise: the int8 MFMAs on the nibbles (pallas_mosaic_gpu_kernel_sm100_i8_quant.py:
+  # 114-190), no gate-up fusion; scale blocks of a power of two >= 64 rows.
+  int8_tiles = (dims == base.DEFAULT_RAGGED_DOT_DIM_NUMS and isinstance(lhs_rows, QArray) and lhs_rows.zero_point is None
+                and _dtype_of(lhs_rows) == torch.int8 and lhs_rows.qvalue.dtype == torch.int8
+                and len(lhs_rows.qvalue.shape) == 2 and rhs.zero_point is None and n % 16 == 0 and not gateup
+                and k % _PACKED_INT4_FP8_TILE_STEP == 0 and blocks is not None
+                and tuple(lhs_rows.scale.shape) in ((lhs_rows.qvalue.shape[0], 1), (lhs_rows.qvalue.shape[0], blocks))
+                and (blocks == 1 or (scale_ok and rows % _PACKED_INT4_TILE_STEP == 0 and lhs_rows.qvalue.shape[0] % 4 == 0)))
+  return rhs if streams or tiles or fp8_tiles or int8_tiles else rhs.unpacked()
 
 
 def _abstract_operand(x):
@@ -886,7 +895,10 @@ class HipRaggedDot(base.RaggedDot):
     # row of waves is small enough for two workgroups to share a CU (64 KB of LDS with two stages of int8 weights, 72 KB
     # with three of int4; 128 registers) and was the fastest or within a few percent of it from 12 rows per group up to
     # 2048 (43 measured shapes per kind).
-    converted_plain = mode == 0 and key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2)
+    # (int8 activations over packed int4 weights likewise: 128 x 256 x 128 with two stages is 64 KB and 128 registers,
+    # and the fastest on 22 of 26 measured shapes)
+    int8_int4 = key[1] == _lib.TKX_I8 and key[2] == _lib.TKX_I4X2
+    converted_plain = mode == 0 and ((key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2)) or int8_int4)
     if mode in (0, 3, 4) and key[1] != _lib.TKX_F32 and rows_per_group >= (12 if converted_plain else 96):
       # The forward kernels other than f32 (16-bit operands without scales are re-ranked by the cost model below): the
       # taller and wider tile pays off earlier than the thresholds above say. Measured on 14 shapes per kind (int8 and
@@ -894,7 +906,7 @@ class HipRaggedDot(base.RaggedDot):
       # rows per group, the 128-row one from about 100, and 256 columns from a few tiles' worth of them.
       want_m = 256 if rows_per_group >= 224 else 128
       want_n = 256 if cols >= 512 else 128
-      if key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2, _lib.TKX_F8E4M3FN):
+      if (key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2, _lib.TKX_F8E4M3FN)) or int8_int4:
         # (also with gate-up fusion, where the tile sits on one row of four waves, likewise two per CU: 6 % ahead of the
         # 256-row tile at the Mixtral shape and 16-31 % at 128 rows per group; and with scales per k-block: 8-13 %
         # ahead at 128-256 rows per group, even at the Mixtral shape)
@@ -944,17 +956,18 @@ class HipRaggedDot(base.RaggedDot):
       # (fp8 activations over packed int4 weights turn nibbles into fp8 bytes the same way: the 128-row tile runs at
       # 2070-2270 TFLOP/s on one row of waves against 1660-2050 on two at the Mixtral shape; their 256-row tile exists
       # on two rows only)
-      two_wave_rows = wm - 1 if converted or (key[1] == _lib.TKX_F8E4M3FN and key[2] == _lib.TKX_I4X2) else 0
+      two_wave_rows = wm - 1 if converted or int8_int4 or (key[1] == _lib.TKX_F8E4M3FN and key[2] == _lib.TKX_I4X2) else 0
       if mode == 4 and key[1] == _lib.TKX_F8E4M3FN and contraction < 1280:
         # (with scales per k-block and a contraction of a few k-steps the tile on two rows of waves was ahead on the
         # three such shapes measured: by 1-2 % at k = 896 and 1152, by 63 % at k = 768 with 12288 columns)
         two_wave_rows = 0
       # ... and among those, the variant whose LDS lets two of its workgroups share a CU (the library gives such a
       # kernel 128 registers: 8 waves on one row, at most 64 accumulators per lane)
-      stage_bytes = (bm * 2 + bn * (0.5 if key[2] == _lib.TKX_I4X2 else 1.0)) * bk + (bn * 4 if mode == 4 else 0)
-      alone_on_cu = 0 if (converted and wm == 1 and wn == 8 and bm * bn <= 128 * 256
+      stage_bytes = ((bm * (1 if int8_int4 else 2) + bn * (0.5 if key[2] == _lib.TKX_I4X2 else 1.0)) * bk
+                     + (bn * 4 if mode == 4 else 0))
+      alone_on_cu = 0 if ((converted or (int8_int4 and mode == 0)) and wm == 1 and wn == 8 and bm * bn <= 128 * 256
                           and 2 * ns * stage_bytes <= 160 * 1024) else 1
-      return (abs(bm - want_m), abs(bn - want_n), two_wave_rows, -(wm * wn), alone_on_cu if converted else 0, -in_flight,
+      return (abs(bm - want_m), abs(bn - want_n), two_wave_rows, -(wm * wn), alone_on_cu if converted or int8_int4 else 0, -in_flight,
               bk if short_k else -bk, ns)
 
     bm, bn, bk, wm, wn, ns = min(usable, key=score)
@@ -994,6 +1007,8 @@ class HipRaggedDot(base.RaggedDot):
       if key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2, _lib.TKX_F8E4M3FN) and wm == 1 and wn == 8:
         stage = (bm * 2 + bn * rb) * bk + (bn * 4 if mode == 4 else 0)
         shares = bm * bn <= 128 * 256 and 2 * ns * stage <= 160 * 1024
+      if int8_int4 and mode == 0 and wm == 1 and wn == 8:
+        shares = bm * bn <= 128 * 256 and 2 * ns * (bm + bn * 0.5) * bk <= 160 * 1024
       estimate = lambda sk: _tile_cost(v, sk, rows, cols, contraction // narrow, num_groups, mode,
                                        rhs_bytes=2.0 if narrow == 2 else rb, shares_cu=shares)
       if key[1] == _lib.TKX_F32 or estimate(4) < estimate(1):

@@ -281,6 +281,10 @@ def ragged_dot_fwd(lhs, rhs, group_sizes, *, config: KernelConfig, out_dtype: to
       raise NotImplementedError("rhs scale must be one f32 per (group, column) or per (group, k-block, column)")
   if lhs_scale_blocks != 1 and lhs_scale_blocks != scale_blocks:
     raise NotImplementedError("lhs and rhs scales must have the same number of blocks along k")
+  if (lhs_scale is not None and lhs_scale_blocks == 1 and scale_blocks > 1 and config.block_m != 16
+      and lhs.dtype in (torch.int8, torch.float8_e4m3fn)):
+    # The kernels that fold both operands' scales in per k-block read the lhs scales as [k-blocks, m].
+    lhs_scale = lhs_scale.view(1, m).expand(scale_blocks, m).contiguous().view(-1)
   if rhs_bias is not None:
     rhs_bias = rhs_bias.to(torch.float32).contiguous().view(-1)
     if rhs_bias.numel() != G * n:
