@@ -73,7 +73,12 @@ def bound_arguments(op, device):
       (torch.rand(w.num_groups, 1, w.n, device=device, generator=gen) + 0.5) / (7 * w.k ** 0.5), None,
       getattr(torch, "int4", torch.int8)))
   yield "mixtral int4 packed weights", op.bind(w.lhs, q4, group_sizes=gs, preferred_element_type=torch.bfloat16)
-  del w, q8, a8, q4
+  # ... and quantised activations over them: the int8 and fp8 MFMAs on the nibbles
+  yield "mixtral int8 x int4 packed", op.bind(a8, q4, group_sizes=gs, preferred_element_type=torch.bfloat16)
+  from tokamax_amd.ragged_dot import hip_ops  # pylint: disable=g-import-not-at-top
+  f8 = tokamax_amd.QArray(*hip_ops.quantize(w.lhs, torch.float8_e4m3fn, (1, w.k)))
+  yield "mixtral fp8 x int4 packed", op.bind(f8, q4, group_sizes=gs, preferred_element_type=torch.bfloat16)
+  del w, q8, a8, q4, f8
   # The reference's own benchmark list (tokamax/_src/ops/ragged_dot/arg_specs.py): its "primary" shapes.
   for spec in arg_specs.ARG_SPECS:
     if "primary" not in spec.tags:
