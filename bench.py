@@ -441,7 +441,13 @@ def main():
     measure("mixtral_gateup_silu_fp8_activations_int4_packed_weights",
             lambda: op(lhs8, q4g, group_sizes=gs, fuse_gateup_activation="silu", preferred_element_type=torch.bfloat16),
             2 * m_ * k_ * 2 * n_, m_ * k_ + m_ * n_ * 2 + 8 * k_ * n_, "mfma", "fp8", cfg48)
-    del q4g, lhs8
+    # ... or to int8: the int8 MFMAs
+    lhsi8 = tokamax_amd.QArray(*_ops.quantize(lhs, torch.int8, (1, k_)))
+    cfg4i = op.bind(lhsi8, q4g, group_sizes=gs, fuse_gateup_activation="silu", preferred_element_type=torch.bfloat16).default_config
+    measure("mixtral_gateup_silu_int8_activations_int4_packed_weights",
+            lambda: op(lhsi8, q4g, group_sizes=gs, fuse_gateup_activation="silu", preferred_element_type=torch.bfloat16),
+            2 * m_ * k_ * 2 * n_, m_ * k_ + m_ * n_ * 2 + 8 * k_ * n_, "mfma", "int8", cfg4i)
+    del q4g, lhs8, lhsi8
     # The whole expert FFN of a Mixtral layer around those two products, as a caller strings it together: tokens
     # permuted into expert order (ragged_gather), gate-up product with silu(gate) * up in the epilogue, down
     # projection, weighted top-2 combine back into token order (ragged_gather_reduce). 8192 tokens, top 2 of 8 experts.

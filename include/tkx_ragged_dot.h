@@ -215,7 +215,7 @@ int32_t tkx_ragged_dot_fwd_static_workspace(const void* lhs, const void* rhs, co
  *   rhs_bias: f32[G,n] added to the scaled accumulator, or NULL.
  *   gateup = 1: rhs is [G,k,n] with its columns [gate | up] (n/2 each) and out is [m, n/2] =
  *     act(lhs.gate + bias_gate) * (lhs.up + bias_up), `activation` naming act (NONE: the plain product); needs
- *     n % 16 == 0, k % block_k == 0 and a variant of mode 3 (see tkx_ragged_dot_variant; bf16 x bf16 and
+ *     n % 16 == 0 (one-byte weights: n % 32 == 0, so that the up half starts on a 16-byte piece), k % block_k == 0 and a variant of mode 3 (see tkx_ragged_dot_variant; bf16 x bf16 and
  *     bf16 x int8 with one scale per (group, column)).
  *   gateup = 0: as tkx_ragged_dot_fwd plus the bias; `activation` applies to the biased result
  *   (TKX_ACT_SWIGLU_OAI and TKX_ACT_SILU_CLAMP need gateup = 1: TKX_ERR_INVALID otherwise).

@@ -359,6 +359,10 @@ def test_every_kernel_variant_through_c_abi(v, device):
     if lt == torch.float8_e4m3fn:  # (over packed int4 weights) one scale per row
       lhs_scale = mk((m, 1), 0.1).abs() + 0.05
       lhs_f = lhs_f * _np(lhs_scale)
+    if lt == torch.int8:  # (likewise)
+      lhs = torch.tensor(rng.integers(-127, 128, (m, k)).astype(np.int8), device=device)
+      lhs_scale = mk((m, 1), 0.01).abs() + 0.005
+      lhs_f = _np(lhs) * _np(lhs_scale)
     if rt == torch.int8:  # int8 weights with one scale per (group, column)
       rhs = torch.tensor(rng.integers(-127, 128, (G, k, n)).astype(np.int8), device=device)
       scale = mk((G, 1, n), 0.005).abs() + 1e-3
@@ -1004,9 +1008,41 @@ def test_tiled_kernels_on_fp8_activations_and_packed_int4_weights(v, device):
   assert torch.count_nonzero(shard[:lo]) == 0 and torch.count_nonzero(shard[hi:]) == 0
 
 
+def test_gateup_over_one_byte_weights_whose_halves_are_not_whole_16_byte_pieces(device):
+  """Gate-up fusion reads the up half of a weight row n / 2 elements in. With one-byte weights that is a whole 16-byte
+  piece only if n % 32 == 0: the library declines other widths, and the op widens such weights to bf16 first (int8
+  weights and packed int4 ones alike) instead of reading up columns from the wrong place."""
+  rng = np.random.default_rng(77)
+  G, k, n, rows = 3, 256, 272, 96
+  m = G * rows
+  gs = torch.full((G,), rows, dtype=torch.int32, device=device)
+  lhs = torch.tensor(rng.normal(0, 1, (m, k)).astype(np.float32), device=device).to(torch.bfloat16)
+  q = torch.tensor(rng.integers(-8, 8, (G, k, n)).astype(np.int8), device=device)
+  scale = torch.tensor((rng.uniform(0.5, 1.5, (G, 1, n)) * 0.02).astype(np.float32), device=device)
+  want = O.ragged_dot_fused(_np(lhs), O.dequantize(q.cpu().numpy(), _np(scale)), np.full(G, rows, np.int32), gateup_activation="silu")
+  op = tokamax_amd.HipRaggedDot()
+  int4 = getattr(torch, "int4", torch.int8)
+  for rhs in (tokamax_amd.QArray(q, scale), tokamax_amd.pack_int4(tokamax_amd.QArray(q, scale, None, int4))):
+    bound = op.bind(lhs, rhs, group_sizes=gs, preferred_element_type=torch.float32, fuse_gateup_activation="silu")
+    assert op._problem(bound)[1] == (3, _lib.TKX_BF16, _lib.TKX_BF16)
+    out = op(lhs, rhs, group_sizes=gs, preferred_element_type=torch.float32, fuse_gateup_activation="silu")
+    assert tuple(out.shape) == (m, n // 2)
+    _check(out, want, 5e-3)  # (weights times scales rounded to bf16)
+  cfg = hip_ops.KernelConfig(128, 256, 64, 2, 4, 3)
+  with pytest.raises(NotImplementedError, match="n % 32"):
+    hip_ops.ragged_dot_fwd(lhs, q, gs, config=cfg, out_dtype=torch.float32, rhs_scale=scale, gateup=True, activation="silu")
+  # 256 columns: the int8 weights are read as they are
+  narrow = tokamax_amd.QArray(q[:, :, :256].contiguous(), scale[:, :, :256].contiguous())
+  bound = op.bind(lhs, narrow, group_sizes=gs, preferred_element_type=torch.float32, fuse_gateup_activation="silu")
+  assert op._problem(bound)[1] == (3, _lib.TKX_BF16, _lib.TKX_I8)
+  out = op(lhs, narrow, group_sizes=gs, preferred_element_type=torch.float32, fuse_gateup_activation="silu")
+  _check(out, O.ragged_dot_fused(_np(lhs), O.dequantize(q[:, :, :256].cpu().numpy(), _np(scale[:, :, :256])),
+                                 np.full(G, rows, np.int32), gateup_activation="silu"), 1e-5)
+
+
 def _int8_over_packed_int4_cases():
   return [pytest.param(v, id="mode{mode}-{block_m}x{block_n}x{block_k}-w{waves_m}x{waves_n}-s{num_stages}".format(**v))
-          for v in _lib.variants(0) if v["rhs_dtype"] == _lib.TKX_I4X2 and v["lhs_dtype"] == _lib.TKX_I8]
+          for v in _lib.variants(0) if v["rhs_dtype"] == _lib.TKX_I4X2 and v["lhs_dtype"] == _lib.TKX_I8 and v["mode"] in (0, 4)]
 
 
 @pytest.mark.parametrize("v", _int8_over_packed_int4_cases())
@@ -1054,6 +1090,23 @@ def test_tiled_kernels_on_int8_activations_and_packed_int4_weights(v, device):
   op = tokamax_amd.HipRaggedDot()
   assert _lib_key(op, q_lhs, q_rhs, gst) == (v["mode"], _lib.TKX_I8, _lib.TKX_I4X2)
   _check(op(q_lhs, q_rhs, group_sizes=gst, preferred_element_type=torch.float32), want, 1e-5)
+  if v["mode"] == 0 and v["block_m"] == 256:
+    # gate-up fusion over the same weights read as [gate | up]: kernels of the same kind
+    # (each half of a weight row must be whole 16-byte pieces, 16 columns of one-byte storage: with n = 272 the
+    # operands are widened to bf16 instead, with n = 256 the weights stay packed)
+    wide = op.bind(q_lhs, q_rhs, group_sizes=gst, preferred_element_type=torch.float32, fuse_gateup_activation="silu")
+    assert op._problem(wide)[1] == (3, _lib.TKX_BF16, _lib.TKX_BF16)
+    fused = op(q_lhs, q_rhs, group_sizes=gst, preferred_element_type=torch.float32, fuse_gateup_activation="silu")
+    _check(fused, O.ragged_dot_fused(lhs_f, O.dequantize(values.astype(np.float64), _np(ws_)), gs, gateup_activation="silu"), 1e-2)
+    with pytest.raises(NotImplementedError, match="n % 32"):
+      hip_ops.ragged_dot_fwd(lhs, packed, gst, config=hip_ops.KernelConfig(256, 256, 128, 2, 4, 3), out_dtype=torch.float32,
+                             lhs_scale=xs, rhs_scale=ws_, gateup=True, activation="silu")
+    q_256 = tokamax_amd.pack_int4(tokamax_amd.QArray(unpacked[:, :, :256].contiguous(), ws_[:, :, :256].contiguous(), None, int4))
+    bound = op.bind(q_lhs, q_256, group_sizes=gst, preferred_element_type=torch.float32, fuse_gateup_activation="silu")
+    assert op._problem(bound)[1] == (3, _lib.TKX_I8, _lib.TKX_I4X2)
+    fused = op(q_lhs, q_256, group_sizes=gst, preferred_element_type=torch.float32, fuse_gateup_activation="silu")
+    _check(fused, O.ragged_dot_fused(lhs_f, O.dequantize(values[:, :, :256].astype(np.float64), _np(ws_[:, :, :256])), gs,
+                                     gateup_activation="silu"), 1e-5)
 
 
 def test_public_op_on_fp8_activations_and_packed_int4_weights(device):

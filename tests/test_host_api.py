@@ -693,7 +693,8 @@ def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   # int8 activations: the int8 MFMAs on the nibbles; the tile whose workgroups share a CU in pairs (two stages: 64 KB)
   xi8 = tokamax_amd.QArray(ShapeDtype((4096, 1024), i8), ShapeDtype((4096, 1), f32))
   assert route8(xi8, packed) == (0, _lib.TKX_I8, _lib.TKX_I4X2) and route8(xi8, blocks) == (4, _lib.TKX_I8, _lib.TKX_I4X2)
-  assert route8(xi8, packed, fuse_gateup_activation="silu")[2] != _lib.TKX_I4X2
+  assert route8(xi8, packed, fuse_gateup_activation="silu") == (3, _lib.TKX_I8, _lib.TKX_I4X2)
+  assert route8(xi8, blocks, fuse_gateup_activation="silu")[2] != _lib.TKX_I4X2
   c = op._get_heuristics_config(op.bind(xi8, wide, group_sizes=gs))
   assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages) == (128, 256, 128, 1, 8, 2)
   x8_blocks = tokamax_amd.QArray(ShapeDtype((4096, 1024), f8), ShapeDtype((4096, 8), f32))

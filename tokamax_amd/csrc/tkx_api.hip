@@ -257,6 +257,9 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
   if (gateup && (n % 16 != 0 || k % c.block_k != 0))
     return set_error(TKX_ERR_UNSUPPORTED, "gate-up fusion needs n %% 16 == 0 and k %% block_k == 0 (k=%lld n=%lld)",
                      (long long)k, (long long)n);
+  // (the up half of a weight row starts n / 2 elements in: whole 16-byte pieces of one-byte weights are 16 columns)
+  if (gateup && rhs_dtype != TKX_BF16 && rhs_dtype != TKX_F16 && rhs_dtype != TKX_F32 && (n / 2) % 16 != 0)
+    return set_error(TKX_ERR_UNSUPPORTED, "gate-up fusion over one-byte weights needs n %% 32 == 0 (n=%lld)", (long long)n);
   if (rhs_bias && (uintptr_t)rhs_bias % 16 != 0) return set_error(TKX_ERR_UNSUPPORTED, "pointers must be 16-byte aligned");
   // Scales that change along k: the streaming small-m kernel (block_m == 16) takes them itself; the tiled
   // kernels have variants of their own (kFwdSubK) that carry the scale rows through LDS.
@@ -266,9 +269,8 @@ int32_t fwd_impl(const void* lhs, const void* rhs, const int32_t* group_sizes, c
     return set_error(TKX_ERR_UNSUPPORTED, "bf16 x fp8 weights: default mode with an rhs scale only");
   // int8 x int8 likewise (the int8 MFMA kernels fold both operands' scales in per k-block).
   const bool a8w8 = lhs_dtype == TKX_I8 && (rhs_dtype == TKX_I8 || rhs_dtype == TKX_I4X2);
-  if (a8w8 && (rhs_scale == nullptr || lhs_scale == nullptr || dlhs || (gateup && rhs_dtype == TKX_I4X2)))
-    return set_error(TKX_ERR_UNSUPPORTED, "int8 x int8 (or packed int4): default mode with lhs and rhs scales only; no"
-                                          " gate-up fusion over packed int4");
+  if (a8w8 && (rhs_scale == nullptr || lhs_scale == nullptr || dlhs))
+    return set_error(TKX_ERR_UNSUPPORTED, "int8 x int8 (or packed int4): default mode with lhs and rhs scales only");
   const bool subk = rhs_scale != nullptr && (rhs_scale_blocks != 1 || a16w8f) && !dlhs && c.block_m != kDecodeBlockM;
   int32_t log2_block_rows = 0;
   if (subk && rhs_scale_blocks == 1) {

@@ -634,7 +634,7 @@ struct GemmKernel {
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes an even number of k-atoms per step");
   static_assert(!SPLIT || (MODE == kFwd && EA == EB && BK % 2 == 0), "split pipeline: plain forward, operands of one type");
   static_assert(!I4 || (((I4P && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK)) || (I4F && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK)) ||
-                        (I4I && (MODE == kFwd || MODE == kFwdSubK))) && !SPLIT),
+                        (I4I && (MODE == kFwd || MODE == kFwdGlu || MODE == kFwdSubK))) && !SPLIT),
                 "packed int4 weights: forward with bf16, fp8 or int8 activations");
   static constexpr int BKB = I4 ? BKC / 2 : BKC;  // rows of a B stage
   typedef TileStage<LA, EA, BM, BK, THREADS> StageA;

@@ -23,6 +23,7 @@ namespace tkx {
 // both sides (the sums of a k-block are folded in at its end).
 #define I8FWD(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwd, kEI8, kEI4, BM, BN, BK, WM, WN, NS)
 #define I8SUBK(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdSubK, kEI8, kEI4, BM, BN, BK, WM, WN, NS)
+#define I8GLU(BM, BN, BK, WM, WN, NS) TKX_VARIANT(kFwdGlu, kEI8, kEI4, BM, BN, BK, WM, WN, NS)
 
 static const Variant kVariants[] = {
     FWD(256, 256, 64, 2, 4, 2),
@@ -60,6 +61,10 @@ static const Variant kVariants[] = {
     I8FWD(128, 256, 128, 1, 8, 2),
     I8FWD(64, 128, 128, 2, 2, 4),
     I8FWD(32, 128, 128, 1, 4, 4),
+    I8GLU(256, 256, 128, 2, 4, 3),
+    I8GLU(128, 256, 128, 2, 4, 3),
+    I8GLU(64, 256, 128, 2, 4, 3),
+    I8GLU(32, 256, 128, 1, 4, 4),
     I8SUBK(128, 256, 128, 2, 4, 3),
     I8SUBK(128, 256, 128, 1, 8, 3),
     I8SUBK(128, 256, 64, 2, 4, 4),

@@ -449,6 +449,12 @@ def _route(lhs, rhs, *, dims, precision, rhs_scale, fuse_gateup_activation, pref
   if mode == 0:
     lhs, rhs = _per_row_lhs_scale(lhs), _per_column_rhs_scale(rhs)
     widen_lhs, widen_rhs, native = _widening_plan(lhs, rhs, allow_native=not gateup)
+    if (gateup and isinstance(rhs, QArray) and not widen_rhs and rhs.qvalue.dtype in (torch.int8, torch.float8_e4m3fn)
+        and rhs.qvalue.shape[2] % 32):
+      # Gate-up fusion reads the up half of a weight row n / 2 elements in, which is a whole 16-byte piece of one-byte
+      # weights only if n % 32 == 0: otherwise the weights are widened first (and quantised activations with them).
+      widen_rhs = True
+      widen_lhs = widen_lhs or isinstance(lhs, QArray)
   else:
     # dlhs / drhs contract unquantised operands (base.py:395-410 rejects quantised ones on the backward path); a
     # quantised operand in a direct call is widened first, as pallas_mosaic_gpu.py:170 does for the drhs product.
@@ -505,6 +511,8 @@ def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True, gateup: bool = Fa
              and lhs.shape[0] * k * 2 < 2**32)
   tiles = (reads_packed and k % _PACKED_INT4_TILE_STEP == 0
            and (blocks == 1 or (scale_ok and not gateup and rows % _PACKED_INT4_TILE_STEP == 0)))
+  if gateup and n % 32:
+    return rhs.unpacked()  # (the up half of a weight row must start on a 16-byte piece: 16 columns of one-byte storage)
   lhs_rows = _per_row_lhs_scale(lhs)
   fp8_tiles = (dims == base.DEFAULT_RAGGED_DOT_DIM_NUMS and isinstance(lhs_rows, QArray) and lhs_rows.zero_point is None
                and lhs_rows.qtype == torch.float8_e4m3fn and len(lhs_rows.qvalue.shape) == 2
@@ -513,13 +521,14 @@ def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True, gateup: bool = Fa
                and (blocks == 1 or (scale_ok and not gateup and rows % _PACKED_INT4_FP8_TILE_STEP == 0
                                     and lhs_rows.qvalue.shape[0] % 4 == 0)))
   # ... or quantised to int8 likewise: the int8 MFMAs on the nibbles (pallas_mosaic_gpu_kernel_sm100_i8_quant.py:
-  # 114-190), no gate-up fusion; scale blocks of a power of two >= 64 rows.
+  # 114-190); scale blocks of a power of two >= 64 rows (not under gate-up fusion).
   int8_tiles = (dims == base.DEFAULT_RAGGED_DOT_DIM_NUMS and isinstance(lhs_rows, QArray) and lhs_rows.zero_point is None
                 and _dtype_of(lhs_rows) == torch.int8 and lhs_rows.qvalue.dtype == torch.int8
-                and len(lhs_rows.qvalue.shape) == 2 and rhs.zero_point is None and n % 16 == 0 and not gateup
+                and len(lhs_rows.qvalue.shape) == 2 and rhs.zero_point is None and n % 16 == 0
                 and k % _PACKED_INT4_FP8_TILE_STEP == 0 and blocks is not None
                 and tuple(lhs_rows.scale.shape) in ((lhs_rows.qvalue.shape[0], 1), (lhs_rows.qvalue.shape[0], blocks))
-                and (blocks == 1 or (scale_ok and rows % _PACKED_INT4_TILE_STEP == 0 and lhs_rows.qvalue.shape[0] % 4 == 0)))
+                and (blocks == 1 or (scale_ok and not gateup and rows % _PACKED_INT4_TILE_STEP == 0
+                                     and lhs_rows.qvalue.shape[0] % 4 == 0)))
   return rhs if streams or tiles or fp8_tiles or int8_tiles else rhs.unpacked()
 
 
@@ -906,7 +915,7 @@ class HipRaggedDot(base.RaggedDot):
       # rows per group, the 128-row one from about 100, and 256 columns from a few tiles' worth of them.
       want_m = 256 if rows_per_group >= 224 else 128
       want_n = 256 if cols >= 512 else 128
-      if (key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2, _lib.TKX_F8E4M3FN)) or int8_int4:
+      if (key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2, _lib.TKX_F8E4M3FN)) or (int8_int4 and mode != 3):
         # (also with gate-up fusion, where the tile sits on one row of four waves, likewise two per CU: 6 % ahead of the
         # 256-row tile at the Mixtral shape and 16-31 % at 128 rows per group; and with scales per k-block: 8-13 %
         # ahead at 128-256 rows per group, even at the Mixtral shape)
