@@ -447,7 +447,7 @@ def main():
     measure("mixtral_gateup_silu_int8_activations_int4_packed_weights",
             lambda: op(lhsi8, q4g, group_sizes=gs, fuse_gateup_activation="silu", preferred_element_type=torch.bfloat16),
             2 * m_ * k_ * 2 * n_, m_ * k_ + m_ * n_ * 2 + 8 * k_ * n_, "mfma", "int8", cfg4i)
-    del q4g, lhs8, lhsi8
+    del lhs8, lhsi8
     # The whole expert FFN of a Mixtral layer around those two products, as a caller strings it together: tokens
     # permuted into expert order (ragged_gather), gate-up product with silu(gate) * up in the epilogue, down
     # projection, weighted top-2 combine back into token order (ragged_gather_reduce). 8192 tokens, top 2 of 8 experts.
@@ -471,7 +471,28 @@ def main():
     block_bytes = (tokens * k_ * 2 + 8 * k_ * 3 * n_) * 2  # tokens in and out, the three weight matrices of every expert
     measure("moe_ffn_block_mixtral_bf16", ffn_block, block_flops, block_bytes, "mfma", "bf16", cfg)
     extras["moe_ffn_block_mixtral_bf16"]["steps"] = "ragged_gather, gate-up ragged_dot (silu fused), down ragged_dot, ragged_gather_reduce (top-2 combine)"
-    del lhs, rhs, h, down
+    del down
+    # The same block with int4 weights packed two to a byte and the activations of both products quantised to fp8 per
+    # row on the way (two quantisation passes): the fp8 MFMAs on the nibbles.
+    q4d = tokamax_amd.pack_int4(tokamax_amd.QArray(
+        torch.randint(-8, 8, (8, n_, k_), device=device, dtype=torch.int8, generator=gen),
+        (torch.rand(8, 1, k_, device=device, generator=gen) + 0.5) / (7 * n_ ** 0.5), None, getattr(torch, "int4", torch.int8)))
+    f8 = torch.float8_e4m3fn
+
+    def ffn_block_w4a8():
+      x = tokamax_amd.ragged_gather(h, token_of_row, 0, tokens)
+      xq = tokamax_amd.QArray(*_ops.quantize(x, f8, (1, k_)))
+      y = op(xq, q4g, group_sizes=gs, fuse_gateup_activation="silu", preferred_element_type=torch.bfloat16)
+      yq = tokamax_amd.QArray(*_ops.quantize(y, f8, (1, n_)))
+      z = op(yq, q4d, group_sizes=gs, preferred_element_type=torch.bfloat16)
+      return tokamax_amd.ragged_gather_reduce(z, inverse, gate_w, valid, 2)
+
+    measure("moe_ffn_block_mixtral_fp8_activations_int4_packed_weights", ffn_block_w4a8, block_flops,
+            tokens * k_ * 2 * 2 + 8 * k_ * 3 * n_ // 2, "mfma", "fp8", cfg48)
+    extras["moe_ffn_block_mixtral_fp8_activations_int4_packed_weights"]["steps"] = (
+        "ragged_gather, quantise rows to fp8, gate-up ragged_dot (silu fused), quantise rows to fp8, down ragged_dot,"
+        " ragged_gather_reduce (top-2 combine)")
+    del lhs, rhs, h, q4g, q4d
 
     # The reference's own benchmark shapes with published timings on other hardware (tokamax/_src/ops/ragged_dot/
     # arg_specs.py:23-60; standard-normal inputs and representative group sizes as its benchmarks make them):
