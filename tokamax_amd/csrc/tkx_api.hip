@@ -77,7 +77,7 @@ struct Registry {
     for (int dtype : {TKX_BF16, TKX_F16})
       for (int depth : {2, 4})
         add({kFwd, dtype, dtype, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
-    for (int depth : {2, 4, 8})  // packed int4 weights: the streaming kernel is their only kernel
+    for (int depth : {2, 4, 8})  // packed int4 weights (their tiled kernels come with variants_i4w)
       add({kFwd, TKX_BF16, TKX_I4X2, kDecodeBlockM, kDecodeBlockN, kDecodeBlockK, 1, kDecodeWaves, depth, 0, nullptr});
   }
 };

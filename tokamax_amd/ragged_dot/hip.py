@@ -495,7 +495,9 @@ def _settle_packed_int4(lhs, rhs, *, dims, plain: bool = True, gateup: bool = Fa
   or under an lhs quantised to fp8 (e4m3fn) with one scale per row (or shared by runs of rows) and k % 128 == 0: the
   tiled kernels that feed the nibbles to the fp8 MFMAs (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:258-300), with one
   scale per (group, column), or, without gate-up fusion and with m % 4 == 0, per (group, k-block, column) with blocks
-  of a power of two >= 128 rows (the lhs scales then per row or per (row, same k-block)).
+  of a power of two >= 128 rows (the lhs scales then per row or per (row, same k-block));
+  or under an lhs quantised to int8 in the same forms (blocks of a power of two >= 64 rows): the int8 MFMAs on the
+  nibbles (pallas_mosaic_gpu_kernel_sm100_i8_quant.py:114-190). Gate-up fusion over packed weights needs n % 32 == 0.
   Every other call gets the values unpacked to int8 storage first (then the int8 paths).
   Works on arrays and on shapes, so the forward pass and the choice of a config settle it alike."""
   if not (isinstance(rhs, QArray) and rhs.packed):
