@@ -225,6 +225,30 @@ def test_e4m3fn_matches_torch_exhaustively():
   np.testing.assert_array_equal(O.e4m3fn_decode(enc), O.e4m3fn_decode(tw))
 
 
+def test_int4_weights_as_fp8_denormals_and_as_int8_times_16():
+  """What the kernels that feed packed int4 weights to the fp8 and int8 matrix instructions rest on
+  (pallas_mosaic_gpu_kernel_sm100_fp8_quant.py:258-300, ..._sm100_i8_quant.py:114-190): the byte 0000uuuu, u = nibble
+  xor 8 = w + 8, decodes as the e4m3 value u / 512 for every int4 w, so sum(x w) = 512 sum(x (w + 8) / 512) - 8 sum(x)
+  in exact arithmetic; and a nibble at the top of a byte is the int8 value 16 w. On a small product against the
+  oracle's definition."""
+  w = np.arange(-8, 8)
+  nibbles = (w & 0xF).astype(np.uint8)
+  np.testing.assert_array_equal(O.e4m3fn_decode(nibbles ^ 8), (w + 8) / 512.0)
+  np.testing.assert_array_equal((nibbles << 4).astype(np.uint8).view(np.int8), 16 * w)
+  rng = np.random.default_rng(4)
+  k, n, rows = 256, 24, 5
+  x = O.e4m3fn_decode(rng.integers(0, 256, (rows, k)).astype(np.uint8) & 0x77 | 0x08).astype(np.float64)  # finite fp8 values
+  values = rng.integers(-8, 8, (1, k, n))
+  want = O.ragged_dot(x, values.astype(np.float64), np.array([rows], np.int32), O.DEFAULT, acc_dtype=np.float64, out_dtype="f64")
+  packed = O.pack_int4(values)[0]
+  as_fp8 = np.empty((k, n))
+  as_fp8[0::2], as_fp8[1::2] = O.e4m3fn_decode((packed & 0xF) ^ 8), O.e4m3fn_decode((packed >> 4) ^ 8)
+  np.testing.assert_allclose(512 * (x @ as_fp8) - 8 * x.sum(axis=1, keepdims=True), want, rtol=0, atol=1e-9)
+  as_int8 = np.empty((k, n))
+  as_int8[0::2], as_int8[1::2] = (packed << 4).astype(np.uint8).view(np.int8), (packed & 0xF0).astype(np.uint8).view(np.int8)
+  np.testing.assert_array_equal((x @ as_int8) / 16, want)
+
+
 def test_fused_epilogue_terms():
   """rhs_bias and gate-up fusion (base.py:205-217): the activations against torch's, the composition
   against brute force on a tiny case."""
