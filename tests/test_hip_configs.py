@@ -167,7 +167,7 @@ def test_packed_int4_weights_at_the_prefill_size(scales, device):
 
 def test_fp8_activations_over_packed_int4_weights_at_the_prefill_size(device):
   """The Mixtral prefill shape with activations quantised to fp8 per row over int4 weights packed two to a byte, on the
-  fp8 MFMAs (the 256-row tile): one row out of every 32-row block of every group against the oracle's definition on
+  fp8 MFMAs (the 128-row tile on one row of four waves): one row out of every 32-row block of every group against the oracle's definition on
   the dequantised operands; scaling the activations' scales by two doubles the result exactly (the affine correction
   with the row sums is applied before the scales); determinism."""
   w = workloads.make("fp8", device)
@@ -179,7 +179,7 @@ def test_fp8_activations_over_packed_int4_weights_at_the_prefill_size(device):
   lhs = tokamax_amd.QArray(w.lhs, w.lhs_scale)
   op = tokamax_amd.HipRaggedDot()
   bound = op.bind(lhs, packed, group_sizes=gs, preferred_element_type=torch.bfloat16)
-  assert op._problem(bound)[1] == (0, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2) and bound.default_config.block_m == 256
+  assert op._problem(bound)[1] == (0, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2) and bound.default_config.block_m == 128
   out = tokamax_amd.ragged_dot(lhs, packed, gs, preferred_element_type=torch.bfloat16)
   assert out.dtype == torch.bfloat16 and tuple(out.shape) == (w.m, w.n)
   rows, groups = _sample_every_block(w.group_sizes, 2)

@@ -673,11 +673,14 @@ def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   shared = tokamax_amd.QArray(ShapeDtype((4096, 1024), f8), ShapeDtype((16, 1), f32))
   assert route8(shared, packed) == (0, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
   wide = tokamax_amd.QArray(ShapeDtype((8, 512, 4096), u8), ShapeDtype((8, 1, 4096), f32), None, int4)
-  c = op._get_heuristics_config(op.bind(x8, wide, group_sizes=gs))   # 512 rows per group: the 256-row tile (two rows of waves)
-  assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages) == (256, 256, 128, 2, 4, 3)
+  # 512 rows per group, and 128: the 128-row tile on one row of four waves, whose workgroups share a CU in pairs
+  c = op._get_heuristics_config(op.bind(x8, wide, group_sizes=gs))
+  assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages) == (128, 256, 128, 1, 4, 2)
   fewer = tokamax_amd.QArray(ShapeDtype((1024, 1024), f8), ShapeDtype((1024, 1), f32))
-  c = op._get_heuristics_config(op.bind(fewer, wide, group_sizes=gs))  # 128 rows per group: 128 rows on one row of waves
-  assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n) == (128, 256, 128, 1, 8)
+  c = op._get_heuristics_config(op.bind(fewer, wide, group_sizes=gs))
+  assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n) == (128, 256, 128, 1, 4)
+  c = op._get_heuristics_config(op.bind(x8, wide, group_sizes=gs, fuse_gateup_activation="silu"))
+  assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n) == (128, 256, 128, 1, 4)
   assert {x.block_k for x in op._get_autotuning_configs(op.bind(x8, wide, group_sizes=gs))} == {128}
   # scale blocks of a power of two >= 128 rows along k (lhs scales per row or per (row, same block)): kernels of the
   # same kind that fold every k-step's products in with its scales; smaller blocks are unpacked and widened
@@ -690,13 +693,13 @@ def test_heuristics_on_abstract_arguments_split_and_packed_int4():
   assert route8(x8, packed, fuse_gateup_activation="silu") == (3, _lib.TKX_F8E4M3FN, _lib.TKX_I4X2)
   assert route8(x8, blocks, fuse_gateup_activation="silu") == (3, _lib.TKX_BF16, _lib.TKX_BF16)
   assert route8(x8, packed.unpacked()) == (0, _lib.TKX_BF16, _lib.TKX_I8)
-  # int8 activations: the int8 MFMAs on the nibbles; the tile whose workgroups share a CU in pairs (two stages: 64 KB)
+  # int8 activations: the int8 MFMAs on the nibbles; again the tile whose 4-wave workgroups share a CU in pairs
   xi8 = tokamax_amd.QArray(ShapeDtype((4096, 1024), i8), ShapeDtype((4096, 1), f32))
   assert route8(xi8, packed) == (0, _lib.TKX_I8, _lib.TKX_I4X2) and route8(xi8, blocks) == (4, _lib.TKX_I8, _lib.TKX_I4X2)
   assert route8(xi8, packed, fuse_gateup_activation="silu") == (3, _lib.TKX_I8, _lib.TKX_I4X2)
   assert route8(xi8, blocks, fuse_gateup_activation="silu")[2] != _lib.TKX_I4X2
   c = op._get_heuristics_config(op.bind(xi8, wide, group_sizes=gs))
-  assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages) == (128, 256, 128, 1, 8, 2)
+  assert (c.block_m, c.block_n, c.block_k, c.waves_m, c.waves_n, c.num_stages) == (128, 256, 128, 1, 4, 2)
   x8_blocks = tokamax_amd.QArray(ShapeDtype((4096, 1024), f8), ShapeDtype((4096, 8), f32))
   assert route8(x8_blocks, packed)[1:] == (_lib.TKX_BF16, _lib.TKX_I8)
   # the key of an autotuning cache entry names the 4-bit type and comes back as the same abstract QArray

@@ -49,6 +49,7 @@ static const Variant kVariants[] = {
     F8FWD(256, 256, 128, 2, 4, 3),
     F8GLU(256, 256, 128, 2, 4, 3),
     F8GLU(128, 256, 128, 2, 4, 3),
+    F8GLU(128, 256, 128, 1, 4, 2),
     F8GLU(64, 256, 128, 2, 4, 3),
     F8GLU(32, 256, 128, 1, 4, 4),
     F8SUBK(128, 256, 128, 2, 4, 3),
@@ -59,10 +60,12 @@ static const Variant kVariants[] = {
     I8FWD(128, 256, 128, 2, 4, 3),
     I8FWD(128, 256, 128, 1, 8, 3),
     I8FWD(128, 256, 128, 1, 8, 2),
+    I8FWD(128, 256, 128, 1, 4, 2),
     I8FWD(64, 128, 128, 2, 2, 4),
     I8FWD(32, 128, 128, 1, 4, 4),
     I8GLU(256, 256, 128, 2, 4, 3),
     I8GLU(128, 256, 128, 2, 4, 3),
+    I8GLU(128, 256, 128, 1, 4, 2),
     I8GLU(64, 256, 128, 2, 4, 3),
     I8GLU(32, 256, 128, 1, 4, 4),
     I8SUBK(128, 256, 128, 2, 4, 3),
@@ -73,6 +76,7 @@ static const Variant kVariants[] = {
     F8FWD(128, 256, 128, 2, 4, 3),
     F8FWD(128, 256, 128, 1, 8, 3),
     F8FWD(128, 256, 128, 1, 8, 4),
+    F8FWD(128, 256, 128, 1, 4, 2),
     F8FWD(128, 128, 128, 2, 2, 4),
     F8FWD(64, 128, 128, 2, 2, 4),
     F8FWD(32, 128, 128, 1, 4, 4),

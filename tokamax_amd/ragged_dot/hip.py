@@ -909,7 +909,14 @@ class HipRaggedDot(base.RaggedDot):
     # (int8 activations over packed int4 weights likewise: 128 x 256 x 128 with two stages is 64 KB and 128 registers,
     # and the fastest on 22 of 26 measured shapes)
     int8_int4 = key[1] == _lib.TKX_I8 and key[2] == _lib.TKX_I4X2
-    converted_plain = mode == 0 and ((key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2)) or int8_int4)
+    f8_int4 = key[1] == _lib.TKX_F8E4M3FN and key[2] == _lib.TKX_I4X2
+    # fp8 or int8 activations over packed int4 weights, plain or with gate-up fusion: 128 x 256 x 128 on one row of
+    # four waves (128 accumulators per lane, one set of converted fragments) with two stages is 64 KB, so two 4-wave
+    # workgroups share a CU behind barriers of their own: the fastest or within 2 % of it on 86 of 95 measured shapes
+    # from 12 rows per group up (the others have too few tiles for it and take the rule below).
+    pairs_of_four = (f8_int4 or int8_int4) and mode in (0, 3)
+    converted_plain = mode == 0 and ((key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2)) or int8_int4
+                                     or f8_int4)
     if mode in (0, 3, 4) and key[1] != _lib.TKX_F32 and rows_per_group >= (12 if converted_plain else 96):
       # The forward kernels other than f32 (16-bit operands without scales are re-ranked by the cost model below): the
       # taller and wider tile pays off earlier than the thresholds above say. Measured on 14 shapes per kind (int8 and
@@ -917,7 +924,7 @@ class HipRaggedDot(base.RaggedDot):
       # rows per group, the 128-row one from about 100, and 256 columns from a few tiles' worth of them.
       want_m = 256 if rows_per_group >= 224 else 128
       want_n = 256 if cols >= 512 else 128
-      if (key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2, _lib.TKX_F8E4M3FN)) or (int8_int4 and mode != 3):
+      if (key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2, _lib.TKX_F8E4M3FN)) or int8_int4 or pairs_of_four:
         # (also with gate-up fusion, where the tile sits on one row of four waves, likewise two per CU: 6 % ahead of the
         # 256-row tile at the Mixtral shape and 16-31 % at 128 rows per group; and with scales per k-block: 8-13 %
         # ahead at 128-256 rows per group, even at the Mixtral shape)
@@ -978,7 +985,9 @@ class HipRaggedDot(base.RaggedDot):
                      + (bn * 4 if mode == 4 else 0))
       alone_on_cu = 0 if ((converted or (int8_int4 and mode == 0)) and wm == 1 and wn == 8 and bm * bn <= 128 * 256
                           and 2 * ns * stage_bytes <= 160 * 1024) else 1
-      return (abs(bm - want_m), abs(bn - want_n), two_wave_rows, -(wm * wn), alone_on_cu if converted or int8_int4 else 0, -in_flight,
+      four_wave_pair = 0 if pairs_of_four and (wm, wn) == (1, 4) and 2 * ns * (bm + bn * 0.5) * bk <= 160 * 1024 else 1
+      return (abs(bm - want_m), abs(bn - want_n), two_wave_rows, four_wave_pair, -(wm * wn),
+              alone_on_cu if converted or int8_int4 else 0, -in_flight,
               bk if short_k else -bk, ns)
 
     bm, bn, bk, wm, wn, ns = min(usable, key=score)
@@ -1020,6 +1029,8 @@ class HipRaggedDot(base.RaggedDot):
         shares = bm * bn <= 128 * 256 and 2 * ns * stage <= 160 * 1024
       if int8_int4 and mode == 0 and wm == 1 and wn == 8:
         shares = bm * bn <= 128 * 256 and 2 * ns * (bm + bn * 0.5) * bk <= 160 * 1024
+      if pairs_of_four and (wm, wn) == (1, 4):
+        shares = 2 * ns * (bm + bn * 0.5) * bk <= 160 * 1024
       estimate = lambda sk: _tile_cost(v, sk, rows, cols, contraction // narrow, num_groups, mode,
                                        rhs_bytes=2.0 if narrow == 2 else rb, shares_cu=shares)
       if key[1] == _lib.TKX_F32 or estimate(4) < estimate(1):
