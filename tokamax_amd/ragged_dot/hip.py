@@ -912,8 +912,8 @@ class HipRaggedDot(base.RaggedDot):
     f8_int4 = key[1] == _lib.TKX_F8E4M3FN and key[2] == _lib.TKX_I4X2
     # fp8 or int8 activations over packed int4 weights, plain or with gate-up fusion: 128 x 256 x 128 on one row of
     # four waves (128 accumulators per lane, one set of converted fragments) with two stages is 64 KB, so two 4-wave
-    # workgroups share a CU behind barriers of their own: the fastest or within 2 % of it on 86 of 95 measured shapes
-    # from 12 rows per group up (the others have too few tiles for it and take the rule below).
+    # workgroups share a CU behind barriers of their own: the fastest or within 2 % of it on 73 of the 87 measured shapes
+    # with 12 rows per group or more (most of the others have too few tiles for it and take the rule below).
     pairs_of_four = (f8_int4 or int8_int4) and mode in (0, 3)
     converted_plain = mode == 0 and ((key[1] == _lib.TKX_BF16 and key[2] in (_lib.TKX_I8, _lib.TKX_I4X2)) or int8_int4
                                      or f8_int4)
