@@ -906,8 +906,8 @@ class HipRaggedDot(base.RaggedDot):
     # row of waves is small enough for two workgroups to share a CU (64 KB of LDS with two stages of int8 weights, 72 KB
     # with three of int4; 128 registers) and was the fastest or within a few percent of it from 12 rows per group up to
     # 2048 (43 measured shapes per kind).
-    # (int8 activations over packed int4 weights likewise: 128 x 256 x 128 with two stages is 64 KB and 128 registers,
-    # and the fastest on 22 of 26 measured shapes)
+    # (int8 activations over packed int4 weights have such a tile too, 128 x 256 x 128 with two stages: the fastest on 22
+    # of 26 shapes until the tile on four waves below, which is 1-2 % ahead of it on most)
     int8_int4 = key[1] == _lib.TKX_I8 and key[2] == _lib.TKX_I4X2
     f8_int4 = key[1] == _lib.TKX_F8E4M3FN and key[2] == _lib.TKX_I4X2
     # fp8 or int8 activations over packed int4 weights, plain or with gate-up fusion: 128 x 256 x 128 on one row of
