@@ -2406,13 +2406,13 @@ def test_timing_tool_collects_every_kind_of_problem(tmp_path, device):
   config among the timed ones."""
   from tokamax_amd.data.autotuning import tile_cost
   path = str(tmp_path / "timings.json")
-  kinds = ["", ",dlhs", ",drhs", ",int8", ",int4", ",fp8", ",fp8i4", ",fp8i4k", ",fp8i4glu", ",int8i4", ",int8i4k", ",int8x8", ",glu",
+  kinds = ["", ",dlhs", ",drhs", ",int8", ",int4", ",fp8", ",fp8i4", ",fp8i4k", ",fp8i4glu", ",int8i4", ",int8i4k", ",int8i4glu", ",int8x8", ",glu",
            ",int8k", ",f32"]
   tile_cost.collect(["768,256,512,4" + k for k in kinds], 2, path=path)
   entries = tile_cost.load(path)
   assert len(entries) == len(kinds) and all(e["timings"] and e["timings"][0][7] > 0 for e in entries)
   assert {e.get("rhs", "bf16") for e in entries} == {"bf16", "int8", "int4", "fp8", "fp8i4", "fp8i4k", "fp8i4glu", "int8i4", "int8i4k",
-                                                     "int8x8", "glu", "int8k", "f32"}
-  assert sorted(e["mode"] for e in entries) == [0] * 13 + [1, 2]
+                                                     "int8i4glu", "int8x8", "glu", "int8k", "f32"}
+  assert sorted(e["mode"] for e in entries) == [0] * 14 + [1, 2]
   for e in entries:
     assert 1.0 <= tile_cost.heuristics_gap(e) < 3.0, e["shape"]

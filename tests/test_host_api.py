@@ -749,7 +749,7 @@ def test_tile_cost_model_picks_near_the_fastest_measured_variant():
   # the config the heuristics hand out for those problems (model, rules for the streaming kernel, split decision), and
   # for quantised operands and drhs, where rules on rows per group and on the fill of the chip choose the tile
   label = lambda e: "drhs" if e["mode"] == 2 else e.get("rhs", "bf16")
-  for kind, count, most in (("bf16", 122, 0.06), ("int8", 26, 0.08), ("int4", 26, 0.06), ("fp8", 26, 0.03), ("fp8i4", 43, 0.04), ("fp8i4k", 26, 0.02), ("fp8i4glu", 26, 0.05), ("int8i4", 26, 0.04), ("int8i4k", 26, 0.03),
+  for kind, count, most in (("bf16", 122, 0.06), ("int8", 26, 0.08), ("int4", 26, 0.06), ("fp8", 26, 0.03), ("fp8i4", 43, 0.04), ("fp8i4k", 26, 0.02), ("fp8i4glu", 26, 0.05), ("int8i4", 26, 0.04), ("int8i4k", 26, 0.03), ("int8i4glu", 26, 0.03),
                             ("int8x8", 12, 0.03), ("drhs", 26, 0.03), ("glu", 26, 0.06), ("int8k", 26, 0.04), ("f32", 12, 0.01)):
     some = [e for e in tile_cost.load() if label(e) == kind]
     mean, worst = tile_cost.summary([tile_cost.heuristics_gap(e) for e in some])

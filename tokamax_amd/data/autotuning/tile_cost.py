@@ -5,14 +5,14 @@ without the split of the last round): entries `{"shape": [rows, contraction, col
 "streaming_best_us": fastest small-m streaming variant or null, "timings": [[block_m, block_n, block_k, waves_m,
 waves_n, num_stages, split_k, microseconds], ...]}`; entries of bf16 activations over quantised weights (one scale per
 (group, column)) carry `"rhs": "int8"` or `"int4"` (packed two to a byte), fp8 x fp8 entries `"rhs": "fp8"`, int8 x int8
-entries `"rhs": "int8x8"`, fp8 activations over packed int4 weights `"fp8i4"` (`"fp8i4k"`: weight scales per 128 k rows, `"fp8i4glu"`: gate-up fusion), int8 activations over them `"int8i4"` / `"int8i4k"`, bf16 gate-up fusion `"glu"`, int8 weights with scales per 128 k rows `"int8k"`, f32 operands `"f32"`; mode 2 is
+entries `"rhs": "int8x8"`, fp8 activations over packed int4 weights `"fp8i4"` (`"fp8i4k"`: weight scales per 128 k rows, `"fp8i4glu"`: gate-up fusion), int8 activations over them `"int8i4"` / `"int8i4k"` / `"int8i4glu"`, bf16 gate-up fusion `"glu"`, int8 weights with scales per 128 k rows `"int8k"`, f32 operands `"f32"`; mode 2 is
 drhs with `"shape": [m, k, n, groups]`. The constants are fitted to the bf16 entries;
 the others are what the rules for quantised weights in `HipRaggedDot._get_heuristics_config` were set by and are
 checked against.
 
   python -m tokamax_amd.data.autotuning.tile_cost check              # how far the model's pick is from the fastest
   python -m tokamax_amd.data.autotuning.tile_cost fit [--iterations N]  # refit; prints the constants to paste
-  python -m tokamax_amd.data.autotuning.tile_cost collect M,K,N,G[,dlhs|drhs|int8|int4|fp8|fp8i4|fp8i4k|fp8i4glu|int8i4|int8i4k|int8x8|glu|int8k|f32] ...   # time shapes on this GPU and add them
+  python -m tokamax_amd.data.autotuning.tile_cost collect M,K,N,G[,dlhs|drhs|int8|int4|fp8|fp8i4|fp8i4k|fp8i4glu|int8i4|int8i4k|int8i4glu|int8x8|glu|int8k|f32] ...   # time shapes on this GPU and add them
 
 `check` and `fit` need no GPU.
 """
@@ -42,7 +42,7 @@ def save(entries: list[dict], path: str | None = None) -> None:
     f.write("[\n" + ",\n".join(json.dumps(e, separators=(",", ":")) for e in entries) + "\n]\n")
 
 
-_RHS_BYTES = {"bf16": 2.0, "int8": 1.0, "int4": 0.5, "fp8i4": 0.5, "fp8i4k": 0.5, "fp8i4glu": 0.5, "int8i4": 0.5, "int8i4k": 0.5}
+_RHS_BYTES = {"bf16": 2.0, "int8": 1.0, "int4": 0.5, "fp8i4": 0.5, "fp8i4k": 0.5, "fp8i4glu": 0.5, "int8i4": 0.5, "int8i4k": 0.5, "int8i4glu": 0.5}
 
 
 def estimate(entry: dict, timing: list, fit: dict) -> float:
@@ -98,7 +98,7 @@ def arguments(entry: dict, array):
     rhs = tokamax_amd.QArray(array(shape, torch.int8, 127), array((groups, 1, cols), f32, 1.0 / (127 * contraction**0.5)))
     return lhs, rhs, dict(kwargs, preferred_element_type=bf16)
   top = 127 if kind == "int8" else 7
-  if kind == "fp8i4glu":  # (`cols` output columns from weights [gate | up] of twice as many)
+  if kind in ("fp8i4glu", "int8i4glu"):  # (`cols` output columns from weights [gate | up] of twice as many)
     shape, kwargs = (groups, contraction, 2 * cols), dict(kwargs, fuse_gateup_activation="silu")
   blocks = contraction // 128 if kind in ("fp8i4k", "int8i4k") else 1
   rhs = tokamax_amd.QArray(array(shape, torch.int8, top), array((groups, blocks, shape[2]), f32, 1.0 / (top * contraction**0.5)),
@@ -196,7 +196,7 @@ def collect(specs: list[str], iterations: int, path: str | None = None) -> None:
     parts = spec.split(",")
     tag = parts[4] if parts[4:] else ""
     mode = {"dlhs": 1, "drhs": 2}.get(tag, 0)
-    kind = tag if tag in ("int8", "int4", "fp8", "fp8i4", "fp8i4k", "fp8i4glu", "int8i4", "int8i4k", "int8x8", "glu", "int8k", "f32") else "bf16"
+    kind = tag if tag in ("int8", "int4", "fp8", "fp8i4", "fp8i4k", "fp8i4glu", "int8i4", "int8i4k", "int8i4glu", "int8x8", "glu", "int8k", "f32") else "bf16"
     dims = [int(x) for x in parts[:4]]
     rng = np.random.default_rng(sum(dims))
     sizes = rng.multinomial(dims[0], rng.dirichlet(np.ones(dims[3]) * 4)).astype(np.int32)
